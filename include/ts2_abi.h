@@ -1,0 +1,159 @@
+/*
+ * ts2_abi.h — C ABI of the MI355X (gfx950) backward path for the TScale2 transformer trainer.
+ *
+ * Every entry point replaces one operator (or kernel launch) of the reference's src/gpt operator surface; the reference
+ * interface it stands for is cited as path:line under the reference tree.  Conventions follow the reference:
+ *   - 2-D device arrays are row-major [y][x] with a byte stride (TCuda2DPtr, src/lib/cuda/cuda_arrays.h:217-253);
+ *   - activations are [token][feature], weights are [out][in], "len" is the number of live token rows;
+ *   - the caller owns every buffer, nothing is allocated or retained by the library, all work is enqueued on the
+ *     caller's stream (a hipStream_t passed as void*) and the call returns without synchronising;
+ *   - device-resident scalars (weight scale, gradient scale) are passed as float* so no host sync is needed
+ *     (TCudaPOD<float>, src/lib/cuda/cuda_arrays.h:54-93).
+ * Errors: the reference aborts (Y_VERIFY, src/util/pch.h:113); here every function returns 0 on success and a negative
+ * TS2_ERR_* code on invalid shapes/alignment/unsupported combinations, and never aborts.
+ */
+#ifndef TS2_ABI_H
+#define TS2_ABI_H
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TS2_OK 0
+#define TS2_ERR_SHAPE (-1)       /* dimension not a multiple of the required tile, or size mismatch */
+#define TS2_ERR_ALIGN (-2)       /* pointer or stride not 16-byte aligned */
+#define TS2_ERR_UNSUPPORTED (-3) /* dtype / epilogue combination not implemented */
+#define TS2_ERR_NULL (-4)        /* required pointer missing */
+#define TS2_ERR_LAUNCH (-5)      /* the HIP runtime refused the launch */
+
+/* element types (TFastModelFloat / TNormStateFloat / TFastGradientFloat choices, src/gpt/compute/cfg_precision.h:20-46) */
+enum ts2_dtype {
+    TS2_I8 = 0,
+    TS2_E4M3 = 1, /* OCP e4m3fn, the format of src/util/fp8.h:4-21 */
+    TS2_BF16 = 2, /* 16-bit activations; the reference uses IEEE half here */
+    TS2_F32 = 3,
+    TS2_I32 = 4
+};
+
+/* row-major 2-D view: TCuda2DPtr<T>{Data, StrideInBytes} + debug sizes, src/lib/cuda/cuda_arrays.h:217-253 */
+typedef struct ts2_mat {
+    void *ptr;
+    int64_t strideBytes;
+    int32_t x; /* columns (elements) */
+    int32_t y; /* rows */
+} ts2_mat;
+
+/* GEMM epilogues = the reference's "store functors", src/lib/cuda/cuda_matmul.cuh:420-559 */
+enum ts2_epilogue {
+    TS2_EPI_STORE = 0,           /* TStore / TStoreScaled        :440-451,467-477 */
+    TS2_EPI_ADD = 1,             /* TStoreAdd / TStoreAddScaled  :455-463,481-490 */
+    TS2_EPI_ROW_TILE_MAXNORM = 2 /* TStoreRowTileMaxNormalize    :530-559  packed delta: i8 + TileScale[n/128][m] */
+};
+
+/*
+ * C[m][n] (op)= alpha * (*alphaPtr) * rowScale[m] * sum_k A[m][k] * B[n][k]
+ * Both operands K-contiguous — the contract of every GEMM core of the reference:
+ *   Int8MatMulKernel / Int8MatMulKernelRowScale / Int8MatMulYScaleKernel  src/lib/cuda/cuda_i8.cuh:157-320
+ *   GenericMatMulKernel (fp8, fp16)                                        src/lib/cuda/cuda_matmul.cuh:396-416
+ * abType: TS2_I8 (int32 accumulate, exact), TS2_E4M3 or TS2_BF16 (fp32 accumulate).
+ * cType : TS2_F32, TS2_BF16, TS2_I32 (raw accumulator, TS2_I8 inputs and TS2_EPI_STORE only) or TS2_I8 (ROW_TILE_MAXNORM).
+ * rowScale  (optional, [m])  : per-row scale of A applied to the accumulator before the epilogue (the dX kernel).
+ * kTileScale (optional, [k/kTile], TS2_I8 only): one scale per kTile contraction rows; each tile's int32 sum is exact and
+ *             tiles are added in fp32 in tile order (the dW kernel).  kTile must be a multiple of 128.
+ * splitK    : >1 splits the contraction over workgroups; partial sums are added with fp32 atomics (TS2_EPI_ADD semantics on a
+ *             C the caller has zeroed, or TS2_EPI_STORE with the library zero-filling first).  1 = deterministic.
+ * Requirements: k a multiple of 128 (8-bit) or 64 (bf16); m, n multiples of 128; 16-byte aligned rows.
+ * Rows >= mLive of C are written as zeros when mLive < m (producers keep pad rows zero, src/lib/cuda/cuda_matmul.cuh:10).
+ */
+typedef struct ts2_gemm_args {
+    ts2_mat a, b, c;
+    int32_t abType, cType;
+    int32_t m, n, k;
+    int32_t mLive; /* 0 = all rows live */
+    const float *rowScale;
+    const float *kTileScale;
+    int32_t kTile;
+    float alpha;
+    const float *alphaPtr;
+    int32_t epilogue;
+    ts2_mat tileScale; /* ROW_TILE_MAXNORM: fp32 [n/128][m] */
+    int32_t splitK;
+    int32_t tileConfig; /* 0 = choose; 1 = 256x256 workgroup tile; 2 = 128x128 */
+} ts2_gemm_args;
+
+int ts2_gemm_nt(const ts2_gemm_args *args, void *stream);
+
+
+/* ------------------------------------------------------------------------------------------------------------------------
+ * Bandwidth-bound fused kernels.  All 2-D operands are [row = token][feature]; feature counts are multiples of 128; per-tile
+ * scale arrays are fp32 [feature/128][row] like the reference's (TFragmentStates::StateScale, layer_cuda_base.cuh:125-149).
+ * "len" = live rows, "lenRound" = rows including padding (multiple of 128) where a kernel also clears the pad rows. */
+
+/* LayerNormalizeStateVecs, src/gpt/compute/gpu_layer_norm.cuh:6-32: per 128-tile scale = sqrt(sum2/128)*vecScale,
+ * normState = state/scale as normType (TS2_I8 | TS2_E4M3 | TS2_BF16), scale 0 and zero data for zero tiles and rows >= len. */
+int ts2_layer_normalize_state_vecs(const ts2_mat *state, int32_t stateType, int32_t len, int32_t lenRound, float vecScale,
+    const ts2_mat *normState, int32_t normType, const ts2_mat *normStateScale, void *stream);
+
+/* BackpropLayerNormalize, src/gpt/compute/gpu_layer_norm.cuh:89-115: g = dNormState * (*combinerScale) * (*gradScale); tile-norm
+ * backward against normState*stateScale; stateGrad += g (fp32, in place); stateGradFast = stateGrad * (*gradMult) as fastType
+ * (TS2_BF16 | TS2_E4M3); atomic max of |stateGrad| into *nextLayerGradMaxNorm.  Scalar pointers may be NULL (= 1). */
+int ts2_backprop_layer_normalize(const ts2_mat *normState, int32_t normType, const ts2_mat *stateScale, const ts2_mat *dNormState,
+    const float *combinerScale, const float *gradScale, const float *gradMult, const ts2_mat *stateGrad, const ts2_mat *stateGradFast,
+    int32_t fastType, float *nextLayerGradMaxNorm, int32_t len, void *stream);
+
+/* BackpropFinalNormalize, src/gpt/compute/gpu_layer_norm.cuh:119-146: same without the residual add; rows >= len are cleared. */
+int ts2_backprop_final_normalize(int32_t len, int32_t lenRound, const ts2_mat *normState, int32_t normType, const ts2_mat *stateScale,
+    const ts2_mat *dNormState, const ts2_mat *stateGrad, const ts2_mat *stateGradFast, int32_t fastType, float *nextLayerGradMaxNorm,
+    void *stream);
+
+/* ScaleGrad + ComputeGradMult, src/gpt/compute/gpu_grad_scale.cuh:33-62: gradMult = 2^floor(log2(128 / *gradMaxNorm)) (1 if the
+ * max is 0); when it differs from *prevGradMult rewrite gradFast = grad * gradMult; publishes *gradScaleOut = 1/gradMult and
+ * *gradMultOut = gradMult. */
+int ts2_scale_grad(const float *gradMaxNorm, const float *prevGradMult, const ts2_mat *grad, const ts2_mat *gradFast, int32_t fastType,
+    int32_t len, float *gradScaleOut, float *gradMultOut, void *stream);
+
+/* MatrixLoLU, src/gpt/compute/gpu_lolu.cuh:41-69: res = vals * sigmoid(2*gate) * resMult as resType; rows in [len, lenRound) zero.
+ * gate and vals are TS2_BF16. */
+int ts2_matrix_lolu(int32_t len, int32_t lenRound, const ts2_mat *gate, const ts2_mat *vals, float resMult, const ts2_mat *res,
+    int32_t resType, void *stream);
+
+/* BackpropRowTileNormalizeLoLU, src/gpt/compute/gpu_lolu.cuh:107-137 (FFN): vals*valsScale is the normalised "wide"; gradGate =
+ * grad*vals*m(1-m)*2, gradVals = tile-norm backward of (grad*m) against vals*valsSrcTileScale; outputs as gradOutType. */
+int ts2_backprop_row_tile_normalize_lolu(int32_t len, int32_t lenRound, const ts2_mat *gate, const ts2_mat *vals, float valsScale,
+    const ts2_mat *valsSrcTileScale, const ts2_mat *grad, int32_t gradType, const ts2_mat *gradGate, const ts2_mat *gradVals,
+    int32_t gradOutType, void *stream);
+
+/* BackpropLoLUdScale, src/gpt/compute/gpu_lolu.cuh:141-173 (attention): gate backward plus dScale[head][t] = <vals*valsScale,
+ * gradVals> per 128-wide head. */
+int ts2_backprop_lolu_dscale(int32_t len, int32_t lenRound, const ts2_mat *gate, const ts2_mat *vals, float valsScale, const ts2_mat *grad,
+    int32_t gradType, const ts2_mat *gradGate, int32_t gradGateType, const ts2_mat *gradVals, int32_t gradValsType, const ts2_mat *dScale,
+    void *stream);
+
+/* NormalizeVecsRowMaxKernel, src/gpt/compute/row_scale.cuh:12-43, deterministic (the reference adds a random dither before rounding):
+ * per row scale = maxabs/127, dst = sat_i8(rne(src/scale)); optional colScale[x] multiplies the source first; rows >= len cleared. */
+int ts2_normalize_vecs_row_max(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, const float *colScale,
+    const ts2_mat *dst, float *rowScale, void *stream);
+
+/* Per-k-tile abs-max of a [len][dim] matrix (optionally times rowMult[t]): tileMax[t/kTile] = max |src|, the first half of
+ * ShuffleMaxScaleTransposeKernel (src/gpt/compute/matmul_fwdbwd.cuh:209-231) without the sort.  tileMax must be zeroed by the
+ * caller or with clear=1. */
+int ts2_tile_absmax(int32_t len, const ts2_mat *src, int32_t srcType, const float *rowMult, int32_t kTile, float *tileMax, int32_t clear,
+    void *stream);
+
+/* Quantise + transpose: dst[x][t] = cvt(src[t][x] * rowMult[t] * mult(t)) for t < len, 0 for len <= t < lenRound.
+ * dstType TS2_I8: mult = 127/tileMax[t/kTile] and tileScale[t/kTile] = tileMax/127 (1 when the tile is all zero) is written;
+ * dstType equal to srcType (1-byte types): pure byte transpose (TransposeI8Matrix, src/lib/cuda/cuda_i8.cuh:14-71;
+ * ShuffleTransposeKernel / ShuffleMaxScaleTransposeKernel, src/gpt/compute/matmul_fwdbwd.cuh:169-280).
+ * rowIndex (optional, [lenRound], -1 = zero row) gathers source rows first (MoeGroupSamples, moe_kernels.cuh:89-143). */
+int ts2_transpose_quant(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, const float *rowMult, const float *tileMax,
+    int32_t kTile, const int32_t *rowIndex, const ts2_mat *dstT, int32_t dstType, float *tileScale, void *stream);
+
+/* peak dense MFMA rate the library prices its kernels against, in T(FL)OP/s, and the CU count it tiles for */
+int ts2_device_info(int *cuCount, int *clockMHz);
+const char *ts2_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -193,5 +193,10 @@ class Oracle:
         self._f("convert_e4m3")(_ptr(d), _ptr(s), s.size, C.c_float(mult))
         return d.reshape(np.shape(src))
 
-    def e4m3_table(self):
-        return np.array([self._f("e4m3_to_float")(c) for c in range(256)], F32)
+    def e4m3_table(self, hw=False):
+        """code -> value.  hw=True gives the hardware (OCP) reading of code 0x80 as -0; the reference's slow decoder
+        (src/util/fp8.h:4-21) only special-cases code 0 and reads 0x80 as -2^-7, a code its own encoder never emits."""
+        tab = np.array([self._f("e4m3_to_float")(c) for c in range(256)], F32)
+        if hw:
+            tab[0x80] = -0.0
+        return tab

@@ -1,0 +1,641 @@
+// Bandwidth-bound fused gradient kernels (tile norm forward/backward + residual add, dynamic gradient scaling, gated sigmoid
+// forward/backward, per-row and per-k-tile int8 quantisation, 8-bit transposes).
+//
+// Mapping for gfx950: one 128-wide tile is held by 32 lanes x 4 elements, so a 64-wide wavefront processes two tiles per
+// instruction with 16-byte (fp32), 8-byte (bf16) or 4-byte (8-bit) accesses per lane; reductions stay inside the 32-lane group
+// (5 cross-lane steps).  Workgroups are 256 threads (8 tiles in flight) and grids cover every (row, tile) once, so each launch puts
+// thousands of workgroups on the 256 CUs; consecutive 32-lane groups walk consecutive tiles of a row, i.e. HBM accesses are fully
+// coalesced 512-byte (fp32) runs.  The reference launches one 32-thread block per (tile, row) (src/lib/cuda/cuda_graph.cuh:359-365).
+#include "vec.h"
+
+namespace
+{
+struct Mat {
+    uint8_t *p;
+    int64_t ld;
+};
+
+__host__ __device__ __forceinline__ Mat M(const ts2_mat &m)
+{
+    Mat r = {(uint8_t *)m.ptr, m.strideBytes};
+    return r;
+}
+
+template <class TT> __device__ __forceinline__ void *At(const Mat &m, int row, int col)
+{
+    return m.p + (int64_t)row * m.ld + (int64_t)col * TT::SIZE;
+}
+
+__device__ __forceinline__ float &ScaleAt(const Mat &m, int tile, int row)
+{
+    return *(float *)(m.p + (int64_t)tile * m.ld + (int64_t)row * 4);
+}
+
+// (row, tile) of this 32-lane group; returns false when out of range
+__device__ __forceinline__ bool Unit(int rows, int tiles, int *row, int *tile, int *lane32)
+{
+    long u = ((long)blockIdx.x * blockDim.x + threadIdx.x) >> 5;
+    *lane32 = threadIdx.x & 31;
+    *row = (int)(u / tiles);
+    *tile = (int)(u - (long)(*row) * tiles);
+    return *row < rows;
+}
+
+inline dim3 GridFor(int rows, int tiles)
+{
+    long units = (long)rows * tiles;
+    return dim3((unsigned)((units * 32 + 255) / 256));
+}
+
+// non-negative float max through the integer ordering, like the reference's atomicMax((int*)p, __float_as_int(x))
+__device__ __forceinline__ void AtomicMaxPos(float *p, float v)
+{
+    atomicMax((int *)p, __float_as_int(v));
+}
+
+// --------------------------------------------------------------------------------------------------------------------------
+template <class TSrc, class TDst>
+__global__ void __launch_bounds__(256) LayerNormalizeStateVecs(int len, int lenRound, int tiles, float vecScale, Mat state, Mat normState, Mat normScale)
+{
+    int t, tile, h;
+    if (!Unit(lenRound, tiles, &t, &tile, &h)) {
+        return;
+    }
+    int col = tile * TILE + h * 4;
+    float discr = 0;
+    F4 v = ZeroF4();
+    if (t < len) {
+        v = Load4<TSrc>(At<TSrc>(state, t, col));
+        float sum2 = Half32Sum(HSum(v * v));
+        if (sum2 > 0) {
+            discr = sqrtf(sum2 / TILE) * vecScale;
+            v = v * (1 / discr);
+        }
+    }
+    Store4<TDst>(At<TDst>(normState, t, col), v);
+    if (h == 0) {
+        ScaleAt(normScale, tile, t) = discr;
+    }
+}
+
+template <class TNorm, class TFast, bool FINAL>
+__global__ void __launch_bounds__(256) BackpropLayerNormalize(int len, int rows, int tiles, Mat normState, Mat stateScale, Mat dNormState,
+    const float *combinerScale, const float *gradScale, const float *gradMult, Mat stateGrad, Mat stateGradFast, float *nextMaxNorm)
+{
+    int t, tile, h;
+    if (!Unit(rows, tiles, &t, &tile, &h)) {
+        return;
+    }
+    int col = tile * TILE + h * 4;
+    if (t >= len) {
+        Store4<TF32>(At<TF32>(stateGrad, t, col), ZeroF4());
+        Store4<TFast>(At<TFast>(stateGradFast, t, col), ZeroF4());
+        return;
+    }
+    F4 vec = Load4<TNorm>(At<TNorm>(normState, t, col)) * ScaleAt(stateScale, tile, t);
+    F4 grad = Load4<TF32>(At<TF32>(dNormState, t, col));
+    if (!FINAL) {
+        float s = 1;
+        if (combinerScale) {
+            s *= *combinerScale;
+        }
+        if (gradScale) {
+            s *= *gradScale;
+        }
+        grad = grad * s;
+    }
+    grad = TileNormBackprop(vec, grad);
+    if (!FINAL) {
+        grad = grad + Load4<TF32>(At<TF32>(stateGrad, t, col));
+    }
+    float gmax = Half32Max(HMaxAbs(grad));
+    Store4<TF32>(At<TF32>(stateGrad, t, col), grad);
+    float gm = (!FINAL && gradMult) ? *gradMult : 1.f;
+    Store4<TFast>(At<TFast>(stateGradFast, t, col), grad * gm);
+    if (h == 0 && nextMaxNorm) {
+        AtomicMaxPos(nextMaxNorm, gmax);
+    }
+}
+
+__device__ __forceinline__ float ComputeGradMult(float gradMaxNorm)
+{
+    if (gradMaxNorm == 0) {
+        return 1;
+    }
+    return __uint_as_float(__float_as_uint(128.f / gradMaxNorm) & 0xff800000u);
+}
+
+template <class TFast>
+__global__ void __launch_bounds__(256) ScaleGrad(int len, int tiles, const float *gradMaxNorm, const float *prevGradMult, Mat grad, Mat gradFast,
+    float *gradScaleOut, float *gradMultOut)
+{
+    int t, tile, h;
+    float gradMult = ComputeGradMult(*gradMaxNorm);
+    bool rewrite = !prevGradMult || gradMult != *prevGradMult;
+    if (Unit(len, tiles, &t, &tile, &h) && rewrite) {
+        int col = tile * TILE + h * 4;
+        F4 v = Load4<TF32>(At<TF32>(grad, t, col));
+        Store4<TFast>(At<TFast>(gradFast, t, col), v * gradMult);
+    }
+}
+
+// published after the rewrite kernel so that a caller may pass the same cell as prevGradMult and gradMultOut
+__global__ void PublishGradMult(const float *gradMaxNorm, float *gradScaleOut, float *gradMultOut)
+{
+    float gradMult = ComputeGradMult(*gradMaxNorm);
+    if (gradScaleOut) {
+        *gradScaleOut = 1 / gradMult;
+    }
+    if (gradMultOut) {
+        *gradMultOut = gradMult;
+    }
+}
+
+template <class TDst>
+__global__ void __launch_bounds__(256) MatrixLoLU(int len, int lenRound, int tiles, Mat gate, Mat vals, float resMult, Mat res)
+{
+    int t, tile, h;
+    if (!Unit(lenRound, tiles, &t, &tile, &h)) {
+        return;
+    }
+    int col = tile * TILE + h * 4;
+    F4 v = ZeroF4();
+    if (t < len) {
+        F4 g = Load4<TBF16>(At<TBF16>(gate, t, col));
+        v = Load4<TBF16>(At<TBF16>(vals, t, col)) * LoLU4(g) * resMult;
+    }
+    Store4<TDst>(At<TDst>(res, t, col), v);
+}
+
+// MODE 0: FFN (tile-norm backward of vals fused); MODE 1: attention (dScale fused)
+template <class TGrad, class TOutG, class TOutV, int MODE>
+__global__ void __launch_bounds__(256) BackpropLoLU(int len, int lenRound, int tiles, Mat gate, Mat vals, float valsScale, Mat valsSrcTileScale,
+    Mat gradArr, Mat gradGate, Mat gradVals, Mat dScale)
+{
+    int t, tile, h;
+    if (!Unit(lenRound, tiles, &t, &tile, &h)) {
+        return;
+    }
+    int col = tile * TILE + h * 4;
+    float ds = 0;
+    if (t < len) {
+        F4 g = Load4<TBF16>(At<TBF16>(gate, t, col));
+        F4 v = Load4<TBF16>(At<TBF16>(vals, t, col)) * valsScale;
+        F4 grad = Load4<TGrad>(At<TGrad>(gradArr, t, col));
+        F4 mult = LoLU4(g);
+        F4 resGate = grad * v * LoLUGrad4(mult);
+        F4 resVals = grad * mult;
+        Store4<TOutG>(At<TOutG>(gradGate, t, col), resGate);
+        if (MODE == 0) {
+            // un-normalised source = normalised * (tile scale / valsScale)
+            F4 src = v * (ScaleAt(valsSrcTileScale, tile, t) / valsScale);
+            resVals = TileNormBackprop(src, resVals);
+        } else {
+            ds = Half32Sum(HSum(v * resVals));
+        }
+        Store4<TOutV>(At<TOutV>(gradVals, t, col), resVals);
+    } else {
+        Store4<TOutG>(At<TOutG>(gradGate, t, col), ZeroF4());
+        Store4<TOutV>(At<TOutV>(gradVals, t, col), ZeroF4());
+    }
+    if (MODE == 1 && h == 0) {
+        ScaleAt(dScale, tile, t) = ds;
+    }
+}
+
+// one workgroup per row: abs-max over the row, then quantise.  The row is read twice (second read served by L2).
+template <class TSrc>
+__global__ void __launch_bounds__(256) NormalizeVecsRowMax(int len, int dim, Mat src, const float *colScale, Mat dst, float *rowScale)
+{
+    __shared__ float red[4];
+    int t = blockIdx.x;
+    int tid = threadIdx.x;
+    if (t >= len) {
+        for (int col = tid * 4; col < dim; col += 1024) {
+            *(uint32_t *)At<TI8>(dst, t, col) = 0;
+        }
+        if (tid == 0) {
+            rowScale[t] = 0;
+        }
+        return;
+    }
+    float mx = 0;
+    for (int col = tid * 4; col < dim; col += 1024) {
+        F4 v = Load4<TSrc>(At<TSrc>(src, t, col));
+        if (colScale) {
+            v = v * Load4<TF32>(colScale + col);
+        }
+        mx = fmaxf(mx, HMaxAbs(v));
+    }
+    mx = WaveMax(mx);
+    if ((tid & 63) == 0) {
+        red[tid >> 6] = mx;
+    }
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    float discr = 0, mult = 0;
+    if (mx > 0) {
+        discr = mx / 127;
+        mult = 1 / discr;
+    }
+    for (int col = tid * 4; col < dim; col += 1024) {
+        F4 v = Load4<TSrc>(At<TSrc>(src, t, col));
+        if (colScale) {
+            v = v * Load4<TF32>(colScale + col);
+        }
+        Store4<TI8>(At<TI8>(dst, t, col), v * mult);
+    }
+    if (tid == 0) {
+        rowScale[t] = discr;
+    }
+}
+
+__global__ void FillFloats(float *p, int n, float v)
+{
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        p[i] = v;
+    }
+}
+
+// grid (dim/1024 rounded up, len/ROWS): every workgroup reduces ROWS rows x 1024 columns and issues one atomic
+template <class TSrc>
+__global__ void __launch_bounds__(256) TileAbsMax(int len, int dim, Mat src, const float *rowMult, int kTile, float *tileMax)
+{
+    constexpr int ROWS = 16;
+    __shared__ float red[4];
+    int tid = threadIdx.x;
+    int col = blockIdx.x * 1024 + tid * 4;
+    int t0 = blockIdx.y * ROWS;
+    float mx = 0;
+    if (col < dim) {
+        for (int r = 0; r < ROWS; ++r) {
+            int t = t0 + r;
+            if (t < len) {
+                F4 v = Load4<TSrc>(At<TSrc>(src, t, col));
+                float m = HMaxAbs(v);
+                if (rowMult) {
+                    m *= fabsf(rowMult[t]);
+                }
+                mx = fmaxf(mx, m);
+            }
+        }
+    }
+    mx = WaveMax(mx);
+    if ((tid & 63) == 0) {
+        red[tid >> 6] = mx;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+        AtomicMaxPos(&tileMax[t0 / kTile], mx);
+    }
+}
+
+// 128 (rows t) x 128 (columns x) tile: coalesced row loads, conversion, byte tile in LDS, 4x4 byte transposes in registers with
+// v_perm_b32, 4-byte stores that are contiguous along t across lanes (128-byte runs per destination row).
+template <class TSrc, bool QUANT>
+__global__ void __launch_bounds__(256) TransposeQuant(int len, int lenRound, Mat src, const float *rowMult, const float *tileMax, int kTile,
+    const int *rowIndex, Mat dst, float *tileScale)
+{
+    constexpr int PITCH = 132; // bytes per LDS row: keeps the column-wise dword reads spread over the banks
+    __shared__ __attribute__((aligned(16))) uint8_t buf[128 * PITCH];
+    int tid = threadIdx.x;
+    int xBlock = blockIdx.x * 128;
+    int tBlock = blockIdx.y * 128;
+    // load + convert: 32 lanes cover one row of 128 columns, 8 rows per pass
+    int h = tid & 31;
+    for (int r = tid >> 5; r < 128; r += 8) {
+        int t = tBlock + r;
+        uint32_t packed = 0;
+        if (t < len) {
+            int srcRow = rowIndex ? rowIndex[t] : t;
+            if (srcRow >= 0) {
+                if (QUANT) {
+                    F4 v = Load4<TSrc>(At<TSrc>(src, srcRow, xBlock + h * 4));
+                    float tm = tileMax[t / kTile];
+                    float mult = tm > 0 ? 127.f / tm : 0.f;
+                    if (rowMult) {
+                        mult *= rowMult[srcRow];
+                    }
+                    v = v * mult;
+                    packed = (uint32_t)(CvtToI8(v.x) & 0xff) | ((uint32_t)(CvtToI8(v.y) & 0xff) << 8) | ((uint32_t)(CvtToI8(v.z) & 0xff) << 16) |
+                             ((uint32_t)(CvtToI8(v.w) & 0xff) << 24);
+                } else {
+                    packed = *(const uint32_t *)(src.p + (int64_t)srcRow * src.ld + xBlock + h * 4);
+                }
+            }
+        }
+        *(uint32_t *)(buf + r * PITCH + h * 4) = packed;
+    }
+    __syncthreads();
+    // transpose: thread -> (tq = t quad, xq = x quad); 32 tq x 32 xq = 1024 quads, 4 per thread
+    int tq = tid & 31;
+    for (int xq = tid >> 5; xq < 32; xq += 8) {
+        uint32_t r0 = *(const uint32_t *)(buf + (tq * 4 + 0) * PITCH + xq * 4);
+        uint32_t r1 = *(const uint32_t *)(buf + (tq * 4 + 1) * PITCH + xq * 4);
+        uint32_t r2 = *(const uint32_t *)(buf + (tq * 4 + 2) * PITCH + xq * 4);
+        uint32_t r3 = *(const uint32_t *)(buf + (tq * 4 + 3) * PITCH + xq * 4);
+        // 4x4 byte transpose.  __builtin_amdgcn_perm(hi, lo, sel): result byte i = byte sel[i] of {hi:lo} (lo = bytes 0-3)
+        uint32_t a = __builtin_amdgcn_perm(r1, r0, 0x05010400); // r0.b0 r1.b0 r0.b1 r1.b1
+        uint32_t b = __builtin_amdgcn_perm(r1, r0, 0x07030602); // r0.b2 r1.b2 r0.b3 r1.b3
+        uint32_t c = __builtin_amdgcn_perm(r3, r2, 0x05010400);
+        uint32_t d = __builtin_amdgcn_perm(r3, r2, 0x07030602);
+        uint32_t c0 = __builtin_amdgcn_perm(c, a, 0x05040100); // column 0: r0.b0 r1.b0 r2.b0 r3.b0
+        uint32_t c1 = __builtin_amdgcn_perm(c, a, 0x07060302);
+        uint32_t c2 = __builtin_amdgcn_perm(d, b, 0x05040100);
+        uint32_t c3 = __builtin_amdgcn_perm(d, b, 0x07060302);
+        int x = xBlock + xq * 4;
+        int tcol = tBlock + tq * 4;
+        *(uint32_t *)(dst.p + (int64_t)(x + 0) * dst.ld + tcol) = c0;
+        *(uint32_t *)(dst.p + (int64_t)(x + 1) * dst.ld + tcol) = c1;
+        *(uint32_t *)(dst.p + (int64_t)(x + 2) * dst.ld + tcol) = c2;
+        *(uint32_t *)(dst.p + (int64_t)(x + 3) * dst.ld + tcol) = c3;
+    }
+    if (QUANT && tileScale && blockIdx.x == 0 && tid == 0) {
+        // one 128-row block lies inside one k-tile (kTile is a multiple of 128)
+        float tm = tileMax[tBlock / kTile];
+        tileScale[tBlock / kTile] = tm > 0 ? tm / 127 : 1.f;
+    }
+}
+
+bool MatOk(const ts2_mat *m, int rows, int cols, int elemSize)
+{
+    return m && m->ptr && m->y >= rows && m->x >= cols && (m->strideBytes % 4) == 0 && m->strideBytes >= (int64_t)cols * elemSize;
+}
+
+int ElemSize(int type)
+{
+    switch (type) {
+    case TS2_F32:
+    case TS2_I32:
+        return 4;
+    case TS2_BF16:
+        return 2;
+    default:
+        return 1;
+    }
+}
+} // namespace
+
+#define STREAM ((hipStream_t)stream)
+
+extern "C" int ts2_layer_normalize_state_vecs(const ts2_mat *state, int32_t stateType, int32_t len, int32_t lenRound, float vecScale,
+    const ts2_mat *normState, int32_t normType, const ts2_mat *normStateScale, void *stream)
+{
+    if (!state || !normState || !normStateScale) {
+        return TS2_ERR_NULL;
+    }
+    int dim = state->x;
+    if (dim % TILE || lenRound < len || !MatOk(state, len, dim, ElemSize(stateType)) || !MatOk(normState, lenRound, dim, ElemSize(normType)) ||
+        !MatOk(normStateScale, dim / TILE, lenRound, 4)) {
+        return TS2_ERR_SHAPE;
+    }
+    int tiles = dim / TILE;
+    TS2_DISPATCH_TYPE(stateType, TS, TS2_DISPATCH_TYPE(normType, TD,
+        hipLaunchKernelGGL((LayerNormalizeStateVecs<TS, TD>), GridFor(lenRound, tiles), dim3(256), 0, STREAM, len, lenRound, tiles, vecScale,
+            M(*state), M(*normState), M(*normStateScale))));
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
+static int BackpropNormImpl(bool final, int len, int rows, const ts2_mat *normState, int normType, const ts2_mat *stateScale,
+    const ts2_mat *dNormState, const float *combinerScale, const float *gradScale, const float *gradMult, const ts2_mat *stateGrad,
+    const ts2_mat *stateGradFast, int fastType, float *nextMaxNorm, void *stream)
+{
+    if (!normState || !stateScale || !dNormState || !stateGrad || !stateGradFast) {
+        return TS2_ERR_NULL;
+    }
+    int dim = dNormState->x;
+    if (dim % TILE || !MatOk(normState, len, dim, ElemSize(normType)) || !MatOk(stateScale, dim / TILE, len, 4) ||
+        !MatOk(dNormState, len, dim, 4) || !MatOk(stateGrad, rows, dim, 4) || !MatOk(stateGradFast, rows, dim, ElemSize(fastType))) {
+        return TS2_ERR_SHAPE;
+    }
+    if (normType == TS2_F32 || (fastType != TS2_BF16 && fastType != TS2_E4M3)) {
+        return TS2_ERR_UNSUPPORTED;
+    }
+    int tiles = dim / TILE;
+#define LAUNCH_BN(TN, TFA)                                                                                                                 \
+    if (final)                                                                                                                             \
+        hipLaunchKernelGGL((BackpropLayerNormalize<TN, TFA, true>), GridFor(rows, tiles), dim3(256), 0, STREAM, len, rows, tiles,         \
+            M(*normState), M(*stateScale), M(*dNormState), combinerScale, gradScale, gradMult, M(*stateGrad), M(*stateGradFast), nextMaxNorm); \
+    else                                                                                                                                   \
+        hipLaunchKernelGGL((BackpropLayerNormalize<TN, TFA, false>), GridFor(rows, tiles), dim3(256), 0, STREAM, len, rows, tiles,        \
+            M(*normState), M(*stateScale), M(*dNormState), combinerScale, gradScale, gradMult, M(*stateGrad), M(*stateGradFast), nextMaxNorm)
+    if (fastType == TS2_BF16) {
+        TS2_DISPATCH_TYPE(normType, TN, LAUNCH_BN(TN, TBF16));
+    } else {
+        TS2_DISPATCH_TYPE(normType, TN, LAUNCH_BN(TN, TE4M3));
+    }
+#undef LAUNCH_BN
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
+extern "C" int ts2_backprop_layer_normalize(const ts2_mat *normState, int32_t normType, const ts2_mat *stateScale, const ts2_mat *dNormState,
+    const float *combinerScale, const float *gradScale, const float *gradMult, const ts2_mat *stateGrad, const ts2_mat *stateGradFast,
+    int32_t fastType, float *nextLayerGradMaxNorm, int32_t len, void *stream)
+{
+    return BackpropNormImpl(false, len, len, normState, normType, stateScale, dNormState, combinerScale, gradScale, gradMult, stateGrad,
+        stateGradFast, fastType, nextLayerGradMaxNorm, stream);
+}
+
+extern "C" int ts2_backprop_final_normalize(int32_t len, int32_t lenRound, const ts2_mat *normState, int32_t normType, const ts2_mat *stateScale,
+    const ts2_mat *dNormState, const ts2_mat *stateGrad, const ts2_mat *stateGradFast, int32_t fastType, float *nextLayerGradMaxNorm,
+    void *stream)
+{
+    return BackpropNormImpl(true, len, lenRound, normState, normType, stateScale, dNormState, nullptr, nullptr, nullptr, stateGrad, stateGradFast,
+        fastType, nextLayerGradMaxNorm, stream);
+}
+
+extern "C" int ts2_scale_grad(const float *gradMaxNorm, const float *prevGradMult, const ts2_mat *grad, const ts2_mat *gradFast, int32_t fastType,
+    int32_t len, float *gradScaleOut, float *gradMultOut, void *stream)
+{
+    if (!gradMaxNorm || !grad || !gradFast) {
+        return TS2_ERR_NULL;
+    }
+    int dim = grad->x;
+    if (dim % TILE || !MatOk(grad, len, dim, 4) || !MatOk(gradFast, len, dim, ElemSize(fastType))) {
+        return TS2_ERR_SHAPE;
+    }
+    int tiles = dim / TILE;
+    if (fastType == TS2_BF16) {
+        hipLaunchKernelGGL((ScaleGrad<TBF16>), GridFor(len, tiles), dim3(256), 0, STREAM, len, tiles, gradMaxNorm, prevGradMult, M(*grad),
+            M(*gradFast), gradScaleOut, gradMultOut);
+    } else if (fastType == TS2_E4M3) {
+        hipLaunchKernelGGL((ScaleGrad<TE4M3>), GridFor(len, tiles), dim3(256), 0, STREAM, len, tiles, gradMaxNorm, prevGradMult, M(*grad),
+            M(*gradFast), gradScaleOut, gradMultOut);
+    } else {
+        return TS2_ERR_UNSUPPORTED;
+    }
+    TS2_CHECK_LAUNCH();
+    hipLaunchKernelGGL(PublishGradMult, dim3(1), dim3(1), 0, STREAM, gradMaxNorm, gradScaleOut, gradMultOut);
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
+extern "C" int ts2_matrix_lolu(int32_t len, int32_t lenRound, const ts2_mat *gate, const ts2_mat *vals, float resMult, const ts2_mat *res,
+    int32_t resType, void *stream)
+{
+    if (!gate || !vals || !res) {
+        return TS2_ERR_NULL;
+    }
+    int dim = res->x;
+    if (dim % TILE || !MatOk(gate, len, dim, 2) || !MatOk(vals, len, dim, 2) || !MatOk(res, lenRound, dim, ElemSize(resType))) {
+        return TS2_ERR_SHAPE;
+    }
+    int tiles = dim / TILE;
+    TS2_DISPATCH_TYPE(resType, TD,
+        hipLaunchKernelGGL((MatrixLoLU<TD>), GridFor(lenRound, tiles), dim3(256), 0, STREAM, len, lenRound, tiles, M(*gate), M(*vals), resMult,
+            M(*res)));
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
+template <int MODE>
+static int BackpropLoluImpl(int len, int lenRound, const ts2_mat *gate, const ts2_mat *vals, float valsScale, const ts2_mat *tileScale,
+    const ts2_mat *grad, int gradType, const ts2_mat *gradGate, int ggType, const ts2_mat *gradVals, int gvType, const ts2_mat *dScale, void *stream)
+{
+    if (!gate || !vals || !grad || !gradGate || !gradVals || (MODE == 0 ? !tileScale : !dScale)) {
+        return TS2_ERR_NULL;
+    }
+    int dim = grad->x;
+    if (dim % TILE || !MatOk(gate, len, dim, 2) || !MatOk(vals, len, dim, 2) || !MatOk(grad, len, dim, ElemSize(gradType)) ||
+        !MatOk(gradGate, lenRound, dim, ElemSize(ggType)) || !MatOk(gradVals, lenRound, dim, ElemSize(gvType))) {
+        return TS2_ERR_SHAPE;
+    }
+    if (MODE == 0 ? !MatOk(tileScale, dim / TILE, len, 4) : !MatOk(dScale, dim / TILE, lenRound, 4)) {
+        return TS2_ERR_SHAPE;
+    }
+    int tiles = dim / TILE;
+    Mat ts = MODE == 0 ? M(*tileScale) : Mat{nullptr, 0};
+    Mat ds = MODE == 1 ? M(*dScale) : Mat{nullptr, 0};
+    if ((gradType != TS2_BF16 && gradType != TS2_F32) || (ggType != TS2_BF16 && ggType != TS2_E4M3) || (gvType != TS2_BF16 && gvType != TS2_E4M3)) {
+        return TS2_ERR_UNSUPPORTED;
+    }
+#define LAUNCH_BL(TG, TOG, TOV)                                                                                                            \
+    hipLaunchKernelGGL((BackpropLoLU<TG, TOG, TOV, MODE>), GridFor(lenRound, tiles), dim3(256), 0, STREAM, len, lenRound, tiles, M(*gate),  \
+        M(*vals), valsScale, ts, M(*grad), M(*gradGate), M(*gradVals), ds)
+    if (gradType == TS2_BF16) {
+        if (ggType == TS2_BF16 && gvType == TS2_BF16) {
+            LAUNCH_BL(TBF16, TBF16, TBF16);
+        } else if (ggType == TS2_E4M3 && gvType == TS2_E4M3) {
+            LAUNCH_BL(TBF16, TE4M3, TE4M3);
+        } else if (ggType == TS2_E4M3 && gvType == TS2_BF16) {
+            LAUNCH_BL(TBF16, TE4M3, TBF16);
+        } else {
+            return TS2_ERR_UNSUPPORTED;
+        }
+    } else {
+        if (ggType == TS2_BF16 && gvType == TS2_BF16) {
+            LAUNCH_BL(TF32, TBF16, TBF16);
+        } else if (ggType == TS2_E4M3 && gvType == TS2_E4M3) {
+            LAUNCH_BL(TF32, TE4M3, TE4M3);
+        } else if (ggType == TS2_E4M3 && gvType == TS2_BF16) {
+            LAUNCH_BL(TF32, TE4M3, TBF16);
+        } else {
+            return TS2_ERR_UNSUPPORTED;
+        }
+    }
+#undef LAUNCH_BL
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
+extern "C" int ts2_backprop_row_tile_normalize_lolu(int32_t len, int32_t lenRound, const ts2_mat *gate, const ts2_mat *vals, float valsScale,
+    const ts2_mat *valsSrcTileScale, const ts2_mat *grad, int32_t gradType, const ts2_mat *gradGate, const ts2_mat *gradVals,
+    int32_t gradOutType, void *stream)
+{
+    return BackpropLoluImpl<0>(len, lenRound, gate, vals, valsScale, valsSrcTileScale, grad, gradType, gradGate, gradOutType, gradVals,
+        gradOutType, nullptr, stream);
+}
+
+extern "C" int ts2_backprop_lolu_dscale(int32_t len, int32_t lenRound, const ts2_mat *gate, const ts2_mat *vals, float valsScale,
+    const ts2_mat *grad, int32_t gradType, const ts2_mat *gradGate, int32_t gradGateType, const ts2_mat *gradVals, int32_t gradValsType,
+    const ts2_mat *dScale, void *stream)
+{
+    return BackpropLoluImpl<1>(len, lenRound, gate, vals, valsScale, nullptr, grad, gradType, gradGate, gradGateType, gradVals, gradValsType,
+        dScale, stream);
+}
+
+extern "C" int ts2_normalize_vecs_row_max(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, const float *colScale,
+    const ts2_mat *dst, float *rowScale, void *stream)
+{
+    if (!src || !dst || !rowScale) {
+        return TS2_ERR_NULL;
+    }
+    int dim = dst->x;
+    if (dim % 4 || lenRound < len || !MatOk(src, len, dim, ElemSize(srcType)) || !MatOk(dst, lenRound, dim, 1)) {
+        return TS2_ERR_SHAPE;
+    }
+    if (srcType == TS2_BF16) {
+        hipLaunchKernelGGL((NormalizeVecsRowMax<TBF16>), dim3(lenRound), dim3(256), 0, STREAM, len, dim, M(*src), colScale, M(*dst), rowScale);
+    } else if (srcType == TS2_F32) {
+        hipLaunchKernelGGL((NormalizeVecsRowMax<TF32>), dim3(lenRound), dim3(256), 0, STREAM, len, dim, M(*src), colScale, M(*dst), rowScale);
+    } else {
+        return TS2_ERR_UNSUPPORTED;
+    }
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
+extern "C" int ts2_tile_absmax(int32_t len, const ts2_mat *src, int32_t srcType, const float *rowMult, int32_t kTile, float *tileMax, int32_t clear,
+    void *stream)
+{
+    if (!src || !tileMax) {
+        return TS2_ERR_NULL;
+    }
+    int dim = src->x;
+    if (dim % 4 || kTile <= 0 || kTile % 128 || !MatOk(src, len, dim, ElemSize(srcType))) {
+        return TS2_ERR_SHAPE;
+    }
+    int nTiles = (len + kTile - 1) / kTile;
+    if (clear) {
+        hipLaunchKernelGGL(FillFloats, dim3((nTiles + 255) / 256), dim3(256), 0, STREAM, tileMax, nTiles, 0.f);
+        TS2_CHECK_LAUNCH();
+    }
+    dim3 grid((dim + 1023) / 1024, (len + 15) / 16);
+    if (srcType == TS2_BF16) {
+        hipLaunchKernelGGL((TileAbsMax<TBF16>), grid, dim3(256), 0, STREAM, len, dim, M(*src), rowMult, kTile, tileMax);
+    } else if (srcType == TS2_F32) {
+        hipLaunchKernelGGL((TileAbsMax<TF32>), grid, dim3(256), 0, STREAM, len, dim, M(*src), rowMult, kTile, tileMax);
+    } else {
+        return TS2_ERR_UNSUPPORTED;
+    }
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
+extern "C" int ts2_transpose_quant(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, const float *rowMult, const float *tileMax,
+    int32_t kTile, const int32_t *rowIndex, const ts2_mat *dstT, int32_t dstType, float *tileScale, void *stream)
+{
+    if (!src || !dstT) {
+        return TS2_ERR_NULL;
+    }
+    int dim = dstT->y;
+    if (dim % 128 || lenRound % 128 || lenRound < len || dstT->x < lenRound || src->x < dim || (dstT->strideBytes % 4) ||
+        dstT->strideBytes < lenRound) {
+        return TS2_ERR_SHAPE;
+    }
+    dim3 grid(dim / 128, lenRound / 128);
+    bool quant = dstType == TS2_I8 && (srcType == TS2_BF16 || srcType == TS2_F32);
+    if (quant) {
+        if (!tileMax || kTile <= 0 || kTile % 128) {
+            return TS2_ERR_SHAPE;
+        }
+        if (srcType == TS2_BF16) {
+            hipLaunchKernelGGL((TransposeQuant<TBF16, true>), grid, dim3(256), 0, STREAM, len, lenRound, M(*src), rowMult, tileMax, kTile, rowIndex,
+                M(*dstT), tileScale);
+        } else {
+            hipLaunchKernelGGL((TransposeQuant<TF32, true>), grid, dim3(256), 0, STREAM, len, lenRound, M(*src), rowMult, tileMax, kTile, rowIndex,
+                M(*dstT), tileScale);
+        }
+    } else if (ElemSize(srcType) == 1 && dstType == srcType) {
+        hipLaunchKernelGGL((TransposeQuant<TI8, false>), grid, dim3(256), 0, STREAM, len, lenRound, M(*src), nullptr, nullptr, 128, rowIndex,
+            M(*dstT), nullptr);
+    } else {
+        return TS2_ERR_UNSUPPORTED;
+    }
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}

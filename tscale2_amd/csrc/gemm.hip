@@ -1,0 +1,547 @@
+// NT GEMM on gfx950 MFMA for 8-bit (i8, e4m3) and bf16 operands:  C[m][n] (op)= scale * sum_k A[m][k] * B[n][k]
+//
+// Replaces the reference's GEMM cores (src/lib/cuda/cuda_i8.cuh:157-320, src/lib/cuda/cuda_matmul.cuh:396-416,
+// src/lib/cuda/sm90_fp8.cuh:171-217) with one CDNA4 design:
+//   * a workgroup = 4 wavefronts (2x2), each wave owns a (32*WTM) x (32*WTN) block of C as WTM x WTN MFMA 32x32 accumulators
+//     (WTM = WTN = 4 -> 256x256 workgroup tile, 256 accumulator registers per lane; 2 -> 128x128);
+//   * K advances 128 bytes per step; A and B tiles are fetched with 16-byte global loads into registers while the MFMAs of the
+//     previous step run, then written to a double-buffered LDS tile whose 16-byte chunks are XOR-swizzled by (row/2)%8 so that both
+//     the ds_write_b128 of the loader and the ds_read_b128 of the MFMA operand fetch are bank-conflict free; one barrier per step;
+//   * MFMA: v_mfma_i32_32x32x32_i8, v_mfma_f32_32x32x64_f8f6f4 (fp8 x fp8), v_mfma_f32_32x32x16_bf16;
+//   * workgroup ids are remapped so that each of the 8 XCDs (which receive ids round-robin) works on a compact band of C tiles
+//     and its L2 sees every A/B panel only a few times;
+//   * the epilogue (per-row scale, alpha, device scalar, store/add, bf16/fp32/i32, packed int8 delta) is fused.
+#include "common.h"
+
+namespace
+{
+struct GemmP {
+    const uint8_t *a;
+    const uint8_t *b;
+    uint8_t *c;
+    int64_t lda, ldb, ldc; // bytes
+    int m, n, kBytes;      // kBytes = K * sizeof(element)
+    int mLive;
+    const float *rowScale;
+    const float *kTileScale;
+    int kTileBytes;
+    float alpha;
+    const float *alphaPtr;
+    float *tileScale;
+    int64_t ldTileScale; // floats
+    int splitK;
+    int tilesM, tilesN;
+};
+
+enum { T_I8 = 0, T_FP8 = 1, T_BF16 = 2 };
+enum { C_F32 = 0, C_BF16 = 1, C_I32 = 2, C_I8PACK = 3 };
+
+constexpr int BKB = 128; // bytes of K per step
+
+template <int TYPE> struct AccT {
+    typedef v16f type;
+};
+template <> struct AccT<T_I8> {
+    typedef v16i type;
+};
+
+__device__ __forceinline__ int SwizzleOffset(int row, int chunk)
+{
+    return row * BKB + ((chunk ^ ((row >> 1) & 7)) << 4);
+}
+
+// tile id -> (tileM, tileN): XCD-aware, then grouped along M
+__device__ __forceinline__ void MapTile(int bid, int nb, int tilesM, int tilesN, int *tm, int *tn)
+{
+    int id = bid;
+    if ((nb & 7) == 0) {
+        id = (bid & 7) * (nb >> 3) + (bid >> 3);
+    }
+    constexpr int GROUP = 8;
+    int perGroup = GROUP * tilesN;
+    int g = id / perGroup;
+    int first = g * GROUP;
+    int gsz = tilesM - first < GROUP ? tilesM - first : GROUP;
+    int r = id - g * perGroup;
+    *tm = first + r % gsz;
+    *tn = r / gsz;
+}
+
+template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT>
+__global__ void __launch_bounds__(256, 1) GemmNT(GemmP p)
+{
+    typedef typename AccT<TYPE>::type TAcc;
+    constexpr int BM = 64 * WTM;
+    constexpr int BN = 64 * WTN;
+    constexpr int LA = BM / 32; // 16-byte loads per thread for the A tile
+    constexpr int LB = BN / 32;
+    constexpr int STAGE = (BM + BN) * BKB;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave >> 1;
+    const int wn = wave & 1;
+
+    int tm, tn;
+    const int tilesMN = p.tilesM * p.tilesN;
+    int bid = blockIdx.x;
+    int split = 0;
+    if (p.splitK > 1) {
+        split = bid / tilesMN;
+        bid -= split * tilesMN;
+    }
+    MapTile(bid, tilesMN, p.tilesM, p.tilesN, &tm, &tn);
+    const int rowBase = tm * BM;
+    const int colBase = tn * BN;
+
+    // contraction range of this workgroup
+    int kSteps = p.kBytes / BKB;
+    int kBeg = 0;
+    if (p.splitK > 1) {
+        int per = (kSteps + p.splitK - 1) / p.splitK;
+        if (KT) {
+            int tileSteps = p.kTileBytes / BKB;
+            per = (per + tileSteps - 1) / tileSteps * tileSteps;
+        }
+        kBeg = split * per;
+        int kEnd = kBeg + per < kSteps ? kBeg + per : kSteps;
+        kSteps = kEnd - kBeg;
+        if (kSteps <= 0) {
+            return;
+        }
+    }
+
+    // global load addressing: thread -> (row = tid/8 + 32*i, 16-byte chunk = tid%8)
+    const int lc = tid & 7;
+    const int lr = tid >> 3;
+    const uint8_t *gaBase = p.a + (int64_t)(rowBase + lr) * p.lda + (int64_t)kBeg * BKB + lc * 16;
+    const uint8_t *gbBase = p.b + (int64_t)(colBase + lr) * p.ldb + (int64_t)kBeg * BKB + lc * 16;
+    v4i ra[LA], rb[LB];
+
+    auto loadGlobal = [&](int step) {
+#pragma unroll
+        for (int i = 0; i < LA; ++i) {
+            ra[i] = *(const v4i *)(gaBase + (int64_t)i * 32 * p.lda + (int64_t)step * BKB);
+        }
+#pragma unroll
+        for (int i = 0; i < LB; ++i) {
+            rb[i] = *(const v4i *)(gbBase + (int64_t)i * 32 * p.ldb + (int64_t)step * BKB);
+        }
+    };
+    auto storeLds = [&](int stage) {
+        uint8_t *sa = lds + stage * STAGE;
+        uint8_t *sb = sa + BM * BKB;
+#pragma unroll
+        for (int i = 0; i < LA; ++i) {
+            *(v4i *)(sa + SwizzleOffset(lr + 32 * i, lc)) = ra[i];
+        }
+#pragma unroll
+        for (int i = 0; i < LB; ++i) {
+            *(v4i *)(sb + SwizzleOffset(lr + 32 * i, lc)) = rb[i];
+        }
+    };
+
+    TAcc acc[WTM][WTN];
+    v16f facc[KT ? WTM : 1][KT ? WTN : 1];
+#pragma unroll
+    for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+        for (int j = 0; j < WTN; ++j) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                acc[i][j][e] = 0;
+            }
+        }
+    }
+    if (KT) {
+#pragma unroll
+        for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+            for (int j = 0; j < WTN; ++j) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    facc[i][j][e] = 0;
+                }
+            }
+        }
+    }
+
+    const int half = lane >> 5;
+    const int l32 = lane & 31;
+    const int aRow0 = wm * (32 * WTM) + l32;
+    const int bRow0 = wn * (32 * WTN) + l32;
+
+    auto compute = [&](int stage) {
+        const uint8_t *sa = lds + stage * STAGE;
+        const uint8_t *sb = sa + BM * BKB;
+        if (TYPE == T_FP8) {
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                v8i fa[WTM], fb[WTN];
+                int ch = s * 4 + half * 2;
+#pragma unroll
+                for (int i = 0; i < WTM; ++i) {
+                    v4i lo = *(const v4i *)(sa + SwizzleOffset(aRow0 + 32 * i, ch));
+                    v4i hi = *(const v4i *)(sa + SwizzleOffset(aRow0 + 32 * i, ch + 1));
+                    fa[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                }
+#pragma unroll
+                for (int j = 0; j < WTN; ++j) {
+                    v4i lo = *(const v4i *)(sb + SwizzleOffset(bRow0 + 32 * j, ch));
+                    v4i hi = *(const v4i *)(sb + SwizzleOffset(bRow0 + 32 * j, ch + 1));
+                    fb[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                }
+#pragma unroll
+                for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+                    for (int j = 0; j < WTN; ++j) {
+                        if constexpr (TYPE == T_FP8) {
+                            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], 0, 0, 0, 0, 0, 0);
+                        }
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                v4i fa[WTM], fb[WTN];
+                int ch = s * 2 + half;
+#pragma unroll
+                for (int i = 0; i < WTM; ++i) {
+                    fa[i] = *(const v4i *)(sa + SwizzleOffset(aRow0 + 32 * i, ch));
+                }
+#pragma unroll
+                for (int j = 0; j < WTN; ++j) {
+                    fb[j] = *(const v4i *)(sb + SwizzleOffset(bRow0 + 32 * j, ch));
+                }
+#pragma unroll
+                for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+                    for (int j = 0; j < WTN; ++j) {
+                        if constexpr (TYPE == T_I8) {
+                            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+                        } else if constexpr (TYPE == T_BF16) {
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                                __builtin_bit_cast(v8bf, fa[i]), __builtin_bit_cast(v8bf, fb[j]), acc[i][j], 0, 0, 0);
+                        }
+                    }
+                }
+            }
+        }
+    };
+
+    // main loop: one barrier per step, LDS double buffered, global loads of step s+1 in flight during the MFMAs of step s
+    loadGlobal(0);
+    storeLds(0);
+    __syncthreads();
+    const int tileSteps = KT ? p.kTileBytes / BKB : 0;
+    for (int s = 0; s < kSteps; ++s) {
+        int cur = s & 1;
+        if (s + 1 < kSteps) {
+            loadGlobal(s + 1);
+        }
+        compute(cur);
+        if (KT) {
+            if ((s + 1) % tileSteps == 0 || s + 1 == kSteps) {
+                float sc = p.kTileScale[(kBeg + s) / tileSteps];
+#pragma unroll
+                for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+                    for (int j = 0; j < WTN; ++j) {
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) {
+                            facc[i][j][e] += sc * (float)acc[i][j][e];
+                            acc[i][j][e] = 0;
+                        }
+                    }
+                }
+            }
+        }
+        if (s + 1 < kSteps) {
+            storeLds(cur ^ 1);
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue.  MFMA 32x32 result: lane holds column l32, rows (e/4)*8 + half*4 + e%4
+    float scale = p.alpha;
+    if (p.alphaPtr) {
+        scale *= *p.alphaPtr;
+    }
+    const int mLive = p.mLive > 0 ? p.mLive : p.m;
+    auto accVal = [&](int i, int j, int e) -> float {
+        if constexpr (KT) {
+            return facc[i][j][e];
+        } else {
+            return (float)acc[i][j][e];
+        }
+    };
+    auto rowLocal = [&](int i, int e) { return wm * (32 * WTM) + i * 32 + (e >> 2) * 8 + half * 4 + (e & 3); };
+
+    if constexpr (CT == C_I8PACK) {
+        // TStoreRowTileMaxNormalize (src/lib/cuda/cuda_matmul.cuh:530-559): per row and 128 columns scale = maxabs/127, bytes =
+        // sat_i8(rne(v/scale)), TileScale[tile][row] = scale.  A 128-column tile is 4 MFMA blocks: inside one wave when WTN == 4,
+        // shared by the two waves along N when WTN == 2 (row maxima exchanged through LDS, which the main loop no longer uses).
+        float *xch = (float *)lds;
+        if (WTN == 2) {
+#pragma unroll
+            for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    float mx = 0;
+#pragma unroll
+                    for (int j = 0; j < WTN; ++j) {
+                        mx = fmaxf(mx, fabsf(accVal(i, j, e)));
+                    }
+                    mx = Half32Max(mx);
+                    if (l32 == 0) {
+                        xch[rowLocal(i, e) * 2 + wn] = mx;
+                    }
+                }
+            }
+            __syncthreads();
+        }
+#pragma unroll
+        for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int rl = rowLocal(i, e);
+                const int row = rowBase + rl;
+                float rs = scale;
+                if (p.rowScale) {
+                    rs *= p.rowScale[row];
+                }
+                rs = fabsf(rs);
+                float mx = 0;
+                if (WTN == 2) {
+                    mx = fmaxf(xch[rl * 2], xch[rl * 2 + 1]);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < WTN; ++j) {
+                        mx = fmaxf(mx, fabsf(accVal(i, j, e)));
+                    }
+                    mx = Half32Max(mx);
+                }
+                mx *= rs;
+                float discr = 0, mult = 0;
+                if (mx > 0 && row < mLive) {
+                    discr = mx / 127;
+                    mult = 1 / discr;
+                }
+                float sgnScale = (p.rowScale ? p.rowScale[row] : 1.f) * scale;
+#pragma unroll
+                for (int j = 0; j < WTN; ++j) {
+                    int col = colBase + wn * (32 * WTN) + j * 32 + l32;
+                    ((int8_t *)p.c)[(int64_t)row * p.ldc + col] = (int8_t)CvtToI8(accVal(i, j, e) * sgnScale * mult);
+                }
+                if (l32 == 0 && (WTN == 4 || wn == 0)) {
+                    int tile = (colBase + wn * (32 * WTN)) / TILE;
+                    p.tileScale[(int64_t)tile * p.ldTileScale + row] = discr;
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int row = rowBase + rowLocal(i, e);
+                const bool live = row < mLive;
+                float rs = scale;
+                if (p.rowScale) {
+                    rs *= p.rowScale[row];
+                }
+                uint8_t *dst = p.c + (int64_t)row * p.ldc;
+#pragma unroll
+                for (int j = 0; j < WTN; ++j) {
+                    const int col = colBase + wn * (32 * WTN) + j * 32 + l32;
+                    if constexpr (CT == C_I32) {
+                        if constexpr (TYPE == T_I8) {
+                            ((int *)dst)[col] = acc[i][j][e];
+                        }
+                    } else {
+                        float v = live ? accVal(i, j, e) * rs : 0.f;
+                        if constexpr (CT == C_F32) {
+                            float *d = (float *)dst + col;
+                            if (p.splitK > 1) {
+                                if (live) {
+                                    atomicAdd(d, v);
+                                }
+                            } else if (EPI == TS2_EPI_ADD) {
+                                if (live) {
+                                    *d += v;
+                                }
+                            } else {
+                                *d = v;
+                            }
+                        } else if constexpr (CT == C_BF16) {
+                            bf16_t *d = (bf16_t *)dst + col;
+                            if (EPI == TS2_EPI_ADD) {
+                                if (live) {
+                                    *d = FloatToBf16(Bf16ToFloat(*d) + v);
+                                }
+                            } else {
+                                *d = FloatToBf16(v);
+                            }
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+__global__ void ZeroRows(uint8_t *c, int64_t ldc, int rowBytes)
+{
+    uint8_t *row = c + (int64_t)blockIdx.x * ldc;
+    for (int x = threadIdx.x * 4; x < rowBytes; x += blockDim.x * 4) {
+        *(int *)(row + x) = 0;
+    }
+}
+
+template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT> int Launch(const GemmP &p, hipStream_t stream)
+{
+    constexpr int BM = 64 * WTM, BN = 64 * WTN;
+    GemmP q = p;
+    q.tilesM = (p.m + BM - 1) / BM;
+    q.tilesN = (p.n + BN - 1) / BN;
+    int ldsBytes = 2 * (BM + BN) * BKB;
+    auto kern = GemmNT<TYPE, WTM, WTN, CT, EPI, KT>;
+    static bool attrDone = false; // per instantiation
+    if (!attrDone) {
+        if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes) != hipSuccess) {
+            return TS2_ERR_LAUNCH;
+        }
+        attrDone = true;
+    }
+    int nb = q.tilesM * q.tilesN * (p.splitK > 1 ? p.splitK : 1);
+    hipLaunchKernelGGL(kern, dim3(nb), dim3(256), ldsBytes, stream, q);
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
+template <int TYPE, int WTM, int WTN> int DispatchEpi(const ts2_gemm_args *a, const GemmP &p, hipStream_t stream)
+{
+    const bool kt = a->kTileScale != nullptr;
+    const int epi = a->epilogue;
+    if (epi == TS2_EPI_ROW_TILE_MAXNORM) {
+        if (a->cType != TS2_I8) {
+            return TS2_ERR_UNSUPPORTED;
+        }
+        if (kt) {
+            if constexpr (TYPE == T_I8 && WTM == 2) {
+                return Launch<TYPE, WTM, WTN, C_I8PACK, TS2_EPI_STORE, true>(p, stream);
+            }
+            return TS2_ERR_UNSUPPORTED;
+        }
+        return Launch<TYPE, WTM, WTN, C_I8PACK, TS2_EPI_STORE, false>(p, stream);
+    }
+    if (a->cType == TS2_I32) {
+        if constexpr (TYPE == T_I8) {
+            if (epi == TS2_EPI_STORE && !kt) {
+                return Launch<TYPE, WTM, WTN, C_I32, TS2_EPI_STORE, false>(p, stream);
+            }
+        }
+        return TS2_ERR_UNSUPPORTED;
+    }
+    if (kt) {
+        if constexpr (TYPE == T_I8 && WTM == 2) {
+            if (a->cType == TS2_F32) {
+                return epi == TS2_EPI_ADD ? Launch<TYPE, WTM, WTN, C_F32, TS2_EPI_ADD, true>(p, stream)
+                                          : Launch<TYPE, WTM, WTN, C_F32, TS2_EPI_STORE, true>(p, stream);
+            }
+        }
+        return TS2_ERR_UNSUPPORTED;
+    }
+    if (a->cType == TS2_F32) {
+        return epi == TS2_EPI_ADD ? Launch<TYPE, WTM, WTN, C_F32, TS2_EPI_ADD, false>(p, stream)
+                                  : Launch<TYPE, WTM, WTN, C_F32, TS2_EPI_STORE, false>(p, stream);
+    }
+    if (a->cType == TS2_BF16) {
+        return epi == TS2_EPI_ADD ? Launch<TYPE, WTM, WTN, C_BF16, TS2_EPI_ADD, false>(p, stream)
+                                  : Launch<TYPE, WTM, WTN, C_BF16, TS2_EPI_STORE, false>(p, stream);
+    }
+    return TS2_ERR_UNSUPPORTED;
+}
+
+template <int TYPE> int DispatchTile(const ts2_gemm_args *a, const GemmP &p, hipStream_t stream)
+{
+    int cfg = a->tileConfig;
+    if (cfg == 0) {
+        // 256x256 tiles only when they still fill the chip; the k-tile-scaled kernel keeps a second accumulator set and needs 128x128
+        long tilesL = (long)(p.m / 256) * (p.n / 256) * (p.splitK > 1 ? p.splitK : 1);
+        cfg = tilesL >= 192 ? 1 : 2;
+    }
+    // the 256x256 kernel needs full tiles and has no room for the second accumulator set of the k-tile-scaled variant
+    if (cfg == 1 && !a->kTileScale && (p.m % 256) == 0 && (p.n % 256) == 0) {
+        return DispatchEpi<TYPE, 4, 4>(a, p, stream);
+    }
+    return DispatchEpi<TYPE, 2, 2>(a, p, stream);
+}
+} // namespace
+
+extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
+{
+    if (!a || !a->a.ptr || !a->b.ptr || !a->c.ptr) {
+        return TS2_ERR_NULL;
+    }
+    hipStream_t stream = (hipStream_t)streamPtr;
+    int esz = a->abType == TS2_BF16 ? 2 : 1;
+    if (a->abType != TS2_I8 && a->abType != TS2_E4M3 && a->abType != TS2_BF16) {
+        return TS2_ERR_UNSUPPORTED;
+    }
+    if (a->m <= 0 || a->n <= 0 || a->k <= 0 || (a->m % 128) || (a->n % 128) || ((int64_t)a->k * esz) % BKB) {
+        return TS2_ERR_SHAPE;
+    }
+    if (!Aligned16(a->a.ptr, a->a.strideBytes) || !Aligned16(a->b.ptr, a->b.strideBytes) || (((uintptr_t)a->c.ptr) & 3)) {
+        return TS2_ERR_ALIGN;
+    }
+    if (a->a.y < a->m || a->b.y < a->n || a->a.x < a->k || a->b.x < a->k || a->c.y < a->m || a->c.x < a->n) {
+        return TS2_ERR_SHAPE;
+    }
+    if (a->kTileScale && (a->abType != TS2_I8 || a->kTile <= 0 || (a->kTile % 128) || (a->k % a->kTile))) {
+        return TS2_ERR_SHAPE;
+    }
+    int splitK = a->splitK > 1 ? a->splitK : 1;
+    if (splitK > 1 && (a->cType != TS2_F32 || a->epilogue == TS2_EPI_ROW_TILE_MAXNORM)) {
+        return TS2_ERR_UNSUPPORTED;
+    }
+    if (a->epilogue == TS2_EPI_ROW_TILE_MAXNORM && (!a->tileScale.ptr || a->tileScale.y < a->n / 128 || a->tileScale.x < a->m)) {
+        return TS2_ERR_SHAPE;
+    }
+    GemmP p;
+    p.a = (const uint8_t *)a->a.ptr;
+    p.b = (const uint8_t *)a->b.ptr;
+    p.c = (uint8_t *)a->c.ptr;
+    p.lda = a->a.strideBytes;
+    p.ldb = a->b.strideBytes;
+    p.ldc = a->epilogue == TS2_EPI_ROW_TILE_MAXNORM ? a->c.strideBytes : a->c.strideBytes;
+    p.m = a->m;
+    p.n = a->n;
+    p.kBytes = a->k * esz;
+    p.mLive = a->mLive;
+    p.rowScale = a->rowScale;
+    p.kTileScale = a->kTileScale;
+    p.kTileBytes = a->kTile * esz;
+    p.alpha = a->alpha;
+    p.alphaPtr = a->alphaPtr;
+    p.tileScale = (float *)a->tileScale.ptr;
+    p.ldTileScale = a->tileScale.strideBytes / 4;
+    p.splitK = splitK;
+    p.tilesM = p.tilesN = 0;
+    if (splitK > 1 && a->epilogue == TS2_EPI_STORE) {
+        // partial sums are accumulated with atomics: clear the live rows first (with a fill kernel, which is safe under graph capture)
+        hipLaunchKernelGGL(ZeroRows, dim3(a->m), dim3(256), 0, stream, (uint8_t *)a->c.ptr, (int64_t)a->c.strideBytes, a->n * 4);
+        TS2_CHECK_LAUNCH();
+    }
+    switch (a->abType) {
+    case TS2_I8:
+        return DispatchTile<T_I8>(a, p, stream);
+    case TS2_E4M3:
+        return DispatchTile<T_FP8>(a, p, stream);
+    default:
+        return DispatchTile<T_BF16>(a, p, stream);
+    }
+}
