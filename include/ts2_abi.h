@@ -149,6 +149,53 @@ int ts2_tile_absmax(int32_t len, const ts2_mat *src, int32_t srcType, const floa
 int ts2_transpose_quant(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, const float *rowMult, const float *tileMax,
     int32_t kTile, const int32_t *rowIndex, const ts2_mat *dstT, int32_t dstType, float *tileScale, void *stream);
 
+/* ------------------------------------------------------------------------------------------------------------------------
+ * Linear-layer backward operator = TMatMulBuffers::{BackpropMulti, BackpropDelta} + Backprop()
+ * (src/gpt/compute/layer_cuda_base.cuh:153-250) over TInt8MatMulBwdBuffers / TFp8MatMulBwdBuffers
+ * (src/gpt/compute/matmul_fwdbwd.cuh:108-163,283-391).  mode = TS2_I8 or TS2_E4M3 (BWD_MATMUL_TYPE, cfg_precision.h:20-35).
+ *
+ * Scratch is caller-owned, like the reference's pool-allocated members; every buffer the mode does not use may be empty:
+ *   grad8 [lenRound][gradDim] i8 + grad8RowScale [lenRound]   (I8: Grad8, Grad8RowScale)
+ *   gradT [gradDim][lenRound] 8-bit                             (I8: Grad8T; E4M3: GradE5T)
+ *   srcT  [srcDim][lenRound] 8-bit                              (I8: Src8T;  E4M3: SrcE4T)
+ *   tileMax, tileScale [lenRound/kTile] fp32                    (I8: SortedTileScale)
+ *   transformT [srcDim][gradDim] 8-bit                          (TransformT)
+ * Differences from the reference, by design: no random dither in the int8 quantisers, no sort of the rows (each kTile
+ * consecutive tokens share the delta GEMM's scale) and exact int32 sums per k-tile added in fp32. */
+typedef struct ts2_matmul_bwd_buffers {
+    ts2_mat grad8;
+    float *grad8RowScale;
+    ts2_mat gradT;
+    ts2_mat srcT;
+    float *tileMax;
+    float *tileScale;
+    ts2_mat transformT;
+} ts2_matmul_bwd_buffers;
+
+/* BackpropMulti (prep of dX): I8: quantise grad (TS2_BF16 | TS2_F32, optionally times gradColScale[gradDim]) per row to
+ * grad8/grad8RowScale and transpose the weight; E4M3: transpose the weight.  transformFast is [gradDim][srcDim]. */
+int ts2_matmul_backprop_multi(int32_t mode, int32_t len, int32_t lenRound, int32_t srcDim, int32_t gradDim, const ts2_mat *transformFast,
+    const ts2_mat *grad, int32_t gradType, const float *gradColScale, const ts2_matmul_bwd_buffers *buf, void *stream);
+
+/* Backprop(): srcGrad[len][srcDim] (+)= alpha * (*alphaPtr) * grad * W.  I8 reads grad8/grad8RowScale from buf; E4M3 reads grad
+ * (e4m3 [lenRound][gradDim]) directly.  srcGradType TS2_F32 | TS2_BF16; add != 0 accumulates (multi-source sum). */
+int ts2_matmul_backprop(int32_t mode, int32_t len, int32_t lenRound, int32_t srcDim, int32_t gradDim, const ts2_mat *grad,
+    const ts2_matmul_bwd_buffers *buf, float alpha, const float *alphaPtr, const ts2_mat *srcGrad, int32_t srcGradType, int32_t add,
+    void *stream);
+
+/* BackpropDelta: delta[gradDim][srcDim] = (*gradScale) * sum_t grad[t][k]*src[t][x] as the packed delta (i8 + tileScale
+ * [srcDim/128][gradDim], TCudaPackedDeltaMatrix, src/gpt/matrix/delta_cuda.h:9-38).  src is the 8-bit layer input
+ * [lenRound][srcDim]; I8: grad (TS2_BF16 | TS2_F32) is requantised per kTile rows (times srcRowScale[t] if given);
+ * E4M3: grad is e4m3 and only transposed. */
+int ts2_matmul_backprop_delta(int32_t mode, int32_t len, int32_t lenRound, int32_t srcDim, int32_t gradDim, const ts2_mat *src,
+    const float *srcRowScale, const ts2_mat *grad, int32_t gradType, const float *gradScale, int32_t kTile,
+    const ts2_matmul_bwd_buffers *buf, const ts2_mat *delta, const ts2_mat *deltaTileScale, void *stream);
+
+/* Forward product of the same operator, TMatMulBuffers::Forward<TStoreScaled> (layer_cuda_base.cuh:183-193):
+ * res[len][dstDim] = alpha * (*alphaPtr) * src * W^T, src and W 8-bit of the same type, resType TS2_F32 | TS2_BF16. */
+int ts2_matmul_forward(int32_t mode, int32_t len, int32_t lenRound, int32_t srcDim, int32_t dstDim, const ts2_mat *src,
+    const ts2_mat *transformFast, float alpha, const float *alphaPtr, const ts2_mat *res, int32_t resType, int32_t add, void *stream);
+
 /* peak dense MFMA rate the library prices its kernels against, in T(FL)OP/s, and the CU count it tiles for */
 int ts2_device_info(int *cuCount, int *clockMHz);
 const char *ts2_version(void);

@@ -1,0 +1,146 @@
+"""Linear-layer backward (dX = dY*W, delta = dY^T*X) on the GPU against the oracle's fp32 CPU path (MulBackwardWithAccum,
+SumRankOne).  The GPU path quantises dY to int8 (per row for dX, per k-tile for the delta) or takes e4m3 operands, so agreement is
+bounded by the quantisation step: max |err| <= 1e-2 * max |ref| (the stated tolerance for 8-bit gradients); int32 partial sums are
+checked bit-exactly in test_gemm_gpu.py."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+from oracle_lib import Oracle, _ptr  # noqa: E402
+
+
+@pytest.fixture(scope="module")
+def L():
+    from tscale2_amd import lib
+    lib.load()
+    return lib
+
+
+@pytest.fixture(scope="module")
+def orc():
+    return Oracle()
+
+
+def make_case(orc, seed, len_, src_dim, grad_dim, fp8):
+    r = np.random.default_rng(seed)
+    w = (r.standard_normal((grad_dim, src_dim)) * 0.02).astype(np.float32)
+    if fp8:
+        fast = np.zeros((grad_dim, src_dim), np.uint8)
+        sko = orc.lib.orc_quantize_matrix_e4m3(_ptr(w), _ptr(fast), grad_dim, src_dim)
+        wq = orc.e4m3_table()[fast] * np.float32(sko / 32)
+    else:
+        fast = np.zeros((grad_dim, src_dim), np.int8)
+        sko = orc.lib.orc_quantize_matrix_i8(_ptr(w), _ptr(fast), grad_dim, src_dim)
+        wq = fast.astype(np.float32) * np.float32(sko / 32)
+    # layer input: unit-rms tiles stored as 8-bit in 1/24 units (the reference's NormState format)
+    x = orc.normalize_state(r.standard_normal((len_, src_dim)).astype(np.float32), src_dim // 128)
+    dy = (r.standard_normal((len_, grad_dim)) * (0.2 + r.random((len_, 1)))).astype(np.float32)
+    return w, fast, float(sko), wq, x, dy
+
+
+@pytest.mark.parametrize("len_,src_dim,grad_dim", [(500, 256, 384), (1024, 512, 256)])
+def test_int8_linear_backward(L, orc, len_, src_dim, grad_dim):
+    print(f"case linear i8 {len_} {src_dim} {grad_dim}", flush=True)
+    len_round = (len_ + 511) // 512 * 512
+    w, fast, sko, wq, x, dy = make_case(orc, 11, len_, src_dim, grad_dim, False)
+    x8 = orc.convert_i8(x, 24.0)
+    xq = x8.astype(np.float32) / 24
+    # oracle on exactly the operands the device sees (dequantised weights and inputs, bf16 gradient)
+    dy16 = torch.from_numpy(dy).bfloat16()
+    dyf = dy16.float().numpy()
+    ref_dx = orc.mul_backward_accum(np.zeros((len_, src_dim), np.float32), wq, dyf)
+    ref_delta = orc.sum_rank_one(xq, dyf)
+
+    bufs = L.MatMulBuffers(L.I8, len_round, src_dim, grad_dim, k_tile=256)
+    x8d = torch.zeros((len_round, src_dim), dtype=torch.int8, device="cuda")
+    x8d[:len_] = torch.from_numpy(x8).cuda()
+    dyd = dy16.cuda()
+    wscale = torch.tensor([sko], device="cuda")
+    dx = torch.full((len_round, src_dim), 9.0, device="cuda")
+    bufs.backprop_multi(len_, torch.from_numpy(fast).cuda(), dyd.view(torch.int16), L.BF16)
+    bufs.backprop(len_, None, (1 / 32) / np.sqrt(src_dim), wscale, dx, L.F32)
+    bufs.backprop_delta(len_, x8d, None, dyd.view(torch.int16), L.BF16)
+    torch.cuda.synchronize()
+    got_dx = dx.cpu().numpy()
+    assert np.all(got_dx[len_:] == 0)
+
+    # (1) same contract on the CPU: identical quantisation, exact int32 sums -> agreement to the last bit of the int8 operands and
+    #     an fp32 epilogue that may differ by rounding order only
+    q8 = np.zeros((len_, grad_dim), np.int8); rsc = np.zeros(len_, np.float32)
+    orc.lib.orc_quant_rowmax_i8(_ptr(dyf), _ptr(q8), _ptr(rsc), len_, grad_dim)
+    np.testing.assert_array_equal(bufs.t["grad8"].cpu().numpy()[:len_], q8)
+    np.testing.assert_array_equal(bufs.t["grad8RowScale"].cpu().numpy()[:len_], rsc)
+    np.testing.assert_array_equal(bufs.t["transformT"].cpu().numpy(), fast.T)
+    same_dx = np.zeros((len_, src_dim), np.float32)
+    import ctypes as C
+    orc.lib.orc_gemm_i8_nt_rowscale(_ptr(q8), _ptr(rsc), _ptr(np.ascontiguousarray(fast.T)), C.c_float(np.float32((1 / 32) / np.sqrt(src_dim)) * np.float32(sko)),
+                                    _ptr(same_dx), len_, src_dim, grad_dim, 0)
+    np.testing.assert_allclose(got_dx[:len_], same_dx, rtol=2e-6, atol=1e-9)
+    kt = 256
+    qk = np.zeros((len_round, grad_dim), np.int8); tsc = np.zeros(len_round // kt, np.float32)
+    dypad = np.zeros((len_round, grad_dim), np.float32); dypad[:len_] = dyf
+    orc.lib.orc_quant_ktile_i8(_ptr(dypad), _ptr(qk), _ptr(tsc), len_round, grad_dim, kt)
+    np.testing.assert_array_equal(bufs.t["gradT"].cpu().numpy(), qk.T)
+    x8pad = np.zeros((len_round, src_dim), np.int8); x8pad[:len_] = x8
+    np.testing.assert_array_equal(bufs.t["srcT"].cpu().numpy(), x8pad.T)
+    acc = np.zeros((grad_dim, src_dim), np.float32)
+    orc.lib.orc_gemm_i8_nt_ktile(_ptr(np.ascontiguousarray(qk.T)), _ptr(np.ascontiguousarray(x8pad.T)), _ptr(tsc), kt, C.c_float(1.0), _ptr(acc),
+                                 grad_dim, src_dim, len_round)
+    want_delta = np.zeros((grad_dim, src_dim), np.int8); want_ts = np.zeros((src_dim // 128, grad_dim), np.float32)
+    orc.lib.orc_compress_delta(_ptr(acc), _ptr(want_delta), _ptr(want_ts), grad_dim, src_dim)
+    np.testing.assert_allclose(bufs.delta_tile_scale.cpu().numpy(), want_ts, rtol=2e-6)
+    dd = np.abs(bufs.delta.cpu().numpy().astype(np.int32) - want_delta)
+    assert dd.max() <= 1 and (dd != 0).mean() < 1e-3
+
+    # (2) against the reference's fp32 CPU path: bounded by the int8 quantisation step of dY (per row: 1/254 of the row maximum per
+    #     element for dX; per k-tile for the delta, plus 1/254 of the row-tile maximum for the packed output)
+    def errs(got, ref):
+        d = got - ref
+        return np.sqrt((d ** 2).mean()) / np.sqrt((ref ** 2).mean()), np.abs(d).max() / np.abs(ref).max()
+    rms, mx = errs(got_dx[:len_], ref_dx)
+    print("dX rel err rms/max", rms, mx)
+    assert rms <= 1e-2 and mx <= 3e-2
+    got_delta = bufs.delta_fp32().cpu().numpy() / 24  # X was stored in 1/24 units
+    rms, mx = errs(got_delta, ref_delta)
+    print("delta rel err rms/max", rms, mx)
+    assert rms <= 2e-2 and mx <= 3e-2
+    # adding a second source accumulates
+    bufs.backprop(len_, None, (1 / 32) / np.sqrt(src_dim), wscale, dx, L.F32, add=True)
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(dx.cpu().numpy(), 2 * got_dx, rtol=1e-6)
+
+
+def test_fp8_linear_backward(L, orc):
+    print("case linear fp8", flush=True)
+    len_, src_dim, grad_dim = 900, 256, 512
+    len_round = 1024
+    w, fast, sko, wq, x, dy = make_case(orc, 12, len_, src_dim, grad_dim, True)
+    tab = orc.e4m3_table(hw=True)
+    xe = np.array([orc.lib.orc_cvt_e4m3_rne(__import__("ctypes").c_float(v)) for v in (x * 24).ravel()], np.uint8).reshape(x.shape)
+    xq = tab[xe] / 24
+    # fast gradient: fp32 gradient times the power-of-two multiplier, stored as e4m3
+    mult = orc.lib.orc_grad_mult(__import__("ctypes").c_float(float(np.abs(dy).max())))
+    dye = np.array([orc.lib.orc_cvt_e4m3_rne(__import__("ctypes").c_float(v)) for v in (dy * mult).ravel()], np.uint8).reshape(dy.shape)
+    dyq = tab[dye] / np.float32(mult)
+    ref_dx = orc.mul_backward_accum(np.zeros((len_, src_dim), np.float32), wq, dyq)
+    ref_delta = orc.sum_rank_one(xq, dyq)
+
+    bufs = L.MatMulBuffers(L.E4M3, len_round, src_dim, grad_dim)
+    xd = torch.zeros((len_round, src_dim), dtype=torch.uint8, device="cuda"); xd[:len_] = torch.from_numpy(xe).cuda()
+    dyd = torch.zeros((len_round, grad_dim), dtype=torch.uint8, device="cuda"); dyd[:len_] = torch.from_numpy(dye).cuda()
+    gscale = torch.tensor([1 / mult], device="cuda")
+    dx = torch.zeros((len_round, src_dim), device="cuda")
+    bufs.backprop_multi(len_, torch.from_numpy(fast).cuda(), None, L.E4M3)
+    bufs.backprop(len_, dyd, (1 / 32) / np.sqrt(src_dim) * sko, gscale, dx, L.F32)
+    bufs.backprop_delta(len_, xd, None, dyd, L.E4M3, gscale)
+    torch.cuda.synchronize()
+    # operands are identical on both sides; only fp32 accumulation differs -> 1e-4 (MFMA fp8 adder-tree precision)
+    err = np.abs(dx.cpu().numpy()[:len_] - ref_dx).max() / np.abs(ref_dx).max()
+    print("fp8 dX rel err", err)
+    assert err <= 1e-4
+    # the packed delta adds its own int8 rounding: 1/254 of each row-tile maximum
+    got_delta = bufs.delta_fp32().cpu().numpy() / 24
+    err = np.abs(got_delta - ref_delta).max() / np.abs(ref_delta).max()
+    print("fp8 delta rel err", err)
+    assert err <= 5e-3

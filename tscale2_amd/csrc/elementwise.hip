@@ -314,9 +314,9 @@ __global__ void __launch_bounds__(256) TransposeQuant(int len, int lenRound, Mat
                 if (QUANT) {
                     F4 v = Load4<TSrc>(At<TSrc>(src, srcRow, xBlock + h * 4));
                     float tm = tileMax[t / kTile];
-                    float mult = tm > 0 ? 127.f / tm : 0.f;
+                    float mult = tm > 0 ? 1 / (tm / 127) : 0.f; // same two roundings as scale = max/127, mult = 1/scale
                     if (rowMult) {
-                        mult *= rowMult[srcRow];
+                        v = v * rowMult[srcRow];
                     }
                     v = v * mult;
                     packed = (uint32_t)(CvtToI8(v.x) & 0xff) | ((uint32_t)(CvtToI8(v.y) & 0xff) << 8) | ((uint32_t)(CvtToI8(v.z) & 0xff) << 16) |

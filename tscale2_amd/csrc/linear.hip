@@ -1,0 +1,148 @@
+// Linear-layer backward operator: the call sequences of TMatMulBuffers (src/gpt/compute/layer_cuda_base.cuh:153-250) expressed
+// over the kernels of this library.  Host code only; every step is enqueued on the caller's stream.
+#include "common.h"
+
+namespace
+{
+bool Is8(int mode)
+{
+    return mode == TS2_I8 || mode == TS2_E4M3;
+}
+} // namespace
+
+extern "C" int ts2_matmul_backprop_multi(int32_t mode, int32_t len, int32_t lenRound, int32_t srcDim, int32_t gradDim,
+    const ts2_mat *transformFast, const ts2_mat *grad, int32_t gradType, const float *gradColScale, const ts2_matmul_bwd_buffers *buf, void *stream)
+{
+    if (!transformFast || !buf) {
+        return TS2_ERR_NULL;
+    }
+    if (!Is8(mode)) {
+        return TS2_ERR_UNSUPPORTED;
+    }
+    if (srcDim % 128 || gradDim % 128 || lenRound % 128 || len > lenRound) {
+        return TS2_ERR_SHAPE;
+    }
+    if (mode == TS2_I8) {
+        if (!grad || !buf->grad8RowScale) {
+            return TS2_ERR_NULL;
+        }
+        int rc = ts2_normalize_vecs_row_max(len, lenRound, grad, gradType, gradColScale, &buf->grad8, buf->grad8RowScale, stream);
+        if (rc) {
+            return rc;
+        }
+    }
+    // W [gradDim][srcDim] -> W^T [srcDim][gradDim] so that the dX GEMM contracts over contiguous bytes
+    return ts2_transpose_quant(gradDim, gradDim, transformFast, mode, nullptr, nullptr, 0, nullptr, &buf->transformT, mode, nullptr, stream);
+}
+
+extern "C" int ts2_matmul_backprop(int32_t mode, int32_t len, int32_t lenRound, int32_t srcDim, int32_t gradDim, const ts2_mat *grad,
+    const ts2_matmul_bwd_buffers *buf, float alpha, const float *alphaPtr, const ts2_mat *srcGrad, int32_t srcGradType, int32_t add, void *stream)
+{
+    if (!buf || !srcGrad) {
+        return TS2_ERR_NULL;
+    }
+    if (!Is8(mode)) {
+        return TS2_ERR_UNSUPPORTED;
+    }
+    ts2_gemm_args g = {};
+    if (mode == TS2_I8) {
+        g.a = buf->grad8;
+        g.rowScale = buf->grad8RowScale;
+    } else {
+        if (!grad) {
+            return TS2_ERR_NULL;
+        }
+        g.a = *grad;
+    }
+    g.b = buf->transformT;
+    g.c = *srcGrad;
+    g.abType = mode;
+    g.cType = srcGradType;
+    g.m = lenRound;
+    g.n = srcDim;
+    g.k = gradDim;
+    g.mLive = len;
+    g.alpha = alpha;
+    g.alphaPtr = alphaPtr;
+    g.epilogue = add ? TS2_EPI_ADD : TS2_EPI_STORE;
+    g.splitK = 1;
+    return ts2_gemm_nt(&g, stream);
+}
+
+extern "C" int ts2_matmul_backprop_delta(int32_t mode, int32_t len, int32_t lenRound, int32_t srcDim, int32_t gradDim, const ts2_mat *src,
+    const float *srcRowScale, const ts2_mat *grad, int32_t gradType, const float *gradScale, int32_t kTile, const ts2_matmul_bwd_buffers *buf,
+    const ts2_mat *delta, const ts2_mat *deltaTileScale, void *stream)
+{
+    if (!buf || !src || !grad || !delta || !deltaTileScale) {
+        return TS2_ERR_NULL;
+    }
+    if (!Is8(mode)) {
+        return TS2_ERR_UNSUPPORTED;
+    }
+    int rc;
+    ts2_gemm_args g = {};
+    if (mode == TS2_I8) {
+        if (kTile <= 0 || kTile % 128 || lenRound % kTile || !buf->tileMax || !buf->tileScale) {
+            return TS2_ERR_SHAPE;
+        }
+        rc = ts2_tile_absmax(len, grad, gradType, srcRowScale, kTile, buf->tileMax, 1, stream);
+        if (rc) {
+            return rc;
+        }
+        rc = ts2_transpose_quant(len, lenRound, grad, gradType, srcRowScale, buf->tileMax, kTile, nullptr, &buf->gradT, TS2_I8, buf->tileScale, stream);
+        if (rc) {
+            return rc;
+        }
+        g.kTileScale = buf->tileScale;
+        g.kTile = kTile;
+    } else {
+        if (gradType != TS2_E4M3) {
+            return TS2_ERR_UNSUPPORTED;
+        }
+        rc = ts2_transpose_quant(len, lenRound, grad, TS2_E4M3, nullptr, nullptr, 0, nullptr, &buf->gradT, TS2_E4M3, nullptr, stream);
+        if (rc) {
+            return rc;
+        }
+    }
+    rc = ts2_transpose_quant(len, lenRound, src, mode, nullptr, nullptr, 0, nullptr, &buf->srcT, mode, nullptr, stream);
+    if (rc) {
+        return rc;
+    }
+    g.a = buf->gradT;
+    g.b = buf->srcT;
+    g.c = *delta;
+    g.abType = mode;
+    g.cType = TS2_I8;
+    g.m = gradDim;
+    g.n = srcDim;
+    g.k = lenRound;
+    g.alpha = 1;
+    g.alphaPtr = gradScale;
+    g.epilogue = TS2_EPI_ROW_TILE_MAXNORM;
+    g.tileScale = *deltaTileScale;
+    g.splitK = 1;
+    return ts2_gemm_nt(&g, stream);
+}
+
+extern "C" int ts2_matmul_forward(int32_t mode, int32_t len, int32_t lenRound, int32_t srcDim, int32_t dstDim, const ts2_mat *src,
+    const ts2_mat *transformFast, float alpha, const float *alphaPtr, const ts2_mat *res, int32_t resType, int32_t add, void *stream)
+{
+    if (!src || !transformFast || !res) {
+        return TS2_ERR_NULL;
+    }
+    ts2_gemm_args g = {};
+    g.a = *src;
+    g.b = *transformFast;
+    g.c = *res;
+    g.abType = mode;
+    g.cType = resType;
+    g.m = lenRound;
+    g.n = dstDim;
+    g.k = srcDim;
+    g.mLive = len;
+    g.alpha = alpha;
+    g.alphaPtr = alphaPtr;
+    g.epilogue = add ? TS2_EPI_ADD : TS2_EPI_STORE;
+    g.splitK = 1;
+    return ts2_gemm_nt(&g, stream);
+}

@@ -114,3 +114,51 @@ def call(name, *args, check=True):
     if check and rc != 0:
         raise RuntimeError(f"{name} failed with code {rc}")
     return rc
+
+
+class BwdBuffers(C.Structure):
+    _fields_ = [("grad8", Mat), ("grad8RowScale", C.c_void_p), ("gradT", Mat), ("srcT", Mat), ("tileMax", C.c_void_p), ("tileScale", C.c_void_p),
+                ("transformT", Mat)]
+
+
+class MatMulBuffers:
+    """Scratch of one linear layer's backward, allocated with torch (the reference allocates the same members from its pools,
+    src/gpt/compute/matmul_fwdbwd.cuh:283-311).  mode: I8 or E4M3."""
+
+    def __init__(self, mode, len_round, src_dim, grad_dim, k_tile=512):
+        import torch
+        self.mode, self.len_round, self.src_dim, self.grad_dim, self.k_tile = mode, len_round, src_dim, grad_dim, k_tile
+        bt = torch.int8 if mode == I8 else torch.uint8
+        dev = "cuda"
+        self.t = {}
+        if mode == I8:
+            self.t["grad8"] = torch.empty((len_round, grad_dim), dtype=torch.int8, device=dev)
+            self.t["grad8RowScale"] = torch.empty(len_round, dtype=torch.float32, device=dev)
+            n_tiles = len_round // k_tile
+            self.t["tileMax"] = torch.empty(n_tiles, dtype=torch.float32, device=dev)
+            self.t["tileScale"] = torch.empty(n_tiles, dtype=torch.float32, device=dev)
+        self.t["gradT"] = torch.empty((grad_dim, len_round), dtype=bt, device=dev)
+        self.t["srcT"] = torch.empty((src_dim, len_round), dtype=bt, device=dev)
+        self.t["transformT"] = torch.empty((src_dim, grad_dim), dtype=bt, device=dev)
+        self.c = BwdBuffers()
+        for k, v in self.t.items():
+            setattr(self.c, k, mat(v) if v.dim() == 2 else v.data_ptr())
+        self.delta = torch.empty((grad_dim, src_dim), dtype=torch.int8, device=dev)
+        self.delta_tile_scale = torch.empty((src_dim // 128, grad_dim), dtype=torch.float32, device=dev)
+
+    def backprop_multi(self, len_, transform_fast, grad, grad_type, grad_col_scale=None):
+        call("ts2_matmul_backprop_multi", self.mode, len_, self.len_round, self.src_dim, self.grad_dim, transform_fast, grad, grad_type,
+             grad_col_scale, C.byref(self.c))
+
+    def backprop(self, len_, grad, alpha, alpha_ptr, src_grad, src_grad_type, add=False):
+        call("ts2_matmul_backprop", self.mode, len_, self.len_round, self.src_dim, self.grad_dim, grad, C.byref(self.c), float(alpha), alpha_ptr,
+             src_grad, src_grad_type, int(add))
+
+    def backprop_delta(self, len_, src, src_row_scale, grad, grad_type, grad_scale=None):
+        call("ts2_matmul_backprop_delta", self.mode, len_, self.len_round, self.src_dim, self.grad_dim, src, src_row_scale, grad, grad_type,
+             grad_scale, self.k_tile, C.byref(self.c), self.delta, self.delta_tile_scale)
+
+    def delta_fp32(self):
+        """dequantised packed delta [gradDim][srcDim]"""
+        sc = self.delta_tile_scale.t().repeat_interleave(128, dim=1)
+        return self.delta.float() * sc
