@@ -196,6 +196,62 @@ int ts2_matmul_backprop_delta(int32_t mode, int32_t len, int32_t lenRound, int32
 int ts2_matmul_forward(int32_t mode, int32_t len, int32_t lenRound, int32_t srcDim, int32_t dstDim, const ts2_mat *src,
     const ts2_mat *transformFast, float alpha, const float *alphaPtr, const ts2_mat *res, int32_t resType, int32_t add, void *stream);
 
+/* ------------------------------------------------------------------------------------------------------------------------
+ * Attention (head dimension 128 = Q_DIM = TT_DIM, src/gpt/compute/cfg_precision.h:79-80).  q, k, v, valLookup, dValLookup are
+ * TS2_BF16 [lenRound][heads*128]; q and k already rotated (RoPE) and q, v head-normalised, as the reference stores them
+ * (src/gpt/compute/layer_att.cu:108-143).  Spans: query row t attends key rows spanStart[t] .. spanFinish[t] inclusive
+ * (finish < start = nothing); both arrays have lenRound entries and pad rows must be empty.  This covers every causal attention
+ * type of src/gpt/att/sliding_window.cpp:111-118,226-240 (one span per row); the reference's general span groups
+ * (TAttentionSpanGroup, src/gpt/att/att.h:86-121) are only needed by its cross-batch attention, which is out of scope.
+ * logit = <q,k> * attDotScale - alibiSlope * (query row - key row); softmax base 2 with the implicit zero "sink" vector.
+ * Stats: sumWeightLog fp32 [heads][lenRound] = max + log2(sum), dScale fp32 [heads][lenRound] (same stride).
+ * Rows >= len of q/k/v/dValLookup must be finite (producers write zeros). */
+typedef struct ts2_att_args {
+    int32_t len, lenRound, heads;
+    ts2_mat q, k, v;
+    const int32_t *spanStart, *spanFinish;
+    float attDotScale, alibiSlope;
+    ts2_mat valLookup;    /* out */
+    ts2_mat sumWeightLog; /* out */
+} ts2_att_args;
+
+/* Fp16Att, src/gpt/compute/gpu_att_fp16.cu:41-215 */
+int ts2_att_forward(const ts2_att_args *args, void *stream);
+
+typedef struct ts2_att_grad_args {
+    int32_t len, lenRound, heads;
+    ts2_mat q, k, v, dValLookup;
+    const int32_t *spanStart, *spanFinish;
+    const int32_t *revLo, *revHi; /* [lenRound/128] from ts2_att_build_rev */
+    float attDotScale, alibiSlope;
+    ts2_mat sumWeightLog, dScale; /* in */
+    ts2_mat dQ, dK, dV;           /* out, gradType = TS2_BF16 | TS2_F32 */
+    int32_t gradType;
+    int32_t which; /* bit 0: dQ (Fp16AttGradQ), bit 1: dK and dV (Fp16AttGradKV) */
+} ts2_att_grad_args;
+
+/* Fp16AttGradQ + Fp16AttGradKV, src/gpt/compute/gpu_att_fp16.cuh:60-358 (their norm/rope epilogues are
+ * ts2_backprop_row_tile_normalize_rope below) */
+int ts2_att_backward(const ts2_att_grad_args *args, void *stream);
+
+/* Transposed span graph reduced to what the dK/dV kernel needs: per block of 128 key rows the first and last query row whose
+ * span touches it (replaces TransposeAttention + GroupAttention on the host, src/gpt/att/att.cpp:25-55, att.h:125-211). */
+int ts2_att_build_rev(int32_t len, int32_t lenRound, const int32_t *spanStart, const int32_t *spanFinish, int32_t *revLo, int32_t *revHi,
+    void *stream);
+
+/* TStoreRowTileNormalize / TStoreRowTileNormalizeRope as a stand-alone pass (src/lib/cuda/cuda_matmul.cuh:495-525,
+ * src/gpt/compute/gpu_rope.cuh:25-60): per row and 128-wide head: v = src*srcMult; if normalize: scale = rms(v)*vecScale
+ * (stored in tileScale[head][row], 0 for zero tiles) and v /= scale; if ropeBuf (fp32 [lenRound][128] = cos,sin pairs of
+ * src/gpt/att/rope.cpp:14-22): rotate pairs by +1; store as TS2_BF16; rows in [len, lenRound) are cleared. */
+int ts2_row_tile_normalize_rope(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, float srcMult, int32_t normalize,
+    float vecScale, const ts2_mat *ropeBuf, const ts2_mat *dst, const ts2_mat *tileScale, void *stream);
+
+/* TStoreAttBackNormalizeRope / TStoreAttBackNormalize / TStoreAttBackRope, src/gpt/compute/gpu_att_utils.cuh:280-352: per row
+ * and head: g = grad*gradMult; if srcNorm: tile-norm backward against srcNorm*srcTileScale (the stored normalised, rotated
+ * vector); if ropeBuf: rotate pairs by -1; store as dstType (TS2_BF16 | TS2_E4M3 | TS2_F32); rows in [len, lenRound) cleared. */
+int ts2_backprop_row_tile_normalize_rope(int32_t len, int32_t lenRound, const ts2_mat *grad, int32_t gradType, float gradMult,
+    const ts2_mat *srcNorm, const ts2_mat *srcTileScale, const ts2_mat *ropeBuf, const ts2_mat *dst, int32_t dstType, void *stream);
+
 /* peak dense MFMA rate the library prices its kernels against, in T(FL)OP/s, and the CU count it tiles for */
 int ts2_device_info(int *cuCount, int *clockMHz);
 const char *ts2_version(void);

@@ -1,0 +1,132 @@
+"""Attention forward / backward on the GPU against the oracle (the reference's TAttentionComputer restated).
+Inputs are bf16-representable so both sides see identical operands; the device rounds probabilities and score gradients to bf16
+before the second product of each pair (fp32 accumulate), hence the tolerance: max |err| <= 1e-2 * max |ref| per tensor."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+from golden_cases import causal_spans  # noqa: E402
+from oracle_lib import Oracle  # noqa: E402
+
+
+@pytest.fixture(scope="module")
+def L():
+    from tscale2_amd import lib
+    lib.load()
+    return lib
+
+
+@pytest.fixture(scope="module")
+def orc():
+    return Oracle()
+
+
+def bf16_round(a):
+    return torch.from_numpy(a).bfloat16().float().numpy()
+
+
+def spans_to_ranges(sp, spans, n, n_round):
+    start = np.zeros(n_round, np.int32)
+    finish = np.full(n_round, -1, np.int32)
+    for t in range(n):
+        assert sp[t + 1] - sp[t] <= 1
+        if sp[t + 1] > sp[t]:
+            start[t], finish[t] = spans[sp[t]]
+    return start, finish
+
+
+def run_case(L, orc, frag_count, frag_len, window, heads, slope, seed, grad_type):
+    n = frag_count * frag_len
+    n_round = (n + 127) // 128 * 128
+    sp, spans = causal_spans(frag_count, frag_len, window)
+    r = np.random.default_rng(seed)
+    # q, v are unit-rms heads and k ~ N(0,1) in the model; scaled so that logits have a realistic spread
+    q = bf16_round(r.standard_normal((n, heads * 128)).astype(np.float32))
+    k = bf16_round(r.standard_normal((n, heads * 128)).astype(np.float32))
+    v = bf16_round(r.standard_normal((n, heads * 128)).astype(np.float32))
+    dval = bf16_round(r.standard_normal((n, heads * 128)).astype(np.float32))
+    ref = orc.attention(heads, 128, 128, slope, sp, spans, q, k, v, dval)
+    att_dot_scale = float(np.float32(np.sqrt(np.float32(1.0 / 128))) * np.float32(0.5 / 0.693147))
+
+    def padded(a):
+        t = torch.zeros((n_round, a.shape[1]), dtype=torch.bfloat16, device="cuda")
+        t[:n] = torch.from_numpy(a).cuda().bfloat16()
+        return t
+    tq, tk, tv, tdv = padded(q), padded(k), padded(v), padded(dval)
+    start, finish = spans_to_ranges(sp, spans, n, n_round)
+    ts, tf = torch.from_numpy(start).cuda(), torch.from_numpy(finish).cuda()
+    val = torch.full((n_round, heads * 128), 7.0, dtype=torch.bfloat16, device="cuda")
+    swl = torch.full((heads, n_round), -5.0, device="cuda")
+    i16 = torch.int16
+    L.att_forward(n, heads, tq.view(i16), tk.view(i16), tv.view(i16), ts, tf, att_dot_scale, slope, val.view(i16), swl)
+    torch.cuda.synchronize()
+    got_val = val.float().cpu().numpy()[:n]
+    err = np.abs(got_val - ref["val"]).max() / np.abs(ref["val"]).max()
+    print("valLookup rel err", err)
+    assert err <= 1e-2
+    want_l = ref["max_dp"] + np.log2(ref["sum_weight"])
+    np.testing.assert_allclose(swl.cpu().numpy()[:, :n], want_l, rtol=1e-4, atol=1e-4)
+    assert np.all(val.float().cpu().numpy()[n:] == 0) and np.all(swl.cpu().numpy()[:, n:] == 0)
+
+    # backward uses the forward's statistics and the oracle's dScale (the device computes dScale in the gate kernel)
+    ds = torch.zeros((heads, n_round), device="cuda")
+    ds[:, :n] = torch.from_numpy(ref["dscale"]).cuda()
+    rev_lo = torch.zeros(n_round // 128, dtype=torch.int32, device="cuda")
+    rev_hi = torch.zeros(n_round // 128, dtype=torch.int32, device="cuda")
+    L.call("ts2_att_build_rev", n, n_round, ts, tf, rev_lo, rev_hi)
+    tdt = torch.float32 if grad_type == L.F32 else torch.bfloat16
+    dq = torch.full((n_round, heads * 128), 3.0, dtype=tdt, device="cuda")
+    dk = torch.full((n_round, heads * 128), 3.0, dtype=tdt, device="cuda")
+    dv = torch.full((n_round, heads * 128), 3.0, dtype=tdt, device="cuda")
+    vw = (lambda t: t) if grad_type == L.F32 else (lambda t: t.view(i16))
+    L.att_backward(n, heads, tq.view(i16), tk.view(i16), tv.view(i16), tdv.view(i16), ts, tf, rev_lo, rev_hi, att_dot_scale, slope, swl, ds,
+                   vw(dq), vw(dk), vw(dv), grad_type)
+    torch.cuda.synchronize()
+    for name, got in (("dq", dq), ("dk", dk), ("dv", dv)):
+        g = got.float().cpu().numpy()
+        err = np.abs(g[:n] - ref[name]).max() / np.abs(ref[name]).max()
+        print(name, "rel err", err)
+        assert err <= 1e-2, name
+        assert np.all(g[n:] == 0), name
+
+
+def test_attention_window_and_slope(L, orc):
+    print("case att window", flush=True)
+    run_case(L, orc, frag_count=3, frag_len=100, window=64, heads=2, slope=0.5, seed=21, grad_type=L.F32)
+
+
+def test_attention_full_causal_bf16_grads(L, orc):
+    print("case att full causal", flush=True)
+    run_case(L, orc, frag_count=2, frag_len=320, window=1024, heads=1, slope=0.0, seed=22, grad_type=L.BF16)
+
+
+def test_attention_window_one(L, orc):
+    print("case att window 1", flush=True)
+    run_case(L, orc, frag_count=2, frag_len=70, window=1, heads=1, slope=0.0, seed=23, grad_type=L.F32)
+
+
+def test_rope_and_head_norm_passes(L, orc):
+    print("case rope/norm passes", flush=True)
+    r = np.random.default_rng(24)
+    n, n_round, heads = 150, 256, 2
+    src = r.standard_normal((n, heads * 128)).astype(np.float32) * 0.3
+    rope = orc.fill_rope_buf(128, n_round)
+    want = orc.apply_rope(rope, 1.0, orc.normalize_state(src, heads))
+    dst = torch.full((n_round, heads * 128), 5.0, dtype=torch.bfloat16, device="cuda")
+    sc = torch.full((heads, n_round), -1.0, device="cuda")
+    tr = torch.from_numpy(rope).cuda()
+    L.call("ts2_row_tile_normalize_rope", n, n_round, torch.from_numpy(src).cuda(), L.F32, 1.0, 1, 1.0, tr, dst.view(torch.int16), sc)
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(dst.float().cpu().numpy()[:n], want, rtol=2 ** -8, atol=2e-3)
+    assert np.all(dst.float().cpu().numpy()[n:] == 0)
+    rms = np.sqrt((src.reshape(n, heads, 128).astype(np.float64) ** 2).mean(-1))
+    np.testing.assert_allclose(sc.cpu().numpy()[:, :n].T, rms, rtol=1e-5)
+    # backward: oracle order = inverse rope, then norm backward against the un-rotated source
+    g = r.standard_normal((n, heads * 128)).astype(np.float32)
+    want_g = orc.normalize_state_backward(src, orc.apply_rope(rope, -1.0, g), heads)
+    out = torch.zeros((n_round, heads * 128), device="cuda")
+    L.call("ts2_backprop_row_tile_normalize_rope", n, n_round, torch.from_numpy(g).cuda(), L.F32, 1.0, dst.view(torch.int16), sc, tr, out, L.F32)
+    torch.cuda.synchronize()
+    # the stored normalised vector is bf16: 2^-8 relative on the source enters the projection
+    assert np.abs(out.cpu().numpy()[:n] - want_g).max() <= 1e-2 * np.abs(want_g).max()

@@ -1,0 +1,580 @@
+// Base-2 "sink" attention of the reference (forward, dQ, dK/dV) on gfx950 bf16 MFMA, head dimension 128.
+//
+// Math (src/gpt/compute/layer_att_reference.h:47-211): for query row q and every key row t of its span [start[q], finish[q]]
+//   dp = <q,k_t> * attDotScale - slope * (q - t);  m = max(0, max dp);  S = 2^-m + sum_t 2^(dp-m)   (a zero vector of weight 1)
+//   out = sum_t w_t v_t,  w_t = 2^(dp-m)/S;  stats L = m + log2 S  (SumWeightLog of src/gpt/compute/gpu_att_fp16.cu:192-205)
+//   dDot = w_t (<dO_q, v_t> - dScale_q) attDotScale ln2;  dq += dDot k_t;  dk_t += dDot q;  dv_t += w_t dO_q
+//
+// Design for CDNA4 (replaces Fp16Att / Fp16AttGradQ / Fp16AttGradKV, src/gpt/compute/gpu_att_fp16.cuh:60-358, whose 16-key
+// mma.sync tiling does not map to MFMA):
+//   * a workgroup = 4 waves x 32 rows = 128 query rows (forward, dQ) or 128 key rows (dK/dV); the other side streams through LDS
+//     in 64-row tiles.  Every product is a v_mfma_f32_32x32x16_bf16 whose N index (the lane) is the wave's own row, so all
+//     softmax statistics are per lane and the running rescale of the accumulators needs no cross-lane traffic:
+//         S^T = K Q^T,  O^T += V^T P^T,  dP^T = V dO^T,  dQ^T += K^T dS^T      (lane = query)
+//         S = Q K^T,  dP = dO V^T,  dV^T += dO^T P,  dK^T += Q^T dS             (lane = key)
+//     The probability / score-gradient tiles never leave registers: an MFMA result register block is fed back as the B operand of
+//     the next product (the contraction index order of an MFMA is free as long as A and B agree).
+//   * products that contract over token rows need the streamed tile with rows along the contraction: each tile is written to LDS
+//     row-major with coalesced 16-byte loads and then re-written transposed (two rows packed per dword with v_perm_b32, padded
+//     pitches chosen so the 8-byte operand reads are bank-conflict free).
+//   * spans are one inclusive key range per query (every causal window / document-start pattern of
+//     src/gpt/att/sliding_window.cpp:111-118,226-240); masking is evaluated per element from those ranges, tiles outside the
+//     workgroup's range are never loaded.
+#include "common.h"
+
+namespace
+{
+constexpr int HD = 128;          // Q_DIM = TT_DIM (src/gpt/compute/cfg_precision.h:79-80)
+constexpr int WROWS = 32;        // rows owned by one wave
+constexpr int BROWS = 128;       // rows owned by one workgroup
+constexpr int TR = 64;           // rows of a streamed tile
+constexpr int RP = HD * 2 + 16;  // row-major tile pitch (bytes)
+constexpr int TP = TR * 2 + 8;   // transposed tile pitch (bytes): 34 dwords -> 8-byte reads of 32 consecutive d hit all 64 banks
+constexpr int RM_BYTES = TR * RP;
+constexpr int T_BYTES = HD * TP;
+constexpr float LN2 = 0.693147f; // LOG2 of src/gpt/model_params/model_dim.h:16
+
+struct AttP {
+    const uint8_t *q, *k, *v, *dO; // bf16 [lenRound][heads*128]
+    int64_t ldq, ldk, ldv, lddo;
+    const int *spanStart, *spanFinish;
+    const int *revLo, *revHi; // per 128-key block: range of query rows that reach it
+    float attDotScale, slope;
+    float *sumWeightLog; // [heads][ldStat]
+    const float *dScale;
+    int64_t ldStat;
+    uint8_t *out0, *out1; // forward: valLookup; dQ kernel: dQ; dK/dV kernel: dK, dV
+    int64_t ldo0, ldo1;
+    int lenRound;
+};
+
+// coalesced copy of a TR x 128 bf16 tile into a row-major LDS tile
+__device__ __forceinline__ void LoadTile(uint8_t *lds, const uint8_t *g, int64_t ld, int tid)
+{
+#pragma unroll
+    for (int i = 0; i < TR * 16 / 256; ++i) {
+        int id = tid + 256 * i;
+        int row = id >> 4, c = id & 15;
+        *(v4i *)(lds + row * RP + c * 16) = *(const v4i *)(g + (int64_t)row * ld + c * 16);
+    }
+}
+
+// row-major LDS tile -> transposed LDS tile T[d][row], two rows per dword
+__device__ __forceinline__ void TransposeTile(uint8_t *t, const uint8_t *rm, int tid)
+{
+    int r2 = tid & 31;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        int c = (tid >> 5) + 8 * i;
+        v4i a0 = *(const v4i *)(rm + (2 * r2) * RP + c * 16);
+        v4i a1 = *(const v4i *)(rm + (2 * r2 + 1) * RP + c * 16);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            uint32_t lo = __builtin_amdgcn_perm((uint32_t)a1[w], (uint32_t)a0[w], 0x05040100);
+            uint32_t hi = __builtin_amdgcn_perm((uint32_t)a1[w], (uint32_t)a0[w], 0x07060302);
+            *(uint32_t *)(t + (8 * c + 2 * w) * TP + 4 * r2) = lo;
+            *(uint32_t *)(t + (8 * c + 2 * w + 1) * TP + 4 * r2) = hi;
+        }
+    }
+}
+
+// A operand from a row-major tile: lane row = rb*32 + l32, 8 consecutive d at ds*16 + half*8
+__device__ __forceinline__ v8bf FragRM(const uint8_t *rm, int rb, int ds, int l32, int half)
+{
+    return __builtin_bit_cast(v8bf, *(const v4i *)(rm + (rb * 32 + l32) * RP + (ds * 16 + half * 8) * 2));
+}
+
+// A operand from a transposed tile: lane row = d = db*32 + l32; contraction slots = tile rows 16*ks + half*4 + {0..3} and +8
+__device__ __forceinline__ v8bf FragT(const uint8_t *t, int db, int ks, int l32, int half)
+{
+    const uint8_t *p = t + (db * 32 + l32) * TP + (16 * ks + half * 4) * 2;
+    uint2 lo = *(const uint2 *)p;
+    uint2 hi = *(const uint2 *)(p + 16);
+    v4i r = {(int)lo.x, (int)lo.y, (int)hi.x, (int)hi.y};
+    return __builtin_bit_cast(v8bf, r);
+}
+
+// B operand of the wave's own rows straight from global memory (loop invariant): lane row = l32
+__device__ __forceinline__ void LoadOwnFrags(v8bf *f, const uint8_t *g, int64_t ld, int l32, int half)
+{
+#pragma unroll
+    for (int ds = 0; ds < 8; ++ds) {
+        f[ds] = __builtin_bit_cast(v8bf, *(const v4i *)(g + (int64_t)l32 * ld + (ds * 16 + half * 8) * 2));
+    }
+}
+
+// result registers 8*s .. 8*s+7 of a 32x32 block -> bf16 B operand whose slots match FragT's row order
+__device__ __forceinline__ v8bf PackB(const float *x, int s)
+{
+    v4i r;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        r[w] = (int)PackBf16x2(x[8 * s + 2 * w], x[8 * s + 2 * w + 1]);
+    }
+    return __builtin_bit_cast(v8bf, r);
+}
+
+// row index inside a 32x32 MFMA result block held in register e by a lane of the given half
+__device__ __forceinline__ int BlkRow(int e, int half)
+{
+    return (e >> 2) * 8 + half * 4 + (e & 3);
+}
+
+template <bool F32> __device__ __forceinline__ void Store4Out(uint8_t *p, float a, float b, float c, float d)
+{
+    if (F32) {
+        *(float4 *)p = make_float4(a, b, c, d);
+    } else {
+        *(uint2 *)p = make_uint2(PackBf16x2(a, b), PackBf16x2(c, d));
+    }
+}
+
+// accumulators acc[db][e] hold X^T[d][own row]; write X[row][d]
+template <bool F32> __device__ __forceinline__ void StoreOwnRows(uint8_t *out, int64_t ld, int col0, v16f *acc, float mult, int l32, int half)
+{
+    constexpr int ES = F32 ? 4 : 2;
+#pragma unroll
+    for (int db = 0; db < 4; ++db) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            int d = db * 32 + g * 8 + half * 4;
+            Store4Out<F32>(out + (int64_t)l32 * ld + (int64_t)(col0 + d) * ES, acc[db][4 * g] * mult, acc[db][4 * g + 1] * mult,
+                acc[db][4 * g + 2] * mult, acc[db][4 * g + 3] * mult);
+        }
+    }
+}
+
+// key range of the workgroup's query rows: min start / max finish over rows with a non-empty span
+__device__ __forceinline__ void BlockKeyRange(int start, int finish, int tid, int *lo, int *hi, int *red)
+{
+    int s = finish >= start ? start : 0x7fffffff;
+    int f = finish >= start ? finish : -1;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        s = min(s, __shfl_xor(s, o, 64));
+        f = max(f, __shfl_xor(f, o, 64));
+    }
+    if ((tid & 63) == 0) {
+        red[(tid >> 6) * 2] = s;
+        red[(tid >> 6) * 2 + 1] = f;
+    }
+    __syncthreads();
+    *lo = min(min(red[0], red[2]), min(red[4], red[6]));
+    *hi = max(max(red[1], red[3]), max(red[5], red[7]));
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
+// forward: grid (lenRound/128, heads)
+__global__ void __launch_bounds__(256) AttForward(AttP p)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    uint8_t *kRm = lds, *vRm = lds + RM_BYTES, *vT = lds + 2 * RM_BYTES;
+    __shared__ int red[8];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
+    const int head = blockIdx.y;
+    const int myRow = blockIdx.x * BROWS + wave * WROWS + l32;
+    const int64_t hoff = (int64_t)head * HD * 2;
+    const int start = p.spanStart[myRow], finish = p.spanFinish[myRow];
+    int kLo, kHi;
+    BlockKeyRange(start, finish, tid, &kLo, &kHi, red);
+
+    v8bf qf[8];
+    LoadOwnFrags(qf, p.q + (int64_t)(myRow - l32) * p.ldq + hoff, p.ldq, l32, half);
+    v16f oacc[4];
+#pragma unroll
+    for (int db = 0; db < 4; ++db) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            oacc[db][e] = 0;
+        }
+    }
+    float m = 0, sum = 1; // the sink: a zero vector with weight 2^-m
+    for (int t0 = kHi >= kLo ? (kLo / TR) * TR : 1; t0 <= kHi; t0 += TR) {
+        __syncthreads();
+        LoadTile(kRm, p.k + (int64_t)t0 * p.ldk + hoff, p.ldk, tid);
+        LoadTile(vRm, p.v + (int64_t)t0 * p.ldv + hoff, p.ldv, tid);
+        __syncthreads();
+        TransposeTile(vT, vRm, tid);
+        __syncthreads();
+#pragma unroll
+        for (int kb = 0; kb < TR / 32; ++kb) {
+            int keyBase = t0 + kb * 32;
+            v16f s;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                s[e] = 0;
+            }
+#pragma unroll
+            for (int ds = 0; ds < 8; ++ds) {
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(kRm, kb, ds, l32, half), qf[ds], s, 0, 0, 0);
+            }
+            float sv[16];
+            float mx = m;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                int key = keyBase + BlkRow(e, half);
+                bool valid = key >= start && key <= finish;
+                float dp = s[e] * p.attDotScale - p.slope * (float)(myRow - key);
+                sv[e] = valid ? dp : -INFINITY;
+                mx = fmaxf(mx, sv[e]);
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            float alpha = exp2f(m - mx);
+            m = mx;
+            float ps = 0;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                sv[e] = exp2f(sv[e] - m); // exp2(-inf) = 0 for masked keys
+                ps += sv[e];
+            }
+            ps += __shfl_xor(ps, 32, 64);
+            sum = sum * alpha + ps;
+#pragma unroll
+            for (int db = 0; db < 4; ++db) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    oacc[db][e] *= alpha;
+                }
+            }
+            v8bf pb0 = PackB(sv, 0), pb1 = PackB(sv, 1);
+#pragma unroll
+            for (int db = 0; db < 4; ++db) {
+                oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(vT, db, kb * 2, l32, half), pb0, oacc[db], 0, 0, 0);
+                oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(vT, db, kb * 2 + 1, l32, half), pb1, oacc[db], 0, 0, 0);
+            }
+        }
+    }
+    StoreOwnRows<false>(p.out0 + (int64_t)(myRow - l32) * p.ldo0, p.ldo0, head * HD, oacc, 1 / sum, l32, half);
+    if (half == 0) {
+        p.sumWeightLog[(int64_t)head * p.ldStat + myRow] = m + log2f(sum);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
+// dQ: grid (lenRound/128, heads)
+template <bool F32> __global__ void __launch_bounds__(256) AttGradQ(AttP p)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    uint8_t *kRm = lds, *vRm = lds + RM_BYTES, *kT = lds + 2 * RM_BYTES;
+    __shared__ int red[8];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
+    const int head = blockIdx.y;
+    const int myRow = blockIdx.x * BROWS + wave * WROWS + l32;
+    const int64_t hoff = (int64_t)head * HD * 2;
+    const int start = p.spanStart[myRow], finish = p.spanFinish[myRow];
+    int kLo, kHi;
+    BlockKeyRange(start, finish, tid, &kLo, &kHi, red);
+
+    v8bf qf[8], dof[8];
+    LoadOwnFrags(qf, p.q + (int64_t)(myRow - l32) * p.ldq + hoff, p.ldq, l32, half);
+    LoadOwnFrags(dof, p.dO + (int64_t)(myRow - l32) * p.lddo + hoff, p.lddo, l32, half);
+    const float L = p.sumWeightLog[(int64_t)head * p.ldStat + myRow];
+    const float dScale = p.dScale[(int64_t)head * p.ldStat + myRow];
+    const float gmul = p.attDotScale * LN2;
+    v16f acc[4];
+#pragma unroll
+    for (int db = 0; db < 4; ++db) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            acc[db][e] = 0;
+        }
+    }
+    for (int t0 = kHi >= kLo ? (kLo / TR) * TR : 1; t0 <= kHi; t0 += TR) {
+        __syncthreads();
+        LoadTile(kRm, p.k + (int64_t)t0 * p.ldk + hoff, p.ldk, tid);
+        LoadTile(vRm, p.v + (int64_t)t0 * p.ldv + hoff, p.ldv, tid);
+        __syncthreads();
+        TransposeTile(kT, kRm, tid);
+        __syncthreads();
+#pragma unroll
+        for (int kb = 0; kb < TR / 32; ++kb) {
+            int keyBase = t0 + kb * 32;
+            v16f s, dp;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                s[e] = 0;
+                dp[e] = 0;
+            }
+#pragma unroll
+            for (int ds = 0; ds < 8; ++ds) {
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(kRm, kb, ds, l32, half), qf[ds], s, 0, 0, 0);
+                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(vRm, kb, ds, l32, half), dof[ds], dp, 0, 0, 0);
+            }
+            float dsv[16];
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                int key = keyBase + BlkRow(e, half);
+                bool valid = key >= start && key <= finish;
+                float x = s[e] * p.attDotScale - p.slope * (float)(myRow - key);
+                float w = valid ? exp2f(x - L) : 0.f;
+                dsv[e] = w * (dp[e] - dScale) * gmul;
+            }
+            v8bf b0 = PackB(dsv, 0), b1 = PackB(dsv, 1);
+#pragma unroll
+            for (int db = 0; db < 4; ++db) {
+                acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(kT, db, kb * 2, l32, half), b0, acc[db], 0, 0, 0);
+                acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(kT, db, kb * 2 + 1, l32, half), b1, acc[db], 0, 0, 0);
+            }
+        }
+    }
+    StoreOwnRows<F32>(p.out0 + (int64_t)(myRow - l32) * p.ldo0, p.ldo0, head * HD, acc, 1.f, l32, half);
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
+// dK, dV: grid (lenRound/128, heads); the workgroup owns 128 key rows and streams the query rows that reach them
+template <bool F32> __global__ void __launch_bounds__(256) AttGradKV(AttP p)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    uint8_t *qRm = lds, *doRm = lds + RM_BYTES, *qT = lds + 2 * RM_BYTES, *doT = lds + 2 * RM_BYTES + T_BYTES;
+    float *stL = (float *)(lds + 2 * RM_BYTES + 2 * T_BYTES); // [TR] each: L, dScale, start, finish
+    float *stD = stL + TR;
+    int *stS = (int *)(stD + TR);
+    int *stF = stS + TR;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
+    const int head = blockIdx.y;
+    const int myRow = blockIdx.x * BROWS + wave * WROWS + l32; // my key
+    const int64_t hoff = (int64_t)head * HD * 2;
+    const int qLo = p.revLo[blockIdx.x], qHi = p.revHi[blockIdx.x];
+
+    v8bf kf[8], vf[8];
+    LoadOwnFrags(kf, p.k + (int64_t)(myRow - l32) * p.ldk + hoff, p.ldk, l32, half);
+    LoadOwnFrags(vf, p.v + (int64_t)(myRow - l32) * p.ldv + hoff, p.ldv, l32, half);
+    const float gmul = p.attDotScale * LN2;
+    v16f dk[4], dv[4];
+#pragma unroll
+    for (int db = 0; db < 4; ++db) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            dk[db][e] = 0;
+            dv[db][e] = 0;
+        }
+    }
+    for (int t0 = qHi >= qLo ? (qLo / TR) * TR : 1; t0 <= qHi; t0 += TR) {
+        __syncthreads();
+        LoadTile(qRm, p.q + (int64_t)t0 * p.ldq + hoff, p.ldq, tid);
+        LoadTile(doRm, p.dO + (int64_t)t0 * p.lddo + hoff, p.lddo, tid);
+        if (tid < TR) {
+            stL[tid] = p.sumWeightLog[(int64_t)head * p.ldStat + t0 + tid];
+            stD[tid] = p.dScale[(int64_t)head * p.ldStat + t0 + tid];
+            stS[tid] = p.spanStart[t0 + tid];
+            stF[tid] = p.spanFinish[t0 + tid];
+        }
+        __syncthreads();
+        TransposeTile(qT, qRm, tid);
+        TransposeTile(doT, doRm, tid);
+        __syncthreads();
+#pragma unroll
+        for (int qb = 0; qb < TR / 32; ++qb) {
+            v16f s, dp;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                s[e] = 0;
+                dp[e] = 0;
+            }
+#pragma unroll
+            for (int ds = 0; ds < 8; ++ds) {
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(qRm, qb, ds, l32, half), kf[ds], s, 0, 0, 0);
+                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(doRm, qb, ds, l32, half), vf[ds], dp, 0, 0, 0);
+            }
+            float pv[16], dsv[16];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                int qi = qb * 32 + g * 8 + half * 4;
+                float4 L4 = *(const float4 *)(stL + qi);
+                float4 D4 = *(const float4 *)(stD + qi);
+                int4 S4 = *(const int4 *)(stS + qi);
+                int4 F4 = *(const int4 *)(stF + qi);
+                const float Ls[4] = {L4.x, L4.y, L4.z, L4.w};
+                const float Ds[4] = {D4.x, D4.y, D4.z, D4.w};
+                const int Ss[4] = {S4.x, S4.y, S4.z, S4.w};
+                const int Fs[4] = {F4.x, F4.y, F4.z, F4.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    int e = g * 4 + j;
+                    int qrow = t0 + qi + j;
+                    bool valid = myRow >= Ss[j] && myRow <= Fs[j];
+                    float x = s[e] * p.attDotScale - p.slope * (float)(qrow - myRow);
+                    float w = valid ? exp2f(x - Ls[j]) : 0.f;
+                    pv[e] = w;
+                    dsv[e] = w * (dp[e] - Ds[j]) * gmul;
+                }
+            }
+            v8bf pb0 = PackB(pv, 0), pb1 = PackB(pv, 1), sb0 = PackB(dsv, 0), sb1 = PackB(dsv, 1);
+#pragma unroll
+            for (int db = 0; db < 4; ++db) {
+                dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(doT, db, qb * 2, l32, half), pb0, dv[db], 0, 0, 0);
+                dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(doT, db, qb * 2 + 1, l32, half), pb1, dv[db], 0, 0, 0);
+                dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(qT, db, qb * 2, l32, half), sb0, dk[db], 0, 0, 0);
+                dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(qT, db, qb * 2 + 1, l32, half), sb1, dk[db], 0, 0, 0);
+            }
+        }
+    }
+    StoreOwnRows<F32>(p.out0 + (int64_t)(myRow - l32) * p.ldo0, p.ldo0, head * HD, dk, 1.f, l32, half);
+    StoreOwnRows<F32>(p.out1 + (int64_t)(myRow - l32) * p.ldo1, p.ldo1, head * HD, dv, 1.f, l32, half);
+}
+
+// reverse ranges: for every 128-key block the first and last query row whose span touches it
+__global__ void RevInit(int *revLo, int *revHi, int n)
+{
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        revLo[i] = 0x7fffffff;
+        revHi[i] = -1;
+    }
+}
+
+__global__ void RevBuild(const int *spanStart, const int *spanFinish, int len, int *revLo, int *revHi)
+{
+    int q = blockIdx.x * blockDim.x + threadIdx.x;
+    if (q >= len) {
+        return;
+    }
+    int s = spanStart[q], f = spanFinish[q];
+    if (f < s) {
+        return;
+    }
+    for (int b = s / BROWS; b <= f / BROWS; ++b) {
+        atomicMin(&revLo[b], q);
+        atomicMax(&revHi[b], q);
+    }
+}
+
+bool ActOk(const ts2_mat *m, int rows, int cols)
+{
+    return m && m->ptr && m->y >= rows && m->x >= cols && Aligned16(m->ptr, m->strideBytes);
+}
+
+int SetAttr(const void *fn, int bytes)
+{
+    return hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess ? 0 : TS2_ERR_LAUNCH;
+}
+} // namespace
+
+extern "C" int ts2_att_build_rev(int32_t len, int32_t lenRound, const int32_t *spanStart, const int32_t *spanFinish, int32_t *revLo, int32_t *revHi,
+    void *stream)
+{
+    if (!spanStart || !spanFinish || !revLo || !revHi) {
+        return TS2_ERR_NULL;
+    }
+    if (lenRound % BROWS || len > lenRound) {
+        return TS2_ERR_SHAPE;
+    }
+    int n = lenRound / BROWS;
+    hipLaunchKernelGGL(RevInit, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream, revLo, revHi, n);
+    TS2_CHECK_LAUNCH();
+    hipLaunchKernelGGL(RevBuild, dim3((len + 255) / 256), dim3(256), 0, (hipStream_t)stream, spanStart, spanFinish, len, revLo, revHi);
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
+extern "C" int ts2_att_forward(const ts2_att_args *a, void *stream)
+{
+    if (!a || !a->spanStart || !a->spanFinish || !a->sumWeightLog.ptr) {
+        return TS2_ERR_NULL;
+    }
+    int cols = a->heads * HD;
+    if (a->lenRound % BROWS || a->heads <= 0 || !ActOk(&a->q, a->lenRound, cols) || !ActOk(&a->k, a->lenRound, cols) ||
+        !ActOk(&a->v, a->lenRound, cols) || !ActOk(&a->valLookup, a->lenRound, cols) || a->sumWeightLog.y < a->heads ||
+        a->sumWeightLog.x < a->lenRound) {
+        return TS2_ERR_SHAPE;
+    }
+    AttP p = {};
+    p.q = (const uint8_t *)a->q.ptr;
+    p.k = (const uint8_t *)a->k.ptr;
+    p.v = (const uint8_t *)a->v.ptr;
+    p.ldq = a->q.strideBytes;
+    p.ldk = a->k.strideBytes;
+    p.ldv = a->v.strideBytes;
+    p.spanStart = a->spanStart;
+    p.spanFinish = a->spanFinish;
+    p.attDotScale = a->attDotScale;
+    p.slope = a->alibiSlope;
+    p.sumWeightLog = (float *)a->sumWeightLog.ptr;
+    p.ldStat = a->sumWeightLog.strideBytes / 4;
+    p.out0 = (uint8_t *)a->valLookup.ptr;
+    p.ldo0 = a->valLookup.strideBytes;
+    p.lenRound = a->lenRound;
+    int ldsBytes = 2 * RM_BYTES + T_BYTES;
+    static bool done = false;
+    if (!done) {
+        if (SetAttr((const void *)AttForward, ldsBytes)) {
+            return TS2_ERR_LAUNCH;
+        }
+        done = true;
+    }
+    hipLaunchKernelGGL(AttForward, dim3(a->lenRound / BROWS, a->heads), dim3(256), ldsBytes, (hipStream_t)stream, p);
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
+extern "C" int ts2_att_backward(const ts2_att_grad_args *a, void *stream)
+{
+    if (!a || !a->spanStart || !a->spanFinish || !a->revLo || !a->revHi || !a->sumWeightLog.ptr || !a->dScale.ptr) {
+        return TS2_ERR_NULL;
+    }
+    int cols = a->heads * HD;
+    bool f32 = a->gradType == TS2_F32;
+    if (!f32 && a->gradType != TS2_BF16) {
+        return TS2_ERR_UNSUPPORTED;
+    }
+    if (a->lenRound % BROWS || a->heads <= 0 || !ActOk(&a->q, a->lenRound, cols) || !ActOk(&a->k, a->lenRound, cols) ||
+        !ActOk(&a->v, a->lenRound, cols) || !ActOk(&a->dValLookup, a->lenRound, cols) || !ActOk(&a->dQ, a->lenRound, cols) ||
+        !ActOk(&a->dK, a->lenRound, cols) || !ActOk(&a->dV, a->lenRound, cols) || a->sumWeightLog.y < a->heads ||
+        a->sumWeightLog.x < a->lenRound || a->dScale.y < a->heads || a->dScale.x < a->lenRound ||
+        a->dScale.strideBytes != a->sumWeightLog.strideBytes) {
+        return TS2_ERR_SHAPE;
+    }
+    AttP p = {};
+    p.q = (const uint8_t *)a->q.ptr;
+    p.k = (const uint8_t *)a->k.ptr;
+    p.v = (const uint8_t *)a->v.ptr;
+    p.dO = (const uint8_t *)a->dValLookup.ptr;
+    p.ldq = a->q.strideBytes;
+    p.ldk = a->k.strideBytes;
+    p.ldv = a->v.strideBytes;
+    p.lddo = a->dValLookup.strideBytes;
+    p.spanStart = a->spanStart;
+    p.spanFinish = a->spanFinish;
+    p.revLo = a->revLo;
+    p.revHi = a->revHi;
+    p.attDotScale = a->attDotScale;
+    p.slope = a->alibiSlope;
+    p.sumWeightLog = (float *)a->sumWeightLog.ptr;
+    p.dScale = (const float *)a->dScale.ptr;
+    p.ldStat = a->sumWeightLog.strideBytes / 4;
+    p.lenRound = a->lenRound;
+    dim3 grid(a->lenRound / BROWS, a->heads);
+    int ldsQ = 2 * RM_BYTES + T_BYTES;
+    int ldsKV = 2 * RM_BYTES + 2 * T_BYTES + 4 * TR * 4;
+    static bool done = false;
+    if (!done) {
+        if (SetAttr((const void *)AttGradQ<true>, ldsQ) || SetAttr((const void *)AttGradQ<false>, ldsQ) ||
+            SetAttr((const void *)AttGradKV<true>, ldsKV) || SetAttr((const void *)AttGradKV<false>, ldsKV)) {
+            return TS2_ERR_LAUNCH;
+        }
+        done = true;
+    }
+    if (a->which & 1) {
+        p.out0 = (uint8_t *)a->dQ.ptr;
+        p.ldo0 = a->dQ.strideBytes;
+        if (f32) {
+            hipLaunchKernelGGL(AttGradQ<true>, grid, dim3(256), ldsQ, (hipStream_t)stream, p);
+        } else {
+            hipLaunchKernelGGL(AttGradQ<false>, grid, dim3(256), ldsQ, (hipStream_t)stream, p);
+        }
+        TS2_CHECK_LAUNCH();
+    }
+    if (a->which & 2) {
+        p.out0 = (uint8_t *)a->dK.ptr;
+        p.ldo0 = a->dK.strideBytes;
+        p.out1 = (uint8_t *)a->dV.ptr;
+        p.ldo1 = a->dV.strideBytes;
+        if (f32) {
+            hipLaunchKernelGGL(AttGradKV<true>, grid, dim3(256), ldsKV, (hipStream_t)stream, p);
+        } else {
+            hipLaunchKernelGGL(AttGradKV<false>, grid, dim3(256), ldsKV, (hipStream_t)stream, p);
+        }
+        TS2_CHECK_LAUNCH();
+    }
+    return TS2_OK;
+}

@@ -359,6 +359,67 @@ __global__ void __launch_bounds__(256) TransposeQuant(int len, int lenRound, Mat
     }
 }
 
+
+// rope pairs are (cos, sin) interleaved: lane holds two pairs
+__device__ __forceinline__ F4 ApplyRope4(F4 v, F4 rope, float dir)
+{
+    float s0 = rope.y * dir, s1 = rope.w * dir;
+    return MakeF4(v.x * rope.x - v.y * s0, v.x * s0 + v.y * rope.x, v.z * rope.z - v.w * s1, v.z * s1 + v.w * rope.z);
+}
+
+template <class TSrc>
+__global__ void __launch_bounds__(256) RowTileNormalizeRope(int len, int lenRound, int tiles, Mat src, float srcMult, int normalize, float vecScale,
+    Mat rope, Mat dst, Mat tileScale)
+{
+    int t, tile, h;
+    if (!Unit(lenRound, tiles, &t, &tile, &h)) {
+        return;
+    }
+    int col = tile * TILE + h * 4;
+    F4 v = ZeroF4();
+    float discr = 0;
+    if (t < len) {
+        v = Load4<TSrc>(At<TSrc>(src, t, col)) * srcMult;
+        if (normalize) {
+            float sum2 = Half32Sum(HSum(v * v));
+            if (sum2 > 0) {
+                discr = sqrtf(sum2 / TILE) * vecScale;
+                v = v * (1 / discr);
+            }
+        }
+        if (rope.p) {
+            v = ApplyRope4(v, Load4<TF32>(At<TF32>(rope, t, h * 4)), 1.f);
+        }
+    }
+    Store4<TBF16>(At<TBF16>(dst, t, col), v);
+    if (normalize && h == 0) {
+        ScaleAt(tileScale, tile, t) = discr;
+    }
+}
+
+template <class TGrad, class TDst>
+__global__ void __launch_bounds__(256) BackpropRowTileNormalizeRope(int len, int lenRound, int tiles, Mat grad, float gradMult, Mat srcNorm,
+    Mat srcTileScale, Mat rope, Mat dst)
+{
+    int t, tile, h;
+    if (!Unit(lenRound, tiles, &t, &tile, &h)) {
+        return;
+    }
+    int col = tile * TILE + h * 4;
+    F4 g = ZeroF4();
+    if (t < len) {
+        g = Load4<TGrad>(At<TGrad>(grad, t, col)) * gradMult;
+        if (srcNorm.p) {
+            F4 src = Load4<TBF16>(At<TBF16>(srcNorm, t, col)) * ScaleAt(srcTileScale, tile, t);
+            g = TileNormBackprop(src, g);
+        }
+        if (rope.p) {
+            g = ApplyRope4(g, Load4<TF32>(At<TF32>(rope, t, h * 4)), -1.f);
+        }
+    }
+    Store4<TDst>(At<TDst>(dst, t, col), g);
+}
+
 bool MatOk(const ts2_mat *m, int rows, int cols, int elemSize)
 {
     return m && m->ptr && m->y >= rows && m->x >= cols && (m->strideBytes % 4) == 0 && m->strideBytes >= (int64_t)cols * elemSize;
@@ -636,6 +697,64 @@ extern "C" int ts2_transpose_quant(int32_t len, int32_t lenRound, const ts2_mat 
     } else {
         return TS2_ERR_UNSUPPORTED;
     }
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
+extern "C" int ts2_row_tile_normalize_rope(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, float srcMult, int32_t normalize,
+    float vecScale, const ts2_mat *ropeBuf, const ts2_mat *dst, const ts2_mat *tileScale, void *stream)
+{
+    if (!src || !dst || (normalize && !tileScale)) {
+        return TS2_ERR_NULL;
+    }
+    int dim = dst->x;
+    if (dim % TILE || !MatOk(src, len, dim, ElemSize(srcType)) || !MatOk(dst, lenRound, dim, 2) ||
+        (normalize && !MatOk(tileScale, dim / TILE, lenRound, 4)) || (ropeBuf && !MatOk(ropeBuf, len, TILE, 4))) {
+        return TS2_ERR_SHAPE;
+    }
+    int tiles = dim / TILE;
+    Mat rope = ropeBuf ? M(*ropeBuf) : Mat{nullptr, 0};
+    Mat ts = normalize ? M(*tileScale) : Mat{nullptr, 0};
+    if (srcType == TS2_F32) {
+        hipLaunchKernelGGL((RowTileNormalizeRope<TF32>), GridFor(lenRound, tiles), dim3(256), 0, STREAM, len, lenRound, tiles, M(*src), srcMult,
+            normalize, vecScale, rope, M(*dst), ts);
+    } else if (srcType == TS2_BF16) {
+        hipLaunchKernelGGL((RowTileNormalizeRope<TBF16>), GridFor(lenRound, tiles), dim3(256), 0, STREAM, len, lenRound, tiles, M(*src), srcMult,
+            normalize, vecScale, rope, M(*dst), ts);
+    } else {
+        return TS2_ERR_UNSUPPORTED;
+    }
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
+extern "C" int ts2_backprop_row_tile_normalize_rope(int32_t len, int32_t lenRound, const ts2_mat *grad, int32_t gradType, float gradMult,
+    const ts2_mat *srcNorm, const ts2_mat *srcTileScale, const ts2_mat *ropeBuf, const ts2_mat *dst, int32_t dstType, void *stream)
+{
+    if (!grad || !dst || (srcNorm && !srcTileScale)) {
+        return TS2_ERR_NULL;
+    }
+    int dim = dst->x;
+    if (dim % TILE || !MatOk(grad, len, dim, ElemSize(gradType)) || !MatOk(dst, lenRound, dim, ElemSize(dstType)) ||
+        (srcNorm && (!MatOk(srcNorm, len, dim, 2) || !MatOk(srcTileScale, dim / TILE, len, 4))) || (ropeBuf && !MatOk(ropeBuf, len, TILE, 4))) {
+        return TS2_ERR_SHAPE;
+    }
+    int tiles = dim / TILE;
+    Mat rope = ropeBuf ? M(*ropeBuf) : Mat{nullptr, 0};
+    Mat sn = srcNorm ? M(*srcNorm) : Mat{nullptr, 0};
+    Mat st = srcNorm ? M(*srcTileScale) : Mat{nullptr, 0};
+    if (gradType != TS2_F32 && gradType != TS2_BF16) {
+        return TS2_ERR_UNSUPPORTED;
+    }
+#define LAUNCH_BR(TG, TD)                                                                                                                  \
+    hipLaunchKernelGGL((BackpropRowTileNormalizeRope<TG, TD>), GridFor(lenRound, tiles), dim3(256), 0, STREAM, len, lenRound, tiles, M(*grad), \
+        gradMult, sn, st, rope, M(*dst))
+    if (gradType == TS2_F32) {
+        TS2_DISPATCH_TYPE(dstType, TD, LAUNCH_BR(TF32, TD));
+    } else {
+        TS2_DISPATCH_TYPE(dstType, TD, LAUNCH_BR(TBF16, TD));
+    }
+#undef LAUNCH_BR
     TS2_CHECK_LAUNCH();
     return TS2_OK;
 }

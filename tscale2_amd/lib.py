@@ -162,3 +162,32 @@ class MatMulBuffers:
         """dequantised packed delta [gradDim][srcDim]"""
         sc = self.delta_tile_scale.t().repeat_interleave(128, dim=1)
         return self.delta.float() * sc
+
+
+class AttArgs(C.Structure):
+    _fields_ = [("len", C.c_int32), ("lenRound", C.c_int32), ("heads", C.c_int32), ("q", Mat), ("k", Mat), ("v", Mat),
+                ("spanStart", C.c_void_p), ("spanFinish", C.c_void_p), ("attDotScale", C.c_float), ("alibiSlope", C.c_float),
+                ("valLookup", Mat), ("sumWeightLog", Mat)]
+
+
+class AttGradArgs(C.Structure):
+    _fields_ = [("len", C.c_int32), ("lenRound", C.c_int32), ("heads", C.c_int32), ("q", Mat), ("k", Mat), ("v", Mat), ("dValLookup", Mat),
+                ("spanStart", C.c_void_p), ("spanFinish", C.c_void_p), ("revLo", C.c_void_p), ("revHi", C.c_void_p),
+                ("attDotScale", C.c_float), ("alibiSlope", C.c_float), ("sumWeightLog", Mat), ("dScale", Mat), ("dQ", Mat), ("dK", Mat),
+                ("dV", Mat), ("gradType", C.c_int32), ("which", C.c_int32)]
+
+
+def att_forward(len_, heads, q, k, v, span_start, span_finish, att_dot_scale, slope, val_lookup, sum_weight_log):
+    a = AttArgs(len_, q.shape[0], heads, mat(q), mat(k), mat(v), span_start.data_ptr(), span_finish.data_ptr(), att_dot_scale, slope,
+                mat(val_lookup), mat(sum_weight_log))
+    lib = load()
+    lib.check(lib.dll.ts2_att_forward(C.byref(a), lib.stream()), "ts2_att_forward")
+
+
+def att_backward(len_, heads, q, k, v, dval, span_start, span_finish, rev_lo, rev_hi, att_dot_scale, slope, sum_weight_log, dscale, dq, dk,
+                 dv, grad_type, which=3):
+    a = AttGradArgs(len_, q.shape[0], heads, mat(q), mat(k), mat(v), mat(dval), span_start.data_ptr(), span_finish.data_ptr(),
+                    rev_lo.data_ptr(), rev_hi.data_ptr(), att_dot_scale, slope, mat(sum_weight_log), mat(dscale), mat(dq), mat(dk), mat(dv),
+                    grad_type, which)
+    lib = load()
+    lib.check(lib.dll.ts2_att_backward(C.byref(a), lib.stream()), "ts2_att_backward")
