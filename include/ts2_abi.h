@@ -80,6 +80,18 @@ typedef struct ts2_gemm_args {
     ts2_mat tileScale; /* ROW_TILE_MAXNORM: fp32 [n/128][m] */
     int32_t splitK;
     int32_t tileConfig; /* 0 = choose; 1 = 256x256 workgroup tile; 2 = 128x128 */
+    /* Expert-grouped products (TMoeMatMulKernelCall / TMoeDeltaMatMulKernelCall, src/gpt/compute/moe_matmul.cuh:47-215):
+     * tileGroup [m/128] (device): rows of A and C are grouped by expert in 128-row tiles; tile i multiplies the B slab
+     *           b + tileGroup[i]*bSlabBytes (n rows each); tiles with group -1 are skipped (XpTileExpertId).
+     * groupOffsets [groups+1] (device): delta mode, one product per group g over contraction rows
+     *           groupOffsets[g] .. groupOffsets[g+1] (multiples of 128; ExpertOffset), written to c + g*cSlabBytes and, for
+     *           ROW_TILE_MAXNORM, tileScale + g*tileScaleSlabBytes. */
+    const int32_t *tileGroup;
+    int64_t bSlabBytes;
+    const int32_t *groupOffsets;
+    int32_t groups;
+    int64_t cSlabBytes;
+    int64_t tileScaleSlabBytes;
 } ts2_gemm_args;
 
 int ts2_gemm_nt(const ts2_gemm_args *args, void *stream);
@@ -183,12 +195,12 @@ int ts2_matmul_backprop(int32_t mode, int32_t len, int32_t lenRound, int32_t src
     const ts2_matmul_bwd_buffers *buf, float alpha, const float *alphaPtr, const ts2_mat *srcGrad, int32_t srcGradType, int32_t add,
     void *stream);
 
-/* BackpropDelta: delta[gradDim][srcDim] = (*gradScale) * sum_t grad[t][k]*src[t][x] as the packed delta (i8 + tileScale
+/* BackpropDelta: delta[gradDim][srcDim] = alpha * (*gradScale) * sum_t grad[t][k]*src[t][x] as the packed delta (i8 + tileScale
  * [srcDim/128][gradDim], TCudaPackedDeltaMatrix, src/gpt/matrix/delta_cuda.h:9-38).  src is the 8-bit layer input
  * [lenRound][srcDim]; I8: grad (TS2_BF16 | TS2_F32) is requantised per kTile rows (times srcRowScale[t] if given);
  * E4M3: grad is e4m3 and only transposed. */
 int ts2_matmul_backprop_delta(int32_t mode, int32_t len, int32_t lenRound, int32_t srcDim, int32_t gradDim, const ts2_mat *src,
-    const float *srcRowScale, const ts2_mat *grad, int32_t gradType, const float *gradScale, int32_t kTile,
+    const float *srcRowScale, const ts2_mat *grad, int32_t gradType, float alpha, const float *gradScale, int32_t kTile,
     const ts2_matmul_bwd_buffers *buf, const ts2_mat *delta, const ts2_mat *deltaTileScale, void *stream);
 
 /* Forward product of the same operator, TMatMulBuffers::Forward<TStoreScaled> (layer_cuda_base.cuh:183-193):
@@ -251,6 +263,107 @@ int ts2_row_tile_normalize_rope(int32_t len, int32_t lenRound, const ts2_mat *sr
  * vector); if ropeBuf: rotate pairs by -1; store as dstType (TS2_BF16 | TS2_E4M3 | TS2_F32); rows in [len, lenRound) cleared. */
 int ts2_backprop_row_tile_normalize_rope(int32_t len, int32_t lenRound, const ts2_mat *grad, int32_t gradType, float gradMult,
     const ts2_mat *srcNorm, const ts2_mat *srcTileScale, const ts2_mat *ropeBuf, const ts2_mat *dst, int32_t dstType, void *stream);
+
+/* ------------------------------------------------------------------------------------------------------------------------
+ * Mixture of experts (src/gpt/compute/layer_moe.cu, moe_kernels.cu, moe_kernels.cuh).  Tables, all device-resident and
+ * caller-owned, named as in the reference (layer_moe.cu:82-89):
+ *   sampleExpertIds / sampleExpertWeights / sampleExpertOffset [len*selected]   per (token, slot)
+ *   expertOffset [experts+2]   first grouped row of each expert (multiples of 128); [experts] = rows in use; [experts+1] = lenMoe
+ *   xpTileExpertId [lenMoe/128]   expert of each 128-row tile, -1 for the unused tail
+ *   xpSampleId [lenMoe] token of each grouped row (-1 = padding), xpSampleWeight [lenMoe] its routing weight
+ * lenMoe is the capacity of the grouped buffers: at least len*selected + 128*experts, a multiple of 128. */
+typedef struct ts2_moe_tables {
+    int32_t *sampleExpertIds;
+    float *sampleExpertWeights;
+    int32_t *sampleExpertOffset;
+    int32_t *expertOffset;
+    int32_t *xpTileExpertId;
+    int32_t *xpSampleId;
+    float *xpSampleWeight;
+    int32_t *blockCounts; /* scratch: [ceil(len*selected/256)][experts] */
+} ts2_moe_tables;
+
+/* MoeCalcSampleExpertLists + GroupPerExpertLists + InitXpTables + FillXpTables (moe_kernels.cu:54-225): top-`selected` logits
+ * per token (ties: lowest index), w = exp((s - max)/2) scaled so that sum w^2 = experts; grouped rows are ordered by
+ * (expert, token, slot) — deterministic, where the reference's order within an expert depends on atomics.
+ * select: TS2_BF16 | TS2_F32 [len][>= experts]. */
+int ts2_moe_route(int32_t len, int32_t lenMoe, int32_t experts, int32_t selected, const ts2_mat *select, int32_t selectType,
+    const ts2_moe_tables *tables, void *stream);
+
+/* MoeGroupSamples (moe_kernels.cuh:89-143): dst[row] = src[xpSampleId[row]] (zeros for padding) for row < lenMoe; elemSize 1 or 2
+ * bytes.  The transposed copy the reference can emit is ts2_transpose_quant with rowIndex = xpSampleId. */
+int ts2_moe_group_samples(int32_t lenMoe, int32_t elemSize, const ts2_mat *src, const int32_t *xpSampleId, const ts2_mat *dst, void *stream);
+
+/* MatrixLoLUmoe (moe_kernels.cuh:15-44): res = vals * sigmoid(2*gate) * xpSampleWeight[row] * resMult over grouped rows */
+int ts2_matrix_lolu_moe(int32_t lenMoe, const float *xpSampleWeight, const ts2_mat *gate, const ts2_mat *vals, float resMult,
+    const ts2_mat *res, int32_t resType, void *stream);
+
+/* BackpropRowTileNormalizeLoLUmoe (moe_kernels.cu:229-302): the FFN gate/norm backward over grouped rows, with the routing
+ * weight folded in and dExpertWeight[row] = sum_x grad*vals*sigmoid(2 gate) */
+int ts2_backprop_row_tile_normalize_lolu_moe(int32_t lenMoe, const float *xpSampleWeight, const ts2_mat *gate, const ts2_mat *vals,
+    float valsScale, const ts2_mat *valsSrcTileScale, const ts2_mat *grad, int32_t gradType, float gradMult, const ts2_mat *gradGate,
+    const ts2_mat *gradVals, int32_t gradOutType, float *dExpertWeight, void *stream);
+
+/* BackpropMoeKernel (moe_kernels.cu:306-355): routing backward per token -> dMoeSelect [lenRound][dMoe->x] (TS2_F32 | TS2_BF16 | TS2_E4M3), columns
+ * >= experts and rows >= len cleared */
+int ts2_backprop_moe(int32_t len, int32_t lenRound, int32_t experts, int32_t selected, const ts2_moe_tables *tables,
+    const float *dExpertWeight, const ts2_mat *dMoe, int32_t dMoeType, void *stream);
+
+/* CombineExperts (moe_kernels.cuh:146-177): res[t] (op)= alpha * (*alphaPtr) * sum over the token's `selected` grouped rows of
+ * src; src TS2_BF16 | TS2_F32 [lenMoe][dim], res TS2_F32 [len][dim]; add != 0 accumulates (TStoreAdd) */
+int ts2_combine_experts(int32_t len, int32_t selected, const ts2_mat *src, int32_t srcType, const ts2_moe_tables *tables, float alpha,
+    const float *alphaPtr, const ts2_mat *res, int32_t add, void *stream);
+
+/* Batched byte transpose: batch slabs of [rows][cols] -> [cols][rows] (MoeTransposeI8Kernel, src/gpt/compute/moe_matmul.cu:9-19);
+ * rows and cols multiples of 128 */
+int ts2_transpose_u8_batched(int32_t batch, int32_t rows, int32_t cols, const void *src, int64_t srcStride, int64_t srcSlabBytes, void *dst,
+    int64_t dstStride, int64_t dstSlabBytes, void *stream);
+
+/* ------------------------------------------------------------------------------------------------------------------------
+ * Layer stack and one-GPU step driver: the counterpart of TCudaLayerBase::{AddForward, AddBackward}
+ * (src/gpt/compute/layer_cuda_base.cuh:290-294) and of the executor's forward/backprop graphs
+ * (src/gpt/compute/gpu_transformer.cu:260-471; IModelImpl::Backprop, src/gpt/compute/model.h:60-67).
+ * The model object owns its device memory (allocated once at creation, like the reference's pools); the per-step entry points
+ * allocate nothing.  Weights are handed over already quantised (fast bytes + matrix scale), exactly what the reference's
+ * ICudaModelMatrixBase<T>::GetFast/GetScale expose (src/gpt/matrix/base_cuda.cuh:19-43). */
+typedef struct ts2_model ts2_model;
+
+enum { TS2_LT_ATT = 0, TS2_LT_FFN = 2, TS2_LT_MOE = 3 }; /* ELayerType, src/gpt/model_params/model_dim.h:57-62 */
+#define TS2_LAYER_EMBED (-1)
+#define TS2_LAYER_FINAL (-2)
+
+typedef struct ts2_model_config {
+    int32_t mode; /* TS2_I8: i8 weights/states, bf16 fast gradients; TS2_E4M3: e4m3 weights/states/fast gradients */
+    int32_t dim, headCount, ffnDim, expertDim, expertCount, moeSelected; /* TModelDims, model_dim.h:118-141 (head dim 128) */
+    int32_t depth;                                                       /* number of layers */
+    const int32_t *layerType;                                            /* [depth] TS2_LT_* */
+    const int32_t *layerAttId;                                           /* [depth] attention type of attention layers */
+    const float *layerSlope;                                             /* [depth] ALiBi slope */
+    int32_t attTypeCount;
+    int32_t vocab, labelCount, maxLen;
+    int32_t kTile; /* rows sharing one scale in the int8 delta GEMM (0 = 512) */
+} ts2_model_config;
+
+ts2_model *ts2_model_create(const ts2_model_config *cfg);
+void ts2_model_destroy(ts2_model *m);
+/* matrixId: MP_ATT_{Q,K,V,GATE,COMBINER} = 0..4, MP_FFN_{EXPAND,GATE,CONTRACT} = 0..2, MP_MOE_{EXPAND,GATE,CONTRACT,SELECT} = 0..3
+ * (model_dim.h:65-80); fastHost is [rows][cols] bytes of the model's 8-bit type, scale the matrix scale. */
+int ts2_model_set_matrix(ts2_model *m, int32_t layer, int32_t matrixId, const void *fastHost, int32_t rows, int32_t cols, float scale);
+int ts2_model_set_bias(ts2_model *m, const float *biasHost);
+/* nodes of one batch (TBatchNodes, src/gpt/att/nodes_batch.h:42-57): label CSR, target token per row (-1 = none), one span per
+ * row and attention type, RoPE table [len][128]; host arrays */
+int ts2_model_set_batch(ts2_model *m, int32_t len, const int32_t *labelPtr, const uint32_t *labels, const int32_t *targetPerRow,
+    const int32_t *const *spanStart, const int32_t *const *spanFinish, const float *ropeBuf, void *stream);
+int ts2_model_forward(ts2_model *m, void *stream);  /* states + predictions ("prediction" array holds probabilities) */
+int ts2_model_backprop(ts2_model *m, void *stream); /* forward, loss gradient, backward through all layers, every delta */
+/* one layer in isolation on the model's buffers ("state" in, "state" out / "stateGrad" in-out) */
+int ts2_layer_forward(ts2_model *m, int32_t layer, void *stream);
+int ts2_layer_backward(ts2_model *m, int32_t layer, void *stream);
+/* dequantised delta of a matrix into hostOut [rows][cols] (synchronises the device) */
+int ts2_model_get_delta(ts2_model *m, int32_t layer, int32_t matrixId, float *hostOut, int32_t rows, int32_t cols);
+/* device view of an internal array: "state", "stateGrad", "stateGradFast", "dNormState", "prediction", "normState"[i], "stateScale"[i] */
+int ts2_model_array(ts2_model *m, const char *name, int32_t index, ts2_mat *out, int32_t *type);
+int ts2_model_scalars(ts2_model *m, float *lossSumHost, int32_t *lenRound, int32_t *lenMoe);
 
 /* peak dense MFMA rate the library prices its kernels against, in T(FL)OP/s, and the CU count it tiles for */
 int ts2_device_info(int *cuCount, int *clockMHz);

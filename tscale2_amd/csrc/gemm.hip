@@ -31,6 +31,13 @@ struct GemmP {
     int64_t ldTileScale; // floats
     int splitK;
     int tilesM, tilesN;
+    // expert-grouped modes (MoE)
+    const int *tileGroup;    // [m/128]: group of each 128-row tile of A/C, -1 = skip; B slab = b + group * bSlab
+    int64_t bSlab;           // bytes
+    const int *groupOffsets; // [groups+1] contraction row ranges (multiples of 128); blockIdx.y = group
+    int64_t cSlab;           // bytes between the C blocks of consecutive groups
+    int64_t tileScaleSlab;   // floats
+    int splitK_groups;       // number of groups when groupOffsets is set
 };
 
 enum { T_I8 = 0, T_FP8 = 1, T_BF16 = 2 };
@@ -99,6 +106,24 @@ __global__ void __launch_bounds__(256, 1) GemmNT(GemmP p)
     // contraction range of this workgroup
     int kSteps = p.kBytes / BKB;
     int kBeg = 0;
+    if (p.tileGroup) {
+        // rows of one 128-row tile belong to one group (BM == 128 is enforced by the host); its B operand is that group's slab
+        int g = p.tileGroup[rowBase / TILE];
+        if (g < 0) {
+            return;
+        }
+        p.b += (int64_t)g * p.bSlab;
+    }
+    if (p.groupOffsets) {
+        // delta of one group: contraction over the group's own rows only
+        int g = blockIdx.y;
+        kBeg = p.groupOffsets[g] * (TYPE == T_BF16 ? 2 : 1) / BKB;
+        kSteps = p.groupOffsets[g + 1] * (TYPE == T_BF16 ? 2 : 1) / BKB - kBeg;
+        p.c += (int64_t)g * p.cSlab;
+        if (p.tileScale) {
+            p.tileScale += (int64_t)g * p.tileScaleSlab;
+        }
+    }
     if (p.splitK > 1) {
         int per = (kSteps + p.splitK - 1) / p.splitK;
         if (KT) {
@@ -233,8 +258,10 @@ __global__ void __launch_bounds__(256, 1) GemmNT(GemmP p)
     };
 
     // main loop: one barrier per step, LDS double buffered, global loads of step s+1 in flight during the MFMAs of step s
-    loadGlobal(0);
-    storeLds(0);
+    if (kSteps > 0) {
+        loadGlobal(0);
+        storeLds(0);
+    }
     __syncthreads();
     const int tileSteps = KT ? p.kTileBytes / BKB : 0;
     for (int s = 0; s < kSteps; ++s) {
@@ -244,7 +271,7 @@ __global__ void __launch_bounds__(256, 1) GemmNT(GemmP p)
         }
         compute(cur);
         if (KT) {
-            if ((s + 1) % tileSteps == 0 || s + 1 == kSteps) {
+            if ((kBeg + s + 1) % tileSteps == 0 || s + 1 == kSteps) {
                 float sc = p.kTileScale[(kBeg + s) / tileSteps];
 #pragma unroll
                 for (int i = 0; i < WTM; ++i) {
@@ -417,7 +444,7 @@ template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT> int Launch(const
         attrDone = true;
     }
     int nb = q.tilesM * q.tilesN * (p.splitK > 1 ? p.splitK : 1);
-    hipLaunchKernelGGL(kern, dim3(nb), dim3(256), ldsBytes, stream, q);
+    hipLaunchKernelGGL(kern, dim3(nb, p.groupOffsets ? p.splitK_groups : 1), dim3(256), ldsBytes, stream, q);
     TS2_CHECK_LAUNCH();
     return TS2_OK;
 }
@@ -475,7 +502,7 @@ template <int TYPE> int DispatchTile(const ts2_gemm_args *a, const GemmP &p, hip
         cfg = tilesL >= 192 ? 1 : 2;
     }
     // the 256x256 kernel needs full tiles and has no room for the second accumulator set of the k-tile-scaled variant
-    if (cfg == 1 && !a->kTileScale && (p.m % 256) == 0 && (p.n % 256) == 0) {
+    if (cfg == 1 && !a->kTileScale && !p.tileGroup && (p.m % 256) == 0 && (p.n % 256) == 0) {
         return DispatchEpi<TYPE, 4, 4>(a, p, stream);
     }
     return DispatchEpi<TYPE, 2, 2>(a, p, stream);
@@ -531,6 +558,18 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
     p.ldTileScale = a->tileScale.strideBytes / 4;
     p.splitK = splitK;
     p.tilesM = p.tilesN = 0;
+    p.tileGroup = a->tileGroup;
+    p.bSlab = a->bSlabBytes;
+    p.groupOffsets = a->groupOffsets;
+    p.cSlab = a->cSlabBytes;
+    p.tileScaleSlab = a->tileScaleSlabBytes / 4;
+    p.splitK_groups = a->groups;
+    if ((a->tileGroup || a->groupOffsets) && splitK > 1) {
+        return TS2_ERR_UNSUPPORTED;
+    }
+    if (a->groupOffsets && a->groups <= 0) {
+        return TS2_ERR_SHAPE;
+    }
     if (splitK > 1 && a->epilogue == TS2_EPI_STORE) {
         // partial sums are accumulated with atomics: clear the live rows first (with a fill kernel, which is safe under graph capture)
         hipLaunchKernelGGL(ZeroRows, dim3(a->m), dim3(256), 0, stream, (uint8_t *)a->c.ptr, (int64_t)a->c.strideBytes, a->n * 4);

@@ -1,0 +1,916 @@
+// Layer orchestration and the one-GPU step driver: the call order of the reference's CUDA layers and executor
+//   TCudaFFLayer::AddForward/AddBackward     src/gpt/compute/layer_ffn.cu:56-113
+//   TCudaAttLayer::AddForward/AddBackward    src/gpt/compute/layer_att.cu:108-226
+//   TCudaMoELayer::AddForward/AddBackward    src/gpt/compute/layer_moe.cu:117-272
+//   AddForwardGraph / CreateBackpropGraph    src/gpt/compute/gpu_transformer.cu:260-471
+// expressed over the C ABI of this library.  Host code only.  Unlike the reference's CUDA path, which drops constant factors
+// (matrix scales, 1/24 storage scales) because its optimiser normalises every delta, this driver keeps every factor of the CPU
+// path (src/gpt/compute/cpu_transformer.cpp, layer_*.cu CPU classes), so its deltas are directly comparable with the CPU oracle.
+#include "common.h"
+#include "internal.h"
+#include <math.h>
+#include <string.h>
+#include <vector>
+
+namespace
+{
+constexpr float VEC = 1 / 24.0f;    // STATE/Q/K/V/FFN/MOE_VEC_SCALE, src/gpt/compute/cfg_precision.h:72-77
+constexpr float DISCR = 1 / 32.0f;  // MODEL_DISCR_SCALE, src/gpt/model_params/model_dim.h:9
+constexpr float LN2F = 0.693147f;   // LOG2, model_dim.h:16
+
+inline float Dot(int dim)
+{
+    return sqrtf(1.0f / dim);
+}
+
+int ElemSz(int type)
+{
+    return (type == TS2_F32 || type == TS2_I32) ? 4 : (type == TS2_BF16 ? 2 : 1);
+}
+
+struct Arr {
+    ts2_mat m = {nullptr, 0, 0, 0};
+    int type = 0;
+    const ts2_mat *P() const { return &m; }
+};
+
+#define CK(x)                                                                                                                              \
+    do {                                                                                                                                   \
+        int rc_ = (x);                                                                                                                     \
+        if (rc_ != 0)                                                                                                                      \
+            return rc_;                                                                                                                    \
+    } while (0)
+
+struct TMatrix {
+    Arr fast;           // [dst][src] 8-bit ([slabs*dst][src] for expert matrices)
+    float *scale = 0;   // device: matrix scale (rms of the fp32 master weights)
+    Arr delta;          // i8 packed delta, same shape
+    Arr deltaTileScale; // fp32 [src/128][rows]
+    int srcDim = 0, dstDim = 0, slabs = 1;
+};
+
+struct TLayer {
+    int type = 0;
+    float slope = 0;
+    int attId = 0;
+    TMatrix w[5];
+};
+
+enum { LT_ATT = 0, LT_FFN = 2, LT_MOE = 3 };
+} // namespace
+
+struct ts2_model {
+    ts2_model_config cfg;
+    std::vector<int> layerType, layerAttId;
+    std::vector<float> layerSlope;
+    std::vector<TLayer> layers;
+    std::vector<void *> allocs;
+    int mode = TS2_I8, fastGradType = TS2_BF16;
+    int R = 0; // lenRound capacity
+    int len = 0;
+    int lenMoe = 0;
+    int kTile = 512;
+    // model
+    TMatrix embed, finalW;
+    float *bias = 0;
+    // batch
+    int *labelPtr = 0;
+    uint32_t *labels = 0;
+    int labelCap = 0;
+    int *target = 0;
+    std::vector<int *> spanStart, spanFinish, revLo, revHi;
+    Arr rope;
+    // states
+    Arr state, stateGrad, stateGradFast, dNormState;
+    std::vector<Arr> normState, stateScale;
+    float *gradMaxNorm = 0, *gradScale = 0, *gradMult = 0, *lossSum = 0;
+    // layer scratch (shared by all layers: one layer runs at a time)
+    Arr raw;                                 // fp32 [R'][maxW]
+    Arr a16[4];                              // bf16 [R'][maxW]: wide/q, gate, k/val, v
+    Arr tsc[3];                              // fp32 [maxW/128][R'] tile scales
+    Arr rg8;                                 // 8-bit [R'][maxW]
+    Arr g32;                                 // fp32 [R'][maxW] gradient scratch (drg / dvlg)
+    Arr gf[4];                               // fast-gradient type [R'][maxW]: dwide/dq, dgate, dk, dv
+    Arr g16[4];                              // bf16 [R'][maxW]: dVal, dQ, dK, dV
+    Arr swl, dScale;                         // fp32 [heads][R]
+    // MoE
+    ts2_moe_tables moe = {};
+    Arr normMoe, sgMoe, moeSel, dMoeSel;     // grouped 8-bit input / gradient, select logits fp32, their gradient
+    float *dExpertWeight = 0;
+    Arr wT;                                  // transposed expert weights scratch
+    // final layer
+    Arr logits, gradV, gradVT, fnT, wfT;
+    // linear backward scratch
+    uint8_t *sGrad8 = 0, *sGradT = 0, *sSrcT = 0, *sWT = 0;
+    float *sRowScale = 0, *sTileMax = 0, *sTileScale = 0;
+    int maxW = 0, RP = 0; // RP = rows of the row-indexed scratch (max(R, lenMoe))
+
+    void *Dev(size_t bytes)
+    {
+        void *p = nullptr;
+        if (hipMalloc(&p, bytes ? bytes : 16) != hipSuccess) {
+            return nullptr;
+        }
+        hipMemset(p, 0, bytes ? bytes : 16);
+        allocs.push_back(p);
+        return p;
+    }
+    bool Alloc(Arr *a, int rows, int cols, int type)
+    {
+        a->type = type;
+        int64_t stride = ((int64_t)cols * ElemSz(type) + 255) / 256 * 256;
+        a->m.ptr = Dev((size_t)stride * rows);
+        a->m.strideBytes = stride;
+        a->m.x = cols;
+        a->m.y = rows;
+        return a->m.ptr != nullptr;
+    }
+    ~ts2_model()
+    {
+        for (void *p : allocs) {
+            hipFree(p);
+        }
+    }
+};
+
+namespace
+{
+// view of the first rows x cols of an array (same storage)
+Arr View(const Arr &a, int rows, int cols)
+{
+    Arr r = a;
+    r.m.x = cols;
+    r.m.y = rows;
+    return r;
+}
+
+Arr Flat(void *p, int rows, int cols, int type)
+{
+    Arr r;
+    r.type = type;
+    r.m.ptr = p;
+    r.m.strideBytes = (int64_t)cols * ElemSz(type);
+    r.m.x = cols;
+    r.m.y = rows;
+    return r;
+}
+
+ts2_matmul_bwd_buffers Scratch(ts2_model *M, int rows, int srcDim, int gradDim)
+{
+    ts2_matmul_bwd_buffers b = {};
+    b.grad8 = Flat(M->sGrad8, rows, gradDim, TS2_I8).m;
+    b.grad8RowScale = M->sRowScale;
+    b.gradT = Flat(M->sGradT, gradDim, rows, M->mode).m;
+    b.srcT = Flat(M->sSrcT, srcDim, rows, M->mode).m;
+    b.tileMax = M->sTileMax;
+    b.tileScale = M->sTileScale;
+    b.transformT = Flat(M->sWT, srcDim, gradDim, M->mode).m;
+    return b;
+}
+
+// res (+)= alpha [* scale] * src8 * W^T
+int Forward(ts2_model *M, TMatrix &W, const Arr &src8, float alpha, bool useScale, const Arr &res, bool add, void *s)
+{
+    return ts2_matmul_forward(M->mode, M->len, M->R, W.srcDim, W.dstDim, src8.P(), W.fast.P(), alpha, useScale ? W.scale : nullptr, res.P(),
+        res.type, add, s);
+}
+
+// srcGrad (+)= alpha [* scale] * gradFast * W   (TMatMulBuffers::BackpropMulti + Backprop)
+int BackpropDX(ts2_model *M, TMatrix &W, const Arr &gradFast, float alpha, bool useScale, const Arr &srcGrad, bool add, void *s)
+{
+    ts2_matmul_bwd_buffers b = Scratch(M, M->R, W.srcDim, W.dstDim);
+    CK(ts2_matmul_backprop_multi(M->mode, M->len, M->R, W.srcDim, W.dstDim, W.fast.P(), gradFast.P(), gradFast.type, nullptr, &b, s));
+    return ts2_matmul_backprop(M->mode, M->len, M->R, W.srcDim, W.dstDim, gradFast.P(), &b, alpha, useScale ? W.scale : nullptr, srcGrad.P(),
+        srcGrad.type, add, s);
+}
+
+// delta = alpha * gradScale * gradFast^T * src8   (TMatMulBuffers::BackpropDelta)
+int BackpropDelta(ts2_model *M, TMatrix &W, const Arr &src8, const Arr &gradFast, float alpha, const float *gradScale, void *s)
+{
+    ts2_matmul_bwd_buffers b = Scratch(M, M->R, W.srcDim, W.dstDim);
+    return ts2_matmul_backprop_delta(M->mode, M->len, M->R, W.srcDim, W.dstDim, src8.P(), nullptr, gradFast.P(), gradFast.type, alpha, gradScale,
+        M->kTile, &b, W.delta.P(), W.deltaTileScale.P(), s);
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
+// FFN: src/gpt/compute/layer_ffn.cu:56-113 (CUDA order) with the CPU path's factors (layer_ffn.cu:190-248)
+int FfnComputeRG(ts2_model *M, TLayer &L, const Arr &norm8, void *s)
+{
+    int D = M->cfg.dim, F = M->cfg.ffnDim, len = M->len, R = M->R;
+    Arr wideRaw = View(M->raw, R, F), wide16 = View(M->a16[0], R, F), gate16 = View(M->a16[1], R, F), wideScale = View(M->tsc[0], F / 128, R);
+    Arr rg8 = View(M->rg8, R, F);
+    // wide = MulForward(n, We) in true units, then per-tile normalisation to 1/24 units + tile scale
+    CK(Forward(M, L.w[0], norm8, VEC * DISCR * Dot(D), true, wideRaw, false, s));
+    CK(ts2_row_tile_normalize_rope(len, R, wideRaw.P(), TS2_F32, 1.f, 1, VEC, nullptr, wide16.P(), wideScale.P(), s));
+    // gate uses the matrix without its scale (GetDataNoScale)
+    CK(Forward(M, L.w[1], norm8, VEC * DISCR * Dot(D), false, gate16, false, s));
+    return ts2_matrix_lolu(len, R, gate16.P(), wide16.P(), 1.f, rg8.P(), M->mode, s);
+}
+
+int FfnForward(ts2_model *M, TLayer &L, const Arr &norm8, void *s)
+{
+    int F = M->cfg.ffnDim;
+    CK(FfnComputeRG(M, L, norm8, s));
+    return Forward(M, L.w[2], View(M->rg8, M->R, F), VEC * DISCR * Dot(F), true, M->state, true, s);
+}
+
+int FfnBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScale, void *s)
+{
+    int D = M->cfg.dim, F = M->cfg.ffnDim, len = M->len, R = M->R;
+    Arr wide16 = View(M->a16[0], R, F), gate16 = View(M->a16[1], R, F), wideScale = View(M->tsc[0], F / 128, R), rg8 = View(M->rg8, R, F);
+    Arr drg = View(M->g32, R, F), dwide = View(M->gf[0], R, F), dgate = View(M->gf[1], R, F);
+    CK(FfnComputeRG(M, L, norm8, s));
+    // contract backward
+    CK(BackpropDX(M, L.w[2], M->stateGradFast, DISCR * Dot(F), true, drg, false, s));
+    CK(ts2_backprop_row_tile_normalize_lolu(len, R, gate16.P(), wide16.P(), VEC, wideScale.P(), drg.P(), TS2_F32, dgate.P(), dwide.P(),
+        M->fastGradType, s));
+    CK(BackpropDX(M, L.w[0], dwide, DISCR * Dot(D), true, M->dNormState, false, s));
+    CK(BackpropDX(M, L.w[1], dgate, DISCR * Dot(D), false, M->dNormState, true, s));
+    // deltas (sources are stored in 1/24 units)
+    CK(BackpropDelta(M, L.w[2], rg8, M->stateGradFast, VEC, gradScale, s));
+    CK(BackpropDelta(M, L.w[0], norm8, dwide, VEC, gradScale, s));
+    return BackpropDelta(M, L.w[1], norm8, dgate, VEC, gradScale, s);
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
+// attention: src/gpt/compute/layer_att.cu:108-226 with the CPU path's factors (layer_att.cu:368-482)
+float AttDotScale()
+{
+    return Dot(128) * (0.5f / LN2F); // CalcDotScale(QDim) * CalcAttentionMult(), layer_att_reference.h:29-32
+}
+
+int AttComputeVLG(ts2_model *M, TLayer &L, const Arr &norm8, void *s)
+{
+    int D = M->cfg.dim, H = M->cfg.headCount, Q = H * 128, len = M->len, R = M->R;
+    Arr raw = View(M->raw, R, Q), q16 = View(M->a16[0], R, Q), gate16 = View(M->a16[1], R, Q), k16 = View(M->a16[2], R, Q), v16 = View(M->a16[3], R, Q);
+    Arr qScale = View(M->tsc[0], H, R), vScale = View(M->tsc[1], H, R), val16 = View(M->g16[0], R, Q), vlg8 = View(M->rg8, R, Q);
+    float a = VEC * DISCR * Dot(D);
+    CK(Forward(M, L.w[0], norm8, a, true, raw, false, s));
+    CK(ts2_row_tile_normalize_rope(len, R, raw.P(), TS2_F32, 1.f, 1, 1.f, M->rope.P(), q16.P(), qScale.P(), s));
+    CK(Forward(M, L.w[1], norm8, a, true, raw, false, s));
+    CK(ts2_row_tile_normalize_rope(len, R, raw.P(), TS2_F32, 1.f, 0, 1.f, M->rope.P(), k16.P(), nullptr, s));
+    CK(Forward(M, L.w[2], norm8, a, true, raw, false, s));
+    CK(ts2_row_tile_normalize_rope(len, R, raw.P(), TS2_F32, 1.f, 1, 1.f, nullptr, v16.P(), vScale.P(), s));
+    CK(Forward(M, L.w[3], norm8, a, false, gate16, false, s));
+    ts2_att_args at = {};
+    at.len = len;
+    at.lenRound = R;
+    at.heads = H;
+    at.q = q16.m;
+    at.k = k16.m;
+    at.v = v16.m;
+    at.spanStart = M->spanStart[L.attId];
+    at.spanFinish = M->spanFinish[L.attId];
+    at.attDotScale = AttDotScale();
+    at.alibiSlope = L.slope;
+    at.valLookup = val16.m;
+    at.sumWeightLog = M->swl.m;
+    CK(ts2_att_forward(&at, s));
+    // VLG = sigmoid(2 gate) * val in 1/24 units
+    return ts2_matrix_lolu(len, R, gate16.P(), val16.P(), 24.f, vlg8.P(), M->mode, s);
+}
+
+int AttForward(ts2_model *M, TLayer &L, const Arr &norm8, void *s)
+{
+    int TT = M->cfg.headCount * 128;
+    CK(AttComputeVLG(M, L, norm8, s));
+    return Forward(M, L.w[4], View(M->rg8, M->R, TT), VEC * DISCR * Dot(TT), true, M->state, true, s);
+}
+
+int AttBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScale, void *s)
+{
+    int D = M->cfg.dim, H = M->cfg.headCount, Q = H * 128, len = M->len, R = M->R;
+    Arr q16 = View(M->a16[0], R, Q), gate16 = View(M->a16[1], R, Q), k16 = View(M->a16[2], R, Q), v16 = View(M->a16[3], R, Q);
+    Arr qScale = View(M->tsc[0], H, R), vScale = View(M->tsc[1], H, R), val16 = View(M->g16[0], R, Q), vlg8 = View(M->rg8, R, Q);
+    Arr dvlg = View(M->g32, R, Q), dGate = View(M->gf[1], R, Q), dVal16 = View(M->g16[1], R, Q);
+    CK(AttComputeVLG(M, L, norm8, s));
+    // combiner backward
+    CK(BackpropDX(M, L.w[4], M->stateGradFast, DISCR * Dot(Q), true, dvlg, false, s));
+    CK(BackpropDelta(M, L.w[4], vlg8, M->stateGradFast, VEC, gradScale, s));
+    // gate backward + dScale
+    CK(ts2_backprop_lolu_dscale(len, R, gate16.P(), val16.P(), 1.f, dvlg.P(), TS2_F32, dGate.P(), M->fastGradType, dVal16.P(), TS2_BF16,
+        M->dScale.P(), s));
+    // attention backward (dQ, dK, dV in bf16; val16's buffer is reused for dQ once dScale is known)
+    Arr dQ = View(M->g16[0], R, Q), dK = View(M->g16[2], R, Q), dV = View(M->g16[3], R, Q);
+    ts2_att_grad_args ag = {};
+    ag.len = len;
+    ag.lenRound = R;
+    ag.heads = H;
+    ag.q = q16.m;
+    ag.k = k16.m;
+    ag.v = v16.m;
+    ag.dValLookup = dVal16.m;
+    ag.spanStart = M->spanStart[L.attId];
+    ag.spanFinish = M->spanFinish[L.attId];
+    ag.revLo = M->revLo[L.attId];
+    ag.revHi = M->revHi[L.attId];
+    ag.attDotScale = AttDotScale();
+    ag.alibiSlope = L.slope;
+    ag.sumWeightLog = M->swl.m;
+    ag.dScale = M->dScale.m;
+    ag.dQ = dQ.m;
+    ag.dK = dK.m;
+    ag.dV = dV.m;
+    ag.gradType = TS2_BF16;
+    ag.which = 3;
+    CK(ts2_att_backward(&ag, s));
+    // epilogues: norm backward against the stored rotated vector, then inverse rope (TStoreAttBack*, gpu_att_utils.cuh:280-352)
+    Arr dQf = View(M->gf[0], R, Q), dKf = View(M->gf[2], R, Q), dVf = View(M->gf[3], R, Q);
+    CK(ts2_backprop_row_tile_normalize_rope(len, R, dQ.P(), TS2_BF16, 1.f, q16.P(), qScale.P(), M->rope.P(), dQf.P(), M->fastGradType, s));
+    CK(ts2_backprop_row_tile_normalize_rope(len, R, dK.P(), TS2_BF16, 1.f, nullptr, nullptr, M->rope.P(), dKf.P(), M->fastGradType, s));
+    CK(ts2_backprop_row_tile_normalize_rope(len, R, dV.P(), TS2_BF16, 1.f, v16.P(), vScale.P(), nullptr, dVf.P(), M->fastGradType, s));
+    float a = DISCR * Dot(D);
+    CK(BackpropDX(M, L.w[0], dQf, a, true, M->dNormState, false, s));
+    CK(BackpropDX(M, L.w[1], dKf, a, true, M->dNormState, true, s));
+    CK(BackpropDX(M, L.w[2], dVf, a, true, M->dNormState, true, s));
+    CK(BackpropDX(M, L.w[3], dGate, a, false, M->dNormState, true, s));
+    CK(BackpropDelta(M, L.w[0], norm8, dQf, VEC, gradScale, s));
+    CK(BackpropDelta(M, L.w[1], norm8, dKf, VEC, gradScale, s));
+    CK(BackpropDelta(M, L.w[2], norm8, dVf, VEC, gradScale, s));
+    return BackpropDelta(M, L.w[3], norm8, dGate, VEC, gradScale, s);
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
+// MoE: src/gpt/compute/layer_moe.cu:117-272 with the CPU path's factors (layer_moe.cu:458-537).  fp8 operands only.
+int GroupedGemm(ts2_model *M, const Arr &a, const Arr &bSlabs, int slabRows, int n, int k, const Arr &c, float alpha, const float *alphaPtr, bool add,
+    void *s)
+{
+    ts2_gemm_args g = {};
+    g.a = a.m;
+    g.b = bSlabs.m;
+    g.b.y = slabRows; // one slab; the kernel offsets by the tile's expert
+    g.c = c.m;
+    g.abType = a.type;
+    g.cType = c.type;
+    g.m = M->lenMoe;
+    g.n = n;
+    g.k = k;
+    g.alpha = alpha;
+    g.alphaPtr = alphaPtr;
+    g.epilogue = add ? TS2_EPI_ADD : TS2_EPI_STORE;
+    g.splitK = 1;
+    g.tileGroup = M->moe.xpTileExpertId;
+    g.bSlabBytes = (int64_t)slabRows * bSlabs.m.strideBytes;
+    return ts2_gemm_nt(&g, s);
+}
+
+// per-expert delta: delta_e[gradDim][srcDim] = alpha * gradScale * sum over the expert's rows of grad^T src
+int GroupedDelta(ts2_model *M, TMatrix &W, const Arr &src8, const Arr &gradFast, float alpha, const float *gradScale, void *s)
+{
+    int E = M->cfg.expertCount, rows = M->lenMoe;
+    Arr gradT = Flat(M->sGradT, W.dstDim, rows, M->mode), srcT = Flat(M->sSrcT, W.srcDim, rows, M->mode);
+    CK(ts2_transpose_quant(rows, rows, gradFast.P(), M->mode, nullptr, nullptr, 0, nullptr, gradT.P(), M->mode, nullptr, s));
+    CK(ts2_transpose_quant(rows, rows, src8.P(), M->mode, nullptr, nullptr, 0, nullptr, srcT.P(), M->mode, nullptr, s));
+    ts2_gemm_args g = {};
+    g.a = gradT.m;
+    g.b = srcT.m;
+    g.c = W.delta.m;
+    g.c.y = W.dstDim;
+    g.abType = M->mode;
+    g.cType = TS2_I8;
+    g.m = W.dstDim;
+    g.n = W.srcDim;
+    g.k = rows;
+    g.alpha = alpha;
+    g.alphaPtr = gradScale;
+    g.epilogue = TS2_EPI_ROW_TILE_MAXNORM;
+    g.tileScale = W.deltaTileScale.m;
+    g.tileScale.x = W.dstDim;
+    g.splitK = 1;
+    g.groupOffsets = M->moe.expertOffset;
+    g.groups = E;
+    g.cSlabBytes = (int64_t)W.dstDim * W.delta.m.strideBytes;
+    g.tileScaleSlabBytes = (int64_t)W.dstDim * 4; // tileScale rows are [src/128][E*dst]: slab e starts at column e*dst
+    return ts2_gemm_nt(&g, s);
+}
+
+int MoeComputeRG(ts2_model *M, TLayer &L, const Arr &norm8, void *s)
+{
+    int D = M->cfg.dim, X = M->cfg.expertDim, E = M->cfg.expertCount, K = M->cfg.moeSelected, len = M->len, R = M->R, RM = M->lenMoe;
+    float a = VEC * DISCR * Dot(D);
+    // select logits (matrix without scale), routing tables, gather of the layer input into expert order
+    CK(Forward(M, L.w[3], norm8, a, false, M->moeSel, false, s));
+    CK(ts2_moe_route(len, RM, E, K, M->moeSel.P(), TS2_F32, &M->moe, s));
+    CK(ts2_moe_group_samples(RM, 1, norm8.P(), M->moe.xpSampleId, M->normMoe.P(), s));
+    Arr wideRaw = View(M->raw, RM, X), wide16 = View(M->a16[0], RM, X), gate16 = View(M->a16[1], RM, X), wideScale = View(M->tsc[0], X / 128, RM);
+    Arr rg8 = View(M->rg8, RM, X);
+    CK(GroupedGemm(M, M->normMoe, L.w[0].fast, X, X, D, wideRaw, a, L.w[0].scale, false, s));
+    CK(ts2_row_tile_normalize_rope(RM, RM, wideRaw.P(), TS2_F32, 1.f, 1, VEC, nullptr, wide16.P(), wideScale.P(), s));
+    CK(GroupedGemm(M, M->normMoe, L.w[1].fast, X, X, D, gate16, a, nullptr, false, s));
+    return ts2_matrix_lolu_moe(RM, M->moe.xpSampleWeight, gate16.P(), wide16.P(), 1.f, rg8.P(), M->mode, s);
+}
+
+int MoeForward(ts2_model *M, TLayer &L, const Arr &norm8, void *s)
+{
+    int D = M->cfg.dim, X = M->cfg.expertDim, E = M->cfg.expertCount, RM = M->lenMoe;
+    CK(MoeComputeRG(M, L, norm8, s));
+    Arr contract = View(M->g32, RM, D);
+    CK(GroupedGemm(M, View(M->rg8, RM, X), L.w[2].fast, D, D, X, contract, VEC * DISCR * Dot(E * X), L.w[2].scale, false, s));
+    return ts2_combine_experts(M->len, M->cfg.moeSelected, contract.P(), TS2_F32, &M->moe, 1.f, nullptr, M->state.P(), 1, s);
+}
+
+int MoeBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScale, void *s)
+{
+    int D = M->cfg.dim, X = M->cfg.expertDim, E = M->cfg.expertCount, K = M->cfg.moeSelected, len = M->len, R = M->R, RM = M->lenMoe;
+    CK(MoeComputeRG(M, L, norm8, s));
+    Arr wide16 = View(M->a16[0], RM, X), gate16 = View(M->a16[1], RM, X), wideScale = View(M->tsc[0], X / 128, RM), rg8 = View(M->rg8, RM, X);
+    // state gradient into expert order
+    CK(ts2_moe_group_samples(RM, 1, M->stateGradFast.P(), M->moe.xpSampleId, M->sgMoe.P(), s));
+    // contract backward: dRG[row][x] = sum_d sg[row][d] Wc_e[d][x]: needs Wc_e^T = [X][D] per expert
+    Arr wcT = View(M->wT, E * X, D);
+    CK(ts2_transpose_u8_batched(E, D, X, L.w[2].fast.m.ptr, L.w[2].fast.m.strideBytes, (int64_t)D * L.w[2].fast.m.strideBytes, wcT.m.ptr,
+        wcT.m.strideBytes, (int64_t)X * wcT.m.strideBytes, s));
+    Arr drg = View(M->g32, RM, X);
+    CK(GroupedGemm(M, M->sgMoe, wcT, X, X, D, drg, DISCR * Dot(E * X), L.w[2].scale, false, s));
+    Arr dwide = View(M->gf[0], RM, X), dgate = View(M->gf[1], RM, X);
+    CK(ts2_backprop_row_tile_normalize_lolu_moe(RM, M->moe.xpSampleWeight, gate16.P(), wide16.P(), VEC, wideScale.P(), drg.P(), TS2_F32, 1.f,
+        dgate.P(), dwide.P(), M->fastGradType, M->dExpertWeight, s));
+    // dExpertWeight was computed against rg in 1/24 units of nothing: vals*valsScale is the true normalised wide, so it is in true
+    // (scaled-gradient) units already
+    CK(ts2_backprop_moe(len, R, E, K, &M->moe, M->dExpertWeight, M->dMoeSel.P(), M->fastGradType, s));
+    // expand + gate backward into grouped rows, then back to token order
+    Arr weT = View(M->wT, E * D, X);
+    Arr sgFull = View(M->raw, RM, D);
+    CK(ts2_transpose_u8_batched(E, X, D, L.w[0].fast.m.ptr, L.w[0].fast.m.strideBytes, (int64_t)X * L.w[0].fast.m.strideBytes, weT.m.ptr,
+        weT.m.strideBytes, (int64_t)D * weT.m.strideBytes, s));
+    CK(GroupedGemm(M, dwide, weT, D, D, X, sgFull, DISCR * Dot(D), L.w[0].scale, false, s));
+    CK(ts2_transpose_u8_batched(E, X, D, L.w[1].fast.m.ptr, L.w[1].fast.m.strideBytes, (int64_t)X * L.w[1].fast.m.strideBytes, weT.m.ptr,
+        weT.m.strideBytes, (int64_t)D * weT.m.strideBytes, s));
+    CK(GroupedGemm(M, dgate, weT, D, D, X, sgFull, DISCR * Dot(D), nullptr, true, s));
+    CK(ts2_combine_experts(len, K, sgFull.P(), TS2_F32, &M->moe, 1.f, nullptr, M->dNormState.P(), 0, s));
+    // select matrix: dNormState += dMoe * Wsel / sqrt(D) and its delta through the same 8-bit operator as every other matrix (the
+    // reference uses its fp16 kernels here, MatmulSelect.BackpropFp16, layer_moe.cu:264); rows >= experts of the matrix are zero
+    CK(BackpropDX(M, L.w[3], M->dMoeSel, DISCR * Dot(D), false, M->dNormState, true, s));
+    CK(BackpropDelta(M, L.w[3], norm8, M->dMoeSel, VEC, gradScale, s));
+    // expert deltas
+    CK(GroupedDelta(M, L.w[2], rg8, M->sgMoe, VEC, gradScale, s));
+    CK(GroupedDelta(M, L.w[0], M->normMoe, dwide, VEC, gradScale, s));
+    return GroupedDelta(M, L.w[1], M->normMoe, dgate, VEC, gradScale, s);
+}
+} // namespace
+
+// ---------------------------------------------------------------------------------------------------------------------------
+// step driver
+namespace
+{
+int InitMatrix(ts2_model *M, TMatrix *W, int srcDim, int dstDim, int slabs)
+{
+    W->srcDim = srcDim;
+    W->dstDim = dstDim;
+    W->slabs = slabs;
+    if (!M->Alloc(&W->fast, dstDim * slabs, srcDim, M->mode) || !M->Alloc(&W->delta, dstDim * slabs, srcDim, TS2_I8) ||
+        !M->Alloc(&W->deltaTileScale, srcDim / 128, dstDim * slabs, TS2_F32)) {
+        return TS2_ERR_LAUNCH;
+    }
+    W->scale = (float *)M->Dev(4);
+    return W->scale ? 0 : TS2_ERR_LAUNCH;
+}
+
+int RoundUp(int x, int m)
+{
+    return (x + m - 1) / m * m;
+}
+
+int LayerForward(ts2_model *M, int d, void *s)
+{
+    TLayer &L = M->layers[d];
+    const Arr &n8 = M->normState[d];
+    if (L.type == LT_FFN) {
+        return FfnForward(M, L, n8, s);
+    } else if (L.type == LT_ATT) {
+        return AttForward(M, L, n8, s);
+    } else if (L.type == LT_MOE) {
+        return MoeForward(M, L, n8, s);
+    }
+    return TS2_ERR_UNSUPPORTED;
+}
+
+int LayerBackward(ts2_model *M, int d, const float *gradScale, void *s)
+{
+    TLayer &L = M->layers[d];
+    const Arr &n8 = M->normState[d];
+    if (L.type == LT_FFN) {
+        return FfnBackward(M, L, n8, gradScale, s);
+    } else if (L.type == LT_ATT) {
+        return AttBackward(M, L, n8, gradScale, s);
+    } else if (L.type == LT_MOE) {
+        return MoeBackward(M, L, n8, gradScale, s);
+    }
+    return TS2_ERR_UNSUPPORTED;
+}
+
+// AddForwardGraph, src/gpt/compute/gpu_transformer.cu:260-309
+int ModelForward(ts2_model *M, void *s)
+{
+    int D = M->cfg.dim, depth = (int)M->layers.size();
+    CK(Ts2EmbedForward(M->len, M->R, D, M->labelPtr, M->labels, M->embed.fast.P(), M->mode, DISCR, M->embed.scale, M->state.P(), s));
+    CK(ts2_layer_normalize_state_vecs(M->state.P(), TS2_F32, M->len, M->R, VEC, M->normState[0].P(), M->mode, M->stateScale[0].P(), s));
+    for (int d = 0; d < depth; ++d) {
+        CK(LayerForward(M, d, s));
+        CK(ts2_layer_normalize_state_vecs(M->state.P(), TS2_F32, M->len, M->R, VEC, M->normState[d + 1].P(), M->mode, M->stateScale[d + 1].P(), s));
+    }
+    return 0;
+}
+
+// final layer: src/gpt/compute/gpu_final.cuh:223-296 / cpu_transformer.cpp:119-172
+int FinalLogits(ts2_model *M, void *s)
+{
+    int D = M->cfg.dim, depth = (int)M->layers.size();
+    return Forward(M, M->finalW, M->normState[depth], VEC * DISCR * Dot(D) / LN2F, true, M->logits, false, s);
+}
+
+int FinalBackward(ts2_model *M, void *s)
+{
+    int D = M->cfg.dim, V = M->cfg.vocab, depth = (int)M->layers.size(), R = M->R;
+    CK(FinalLogits(M, s));
+    CK(Ts2ZeroRows(Flat(M->lossSum, 1, 1, TS2_F32).P(), 1, 4, s));
+    CK(Ts2FinalSoftmaxGrad(R, V, M->logits.P(), M->bias, M->target, 1.f, M->gradV.P(), M->lossSum, 0, s));
+    // dfn = grad * Wf / sqrt(D): bf16 product, the 8-bit weights converted exactly
+    CK(Ts2TransposeToBf16(V, V, D, M->finalW.fast.P(), M->mode, M->wfT.P(), s));
+    ts2_gemm_args g = {};
+    g.a = M->gradV.m;
+    g.b = M->wfT.m;
+    g.c = M->dNormState.m;
+    g.abType = TS2_BF16;
+    g.cType = TS2_F32;
+    g.m = R;
+    g.n = D;
+    g.k = V;
+    g.mLive = M->len;
+    g.alpha = DISCR * Dot(D);
+    g.alphaPtr = M->finalW.scale;
+    g.epilogue = TS2_EPI_STORE;
+    g.splitK = 1;
+    CK(ts2_gemm_nt(&g, s));
+    // delta_final[v][d] = sum_t grad[t][v] * fn[t][d]
+    CK(Ts2TransposeToBf16(M->len, R, V, M->gradV.P(), TS2_BF16, M->gradVT.P(), s));
+    CK(Ts2TransposeToBf16(M->len, R, D, M->normState[depth].P(), M->mode, M->fnT.P(), s));
+    ts2_gemm_args h = {};
+    h.a = M->gradVT.m;
+    h.b = M->fnT.m;
+    h.c = M->finalW.delta.m;
+    h.abType = TS2_BF16;
+    h.cType = TS2_I8;
+    h.m = V;
+    h.n = D;
+    h.k = R;
+    h.alpha = VEC;
+    h.epilogue = TS2_EPI_ROW_TILE_MAXNORM;
+    h.tileScale = M->finalW.deltaTileScale.m;
+    h.splitK = 1;
+    CK(ts2_gemm_nt(&h, s));
+    return ts2_backprop_final_normalize(M->len, R, M->normState[depth].P(), M->mode, M->stateScale[depth].P(), M->dNormState.P(), M->stateGrad.P(),
+        M->stateGradFast.P(), M->fastGradType, M->gradMaxNorm, s);
+}
+
+// CreateBackpropGraph, src/gpt/compute/gpu_transformer.cu:326-471 (one device, one micro batch)
+int ModelBackprop(ts2_model *M, void *s)
+{
+    int D = M->cfg.dim, depth = (int)M->layers.size();
+    CK(ModelForward(M, s));
+    CK(Ts2ZeroRows(Flat(M->gradMaxNorm, 1, depth + 2, TS2_F32).P(), 1, (depth + 2) * 4, s));
+    CK(FinalBackward(M, s));
+    int stepId = 0;
+    for (int d = depth - 1; d >= 0; --d, ++stepId) {
+        float *prevMax = M->gradMaxNorm + stepId, *nextMax = M->gradMaxNorm + stepId + 1;
+        float *gradScale = M->gradScale + stepId + 1, *gradMult = M->gradMult + stepId + 1;
+        // the fast gradient is rewritten unconditionally: its multiplier history does not survive between steps here
+        CK(ts2_scale_grad(prevMax, nullptr, M->stateGrad.P(), M->stateGradFast.P(), M->fastGradType, M->len, gradScale, gradMult, s));
+        CK(LayerBackward(M, d, gradScale, s));
+        CK(ts2_backprop_layer_normalize(M->normState[d].P(), M->mode, M->stateScale[d].P(), M->dNormState.P(), nullptr, gradScale, gradMult,
+            M->stateGrad.P(), M->stateGradFast.P(), M->fastGradType, nextMax, M->len, s));
+    }
+    return Ts2EmbedBackward(M->len, D, M->labelPtr, M->labels, M->stateGrad.P(), Flat(M->embed.delta.m.ptr, M->cfg.labelCount, D, TS2_F32).P(),
+        M->cfg.labelCount, s);
+}
+} // namespace
+
+extern "C" ts2_model *ts2_model_create(const ts2_model_config *cfg)
+{
+    if (!cfg || cfg->depth <= 0 || cfg->dim % 128 || cfg->vocab % 128 || cfg->maxLen <= 0 || (cfg->mode != TS2_I8 && cfg->mode != TS2_E4M3)) {
+        return nullptr;
+    }
+    ts2_model *M = new ts2_model();
+    M->cfg = *cfg;
+    M->mode = cfg->mode;
+    M->fastGradType = cfg->mode == TS2_I8 ? TS2_BF16 : TS2_E4M3;
+    M->kTile = cfg->kTile > 0 ? cfg->kTile : 512;
+    M->R = RoundUp(cfg->maxLen, M->kTile > 128 ? M->kTile : 128);
+    int D = cfg->dim, H = cfg->headCount, F = cfg->ffnDim, X = cfg->expertDim, E = cfg->expertCount, V = cfg->vocab, R = M->R;
+    int SelectDim = E > 0 ? RoundUp(E, 128) : 0;
+    bool hasMoe = false;
+    for (int d = 0; d < cfg->depth; ++d) {
+        M->layerType.push_back(cfg->layerType[d]);
+        M->layerAttId.push_back(cfg->layerAttId[d]);
+        M->layerSlope.push_back(cfg->layerSlope[d]);
+        hasMoe |= cfg->layerType[d] == LT_MOE;
+    }
+    if (hasMoe && (cfg->mode != TS2_E4M3 || E <= 0 || X % 128)) {
+        delete M;
+        return nullptr;
+    }
+    M->lenMoe = hasMoe ? RoundUp(R * cfg->moeSelected + 128 * E, 128) : 0;
+    M->RP = R > M->lenMoe ? R : M->lenMoe;
+    int maxW = D;
+    maxW = F > maxW ? F : maxW;
+    maxW = H * 128 > maxW ? H * 128 : maxW;
+    if (hasMoe) {
+        maxW = X > maxW ? X : maxW;
+        maxW = SelectDim > maxW ? SelectDim : maxW;
+    }
+    M->maxW = maxW;
+    bool ok = true;
+    ok &= InitMatrix(M, &M->embed, D, cfg->labelCount, 1) == 0; // delta storage reused as fp32 [labelCount][D]: allocate separately below
+    ok &= M->Alloc(&M->embed.delta, cfg->labelCount, D, TS2_F32);
+    ok &= InitMatrix(M, &M->finalW, D, V, 1) == 0;
+    M->bias = (float *)M->Dev((size_t)V * 4);
+    M->layers.resize(cfg->depth);
+    for (int d = 0; d < cfg->depth && ok; ++d) {
+        TLayer &L = M->layers[d];
+        L.type = cfg->layerType[d];
+        L.slope = cfg->layerSlope[d];
+        L.attId = cfg->layerAttId[d];
+        if (L.type == LT_ATT) {
+            for (int k = 0; k < 4; ++k) {
+                ok &= InitMatrix(M, &L.w[k], D, H * 128, 1) == 0;
+            }
+            ok &= InitMatrix(M, &L.w[4], H * 128, D, 1) == 0;
+        } else if (L.type == LT_FFN) {
+            ok &= InitMatrix(M, &L.w[0], D, F, 1) == 0;
+            ok &= InitMatrix(M, &L.w[1], D, F, 1) == 0;
+            ok &= InitMatrix(M, &L.w[2], F, D, 1) == 0;
+        } else if (L.type == LT_MOE) {
+            ok &= InitMatrix(M, &L.w[0], D, X, E) == 0;
+            ok &= InitMatrix(M, &L.w[1], D, X, E) == 0;
+            ok &= InitMatrix(M, &L.w[2], X, D, E) == 0;
+            ok &= InitMatrix(M, &L.w[3], D, SelectDim, 1) == 0;
+        } else {
+            ok = false;
+        }
+    }
+    // batch
+    M->labelCap = R * 4;
+    M->labelPtr = (int *)M->Dev((size_t)(R + 1) * 4);
+    M->labels = (uint32_t *)M->Dev((size_t)M->labelCap * 4);
+    M->target = (int *)M->Dev((size_t)R * 4);
+    for (int a = 0; a < cfg->attTypeCount; ++a) {
+        M->spanStart.push_back((int *)M->Dev((size_t)R * 4));
+        M->spanFinish.push_back((int *)M->Dev((size_t)R * 4));
+        M->revLo.push_back((int *)M->Dev((size_t)(R / 128) * 4));
+        M->revHi.push_back((int *)M->Dev((size_t)(R / 128) * 4));
+    }
+    ok &= M->Alloc(&M->rope, R, 128, TS2_F32);
+    // states
+    ok &= M->Alloc(&M->state, R, D, TS2_F32) && M->Alloc(&M->stateGrad, R, D, TS2_F32) && M->Alloc(&M->stateGradFast, R, D, M->fastGradType) &&
+          M->Alloc(&M->dNormState, R, D, TS2_F32);
+    M->normState.resize(cfg->depth + 1);
+    M->stateScale.resize(cfg->depth + 1);
+    for (int d = 0; d <= cfg->depth; ++d) {
+        ok &= M->Alloc(&M->normState[d], R, D, M->mode) && M->Alloc(&M->stateScale[d], D / 128, R, TS2_F32);
+    }
+    M->gradMaxNorm = (float *)M->Dev((size_t)(cfg->depth + 2) * 4);
+    M->gradScale = (float *)M->Dev((size_t)(cfg->depth + 2) * 4);
+    M->gradMult = (float *)M->Dev((size_t)(cfg->depth + 2) * 4);
+    M->lossSum = (float *)M->Dev(4);
+    // layer scratch
+    int RP = M->RP;
+    ok &= M->Alloc(&M->raw, RP, maxW, TS2_F32) && M->Alloc(&M->g32, RP, maxW, TS2_F32) && M->Alloc(&M->rg8, RP, maxW, M->mode);
+    for (int k = 0; k < 4; ++k) {
+        ok &= M->Alloc(&M->a16[k], RP, maxW, TS2_BF16) && M->Alloc(&M->g16[k], RP, maxW, TS2_BF16) && M->Alloc(&M->gf[k], RP, maxW, M->fastGradType);
+    }
+    for (int k = 0; k < 3; ++k) {
+        ok &= M->Alloc(&M->tsc[k], maxW / 128, RP, TS2_F32);
+    }
+    ok &= M->Alloc(&M->swl, H > 0 ? H : 1, R, TS2_F32) && M->Alloc(&M->dScale, H > 0 ? H : 1, R, TS2_F32);
+    // keep the two statistics arrays on one stride
+    M->sGrad8 = (uint8_t *)M->Dev((size_t)RP * maxW);
+    M->sGradT = (uint8_t *)M->Dev((size_t)RP * maxW);
+    M->sSrcT = (uint8_t *)M->Dev((size_t)RP * maxW);
+    M->sWT = (uint8_t *)M->Dev((size_t)maxW * maxW);
+    M->sRowScale = (float *)M->Dev((size_t)RP * 4);
+    M->sTileMax = (float *)M->Dev((size_t)(RP / 128 + 1) * 4);
+    M->sTileScale = (float *)M->Dev((size_t)(RP / 128 + 1) * 4);
+    if (hasMoe) {
+        int total = R * cfg->moeSelected;
+        M->moe.sampleExpertIds = (int *)M->Dev((size_t)total * 4);
+        M->moe.sampleExpertWeights = (float *)M->Dev((size_t)total * 4);
+        M->moe.sampleExpertOffset = (int *)M->Dev((size_t)total * 4);
+        M->moe.expertOffset = (int *)M->Dev((size_t)(E + 2) * 4);
+        M->moe.xpTileExpertId = (int *)M->Dev((size_t)(M->lenMoe / 128) * 4);
+        M->moe.xpSampleId = (int *)M->Dev((size_t)M->lenMoe * 4);
+        M->moe.xpSampleWeight = (float *)M->Dev((size_t)M->lenMoe * 4);
+        M->moe.blockCounts = (int *)M->Dev((size_t)((total + 255) / 256) * E * 4);
+        M->dExpertWeight = (float *)M->Dev((size_t)M->lenMoe * 4);
+        ok &= M->Alloc(&M->normMoe, M->lenMoe, D, M->mode) && M->Alloc(&M->sgMoe, M->lenMoe, D, M->fastGradType) &&
+              M->Alloc(&M->moeSel, R, SelectDim, TS2_F32) && M->Alloc(&M->dMoeSel, R, SelectDim, M->fastGradType);
+        int wtRows = E * (X > D ? X : D), wtCols = X > D ? X : D;
+        ok &= M->Alloc(&M->wT, wtRows, wtCols, M->mode);
+    }
+    ok &= M->Alloc(&M->logits, R, V, TS2_F32) && M->Alloc(&M->gradV, R, V, TS2_BF16) && M->Alloc(&M->gradVT, V, R, TS2_BF16) &&
+          M->Alloc(&M->fnT, D, R, TS2_BF16) && M->Alloc(&M->wfT, D, V, TS2_BF16);
+    if (!ok || !M->sGrad8 || !M->sGradT || !M->sSrcT || !M->sWT) {
+        delete M;
+        return nullptr;
+    }
+    return M;
+}
+
+extern "C" void ts2_model_destroy(ts2_model *M)
+{
+    delete M;
+}
+
+static TMatrix *FindMatrix(ts2_model *M, int layer, int matrixId)
+{
+    if (layer == TS2_LAYER_EMBED) {
+        return &M->embed;
+    }
+    if (layer == TS2_LAYER_FINAL) {
+        return &M->finalW;
+    }
+    if (layer < 0 || layer >= (int)M->layers.size() || matrixId < 0 || matrixId >= 5 || !M->layers[layer].w[matrixId].fast.m.ptr) {
+        return nullptr;
+    }
+    return &M->layers[layer].w[matrixId];
+}
+
+extern "C" int ts2_model_set_matrix(ts2_model *M, int32_t layer, int32_t matrixId, const void *fastHost, int32_t rows, int32_t cols, float scale)
+{
+    TMatrix *W = M ? FindMatrix(M, layer, matrixId) : nullptr;
+    if (!W || !fastHost) {
+        return TS2_ERR_NULL;
+    }
+    if (cols != W->srcDim || rows > W->dstDim * W->slabs) {
+        return TS2_ERR_SHAPE;
+    }
+    if (hipMemcpy2D(W->fast.m.ptr, W->fast.m.strideBytes, fastHost, cols, cols, rows, hipMemcpyHostToDevice) != hipSuccess ||
+        hipMemcpy(W->scale, &scale, 4, hipMemcpyHostToDevice) != hipSuccess) {
+        return TS2_ERR_LAUNCH;
+    }
+    return 0;
+}
+
+extern "C" int ts2_model_set_bias(ts2_model *M, const float *biasHost)
+{
+    if (!M || !biasHost) {
+        return TS2_ERR_NULL;
+    }
+    return hipMemcpy(M->bias, biasHost, (size_t)M->cfg.vocab * 4, hipMemcpyHostToDevice) == hipSuccess ? 0 : TS2_ERR_LAUNCH;
+}
+
+extern "C" int ts2_model_set_batch(ts2_model *M, int32_t len, const int32_t *labelPtr, const uint32_t *labels, const int32_t *targetPerRow,
+    const int32_t *const *spanStart, const int32_t *const *spanFinish, const float *ropeBuf, void *stream)
+{
+    if (!M || !labelPtr || !labels || !targetPerRow || !ropeBuf) {
+        return TS2_ERR_NULL;
+    }
+    if (len <= 0 || len > M->cfg.maxLen || labelPtr[len] > M->labelCap) {
+        return TS2_ERR_SHAPE;
+    }
+    M->len = len;
+    int R = M->R;
+    std::vector<int> tg(R, -1), st(R, 0), fi(R, -1);
+    memcpy(tg.data(), targetPerRow, (size_t)len * 4);
+    bool ok = hipMemcpy(M->labelPtr, labelPtr, (size_t)(len + 1) * 4, hipMemcpyHostToDevice) == hipSuccess;
+    ok &= hipMemcpy(M->labels, labels, (size_t)labelPtr[len] * 4, hipMemcpyHostToDevice) == hipSuccess;
+    ok &= hipMemcpy(M->target, tg.data(), (size_t)R * 4, hipMemcpyHostToDevice) == hipSuccess;
+    ok &= hipMemcpy2D(M->rope.m.ptr, M->rope.m.strideBytes, ropeBuf, 128 * 4, 128 * 4, len, hipMemcpyHostToDevice) == hipSuccess;
+    for (int a = 0; a < M->cfg.attTypeCount && ok; ++a) {
+        std::fill(st.begin(), st.end(), 0);
+        std::fill(fi.begin(), fi.end(), -1);
+        memcpy(st.data(), spanStart[a], (size_t)len * 4);
+        memcpy(fi.data(), spanFinish[a], (size_t)len * 4);
+        ok &= hipMemcpy(M->spanStart[a], st.data(), (size_t)R * 4, hipMemcpyHostToDevice) == hipSuccess;
+        ok &= hipMemcpy(M->spanFinish[a], fi.data(), (size_t)R * 4, hipMemcpyHostToDevice) == hipSuccess;
+        if (ok) {
+            int rc = ts2_att_build_rev(len, R, M->spanStart[a], M->spanFinish[a], M->revLo[a], M->revHi[a], stream);
+            if (rc) {
+                return rc;
+            }
+        }
+    }
+    return ok ? 0 : TS2_ERR_LAUNCH;
+}
+
+extern "C" int ts2_model_forward(ts2_model *M, void *stream)
+{
+    if (!M || M->len <= 0) {
+        return TS2_ERR_NULL;
+    }
+    CK(ModelForward(M, stream));
+    CK(FinalLogits(M, stream));
+    // probabilities in place of the logits; the gradient buffer is scratch here
+    return Ts2FinalSoftmaxGrad(M->R, M->cfg.vocab, M->logits.P(), M->bias, M->target, 1.f, M->gradV.P(), nullptr, 1, stream);
+}
+
+extern "C" int ts2_model_backprop(ts2_model *M, void *stream)
+{
+    if (!M || M->len <= 0) {
+        return TS2_ERR_NULL;
+    }
+    return ModelBackprop(M, stream);
+}
+
+extern "C" int ts2_layer_backward(ts2_model *M, int32_t layer, void *stream)
+{
+    if (!M || M->len <= 0 || layer < 0 || layer >= (int)M->layers.size()) {
+        return TS2_ERR_NULL;
+    }
+    // gradient scale bookkeeping of one step of the backward loop, fed from stateGrad as it stands
+    CK(ts2_scale_grad(M->gradMaxNorm, nullptr, M->stateGrad.P(), M->stateGradFast.P(), M->fastGradType, M->len, M->gradScale, M->gradMult, stream));
+    CK(LayerBackward(M, layer, M->gradScale, stream));
+    return ts2_backprop_layer_normalize(M->normState[layer].P(), M->mode, M->stateScale[layer].P(), M->dNormState.P(), nullptr, M->gradScale,
+        M->gradMult, M->stateGrad.P(), M->stateGradFast.P(), M->fastGradType, M->gradMaxNorm + 1, M->len, stream);
+}
+
+extern "C" int ts2_layer_forward(ts2_model *M, int32_t layer, void *stream)
+{
+    if (!M || M->len <= 0 || layer < 0 || layer >= (int)M->layers.size()) {
+        return TS2_ERR_NULL;
+    }
+    CK(ts2_layer_normalize_state_vecs(M->state.P(), TS2_F32, M->len, M->R, VEC, M->normState[layer].P(), M->mode, M->stateScale[layer].P(), stream));
+    return LayerForward(M, layer, stream);
+}
+
+extern "C" int ts2_model_get_delta(ts2_model *M, int32_t layer, int32_t matrixId, float *hostOut, int32_t rows, int32_t cols)
+{
+    TMatrix *W = M ? FindMatrix(M, layer, matrixId) : nullptr;
+    if (!W || !hostOut) {
+        return TS2_ERR_NULL;
+    }
+    if (cols != W->srcDim || rows > W->dstDim * W->slabs) {
+        return TS2_ERR_SHAPE;
+    }
+    if (hipDeviceSynchronize() != hipSuccess) {
+        return TS2_ERR_LAUNCH;
+    }
+    if (layer == TS2_LAYER_EMBED) {
+        return hipMemcpy2D(hostOut, (size_t)cols * 4, W->delta.m.ptr, W->delta.m.strideBytes, (size_t)cols * 4, rows, hipMemcpyDeviceToHost) ==
+                       hipSuccess
+                   ? 0
+                   : TS2_ERR_LAUNCH;
+    }
+    int allRows = W->dstDim * W->slabs;
+    std::vector<int8_t> d((size_t)rows * cols);
+    std::vector<float> ts((size_t)(cols / 128) * allRows);
+    if (hipMemcpy2D(d.data(), cols, W->delta.m.ptr, W->delta.m.strideBytes, cols, rows, hipMemcpyDeviceToHost) != hipSuccess ||
+        hipMemcpy2D(ts.data(), (size_t)allRows * 4, W->deltaTileScale.m.ptr, W->deltaTileScale.m.strideBytes, (size_t)allRows * 4, cols / 128,
+            hipMemcpyDeviceToHost) != hipSuccess) {
+        return TS2_ERR_LAUNCH;
+    }
+    for (int y = 0; y < rows; ++y) {
+        for (int x = 0; x < cols; ++x) {
+            hostOut[(size_t)y * cols + x] = d[(size_t)y * cols + x] * ts[(size_t)(x / 128) * allRows + y];
+        }
+    }
+    return 0;
+}
+
+extern "C" int ts2_model_array(ts2_model *M, const char *name, int32_t index, ts2_mat *out, int32_t *type)
+{
+    if (!M || !name || !out) {
+        return TS2_ERR_NULL;
+    }
+    const Arr *a = nullptr;
+    if (!strcmp(name, "state")) {
+        a = &M->state;
+    } else if (!strcmp(name, "stateGrad")) {
+        a = &M->stateGrad;
+    } else if (!strcmp(name, "stateGradFast")) {
+        a = &M->stateGradFast;
+    } else if (!strcmp(name, "dNormState")) {
+        a = &M->dNormState;
+    } else if (!strcmp(name, "prediction")) {
+        a = &M->logits;
+    } else if (!strcmp(name, "normState") && index >= 0 && index < (int)M->normState.size()) {
+        a = &M->normState[index];
+    } else if (!strcmp(name, "stateScale") && index >= 0 && index < (int)M->stateScale.size()) {
+        a = &M->stateScale[index];
+    } else {
+        return TS2_ERR_UNSUPPORTED;
+    }
+    *out = a->m;
+    if (type) {
+        *type = a->type;
+    }
+    return 0;
+}
+
+extern "C" int ts2_model_scalars(ts2_model *M, float *lossSumHost, int32_t *lenRound, int32_t *lenMoe)
+{
+    if (!M) {
+        return TS2_ERR_NULL;
+    }
+    if (lossSumHost) {
+        if (hipDeviceSynchronize() != hipSuccess || hipMemcpy(lossSumHost, M->lossSum, 4, hipMemcpyDeviceToHost) != hipSuccess) {
+            return TS2_ERR_LAUNCH;
+        }
+    }
+    if (lenRound) {
+        *lenRound = M->R;
+    }
+    if (lenMoe) {
+        *lenMoe = M->lenMoe;
+    }
+    return 0;
+}

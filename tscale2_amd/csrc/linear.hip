@@ -70,7 +70,7 @@ extern "C" int ts2_matmul_backprop(int32_t mode, int32_t len, int32_t lenRound, 
 }
 
 extern "C" int ts2_matmul_backprop_delta(int32_t mode, int32_t len, int32_t lenRound, int32_t srcDim, int32_t gradDim, const ts2_mat *src,
-    const float *srcRowScale, const ts2_mat *grad, int32_t gradType, const float *gradScale, int32_t kTile, const ts2_matmul_bwd_buffers *buf,
+    const float *srcRowScale, const ts2_mat *grad, int32_t gradType, float alpha, const float *gradScale, int32_t kTile, const ts2_matmul_bwd_buffers *buf,
     const ts2_mat *delta, const ts2_mat *deltaTileScale, void *stream)
 {
     if (!buf || !src || !grad || !delta || !deltaTileScale) {
@@ -116,7 +116,7 @@ extern "C" int ts2_matmul_backprop_delta(int32_t mode, int32_t len, int32_t lenR
     g.m = gradDim;
     g.n = srcDim;
     g.k = lenRound;
-    g.alpha = 1;
+    g.alpha = alpha;
     g.alphaPtr = gradScale;
     g.epilogue = TS2_EPI_ROW_TILE_MAXNORM;
     g.tileScale = *deltaTileScale;

@@ -1,0 +1,205 @@
+// Kernels around the layer stack: label embedding, final soft-max / loss gradient and 16-bit transposed copies for the
+// final layer's bf16 products (the reference runs them in fp16: src/gpt/compute/gpu_final.cuh:223-296, gpu_embedding.cuh:126-218).
+#include "vec.h"
+#include "internal.h"
+
+namespace
+{
+// state0[t] = sum over labels of +-E[label] * scale (ComputeEmbedding, src/gpt/compute/cpu_transformer.cpp:76-100); one workgroup per row
+template <class TEmb>
+__global__ void __launch_bounds__(256) EmbedForward(int len, int dim, const int *labelPtr, const uint32_t *labels, const uint8_t *embed,
+    int64_t ldEmb, float mult, const float *scalePtr, float *state, int64_t ldState)
+{
+    int t = blockIdx.x;
+    float s = mult * (scalePtr ? *scalePtr : 1.f);
+    for (int col = threadIdx.x * 4; col < dim; col += 1024) {
+        F4 acc = ZeroF4();
+        if (t < len) {
+            for (int k = labelPtr[t]; k < labelPtr[t + 1]; ++k) {
+                uint32_t label = labels[k];
+                float w = (label & 0x80000000u) ? -s : s;
+                label &= 0x7fffffffu;
+                acc = acc + Load4<TEmb>(embed + (int64_t)label * ldEmb + col * TEmb::SIZE) * w;
+            }
+        }
+        Store4<TF32>((uint8_t *)state + (int64_t)t * ldState + col * 4, acc);
+    }
+}
+
+// deltaLabel[label] += +-grad[t]  (src/gpt/compute/cpu_transformer.cpp:182-197); fp32 atomics, delta cleared by the caller
+__global__ void __launch_bounds__(256) EmbedBackward(int len, int dim, const int *labelPtr, const uint32_t *labels, const float *grad, int64_t ldGrad,
+    float *delta, int64_t ldDelta)
+{
+    int t = blockIdx.x;
+    for (int k = labelPtr[t]; k < labelPtr[t + 1]; ++k) {
+        uint32_t label = labels[k];
+        float w = (label & 0x80000000u) ? -1.f : 1.f;
+        label &= 0x7fffffffu;
+        for (int col = threadIdx.x; col < dim; col += 256) {
+            atomicAdd(delta + (int64_t)label * ldDelta / 4 + col, grad[(int64_t)t * ldGrad / 4 + col] * w);
+        }
+    }
+}
+
+// SoftMax base 2 with running max starting at 0 and the (onehot - p) gradient (src/gpt/compute/cpu_transformer.cpp:12-37,146-159).
+// One workgroup per row; logits fp32 [row][vocab] are overwritten by probabilities when keepProb, grad is bf16.
+__global__ void __launch_bounds__(256) FinalSoftmaxGrad(int vocab, float *logits, int64_t ldLogits, const float *bias, const int *target,
+    float gradMult, bf16_t *grad, int64_t ldGrad, float *lossSum, int keepProb)
+{
+    __shared__ float red[4];
+    __shared__ float bc;
+    int t = blockIdx.x;
+    int tid = threadIdx.x;
+    float *row = (float *)((uint8_t *)logits + (int64_t)t * ldLogits);
+    bf16_t *grow = (bf16_t *)((uint8_t *)grad + (int64_t)t * ldGrad);
+    int tg = target[t];
+    if (tg < 0) {
+        for (int k = tid; k < vocab; k += 256) {
+            grow[k] = 0;
+        }
+        if (!keepProb) {
+            return;
+        }
+    }
+    float mx = 0;
+    for (int k = tid; k < vocab; k += 256) {
+        mx = fmaxf(mx, row[k]);
+    }
+    mx = WaveMax(mx);
+    if ((tid & 63) == 0) {
+        red[tid >> 6] = mx;
+    }
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    float sum = 0;
+    for (int k = tid; k < vocab; k += 256) {
+        sum += exp2f(row[k] + bias[k] - mx);
+    }
+    sum = WaveSum(sum);
+    if ((tid & 63) == 0) {
+        red[tid >> 6] = sum;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        bc = 1 / ((red[0] + red[1]) + (red[2] + red[3]));
+    }
+    __syncthreads();
+    float scale = bc;
+    for (int k = tid; k < vocab; k += 256) {
+        float p = exp2f(row[k] + bias[k] - mx) * scale;
+        if (keepProb) {
+            row[k] = p;
+        }
+        if (tg >= 0) {
+            float g = (k == tg ? 1.f : 0.f) - p;
+            grow[k] = FloatToBf16(g * gradMult);
+            if (k == tg && lossSum) {
+                atomicAdd(lossSum, logf(p));
+            }
+        }
+    }
+}
+
+// dst[x][t] = bf16(src[t][x]) for t < rows, 0 up to rowsRound; 64x64 tiles through LDS
+template <class TSrc>
+__global__ void __launch_bounds__(256) TransposeToBf16(int rows, int rowsRound, int cols, const uint8_t *src, int64_t ldSrc, uint8_t *dst, int64_t ldDst)
+{
+    __shared__ float tile[64][65];
+    int x0 = blockIdx.x * 64, t0 = blockIdx.y * 64;
+    int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int r = ty; r < 64; r += 4) {
+        int t = t0 + r, x = x0 + tx;
+        float v = 0;
+        if (t < rows && x < cols) {
+            const uint8_t *p = src + (int64_t)t * ldSrc + (int64_t)x * TSrc::SIZE;
+            if (TSrc::SIZE == 2) {
+                v = Bf16ToFloat(*(const bf16_t *)p);
+            } else if (std::is_same<TSrc, TI8>::value) {
+                v = (float)*(const int8_t *)p;
+            } else {
+                v = __builtin_amdgcn_cvt_f32_fp8((int)*p, 0);
+            }
+        }
+        tile[r][tx] = v;
+    }
+    __syncthreads();
+    for (int r = ty; r < 64; r += 4) {
+        int x = x0 + r, t = t0 + tx;
+        if (x < cols && t < rowsRound) {
+            *(bf16_t *)(dst + (int64_t)x * ldDst + (int64_t)t * 2) = FloatToBf16(tile[tx][r]);
+        }
+    }
+}
+
+__global__ void ZeroBytes(uint8_t *p, int64_t ld, int rowBytes)
+{
+    uint8_t *row = p + (int64_t)blockIdx.x * ld;
+    for (int x = threadIdx.x * 4; x < rowBytes; x += blockDim.x * 4) {
+        *(uint32_t *)(row + x) = 0;
+    }
+}
+} // namespace
+
+#define STREAM ((hipStream_t)stream)
+
+int Ts2EmbedForward(int len, int lenRound, int dim, const int *labelPtr, const uint32_t *labels, const ts2_mat *embed, int embType, float mult,
+    const float *scalePtr, const ts2_mat *state, void *stream)
+{
+    if (embType == TS2_I8) {
+        hipLaunchKernelGGL((EmbedForward<TI8>), dim3(lenRound), dim3(256), 0, STREAM, len, dim, labelPtr, labels, (const uint8_t *)embed->ptr,
+            embed->strideBytes, mult, scalePtr, (float *)state->ptr, state->strideBytes);
+    } else if (embType == TS2_E4M3) {
+        hipLaunchKernelGGL((EmbedForward<TE4M3>), dim3(lenRound), dim3(256), 0, STREAM, len, dim, labelPtr, labels, (const uint8_t *)embed->ptr,
+            embed->strideBytes, mult, scalePtr, (float *)state->ptr, state->strideBytes);
+    } else {
+        return TS2_ERR_UNSUPPORTED;
+    }
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
+int Ts2EmbedBackward(int len, int dim, const int *labelPtr, const uint32_t *labels, const ts2_mat *grad, const ts2_mat *delta, int labelCount,
+    void *stream)
+{
+    hipLaunchKernelGGL(ZeroBytes, dim3(labelCount), dim3(256), 0, STREAM, (uint8_t *)delta->ptr, delta->strideBytes, dim * 4);
+    TS2_CHECK_LAUNCH();
+    hipLaunchKernelGGL(EmbedBackward, dim3(len), dim3(256), 0, STREAM, len, dim, labelPtr, labels, (const float *)grad->ptr, grad->strideBytes,
+        (float *)delta->ptr, delta->strideBytes);
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
+int Ts2FinalSoftmaxGrad(int rows, int vocab, const ts2_mat *logits, const float *bias, const int *target, float gradMult, const ts2_mat *grad,
+    float *lossSum, int keepProb, void *stream)
+{
+    hipLaunchKernelGGL(FinalSoftmaxGrad, dim3(rows), dim3(256), 0, STREAM, vocab, (float *)logits->ptr, logits->strideBytes, bias, target, gradMult,
+        (bf16_t *)grad->ptr, grad->strideBytes, lossSum, keepProb);
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
+int Ts2TransposeToBf16(int rows, int rowsRound, int cols, const ts2_mat *src, int srcType, const ts2_mat *dst, void *stream)
+{
+    dim3 grid((cols + 63) / 64, (rowsRound + 63) / 64);
+    const uint8_t *s = (const uint8_t *)src->ptr;
+    uint8_t *d = (uint8_t *)dst->ptr;
+    if (srcType == TS2_I8) {
+        hipLaunchKernelGGL((TransposeToBf16<TI8>), grid, dim3(256), 0, STREAM, rows, rowsRound, cols, s, src->strideBytes, d, dst->strideBytes);
+    } else if (srcType == TS2_E4M3) {
+        hipLaunchKernelGGL((TransposeToBf16<TE4M3>), grid, dim3(256), 0, STREAM, rows, rowsRound, cols, s, src->strideBytes, d, dst->strideBytes);
+    } else if (srcType == TS2_BF16) {
+        hipLaunchKernelGGL((TransposeToBf16<TBF16>), grid, dim3(256), 0, STREAM, rows, rowsRound, cols, s, src->strideBytes, d, dst->strideBytes);
+    } else {
+        return TS2_ERR_UNSUPPORTED;
+    }
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
+int Ts2ZeroRows(const ts2_mat *m, int rows, int rowBytes, void *stream)
+{
+    hipLaunchKernelGGL(ZeroBytes, dim3(rows), dim3(256), 0, STREAM, (uint8_t *)m->ptr, m->strideBytes, rowBytes);
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}

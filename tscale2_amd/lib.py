@@ -18,7 +18,8 @@ class GemmArgs(C.Structure):
     _fields_ = [("a", Mat), ("b", Mat), ("c", Mat), ("abType", C.c_int32), ("cType", C.c_int32), ("m", C.c_int32), ("n", C.c_int32),
                 ("k", C.c_int32), ("mLive", C.c_int32), ("rowScale", C.c_void_p), ("kTileScale", C.c_void_p), ("kTile", C.c_int32),
                 ("alpha", C.c_float), ("alphaPtr", C.c_void_p), ("epilogue", C.c_int32), ("tileScale", Mat), ("splitK", C.c_int32),
-                ("tileConfig", C.c_int32)]
+                ("tileConfig", C.c_int32), ("tileGroup", C.c_void_p), ("bSlabBytes", C.c_int64), ("groupOffsets", C.c_void_p),
+                ("groups", C.c_int32), ("cSlabBytes", C.c_int64), ("tileScaleSlabBytes", C.c_int64)]
 
 
 def mat(t):
@@ -53,11 +54,15 @@ class Lib:
             raise RuntimeError(f"{what} failed with code {rc}")
 
     def gemm_nt(self, a, b, c, ab_type, c_type, row_scale=None, k_tile_scale=None, k_tile=0, alpha=1.0, alpha_ptr=None,
-                epilogue=EPI_STORE, tile_scale=None, split_k=1, m_live=0, tile_config=0, k=None, check=True):
+                epilogue=EPI_STORE, tile_scale=None, split_k=1, m_live=0, tile_config=0, k=None, check=True, m=None, n=None,
+                tile_group=None, b_slab_bytes=0, group_offsets=None, groups=0, c_slab_bytes=0, tile_scale_slab_bytes=0):
         args = GemmArgs()
         args.a, args.b, args.c = mat(a), mat(b), mat(c)
         args.abType, args.cType = ab_type, c_type
-        args.m, args.n = a.shape[0], b.shape[0]
+        args.m = a.shape[0] if m is None else m
+        args.n = b.shape[0] if n is None else n
+        args.tileGroup, args.bSlabBytes = ptr(tile_group), b_slab_bytes
+        args.groupOffsets, args.groups, args.cSlabBytes, args.tileScaleSlabBytes = ptr(group_offsets), groups, c_slab_bytes, tile_scale_slab_bytes
         args.k = a.shape[1] if k is None else k
         args.mLive = m_live
         args.rowScale = ptr(row_scale)
@@ -154,9 +159,9 @@ class MatMulBuffers:
         call("ts2_matmul_backprop", self.mode, len_, self.len_round, self.src_dim, self.grad_dim, grad, C.byref(self.c), float(alpha), alpha_ptr,
              src_grad, src_grad_type, int(add))
 
-    def backprop_delta(self, len_, src, src_row_scale, grad, grad_type, grad_scale=None):
+    def backprop_delta(self, len_, src, src_row_scale, grad, grad_type, grad_scale=None, alpha=1.0):
         call("ts2_matmul_backprop_delta", self.mode, len_, self.len_round, self.src_dim, self.grad_dim, src, src_row_scale, grad, grad_type,
-             grad_scale, self.k_tile, C.byref(self.c), self.delta, self.delta_tile_scale)
+             float(alpha), grad_scale, self.k_tile, C.byref(self.c), self.delta, self.delta_tile_scale)
 
     def delta_fp32(self):
         """dequantised packed delta [gradDim][srcDim]"""
@@ -191,3 +196,105 @@ def att_backward(len_, heads, q, k, v, dval, span_start, span_finish, rev_lo, re
                     grad_type, which)
     lib = load()
     lib.check(lib.dll.ts2_att_backward(C.byref(a), lib.stream()), "ts2_att_backward")
+
+
+class ModelConfig(C.Structure):
+    _fields_ = [("mode", C.c_int32), ("dim", C.c_int32), ("headCount", C.c_int32), ("ffnDim", C.c_int32), ("expertDim", C.c_int32),
+                ("expertCount", C.c_int32), ("moeSelected", C.c_int32), ("depth", C.c_int32), ("layerType", C.c_void_p),
+                ("layerAttId", C.c_void_p), ("layerSlope", C.c_void_p), ("attTypeCount", C.c_int32), ("vocab", C.c_int32),
+                ("labelCount", C.c_int32), ("maxLen", C.c_int32), ("kTile", C.c_int32)]
+
+
+LAYER_EMBED, LAYER_FINAL = -1, -2
+
+
+class Model:
+    """Step driver object of the library (ts2_model_*): owns device buffers, runs forward / backprop of a layer stack."""
+
+    def __init__(self, mode, dim, heads, ffn_dim, layer_type, layer_att_id, layer_slope, att_type_count, vocab, label_count, max_len,
+                 expert_dim=0, expert_count=0, moe_selected=0, k_tile=0):
+        import numpy as np
+        self.lib = load()
+        dll = self.lib.dll
+        dll.ts2_model_create.restype = C.c_void_p
+        self._lt = np.ascontiguousarray(layer_type, np.int32)
+        self._la = np.ascontiguousarray(layer_att_id, np.int32)
+        self._ls = np.ascontiguousarray(layer_slope, np.float32)
+        cfg = ModelConfig(mode, dim, heads, ffn_dim, expert_dim, expert_count, moe_selected, len(self._lt), self._lt.ctypes.data,
+                          self._la.ctypes.data, self._ls.ctypes.data, att_type_count, vocab, label_count, max_len, k_tile)
+        self.h = dll.ts2_model_create(C.byref(cfg))
+        if not self.h:
+            raise RuntimeError("ts2_model_create failed")
+        self.h = C.c_void_p(self.h)
+        self.att_type_count = att_type_count
+
+    def close(self):
+        if self.h:
+            self.lib.dll.ts2_model_destroy(self.h)
+            self.h = None
+
+    def _ck(self, rc, what):
+        if rc != 0:
+            raise RuntimeError(f"{what} failed with code {rc}")
+
+    def set_matrix(self, layer, matrix_id, fast, scale):
+        import numpy as np
+        fast = np.ascontiguousarray(fast)
+        self._ck(self.lib.dll.ts2_model_set_matrix(self.h, layer, matrix_id, fast.ctypes.data_as(C.c_void_p), fast.shape[0], fast.shape[1],
+                                                   C.c_float(scale)), "ts2_model_set_matrix")
+
+    def set_bias(self, bias):
+        import numpy as np
+        b = np.ascontiguousarray(bias, np.float32)
+        self._ck(self.lib.dll.ts2_model_set_bias(self.h, b.ctypes.data_as(C.c_void_p)), "ts2_model_set_bias")
+
+    def set_batch(self, label_ptr, labels, target_per_row, span_start, span_finish, rope):
+        import numpy as np
+        lp = np.ascontiguousarray(label_ptr, np.int32); lb = np.ascontiguousarray(labels, np.uint32)
+        tg = np.ascontiguousarray(target_per_row, np.int32); rp = np.ascontiguousarray(rope, np.float32)
+        ss = [np.ascontiguousarray(a, np.int32) for a in span_start]; sf = [np.ascontiguousarray(a, np.int32) for a in span_finish]
+        pa = (C.c_void_p * len(ss))(*[a.ctypes.data for a in ss]); pf = (C.c_void_p * len(sf))(*[a.ctypes.data for a in sf])
+        self._ck(self.lib.dll.ts2_model_set_batch(self.h, len(tg), lp.ctypes.data_as(C.c_void_p), lb.ctypes.data_as(C.c_void_p),
+                                                  tg.ctypes.data_as(C.c_void_p), pa, pf, rp.ctypes.data_as(C.c_void_p), self.lib.stream()),
+                 "ts2_model_set_batch")
+
+    def forward(self):
+        self._ck(self.lib.dll.ts2_model_forward(self.h, self.lib.stream()), "ts2_model_forward")
+
+    def backprop(self):
+        self._ck(self.lib.dll.ts2_model_backprop(self.h, self.lib.stream()), "ts2_model_backprop")
+
+    def layer_forward(self, layer):
+        self._ck(self.lib.dll.ts2_layer_forward(self.h, layer, self.lib.stream()), "ts2_layer_forward")
+
+    def layer_backward(self, layer):
+        self._ck(self.lib.dll.ts2_layer_backward(self.h, layer, self.lib.stream()), "ts2_layer_backward")
+
+    def get_delta(self, layer, matrix_id, rows, cols):
+        import numpy as np
+        out = np.empty((rows, cols), np.float32)
+        self._ck(self.lib.dll.ts2_model_get_delta(self.h, layer, matrix_id, out.ctypes.data_as(C.c_void_p), rows, cols), "ts2_model_get_delta")
+        return out
+
+    def array(self, name, index=0):
+        """torch view (no copy) of an internal device array"""
+        import torch
+        m = Mat(); t = C.c_int32(0)
+        self._ck(self.lib.dll.ts2_model_array(self.h, name.encode(), index, C.byref(m), C.byref(t)), "ts2_model_array")
+        dt = {I8: torch.int8, E4M3: torch.uint8, BF16: torch.bfloat16, F32: torch.float32}[t.value]
+        es = {I8: 1, E4M3: 1, BF16: 2, F32: 4}[t.value]
+        n = m.strideBytes // es * m.y
+
+        class _Holder:
+            __cuda_array_interface__ = {"shape": (n,), "typestr": {1: "|u1", 2: "<u2", 4: "<f4"}[es], "data": (m.ptr, False), "version": 2}
+        flat = torch.as_tensor(_Holder(), device="cuda")
+        if dt == torch.bfloat16:
+            flat = flat.view(torch.int16).view(torch.bfloat16)
+        elif dt == torch.int8:
+            flat = flat.view(torch.int8)
+        return flat.view(m.y, m.strideBytes // es)[:, :m.x]
+
+    def loss_sum(self):
+        v = C.c_float(0)
+        self._ck(self.lib.dll.ts2_model_scalars(self.h, C.byref(v), None, None), "ts2_model_scalars")
+        return v.value
