@@ -125,7 +125,151 @@ def bench_linear_i8(args):
     return out
 
 
-WORKLOADS = {"linear_i8_bwd": bench_linear_i8}
+def _fast_weights(torch, rows, cols, mode_e4m3, gen):
+    """random per-matrix quantised weights: N(0,1) * 32 in the 8-bit type (fast = w / (rms/32)), matrix scale 0.02"""
+    w = torch.randn((rows, cols), device="cuda", generator=gen) * 32
+    if mode_e4m3:
+        return w.to(torch.float8_e4m3fn).view(torch.uint8).cpu().numpy(), 0.02
+    return torch.clamp(torch.round(w), -128, 127).to(torch.int8).cpu().numpy(), 0.02
+
+
+def bench_step_fp8(args):
+    """BASELINE config[2]: e2048 h16 d12 ffn64 w1024 (24 layers), vocab 50304, 32 sequences x 1024 tokens, e4m3 weights/states/gradients,
+    bf16 activations.  One step = forward + loss gradient + backward through all layers with every delta (no optimiser)."""
+    import numpy as np
+    import torch
+    from model_harness import LT_ATT, layer_shapes, schedule
+    from oracle_lib import Oracle
+    from tscale2_amd import lib as L
+    L.load()
+    orc = Oracle()
+    dim, heads, ffn, depth, vocab, frags, frag_len, wide = 2048, 16, 8192, 12, 50304, 32, 1024, 1024
+    if args.small:
+        dim, heads, ffn, depth, vocab, frags, frag_len, wide = 512, 4, 2048, 4, 1024, 8, 512, 512
+    lt, la, ls, aw = schedule(orc, depth, 0, wide)
+    n = frags * frag_len
+    m = L.Model(L.E4M3, dim, heads, ffn, lt, la, ls, len(aw), vocab, vocab + 1, n)
+    gen = torch.Generator(device="cuda").manual_seed(2)
+    params = 0
+    for d in range(len(lt)):
+        for i, (rows, cols) in enumerate(layer_shapes(int(lt[d]), dim, heads, ffn, 0, 0)):
+            fast, sc = _fast_weights(torch, rows, cols, True, gen)
+            m.set_matrix(d, i, fast, sc)
+            params += rows * cols
+    fast, sc = _fast_weights(torch, vocab + 1, dim, True, gen)
+    m.set_matrix(L.LAYER_EMBED, 0, fast, sc)
+    fast, sc = _fast_weights(torch, vocab, dim, True, gen)
+    m.set_matrix(L.LAYER_FINAL, 0, fast, sc)
+    params += vocab * dim
+    m.set_bias(np.zeros(vocab, np.float32))
+    r = np.random.default_rng(3)
+    tokens = r.integers(0, vocab, (frags, frag_len))
+    tg = np.full((frags, frag_len), -1, np.int32); tg[:, :-1] = tokens[:, 1:]
+    t = np.arange(n, dtype=np.int32); frag0 = (t // frag_len) * frag_len
+    starts = [np.maximum(frag0, t - int(w)).astype(np.int32) for w in aw]
+    finishes = [(t - 1).astype(np.int32) for _ in aw]
+    for a in range(len(aw)):
+        finishes[a][t == frag0] = -1
+    m.set_batch(np.arange(n + 1, dtype=np.int32), (1 + tokens).astype(np.uint32).ravel(), tg.ravel(), starts, finishes, orc.fill_rope_buf(128, n))
+    for _ in range(args.warmup):
+        m.backprop()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        m.backprop()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    loss = m.loss_sum() / (tg >= 0).sum()
+    assert np.isfinite(loss), "loss is not finite"
+    # useful work: 6 flop per matmul parameter and token + causal attention (2 fwd + 5 bwd products of S*S/2 x 128 per head)
+    att_layers = int((lt == LT_ATT).sum())
+    att = 0.0
+    for d in range(len(lt)):
+        if lt[d] == LT_ATT:
+            w = int(aw[la[d]])
+            pairs = sum(min(i, w) for i in range(frag_len)) * frags
+            att += 7 * 2.0 * pairs * 128 * heads
+    flop = 6.0 * params * n + att
+    # dominant kernel: the e4m3 GEMM, timed alone on the biggest backward shape of the model (dX of the FFN expand: M=tokens, K=ffn, N=dim)
+    a = torch.randint(0, 120, (n, ffn), dtype=torch.uint8, device="cuda"); b = torch.randint(0, 120, (dim, ffn), dtype=torch.uint8, device="cuda")
+    c = torch.empty((n, dim), dtype=torch.float32, device="cuda")
+    lib = L.load()
+    ms_g = event_time_ms(lambda: lib.gemm_nt(a, b, c, L.E4M3, L.F32), 10)
+    gops = 2.0 * n * ffn * dim
+    roof = {"bound": "mfma", "achieved": gops / (ms_g * 1e-3) / 1e12, "peak": PEAK_FP8 / 1e12, "unit": "TFLOP/s",
+            "frac": gops / (ms_g * 1e-3) / PEAK_FP8, "traffic": None,
+            "kernel": "GemmNT<e4m3> %dx%dx%d (%.1f us per launch)" % (n, dim, ffn, ms_g * 1e3)}
+    out = {"metric": "fwd+bwd tokens/sec on 1 MI355X; bwd GEMM TFLOPS as % of MFMA peak", "value": n / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1,
+           "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "fp8_e4m3", "data": "synthetic",
+           "config": {"workload": "dense GPT fwd+bwd step, e%dh%dd%dffn%dw%d (%d layers), vocab %d, %d x %d tokens, e4m3 matmuls, bf16 activations"
+                                  % (dim, heads, depth, ffn // 128, wide, len(lt), vocab, frags, frag_len),
+                      "tokens_per_step": n, "matmul_params": params, "useful_tflop_per_step": flop / 1e12},
+           "step_tflops": flop / (ms * 1e-3) / 1e12, "bwd_gemm_pct_of_peak": 100 * roof["frac"], "loss": loss, "roofline": roof}
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline_step(orc, dim, heads, ffn, lt, la, ls, aw, vocab)
+    m.close()
+    return out
+
+
+def cpu_baseline_step(orc, dim, heads, ffn, lt, la, ls, aw, vocab):
+    """the oracle's full step (the reference's CPU ComputeBackprop restated) on a bounded sample of the same model: one layer pair
+    (attention + FFN) of the real width on 256 tokens, extrapolated per token and per layer"""
+    import numpy as np
+    from model_harness import Harness
+    cores = min(len(os.sched_getaffinity(0)), 16)
+    os.environ["OMP_NUM_THREADS"] = str(cores)
+    h = Harness(1, dim=dim, heads=heads, ffn_tiles=ffn // 128, depth=1, vocab=256, frag_count=2, frag_len=128, wide_window=128, seed=1)
+    t0 = time.perf_counter()
+    h.oracle_step()
+    dt = time.perf_counter() - t0
+    layers_full = len(lt)
+    # depth=1 schedule = 1 attention + 1 ffn layer; the full model has layers_full/2 such pairs; the head (vocab) is left out of the sample
+    tok_s = h.n / (dt * layers_full / 2)
+    return {"value": tok_s, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": "one attention+FFN layer pair of the full width on %d tokens (%.1f s), scaled by %d layer pairs; final layer excluded"
+                      % (h.n, dt, layers_full // 2)}
+
+
+def bench_att_bwd(args):
+    """BASELINE config[3]: causal attention backward alone, 16 sequences x 2048, 16 heads x 128, bf16"""
+    import torch
+    from tscale2_amd import lib as L
+    L.load()
+    B, S, H = 16, 2048, 16
+    n = B * S
+    i16 = torch.int16
+    gen = torch.Generator(device="cuda").manual_seed(4)
+    q, k, v, do = [torch.randn((n, H * 128), device="cuda", generator=gen).bfloat16() for _ in range(4)]
+    t = torch.arange(n, device="cuda", dtype=torch.int32)
+    start = ((t // S) * S).int().contiguous()
+    finish = torch.where(t - 1 >= start, t - 1, torch.full_like(t, -1)).int().contiguous()
+    val = torch.empty_like(q); swl = torch.empty((H, n), device="cuda"); ds = torch.zeros((H, n), device="cuda")
+    rl = torch.zeros(n // 128, dtype=torch.int32, device="cuda"); rh = torch.zeros_like(rl)
+    L.call("ts2_att_build_rev", n, n, start, finish, rl, rh)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+    sc = 0.0637
+    L.att_forward(n, H, q.view(i16), k.view(i16), v.view(i16), start, finish, sc, 0.0, val.view(i16), swl)
+    ds.copy_((val.float() * do.float()).view(n, H, 128).sum(-1).t())
+
+    def step():
+        L.att_backward(n, H, q.view(i16), k.view(i16), v.view(i16), do.view(i16), start, finish, rl, rh, sc, 0.0, swl, ds, dq.view(i16), dk.view(i16),
+                       dv.view(i16), L.BF16, 3)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ms = event_time_ms(step, args.steps)
+    pairs = B * H * (S * (S - 1) / 2)
+    flop5 = 5 * 2.0 * pairs * 128
+    roof = {"bound": "mfma", "achieved": flop5 / (ms * 1e-3) / 1e12, "peak": PEAK_BF16 / 1e12, "unit": "TFLOP/s", "frac": flop5 / (ms * 1e-3) / PEAK_BF16,
+            "traffic": None, "kernel": "AttGradQ + AttGradKV, 5-product causal count (7 products executed)"}
+    return {"metric": "fwd+bwd tokens/sec on 1 MI355X; bwd GEMM TFLOPS as % of MFMA peak", "value": n / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16", "data": "synthetic", "config": {"workload": "causal attention backward, 16 x 2048 tokens, 16 heads x 128, bf16"},
+            "roofline": roof}
+
+
+WORKLOADS = {"linear_i8_bwd": bench_linear_i8, "step_fp8": bench_step_fp8, "att_bwd": bench_att_bwd}
 
 
 def main():
@@ -135,6 +279,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="linear_i8_bwd", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--small", action="store_true", help="step_fp8: a reduced model for quick checks (not a valid benchmark figure)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the path has no multi-GPU leg); use --gpus 1", file=sys.stderr)

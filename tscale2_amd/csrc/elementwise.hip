@@ -78,42 +78,56 @@ __global__ void __launch_bounds__(256) LayerNormalizeStateVecs(int len, int lenR
     }
 }
 
+// Every workgroup walks many (row, tile) units and issues ONE atomic max at the end: one atomic per unit (the reference's scheme,
+// gpu_layer_norm.cuh:111-114) serialises half a million updates of a single address at this problem size.
 template <class TNorm, class TFast, bool FINAL>
 __global__ void __launch_bounds__(256) BackpropLayerNormalize(int len, int rows, int tiles, Mat normState, Mat stateScale, Mat dNormState,
     const float *combinerScale, const float *gradScale, const float *gradMult, Mat stateGrad, Mat stateGradFast, float *nextMaxNorm)
 {
-    int t, tile, h;
-    if (!Unit(rows, tiles, &t, &tile, &h)) {
-        return;
-    }
-    int col = tile * TILE + h * 4;
-    if (t >= len) {
-        Store4<TF32>(At<TF32>(stateGrad, t, col), ZeroF4());
-        Store4<TFast>(At<TFast>(stateGradFast, t, col), ZeroF4());
-        return;
-    }
-    F4 vec = Load4<TNorm>(At<TNorm>(normState, t, col)) * ScaleAt(stateScale, tile, t);
-    F4 grad = Load4<TF32>(At<TF32>(dNormState, t, col));
+    __shared__ float red[8];
+    const int h = threadIdx.x & 31;
+    const long units = (long)rows * tiles;
+    float s = 1;
     if (!FINAL) {
-        float s = 1;
         if (combinerScale) {
             s *= *combinerScale;
         }
         if (gradScale) {
             s *= *gradScale;
         }
-        grad = grad * s;
     }
-    grad = TileNormBackprop(vec, grad);
-    if (!FINAL) {
-        grad = grad + Load4<TF32>(At<TF32>(stateGrad, t, col));
+    const float gm = (!FINAL && gradMult) ? *gradMult : 1.f;
+    float gmax = 0;
+    for (long u = ((long)blockIdx.x * 256 + threadIdx.x) >> 5; u < units; u += (long)gridDim.x * 8) {
+        int t = (int)(u / tiles);
+        int tile = (int)(u - (long)t * tiles);
+        int col = tile * TILE + h * 4;
+        if (t >= len) {
+            Store4<TF32>(At<TF32>(stateGrad, t, col), ZeroF4());
+            Store4<TFast>(At<TFast>(stateGradFast, t, col), ZeroF4());
+            continue;
+        }
+        F4 vec = Load4<TNorm>(At<TNorm>(normState, t, col)) * ScaleAt(stateScale, tile, t);
+        F4 grad = Load4<TF32>(At<TF32>(dNormState, t, col));
+        if (!FINAL) {
+            grad = grad * s;
+        }
+        grad = TileNormBackprop(vec, grad);
+        if (!FINAL) {
+            grad = grad + Load4<TF32>(At<TF32>(stateGrad, t, col));
+        }
+        gmax = fmaxf(gmax, HMaxAbs(grad));
+        Store4<TF32>(At<TF32>(stateGrad, t, col), grad);
+        Store4<TFast>(At<TFast>(stateGradFast, t, col), grad * gm);
     }
-    float gmax = Half32Max(HMaxAbs(grad));
-    Store4<TF32>(At<TF32>(stateGrad, t, col), grad);
-    float gm = (!FINAL && gradMult) ? *gradMult : 1.f;
-    Store4<TFast>(At<TFast>(stateGradFast, t, col), grad * gm);
-    if (h == 0 && nextMaxNorm) {
-        AtomicMaxPos(nextMaxNorm, gmax);
+    gmax = Half32Max(gmax);
+    if (h == 0) {
+        red[threadIdx.x >> 5] = gmax;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0 && nextMaxNorm) {
+        float m = fmaxf(fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])), fmaxf(fmaxf(red[4], red[5]), fmaxf(red[6], red[7])));
+        AtomicMaxPos(nextMaxNorm, m);
     }
 }
 
@@ -476,12 +490,14 @@ static int BackpropNormImpl(bool final, int len, int rows, const ts2_mat *normSt
         return TS2_ERR_UNSUPPORTED;
     }
     int tiles = dim / TILE;
+    long nUnits = (long)rows * tiles;
+    dim3 bnGrid((unsigned)((nUnits + 7) / 8 < 4096 ? (nUnits + 7) / 8 : 4096));
 #define LAUNCH_BN(TN, TFA)                                                                                                                 \
     if (final)                                                                                                                             \
-        hipLaunchKernelGGL((BackpropLayerNormalize<TN, TFA, true>), GridFor(rows, tiles), dim3(256), 0, STREAM, len, rows, tiles,         \
+        hipLaunchKernelGGL((BackpropLayerNormalize<TN, TFA, true>), bnGrid, dim3(256), 0, STREAM, len, rows, tiles,         \
             M(*normState), M(*stateScale), M(*dNormState), combinerScale, gradScale, gradMult, M(*stateGrad), M(*stateGradFast), nextMaxNorm); \
     else                                                                                                                                   \
-        hipLaunchKernelGGL((BackpropLayerNormalize<TN, TFA, false>), GridFor(rows, tiles), dim3(256), 0, STREAM, len, rows, tiles,        \
+        hipLaunchKernelGGL((BackpropLayerNormalize<TN, TFA, false>), bnGrid, dim3(256), 0, STREAM, len, rows, tiles,        \
             M(*normState), M(*stateScale), M(*dNormState), combinerScale, gradScale, gradMult, M(*stateGrad), M(*stateGradFast), nextMaxNorm)
     if (fastType == TS2_BF16) {
         TS2_DISPATCH_TYPE(normType, TN, LAUNCH_BN(TN, TBF16));

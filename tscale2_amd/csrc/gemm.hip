@@ -12,6 +12,7 @@
 //     and its L2 sees every A/B panel only a few times;
 //   * the epilogue (per-row scale, alpha, device scalar, store/add, bf16/fp32/i32, packed int8 delta) is fused.
 #include "common.h"
+#include <type_traits>
 
 namespace
 {
@@ -38,6 +39,7 @@ struct GemmP {
     int64_t cSlab;           // bytes between the C blocks of consecutive groups
     int64_t tileScaleSlab;   // floats
     int splitK_groups;       // number of groups when groupOffsets is set
+    int direct;              // 1: direct global->LDS loader
 };
 
 enum { T_I8 = 0, T_FP8 = 1, T_BF16 = 2 };
@@ -74,224 +76,10 @@ __device__ __forceinline__ void MapTile(int bid, int nb, int tilesM, int tilesN,
     *tn = r / gsz;
 }
 
-template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT>
-__global__ void __launch_bounds__(256, 1) GemmNT(GemmP p)
+template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT, class TAcc, class TFAcc>
+__device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], TFAcc &facc, uint8_t *lds, int rowBase, int colBase, int wm, int wn,
+    int half, int l32)
 {
-    typedef typename AccT<TYPE>::type TAcc;
-    constexpr int BM = 64 * WTM;
-    constexpr int BN = 64 * WTN;
-    constexpr int LA = BM / 32; // 16-byte loads per thread for the A tile
-    constexpr int LB = BN / 32;
-    constexpr int STAGE = (BM + BN) * BKB;
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int wm = wave >> 1;
-    const int wn = wave & 1;
-
-    int tm, tn;
-    const int tilesMN = p.tilesM * p.tilesN;
-    int bid = blockIdx.x;
-    int split = 0;
-    if (p.splitK > 1) {
-        split = bid / tilesMN;
-        bid -= split * tilesMN;
-    }
-    MapTile(bid, tilesMN, p.tilesM, p.tilesN, &tm, &tn);
-    const int rowBase = tm * BM;
-    const int colBase = tn * BN;
-
-    // contraction range of this workgroup
-    int kSteps = p.kBytes / BKB;
-    int kBeg = 0;
-    if (p.tileGroup) {
-        // rows of one 128-row tile belong to one group (BM == 128 is enforced by the host); its B operand is that group's slab
-        int g = p.tileGroup[rowBase / TILE];
-        if (g < 0) {
-            return;
-        }
-        p.b += (int64_t)g * p.bSlab;
-    }
-    if (p.groupOffsets) {
-        // delta of one group: contraction over the group's own rows only
-        int g = blockIdx.y;
-        kBeg = p.groupOffsets[g] * (TYPE == T_BF16 ? 2 : 1) / BKB;
-        kSteps = p.groupOffsets[g + 1] * (TYPE == T_BF16 ? 2 : 1) / BKB - kBeg;
-        p.c += (int64_t)g * p.cSlab;
-        if (p.tileScale) {
-            p.tileScale += (int64_t)g * p.tileScaleSlab;
-        }
-    }
-    if (p.splitK > 1) {
-        int per = (kSteps + p.splitK - 1) / p.splitK;
-        if (KT) {
-            int tileSteps = p.kTileBytes / BKB;
-            per = (per + tileSteps - 1) / tileSteps * tileSteps;
-        }
-        kBeg = split * per;
-        int kEnd = kBeg + per < kSteps ? kBeg + per : kSteps;
-        kSteps = kEnd - kBeg;
-        if (kSteps <= 0) {
-            return;
-        }
-    }
-
-    // global load addressing: thread -> (row = tid/8 + 32*i, 16-byte chunk = tid%8)
-    const int lc = tid & 7;
-    const int lr = tid >> 3;
-    const uint8_t *gaBase = p.a + (int64_t)(rowBase + lr) * p.lda + (int64_t)kBeg * BKB + lc * 16;
-    const uint8_t *gbBase = p.b + (int64_t)(colBase + lr) * p.ldb + (int64_t)kBeg * BKB + lc * 16;
-    v4i ra[LA], rb[LB];
-
-    auto loadGlobal = [&](int step) {
-#pragma unroll
-        for (int i = 0; i < LA; ++i) {
-            ra[i] = *(const v4i *)(gaBase + (int64_t)i * 32 * p.lda + (int64_t)step * BKB);
-        }
-#pragma unroll
-        for (int i = 0; i < LB; ++i) {
-            rb[i] = *(const v4i *)(gbBase + (int64_t)i * 32 * p.ldb + (int64_t)step * BKB);
-        }
-    };
-    auto storeLds = [&](int stage) {
-        uint8_t *sa = lds + stage * STAGE;
-        uint8_t *sb = sa + BM * BKB;
-#pragma unroll
-        for (int i = 0; i < LA; ++i) {
-            *(v4i *)(sa + SwizzleOffset(lr + 32 * i, lc)) = ra[i];
-        }
-#pragma unroll
-        for (int i = 0; i < LB; ++i) {
-            *(v4i *)(sb + SwizzleOffset(lr + 32 * i, lc)) = rb[i];
-        }
-    };
-
-    TAcc acc[WTM][WTN];
-    v16f facc[KT ? WTM : 1][KT ? WTN : 1];
-#pragma unroll
-    for (int i = 0; i < WTM; ++i) {
-#pragma unroll
-        for (int j = 0; j < WTN; ++j) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                acc[i][j][e] = 0;
-            }
-        }
-    }
-    if (KT) {
-#pragma unroll
-        for (int i = 0; i < WTM; ++i) {
-#pragma unroll
-            for (int j = 0; j < WTN; ++j) {
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    facc[i][j][e] = 0;
-                }
-            }
-        }
-    }
-
-    const int half = lane >> 5;
-    const int l32 = lane & 31;
-    const int aRow0 = wm * (32 * WTM) + l32;
-    const int bRow0 = wn * (32 * WTN) + l32;
-
-    auto compute = [&](int stage) {
-        const uint8_t *sa = lds + stage * STAGE;
-        const uint8_t *sb = sa + BM * BKB;
-        if (TYPE == T_FP8) {
-#pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                v8i fa[WTM], fb[WTN];
-                int ch = s * 4 + half * 2;
-#pragma unroll
-                for (int i = 0; i < WTM; ++i) {
-                    v4i lo = *(const v4i *)(sa + SwizzleOffset(aRow0 + 32 * i, ch));
-                    v4i hi = *(const v4i *)(sa + SwizzleOffset(aRow0 + 32 * i, ch + 1));
-                    fa[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                }
-#pragma unroll
-                for (int j = 0; j < WTN; ++j) {
-                    v4i lo = *(const v4i *)(sb + SwizzleOffset(bRow0 + 32 * j, ch));
-                    v4i hi = *(const v4i *)(sb + SwizzleOffset(bRow0 + 32 * j, ch + 1));
-                    fb[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                }
-#pragma unroll
-                for (int i = 0; i < WTM; ++i) {
-#pragma unroll
-                    for (int j = 0; j < WTN; ++j) {
-                        if constexpr (TYPE == T_FP8) {
-                            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], 0, 0, 0, 0, 0, 0);
-                        }
-                    }
-                }
-            }
-        } else {
-#pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                v4i fa[WTM], fb[WTN];
-                int ch = s * 2 + half;
-#pragma unroll
-                for (int i = 0; i < WTM; ++i) {
-                    fa[i] = *(const v4i *)(sa + SwizzleOffset(aRow0 + 32 * i, ch));
-                }
-#pragma unroll
-                for (int j = 0; j < WTN; ++j) {
-                    fb[j] = *(const v4i *)(sb + SwizzleOffset(bRow0 + 32 * j, ch));
-                }
-#pragma unroll
-                for (int i = 0; i < WTM; ++i) {
-#pragma unroll
-                    for (int j = 0; j < WTN; ++j) {
-                        if constexpr (TYPE == T_I8) {
-                            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
-                        } else if constexpr (TYPE == T_BF16) {
-                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                                __builtin_bit_cast(v8bf, fa[i]), __builtin_bit_cast(v8bf, fb[j]), acc[i][j], 0, 0, 0);
-                        }
-                    }
-                }
-            }
-        }
-    };
-
-    // main loop: one barrier per step, LDS double buffered, global loads of step s+1 in flight during the MFMAs of step s
-    if (kSteps > 0) {
-        loadGlobal(0);
-        storeLds(0);
-    }
-    __syncthreads();
-    const int tileSteps = KT ? p.kTileBytes / BKB : 0;
-    for (int s = 0; s < kSteps; ++s) {
-        int cur = s & 1;
-        if (s + 1 < kSteps) {
-            loadGlobal(s + 1);
-        }
-        compute(cur);
-        if (KT) {
-            if ((kBeg + s + 1) % tileSteps == 0 || s + 1 == kSteps) {
-                float sc = p.kTileScale[(kBeg + s) / tileSteps];
-#pragma unroll
-                for (int i = 0; i < WTM; ++i) {
-#pragma unroll
-                    for (int j = 0; j < WTN; ++j) {
-#pragma unroll
-                        for (int e = 0; e < 16; ++e) {
-                            facc[i][j][e] += sc * (float)acc[i][j][e];
-                            acc[i][j][e] = 0;
-                        }
-                    }
-                }
-            }
-        }
-        if (s + 1 < kSteps) {
-            storeLds(cur ^ 1);
-        }
-        __syncthreads();
-    }
-
     // ---- epilogue.  MFMA 32x32 result: lane holds column l32, rows (e/4)*8 + half*4 + e%4
     float scale = p.alpha;
     if (p.alphaPtr) {
@@ -420,12 +208,435 @@ __global__ void __launch_bounds__(256, 1) GemmNT(GemmP p)
     }
 }
 
+template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT>
+__global__ void __launch_bounds__(256, 1) GemmNT(GemmP p)
+{
+    typedef typename AccT<TYPE>::type TAcc;
+    constexpr int BM = 64 * WTM;
+    constexpr int BN = 64 * WTN;
+    constexpr int LA = BM / 32; // 16-byte loads per thread for the A tile
+    constexpr int LB = BN / 32;
+    constexpr int STAGE = (BM + BN) * BKB;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave >> 1;
+    const int wn = wave & 1;
+
+    int tm, tn;
+    const int tilesMN = p.tilesM * p.tilesN;
+    int bid = blockIdx.x;
+    int split = 0;
+    if (p.splitK > 1) {
+        split = bid / tilesMN;
+        bid -= split * tilesMN;
+    }
+    MapTile(bid, tilesMN, p.tilesM, p.tilesN, &tm, &tn);
+    const int rowBase = tm * BM;
+    const int colBase = tn * BN;
+
+    // contraction range of this workgroup
+    int kSteps = p.kBytes / BKB;
+    int kBeg = 0;
+    if (p.tileGroup) {
+        // rows of one 128-row tile belong to one group (BM == 128 is enforced by the host); its B operand is that group's slab
+        int g = p.tileGroup[rowBase / TILE];
+        if (g < 0) {
+            return;
+        }
+        p.b += (int64_t)g * p.bSlab;
+    }
+    if (p.groupOffsets) {
+        // delta of one group: contraction over the group's own rows only
+        int g = blockIdx.y;
+        kBeg = p.groupOffsets[g] * (TYPE == T_BF16 ? 2 : 1) / BKB;
+        kSteps = p.groupOffsets[g + 1] * (TYPE == T_BF16 ? 2 : 1) / BKB - kBeg;
+        p.c += (int64_t)g * p.cSlab;
+        if (p.tileScale) {
+            p.tileScale += (int64_t)g * p.tileScaleSlab;
+        }
+    }
+    if (p.splitK > 1) {
+        int per = (kSteps + p.splitK - 1) / p.splitK;
+        if (KT) {
+            int tileSteps = p.kTileBytes / BKB;
+            per = (per + tileSteps - 1) / tileSteps * tileSteps;
+        }
+        kBeg = split * per;
+        int kEnd = kBeg + per < kSteps ? kBeg + per : kSteps;
+        kSteps = kEnd - kBeg;
+        if (kSteps <= 0) {
+            return;
+        }
+    }
+
+    // global load addressing: thread -> (row = tid/8 + 32*i, 16-byte chunk = tid%8)
+    const int lc = tid & 7;
+    const int lr = tid >> 3;
+    const uint8_t *gaBase = p.a + (int64_t)(rowBase + lr) * p.lda + (int64_t)kBeg * BKB + lc * 16;
+    const uint8_t *gbBase = p.b + (int64_t)(colBase + lr) * p.ldb + (int64_t)kBeg * BKB + lc * 16;
+    v4i ra[LA], rb[LB];
+
+    auto loadGlobal = [&](int step) {
+#pragma unroll
+        for (int i = 0; i < LA; ++i) {
+            ra[i] = *(const v4i *)(gaBase + (int64_t)i * 32 * p.lda + (int64_t)step * BKB);
+        }
+#pragma unroll
+        for (int i = 0; i < LB; ++i) {
+            rb[i] = *(const v4i *)(gbBase + (int64_t)i * 32 * p.ldb + (int64_t)step * BKB);
+        }
+    };
+    auto storeLds = [&](int stage) {
+        uint8_t *sa = lds + stage * STAGE;
+        uint8_t *sb = sa + BM * BKB;
+#pragma unroll
+        for (int i = 0; i < LA; ++i) {
+            *(v4i *)(sa + SwizzleOffset(lr + 32 * i, lc)) = ra[i];
+        }
+#pragma unroll
+        for (int i = 0; i < LB; ++i) {
+            *(v4i *)(sb + SwizzleOffset(lr + 32 * i, lc)) = rb[i];
+        }
+    };
+
+    TAcc acc[WTM][WTN];
+    v16f facc[KT ? WTM : 1][KT ? WTN : 1];
+#pragma unroll
+    for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+        for (int j = 0; j < WTN; ++j) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                acc[i][j][e] = 0;
+            }
+        }
+    }
+    if (KT) {
+#pragma unroll
+        for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+            for (int j = 0; j < WTN; ++j) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    facc[i][j][e] = 0;
+                }
+            }
+        }
+    }
+
+    const int half = lane >> 5;
+    const int l32 = lane & 31;
+    const int aRow0 = wm * (32 * WTM) + l32;
+    const int bRow0 = wn * (32 * WTN) + l32;
+
+    // MFMA operand fragments, two register sets: the set of slice s+1 is fetched from LDS while the MFMAs of slice s run
+    constexpr int NS = TYPE == T_FP8 ? 2 : 4; // K slices per step: 64 bytes (f8f6f4 32x32x64) or 32 bytes (i8 32x32x32, bf16 32x32x16)
+    typedef typename std::conditional<TYPE == T_FP8, v8i, v4i>::type TFrag;
+    TFrag fa[2][WTM], fb[2][WTN];
+    auto loadOne = [&](const uint8_t *base, int row, int sl) -> TFrag {
+        if constexpr (TYPE == T_FP8) {
+            int ch = sl * 4 + half * 2;
+            v4i lo = *(const v4i *)(base + SwizzleOffset(row, ch));
+            v4i hi = *(const v4i *)(base + SwizzleOffset(row, ch + 1));
+            return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        } else {
+            return *(const v4i *)(base + SwizzleOffset(row, sl * 2 + half));
+        }
+    };
+    auto mfma = [&](TFrag a, TFrag b, TAcc c) -> TAcc {
+        if constexpr (TYPE == T_I8) {
+            return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+        } else if constexpr (TYPE == T_FP8) {
+            return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+        } else {
+            return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+        }
+    };
+#define LOAD_FRAGS(SET, STAGE, SL)                                                                                                         \
+    do {                                                                                                                                   \
+        const uint8_t *sa_ = lds + (STAGE)*STAGE_BYTES;                                                                                    \
+        const uint8_t *sb_ = sa_ + BM * BKB;                                                                                               \
+        _Pragma("unroll") for (int i = 0; i < WTM; ++i) fa[SET][i] = loadOne(sa_, aRow0 + 32 * i, SL);                                     \
+        _Pragma("unroll") for (int j = 0; j < WTN; ++j) fb[SET][j] = loadOne(sb_, bRow0 + 32 * j, SL);                                     \
+    } while (0)
+#define MFMA_ROWS(SET, I0, I1)                                                                                                             \
+    do {                                                                                                                                   \
+        _Pragma("unroll") for (int i = I0; i < I1; ++i) _Pragma("unroll") for (int j = 0; j < WTN; ++j) acc[i][j] =                        \
+            mfma(fa[SET][i], fb[SET][j], acc[i][j]);                                                                                       \
+    } while (0)
+
+    // main loop: LDS double buffered; global loads of step s+1 are in flight during step s, are written to LDS before the last
+    // slice's MFMAs, the barrier sits in the middle of that slice and the first fragments of step s+1 are fetched behind it
+    constexpr int STAGE_BYTES = STAGE;
+    if (kSteps > 0) {
+        loadGlobal(0);
+        storeLds(0);
+    }
+    __syncthreads();
+    if (kSteps > 0) {
+        LOAD_FRAGS(0, 0, 0);
+    }
+    const int tileSteps = KT ? p.kTileBytes / BKB : 0;
+    for (int s = 0; s < kSteps; ++s) {
+        const int cur = s & 1;
+        const bool more = s + 1 < kSteps;
+        if (more) {
+            loadGlobal(s + 1);
+        }
+#pragma unroll
+        for (int sl = 0; sl < NS - 1; ++sl) {
+            if ((sl & 1) == 0) {
+                LOAD_FRAGS(1, cur, sl + 1);
+                MFMA_ROWS(0, 0, WTM);
+            } else {
+                LOAD_FRAGS(0, cur, sl + 1);
+                MFMA_ROWS(1, 0, WTM);
+            }
+        }
+        // last slice lives in set 1 (NS is even)
+        if (more) {
+            storeLds(cur ^ 1);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        MFMA_ROWS(1, 0, WTM / 2);
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+        if (more) {
+            LOAD_FRAGS(0, cur ^ 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0); // keep the LDS reads ahead of the remaining MFMAs, which hide their latency
+        MFMA_ROWS(1, WTM / 2, WTM);
+        if (KT) {
+            if ((kBeg + s + 1) % tileSteps == 0 || s + 1 == kSteps) {
+                float sc = p.kTileScale[(kBeg + s) / tileSteps];
+#pragma unroll
+                for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+                    for (int j = 0; j < WTN; ++j) {
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) {
+                            facc[i][j][e] += sc * (float)acc[i][j][e];
+                            acc[i][j][e] = 0;
+                        }
+                    }
+                }
+            }
+        }
+    }
+#undef LOAD_FRAGS
+#undef MFMA_ROWS
+    __syncthreads();
+
+    Epilogue<TYPE, WTM, WTN, CT, EPI, KT>(p, acc, facc, lds, rowBase, colBase, wm, wn, half, l32);
+}
+
 __global__ void ZeroRows(uint8_t *c, int64_t ldc, int rowBytes)
 {
     uint8_t *row = c + (int64_t)blockIdx.x * ldc;
     for (int x = threadIdx.x * 4; x < rowBytes; x += blockDim.x * 4) {
         *(int *)(row + x) = 0;
     }
+}
+
+
+// ---------------------------------------------------------------------------------------------------------------------------
+// Variant with direct global -> LDS loads (global_load_lds_dwordx4): no staging registers and no ds_write instructions.  A wave-level
+// load deposits 64 x 16 bytes contiguously in LDS, i.e. one block of 8 tile rows; which 16-byte chunk of the row a lane fetches is
+// chosen so that the block lands already XOR-swizzled.  The two LDS stages are separate static arrays: the compiler can then prove
+// that the operand reads of one stage do not alias the in-flight loads into the other and does not serialise them.
+#define TS2_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
+#define TS2_GLB_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
+
+template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT>
+__global__ void __launch_bounds__(256, 1) GemmNTDirect(GemmP p)
+{
+    typedef typename AccT<TYPE>::type TAcc;
+    constexpr int BM = 64 * WTM;
+    constexpr int BN = 64 * WTN;
+    __shared__ __attribute__((aligned(1024))) uint8_t sA0[BM * BKB];
+    __shared__ __attribute__((aligned(1024))) uint8_t sB0[BN * BKB];
+    __shared__ __attribute__((aligned(1024))) uint8_t sA1[BM * BKB];
+    __shared__ __attribute__((aligned(1024))) uint8_t sB1[BN * BKB];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave >> 1;
+    const int wn = wave & 1;
+
+    int tm, tn;
+    const int tilesMN = p.tilesM * p.tilesN;
+    int bid = blockIdx.x;
+    MapTile(bid, tilesMN, p.tilesM, p.tilesN, &tm, &tn);
+    const int rowBase = tm * BM;
+    const int colBase = tn * BN;
+    int kSteps = p.kBytes / BKB;
+    int kBeg = 0;
+    if (p.tileGroup) {
+        int g = p.tileGroup[rowBase / TILE];
+        if (g < 0) {
+            return;
+        }
+        p.b += (int64_t)g * p.bSlab;
+    }
+    if (p.groupOffsets) {
+        int g = blockIdx.y;
+        kBeg = p.groupOffsets[g] * (TYPE == T_BF16 ? 2 : 1) / BKB;
+        kSteps = p.groupOffsets[g + 1] * (TYPE == T_BF16 ? 2 : 1) / BKB - kBeg;
+        p.c += (int64_t)g * p.cSlab;
+        if (p.tileScale) {
+            p.tileScale += (int64_t)g * p.tileScaleSlab;
+        }
+    }
+
+    // loader: wave w fills the 8-row blocks w, w+4, w+8, ... of each operand tile; inside a block lane -> (row = lane/8, slot = lane%8)
+    // and the slot holds chunk slot ^ ((row >> 1) & 7) of the row.  All blocks of one wave have the same parity, so the chunk is fixed.
+    const int lrow = wave * 8 + (lane >> 3);
+    const int lchunk = (lane & 7) ^ ((lrow >> 1) & 7);
+    // address = wave-uniform base (scalar registers) + one 32-bit per-lane offset per operand
+    const uint8_t *gaTile = p.a + (int64_t)rowBase * p.lda + (int64_t)kBeg * BKB;
+    const uint8_t *gbTile = p.b + (int64_t)colBase * p.ldb + (int64_t)kBeg * BKB;
+    const uint32_t gaLane = (uint32_t)(lrow * (int)p.lda + lchunk * 16);
+    const uint32_t gbLane = (uint32_t)(lrow * (int)p.ldb + lchunk * 16);
+    constexpr int LA = BM / 32;
+    constexpr int LB = BN / 32;
+#define DIRECT_LOAD(SA, SB, STEP)                                                                                                          \
+    do {                                                                                                                                   \
+        _Pragma("unroll") for (int i = 0; i < LA; ++i) __builtin_amdgcn_global_load_lds(                                                   \
+            TS2_GLB_PTR(gaTile + ((int64_t)i * 32 * p.lda + (int64_t)(STEP)*BKB) + gaLane), TS2_LDS_PTR(SA + (wave + 4 * i) * 1024), 16, 0, 0); \
+        _Pragma("unroll") for (int i = 0; i < LB; ++i) __builtin_amdgcn_global_load_lds(                                                   \
+            TS2_GLB_PTR(gbTile + ((int64_t)i * 32 * p.ldb + (int64_t)(STEP)*BKB) + gbLane), TS2_LDS_PTR(SB + (wave + 4 * i) * 1024), 16, 0, 0); \
+    } while (0)
+
+    TAcc acc[WTM][WTN];
+    v16f facc[KT ? WTM : 1][KT ? WTN : 1];
+#pragma unroll
+    for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+        for (int j = 0; j < WTN; ++j) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                acc[i][j][e] = 0;
+            }
+        }
+    }
+    if (KT) {
+#pragma unroll
+        for (int i = 0; i < (KT ? WTM : 1); ++i) {
+#pragma unroll
+            for (int j = 0; j < (KT ? WTN : 1); ++j) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    facc[i][j][e] = 0;
+                }
+            }
+        }
+    }
+    const int half = lane >> 5;
+    const int l32 = lane & 31;
+    const int aRow0 = wm * (32 * WTM) + l32;
+    const int bRow0 = wn * (32 * WTN) + l32;
+    constexpr int NS = TYPE == T_FP8 ? 2 : 4;
+    typedef typename std::conditional<TYPE == T_FP8, v8i, v4i>::type TFrag;
+    TFrag fa[2][WTM], fb[2][WTN];
+    auto loadOne = [&](const uint8_t *base, int row, int sl) -> TFrag {
+        if constexpr (TYPE == T_FP8) {
+            int ch = sl * 4 + half * 2;
+            v4i lo = *(const v4i *)(base + SwizzleOffset(row, ch));
+            v4i hi = *(const v4i *)(base + SwizzleOffset(row, ch + 1));
+            return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        } else {
+            return *(const v4i *)(base + SwizzleOffset(row, sl * 2 + half));
+        }
+    };
+    auto mfma = [&](TFrag a, TFrag b, TAcc c) -> TAcc {
+        if constexpr (TYPE == T_I8) {
+            return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+        } else if constexpr (TYPE == T_FP8) {
+            return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+        } else {
+            return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+        }
+    };
+#define LOAD_FRAGS(SET, SA, SB, SL)                                                                                                        \
+    do {                                                                                                                                   \
+        _Pragma("unroll") for (int i = 0; i < WTM; ++i) fa[SET][i] = loadOne(SA, aRow0 + 32 * i, SL);                                      \
+        _Pragma("unroll") for (int j = 0; j < WTN; ++j) fb[SET][j] = loadOne(SB, bRow0 + 32 * j, SL);                                      \
+    } while (0)
+#define MFMA_ROWS(SET, I0, I1)                                                                                                             \
+    do {                                                                                                                                   \
+        _Pragma("unroll") for (int i = I0; i < I1; ++i) _Pragma("unroll") for (int j = 0; j < WTN; ++j) acc[i][j] =                        \
+            mfma(fa[SET][i], fb[SET][j], acc[i][j]);                                                                                       \
+    } while (0)
+#define WAIT_VM0() __builtin_amdgcn_s_waitcnt(0x0F70) /* vmcnt(0): the direct loads have landed in LDS */
+    const int tileSteps = KT ? p.kTileBytes / BKB : 0;
+    // one K step computing from stage (CA, CB) while the next tile streams into (NA, NB)
+#define STEP(CA, CB, NA, NB, S)                                                                                                            \
+    do {                                                                                                                                   \
+        const bool more_ = (S) + 1 < kSteps;                                                                                               \
+        if (more_) {                                                                                                                       \
+            DIRECT_LOAD(NA, NB, (S) + 1);                                                                                                  \
+        }                                                                                                                                  \
+        _Pragma("unroll") for (int sl = 0; sl < NS - 1; ++sl)                                                                              \
+        {                                                                                                                                  \
+            if ((sl & 1) == 0) {                                                                                                           \
+                LOAD_FRAGS(1, CA, CB, sl + 1);                                                                                             \
+                MFMA_ROWS(0, 0, WTM);                                                                                                      \
+            } else {                                                                                                                       \
+                LOAD_FRAGS(0, CA, CB, sl + 1);                                                                                             \
+                MFMA_ROWS(1, 0, WTM);                                                                                                      \
+            }                                                                                                                              \
+        }                                                                                                                                  \
+        __builtin_amdgcn_sched_barrier(0);                                                                                                 \
+        MFMA_ROWS(1, 0, WTM / 2);                                                                                                          \
+        __builtin_amdgcn_sched_barrier(0);                                                                                                 \
+        WAIT_VM0();                                                                                                                        \
+        __syncthreads();                                                                                                                   \
+        if (more_) {                                                                                                                       \
+            LOAD_FRAGS(0, NA, NB, 0);                                                                                                      \
+        }                                                                                                                                  \
+        __builtin_amdgcn_sched_barrier(0);                                                                                                 \
+        MFMA_ROWS(1, WTM / 2, WTM);                                                                                                        \
+        if (KT) {                                                                                                                          \
+            if ((kBeg + (S) + 1) % tileSteps == 0 || (S) + 1 == kSteps) {                                                                  \
+                float sc = p.kTileScale[(kBeg + (S)) / tileSteps];                                                                         \
+                _Pragma("unroll") for (int i = 0; i < (KT ? WTM : 1); ++i) _Pragma("unroll") for (int j = 0; j < (KT ? WTN : 1); ++j)      \
+                    _Pragma("unroll") for (int e = 0; e < 16; ++e)                                                                         \
+                {                                                                                                                          \
+                    facc[i][j][e] += sc * (float)acc[i][j][e];                                                                             \
+                    acc[i][j][e] = 0;                                                                                                      \
+                }                                                                                                                          \
+            }                                                                                                                              \
+        }                                                                                                                                  \
+    } while (0)
+
+    if (kSteps > 0) {
+        DIRECT_LOAD(sA0, sB0, 0);
+    }
+    WAIT_VM0();
+    __syncthreads();
+    if (kSteps > 0) {
+        LOAD_FRAGS(0, sA0, sB0, 0);
+    }
+    // two steps per iteration so that each stage is a compile-time array; an odd tail step is peeled off behind the loop
+    int s = 0;
+    for (; s + 1 < kSteps; s += 2) {
+        STEP(sA0, sB0, sA1, sB1, s);
+        STEP(sA1, sB1, sA0, sB0, s + 1);
+    }
+    if (s < kSteps) {
+        STEP(sA0, sB0, sA1, sB1, s);
+    }
+#undef STEP
+#undef LOAD_FRAGS
+#undef MFMA_ROWS
+#undef DIRECT_LOAD
+#undef WAIT_VM0
+    __syncthreads();
+    Epilogue<TYPE, WTM, WTN, CT, EPI, KT>(p, acc, facc, sA0, rowBase, colBase, wm, wn, half, l32);
 }
 
 template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT> int Launch(const GemmP &p, hipStream_t stream)
@@ -444,6 +655,11 @@ template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT> int Launch(const
         attrDone = true;
     }
     int nb = q.tilesM * q.tilesN * (p.splitK > 1 ? p.splitK : 1);
+    if (p.direct && p.splitK <= 1) {
+        hipLaunchKernelGGL((GemmNTDirect<TYPE, WTM, WTN, CT, EPI, KT>), dim3(nb, p.groupOffsets ? p.splitK_groups : 1), dim3(256), 0, stream, q);
+        TS2_CHECK_LAUNCH();
+        return TS2_OK;
+    }
     hipLaunchKernelGGL(kern, dim3(nb, p.groupOffsets ? p.splitK_groups : 1), dim3(256), ldsBytes, stream, q);
     TS2_CHECK_LAUNCH();
     return TS2_OK;
@@ -495,7 +711,7 @@ template <int TYPE, int WTM, int WTN> int DispatchEpi(const ts2_gemm_args *a, co
 
 template <int TYPE> int DispatchTile(const ts2_gemm_args *a, const GemmP &p, hipStream_t stream)
 {
-    int cfg = a->tileConfig;
+    int cfg = a->tileConfig & 3;
     if (cfg == 0) {
         // 256x256 tiles only when they still fill the chip; the k-tile-scaled kernel keeps a second accumulator set and needs 128x128
         long tilesL = (long)(p.m / 256) * (p.n / 256) * (p.splitK > 1 ? p.splitK : 1);
@@ -564,6 +780,7 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
     p.cSlab = a->cSlabBytes;
     p.tileScaleSlab = a->tileScaleSlabBytes / 4;
     p.splitK_groups = a->groups;
+    p.direct = (a->tileConfig & 4) ? 0 : 1; // bit 2 of tileConfig selects the register-staged loader (kept for comparison)
     if ((a->tileGroup || a->groupOffsets) && splitK > 1) {
         return TS2_ERR_UNSUPPORTED;
     }
