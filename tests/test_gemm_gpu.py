@@ -176,3 +176,17 @@ def test_rejects_bad_shapes(lib):
     assert lib.gemm_nt(a, a, c, L.I8, L.F32, check=False) == -1
     a2 = torch.zeros((100, 128), dtype=torch.int8, device="cuda")
     assert lib.gemm_nt(a2, a2, c, L.I8, L.F32, check=False) == -1
+
+
+def test_eight_wave_configuration_is_bit_exact(lib, orc):
+    print("case 8-wave config", flush=True)
+    from tscale2_amd import lib as L
+    m, n, k = 512, 256, 768
+    r = np.random.default_rng(10)
+    a = r.integers(-128, 128, (m, k), dtype=np.int8)
+    b = r.integers(-128, 128, (n, k), dtype=np.int8)
+    ref = orc_gemm_i8(orc, a, b).astype(np.float32)  # fp32 store of exact int32 sums (|sum| < 2^24 here)
+    tc = torch.empty((m, n), dtype=torch.float32, device="cuda")
+    lib.gemm_nt(torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(), tc, L.I8, L.F32, tile_config=9)
+    torch.cuda.synchronize()
+    assert np.array_equal(tc.cpu().numpy(), ref.astype(np.float32))

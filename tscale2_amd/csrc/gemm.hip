@@ -450,12 +450,13 @@ __global__ void ZeroRows(uint8_t *c, int64_t ldc, int rowBytes)
 #define TS2_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 #define TS2_GLB_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
 
-template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT>
-__global__ void __launch_bounds__(256, 1) GemmNTDirect(GemmP p)
+template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT, int WM = 2, int WN = 2>
+__global__ void __launch_bounds__(64 * WM * WN, (WM * WN) / 4) GemmNTDirect(GemmP p)
 {
     typedef typename AccT<TYPE>::type TAcc;
-    constexpr int BM = 64 * WTM;
-    constexpr int BN = 64 * WTN;
+    constexpr int NW = WM * WN; // waves per workgroup
+    constexpr int BM = 32 * WTM * WM;
+    constexpr int BN = 32 * WTN * WN;
     __shared__ __attribute__((aligned(1024))) uint8_t sA0[BM * BKB];
     __shared__ __attribute__((aligned(1024))) uint8_t sB0[BN * BKB];
     __shared__ __attribute__((aligned(1024))) uint8_t sA1[BM * BKB];
@@ -464,8 +465,8 @@ __global__ void __launch_bounds__(256, 1) GemmNTDirect(GemmP p)
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int wm = wave >> 1;
-    const int wn = wave & 1;
+    const int wm = wave / WN;
+    const int wn = wave % WN;
 
     int tm, tn;
     const int tilesMN = p.tilesM * p.tilesN;
@@ -501,14 +502,14 @@ __global__ void __launch_bounds__(256, 1) GemmNTDirect(GemmP p)
     const uint8_t *gbTile = p.b + (int64_t)colBase * p.ldb + (int64_t)kBeg * BKB;
     const uint32_t gaLane = (uint32_t)(lrow * (int)p.lda + lchunk * 16);
     const uint32_t gbLane = (uint32_t)(lrow * (int)p.ldb + lchunk * 16);
-    constexpr int LA = BM / 32;
-    constexpr int LB = BN / 32;
+    constexpr int LA = BM / (8 * NW);
+    constexpr int LB = BN / (8 * NW);
 #define DIRECT_LOAD(SA, SB, STEP)                                                                                                          \
     do {                                                                                                                                   \
         _Pragma("unroll") for (int i = 0; i < LA; ++i) __builtin_amdgcn_global_load_lds(                                                   \
-            TS2_GLB_PTR(gaTile + ((int64_t)i * 32 * p.lda + (int64_t)(STEP)*BKB) + gaLane), TS2_LDS_PTR(SA + (wave + 4 * i) * 1024), 16, 0, 0); \
+            TS2_GLB_PTR(gaTile + ((int64_t)i * (8 * NW) * p.lda + (int64_t)(STEP)*BKB) + gaLane), TS2_LDS_PTR(SA + (wave + NW * i) * 1024), 16, 0, 0); \
         _Pragma("unroll") for (int i = 0; i < LB; ++i) __builtin_amdgcn_global_load_lds(                                                   \
-            TS2_GLB_PTR(gbTile + ((int64_t)i * 32 * p.ldb + (int64_t)(STEP)*BKB) + gbLane), TS2_LDS_PTR(SB + (wave + 4 * i) * 1024), 16, 0, 0); \
+            TS2_GLB_PTR(gbTile + ((int64_t)i * (8 * NW) * p.ldb + (int64_t)(STEP)*BKB) + gbLane), TS2_LDS_PTR(SB + (wave + NW * i) * 1024), 16, 0, 0); \
     } while (0)
 
     TAcc acc[WTM][WTN];
@@ -665,6 +666,18 @@ template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT> int Launch(const
     return TS2_OK;
 }
 
+// 256x256 tile with 8 waves (2 x 4, wave tile 128x64): two waves per SIMD hide each other's LDS and barrier stalls
+template <int TYPE, int CT, int EPI> int Launch8(const GemmP &p, hipStream_t stream)
+{
+    GemmP q = p;
+    q.tilesM = p.m / 256;
+    q.tilesN = p.n / 256;
+    hipLaunchKernelGGL((GemmNTDirect<TYPE, 4, 2, CT, EPI, false, 2, 4>), dim3(q.tilesM * q.tilesN, p.groupOffsets ? p.splitK_groups : 1), dim3(512), 0,
+        stream, q);
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
 template <int TYPE, int WTM, int WTN> int DispatchEpi(const ts2_gemm_args *a, const GemmP &p, hipStream_t stream)
 {
     const bool kt = a->kTileScale != nullptr;
@@ -698,11 +711,18 @@ template <int TYPE, int WTM, int WTN> int DispatchEpi(const ts2_gemm_args *a, co
         }
         return TS2_ERR_UNSUPPORTED;
     }
+    const bool eight = WTM == 4 && (a->tileConfig & 8) && p.splitK <= 1;
     if (a->cType == TS2_F32) {
+        if (eight) {
+            return epi == TS2_EPI_ADD ? Launch8<TYPE, C_F32, TS2_EPI_ADD>(p, stream) : Launch8<TYPE, C_F32, TS2_EPI_STORE>(p, stream);
+        }
         return epi == TS2_EPI_ADD ? Launch<TYPE, WTM, WTN, C_F32, TS2_EPI_ADD, false>(p, stream)
                                   : Launch<TYPE, WTM, WTN, C_F32, TS2_EPI_STORE, false>(p, stream);
     }
     if (a->cType == TS2_BF16) {
+        if (eight) {
+            return epi == TS2_EPI_ADD ? Launch8<TYPE, C_BF16, TS2_EPI_ADD>(p, stream) : Launch8<TYPE, C_BF16, TS2_EPI_STORE>(p, stream);
+        }
         return epi == TS2_EPI_ADD ? Launch<TYPE, WTM, WTN, C_BF16, TS2_EPI_ADD, false>(p, stream)
                                   : Launch<TYPE, WTM, WTN, C_BF16, TS2_EPI_STORE, false>(p, stream);
     }
