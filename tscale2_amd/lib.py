@@ -121,6 +121,28 @@ def call(name, *args, check=True):
     return rc
 
 
+def probe_mfma_rate(ab_type, random_data, iters=20000):
+    """Sustained rate, in T(FL)OP/s, of a kernel that issues nothing but MFMAs of the given operand type on every CU."""
+    import torch
+    lib = load()
+    scratch = torch.empty(1024 * 256, dtype=torch.int32, device="cuda")
+    out = C.c_double(0)
+    lib.check(lib.dll.ts2_probe_mfma_rate(C.c_int32(ab_type), C.c_int32(int(random_data)), C.c_int32(iters), ptr(scratch),
+                                          C.c_int64(scratch.numel()), C.byref(out), lib.stream()), "ts2_probe_mfma_rate")
+    return out.value
+
+
+def probe_copy_rate(nbytes=1 << 30):
+    """Read + write GB/s of a plain 16-byte-per-lane copy of nbytes bytes."""
+    import torch
+    lib = load()
+    src = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    dst = torch.empty_like(src)
+    out = C.c_double(0)
+    lib.check(lib.dll.ts2_probe_copy_rate(ptr(src), ptr(dst), C.c_int64(nbytes), C.byref(out), lib.stream()), "ts2_probe_copy_rate")
+    return out.value
+
+
 class BwdBuffers(C.Structure):
     _fields_ = [("grad8", Mat), ("grad8RowScale", C.c_void_p), ("gradT", Mat), ("srcT", Mat), ("tileMax", C.c_void_p), ("tileScale", C.c_void_p),
                 ("transformT", Mat)]
