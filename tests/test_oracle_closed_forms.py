@@ -191,7 +191,7 @@ def _fd_ratio(h, mat, delta, r, eps):
 def _check_ratio(h, mat, delta, expect, eps, what):
     """With experts in the model a finite step can flip a selection (a jump in the loss); the same direction is then retried with
     smaller steps and two of them have to agree with the analytic value -- a wrong gradient agrees at none."""
-    steps = [eps] if h.experts == 0 else [eps, eps / 2.5, eps / 5, eps / 10]
+    steps = [eps] if h.experts == 0 else [eps / k for k in (1, 2.5, 5, 10, 25, 50, 100)]
     need = 1 if h.experts == 0 else 2
     seed = zlib.crc32(str(what).encode())
     got = []
