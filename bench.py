@@ -37,6 +37,15 @@ def event_time_ms(fn, iters):
     return e0.elapsed_time(e1) / iters
 
 
+def sustained(ab_type):
+    """What the device sustains with nothing else running: an MFMA-only kernel with per-lane random operand bits (the chip is power
+    limited below its boost clock under such data) and a streaming copy.  Reported beside the published peaks, never instead of them."""
+    from tscale2_amd import lib as L
+    return {"mfma_only_random_operands_tops": round(L.probe_mfma_rate(ab_type, 1, 100000), 1),
+            "mfma_only_constant_operands_tops": round(L.probe_mfma_rate(ab_type, 0, 100000), 1),
+            "copy_read_plus_write_gbps": round(L.probe_copy_rate(1 << 30), 1)}
+
+
 def cpu_baseline_linear(len_full, src_dim, grad_dim, sample_rows):
     """The oracle's restatement of the reference CPU path (MulBackwardWithAccum + SumRankOne, cpu_util.cpp:30-67), OpenMP over
     independent output rows, on a row subsample; tokens/s = sample_rows / time."""
@@ -120,6 +129,7 @@ def bench_linear_i8(args):
                                   "per-channel scales, k-tile 512", "tokens_per_step": len_, "gemm_gop_per_step": 2 * gemm_ops / 1e9},
            "bwd_gemm_tflops": 2 * gemm_ops / ((ms_dx + ms_dw) * 1e-3) / 1e12, "bwd_gemm_pct_of_peak": 100 * roof["frac"],
            "roofline": roof}
+    roof["device_sustained"] = sustained(L.I8)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_linear(len_, src_dim, grad_dim, 2048)
     return out
@@ -206,6 +216,7 @@ def bench_step_fp8(args):
                                   % (dim, heads, depth, ffn // 128, wide, len(lt), vocab, frags, frag_len),
                       "tokens_per_step": n, "matmul_params": params, "useful_tflop_per_step": flop / 1e12},
            "step_tflops": flop / (ms * 1e-3) / 1e12, "bwd_gemm_pct_of_peak": 100 * roof["frac"], "loss": loss, "roofline": roof}
+    roof["device_sustained"] = sustained(L.E4M3)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_step(orc, dim, heads, ffn, lt, la, ls, aw, vocab)
     m.close()
