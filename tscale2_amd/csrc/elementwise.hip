@@ -31,19 +31,24 @@ __device__ __forceinline__ float &ScaleAt(const Mat &m, int tile, int row)
     return *(float *)(m.p + (int64_t)tile * m.ld + (int64_t)row * 4);
 }
 
-// (row, tile) of this 32-lane group; returns false when out of range
-__device__ __forceinline__ bool Unit(int rows, int tiles, int *row, int *tile, int *lane32)
+// Every 32-lane group owns U consecutive rows of one tile column and issues the loads of all U rows before it touches any of them:
+// with one row per group a wave has a single 4-16 byte load per lane in flight and the kernels sit at 30-50 % of what a copy reaches.
+constexpr int U = 4;
+
+// first row and tile of this 32-lane group; returns false when the whole group is out of range
+__device__ __forceinline__ bool Unit(int rows, int tiles, int *row0, int *tile, int *lane32)
 {
     long u = ((long)blockIdx.x * blockDim.x + threadIdx.x) >> 5;
     *lane32 = threadIdx.x & 31;
-    *row = (int)(u / tiles);
-    *tile = (int)(u - (long)(*row) * tiles);
-    return *row < rows;
+    long rb = u / tiles;
+    *tile = (int)(u - rb * tiles);
+    *row0 = (int)(rb * U);
+    return *row0 < rows;
 }
 
 inline dim3 GridFor(int rows, int tiles)
 {
-    long units = (long)rows * tiles;
+    long units = (long)((rows + U - 1) / U) * tiles;
     return dim3((unsigned)((units * 32 + 255) / 256));
 }
 
@@ -53,32 +58,50 @@ __device__ __forceinline__ void AtomicMaxPos(float *p, float v)
     atomicMax((int *)p, __float_as_int(v));
 }
 
+// lanes 0..U-1 of the group store the U per-row scalars of one tile column (16 contiguous bytes)
+__device__ __forceinline__ void StoreScales(const Mat &m, int tile, int row0, int rows, int h, const float (&v)[U])
+{
+    float mine = 0;
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+        mine = h == k ? v[k] : mine;
+    }
+    if (h < U && row0 + h < rows) {
+        ScaleAt(m, tile, row0 + h) = mine;
+    }
+}
+
 // --------------------------------------------------------------------------------------------------------------------------
 template <class TSrc, class TDst>
 __global__ void __launch_bounds__(256) LayerNormalizeStateVecs(int len, int lenRound, int tiles, float vecScale, Mat state, Mat normState, Mat normScale)
 {
-    int t, tile, h;
-    if (!Unit(lenRound, tiles, &t, &tile, &h)) {
+    int t0, tile, h;
+    if (!Unit(lenRound, tiles, &t0, &tile, &h)) {
         return;
     }
     int col = tile * TILE + h * 4;
-    float discr = 0;
-    F4 v = ZeroF4();
-    if (t < len) {
-        v = Load4<TSrc>(At<TSrc>(state, t, col));
-        float sum2 = Half32Sum(HSum(v * v));
+    F4 v[U];
+    float discr[U];
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+        v[k] = t0 + k < len ? Load4<TSrc>(At<TSrc>(state, t0 + k, col)) : ZeroF4();
+    }
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+        discr[k] = 0;
+        float sum2 = Half32Sum(HSum(v[k] * v[k]));
         if (sum2 > 0) {
-            discr = sqrtf(sum2 / TILE) * vecScale;
-            v = v * (1 / discr);
+            discr[k] = sqrtf(sum2 / TILE) * vecScale;
+            v[k] = v[k] * (1 / discr[k]);
+        }
+        if (t0 + k < lenRound) {
+            Store4<TDst>(At<TDst>(normState, t0 + k, col), v[k]);
         }
     }
-    Store4<TDst>(At<TDst>(normState, t, col), v);
-    if (h == 0) {
-        ScaleAt(normScale, tile, t) = discr;
-    }
+    StoreScales(normScale, tile, t0, lenRound, h, discr);
 }
 
-// Every workgroup walks many (row, tile) units and issues ONE atomic max at the end: one atomic per unit (the reference's scheme,
+// Every workgroup walks many units and issues ONE atomic max at the end: one atomic per unit (the reference's scheme,
 // gpu_layer_norm.cuh:111-114) serialises half a million updates of a single address at this problem size.
 template <class TNorm, class TFast, bool FINAL>
 __global__ void __launch_bounds__(256) BackpropLayerNormalize(int len, int rows, int tiles, Mat normState, Mat stateScale, Mat dNormState,
@@ -86,7 +109,7 @@ __global__ void __launch_bounds__(256) BackpropLayerNormalize(int len, int rows,
 {
     __shared__ float red[8];
     const int h = threadIdx.x & 31;
-    const long units = (long)rows * tiles;
+    const long units = (long)((rows + U - 1) / U) * tiles;
     float s = 1;
     if (!FINAL) {
         if (combinerScale) {
@@ -99,26 +122,39 @@ __global__ void __launch_bounds__(256) BackpropLayerNormalize(int len, int rows,
     const float gm = (!FINAL && gradMult) ? *gradMult : 1.f;
     float gmax = 0;
     for (long u = ((long)blockIdx.x * 256 + threadIdx.x) >> 5; u < units; u += (long)gridDim.x * 8) {
-        int t = (int)(u / tiles);
-        int tile = (int)(u - (long)t * tiles);
+        long rb = u / tiles;
+        int tile = (int)(u - rb * tiles);
+        int t0 = (int)rb * U;
         int col = tile * TILE + h * 4;
-        if (t >= len) {
-            Store4<TF32>(At<TF32>(stateGrad, t, col), ZeroF4());
-            Store4<TFast>(At<TFast>(stateGradFast, t, col), ZeroF4());
-            continue;
+        F4 vec[U], grad[U], prev[U];
+        float sc[U];
+#pragma unroll
+        for (int k = 0; k < U; ++k) {
+            int t = t0 + k;
+            bool live = t < len;
+            vec[k] = live ? Load4<TNorm>(At<TNorm>(normState, t, col)) : ZeroF4();
+            grad[k] = live ? Load4<TF32>(At<TF32>(dNormState, t, col)) : ZeroF4();
+            prev[k] = (live && !FINAL) ? Load4<TF32>(At<TF32>(stateGrad, t, col)) : ZeroF4();
+            sc[k] = live ? ScaleAt(stateScale, tile, t) : 0.f;
         }
-        F4 vec = Load4<TNorm>(At<TNorm>(normState, t, col)) * ScaleAt(stateScale, tile, t);
-        F4 grad = Load4<TF32>(At<TF32>(dNormState, t, col));
-        if (!FINAL) {
-            grad = grad * s;
+#pragma unroll
+        for (int k = 0; k < U; ++k) {
+            int t = t0 + k;
+            if (t >= rows) {
+                continue;
+            }
+            F4 g = ZeroF4();
+            if (t < len) {
+                g = FINAL ? grad[k] : grad[k] * s;
+                g = TileNormBackprop(vec[k] * sc[k], g);
+                if (!FINAL) {
+                    g = g + prev[k];
+                }
+                gmax = fmaxf(gmax, HMaxAbs(g));
+            }
+            Store4<TF32>(At<TF32>(stateGrad, t, col), g);
+            Store4<TFast>(At<TFast>(stateGradFast, t, col), g * gm);
         }
-        grad = TileNormBackprop(vec, grad);
-        if (!FINAL) {
-            grad = grad + Load4<TF32>(At<TF32>(stateGrad, t, col));
-        }
-        gmax = fmaxf(gmax, HMaxAbs(grad));
-        Store4<TF32>(At<TF32>(stateGrad, t, col), grad);
-        Store4<TFast>(At<TFast>(stateGradFast, t, col), grad * gm);
     }
     gmax = Half32Max(gmax);
     if (h == 0) {
@@ -143,13 +179,22 @@ template <class TFast>
 __global__ void __launch_bounds__(256) ScaleGrad(int len, int tiles, const float *gradMaxNorm, const float *prevGradMult, Mat grad, Mat gradFast,
     float *gradScaleOut, float *gradMultOut)
 {
-    int t, tile, h;
+    int t0, tile, h;
     float gradMult = ComputeGradMult(*gradMaxNorm);
     bool rewrite = !prevGradMult || gradMult != *prevGradMult;
-    if (Unit(len, tiles, &t, &tile, &h) && rewrite) {
+    if (Unit(len, tiles, &t0, &tile, &h) && rewrite) {
         int col = tile * TILE + h * 4;
-        F4 v = Load4<TF32>(At<TF32>(grad, t, col));
-        Store4<TFast>(At<TFast>(gradFast, t, col), v * gradMult);
+        F4 v[U];
+#pragma unroll
+        for (int k = 0; k < U; ++k) {
+            v[k] = t0 + k < len ? Load4<TF32>(At<TF32>(grad, t0 + k, col)) : ZeroF4();
+        }
+#pragma unroll
+        for (int k = 0; k < U; ++k) {
+            if (t0 + k < len) {
+                Store4<TFast>(At<TFast>(gradFast, t0 + k, col), v[k] * gradMult);
+            }
+        }
     }
 }
 
@@ -168,17 +213,24 @@ __global__ void PublishGradMult(const float *gradMaxNorm, float *gradScaleOut, f
 template <class TDst>
 __global__ void __launch_bounds__(256) MatrixLoLU(int len, int lenRound, int tiles, Mat gate, Mat vals, float resMult, Mat res)
 {
-    int t, tile, h;
-    if (!Unit(lenRound, tiles, &t, &tile, &h)) {
+    int t0, tile, h;
+    if (!Unit(lenRound, tiles, &t0, &tile, &h)) {
         return;
     }
     int col = tile * TILE + h * 4;
-    F4 v = ZeroF4();
-    if (t < len) {
-        F4 g = Load4<TBF16>(At<TBF16>(gate, t, col));
-        v = Load4<TBF16>(At<TBF16>(vals, t, col)) * LoLU4(g) * resMult;
+    F4 g[U], v[U];
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+        bool live = t0 + k < len;
+        g[k] = live ? Load4<TBF16>(At<TBF16>(gate, t0 + k, col)) : ZeroF4();
+        v[k] = live ? Load4<TBF16>(At<TBF16>(vals, t0 + k, col)) : ZeroF4();
     }
-    Store4<TDst>(At<TDst>(res, t, col), v);
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+        if (t0 + k < lenRound) {
+            Store4<TDst>(At<TDst>(res, t0 + k, col), t0 + k < len ? v[k] * LoLU4(g[k]) * resMult : ZeroF4());
+        }
+    }
 }
 
 // MODE 0: FFN (tile-norm backward of vals fused); MODE 1: attention (dScale fused)
@@ -186,39 +238,54 @@ template <class TGrad, class TOutG, class TOutV, int MODE>
 __global__ void __launch_bounds__(256) BackpropLoLU(int len, int lenRound, int tiles, Mat gate, Mat vals, float valsScale, Mat valsSrcTileScale,
     Mat gradArr, Mat gradGate, Mat gradVals, Mat dScale)
 {
-    int t, tile, h;
-    if (!Unit(lenRound, tiles, &t, &tile, &h)) {
+    int t0, tile, h;
+    if (!Unit(lenRound, tiles, &t0, &tile, &h)) {
         return;
     }
     int col = tile * TILE + h * 4;
-    float ds = 0;
-    if (t < len) {
-        F4 g = Load4<TBF16>(At<TBF16>(gate, t, col));
-        F4 v = Load4<TBF16>(At<TBF16>(vals, t, col)) * valsScale;
-        F4 grad = Load4<TGrad>(At<TGrad>(gradArr, t, col));
-        F4 mult = LoLU4(g);
-        F4 resGate = grad * v * LoLUGrad4(mult);
-        F4 resVals = grad * mult;
-        Store4<TOutG>(At<TOutG>(gradGate, t, col), resGate);
-        if (MODE == 0) {
-            // un-normalised source = normalised * (tile scale / valsScale)
-            F4 src = v * (ScaleAt(valsSrcTileScale, tile, t) / valsScale);
-            resVals = TileNormBackprop(src, resVals);
-        } else {
-            ds = Half32Sum(HSum(v * resVals));
-        }
-        Store4<TOutV>(At<TOutV>(gradVals, t, col), resVals);
-    } else {
-        Store4<TOutG>(At<TOutG>(gradGate, t, col), ZeroF4());
-        Store4<TOutV>(At<TOutV>(gradVals, t, col), ZeroF4());
+    F4 g[U], v[U], grad[U];
+    float ts[U], ds[U];
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+        int t = t0 + k;
+        bool live = t < len;
+        g[k] = live ? Load4<TBF16>(At<TBF16>(gate, t, col)) : ZeroF4();
+        v[k] = live ? Load4<TBF16>(At<TBF16>(vals, t, col)) : ZeroF4();
+        grad[k] = live ? Load4<TGrad>(At<TGrad>(gradArr, t, col)) : ZeroF4();
+        ts[k] = (MODE == 0 && live) ? ScaleAt(valsSrcTileScale, tile, t) : 0.f;
     }
-    if (MODE == 1 && h == 0) {
-        ScaleAt(dScale, tile, t) = ds;
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+        int t = t0 + k;
+        ds[k] = 0;
+        if (t >= lenRound) {
+            continue;
+        }
+        F4 resGate = ZeroF4(), resVals = ZeroF4();
+        if (t < len) {
+            F4 vv = v[k] * valsScale;
+            F4 mult = LoLU4(g[k]);
+            resGate = grad[k] * vv * LoLUGrad4(mult);
+            resVals = grad[k] * mult;
+            if (MODE == 0) {
+                // un-normalised source = normalised * (tile scale / valsScale)
+                F4 src = vv * (ts[k] / valsScale);
+                resVals = TileNormBackprop(src, resVals);
+            } else {
+                ds[k] = Half32Sum(HSum(vv * resVals));
+            }
+        }
+        Store4<TOutG>(At<TOutG>(gradGate, t, col), resGate);
+        Store4<TOutV>(At<TOutV>(gradVals, t, col), resVals);
+    }
+    if (MODE == 1) {
+        StoreScales(dScale, tile, t0, lenRound, h, ds);
     }
 }
 
-// one workgroup per row: abs-max over the row, then quantise.  The row is read twice (second read served by L2).
-template <class TSrc>
+// One workgroup per row; the row stays in registers between the abs-max pass and the quantise pass when it has at most 4096
+// elements (REG), otherwise it is read twice (the second read is served by L2).
+template <class TSrc, bool REG>
 __global__ void __launch_bounds__(256) NormalizeVecsRowMax(int len, int dim, Mat src, const float *colScale, Mat dst, float *rowScale)
 {
     __shared__ float red[4];
@@ -234,12 +301,34 @@ __global__ void __launch_bounds__(256) NormalizeVecsRowMax(int len, int dim, Mat
         return;
     }
     float mx = 0;
-    for (int col = tid * 4; col < dim; col += 1024) {
-        F4 v = Load4<TSrc>(At<TSrc>(src, t, col));
-        if (colScale) {
-            v = v * Load4<TF32>(colScale + col);
+    F4 keep[4];
+    if (REG) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            int col = tid * 4 + i * 1024;
+            keep[i] = col < dim ? Load4<TSrc>(At<TSrc>(src, t, col)) : ZeroF4();
         }
-        mx = fmaxf(mx, HMaxAbs(v));
+        if (colScale) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                int col = tid * 4 + i * 1024;
+                if (col < dim) {
+                    keep[i] = keep[i] * Load4<TF32>(colScale + col);
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            mx = fmaxf(mx, HMaxAbs(keep[i]));
+        }
+    } else {
+        for (int col = tid * 4; col < dim; col += 1024) {
+            F4 v = Load4<TSrc>(At<TSrc>(src, t, col));
+            if (colScale) {
+                v = v * Load4<TF32>(colScale + col);
+            }
+            mx = fmaxf(mx, HMaxAbs(v));
+        }
     }
     mx = WaveMax(mx);
     if ((tid & 63) == 0) {
@@ -252,12 +341,22 @@ __global__ void __launch_bounds__(256) NormalizeVecsRowMax(int len, int dim, Mat
         discr = mx / 127;
         mult = 1 / discr;
     }
-    for (int col = tid * 4; col < dim; col += 1024) {
-        F4 v = Load4<TSrc>(At<TSrc>(src, t, col));
-        if (colScale) {
-            v = v * Load4<TF32>(colScale + col);
+    if (REG) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            int col = tid * 4 + i * 1024;
+            if (col < dim) {
+                Store4<TI8>(At<TI8>(dst, t, col), keep[i] * mult);
+            }
         }
-        Store4<TI8>(At<TI8>(dst, t, col), v * mult);
+    } else {
+        for (int col = tid * 4; col < dim; col += 1024) {
+            F4 v = Load4<TSrc>(At<TSrc>(src, t, col));
+            if (colScale) {
+                v = v * Load4<TF32>(colScale + col);
+            }
+            Store4<TI8>(At<TI8>(dst, t, col), v * mult);
+        }
     }
     if (tid == 0) {
         rowScale[t] = discr;
@@ -272,26 +371,46 @@ __global__ void FillFloats(float *p, int n, float v)
     }
 }
 
-// grid (dim/1024 rounded up, len/ROWS): every workgroup reduces ROWS rows x 1024 columns and issues one atomic
+// abs-max of 16 raw bytes holding fp32 or bf16 values
+template <class TSrc> __device__ __forceinline__ float AbsMax16(v4i raw)
+{
+    float m = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        uint32_t w = (uint32_t)raw[e];
+        if (TSrc::SIZE == 4) {
+            m = fmaxf(m, fabsf(__uint_as_float(w)));
+        } else {
+            m = fmaxf(m, fmaxf(fabsf(__uint_as_float(w << 16)), fabsf(__uint_as_float(w & 0xffff0000u))));
+        }
+    }
+    return m;
+}
+
+// grid (row bytes / 4096 rounded up, len/ROWS): a workgroup reduces ROWS rows x 4096 bytes with 16-byte loads, four rows in flight,
+// and issues one atomic.  ROWS divides 128, hence kTile.
 template <class TSrc>
 __global__ void __launch_bounds__(256) TileAbsMax(int len, int dim, Mat src, const float *rowMult, int kTile, float *tileMax)
 {
     constexpr int ROWS = 16;
     __shared__ float red[4];
     int tid = threadIdx.x;
-    int col = blockIdx.x * 1024 + tid * 4;
+    int byteCol = blockIdx.x * 4096 + tid * 16;
     int t0 = blockIdx.y * ROWS;
     float mx = 0;
-    if (col < dim) {
-        for (int r = 0; r < ROWS; ++r) {
-            int t = t0 + r;
-            if (t < len) {
-                F4 v = Load4<TSrc>(At<TSrc>(src, t, col));
-                float m = HMaxAbs(v);
-                if (rowMult) {
-                    m *= fabsf(rowMult[t]);
-                }
-                mx = fmaxf(mx, m);
+    if (byteCol < dim * TSrc::SIZE) {
+        for (int r = 0; r < ROWS; r += 4) {
+            v4i raw[4];
+            float rm[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                int t = t0 + r + k;
+                raw[k] = t < len ? *(const v4i *)(src.p + (int64_t)t * src.ld + byteCol) : (v4i){0, 0, 0, 0};
+                rm[k] = (rowMult && t < len) ? fabsf(rowMult[t]) : 1.f;
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                mx = fmaxf(mx, AbsMax16<TSrc>(raw[k]) * rm[k]);
             }
         }
     }
@@ -306,68 +425,114 @@ __global__ void __launch_bounds__(256) TileAbsMax(int len, int dim, Mat src, con
     }
 }
 
-// 128 (rows t) x 128 (columns x) tile: coalesced row loads, conversion, byte tile in LDS, 4x4 byte transposes in registers with
-// v_perm_b32, 4-byte stores that are contiguous along t across lanes (128-byte runs per destination row).
+// 128 (rows t) x 128 (columns x) tile.  Loads are 16 bytes per lane with four rows in flight, conversion, byte tile in LDS, then
+// every thread transposes a 16 (t) x 4 (x) block with v_perm_b32 and stores 16 bytes to each of 4 destination rows; 8 neighbouring
+// lanes cover the 128 bytes of one destination row.
 template <class TSrc, bool QUANT>
 __global__ void __launch_bounds__(256) TransposeQuant(int len, int lenRound, Mat src, const float *rowMult, const float *tileMax, int kTile,
     const int *rowIndex, Mat dst, float *tileScale)
 {
-    constexpr int PITCH = 132; // bytes per LDS row: keeps the column-wise dword reads spread over the banks
+    constexpr int PITCH = 132;
     __shared__ __attribute__((aligned(16))) uint8_t buf[128 * PITCH];
     int tid = threadIdx.x;
     int xBlock = blockIdx.x * 128;
     int tBlock = blockIdx.y * 128;
-    // load + convert: 32 lanes cover one row of 128 columns, 8 rows per pass
-    int h = tid & 31;
-    for (int r = tid >> 5; r < 128; r += 8) {
-        int t = tBlock + r;
-        uint32_t packed = 0;
-        if (t < len) {
-            int srcRow = rowIndex ? rowIndex[t] : t;
-            if (srcRow >= 0) {
-                if (QUANT) {
-                    F4 v = Load4<TSrc>(At<TSrc>(src, srcRow, xBlock + h * 4));
-                    float tm = tileMax[t / kTile];
-                    float mult = tm > 0 ? 1 / (tm / 127) : 0.f; // same two roundings as scale = max/127, mult = 1/scale
-                    if (rowMult) {
-                        v = v * rowMult[srcRow];
-                    }
-                    v = v * mult;
-                    packed = (uint32_t)(CvtToI8(v.x) & 0xff) | ((uint32_t)(CvtToI8(v.y) & 0xff) << 8) | ((uint32_t)(CvtToI8(v.z) & 0xff) << 16) |
-                             ((uint32_t)(CvtToI8(v.w) & 0xff) << 24);
-                } else {
-                    packed = *(const uint32_t *)(src.p + (int64_t)srcRow * src.ld + xBlock + h * 4);
+    constexpr int SB = QUANT ? TSrc::SIZE : 1;     // source bytes per element
+    constexpr int LPR = 128 * SB / 16;             // lanes per row: 8 (1-byte), 16 (bf16), 32 (fp32)
+    constexpr int RPP = 256 / LPR;                 // rows per pass
+    constexpr int EPL = 16 / SB;                   // elements per lane
+    const int lr = tid / LPR, lc = tid % LPR;
+    float mult = 0;
+    if (QUANT) {
+        float tm = tileMax[tBlock / kTile];          // one 128-row block lies inside one k-tile (kTile is a multiple of 128)
+        mult = tm > 0 ? 1 / (tm / 127) : 0.f;        // same two roundings as scale = max/127, mult = 1/scale
+    }
+    for (int r0 = 0; r0 < 128; r0 += RPP * 4) {
+        v4i raw[4];
+        float rm[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            int r = r0 + k * RPP + lr;
+            int t = tBlock + r;
+            raw[k] = (v4i){0, 0, 0, 0};
+            rm[k] = 0;
+            if (t < len) {
+                int srcRow = rowIndex ? rowIndex[t] : t;
+                if (srcRow >= 0) {
+                    raw[k] = *(const v4i *)(src.p + (int64_t)srcRow * src.ld + (int64_t)(xBlock + lc * EPL) * SB);
+                    rm[k] = (QUANT && rowMult) ? rowMult[srcRow] : 1.f;
                 }
             }
         }
-        *(uint32_t *)(buf + r * PITCH + h * 4) = packed;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            int r = r0 + k * RPP + lr;
+            uint8_t *d = buf + r * PITCH + lc * EPL;
+            if (!QUANT) {
+                *(uint32_t *)d = (uint32_t)raw[k][0];
+                *(uint32_t *)(d + 4) = (uint32_t)raw[k][1];
+                *(uint32_t *)(d + 8) = (uint32_t)raw[k][2];
+                *(uint32_t *)(d + 12) = (uint32_t)raw[k][3];
+            } else {
+                float f[EPL];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    uint32_t w = (uint32_t)raw[k][e];
+                    if (SB == 4) {
+                        f[e] = __uint_as_float(w);
+                    } else {
+                        f[(2 * e) % EPL] = __uint_as_float(w << 16);
+                        f[(2 * e + 1) % EPL] = __uint_as_float(w & 0xffff0000u);
+                    }
+                }
+                uint32_t packed[EPL / 4];
+#pragma unroll
+                for (int q = 0; q < EPL / 4; ++q) {
+                    packed[q] = 0;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        float x = f[q * 4 + e];
+                        if (rowMult) {
+                            x = x * rm[k];
+                        }
+                        packed[q] |= (uint32_t)(CvtToI8(x * mult) & 0xff) << (8 * e);
+                    }
+                }
+                *(uint32_t *)d = packed[0];
+                if (EPL == 8) {
+                    *(uint32_t *)(d + 4) = packed[EPL / 4 - 1];
+                }
+            }
+        }
     }
     __syncthreads();
-    // transpose: thread -> (tq = t quad, xq = x quad); 32 tq x 32 xq = 1024 quads, 4 per thread
-    int tq = tid & 31;
-    for (int xq = tid >> 5; xq < 32; xq += 8) {
-        uint32_t r0 = *(const uint32_t *)(buf + (tq * 4 + 0) * PITCH + xq * 4);
-        uint32_t r1 = *(const uint32_t *)(buf + (tq * 4 + 1) * PITCH + xq * 4);
-        uint32_t r2 = *(const uint32_t *)(buf + (tq * 4 + 2) * PITCH + xq * 4);
-        uint32_t r3 = *(const uint32_t *)(buf + (tq * 4 + 3) * PITCH + xq * 4);
+    // transpose: thread -> (tq = block of 16 t, xq = x quad)
+    const int tq = tid & 7, xq = tid >> 3;
+    uint32_t out[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint8_t *b = buf + (tq * 16 + j * 4) * PITCH + xq * 4;
+        uint32_t r0 = *(const uint32_t *)(b);
+        uint32_t r1 = *(const uint32_t *)(b + PITCH);
+        uint32_t r2 = *(const uint32_t *)(b + 2 * PITCH);
+        uint32_t r3 = *(const uint32_t *)(b + 3 * PITCH);
         // 4x4 byte transpose.  __builtin_amdgcn_perm(hi, lo, sel): result byte i = byte sel[i] of {hi:lo} (lo = bytes 0-3)
         uint32_t a = __builtin_amdgcn_perm(r1, r0, 0x05010400); // r0.b0 r1.b0 r0.b1 r1.b1
-        uint32_t b = __builtin_amdgcn_perm(r1, r0, 0x07030602); // r0.b2 r1.b2 r0.b3 r1.b3
+        uint32_t bb = __builtin_amdgcn_perm(r1, r0, 0x07030602); // r0.b2 r1.b2 r0.b3 r1.b3
         uint32_t c = __builtin_amdgcn_perm(r3, r2, 0x05010400);
         uint32_t d = __builtin_amdgcn_perm(r3, r2, 0x07030602);
-        uint32_t c0 = __builtin_amdgcn_perm(c, a, 0x05040100); // column 0: r0.b0 r1.b0 r2.b0 r3.b0
-        uint32_t c1 = __builtin_amdgcn_perm(c, a, 0x07060302);
-        uint32_t c2 = __builtin_amdgcn_perm(d, b, 0x05040100);
-        uint32_t c3 = __builtin_amdgcn_perm(d, b, 0x07060302);
-        int x = xBlock + xq * 4;
-        int tcol = tBlock + tq * 4;
-        *(uint32_t *)(dst.p + (int64_t)(x + 0) * dst.ld + tcol) = c0;
-        *(uint32_t *)(dst.p + (int64_t)(x + 1) * dst.ld + tcol) = c1;
-        *(uint32_t *)(dst.p + (int64_t)(x + 2) * dst.ld + tcol) = c2;
-        *(uint32_t *)(dst.p + (int64_t)(x + 3) * dst.ld + tcol) = c3;
+        out[0][j] = __builtin_amdgcn_perm(c, a, 0x05040100); // column 0: r0.b0 r1.b0 r2.b0 r3.b0
+        out[1][j] = __builtin_amdgcn_perm(c, a, 0x07060302);
+        out[2][j] = __builtin_amdgcn_perm(d, bb, 0x05040100);
+        out[3][j] = __builtin_amdgcn_perm(d, bb, 0x07060302);
+    }
+    int x = xBlock + xq * 4;
+    int tcol = tBlock + tq * 16;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        *(uint4 *)(dst.p + (int64_t)(x + i) * dst.ld + tcol) = make_uint4(out[i][0], out[i][1], out[i][2], out[i][3]);
     }
     if (QUANT && tileScale && blockIdx.x == 0 && tid == 0) {
-        // one 128-row block lies inside one k-tile (kTile is a multiple of 128)
         float tm = tileMax[tBlock / kTile];
         tileScale[tBlock / kTile] = tm > 0 ? tm / 127 : 1.f;
     }
@@ -385,29 +550,42 @@ template <class TSrc>
 __global__ void __launch_bounds__(256) RowTileNormalizeRope(int len, int lenRound, int tiles, Mat src, float srcMult, int normalize, float vecScale,
     Mat rope, Mat dst, Mat tileScale)
 {
-    int t, tile, h;
-    if (!Unit(lenRound, tiles, &t, &tile, &h)) {
+    int t0, tile, h;
+    if (!Unit(lenRound, tiles, &t0, &tile, &h)) {
         return;
     }
     int col = tile * TILE + h * 4;
-    F4 v = ZeroF4();
-    float discr = 0;
-    if (t < len) {
-        v = Load4<TSrc>(At<TSrc>(src, t, col)) * srcMult;
-        if (normalize) {
-            float sum2 = Half32Sum(HSum(v * v));
-            if (sum2 > 0) {
-                discr = sqrtf(sum2 / TILE) * vecScale;
-                v = v * (1 / discr);
+    F4 v[U], rp[U];
+    float discr[U];
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+        bool live = t0 + k < len;
+        v[k] = live ? Load4<TSrc>(At<TSrc>(src, t0 + k, col)) : ZeroF4();
+        rp[k] = (live && rope.p) ? Load4<TF32>(At<TF32>(rope, t0 + k, h * 4)) : ZeroF4();
+    }
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+        discr[k] = 0;
+        if (t0 + k >= lenRound) {
+            continue;
+        }
+        F4 x = v[k] * srcMult;
+        if (t0 + k < len) {
+            if (normalize) {
+                float sum2 = Half32Sum(HSum(x * x));
+                if (sum2 > 0) {
+                    discr[k] = sqrtf(sum2 / TILE) * vecScale;
+                    x = x * (1 / discr[k]);
+                }
+            }
+            if (rope.p) {
+                x = ApplyRope4(x, rp[k], 1.f);
             }
         }
-        if (rope.p) {
-            v = ApplyRope4(v, Load4<TF32>(At<TF32>(rope, t, h * 4)), 1.f);
-        }
+        Store4<TBF16>(At<TBF16>(dst, t0 + k, col), x);
     }
-    Store4<TBF16>(At<TBF16>(dst, t, col), v);
-    if (normalize && h == 0) {
-        ScaleAt(tileScale, tile, t) = discr;
+    if (normalize) {
+        StoreScales(tileScale, tile, t0, lenRound, h, discr);
     }
 }
 
@@ -415,23 +593,39 @@ template <class TGrad, class TDst>
 __global__ void __launch_bounds__(256) BackpropRowTileNormalizeRope(int len, int lenRound, int tiles, Mat grad, float gradMult, Mat srcNorm,
     Mat srcTileScale, Mat rope, Mat dst)
 {
-    int t, tile, h;
-    if (!Unit(lenRound, tiles, &t, &tile, &h)) {
+    int t0, tile, h;
+    if (!Unit(lenRound, tiles, &t0, &tile, &h)) {
         return;
     }
     int col = tile * TILE + h * 4;
-    F4 g = ZeroF4();
-    if (t < len) {
-        g = Load4<TGrad>(At<TGrad>(grad, t, col)) * gradMult;
-        if (srcNorm.p) {
-            F4 src = Load4<TBF16>(At<TBF16>(srcNorm, t, col)) * ScaleAt(srcTileScale, tile, t);
-            g = TileNormBackprop(src, g);
-        }
-        if (rope.p) {
-            g = ApplyRope4(g, Load4<TF32>(At<TF32>(rope, t, h * 4)), -1.f);
-        }
+    F4 g[U], sn[U], rp[U];
+    float sc[U];
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+        int t = t0 + k;
+        bool live = t < len;
+        g[k] = live ? Load4<TGrad>(At<TGrad>(grad, t, col)) : ZeroF4();
+        sn[k] = (live && srcNorm.p) ? Load4<TBF16>(At<TBF16>(srcNorm, t, col)) : ZeroF4();
+        sc[k] = (live && srcNorm.p) ? ScaleAt(srcTileScale, tile, t) : 0.f;
+        rp[k] = (live && rope.p) ? Load4<TF32>(At<TF32>(rope, t, h * 4)) : ZeroF4();
     }
-    Store4<TDst>(At<TDst>(dst, t, col), g);
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+        int t = t0 + k;
+        if (t >= lenRound) {
+            continue;
+        }
+        F4 x = g[k] * gradMult;
+        if (t < len) {
+            if (srcNorm.p) {
+                x = TileNormBackprop(sn[k] * sc[k], x);
+            }
+            if (rope.p) {
+                x = ApplyRope4(x, rp[k], -1.f);
+            }
+        }
+        Store4<TDst>(At<TDst>(dst, t, col), x);
+    }
 }
 
 bool MatOk(const ts2_mat *m, int rows, int cols, int elemSize)
@@ -645,10 +839,20 @@ extern "C" int ts2_normalize_vecs_row_max(int32_t len, int32_t lenRound, const t
     if (dim % 4 || lenRound < len || !MatOk(src, len, dim, ElemSize(srcType)) || !MatOk(dst, lenRound, dim, 1)) {
         return TS2_ERR_SHAPE;
     }
+    const bool reg = dim <= 4096;
+#define LAUNCH_RM(TS, REG) hipLaunchKernelGGL((NormalizeVecsRowMax<TS, REG>), dim3(lenRound), dim3(256), 0, STREAM, len, dim, M(*src), colScale, M(*dst), rowScale)
     if (srcType == TS2_BF16) {
-        hipLaunchKernelGGL((NormalizeVecsRowMax<TBF16>), dim3(lenRound), dim3(256), 0, STREAM, len, dim, M(*src), colScale, M(*dst), rowScale);
+        if (reg) {
+            LAUNCH_RM(TBF16, true);
+        } else {
+            LAUNCH_RM(TBF16, false);
+        }
     } else if (srcType == TS2_F32) {
-        hipLaunchKernelGGL((NormalizeVecsRowMax<TF32>), dim3(lenRound), dim3(256), 0, STREAM, len, dim, M(*src), colScale, M(*dst), rowScale);
+        if (reg) {
+            LAUNCH_RM(TF32, true);
+        } else {
+            LAUNCH_RM(TF32, false);
+        }
     } else {
         return TS2_ERR_UNSUPPORTED;
     }
@@ -666,12 +870,15 @@ extern "C" int ts2_tile_absmax(int32_t len, const ts2_mat *src, int32_t srcType,
     if (dim % 4 || kTile <= 0 || kTile % 128 || !MatOk(src, len, dim, ElemSize(srcType))) {
         return TS2_ERR_SHAPE;
     }
+    if (((uintptr_t)src->ptr % 16) || (src->strideBytes % 16) || ((int64_t)dim * ElemSize(srcType)) % 16) {
+        return TS2_ERR_ALIGN;
+    }
     int nTiles = (len + kTile - 1) / kTile;
     if (clear) {
         hipLaunchKernelGGL(FillFloats, dim3((nTiles + 255) / 256), dim3(256), 0, STREAM, tileMax, nTiles, 0.f);
         TS2_CHECK_LAUNCH();
     }
-    dim3 grid((dim + 1023) / 1024, (len + 15) / 16);
+    dim3 grid((dim * ElemSize(srcType) + 4095) / 4096, (len + 15) / 16);
     if (srcType == TS2_BF16) {
         hipLaunchKernelGGL((TileAbsMax<TBF16>), grid, dim3(256), 0, STREAM, len, dim, M(*src), rowMult, kTile, tileMax);
     } else if (srcType == TS2_F32) {
@@ -693,6 +900,9 @@ extern "C" int ts2_transpose_quant(int32_t len, int32_t lenRound, const ts2_mat 
     if (dim % 128 || lenRound % 128 || lenRound < len || dstT->x < lenRound || src->x < dim || (dstT->strideBytes % 4) ||
         dstT->strideBytes < lenRound) {
         return TS2_ERR_SHAPE;
+    }
+    if (((uintptr_t)src->ptr % 16) || (src->strideBytes % 16) || ((uintptr_t)dstT->ptr % 16) || (dstT->strideBytes % 16)) {
+        return TS2_ERR_ALIGN;
     }
     dim3 grid(dim / 128, lenRound / 128);
     bool quant = dstType == TS2_I8 && (srcType == TS2_BF16 || srcType == TS2_F32);

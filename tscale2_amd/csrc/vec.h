@@ -149,8 +149,9 @@ __device__ __forceinline__ F4 TileNormBackprop(F4 src, F4 grad)
         return ZeroF4();
     }
     float dp = Half32Sum(HSum(src * grad));
-    float sigma = dp / sum2;
-    float scale = sqrtf(TILE / sum2);
+    float inv = 1 / sum2; // one division per tile; the two quotients below differ from dp/sum2 and TILE/sum2 by an ulp at most
+    float sigma = dp * inv;
+    float scale = sqrtf(TILE * inv);
     return (grad - src * sigma) * scale;
 }
 
@@ -158,13 +159,11 @@ __device__ __forceinline__ F4 TileNormBackprop(F4 src, F4 grad)
 __device__ __forceinline__ float LoLU1(float x)
 {
     float arg = x * 2.f;
-    if (arg < -20) {
-        return 0;
-    } else if (arg > 20) {
-        return 1;
-    }
-    float w = expf(arg);
-    return w / (1 + w);
+    // hardware exp2 and reciprocal (about 1 ulp each): these kernels are otherwise bound by the expf/division instruction count
+    float w = __builtin_amdgcn_exp2f(arg * 1.44269504088896341f);
+    float r = w * __builtin_amdgcn_rcpf(1 + w);
+    r = arg > 20 ? 1.f : r;
+    return arg < -20 ? 0.f : r;
 }
 
 __device__ __forceinline__ F4 LoLU4(F4 g)
