@@ -342,6 +342,9 @@ typedef struct ts2_model_config {
     int32_t attTypeCount;
     int32_t vocab, labelCount, maxLen;
     int32_t kTile; /* rows sharing one scale in the int8 delta GEMM (0 = 512) */
+    /* 0: every FFN and attention layer keeps what its forward pass computed for its backward pass when that fits into half of the
+     * free device memory; 1: the backward recomputes it, as the reference's AddBackward does (layer_ffn.cu:83-113, layer_att.cu:160-226) */
+    int32_t recompute;
 } ts2_model_config;
 
 ts2_model *ts2_model_create(const ts2_model_config *cfg);

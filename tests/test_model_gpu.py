@@ -53,6 +53,27 @@ def check_model(h, tol_state, tol_grad, tol_delta):
         m.close()
 
 
+@pytest.mark.parametrize("mode", [I8, E4M3])
+def test_kept_activations_give_the_same_deltas_as_recomputation(mode):
+    """the default driver keeps each layer's forward activations for its backward; recompute mode rebuilds them as the reference does.
+    Same kernels on the same inputs: every delta must be bit-identical, also on the second step of the same model object."""
+    print("case kept vs recomputed activations", mode, flush=True)
+    h = Harness(mode, dim=256, heads=2, ffn_tiles=4, depth=2, vocab=256, frag_count=4, frag_len=64, wide_window=64, seed=9)
+    res = []
+    for recompute in (False, True):
+        m = h.device_model(recompute=recompute)
+        try:
+            for _ in range(2):
+                m.backprop()
+            torch.cuda.synchronize()
+            res.append([m.get_delta(d, i, *q.fast.shape) for d in range(h.depth) for i, q in enumerate(h.layers[d])] +
+                       [m.array("stateGrad").float().cpu().numpy()])
+        finally:
+            m.close()
+    for a, b in zip(*res):
+        assert np.array_equal(a, b)
+
+
 def test_tiny_dense_int8_step():
     """BASELINE config[0]: e256 h2 d4 ffn8 w64 (8 layers), byte vocab, 8 fragments of 64 tokens, weights N(0, 0.02)"""
     print("case tiny dense int8", flush=True)

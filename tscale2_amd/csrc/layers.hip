@@ -49,14 +49,29 @@ struct TMatrix {
     int srcDim = 0, dstDim = 0, slabs = 1;
 };
 
+struct TActs;
 struct TLayer {
     int type = 0;
     float slope = 0;
     int attId = 0;
     TMatrix w[5];
+    TActs *acts = nullptr;
 };
 
 enum { LT_ATT = 0, LT_FFN = 2, LT_MOE = 3 };
+
+// What a layer's forward pass leaves behind for its backward pass.  The reference recomputes all of it inside AddBackward (its
+// Fwd/Bwd pools are shared between layers, layer_cuda_base.cuh:101-121); with 288 GB of HBM every FFN and attention layer keeps its own
+// set (about 1.35 GB per FFN layer and 0.75 GB per attention layer at dim 2048, ffn 8192, 32768 tokens) and the backward starts
+// from it.  One shared set (recompute mode) serves all layers otherwise.
+struct TActs {
+    Arr a16[4]; // bf16: wide/q, gate, k, v
+    Arr tsc[2]; // fp32 tile scales: wide/q, v
+    Arr rg8;    // 8-bit rg / vlg
+    Arr val16;  // bf16 attention output (its storage is reused for dQ by the backward)
+    Arr swl;    // fp32 [heads][R] softmax statistics
+    bool valid = false;
+};
 } // namespace
 
 struct ts2_model {
@@ -86,13 +101,14 @@ struct ts2_model {
     float *gradMaxNorm = 0, *gradScale = 0, *gradMult = 0, *lossSum = 0;
     // layer scratch (shared by all layers: one layer runs at a time)
     Arr raw;                                 // fp32 [R'][maxW]
-    Arr a16[4];                              // bf16 [R'][maxW]: wide/q, gate, k/val, v
-    Arr tsc[3];                              // fp32 [maxW/128][R'] tile scales
-    Arr rg8;                                 // 8-bit [R'][maxW]
+    TActs shared;                            // the one activation set of recompute mode (and of MoE layers)
+    std::vector<TActs> acts;                 // per layer; entries of kept layers own storage, the others alias `shared`
+    bool keep = false;      // FFN and attention layers own activation sets
+    bool useKept = false;   // inside ModelBackprop: the backward of a layer starts from what its forward left
     Arr g32;                                 // fp32 [R'][maxW] gradient scratch (drg / dvlg)
     Arr gf[4];                               // fast-gradient type [R'][maxW]: dwide/dq, dgate, dk, dv
-    Arr g16[4];                              // bf16 [R'][maxW]: dVal, dQ, dK, dV
-    Arr swl, dScale;                         // fp32 [heads][R]
+    Arr g16[4];                              // bf16 [R'][maxW]: -, dVal, dK, dV
+    Arr dScale;                              // fp32 [heads][R]
     // MoE
     ts2_moe_tables moe = {};
     Arr normMoe, sgMoe, moeSel, dMoeSel;     // grouped 8-bit input / gradient, select logits fp32, their gradient
@@ -197,8 +213,9 @@ int BackpropDelta(ts2_model *M, TMatrix &W, const Arr &src8, const Arr &gradFast
 int FfnComputeRG(ts2_model *M, TLayer &L, const Arr &norm8, void *s)
 {
     int D = M->cfg.dim, F = M->cfg.ffnDim, len = M->len, R = M->R;
-    Arr wideRaw = View(M->raw, R, F), wide16 = View(M->a16[0], R, F), gate16 = View(M->a16[1], R, F), wideScale = View(M->tsc[0], F / 128, R);
-    Arr rg8 = View(M->rg8, R, F);
+    TActs &A = *L.acts;
+    Arr wideRaw = View(M->raw, R, F), wide16 = View(A.a16[0], R, F), gate16 = View(A.a16[1], R, F), wideScale = View(A.tsc[0], F / 128, R);
+    Arr rg8 = View(A.rg8, R, F);
     // wide = MulForward(n, We) in true units, then per-tile normalisation to 1/24 units + tile scale
     CK(Forward(M, L.w[0], norm8, VEC * DISCR * Dot(D), true, wideRaw, false, s));
     CK(ts2_row_tile_normalize_rope(len, R, wideRaw.P(), TS2_F32, 1.f, 1, VEC, nullptr, wide16.P(), wideScale.P(), s));
@@ -211,15 +228,18 @@ int FfnForward(ts2_model *M, TLayer &L, const Arr &norm8, void *s)
 {
     int F = M->cfg.ffnDim;
     CK(FfnComputeRG(M, L, norm8, s));
-    return Forward(M, L.w[2], View(M->rg8, M->R, F), VEC * DISCR * Dot(F), true, M->state, true, s);
+    return Forward(M, L.w[2], View(L.acts->rg8, M->R, F), VEC * DISCR * Dot(F), true, M->state, true, s);
 }
 
 int FfnBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScale, void *s)
 {
     int D = M->cfg.dim, F = M->cfg.ffnDim, len = M->len, R = M->R;
-    Arr wide16 = View(M->a16[0], R, F), gate16 = View(M->a16[1], R, F), wideScale = View(M->tsc[0], F / 128, R), rg8 = View(M->rg8, R, F);
+    TActs &A = *L.acts;
+    Arr wide16 = View(A.a16[0], R, F), gate16 = View(A.a16[1], R, F), wideScale = View(A.tsc[0], F / 128, R), rg8 = View(A.rg8, R, F);
     Arr drg = View(M->g32, R, F), dwide = View(M->gf[0], R, F), dgate = View(M->gf[1], R, F);
-    CK(FfnComputeRG(M, L, norm8, s));
+    if (!(M->useKept && A.valid)) {
+        CK(FfnComputeRG(M, L, norm8, s));
+    }
     // contract backward
     CK(BackpropDX(M, L.w[2], M->stateGradFast, DISCR * Dot(F), true, drg, false, s));
     CK(ts2_backprop_row_tile_normalize_lolu(len, R, gate16.P(), wide16.P(), VEC, wideScale.P(), drg.P(), TS2_F32, dgate.P(), dwide.P(),
@@ -242,8 +262,9 @@ float AttDotScale()
 int AttComputeVLG(ts2_model *M, TLayer &L, const Arr &norm8, void *s)
 {
     int D = M->cfg.dim, H = M->cfg.headCount, Q = H * 128, len = M->len, R = M->R;
-    Arr raw = View(M->raw, R, Q), q16 = View(M->a16[0], R, Q), gate16 = View(M->a16[1], R, Q), k16 = View(M->a16[2], R, Q), v16 = View(M->a16[3], R, Q);
-    Arr qScale = View(M->tsc[0], H, R), vScale = View(M->tsc[1], H, R), val16 = View(M->g16[0], R, Q), vlg8 = View(M->rg8, R, Q);
+    TActs &A = *L.acts;
+    Arr raw = View(M->raw, R, Q), q16 = View(A.a16[0], R, Q), gate16 = View(A.a16[1], R, Q), k16 = View(A.a16[2], R, Q), v16 = View(A.a16[3], R, Q);
+    Arr qScale = View(A.tsc[0], H, R), vScale = View(A.tsc[1], H, R), val16 = View(A.val16, R, Q), vlg8 = View(A.rg8, R, Q);
     float a = VEC * DISCR * Dot(D);
     CK(Forward(M, L.w[0], norm8, a, true, raw, false, s));
     CK(ts2_row_tile_normalize_rope(len, R, raw.P(), TS2_F32, 1.f, 1, 1.f, M->rope.P(), q16.P(), qScale.P(), s));
@@ -264,7 +285,7 @@ int AttComputeVLG(ts2_model *M, TLayer &L, const Arr &norm8, void *s)
     at.attDotScale = AttDotScale();
     at.alibiSlope = L.slope;
     at.valLookup = val16.m;
-    at.sumWeightLog = M->swl.m;
+    at.sumWeightLog = A.swl.m;
     CK(ts2_att_forward(&at, s));
     // VLG = sigmoid(2 gate) * val in 1/24 units
     return ts2_matrix_lolu(len, R, gate16.P(), val16.P(), 24.f, vlg8.P(), M->mode, s);
@@ -274,16 +295,20 @@ int AttForward(ts2_model *M, TLayer &L, const Arr &norm8, void *s)
 {
     int TT = M->cfg.headCount * 128;
     CK(AttComputeVLG(M, L, norm8, s));
-    return Forward(M, L.w[4], View(M->rg8, M->R, TT), VEC * DISCR * Dot(TT), true, M->state, true, s);
+    return Forward(M, L.w[4], View(L.acts->rg8, M->R, TT), VEC * DISCR * Dot(TT), true, M->state, true, s);
 }
 
 int AttBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScale, void *s)
 {
     int D = M->cfg.dim, H = M->cfg.headCount, Q = H * 128, len = M->len, R = M->R;
-    Arr q16 = View(M->a16[0], R, Q), gate16 = View(M->a16[1], R, Q), k16 = View(M->a16[2], R, Q), v16 = View(M->a16[3], R, Q);
-    Arr qScale = View(M->tsc[0], H, R), vScale = View(M->tsc[1], H, R), val16 = View(M->g16[0], R, Q), vlg8 = View(M->rg8, R, Q);
+    TActs &A = *L.acts;
+    Arr q16 = View(A.a16[0], R, Q), gate16 = View(A.a16[1], R, Q), k16 = View(A.a16[2], R, Q), v16 = View(A.a16[3], R, Q);
+    Arr qScale = View(A.tsc[0], H, R), vScale = View(A.tsc[1], H, R), val16 = View(A.val16, R, Q), vlg8 = View(A.rg8, R, Q);
     Arr dvlg = View(M->g32, R, Q), dGate = View(M->gf[1], R, Q), dVal16 = View(M->g16[1], R, Q);
-    CK(AttComputeVLG(M, L, norm8, s));
+    if (!(M->useKept && A.valid)) {
+        CK(AttComputeVLG(M, L, norm8, s));
+    }
+    A.valid = false; // the backward reuses val16's storage for dQ
     // combiner backward
     CK(BackpropDX(M, L.w[4], M->stateGradFast, DISCR * Dot(Q), true, dvlg, false, s));
     CK(BackpropDelta(M, L.w[4], vlg8, M->stateGradFast, VEC, gradScale, s));
@@ -291,7 +316,7 @@ int AttBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
     CK(ts2_backprop_lolu_dscale(len, R, gate16.P(), val16.P(), 1.f, dvlg.P(), TS2_F32, dGate.P(), M->fastGradType, dVal16.P(), TS2_BF16,
         M->dScale.P(), s));
     // attention backward (dQ, dK, dV in bf16; val16's buffer is reused for dQ once dScale is known)
-    Arr dQ = View(M->g16[0], R, Q), dK = View(M->g16[2], R, Q), dV = View(M->g16[3], R, Q);
+    Arr dQ = View(A.val16, R, Q), dK = View(M->g16[2], R, Q), dV = View(M->g16[3], R, Q);
     ts2_att_grad_args ag = {};
     ag.len = len;
     ag.lenRound = R;
@@ -306,7 +331,7 @@ int AttBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
     ag.revHi = M->revHi[L.attId];
     ag.attDotScale = AttDotScale();
     ag.alibiSlope = L.slope;
-    ag.sumWeightLog = M->swl.m;
+    ag.sumWeightLog = A.swl.m;
     ag.dScale = M->dScale.m;
     ag.dQ = dQ.m;
     ag.dK = dK.m;
@@ -392,8 +417,9 @@ int MoeComputeRG(ts2_model *M, TLayer &L, const Arr &norm8, void *s)
     CK(Forward(M, L.w[3], norm8, a, false, M->moeSel, false, s));
     CK(ts2_moe_route(len, RM, E, K, M->moeSel.P(), TS2_F32, &M->moe, s));
     CK(ts2_moe_group_samples(RM, 1, norm8.P(), M->moe.xpSampleId, M->normMoe.P(), s));
-    Arr wideRaw = View(M->raw, RM, X), wide16 = View(M->a16[0], RM, X), gate16 = View(M->a16[1], RM, X), wideScale = View(M->tsc[0], X / 128, RM);
-    Arr rg8 = View(M->rg8, RM, X);
+    TActs &A = M->shared;
+    Arr wideRaw = View(M->raw, RM, X), wide16 = View(A.a16[0], RM, X), gate16 = View(A.a16[1], RM, X), wideScale = View(A.tsc[0], X / 128, RM);
+    Arr rg8 = View(A.rg8, RM, X);
     CK(GroupedGemm(M, M->normMoe, L.w[0].fast, X, X, D, wideRaw, a, L.w[0].scale, false, s));
     CK(ts2_row_tile_normalize_rope(RM, RM, wideRaw.P(), TS2_F32, 1.f, 1, VEC, nullptr, wide16.P(), wideScale.P(), s));
     CK(GroupedGemm(M, M->normMoe, L.w[1].fast, X, X, D, gate16, a, nullptr, false, s));
@@ -405,7 +431,7 @@ int MoeForward(ts2_model *M, TLayer &L, const Arr &norm8, void *s)
     int D = M->cfg.dim, X = M->cfg.expertDim, E = M->cfg.expertCount, RM = M->lenMoe;
     CK(MoeComputeRG(M, L, norm8, s));
     Arr contract = View(M->g32, RM, D);
-    CK(GroupedGemm(M, View(M->rg8, RM, X), L.w[2].fast, D, D, X, contract, VEC * DISCR * Dot(E * X), L.w[2].scale, false, s));
+    CK(GroupedGemm(M, View(M->shared.rg8, RM, X), L.w[2].fast, D, D, X, contract, VEC * DISCR * Dot(E * X), L.w[2].scale, false, s));
     return ts2_combine_experts(M->len, M->cfg.moeSelected, contract.P(), TS2_F32, &M->moe, 1.f, nullptr, M->state.P(), 1, s);
 }
 
@@ -413,7 +439,8 @@ int MoeBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
 {
     int D = M->cfg.dim, X = M->cfg.expertDim, E = M->cfg.expertCount, K = M->cfg.moeSelected, len = M->len, R = M->R, RM = M->lenMoe;
     CK(MoeComputeRG(M, L, norm8, s));
-    Arr wide16 = View(M->a16[0], RM, X), gate16 = View(M->a16[1], RM, X), wideScale = View(M->tsc[0], X / 128, RM), rg8 = View(M->rg8, RM, X);
+    TActs &A = M->shared;
+    Arr wide16 = View(A.a16[0], RM, X), gate16 = View(A.a16[1], RM, X), wideScale = View(A.tsc[0], X / 128, RM), rg8 = View(A.rg8, RM, X);
     // state gradient into expert order
     CK(ts2_moe_group_samples(RM, 1, M->stateGradFast.P(), M->moe.xpSampleId, M->sgMoe.P(), s));
     // contract backward: dRG[row][x] = sum_d sg[row][d] Wc_e[d][x]: needs Wc_e^T = [X][D] per expert
@@ -476,13 +503,16 @@ int LayerForward(ts2_model *M, int d, void *s)
     TLayer &L = M->layers[d];
     const Arr &n8 = M->normState[d];
     if (L.type == LT_FFN) {
-        return FfnForward(M, L, n8, s);
+        CK(FfnForward(M, L, n8, s));
     } else if (L.type == LT_ATT) {
-        return AttForward(M, L, n8, s);
+        CK(AttForward(M, L, n8, s));
     } else if (L.type == LT_MOE) {
         return MoeForward(M, L, n8, s);
+    } else {
+        return TS2_ERR_UNSUPPORTED;
     }
-    return TS2_ERR_UNSUPPORTED;
+    L.acts->valid = L.acts != &M->shared; // a set of its own still holds this layer's activations when its backward runs
+    return 0;
 }
 
 int LayerBackward(ts2_model *M, int d, const float *gradScale, void *s)
@@ -570,6 +600,11 @@ int ModelBackprop(ts2_model *M, void *s)
     CK(ModelForward(M, s));
     CK(Ts2ZeroRows(Flat(M->gradMaxNorm, 1, depth + 2, TS2_F32).P(), 1, (depth + 2) * 4, s));
     CK(FinalBackward(M, s));
+    M->useKept = M->keep;
+    struct TReset {
+        ts2_model *M;
+        ~TReset() { M->useKept = false; }
+    } reset = {M};
     int stepId = 0;
     for (int d = depth - 1; d >= 0; --d, ++stepId) {
         float *prevMax = M->gradMaxNorm + stepId, *nextMax = M->gradMaxNorm + stepId + 1;
@@ -674,14 +709,52 @@ extern "C" ts2_model *ts2_model_create(const ts2_model_config *cfg)
     M->lossSum = (float *)M->Dev(4);
     // layer scratch
     int RP = M->RP;
-    ok &= M->Alloc(&M->raw, RP, maxW, TS2_F32) && M->Alloc(&M->g32, RP, maxW, TS2_F32) && M->Alloc(&M->rg8, RP, maxW, M->mode);
+    ok &= M->Alloc(&M->raw, RP, maxW, TS2_F32) && M->Alloc(&M->g32, RP, maxW, TS2_F32) && M->Alloc(&M->shared.rg8, RP, maxW, M->mode);
     for (int k = 0; k < 4; ++k) {
-        ok &= M->Alloc(&M->a16[k], RP, maxW, TS2_BF16) && M->Alloc(&M->g16[k], RP, maxW, TS2_BF16) && M->Alloc(&M->gf[k], RP, maxW, M->fastGradType);
+        ok &= M->Alloc(&M->shared.a16[k], RP, maxW, TS2_BF16) && M->Alloc(&M->g16[k], RP, maxW, TS2_BF16) &&
+              M->Alloc(&M->gf[k], RP, maxW, M->fastGradType);
     }
-    for (int k = 0; k < 3; ++k) {
-        ok &= M->Alloc(&M->tsc[k], maxW / 128, RP, TS2_F32);
+    for (int k = 0; k < 2; ++k) {
+        ok &= M->Alloc(&M->shared.tsc[k], maxW / 128, RP, TS2_F32);
     }
-    ok &= M->Alloc(&M->swl, H > 0 ? H : 1, R, TS2_F32) && M->Alloc(&M->dScale, H > 0 ? H : 1, R, TS2_F32);
+    ok &= M->Alloc(&M->shared.val16, RP, maxW, TS2_BF16);
+    ok &= M->Alloc(&M->shared.swl, H > 0 ? H : 1, R, TS2_F32) && M->Alloc(&M->dScale, H > 0 ? H : 1, R, TS2_F32);
+    // per-layer activation sets when they fit into half of the free device memory, else every layer shares one set and recomputes
+    {
+        size_t need = 0;
+        for (int d = 0; d < cfg->depth; ++d) {
+            int w = M->layers[d].type == LT_FFN ? F : H * 128;
+            if (M->layers[d].type == LT_FFN) {
+                need += (size_t)R * w * 5 + (size_t)R * (w / 128) * 4;
+            } else if (M->layers[d].type == LT_ATT) {
+                need += (size_t)R * w * 11 + (size_t)R * H * 12;
+            }
+        }
+        size_t freeB = 0, totalB = 0;
+        bool fits = hipMemGetInfo(&freeB, &totalB) == hipSuccess && need < freeB / 2;
+        M->keep = ok && fits && cfg->recompute == 0;
+        M->acts.resize(cfg->depth);
+        for (int d = 0; d < cfg->depth && ok; ++d) {
+            TLayer &L = M->layers[d];
+            TActs &A = M->acts[d];
+            L.acts = &M->shared;
+            if (!M->keep || L.type == LT_MOE) {
+                continue;
+            }
+            L.acts = &A;
+            if (L.type == LT_FFN) {
+                ok &= M->Alloc(&A.a16[0], R, F, TS2_BF16) && M->Alloc(&A.a16[1], R, F, TS2_BF16) && M->Alloc(&A.tsc[0], F / 128, R, TS2_F32) &&
+                      M->Alloc(&A.rg8, R, F, M->mode);
+            } else {
+                int Q = H * 128;
+                for (int k = 0; k < 4; ++k) {
+                    ok &= M->Alloc(&A.a16[k], R, Q, TS2_BF16);
+                }
+                ok &= M->Alloc(&A.tsc[0], H, R, TS2_F32) && M->Alloc(&A.tsc[1], H, R, TS2_F32) && M->Alloc(&A.val16, R, Q, TS2_BF16) &&
+                      M->Alloc(&A.rg8, R, Q, M->mode) && M->Alloc(&A.swl, H, R, TS2_F32);
+            }
+        }
+    }
     // keep the two statistics arrays on one stride
     M->sGrad8 = (uint8_t *)M->Dev((size_t)RP * maxW);
     M->sGradT = (uint8_t *)M->Dev((size_t)RP * maxW);
