@@ -48,32 +48,50 @@ struct AttP {
     int lenRound;
 };
 
-// coalesced copy of a TR x 128 bf16 tile into a row-major LDS tile
-__device__ __forceinline__ void LoadTile(uint8_t *lds, const uint8_t *g, int64_t ld, int tid)
+// Streamed tiles are fetched one tile ahead into registers (the loads of tile i+1 are in flight while tile i is multiplied) and go
+// from there to LDS row-major and/or transposed, so a tile costs two workgroup barriers and no LDS-to-LDS pass.  A thread holds two
+// pairs of neighbouring rows (16 bytes of each): lane -> 64 contiguous bytes of a row per 4 lanes, 16 row pairs per wave; with
+// this mapping the dword writes of the transposed copy (two rows per dword) fall into 64 different banks.
+struct TilePref {
+    v4i a[2][2];
+};
+
+__device__ __forceinline__ void TileSlot(int tid, int i, int *r2, int *c)
+{
+    int lane = tid & 63, combo = (tid >> 6) + 4 * i;
+    *r2 = (combo & 1) * 16 + (lane >> 2);
+    *c = (combo >> 1) * 4 + (lane & 3);
+}
+
+__device__ __forceinline__ void PrefetchTile(TilePref &r, const uint8_t *g, int64_t ld, int tid)
 {
 #pragma unroll
-    for (int i = 0; i < TR * 16 / 256; ++i) {
-        int id = tid + 256 * i;
-        int row = id >> 4, c = id & 15;
-        *(v4i *)(lds + row * RP + c * 16) = *(const v4i *)(g + (int64_t)row * ld + c * 16);
+    for (int i = 0; i < 2; ++i) {
+        int r2, c;
+        TileSlot(tid, i, &r2, &c);
+        r.a[i][0] = *(const v4i *)(g + (int64_t)(2 * r2) * ld + c * 16);
+        r.a[i][1] = *(const v4i *)(g + (int64_t)(2 * r2 + 1) * ld + c * 16);
     }
 }
 
-// row-major LDS tile -> transposed LDS tile T[d][row], two rows per dword
-__device__ __forceinline__ void TransposeTile(uint8_t *t, const uint8_t *rm, int tid)
+template <bool RM, bool T> __device__ __forceinline__ void StoreTile(const TilePref &r, uint8_t *rm, uint8_t *t, int tid)
 {
-    int r2 = tid & 31;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-        int c = (tid >> 5) + 8 * i;
-        v4i a0 = *(const v4i *)(rm + (2 * r2) * RP + c * 16);
-        v4i a1 = *(const v4i *)(rm + (2 * r2 + 1) * RP + c * 16);
+        int r2, c;
+        TileSlot(tid, i, &r2, &c);
+        if (RM) {
+            *(v4i *)(rm + (2 * r2) * RP + c * 16) = r.a[i][0];
+            *(v4i *)(rm + (2 * r2 + 1) * RP + c * 16) = r.a[i][1];
+        }
+        if (T) {
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            uint32_t lo = __builtin_amdgcn_perm((uint32_t)a1[w], (uint32_t)a0[w], 0x05040100);
-            uint32_t hi = __builtin_amdgcn_perm((uint32_t)a1[w], (uint32_t)a0[w], 0x07060302);
-            *(uint32_t *)(t + (8 * c + 2 * w) * TP + 4 * r2) = lo;
-            *(uint32_t *)(t + (8 * c + 2 * w + 1) * TP + 4 * r2) = hi;
+            for (int w = 0; w < 4; ++w) {
+                uint32_t lo = __builtin_amdgcn_perm((uint32_t)r.a[i][1][w], (uint32_t)r.a[i][0][w], 0x05040100);
+                uint32_t hi = __builtin_amdgcn_perm((uint32_t)r.a[i][1][w], (uint32_t)r.a[i][0][w], 0x07060302);
+                *(uint32_t *)(t + (8 * c + 2 * w) * TP + 4 * r2) = lo;
+                *(uint32_t *)(t + (8 * c + 2 * w + 1) * TP + 4 * r2) = hi;
+            }
         }
     }
 }
@@ -163,20 +181,56 @@ __device__ __forceinline__ void BlockKeyRange(int start, int finish, int tid, in
     *hi = max(max(red[1], red[3]), max(red[5], red[7]));
 }
 
+// span of the lane's own row in a form that needs one unsigned compare per key, plus the wave-wide bounds that tell whether a tile
+// is seen completely, partly or not at all by the 32 rows of the wave
+struct TRowSpan {
+    int start;     // 0x7fffffff for an empty span
+    unsigned len;  // finish - start (0 for an empty span, whose start makes every compare fail)
+    int waveMaxStart, waveMinFinish, waveMinStart, waveMaxFinish;
+};
+
+__device__ __forceinline__ TRowSpan MakeRowSpan(int start, int finish)
+{
+    TRowSpan r;
+    bool some = finish >= start;
+    r.start = some ? start : 0x7fffffff;
+    r.len = some ? (unsigned)(finish - start) : 0u;
+    int a = r.start, b = some ? finish : -1, c = r.start, d = b;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        a = max(a, __shfl_xor(a, o, 64));
+        b = min(b, __shfl_xor(b, o, 64));
+        c = min(c, __shfl_xor(c, o, 64));
+        d = max(d, __shfl_xor(d, o, 64));
+    }
+    r.waveMaxStart = a;
+    r.waveMinFinish = b;
+    r.waveMinStart = c;
+    r.waveMaxFinish = d;
+    return r;
+}
+
 // ---------------------------------------------------------------------------------------------------------------------------
 // forward: grid (lenRound/128, heads)
 __global__ void __launch_bounds__(256) AttForward(AttP p)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    uint8_t *kRm = lds, *vRm = lds + RM_BYTES, *vT = lds + 2 * RM_BYTES;
+    uint8_t *kRm = lds, *vT = lds + RM_BYTES;
     __shared__ int red[8];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
     const int head = blockIdx.y;
-    const int myRow = blockIdx.x * BROWS + wave * WROWS + l32;
+    // later query blocks of a causal sequence see more keys: they start first so that the short ones fill the tail of the launch
+    const int myRow = (gridDim.x - 1 - blockIdx.x) * BROWS + wave * WROWS + l32;
     const int64_t hoff = (int64_t)head * HD * 2;
     const int start = p.spanStart[myRow], finish = p.spanFinish[myRow];
     int kLo, kHi;
     BlockKeyRange(start, finish, tid, &kLo, &kHi, red);
+    const int tFirst = kHi >= kLo ? (kLo / TR) * TR : 1;
+    TilePref pk, pv;
+    if (tFirst <= kHi) {
+        PrefetchTile(pk, p.k + (int64_t)tFirst * p.ldk + hoff, p.ldk, tid);
+        PrefetchTile(pv, p.v + (int64_t)tFirst * p.ldv + hoff, p.ldv, tid);
+    }
 
     v8bf qf[8];
     LoadOwnFrags(qf, p.q + (int64_t)(myRow - l32) * p.ldq + hoff, p.ldq, l32, half);
@@ -189,46 +243,80 @@ __global__ void __launch_bounds__(256) AttForward(AttP p)
         }
     }
     float m = 0, sum = 1; // the sink: a zero vector with weight 2^-m
-    for (int t0 = kHi >= kLo ? (kLo / TR) * TR : 1; t0 <= kHi; t0 += TR) {
+    const TRowSpan sp = MakeRowSpan(start, finish);
+    for (int t0 = tFirst; t0 <= kHi; t0 += TR) {
         __syncthreads();
-        LoadTile(kRm, p.k + (int64_t)t0 * p.ldk + hoff, p.ldk, tid);
-        LoadTile(vRm, p.v + (int64_t)t0 * p.ldv + hoff, p.ldv, tid);
+        StoreTile<true, false>(pk, kRm, nullptr, tid);
+        StoreTile<false, true>(pv, nullptr, vT, tid);
         __syncthreads();
-        TransposeTile(vT, vRm, tid);
-        __syncthreads();
+        if (t0 + TR <= kHi) {
+            PrefetchTile(pk, p.k + (int64_t)(t0 + TR) * p.ldk + hoff, p.ldk, tid);
+            PrefetchTile(pv, p.v + (int64_t)(t0 + TR) * p.ldv + hoff, p.ldv, tid);
+        }
+        if (t0 > sp.waveMaxFinish || t0 + TR - 1 < sp.waveMinStart) {
+            continue; // no row of this wave sees a key of the tile (wave-uniform)
+        }
+        // phase 1: scores of all 64 keys of the tile (two independent accumulator chains)
+        constexpr int NB = TR / 32;
+        v16f s[NB];
 #pragma unroll
-        for (int kb = 0; kb < TR / 32; ++kb) {
-            int keyBase = t0 + kb * 32;
-            v16f s;
+        for (int kb = 0; kb < NB; ++kb) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                s[e] = 0;
+                s[kb][e] = 0;
             }
+        }
 #pragma unroll
-            for (int ds = 0; ds < 8; ++ds) {
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(kRm, kb, ds, l32, half), qf[ds], s, 0, 0, 0);
+        for (int ds = 0; ds < 8; ++ds) {
+#pragma unroll
+            for (int kb = 0; kb < NB; ++kb) {
+                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(kRm, kb, ds, l32, half), qf[ds], s[kb], 0, 0, 0);
             }
-            float sv[16];
-            float mx = m;
+        }
+        // phase 2: one running-max update per tile.  logit = s*scale - slope*(row - key); tiles that every row of the wave sees
+        // completely skip the span tests
+        float sv[NB][16];
+        float mx = m;
+        const float kc = p.slope * (float)(t0 + half * 4 - myRow); // small exact integer times the slope
+        const bool full = t0 >= sp.waveMaxStart && t0 + TR - 1 <= sp.waveMinFinish;
+        if (full) {
+#pragma unroll
+            for (int kb = 0; kb < NB; ++kb) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    sv[kb][e] = fmaf(s[kb][e], p.attDotScale, fmaf(p.slope, (float)(kb * 32 + BlkRow(e, 0)), kc));
+                    mx = fmaxf(mx, sv[kb][e]);
+                }
+            }
+        } else {
+            const int rel0 = t0 + half * 4 - sp.start;
+#pragma unroll
+            for (int kb = 0; kb < NB; ++kb) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    bool valid = (unsigned)(rel0 + kb * 32 + BlkRow(e, 0)) <= sp.len;
+                    float x = fmaf(s[kb][e], p.attDotScale, fmaf(p.slope, (float)(kb * 32 + BlkRow(e, 0)), kc));
+                    sv[kb][e] = valid ? x : -INFINITY;
+                    mx = fmaxf(mx, sv[kb][e]);
+                }
+            }
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        float alpha = __builtin_amdgcn_exp2f(m - mx);
+        const bool rescale = __any(mx != m);
+        m = mx;
+        float ps = 0;
+#pragma unroll
+        for (int kb = 0; kb < NB; ++kb) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                int key = keyBase + BlkRow(e, half);
-                bool valid = key >= start && key <= finish;
-                float dp = s[e] * p.attDotScale - p.slope * (float)(myRow - key);
-                sv[e] = valid ? dp : -INFINITY;
-                mx = fmaxf(mx, sv[e]);
+                sv[kb][e] = __builtin_amdgcn_exp2f(sv[kb][e] - m); // exp2(-inf) = 0 for masked keys
+                ps += sv[kb][e];
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            float alpha = exp2f(m - mx);
-            m = mx;
-            float ps = 0;
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                sv[e] = exp2f(sv[e] - m); // exp2(-inf) = 0 for masked keys
-                ps += sv[e];
-            }
-            ps += __shfl_xor(ps, 32, 64);
-            sum = sum * alpha + ps;
+        }
+        ps += __shfl_xor(ps, 32, 64);
+        sum = sum * alpha + ps;
+        if (rescale) { // wave-uniform: the maximum of no row moved in most tiles
 #pragma unroll
             for (int db = 0; db < 4; ++db) {
 #pragma unroll
@@ -236,11 +324,19 @@ __global__ void __launch_bounds__(256) AttForward(AttP p)
                     oacc[db][e] *= alpha;
                 }
             }
-            v8bf pb0 = PackB(sv, 0), pb1 = PackB(sv, 1);
+        }
+        // phase 3: O^T += V^T P^T, neighbouring MFMAs on different accumulators
+        v8bf pb[NB][2];
+#pragma unroll
+        for (int kb = 0; kb < NB; ++kb) {
+            pb[kb][0] = PackB(sv[kb], 0);
+            pb[kb][1] = PackB(sv[kb], 1);
+        }
+#pragma unroll
+        for (int ks = 0; ks < 2 * NB; ++ks) {
 #pragma unroll
             for (int db = 0; db < 4; ++db) {
-                oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(vT, db, kb * 2, l32, half), pb0, oacc[db], 0, 0, 0);
-                oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(vT, db, kb * 2 + 1, l32, half), pb1, oacc[db], 0, 0, 0);
+                oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(vT, db, ks, l32, half), pb[ks >> 1][ks & 1], oacc[db], 0, 0, 0);
             }
         }
     }
@@ -259,11 +355,18 @@ template <bool F32> __global__ void __launch_bounds__(256) AttGradQ(AttP p)
     __shared__ int red[8];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
     const int head = blockIdx.y;
-    const int myRow = blockIdx.x * BROWS + wave * WROWS + l32;
+    // later query blocks of a causal sequence see more keys: they start first so that the short ones fill the tail of the launch
+    const int myRow = (gridDim.x - 1 - blockIdx.x) * BROWS + wave * WROWS + l32;
     const int64_t hoff = (int64_t)head * HD * 2;
     const int start = p.spanStart[myRow], finish = p.spanFinish[myRow];
     int kLo, kHi;
     BlockKeyRange(start, finish, tid, &kLo, &kHi, red);
+    const int tFirst = kHi >= kLo ? (kLo / TR) * TR : 1;
+    TilePref pk, pv;
+    if (tFirst <= kHi) {
+        PrefetchTile(pk, p.k + (int64_t)tFirst * p.ldk + hoff, p.ldk, tid);
+        PrefetchTile(pv, p.v + (int64_t)tFirst * p.ldv + hoff, p.ldv, tid);
+    }
 
     v8bf qf[8], dof[8];
     LoadOwnFrags(qf, p.q + (int64_t)(myRow - l32) * p.ldq + hoff, p.ldq, l32, half);
@@ -271,6 +374,7 @@ template <bool F32> __global__ void __launch_bounds__(256) AttGradQ(AttP p)
     const float L = p.sumWeightLog[(int64_t)head * p.ldStat + myRow];
     const float dScale = p.dScale[(int64_t)head * p.ldStat + myRow];
     const float gmul = p.attDotScale * LN2;
+    const TRowSpan sp = MakeRowSpan(start, finish);
     v16f acc[4];
 #pragma unroll
     for (int db = 0; db < 4; ++db) {
@@ -279,41 +383,60 @@ template <bool F32> __global__ void __launch_bounds__(256) AttGradQ(AttP p)
             acc[db][e] = 0;
         }
     }
-    for (int t0 = kHi >= kLo ? (kLo / TR) * TR : 1; t0 <= kHi; t0 += TR) {
+    for (int t0 = tFirst; t0 <= kHi; t0 += TR) {
         __syncthreads();
-        LoadTile(kRm, p.k + (int64_t)t0 * p.ldk + hoff, p.ldk, tid);
-        LoadTile(vRm, p.v + (int64_t)t0 * p.ldv + hoff, p.ldv, tid);
+        StoreTile<true, true>(pk, kRm, kT, tid);
+        StoreTile<true, false>(pv, vRm, nullptr, tid);
         __syncthreads();
-        TransposeTile(kT, kRm, tid);
-        __syncthreads();
+        if (t0 + TR <= kHi) {
+            PrefetchTile(pk, p.k + (int64_t)(t0 + TR) * p.ldk + hoff, p.ldk, tid);
+            PrefetchTile(pv, p.v + (int64_t)(t0 + TR) * p.ldv + hoff, p.ldv, tid);
+        }
+        if (t0 > sp.waveMaxFinish || t0 + TR - 1 < sp.waveMinStart) {
+            continue; // no row of this wave sees a key of the tile (wave-uniform)
+        }
+        constexpr int NB = TR / 32;
+        v16f s[NB], dp[NB];
 #pragma unroll
-        for (int kb = 0; kb < TR / 32; ++kb) {
-            int keyBase = t0 + kb * 32;
-            v16f s, dp;
+        for (int kb = 0; kb < NB; ++kb) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                s[e] = 0;
-                dp[e] = 0;
+                s[kb][e] = 0;
+                dp[kb][e] = 0;
             }
+        }
+        // phase 1: S^T and dP^T of the whole tile, four independent accumulator chains
 #pragma unroll
-            for (int ds = 0; ds < 8; ++ds) {
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(kRm, kb, ds, l32, half), qf[ds], s, 0, 0, 0);
-                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(vRm, kb, ds, l32, half), dof[ds], dp, 0, 0, 0);
+        for (int ds = 0; ds < 8; ++ds) {
+#pragma unroll
+            for (int kb = 0; kb < NB; ++kb) {
+                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(kRm, kb, ds, l32, half), qf[ds], s[kb], 0, 0, 0);
+                dp[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(vRm, kb, ds, l32, half), dof[ds], dp[kb], 0, 0, 0);
             }
+        }
+        // phase 2: dS
+        v8bf sb[NB][2];
+        const float kc = p.slope * (float)(t0 + half * 4 - myRow) - L; // logit - L in one fma chain
+        const int rel0 = t0 + half * 4 - sp.start;
+#pragma unroll
+        for (int kb = 0; kb < NB; ++kb) {
             float dsv[16];
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                int key = keyBase + BlkRow(e, half);
-                bool valid = key >= start && key <= finish;
-                float x = s[e] * p.attDotScale - p.slope * (float)(myRow - key);
-                float w = valid ? exp2f(x - L) : 0.f;
-                dsv[e] = w * (dp[e] - dScale) * gmul;
+                float x = fmaf(s[kb][e], p.attDotScale, fmaf(p.slope, (float)(kb * 32 + BlkRow(e, 0)), kc));
+                float w = __builtin_amdgcn_exp2f(x);
+                w = (unsigned)(rel0 + kb * 32 + BlkRow(e, 0)) <= sp.len ? w : 0.f;
+                dsv[e] = w * (dp[kb][e] - dScale) * gmul;
             }
-            v8bf b0 = PackB(dsv, 0), b1 = PackB(dsv, 1);
+            sb[kb][0] = PackB(dsv, 0);
+            sb[kb][1] = PackB(dsv, 1);
+        }
+        // phase 3: dQ^T += K^T dS^T
+#pragma unroll
+        for (int ks = 0; ks < 2 * NB; ++ks) {
 #pragma unroll
             for (int db = 0; db < 4; ++db) {
-                acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(kT, db, kb * 2, l32, half), b0, acc[db], 0, 0, 0);
-                acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(kT, db, kb * 2 + 1, l32, half), b1, acc[db], 0, 0, 0);
+                acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(kT, db, ks, l32, half), sb[ks >> 1][ks & 1], acc[db], 0, 0, 0);
             }
         }
     }
@@ -330,11 +453,32 @@ template <bool F32> __global__ void __launch_bounds__(256) AttGradKV(AttP p)
     float *stD = stL + TR;
     int *stS = (int *)(stD + TR);
     int *stF = stS + TR;
+    int *stT = stF + TR; // [4] bounds over the tile's queries
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
     const int head = blockIdx.y;
     const int myRow = blockIdx.x * BROWS + wave * WROWS + l32; // my key
     const int64_t hoff = (int64_t)head * HD * 2;
     const int qLo = p.revLo[blockIdx.x], qHi = p.revHi[blockIdx.x];
+    const int tFirst = qHi >= qLo ? (qLo / TR) * TR : 1;
+    TilePref pq, pdo;
+    float preL = 0, preD = 0;
+    int preS = 0x7fffffff, preF = -1;
+    const int keyBase = blockIdx.x * BROWS;
+    auto prefetch = [&](int t0) {
+        PrefetchTile(pq, p.q + (int64_t)t0 * p.ldq + hoff, p.ldq, tid);
+        PrefetchTile(pdo, p.dO + (int64_t)t0 * p.lddo + hoff, p.lddo, tid);
+        if (tid < TR) {
+            // per query: -L - slope * (query - first key of the workgroup), dScale, span start (0x7fffffff if empty) and finish
+            preL = -p.sumWeightLog[(int64_t)head * p.ldStat + t0 + tid] - p.slope * (float)(t0 + tid - keyBase);
+            preD = p.dScale[(int64_t)head * p.ldStat + t0 + tid];
+            int st = p.spanStart[t0 + tid], fi = p.spanFinish[t0 + tid];
+            preS = fi >= st ? st : 0x7fffffff;
+            preF = fi >= st ? fi : -1;
+        }
+    };
+    if (tFirst <= qHi) {
+        prefetch(tFirst);
+    }
 
     v8bf kf[8], vf[8];
     LoadOwnFrags(kf, p.k + (int64_t)(myRow - l32) * p.ldk + hoff, p.ldk, l32, half);
@@ -349,63 +493,95 @@ template <bool F32> __global__ void __launch_bounds__(256) AttGradKV(AttP p)
             dv[db][e] = 0;
         }
     }
-    for (int t0 = qHi >= qLo ? (qLo / TR) * TR : 1; t0 <= qHi; t0 += TR) {
+    for (int t0 = tFirst; t0 <= qHi; t0 += TR) {
         __syncthreads();
-        LoadTile(qRm, p.q + (int64_t)t0 * p.ldq + hoff, p.ldq, tid);
-        LoadTile(doRm, p.dO + (int64_t)t0 * p.lddo + hoff, p.lddo, tid);
-        if (tid < TR) {
-            stL[tid] = p.sumWeightLog[(int64_t)head * p.ldStat + t0 + tid];
-            stD[tid] = p.dScale[(int64_t)head * p.ldStat + t0 + tid];
-            stS[tid] = p.spanStart[t0 + tid];
-            stF[tid] = p.spanFinish[t0 + tid];
+        StoreTile<true, true>(pq, qRm, qT, tid);
+        StoreTile<true, true>(pdo, doRm, doT, tid);
+        if (tid < TR) { // wave 0
+            stL[tid] = preL;
+            stD[tid] = preD;
+            stS[tid] = preS;
+            stF[tid] = (int)(preF >= preS ? (unsigned)(preF - preS) : 0u); // span length
+            int a = preS, b = preF, c = preS, d = preF;
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                a = max(a, __shfl_xor(a, o, 64));
+                b = min(b, __shfl_xor(b, o, 64));
+                c = min(c, __shfl_xor(c, o, 64));
+                d = max(d, __shfl_xor(d, o, 64));
+            }
+            if (tid == 0) {
+                stT[0] = a; // latest span start of the tile's queries
+                stT[1] = b; // earliest finish
+                stT[2] = c; // earliest start
+                stT[3] = d; // latest finish
+            }
         }
         __syncthreads();
-        TransposeTile(qT, qRm, tid);
-        TransposeTile(doT, doRm, tid);
-        __syncthreads();
+        if (t0 + TR <= qHi) {
+            prefetch(t0 + TR);
+        }
+        const int kw0 = myRow - l32; // first key of this wave
+        if (stT[3] < kw0 || stT[2] > kw0 + 31) {
+            continue; // no query of the tile sees a key of this wave (wave-uniform)
+        }
+        constexpr int NB = TR / 32;
+        v16f s[NB], dp[NB];
 #pragma unroll
-        for (int qb = 0; qb < TR / 32; ++qb) {
-            v16f s, dp;
+        for (int qb = 0; qb < NB; ++qb) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                s[e] = 0;
-                dp[e] = 0;
+                s[qb][e] = 0;
+                dp[qb][e] = 0;
             }
+        }
+        // phase 1: S and dP of the whole tile, four independent accumulator chains
 #pragma unroll
-            for (int ds = 0; ds < 8; ++ds) {
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(qRm, qb, ds, l32, half), kf[ds], s, 0, 0, 0);
-                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(doRm, qb, ds, l32, half), vf[ds], dp, 0, 0, 0);
+        for (int ds = 0; ds < 8; ++ds) {
+#pragma unroll
+            for (int qb = 0; qb < NB; ++qb) {
+                s[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(qRm, qb, ds, l32, half), kf[ds], s[qb], 0, 0, 0);
+                dp[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(doRm, qb, ds, l32, half), vf[ds], dp[qb], 0, 0, 0);
             }
+        }
+        // phase 2: P and dS from the per-query statistics of the tile
+        v8bf pb[NB][2], sb[NB][2];
+        const float ck = p.slope * (float)(myRow - keyBase);
+#pragma unroll
+        for (int qb = 0; qb < NB; ++qb) {
             float pv[16], dsv[16];
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 int qi = qb * 32 + g * 8 + half * 4;
                 float4 L4 = *(const float4 *)(stL + qi);
                 float4 D4 = *(const float4 *)(stD + qi);
-                int4 S4 = *(const int4 *)(stS + qi);
-                int4 F4 = *(const int4 *)(stF + qi);
                 const float Ls[4] = {L4.x, L4.y, L4.z, L4.w};
                 const float Ds[4] = {D4.x, D4.y, D4.z, D4.w};
+                int4 S4 = *(const int4 *)(stS + qi);
+                int4 N4 = *(const int4 *)(stF + qi);
                 const int Ss[4] = {S4.x, S4.y, S4.z, S4.w};
-                const int Fs[4] = {F4.x, F4.y, F4.z, F4.w};
+                const unsigned Ns[4] = {(unsigned)N4.x, (unsigned)N4.y, (unsigned)N4.z, (unsigned)N4.w};
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     int e = g * 4 + j;
-                    int qrow = t0 + qi + j;
-                    bool valid = myRow >= Ss[j] && myRow <= Fs[j];
-                    float x = s[e] * p.attDotScale - p.slope * (float)(qrow - myRow);
-                    float w = valid ? exp2f(x - Ls[j]) : 0.f;
+                    float w = __builtin_amdgcn_exp2f(fmaf(s[qb][e], p.attDotScale, Ls[j] + ck));
+                    w = (unsigned)(myRow - Ss[j]) <= Ns[j] ? w : 0.f;
                     pv[e] = w;
-                    dsv[e] = w * (dp[e] - Ds[j]) * gmul;
+                    dsv[e] = w * (dp[qb][e] - Ds[j]) * gmul;
                 }
             }
-            v8bf pb0 = PackB(pv, 0), pb1 = PackB(pv, 1), sb0 = PackB(dsv, 0), sb1 = PackB(dsv, 1);
+            pb[qb][0] = PackB(pv, 0);
+            pb[qb][1] = PackB(pv, 1);
+            sb[qb][0] = PackB(dsv, 0);
+            sb[qb][1] = PackB(dsv, 1);
+        }
+        // phase 3: dV^T += dO^T P, dK^T += Q^T dS; eight accumulators in turn
+#pragma unroll
+        for (int ks = 0; ks < 2 * NB; ++ks) {
 #pragma unroll
             for (int db = 0; db < 4; ++db) {
-                dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(doT, db, qb * 2, l32, half), pb0, dv[db], 0, 0, 0);
-                dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(doT, db, qb * 2 + 1, l32, half), pb1, dv[db], 0, 0, 0);
-                dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(qT, db, qb * 2, l32, half), sb0, dk[db], 0, 0, 0);
-                dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(qT, db, qb * 2 + 1, l32, half), sb1, dk[db], 0, 0, 0);
+                dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(doT, db, ks, l32, half), pb[ks >> 1][ks & 1], dv[db], 0, 0, 0);
+                dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(qT, db, ks, l32, half), sb[ks >> 1][ks & 1], dk[db], 0, 0, 0);
             }
         }
     }
@@ -494,7 +670,7 @@ extern "C" int ts2_att_forward(const ts2_att_args *a, void *stream)
     p.out0 = (uint8_t *)a->valLookup.ptr;
     p.ldo0 = a->valLookup.strideBytes;
     p.lenRound = a->lenRound;
-    int ldsBytes = 2 * RM_BYTES + T_BYTES;
+    int ldsBytes = RM_BYTES + T_BYTES;
     static bool done = false;
     if (!done) {
         if (SetAttr((const void *)AttForward, ldsBytes)) {
@@ -545,7 +721,7 @@ extern "C" int ts2_att_backward(const ts2_att_grad_args *a, void *stream)
     p.lenRound = a->lenRound;
     dim3 grid(a->lenRound / BROWS, a->heads);
     int ldsQ = 2 * RM_BYTES + T_BYTES;
-    int ldsKV = 2 * RM_BYTES + 2 * T_BYTES + 4 * TR * 4;
+    int ldsKV = 2 * RM_BYTES + 2 * T_BYTES + 4 * TR * 4 + 16;
     static bool done = false;
     if (!done) {
         if (SetAttr((const void *)AttGradQ<true>, ldsQ) || SetAttr((const void *)AttGradQ<false>, ldsQ) ||

@@ -42,60 +42,91 @@ __global__ void __launch_bounds__(256) EmbedBackward(int len, int dim, const int
 }
 
 // SoftMax base 2 with running max starting at 0 and the (onehot - p) gradient (src/gpt/compute/cpu_transformer.cpp:12-37,146-159).
-// One workgroup per row; logits fp32 [row][vocab] are overwritten by probabilities when keepProb, grad is bf16.
+// One workgroup per row; logits fp32 [row][vocab] are overwritten by probabilities when keepProb, grad is bf16.  Two passes over the
+// row with 16-byte accesses: the first finds the maximum and the sum together (the sum is rescaled whenever a lane's maximum grows),
+// the second, served by the caches, writes the gradient.  vocab is a multiple of 4.
 __global__ void __launch_bounds__(256) FinalSoftmaxGrad(int vocab, float *logits, int64_t ldLogits, const float *bias, const int *target,
     float gradMult, bf16_t *grad, int64_t ldGrad, float *lossSum, int keepProb)
 {
-    __shared__ float red[4];
-    __shared__ float bc;
+    __shared__ float redM[4], redS[4];
     int t = blockIdx.x;
     int tid = threadIdx.x;
     float *row = (float *)((uint8_t *)logits + (int64_t)t * ldLogits);
     bf16_t *grow = (bf16_t *)((uint8_t *)grad + (int64_t)t * ldGrad);
     int tg = target[t];
     if (tg < 0) {
-        for (int k = tid; k < vocab; k += 256) {
-            grow[k] = 0;
+        for (int k = tid * 4; k < vocab; k += 1024) {
+            *(uint2 *)(grow + k) = make_uint2(0, 0);
         }
         if (!keepProb) {
             return;
         }
     }
-    float mx = 0;
-    for (int k = tid; k < vocab; k += 256) {
-        mx = fmaxf(mx, row[k]);
-    }
-    mx = WaveMax(mx);
-    if ((tid & 63) == 0) {
-        red[tid >> 6] = mx;
-    }
-    __syncthreads();
-    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    __syncthreads();
-    float sum = 0;
-    for (int k = tid; k < vocab; k += 256) {
-        sum += exp2f(row[k] + bias[k] - mx);
-    }
-    sum = WaveSum(sum);
-    if ((tid & 63) == 0) {
-        red[tid >> 6] = sum;
-    }
-    __syncthreads();
-    if (tid == 0) {
-        bc = 1 / ((red[0] + red[1]) + (red[2] + red[3]));
-    }
-    __syncthreads();
-    float scale = bc;
-    for (int k = tid; k < vocab; k += 256) {
-        float p = exp2f(row[k] + bias[k] - mx) * scale;
-        if (keepProb) {
-            row[k] = p;
+    // lane-local running maximum m (of the logits without bias, never below 0) and sum of 2^(x + bias - m)
+    float m = 0, sum = 0;
+    for (int k0 = tid * 4; k0 < vocab; k0 += 4096) {
+        float4 x[4], bv[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            int k = k0 + i * 1024;
+            bool in = k < vocab;
+            x[i] = in ? *(const float4 *)(row + k) : make_float4(-1e30f, -1e30f, -1e30f, -1e30f);
+            bv[i] = in ? *(const float4 *)(bias + k) : make_float4(0, 0, 0, 0);
         }
-        if (tg >= 0) {
-            float g = (k == tg ? 1.f : 0.f) - p;
-            grow[k] = FloatToBf16(g * gradMult);
-            if (k == tg && lossSum) {
-                atomicAdd(lossSum, logf(p));
+        float mNew = m;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            mNew = fmaxf(mNew, fmaxf(fmaxf(x[i].x, x[i].y), fmaxf(x[i].z, x[i].w)));
+        }
+        sum *= exp2f(m - mNew);
+        m = mNew;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            sum += (exp2f(x[i].x + bv[i].x - m) + exp2f(x[i].y + bv[i].y - m)) + (exp2f(x[i].z + bv[i].z - m) + exp2f(x[i].w + bv[i].w - m));
+        }
+    }
+    float mx = WaveMax(m);
+    if ((tid & 63) == 0) {
+        redM[tid >> 6] = mx;
+    }
+    __syncthreads();
+    mx = fmaxf(fmaxf(redM[0], redM[1]), fmaxf(redM[2], redM[3]));
+    sum = WaveSum(sum * exp2f(m - mx));
+    if ((tid & 63) == 0) {
+        redS[tid >> 6] = sum;
+    }
+    __syncthreads();
+    float scale = 1 / ((redS[0] + redS[1]) + (redS[2] + redS[3]));
+    for (int k0 = tid * 4; k0 < vocab; k0 += 4096) {
+        float4 x[4], bv[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            int k = k0 + i * 1024;
+            bool in = k < vocab;
+            x[i] = in ? *(const float4 *)(row + k) : make_float4(0, 0, 0, 0);
+            bv[i] = in ? *(const float4 *)(bias + k) : make_float4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            int k = k0 + i * 1024;
+            if (k >= vocab) {
+                continue;
+            }
+            float p[4] = {exp2f(x[i].x + bv[i].x - mx) * scale, exp2f(x[i].y + bv[i].y - mx) * scale, exp2f(x[i].z + bv[i].z - mx) * scale,
+                exp2f(x[i].w + bv[i].w - mx) * scale};
+            if (keepProb) {
+                *(float4 *)(row + k) = make_float4(p[0], p[1], p[2], p[3]);
+            }
+            if (tg >= 0) {
+                float g[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    g[e] = ((k + e == tg ? 1.f : 0.f) - p[e]) * gradMult;
+                    if (k + e == tg && lossSum) {
+                        atomicAdd(lossSum, logf(p[e]));
+                    }
+                }
+                *(uint2 *)(grow + k) = make_uint2(PackBf16x2(g[0], g[1]), PackBf16x2(g[2], g[3]));
             }
         }
     }
@@ -128,6 +159,49 @@ __global__ void __launch_bounds__(256) TransposeToBf16(int rows, int rowsRound, 
         int x = x0 + r, t = t0 + tx;
         if (x < cols && t < rowsRound) {
             *(bf16_t *)(dst + (int64_t)x * ldDst + (int64_t)t * 2) = FloatToBf16(tile[tx][r]);
+        }
+    }
+}
+
+// dst[x][t] = src[t][x] for 2-byte elements, zeros for rows <= t < rowsRound; 64x64 tiles, 16-byte loads and stores.
+// cols and rowsRound are multiples of 8, rows of both matrices 16-byte aligned.
+__global__ void __launch_bounds__(256) Transpose16(int rows, int rowsRound, int cols, const uint8_t *src, int64_t ldSrc, uint8_t *dst, int64_t ldDst)
+{
+    constexpr int PITCH = 66; // 2-byte elements per LDS row: column reads of neighbouring lanes fall into different banks
+    __shared__ __attribute__((aligned(16))) uint16_t tile[64 * PITCH];
+    int x0 = blockIdx.x * 64, t0 = blockIdx.y * 64;
+    int tid = threadIdx.x;
+    int lc = tid & 7, lr = tid >> 3; // 8 lanes x 16 bytes per row, 32 rows per pass
+    v4i raw[2];
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        int t = t0 + lr + 32 * k, x = x0 + lc * 8;
+        raw[k] = (t < rows && x < cols) ? *(const v4i *)(src + (int64_t)t * ldSrc + (int64_t)x * 2) : (v4i){0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        uint32_t *d = (uint32_t *)(tile + (lr + 32 * k) * PITCH + lc * 8);
+        d[0] = (uint32_t)raw[k][0];
+        d[1] = (uint32_t)raw[k][1];
+        d[2] = (uint32_t)raw[k][2];
+        d[3] = (uint32_t)raw[k][3];
+    }
+    __syncthreads();
+    // thread -> destination row x (64 of them), 8 consecutive t (8 blocks): 2 units per thread
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        int u = tid + 256 * k;
+        int tb = u & 7, xr = u >> 3;
+        uint32_t w[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            uint32_t lo = tile[(tb * 8 + 2 * e) * PITCH + xr];
+            uint32_t hi = tile[(tb * 8 + 2 * e + 1) * PITCH + xr];
+            w[e] = lo | (hi << 16);
+        }
+        int x = x0 + xr, t = t0 + tb * 8;
+        if (x < cols && t < rowsRound) {
+            *(uint4 *)(dst + (int64_t)x * ldDst + (int64_t)t * 2) = make_uint4(w[0], w[1], w[2], w[3]);
         }
     }
 }
@@ -189,7 +263,12 @@ int Ts2TransposeToBf16(int rows, int rowsRound, int cols, const ts2_mat *src, in
     } else if (srcType == TS2_E4M3) {
         hipLaunchKernelGGL((TransposeToBf16<TE4M3>), grid, dim3(256), 0, STREAM, rows, rowsRound, cols, s, src->strideBytes, d, dst->strideBytes);
     } else if (srcType == TS2_BF16) {
-        hipLaunchKernelGGL((TransposeToBf16<TBF16>), grid, dim3(256), 0, STREAM, rows, rowsRound, cols, s, src->strideBytes, d, dst->strideBytes);
+        if (cols % 8 == 0 && rowsRound % 8 == 0 && src->strideBytes % 16 == 0 && dst->strideBytes % 16 == 0 && (uintptr_t)s % 16 == 0 &&
+            (uintptr_t)d % 16 == 0) {
+            hipLaunchKernelGGL(Transpose16, grid, dim3(256), 0, STREAM, rows, rowsRound, cols, s, src->strideBytes, d, dst->strideBytes);
+        } else {
+            hipLaunchKernelGGL((TransposeToBf16<TBF16>), grid, dim3(256), 0, STREAM, rows, rowsRound, cols, s, src->strideBytes, d, dst->strideBytes);
+        }
     } else {
         return TS2_ERR_UNSUPPORTED;
     }
