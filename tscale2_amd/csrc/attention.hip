@@ -112,13 +112,23 @@ __device__ __forceinline__ v8bf FragT(const uint8_t *t, int db, int ks, int l32,
     return __builtin_bit_cast(v8bf, r);
 }
 
-// B operand of the wave's own rows straight from global memory (loop invariant): lane row = l32
-__device__ __forceinline__ void LoadOwnFrags(v8bf *f, const uint8_t *g, int64_t ld, int l32, int half)
+// The wave's own rows are a loop-invariant B operand.  Held in registers they cost 32 VGPRs per matrix for the whole kernel, which
+// pushes the kernels over the 256 VGPRs a wave can address directly and makes the compiler shuttle values through AGPRs in the
+// inner loop; parked in LDS in fragment order (lane-linear 16-byte slots: conflict-free ds_read_b128) they cost 8 reads per tile.
+constexpr int OWN_BYTES = 4 * 8 * 64 * 16; // 4 waves x 8 fragments x 64 lanes x 16 bytes
+
+__device__ __forceinline__ void ParkOwnFrags(uint8_t *own, const uint8_t *g, int64_t ld, int wave, int lane)
 {
+    int l32 = lane & 31, half = lane >> 5;
 #pragma unroll
     for (int ds = 0; ds < 8; ++ds) {
-        f[ds] = __builtin_bit_cast(v8bf, *(const v4i *)(g + (int64_t)l32 * ld + (ds * 16 + half * 8) * 2));
+        *(v4i *)(own + (wave * 8 + ds) * 1024 + lane * 16) = *(const v4i *)(g + (int64_t)l32 * ld + (ds * 16 + half * 8) * 2);
     }
+}
+
+__device__ __forceinline__ v8bf OwnFrag(const uint8_t *own, int wave, int ds, int lane)
+{
+    return __builtin_bit_cast(v8bf, *(const v4i *)(own + (wave * 8 + ds) * 1024 + lane * 16));
 }
 
 // result registers 8*s .. 8*s+7 of a 32x32 block -> bf16 B operand whose slots match FragT's row order
@@ -212,10 +222,11 @@ __device__ __forceinline__ TRowSpan MakeRowSpan(int start, int finish)
 
 // ---------------------------------------------------------------------------------------------------------------------------
 // forward: grid (lenRound/128, heads)
-__global__ void __launch_bounds__(256) AttForward(AttP p)
+// two workgroups per CU (256 registers per wave, no AGPR form): their barriers and tile latencies overlap
+__global__ void __launch_bounds__(256, 2) AttForward(AttP p)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    uint8_t *kRm = lds, *vT = lds + RM_BYTES;
+    uint8_t *kRm = lds, *vT = lds + RM_BYTES, *ownQ = lds + RM_BYTES + T_BYTES;
     __shared__ int red[8];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
     const int head = blockIdx.y;
@@ -232,8 +243,7 @@ __global__ void __launch_bounds__(256) AttForward(AttP p)
         PrefetchTile(pv, p.v + (int64_t)tFirst * p.ldv + hoff, p.ldv, tid);
     }
 
-    v8bf qf[8];
-    LoadOwnFrags(qf, p.q + (int64_t)(myRow - l32) * p.ldq + hoff, p.ldq, l32, half);
+    ParkOwnFrags(ownQ, p.q + (int64_t)(myRow - l32) * p.ldq + hoff, p.ldq, wave, lane);
     v16f oacc[4];
 #pragma unroll
     for (int db = 0; db < 4; ++db) {
@@ -268,9 +278,10 @@ __global__ void __launch_bounds__(256) AttForward(AttP p)
         }
 #pragma unroll
         for (int ds = 0; ds < 8; ++ds) {
+            v8bf qf = OwnFrag(ownQ, wave, ds, lane);
 #pragma unroll
             for (int kb = 0; kb < NB; ++kb) {
-                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(kRm, kb, ds, l32, half), qf[ds], s[kb], 0, 0, 0);
+                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(kRm, kb, ds, l32, half), qf, s[kb], 0, 0, 0);
             }
         }
         // phase 2: one running-max update per tile.  logit = s*scale - slope*(row - key); tiles that every row of the wave sees
@@ -348,10 +359,10 @@ __global__ void __launch_bounds__(256) AttForward(AttP p)
 
 // ---------------------------------------------------------------------------------------------------------------------------
 // dQ: grid (lenRound/128, heads)
-template <bool F32> __global__ void __launch_bounds__(256) AttGradQ(AttP p)
+template <bool F32> __global__ void __launch_bounds__(256, 2) AttGradQ(AttP p)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    uint8_t *kRm = lds, *vRm = lds + RM_BYTES, *kT = lds + 2 * RM_BYTES;
+    uint8_t *kRm = lds, *vRm = lds + RM_BYTES, *kT = lds + 2 * RM_BYTES, *ownQ = lds + 2 * RM_BYTES + T_BYTES, *ownDO = ownQ + OWN_BYTES;
     __shared__ int red[8];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
     const int head = blockIdx.y;
@@ -368,9 +379,8 @@ template <bool F32> __global__ void __launch_bounds__(256) AttGradQ(AttP p)
         PrefetchTile(pv, p.v + (int64_t)tFirst * p.ldv + hoff, p.ldv, tid);
     }
 
-    v8bf qf[8], dof[8];
-    LoadOwnFrags(qf, p.q + (int64_t)(myRow - l32) * p.ldq + hoff, p.ldq, l32, half);
-    LoadOwnFrags(dof, p.dO + (int64_t)(myRow - l32) * p.lddo + hoff, p.lddo, l32, half);
+    ParkOwnFrags(ownQ, p.q + (int64_t)(myRow - l32) * p.ldq + hoff, p.ldq, wave, lane);
+    ParkOwnFrags(ownDO, p.dO + (int64_t)(myRow - l32) * p.lddo + hoff, p.lddo, wave, lane);
     const float L = p.sumWeightLog[(int64_t)head * p.ldStat + myRow];
     const float dScale = p.dScale[(int64_t)head * p.ldStat + myRow];
     const float gmul = p.attDotScale * LN2;
@@ -408,10 +418,11 @@ template <bool F32> __global__ void __launch_bounds__(256) AttGradQ(AttP p)
         // phase 1: S^T and dP^T of the whole tile, four independent accumulator chains
 #pragma unroll
         for (int ds = 0; ds < 8; ++ds) {
+            v8bf qf = OwnFrag(ownQ, wave, ds, lane), dof = OwnFrag(ownDO, wave, ds, lane);
 #pragma unroll
             for (int kb = 0; kb < NB; ++kb) {
-                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(kRm, kb, ds, l32, half), qf[ds], s[kb], 0, 0, 0);
-                dp[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(vRm, kb, ds, l32, half), dof[ds], dp[kb], 0, 0, 0);
+                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(kRm, kb, ds, l32, half), qf, s[kb], 0, 0, 0);
+                dp[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(vRm, kb, ds, l32, half), dof, dp[kb], 0, 0, 0);
             }
         }
         // phase 2: dS
@@ -454,6 +465,7 @@ template <bool F32> __global__ void __launch_bounds__(256) AttGradKV(AttP p)
     int *stS = (int *)(stD + TR);
     int *stF = stS + TR;
     int *stT = stF + TR; // [4] bounds over the tile's queries
+    uint8_t *ownK = (uint8_t *)(stT + 4), *ownV = ownK + OWN_BYTES;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
     const int head = blockIdx.y;
     const int myRow = blockIdx.x * BROWS + wave * WROWS + l32; // my key
@@ -480,9 +492,8 @@ template <bool F32> __global__ void __launch_bounds__(256) AttGradKV(AttP p)
         prefetch(tFirst);
     }
 
-    v8bf kf[8], vf[8];
-    LoadOwnFrags(kf, p.k + (int64_t)(myRow - l32) * p.ldk + hoff, p.ldk, l32, half);
-    LoadOwnFrags(vf, p.v + (int64_t)(myRow - l32) * p.ldv + hoff, p.ldv, l32, half);
+    ParkOwnFrags(ownK, p.k + (int64_t)(myRow - l32) * p.ldk + hoff, p.ldk, wave, lane);
+    ParkOwnFrags(ownV, p.v + (int64_t)(myRow - l32) * p.ldv + hoff, p.ldv, wave, lane);
     const float gmul = p.attDotScale * LN2;
     v16f dk[4], dv[4];
 #pragma unroll
@@ -525,63 +536,53 @@ template <bool F32> __global__ void __launch_bounds__(256) AttGradKV(AttP p)
         if (stT[3] < kw0 || stT[2] > kw0 + 31) {
             continue; // no query of the tile sees a key of this wave (wave-uniform)
         }
-        constexpr int NB = TR / 32;
-        v16f s[NB], dp[NB];
+        const float ck = p.slope * (float)(myRow - keyBase);
+        // 32 queries at a time: with both halves of the tile in flight the kernel does not fit into 256 registers
 #pragma unroll
-        for (int qb = 0; qb < NB; ++qb) {
+        for (int qb = 0; qb < TR / 32; ++qb) {
+            v16f s, dp;
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                s[qb][e] = 0;
-                dp[qb][e] = 0;
+                s[e] = 0;
+                dp[e] = 0;
             }
-        }
-        // phase 1: S and dP of the whole tile, four independent accumulator chains
+            // phase 1: S and dP
 #pragma unroll
-        for (int ds = 0; ds < 8; ++ds) {
-#pragma unroll
-            for (int qb = 0; qb < NB; ++qb) {
-                s[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(qRm, qb, ds, l32, half), kf[ds], s[qb], 0, 0, 0);
-                dp[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(doRm, qb, ds, l32, half), vf[ds], dp[qb], 0, 0, 0);
+            for (int ds = 0; ds < 8; ++ds) {
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(qRm, qb, ds, l32, half), OwnFrag(ownK, wave, ds, lane), s, 0, 0, 0);
+                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(doRm, qb, ds, l32, half), OwnFrag(ownV, wave, ds, lane), dp, 0, 0, 0);
             }
-        }
-        // phase 2: P and dS from the per-query statistics of the tile
-        v8bf pb[NB][2], sb[NB][2];
-        const float ck = p.slope * (float)(myRow - keyBase);
-#pragma unroll
-        for (int qb = 0; qb < NB; ++qb) {
+            // phase 2: P and dS from the per-query statistics of the tile
             float pv[16], dsv[16];
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 int qi = qb * 32 + g * 8 + half * 4;
                 float4 L4 = *(const float4 *)(stL + qi);
                 float4 D4 = *(const float4 *)(stD + qi);
-                const float Ls[4] = {L4.x, L4.y, L4.z, L4.w};
-                const float Ds[4] = {D4.x, D4.y, D4.z, D4.w};
                 int4 S4 = *(const int4 *)(stS + qi);
                 int4 N4 = *(const int4 *)(stF + qi);
+                const float Ls[4] = {L4.x, L4.y, L4.z, L4.w};
+                const float Ds[4] = {D4.x, D4.y, D4.z, D4.w};
                 const int Ss[4] = {S4.x, S4.y, S4.z, S4.w};
                 const unsigned Ns[4] = {(unsigned)N4.x, (unsigned)N4.y, (unsigned)N4.z, (unsigned)N4.w};
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     int e = g * 4 + j;
-                    float w = __builtin_amdgcn_exp2f(fmaf(s[qb][e], p.attDotScale, Ls[j] + ck));
+                    float w = __builtin_amdgcn_exp2f(fmaf(s[e], p.attDotScale, Ls[j] + ck));
                     w = (unsigned)(myRow - Ss[j]) <= Ns[j] ? w : 0.f;
                     pv[e] = w;
-                    dsv[e] = w * (dp[qb][e] - Ds[j]) * gmul;
+                    dsv[e] = w * (dp[e] - Ds[j]) * gmul;
                 }
             }
-            pb[qb][0] = PackB(pv, 0);
-            pb[qb][1] = PackB(pv, 1);
-            sb[qb][0] = PackB(dsv, 0);
-            sb[qb][1] = PackB(dsv, 1);
-        }
-        // phase 3: dV^T += dO^T P, dK^T += Q^T dS; eight accumulators in turn
+            v8bf pb[2] = {PackB(pv, 0), PackB(pv, 1)}, sb[2] = {PackB(dsv, 0), PackB(dsv, 1)};
+            // phase 3: dV^T += dO^T P, dK^T += Q^T dS; eight accumulators in turn
 #pragma unroll
-        for (int ks = 0; ks < 2 * NB; ++ks) {
+            for (int j = 0; j < 2; ++j) {
 #pragma unroll
-            for (int db = 0; db < 4; ++db) {
-                dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(doT, db, ks, l32, half), pb[ks >> 1][ks & 1], dv[db], 0, 0, 0);
-                dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(qT, db, ks, l32, half), sb[ks >> 1][ks & 1], dk[db], 0, 0, 0);
+                for (int db = 0; db < 4; ++db) {
+                    dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(doT, db, qb * 2 + j, l32, half), pb[j], dv[db], 0, 0, 0);
+                    dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(qT, db, qb * 2 + j, l32, half), sb[j], dk[db], 0, 0, 0);
+                }
             }
         }
     }
@@ -670,7 +671,7 @@ extern "C" int ts2_att_forward(const ts2_att_args *a, void *stream)
     p.out0 = (uint8_t *)a->valLookup.ptr;
     p.ldo0 = a->valLookup.strideBytes;
     p.lenRound = a->lenRound;
-    int ldsBytes = RM_BYTES + T_BYTES;
+    int ldsBytes = RM_BYTES + T_BYTES + OWN_BYTES;
     static bool done = false;
     if (!done) {
         if (SetAttr((const void *)AttForward, ldsBytes)) {
@@ -720,8 +721,8 @@ extern "C" int ts2_att_backward(const ts2_att_grad_args *a, void *stream)
     p.ldStat = a->sumWeightLog.strideBytes / 4;
     p.lenRound = a->lenRound;
     dim3 grid(a->lenRound / BROWS, a->heads);
-    int ldsQ = 2 * RM_BYTES + T_BYTES;
-    int ldsKV = 2 * RM_BYTES + 2 * T_BYTES + 4 * TR * 4 + 16;
+    int ldsQ = 2 * RM_BYTES + T_BYTES + 2 * OWN_BYTES;
+    int ldsKV = 2 * RM_BYTES + 2 * T_BYTES + 4 * TR * 4 + 16 + 2 * OWN_BYTES;
     static bool done = false;
     if (!done) {
         if (SetAttr((const void *)AttGradQ<true>, ldsQ) || SetAttr((const void *)AttGradQ<false>, ldsQ) ||
