@@ -48,7 +48,13 @@ typedef struct ts2_mat {
 enum ts2_epilogue {
     TS2_EPI_STORE = 0,           /* TStore / TStoreScaled        :440-451,467-477 */
     TS2_EPI_ADD = 1,             /* TStoreAdd / TStoreAddScaled  :455-463,481-490 */
-    TS2_EPI_ROW_TILE_MAXNORM = 2 /* TStoreRowTileMaxNormalize    :530-559  packed delta: i8 + TileScale[n/128][m] */
+    TS2_EPI_ROW_TILE_MAXNORM = 2, /* TStoreRowTileMaxNormalize    :530-559  packed delta: i8 + TileScale[n/128][m] */
+    /* TStoreRowTileNormalize :495-525 and TStoreRowTileNormalizeRope (src/gpt/compute/gpu_rope.cuh:25-60): cType TS2_BF16;
+     * v = alpha*acc; if normalize: tileScale[n/128][m] = rms over each 128-column tile * vecScale (0 for zero tiles), v /= it;
+     * if rope.ptr: rotate (even, odd) column pairs of each 128-wide head by the row's (cos, sin) table fp32 [m][128].
+     * Only the 256x256-tile kernel carries it: m, n multiples of 256 and (m/256)*(n/256) >= 192 (or tileConfig 1), else
+     * TS2_ERR_UNSUPPORTED and the caller runs ts2_row_tile_normalize_rope on a plain product. */
+    TS2_EPI_ROW_TILE_NORM = 3
 };
 
 /*
@@ -92,6 +98,10 @@ typedef struct ts2_gemm_args {
     int32_t groups;
     int64_t cSlabBytes;
     int64_t tileScaleSlabBytes;
+    /* TS2_EPI_ROW_TILE_NORM */
+    int32_t normalize;
+    float vecScale;
+    ts2_mat rope;
 } ts2_gemm_args;
 
 int ts2_gemm_nt(const ts2_gemm_args *args, void *stream);
@@ -207,6 +217,15 @@ int ts2_matmul_backprop_delta(int32_t mode, int32_t len, int32_t lenRound, int32
  * res[len][dstDim] = alpha * (*alphaPtr) * src * W^T, src and W 8-bit of the same type, resType TS2_F32 | TS2_BF16. */
 int ts2_matmul_forward(int32_t mode, int32_t len, int32_t lenRound, int32_t srcDim, int32_t dstDim, const ts2_mat *src,
     const ts2_mat *transformFast, float alpha, const float *alphaPtr, const ts2_mat *res, int32_t resType, int32_t add, void *stream);
+
+/* Forward<TStoreRowTileNormalize> / Forward<TStoreRowTileNormalizeRope> of the same operator (store functors of
+ * src/lib/cuda/cuda_matmul.cuh:495-525 and src/gpt/compute/gpu_rope.cuh:25-60): res (TS2_BF16) = rope(normalise(alpha * (*alphaPtr) *
+ * src * W^T)), tileScale fp32 [dstDim/128][lenRound] when normalize.  Fused into the product's epilogue where the 256x256-tile kernel
+ * applies (lenRound, dstDim multiples of 256, at least 192 tiles); otherwise the product goes to `raw` (fp32 [lenRound][dstDim]
+ * scratch) and ts2_row_tile_normalize_rope finishes it. */
+int ts2_matmul_forward_norm_rope(int32_t mode, int32_t len, int32_t lenRound, int32_t srcDim, int32_t dstDim, const ts2_mat *src,
+    const ts2_mat *transformFast, float alpha, const float *alphaPtr, int32_t normalize, float vecScale, const ts2_mat *ropeBuf,
+    const ts2_mat *res, const ts2_mat *tileScale, const ts2_mat *raw, void *stream);
 
 /* ------------------------------------------------------------------------------------------------------------------------
  * Attention (head dimension 128 = Q_DIM = TT_DIM, src/gpt/compute/cfg_precision.h:79-80).  q, k, v, valLookup, dValLookup are

@@ -190,3 +190,51 @@ def test_eight_wave_configuration_is_bit_exact(lib, orc):
     lib.gemm_nt(torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(), tc, L.I8, L.F32, tile_config=9)
     torch.cuda.synchronize()
     assert np.array_equal(tc.cpu().numpy(), ref.astype(np.float32))
+
+
+@pytest.mark.parametrize("ab", ["i8", "e4m3"])
+@pytest.mark.parametrize("normalize,use_rope", [(True, True), (True, False), (False, True)])
+def test_fused_row_tile_normalize_rope_epilogue_matches_the_two_pass_path(ab, normalize, use_rope):
+    """TS2_EPI_ROW_TILE_NORM against the same product stored in fp32 followed by ts2_row_tile_normalize_rope: same arithmetic except
+    for the order of the 128 squares in the tile sum, so the bf16 results may differ by one unit in the last place at most."""
+    print("case fused norm/rope epilogue", ab, normalize, use_rope, flush=True)
+    from tscale2_amd import lib as L
+    lib = L.load()
+    m, n, k = 512, 768, 256
+    g = torch.Generator(device="cuda").manual_seed(5)
+    if ab == "i8":
+        a = torch.randint(-90, 90, (m, k), dtype=torch.int8, device="cuda", generator=g)
+        b = torch.randint(-90, 90, (n, k), dtype=torch.int8, device="cuda", generator=g)
+        t = L.I8
+    else:
+        a = (torch.randn((m, k), device="cuda", generator=g) * 8).to(torch.float8_e4m3fn).view(torch.uint8)
+        b = (torch.randn((n, k), device="cuda", generator=g) * 8).to(torch.float8_e4m3fn).view(torch.uint8)
+        t = L.E4M3
+    a[300:310] = 0                                                   # zero rows: tile scale 0, zero output
+    m_live = 500
+    rope = None
+    if use_rope:
+        ang = torch.rand((m, 64), device="cuda", generator=g) * 6.28
+        rope = torch.stack([torch.cos(ang), torch.sin(ang)], dim=2).reshape(m, 128).contiguous()
+    alpha = 0.37
+    raw = torch.empty((m, n), dtype=torch.float32, device="cuda")
+    lib.gemm_nt(a, b, raw, t, L.F32, alpha=alpha, m_live=m_live, tile_config=1)
+    want = torch.full((m, n), 7, dtype=torch.int16, device="cuda")
+    want_sc = torch.full((n // 128, m), -1.0, device="cuda")
+    L.call("ts2_row_tile_normalize_rope", m_live, m, raw, L.F32, 1.0, int(normalize), 1 / 24.0, rope, want, want_sc if normalize else None)
+    got = torch.full((m, n), 9, dtype=torch.int16, device="cuda")
+    got_sc = torch.full((n // 128, m), -2.0, device="cuda")
+    lib.gemm_nt(a, b, got, t, L.BF16, alpha=alpha, m_live=m_live, tile_config=1, epilogue=L.EPI_ROW_TILE_NORM, normalize=normalize,
+                vec_scale=1 / 24.0, rope=rope, tile_scale=got_sc if normalize else None)
+    torch.cuda.synchronize()
+    gf, wf = got.view(torch.bfloat16).float(), want.view(torch.bfloat16).float()
+    assert (gf[m_live:] == 0).all() and (gf[300:310] == 0).all()
+    tol = wf.abs() * 2.0 ** -7 + 1e-30                               # one bf16 ulp
+    assert ((gf - wf).abs() <= tol).all()
+    assert (gf == wf).float().mean() > 0.99
+    if normalize:
+        assert torch.allclose(got_sc[:, :m_live], want_sc[:, :m_live], rtol=1e-6, atol=0)
+        assert (got_sc[:, 300:310] == 0).all()
+    # unsupported with 128x128 tiles: the caller falls back to the two-pass path
+    assert lib.gemm_nt(a, b, got, t, L.BF16, tile_config=2, epilogue=L.EPI_ROW_TILE_NORM, normalize=True, vec_scale=1.0, tile_scale=got_sc,
+                       check=False) == -3

@@ -40,10 +40,15 @@ struct GemmP {
     int64_t tileScaleSlab;   // floats
     int splitK_groups;       // number of groups when groupOffsets is set
     int direct;              // 1: direct global->LDS loader
+    // row-tile normalise / rope epilogue (C_BF16NORM)
+    int normalize;
+    float vecScale;
+    const float *rope; // [m][128] (cos, sin) pairs, may be null
+    int64_t ldRope;    // floats
 };
 
 enum { T_I8 = 0, T_FP8 = 1, T_BF16 = 2 };
-enum { C_F32 = 0, C_BF16 = 1, C_I32 = 2, C_I8PACK = 3 };
+enum { C_F32 = 0, C_BF16 = 1, C_I32 = 2, C_I8PACK = 3, C_BF16NORM = 4 };
 
 constexpr int BKB = 128; // bytes of K per step
 
@@ -76,6 +81,26 @@ __device__ __forceinline__ void MapTile(int bid, int nb, int tilesM, int tilesN,
     *tn = r / gsz;
 }
 
+// bf16 store of one 32x32 block held as v[e] (lane = column, e -> row): neighbouring lanes swap one value so that even lanes store
+// columns (c, c+1) of the even row of a row pair and odd lanes those of the odd row: 4-byte stores instead of 2-byte ones.
+// rowOf(e) gives the global row; rows >= mLive are written as zeros.
+template <class TRow>
+__device__ __forceinline__ void StoreBlockBf16(uint8_t *c, int64_t ldc, int col, int l32, int mLive, const float (&v)[16], TRow rowOf)
+{
+    const bool odd = l32 & 1;
+#pragma unroll
+    for (int e = 0; e < 16; e += 2) {
+        // rows e and e+1 are consecutive rows of the block (e%4 = 0,1 or 2,3)
+        float give = odd ? v[e] : v[e + 1];
+        float got = __shfl_xor(give, 1, 64);
+        float lo = odd ? got : v[e];
+        float hi = odd ? v[e + 1] : got;
+        int row = rowOf(odd ? e + 1 : e);
+        uint32_t packed = row < mLive ? PackBf16x2(lo, hi) : 0u;
+        *(uint32_t *)(c + (int64_t)row * ldc + (int64_t)(col & ~1) * 2) = packed;
+    }
+}
+
 template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT, class TAcc, class TFAcc>
 __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], TFAcc &facc, uint8_t *lds, int rowBase, int colBase, int wm, int wn,
     int half, int l32)
@@ -95,7 +120,65 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
     };
     auto rowLocal = [&](int i, int e) { return wm * (32 * WTM) + i * 32 + (e >> 2) * 8 + half * 4 + (e & 3); };
 
-    if constexpr (CT == C_I8PACK) {
+    if constexpr (CT == C_BF16NORM) {
+        // TStoreRowTileNormalize / TStoreRowTileNormalizeRope (src/lib/cuda/cuda_matmul.cuh:495-525, src/gpt/compute/gpu_rope.cuh:25-60):
+        // per row and 128-column tile v = acc*scale; scale_t = rms(v)*vecScale, v /= scale_t; rotate (even, odd) column pairs by the
+        // row's (cos, sin) table; bf16.  The wave's 128 columns (WTN == 4) are exactly one tile, so the reduction stays inside the
+        // 32-lane group.
+        static_assert(WTN == 4 || CT != C_BF16NORM, "the normalising epilogue needs the 128-column wave tile");
+        const int tile = (colBase + wn * (32 * WTN)) / TILE;
+#pragma unroll
+        for (int i = 0; i < WTM; ++i) {
+            float out[WTN][16];
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int row = rowBase + rowLocal(i, e);
+                float rs = scale;
+                if (p.rowScale) {
+                    rs *= p.rowScale[row];
+                }
+                float v[WTN];
+                float sum2 = 0;
+#pragma unroll
+                for (int j = 0; j < WTN; ++j) {
+                    v[j] = accVal(i, j, e) * rs;
+                    sum2 += v[j] * v[j];
+                }
+                float discr = 0;
+                if (p.normalize) {
+                    sum2 = Half32Sum(sum2);
+                    if (sum2 > 0 && row < mLive) {
+                        discr = sqrtf(sum2 / TILE) * p.vecScale;
+                        float inv = 1 / discr;
+#pragma unroll
+                        for (int j = 0; j < WTN; ++j) {
+                            v[j] *= inv;
+                        }
+                    }
+                    if (l32 == 0) {
+                        p.tileScale[(int64_t)tile * p.ldTileScale + row] = discr;
+                    }
+                }
+                if (p.rope) {
+#pragma unroll
+                    for (int j = 0; j < WTN; ++j) {
+                        float2 cs = *(const float2 *)(p.rope + (int64_t)row * p.ldRope + ((j * 32 + l32) & ~1));
+                        float other = __shfl_xor(v[j], 1, 64);
+                        v[j] = (l32 & 1) ? other * cs.y + v[j] * cs.x : v[j] * cs.x - other * cs.y;
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < WTN; ++j) {
+                    out[j][e] = v[j];
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < WTN; ++j) {
+                StoreBlockBf16(p.c, p.ldc, colBase + wn * (32 * WTN) + j * 32 + l32, l32, mLive, out[j],
+                    [&](int e) { return rowBase + rowLocal(i, e); });
+            }
+        }
+    } else if constexpr (CT == C_I8PACK) {
         // TStoreRowTileMaxNormalize (src/lib/cuda/cuda_matmul.cuh:530-559): per row and 128 columns scale = maxabs/127, bytes =
         // sat_i8(rne(v/scale)), TileScale[tile][row] = scale.  A 128-column tile is 4 MFMA blocks: inside one wave when WTN == 4,
         // shared by the two waves along N when WTN == 2 (row maxima exchanged through LDS, which the main loop no longer uses).
@@ -158,25 +241,53 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
             }
         }
     } else {
+        // one 32x32 block at a time: for the accumulate epilogues all 16 old values of the block are fetched before the first store,
+        // so the loads are in flight together instead of alternating with the stores they could alias
 #pragma unroll
         for (int i = 0; i < WTM; ++i) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int row = rowBase + rowLocal(i, e);
-                const bool live = row < mLive;
-                float rs = scale;
-                if (p.rowScale) {
-                    rs *= p.rowScale[row];
-                }
-                uint8_t *dst = p.c + (int64_t)row * p.ldc;
+            for (int j = 0; j < WTN; ++j) {
+                const int col = colBase + wn * (32 * WTN) + j * 32 + l32;
+                if constexpr (CT == C_BF16 && EPI == TS2_EPI_STORE) {
+                    float v[16];
 #pragma unroll
-                for (int j = 0; j < WTN; ++j) {
-                    const int col = colBase + wn * (32 * WTN) + j * 32 + l32;
+                    for (int e = 0; e < 16; ++e) {
+                        float rs = scale;
+                        if (p.rowScale) {
+                            rs *= p.rowScale[rowBase + rowLocal(i, e)];
+                        }
+                        v[e] = accVal(i, j, e) * rs;
+                    }
+                    StoreBlockBf16(p.c, p.ldc, col, l32, mLive, v, [&](int e) { return rowBase + rowLocal(i, e); });
+                    continue;
+                }
+                float old[16];
+                if (EPI == TS2_EPI_ADD && p.splitK <= 1 && (CT == C_F32 || CT == C_BF16)) {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const int row = rowBase + rowLocal(i, e);
+                        const uint8_t *src = p.c + (int64_t)row * p.ldc;
+                        if (CT == C_F32) {
+                            old[e] = row < mLive ? ((const float *)src)[col] : 0.f;
+                        } else {
+                            old[e] = row < mLive ? Bf16ToFloat(((const bf16_t *)src)[col]) : 0.f;
+                        }
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int row = rowBase + rowLocal(i, e);
+                    const bool live = row < mLive;
+                    uint8_t *dst = p.c + (int64_t)row * p.ldc;
                     if constexpr (CT == C_I32) {
                         if constexpr (TYPE == T_I8) {
                             ((int *)dst)[col] = acc[i][j][e];
                         }
                     } else {
+                        float rs = scale;
+                        if (p.rowScale) {
+                            rs *= p.rowScale[row];
+                        }
                         float v = live ? accVal(i, j, e) * rs : 0.f;
                         if constexpr (CT == C_F32) {
                             float *d = (float *)dst + col;
@@ -186,7 +297,7 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
                                 }
                             } else if (EPI == TS2_EPI_ADD) {
                                 if (live) {
-                                    *d += v;
+                                    *d = old[e] + v;
                                 }
                             } else {
                                 *d = v;
@@ -195,7 +306,7 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
                             bf16_t *d = (bf16_t *)dst + col;
                             if (EPI == TS2_EPI_ADD) {
                                 if (live) {
-                                    *d = FloatToBf16(Bf16ToFloat(*d) + v);
+                                    *d = FloatToBf16(old[e] + v);
                                 }
                             } else {
                                 *d = FloatToBf16(v);
@@ -711,6 +822,14 @@ template <int TYPE, int WTM, int WTN> int DispatchEpi(const ts2_gemm_args *a, co
         }
         return TS2_ERR_UNSUPPORTED;
     }
+    if (epi == TS2_EPI_ROW_TILE_NORM) {
+        if constexpr (WTN == 4) {
+            if (a->cType == TS2_BF16 && !kt && p.splitK <= 1) {
+                return Launch<TYPE, WTM, WTN, C_BF16NORM, TS2_EPI_STORE, false>(p, stream);
+            }
+        }
+        return TS2_ERR_UNSUPPORTED;
+    }
     const bool eight = WTM == 4 && (a->tileConfig & 8) && p.splitK <= 1;
     if (a->cType == TS2_F32) {
         if (eight) {
@@ -767,6 +886,9 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
     if (a->kTileScale && (a->abType != TS2_I8 || a->kTile <= 0 || (a->kTile % 128) || (a->k % a->kTile))) {
         return TS2_ERR_SHAPE;
     }
+    if (a->cType == TS2_BF16 && (a->c.strideBytes & 3)) {
+        return TS2_ERR_ALIGN; // bf16 results are stored two columns at a time
+    }
     int splitK = a->splitK > 1 ? a->splitK : 1;
     if (splitK > 1 && (a->cType != TS2_F32 || a->epilogue == TS2_EPI_ROW_TILE_MAXNORM)) {
         return TS2_ERR_UNSUPPORTED;
@@ -800,6 +922,19 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
     p.cSlab = a->cSlabBytes;
     p.tileScaleSlab = a->tileScaleSlabBytes / 4;
     p.splitK_groups = a->groups;
+    p.normalize = a->normalize;
+    p.vecScale = a->vecScale;
+    p.rope = (const float *)a->rope.ptr;
+    p.ldRope = a->rope.strideBytes / 4;
+    if (a->epilogue == TS2_EPI_ROW_TILE_NORM) {
+        if (a->cType != TS2_BF16 || (a->c.strideBytes & 3)) {
+            return TS2_ERR_UNSUPPORTED;
+        }
+        if ((a->normalize && (!a->tileScale.ptr || a->tileScale.y < a->n / 128 || a->tileScale.x < a->m)) ||
+            (a->rope.ptr && (a->rope.y < (a->mLive > 0 ? a->mLive : a->m) || a->rope.x < 128 || (a->rope.strideBytes & 7) || ((uintptr_t)a->rope.ptr & 7)))) {
+            return TS2_ERR_SHAPE;
+        }
+    }
     p.direct = (a->tileConfig & 4) ? 0 : 1; // bit 2 of tileConfig selects the register-staged loader (kept for comparison)
     if ((a->tileGroup || a->groupOffsets) && splitK > 1) {
         return TS2_ERR_UNSUPPORTED;

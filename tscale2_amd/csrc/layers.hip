@@ -191,6 +191,15 @@ int Forward(ts2_model *M, TMatrix &W, const Arr &src8, float alpha, bool useScal
         res.type, add, s);
 }
 
+// dst16 = rope(normalise(alpha [* scale] * src8 * W^T)), tile scales to tileScale (fused into the product where the big tile applies)
+int ForwardNormRope(ts2_model *M, TMatrix &W, const Arr &src8, float alpha, bool useScale, bool normalize, float vecScale, const Arr *rope,
+    const Arr &dst16, const Arr *tileScale, void *s)
+{
+    Arr raw = View(M->raw, M->R, W.dstDim);
+    return ts2_matmul_forward_norm_rope(M->mode, M->len, M->R, W.srcDim, W.dstDim, src8.P(), W.fast.P(), alpha, useScale ? W.scale : nullptr,
+        normalize, vecScale, rope ? rope->P() : nullptr, dst16.P(), tileScale ? tileScale->P() : nullptr, raw.P(), s);
+}
+
 // srcGrad (+)= alpha [* scale] * gradFast * W   (TMatMulBuffers::BackpropMulti + Backprop)
 int BackpropDX(ts2_model *M, TMatrix &W, const Arr &gradFast, float alpha, bool useScale, const Arr &srcGrad, bool add, void *s)
 {
@@ -217,8 +226,7 @@ int FfnComputeRG(ts2_model *M, TLayer &L, const Arr &norm8, void *s)
     Arr wideRaw = View(M->raw, R, F), wide16 = View(A.a16[0], R, F), gate16 = View(A.a16[1], R, F), wideScale = View(A.tsc[0], F / 128, R);
     Arr rg8 = View(A.rg8, R, F);
     // wide = MulForward(n, We) in true units, then per-tile normalisation to 1/24 units + tile scale
-    CK(Forward(M, L.w[0], norm8, VEC * DISCR * Dot(D), true, wideRaw, false, s));
-    CK(ts2_row_tile_normalize_rope(len, R, wideRaw.P(), TS2_F32, 1.f, 1, VEC, nullptr, wide16.P(), wideScale.P(), s));
+    CK(ForwardNormRope(M, L.w[0], norm8, VEC * DISCR * Dot(D), true, true, VEC, nullptr, wide16, &wideScale, s));
     // gate uses the matrix without its scale (GetDataNoScale)
     CK(Forward(M, L.w[1], norm8, VEC * DISCR * Dot(D), false, gate16, false, s));
     return ts2_matrix_lolu(len, R, gate16.P(), wide16.P(), 1.f, rg8.P(), M->mode, s);
@@ -266,12 +274,9 @@ int AttComputeVLG(ts2_model *M, TLayer &L, const Arr &norm8, void *s)
     Arr raw = View(M->raw, R, Q), q16 = View(A.a16[0], R, Q), gate16 = View(A.a16[1], R, Q), k16 = View(A.a16[2], R, Q), v16 = View(A.a16[3], R, Q);
     Arr qScale = View(A.tsc[0], H, R), vScale = View(A.tsc[1], H, R), val16 = View(A.val16, R, Q), vlg8 = View(A.rg8, R, Q);
     float a = VEC * DISCR * Dot(D);
-    CK(Forward(M, L.w[0], norm8, a, true, raw, false, s));
-    CK(ts2_row_tile_normalize_rope(len, R, raw.P(), TS2_F32, 1.f, 1, 1.f, M->rope.P(), q16.P(), qScale.P(), s));
-    CK(Forward(M, L.w[1], norm8, a, true, raw, false, s));
-    CK(ts2_row_tile_normalize_rope(len, R, raw.P(), TS2_F32, 1.f, 0, 1.f, M->rope.P(), k16.P(), nullptr, s));
-    CK(Forward(M, L.w[2], norm8, a, true, raw, false, s));
-    CK(ts2_row_tile_normalize_rope(len, R, raw.P(), TS2_F32, 1.f, 1, 1.f, nullptr, v16.P(), vScale.P(), s));
+    CK(ForwardNormRope(M, L.w[0], norm8, a, true, true, 1.f, &M->rope, q16, &qScale, s));
+    CK(ForwardNormRope(M, L.w[1], norm8, a, true, false, 1.f, &M->rope, k16, nullptr, s));
+    CK(ForwardNormRope(M, L.w[2], norm8, a, true, true, 1.f, nullptr, v16, &vScale, s));
     CK(Forward(M, L.w[3], norm8, a, false, gate16, false, s));
     ts2_att_args at = {};
     at.len = len;

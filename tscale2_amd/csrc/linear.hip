@@ -146,3 +146,53 @@ extern "C" int ts2_matmul_forward(int32_t mode, int32_t len, int32_t lenRound, i
     g.splitK = 1;
     return ts2_gemm_nt(&g, stream);
 }
+
+// Forward<TStoreRowTileNormalize> / Forward<TStoreRowTileNormalizeRope> of the same operator (layer_cuda_base.cuh:183-193 with the store
+// functors of cuda_matmul.cuh:495-525 and gpu_rope.cuh:25-60): res = rope(normalise(alpha * (*alphaPtr) * src * W^T)) as bf16 plus the
+// per-tile scales.  The product carries the epilogue itself where the 256x256-tile kernel applies; otherwise it is stored in fp32 into
+// `raw` (caller scratch [lenRound][dstDim], may be null only when the fused form applies) and finished by the stand-alone pass.
+extern "C" int ts2_matmul_forward_norm_rope(int32_t mode, int32_t len, int32_t lenRound, int32_t srcDim, int32_t dstDim, const ts2_mat *src,
+    const ts2_mat *transformFast, float alpha, const float *alphaPtr, int32_t normalize, float vecScale, const ts2_mat *ropeBuf,
+    const ts2_mat *res, const ts2_mat *tileScale, const ts2_mat *raw, void *stream)
+{
+    if (!src || !transformFast || !res || (normalize && !tileScale)) {
+        return TS2_ERR_NULL;
+    }
+    ts2_gemm_args g = {};
+    g.a = *src;
+    g.b = *transformFast;
+    g.abType = mode;
+    g.m = lenRound;
+    g.n = dstDim;
+    g.k = srcDim;
+    g.mLive = len;
+    g.alpha = alpha;
+    g.alphaPtr = alphaPtr;
+    g.splitK = 1;
+    const bool fused = lenRound % 256 == 0 && dstDim % 256 == 0 && (int64_t)(lenRound / 256) * (dstDim / 256) >= 192;
+    if (fused) {
+        g.c = *res;
+        g.cType = TS2_BF16;
+        g.epilogue = TS2_EPI_ROW_TILE_NORM;
+        g.normalize = normalize;
+        g.vecScale = vecScale;
+        if (ropeBuf) {
+            g.rope = *ropeBuf;
+        }
+        if (normalize) {
+            g.tileScale = *tileScale;
+        }
+        return ts2_gemm_nt(&g, stream);
+    }
+    if (!raw) {
+        return TS2_ERR_NULL;
+    }
+    g.c = *raw;
+    g.cType = TS2_F32;
+    g.epilogue = TS2_EPI_STORE;
+    int rc = ts2_gemm_nt(&g, stream);
+    if (rc != TS2_OK) {
+        return rc;
+    }
+    return ts2_row_tile_normalize_rope(len, lenRound, raw, TS2_F32, 1.f, normalize, vecScale, ropeBuf, res, tileScale, stream);
+}

@@ -7,7 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 SO = os.path.join(HERE, "libts2amd.so")
 
 I8, E4M3, BF16, F32, I32 = 0, 1, 2, 3, 4
-EPI_STORE, EPI_ADD, EPI_ROW_TILE_MAXNORM = 0, 1, 2
+EPI_STORE, EPI_ADD, EPI_ROW_TILE_MAXNORM, EPI_ROW_TILE_NORM = 0, 1, 2, 3
 
 
 class Mat(C.Structure):
@@ -19,7 +19,8 @@ class GemmArgs(C.Structure):
                 ("k", C.c_int32), ("mLive", C.c_int32), ("rowScale", C.c_void_p), ("kTileScale", C.c_void_p), ("kTile", C.c_int32),
                 ("alpha", C.c_float), ("alphaPtr", C.c_void_p), ("epilogue", C.c_int32), ("tileScale", Mat), ("splitK", C.c_int32),
                 ("tileConfig", C.c_int32), ("tileGroup", C.c_void_p), ("bSlabBytes", C.c_int64), ("groupOffsets", C.c_void_p),
-                ("groups", C.c_int32), ("cSlabBytes", C.c_int64), ("tileScaleSlabBytes", C.c_int64)]
+                ("groups", C.c_int32), ("cSlabBytes", C.c_int64), ("tileScaleSlabBytes", C.c_int64), ("normalize", C.c_int32),
+                ("vecScale", C.c_float), ("rope", Mat)]
 
 
 def mat(t):
@@ -55,7 +56,8 @@ class Lib:
 
     def gemm_nt(self, a, b, c, ab_type, c_type, row_scale=None, k_tile_scale=None, k_tile=0, alpha=1.0, alpha_ptr=None,
                 epilogue=EPI_STORE, tile_scale=None, split_k=1, m_live=0, tile_config=0, k=None, check=True, m=None, n=None,
-                tile_group=None, b_slab_bytes=0, group_offsets=None, groups=0, c_slab_bytes=0, tile_scale_slab_bytes=0):
+                tile_group=None, b_slab_bytes=0, group_offsets=None, groups=0, c_slab_bytes=0, tile_scale_slab_bytes=0,
+                normalize=False, vec_scale=1.0, rope=None):
         args = GemmArgs()
         args.a, args.b, args.c = mat(a), mat(b), mat(c)
         args.abType, args.cType = ab_type, c_type
@@ -74,6 +76,7 @@ class Lib:
         args.tileScale = mat(tile_scale)
         args.splitK = split_k
         args.tileConfig = tile_config
+        args.normalize, args.vecScale, args.rope = int(normalize), vec_scale, mat(rope)
         rc = self.dll.ts2_gemm_nt(C.byref(args), self.stream())
         if check:
             self.check(rc, "ts2_gemm_nt")
