@@ -244,13 +244,14 @@ int FfnBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
     int D = M->cfg.dim, F = M->cfg.ffnDim, len = M->len, R = M->R;
     TActs &A = *L.acts;
     Arr wide16 = View(A.a16[0], R, F), gate16 = View(A.a16[1], R, F), wideScale = View(A.tsc[0], F / 128, R), rg8 = View(A.rg8, R, F);
-    Arr drg = View(M->g32, R, F), dwide = View(M->gf[0], R, F), dgate = View(M->gf[1], R, F);
+    // drg travels in bf16 (the reference uses half here): its consumer rounds to the 8-bit gradient type anyway
+    Arr drg = View(M->g16[0], R, F), dwide = View(M->gf[0], R, F), dgate = View(M->gf[1], R, F);
     if (!(M->useKept && A.valid)) {
         CK(FfnComputeRG(M, L, norm8, s));
     }
     // contract backward
     CK(BackpropDX(M, L.w[2], M->stateGradFast, DISCR * Dot(F), true, drg, false, s));
-    CK(ts2_backprop_row_tile_normalize_lolu(len, R, gate16.P(), wide16.P(), VEC, wideScale.P(), drg.P(), TS2_F32, dgate.P(), dwide.P(),
+    CK(ts2_backprop_row_tile_normalize_lolu(len, R, gate16.P(), wide16.P(), VEC, wideScale.P(), drg.P(), TS2_BF16, dgate.P(), dwide.P(),
         M->fastGradType, s));
     CK(BackpropDX(M, L.w[0], dwide, DISCR * Dot(D), true, M->dNormState, false, s));
     CK(BackpropDX(M, L.w[1], dgate, DISCR * Dot(D), false, M->dNormState, true, s));
@@ -309,7 +310,7 @@ int AttBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
     TActs &A = *L.acts;
     Arr q16 = View(A.a16[0], R, Q), gate16 = View(A.a16[1], R, Q), k16 = View(A.a16[2], R, Q), v16 = View(A.a16[3], R, Q);
     Arr qScale = View(A.tsc[0], H, R), vScale = View(A.tsc[1], H, R), val16 = View(A.val16, R, Q), vlg8 = View(A.rg8, R, Q);
-    Arr dvlg = View(M->g32, R, Q), dGate = View(M->gf[1], R, Q), dVal16 = View(M->g16[1], R, Q);
+    Arr dvlg = View(M->g16[0], R, Q), dGate = View(M->gf[1], R, Q), dVal16 = View(M->g16[1], R, Q);
     if (!(M->useKept && A.valid)) {
         CK(AttComputeVLG(M, L, norm8, s));
     }
@@ -318,7 +319,7 @@ int AttBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
     CK(BackpropDX(M, L.w[4], M->stateGradFast, DISCR * Dot(Q), true, dvlg, false, s));
     CK(BackpropDelta(M, L.w[4], vlg8, M->stateGradFast, VEC, gradScale, s));
     // gate backward + dScale
-    CK(ts2_backprop_lolu_dscale(len, R, gate16.P(), val16.P(), 1.f, dvlg.P(), TS2_F32, dGate.P(), M->fastGradType, dVal16.P(), TS2_BF16,
+    CK(ts2_backprop_lolu_dscale(len, R, gate16.P(), val16.P(), 1.f, dvlg.P(), TS2_BF16, dGate.P(), M->fastGradType, dVal16.P(), TS2_BF16,
         M->dScale.P(), s));
     // attention backward (dQ, dK, dV in bf16; val16's buffer is reused for dQ once dScale is known)
     Arr dQ = View(A.val16, R, Q), dK = View(M->g16[2], R, Q), dV = View(M->g16[3], R, Q);
