@@ -241,14 +241,14 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
             }
         }
     } else {
-        // one 32x32 block at a time: for the accumulate epilogues all 16 old values of the block are fetched before the first store,
-        // so the loads are in flight together instead of alternating with the stores they could alias
+        // four consecutive rows (one e-quad) across the wave's whole width at a time: a row's WTN 128-byte segments are written back
+        // to back, and for the accumulate epilogues the 4 x WTN old values are all fetched before the first store
 #pragma unroll
         for (int i = 0; i < WTM; ++i) {
+            if constexpr (CT == C_BF16 && EPI == TS2_EPI_STORE) {
 #pragma unroll
-            for (int j = 0; j < WTN; ++j) {
-                const int col = colBase + wn * (32 * WTN) + j * 32 + l32;
-                if constexpr (CT == C_BF16 && EPI == TS2_EPI_STORE) {
+                for (int j = 0; j < WTN; ++j) {
+                    const int col = colBase + wn * (32 * WTN) + j * 32 + l32;
                     float v[16];
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
@@ -259,57 +259,65 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
                         v[e] = accVal(i, j, e) * rs;
                     }
                     StoreBlockBf16(p.c, p.ldc, col, l32, mLive, v, [&](int e) { return rowBase + rowLocal(i, e); });
-                    continue;
                 }
-                float old[16];
-                if (EPI == TS2_EPI_ADD && p.splitK <= 1 && (CT == C_F32 || CT == C_BF16)) {
+            } else {
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) {
-                        const int row = rowBase + rowLocal(i, e);
-                        const uint8_t *src = p.c + (int64_t)row * p.ldc;
-                        if (CT == C_F32) {
-                            old[e] = row < mLive ? ((const float *)src)[col] : 0.f;
-                        } else {
-                            old[e] = row < mLive ? Bf16ToFloat(((const bf16_t *)src)[col]) : 0.f;
+                for (int eq = 0; eq < 4; ++eq) {
+                    float old[4][WTN];
+                    if (EPI == TS2_EPI_ADD && p.splitK <= 1 && (CT == C_F32 || CT == C_BF16)) {
+#pragma unroll
+                        for (int ee = 0; ee < 4; ++ee) {
+                            const int row = rowBase + rowLocal(i, eq * 4 + ee);
+                            const uint8_t *src = p.c + (int64_t)row * p.ldc;
+#pragma unroll
+                            for (int j = 0; j < WTN; ++j) {
+                                const int col = colBase + wn * (32 * WTN) + j * 32 + l32;
+                                if (CT == C_F32) {
+                                    old[ee][j] = row < mLive ? ((const float *)src)[col] : 0.f;
+                                } else {
+                                    old[ee][j] = row < mLive ? Bf16ToFloat(((const bf16_t *)src)[col]) : 0.f;
+                                }
+                            }
                         }
                     }
-                }
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    const int row = rowBase + rowLocal(i, e);
-                    const bool live = row < mLive;
-                    uint8_t *dst = p.c + (int64_t)row * p.ldc;
-                    if constexpr (CT == C_I32) {
-                        if constexpr (TYPE == T_I8) {
-                            ((int *)dst)[col] = acc[i][j][e];
-                        }
-                    } else {
+                    for (int ee = 0; ee < 4; ++ee) {
+                        const int e = eq * 4 + ee;
+                        const int row = rowBase + rowLocal(i, e);
+                        const bool live = row < mLive;
+                        uint8_t *dst = p.c + (int64_t)row * p.ldc;
                         float rs = scale;
                         if (p.rowScale) {
                             rs *= p.rowScale[row];
                         }
-                        float v = live ? accVal(i, j, e) * rs : 0.f;
-                        if constexpr (CT == C_F32) {
-                            float *d = (float *)dst + col;
-                            if (p.splitK > 1) {
-                                if (live) {
-                                    atomicAdd(d, v);
-                                }
-                            } else if (EPI == TS2_EPI_ADD) {
-                                if (live) {
-                                    *d = old[e] + v;
+#pragma unroll
+                        for (int j = 0; j < WTN; ++j) {
+                            const int col = colBase + wn * (32 * WTN) + j * 32 + l32;
+                            if constexpr (CT == C_I32) {
+                                if constexpr (TYPE == T_I8) {
+                                    ((int *)dst)[col] = acc[i][j][e];
                                 }
                             } else {
-                                *d = v;
-                            }
-                        } else if constexpr (CT == C_BF16) {
-                            bf16_t *d = (bf16_t *)dst + col;
-                            if (EPI == TS2_EPI_ADD) {
-                                if (live) {
-                                    *d = FloatToBf16(old[e] + v);
+                                float v = live ? accVal(i, j, e) * rs : 0.f;
+                                if constexpr (CT == C_F32) {
+                                    float *d = (float *)dst + col;
+                                    if (p.splitK > 1) {
+                                        if (live) {
+                                            atomicAdd(d, v);
+                                        }
+                                    } else if (EPI == TS2_EPI_ADD) {
+                                        if (live) {
+                                            *d = old[ee][j] + v;
+                                        }
+                                    } else {
+                                        *d = v;
+                                    }
+                                } else if constexpr (CT == C_BF16) {
+                                    bf16_t *d = (bf16_t *)dst + col;
+                                    if (live) {
+                                        *d = FloatToBf16(old[ee][j] + v);
+                                    }
                                 }
-                            } else {
-                                *d = FloatToBf16(v);
                             }
                         }
                     }
