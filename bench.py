@@ -280,7 +280,77 @@ def bench_att_bwd(args):
             "roofline": roof}
 
 
-WORKLOADS = {"linear_i8_bwd": bench_linear_i8, "step_fp8": bench_step_fp8, "att_bwd": bench_att_bwd}
+def bench_moe_fp8(args):
+    """BASELINE config[4]: one MoE layer forward + backward: 64 experts, top-2, dim 1024, expert width 512, 65536 tokens, e4m3 expert
+    weights; the router logits come from a random select matrix on tile-normalised N(0,1) states (mildly imbalanced load).
+    One step = ts2_layer_forward + ts2_layer_backward of that layer (routing, gather, grouped expand/gate/contract products, combine,
+    routing backward, grouped dX products, grouped deltas, select-matrix backward)."""
+    import numpy as np
+    import torch
+    from tscale2_amd import lib as L
+    from oracle_lib import Oracle
+    L.load()
+    orc = Oracle()
+    dim, xp, experts, selected, n, vocab = 1024, 512, 64, 2, 65536, 128
+    if args.small:
+        n = 8192
+    lt = np.array([3], np.int32); la = np.zeros(1, np.int32); ls = np.zeros(1, np.float32)
+    # every token carries its own label: the embedding rows are the N(0,1) token states the configuration asks for
+    m = L.Model(L.E4M3, dim, 8, 1024, lt, la, ls, 1, vocab, n + 1, n, xp, experts, selected)
+    gen = torch.Generator(device="cuda").manual_seed(6)
+    shapes = [(xp * experts, dim), (xp * experts, dim), (dim * experts, xp), (experts, dim)]
+    for i, (rows, cols) in enumerate(shapes):
+        fast, sc = _fast_weights(torch, rows, cols, True, gen)
+        # the timed loop re-runs the layer on its own output state: a tiny contract scale keeps that state, and with it the routing,
+        # the same in every step (the arithmetic does not depend on the scale)
+        m.set_matrix(0, i, fast, 1e-6 if i == 2 else sc)
+    fast, sc = _fast_weights(torch, n + 1, dim, True, gen)
+    m.set_matrix(L.LAYER_EMBED, 0, fast, sc)
+    fast, sc = _fast_weights(torch, vocab, dim, True, gen)
+    m.set_matrix(L.LAYER_FINAL, 0, fast, sc)
+    m.set_bias(np.zeros(vocab, np.float32))
+    r = np.random.default_rng(7)
+    tg = r.integers(0, vocab, n).astype(np.int32)
+    t = np.arange(n, dtype=np.int32)
+    m.set_batch(np.arange(n + 1, dtype=np.int32), (1 + t).astype(np.uint32), tg, [np.maximum(t - 1, 0).astype(np.int32)],
+                [(t - 1).astype(np.int32)], orc.fill_rope_buf(128, n))
+    m.backprop()                                  # fills state, stateGrad and the gradient scales once
+
+    def step():
+        m.layer_forward(0)
+        m.layer_backward(0)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ms = event_time_ms(step, args.steps)
+    offs = m.read("expertOffset").ravel()
+    per_expert = np.diff(offs[:experts + 1])
+    routed = n * selected
+    flop = 3 * 3 * 2.0 * dim * xp * routed         # three slabs, forward + dX + delta
+    # dominant kernel: the grouped e4m3 product; timed alone through the same entry point on a balanced routing of the same size
+    lib = L.load()
+    rows = routed + 128 * experts
+    a = torch.randint(0, 120, (rows, dim), dtype=torch.uint8, device="cuda")
+    b = torch.randint(0, 120, (experts * xp, dim), dtype=torch.uint8, device="cuda")
+    c = torch.empty((rows, xp), dtype=torch.float32, device="cuda")
+    grp = (torch.arange(rows // 128, device="cuda", dtype=torch.int32) * experts // (rows // 128)).int().contiguous()
+    ms_g = event_time_ms(lambda: lib.gemm_nt(a, b, c, L.E4M3, L.F32, n=xp, tile_group=grp, b_slab_bytes=xp * dim), 10)
+    gops = 2.0 * rows * xp * dim
+    roof = {"bound": "mfma", "achieved": gops / (ms_g * 1e-3) / 1e12, "peak": PEAK_FP8 / 1e12, "unit": "TFLOP/s",
+            "frac": gops / (ms_g * 1e-3) / PEAK_FP8, "traffic": None,
+            "kernel": "GemmNT<e4m3>, expert-grouped rows: %d x %d x %d, %d slabs (%.1f us per launch)" % (rows, xp, dim, experts, ms_g * 1e3)}
+    out = {"metric": "fwd+bwd tokens/sec on 1 MI355X; bwd GEMM TFLOPS as % of MFMA peak", "value": n / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1,
+           "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "fp8_e4m3", "data": "synthetic",
+           "config": {"workload": "MoE layer fwd+bwd: %d experts, top-%d, dim %d, expert width %d, %d tokens, e4m3" % (experts, selected, dim, xp, n),
+                      "routed_rows": routed, "useful_tflop_per_step": flop / 1e12,
+                      "rows_per_expert_min_mean_max": [int(per_expert.min()), float(per_expert.mean()), int(per_expert.max())]},
+           "layer_tflops": flop / (ms * 1e-3) / 1e12, "roofline": roof}
+    m.close()
+    return out
+
+
+WORKLOADS = {"linear_i8_bwd": bench_linear_i8, "step_fp8": bench_step_fp8, "att_bwd": bench_att_bwd, "moe_fp8": bench_moe_fp8}
 
 
 def main():
@@ -290,7 +360,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="linear_i8_bwd", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--small", action="store_true", help="step_fp8: a reduced model for quick checks (not a valid benchmark figure)")
+    ap.add_argument("--small", action="store_true", help="step_fp8 / moe_fp8: a reduced model for quick checks (not a valid benchmark figure)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the path has no multi-GPU leg); use --gpus 1", file=sys.stderr)

@@ -383,8 +383,11 @@ int ts2_layer_forward(ts2_model *m, int32_t layer, void *stream);
 int ts2_layer_backward(ts2_model *m, int32_t layer, void *stream);
 /* dequantised delta of a matrix into hostOut [rows][cols] (synchronises the device) */
 int ts2_model_get_delta(ts2_model *m, int32_t layer, int32_t matrixId, float *hostOut, int32_t rows, int32_t cols);
-/* device view of an internal array: "state", "stateGrad", "stateGradFast", "dNormState", "prediction", "normState"[i], "stateScale"[i] */
+/* device view of an internal array: "state", "stateGrad", "stateGradFast", "dNormState", "prediction", "normState"[i], "stateScale"[i],
+ * "expertOffset" (TS2_I32 [1][experts+2], MoE models: the routing of the last MoE layer that ran) */
 int ts2_model_array(ts2_model *m, const char *name, int32_t index, ts2_mat *out, int32_t *type);
+/* host copy of the same arrays, rows packed ([y][x] elements); synchronises the device */
+int ts2_model_read(ts2_model *m, const char *name, int32_t index, void *hostOut, int64_t hostBytes);
 int ts2_model_scalars(ts2_model *m, float *lossSumHost, int32_t *lenRound, int32_t *lenMoe);
 
 /* peak dense MFMA rate the library prices its kernels against, in T(FL)OP/s, and the CU count it tiles for */

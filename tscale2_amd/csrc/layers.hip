@@ -23,6 +23,21 @@ inline float Dot(int dim)
     return sqrtf(1.0f / dim);
 }
 
+// pitched host<->device copy as plain 1-D copies (one when both sides are dense, else one per row)
+hipError_t Copy2D(void *dst, size_t dpitch, const void *src, size_t spitch, size_t width, size_t height, hipMemcpyKind kind)
+{
+    if (dpitch == width && spitch == width) {
+        return hipMemcpy(dst, src, width * height, kind);
+    }
+    for (size_t y = 0; y < height; ++y) {
+        hipError_t e = hipMemcpy((uint8_t *)dst + y * dpitch, (const uint8_t *)src + y * spitch, width, kind);
+        if (e != hipSuccess) {
+            return e;
+        }
+    }
+    return hipSuccess;
+}
+
 int ElemSz(int type)
 {
     return (type == TS2_F32 || type == TS2_I32) ? 4 : (type == TS2_BF16 ? 2 : 1);
@@ -822,7 +837,7 @@ extern "C" int ts2_model_set_matrix(ts2_model *M, int32_t layer, int32_t matrixI
     if (cols != W->srcDim || rows > W->dstDim * W->slabs) {
         return TS2_ERR_SHAPE;
     }
-    if (hipMemcpy2D(W->fast.m.ptr, W->fast.m.strideBytes, fastHost, cols, cols, rows, hipMemcpyHostToDevice) != hipSuccess ||
+    if (Copy2D(W->fast.m.ptr, W->fast.m.strideBytes, fastHost, cols, cols, rows, hipMemcpyHostToDevice) != hipSuccess ||
         hipMemcpy(W->scale, &scale, 4, hipMemcpyHostToDevice) != hipSuccess) {
         return TS2_ERR_LAUNCH;
     }
@@ -853,7 +868,7 @@ extern "C" int ts2_model_set_batch(ts2_model *M, int32_t len, const int32_t *lab
     bool ok = hipMemcpy(M->labelPtr, labelPtr, (size_t)(len + 1) * 4, hipMemcpyHostToDevice) == hipSuccess;
     ok &= hipMemcpy(M->labels, labels, (size_t)labelPtr[len] * 4, hipMemcpyHostToDevice) == hipSuccess;
     ok &= hipMemcpy(M->target, tg.data(), (size_t)R * 4, hipMemcpyHostToDevice) == hipSuccess;
-    ok &= hipMemcpy2D(M->rope.m.ptr, M->rope.m.strideBytes, ropeBuf, 128 * 4, 128 * 4, len, hipMemcpyHostToDevice) == hipSuccess;
+    ok &= Copy2D(M->rope.m.ptr, M->rope.m.strideBytes, ropeBuf, 128 * 4, 128 * 4, len, hipMemcpyHostToDevice) == hipSuccess;
     for (int a = 0; a < M->cfg.attTypeCount && ok; ++a) {
         std::fill(st.begin(), st.end(), 0);
         std::fill(fi.begin(), fi.end(), -1);
@@ -924,7 +939,7 @@ extern "C" int ts2_model_get_delta(ts2_model *M, int32_t layer, int32_t matrixId
         return TS2_ERR_LAUNCH;
     }
     if (layer == TS2_LAYER_EMBED) {
-        return hipMemcpy2D(hostOut, (size_t)cols * 4, W->delta.m.ptr, W->delta.m.strideBytes, (size_t)cols * 4, rows, hipMemcpyDeviceToHost) ==
+        return Copy2D(hostOut, (size_t)cols * 4, W->delta.m.ptr, W->delta.m.strideBytes, (size_t)cols * 4, rows, hipMemcpyDeviceToHost) ==
                        hipSuccess
                    ? 0
                    : TS2_ERR_LAUNCH;
@@ -932,8 +947,8 @@ extern "C" int ts2_model_get_delta(ts2_model *M, int32_t layer, int32_t matrixId
     int allRows = W->dstDim * W->slabs;
     std::vector<int8_t> d((size_t)rows * cols);
     std::vector<float> ts((size_t)(cols / 128) * allRows);
-    if (hipMemcpy2D(d.data(), cols, W->delta.m.ptr, W->delta.m.strideBytes, cols, rows, hipMemcpyDeviceToHost) != hipSuccess ||
-        hipMemcpy2D(ts.data(), (size_t)allRows * 4, W->deltaTileScale.m.ptr, W->deltaTileScale.m.strideBytes, (size_t)allRows * 4, cols / 128,
+    if (Copy2D(d.data(), cols, W->delta.m.ptr, W->delta.m.strideBytes, cols, rows, hipMemcpyDeviceToHost) != hipSuccess ||
+        Copy2D(ts.data(), (size_t)allRows * 4, W->deltaTileScale.m.ptr, W->deltaTileScale.m.strideBytes, (size_t)allRows * 4, cols / 128,
             hipMemcpyDeviceToHost) != hipSuccess) {
         return TS2_ERR_LAUNCH;
     }
@@ -951,7 +966,11 @@ extern "C" int ts2_model_array(ts2_model *M, const char *name, int32_t index, ts
         return TS2_ERR_NULL;
     }
     const Arr *a = nullptr;
-    if (!strcmp(name, "state")) {
+    Arr tmp;
+    if (!strcmp(name, "expertOffset") && M->moe.expertOffset) {
+        tmp = Flat(M->moe.expertOffset, 1, M->cfg.expertCount + 2, TS2_I32); // first grouped row of each expert, rows in use, capacity
+        a = &tmp;
+    } else if (!strcmp(name, "state")) {
         a = &M->state;
     } else if (!strcmp(name, "stateGrad")) {
         a = &M->stateGrad;
@@ -971,6 +990,25 @@ extern "C" int ts2_model_array(ts2_model *M, const char *name, int32_t index, ts
     *out = a->m;
     if (type) {
         *type = a->type;
+    }
+    return 0;
+}
+
+extern "C" int ts2_model_read(ts2_model *M, const char *name, int32_t index, void *hostOut, int64_t hostBytes)
+{
+    ts2_mat m;
+    int32_t type = 0;
+    int rc = ts2_model_array(M, name, index, &m, &type);
+    if (rc != 0) {
+        return rc;
+    }
+    int64_t rowBytes = (int64_t)m.x * ElemSz(type);
+    if (!hostOut || hostBytes < rowBytes * m.y) {
+        return TS2_ERR_SHAPE;
+    }
+    if (hipDeviceSynchronize() != hipSuccess ||
+        Copy2D(hostOut, rowBytes, m.ptr, m.strideBytes, rowBytes, m.y, hipMemcpyDeviceToHost) != hipSuccess) {
+        return TS2_ERR_LAUNCH;
     }
     return 0;
 }

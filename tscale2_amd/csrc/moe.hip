@@ -118,19 +118,39 @@ __global__ void __launch_bounds__(RB) MoeLocalRank(int total, int experts, const
     }
 }
 
-// step 2 (one workgroup): per expert exclusive prefix over blocks, padded expert offsets, tile -> expert table
+// step 2 (one workgroup): per expert exclusive prefix over blocks, padded expert offsets, tile -> expert table.  The blocks are cut
+// into 256/experts chunks (experts <= 256) that are summed by different threads, so no thread walks a long chain of dependent loads.
 __global__ void __launch_bounds__(256) MoeOffsets(int nBlocks, int experts, int lenMoe, int *blockCounts, int *expertOffset, int *xpTileExpertId)
 {
+    __shared__ int chunkSum[256];
     __shared__ int counts[256];
-    int e = threadIdx.x;
+    const int chunks = 256 / experts > 0 ? 256 / experts : 1;
+    const int e = threadIdx.x % experts, ch = threadIdx.x / experts;
+    const int per = (nBlocks + chunks - 1) / chunks;
+    const int b0 = ch * per, b1 = min(nBlocks, b0 + per);
+    const bool active = ch < chunks && threadIdx.x < experts * chunks;
     int sum = 0;
-    if (e < experts) {
-        for (int b = 0; b < nBlocks; ++b) {
-            int c = blockCounts[b * experts + e];
-            blockCounts[b * experts + e] = sum;
-            sum += c;
+    if (active) {
+        for (int b = b0; b < b1; ++b) {
+            sum += blockCounts[b * experts + e];
         }
-        counts[e] = (sum + TILE - 1) & ~(TILE - 1);
+    }
+    chunkSum[threadIdx.x] = active ? sum : 0;
+    __syncthreads();
+    if (active) {
+        int base = 0;
+        for (int c = 0; c < ch; ++c) {
+            base += chunkSum[c * experts + e];
+        }
+        int run = base;
+        for (int b = b0; b < b1; ++b) {
+            int c = blockCounts[b * experts + e];
+            blockCounts[b * experts + e] = run;
+            run += c;
+        }
+        if (ch == chunks - 1) {
+            counts[e] = (run + TILE - 1) & ~(TILE - 1);
+        }
     }
     __syncthreads();
     if (threadIdx.x == 0) {

@@ -306,8 +306,8 @@ class Model:
         import torch
         m = Mat(); t = C.c_int32(0)
         self._ck(self.lib.dll.ts2_model_array(self.h, name.encode(), index, C.byref(m), C.byref(t)), "ts2_model_array")
-        dt = {I8: torch.int8, E4M3: torch.uint8, BF16: torch.bfloat16, F32: torch.float32}[t.value]
-        es = {I8: 1, E4M3: 1, BF16: 2, F32: 4}[t.value]
+        dt = {I8: torch.int8, E4M3: torch.uint8, BF16: torch.bfloat16, F32: torch.float32, I32: torch.int32}[t.value]
+        es = {I8: 1, E4M3: 1, BF16: 2, F32: 4, I32: 4}[t.value]
         n = m.strideBytes // es * m.y
 
         class _Holder:
@@ -317,7 +317,19 @@ class Model:
             flat = flat.view(torch.int16).view(torch.bfloat16)
         elif dt == torch.int8:
             flat = flat.view(torch.int8)
+        elif dt == torch.int32:
+            flat = flat.view(torch.int32)
         return flat.view(m.y, m.strideBytes // es)[:, :m.x]
+
+    def read(self, name, index=0):
+        """host copy (numpy) of an internal device array"""
+        import numpy as np
+        m = Mat(); t = C.c_int32(0)
+        self._ck(self.lib.dll.ts2_model_array(self.h, name.encode(), index, C.byref(m), C.byref(t)), "ts2_model_array")
+        dt = {I8: np.int8, E4M3: np.uint8, BF16: np.uint16, F32: np.float32, I32: np.int32}[t.value]
+        out = np.empty((m.y, m.x), dt)
+        self._ck(self.lib.dll.ts2_model_read(self.h, name.encode(), index, out.ctypes.data_as(C.c_void_p), C.c_int64(out.nbytes)), "ts2_model_read")
+        return out
 
     def loss_sum(self):
         v = C.c_float(0)
