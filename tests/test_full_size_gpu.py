@@ -1,0 +1,118 @@
+"""The kernels at the full sizes of the benchmark configurations, checked through properties that need no CPU reference of that size:
+row/column checksums of a product (exact for int32-accumulated int8), independence of the sequences of a causal batch, and
+linearity of dK/dV in dO."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def L():
+    from tscale2_amd import lib
+    lib.load()
+    return lib
+
+
+def checksums(a, b):
+    """sum_i C[i][j] and sum_j C[i][j] of C = A B^T from the operand sums, in float64 (exact below 2^53)"""
+    a64, b64 = a.double(), b.double()
+    col = (a64.sum(0, keepdim=True) @ b64.t()).ravel()      # [n]
+    row = (a64 @ b64.sum(0, keepdim=True).t()).ravel()      # [m]
+    return col, row
+
+
+@pytest.mark.parametrize("m,n,k", [(16384, 1024, 4096), (4096, 1024, 16384)])
+def test_int8_products_of_the_linear_backward_are_exact_at_full_size(L, m, n, k):
+    """config[1]: dX is [16384 x 4096] x [1024 x 4096]^T, the delta [4096 x 16384] x [1024 x 16384]^T; every row sum and every column sum
+    of the int32 result must equal the value computed from the operand sums -- bit-exact"""
+    print("case int8 full size", m, n, k, flush=True)
+    lib = L.load()
+    g = torch.Generator(device="cuda").manual_seed(m + k)
+    a = torch.randint(-127, 128, (m, k), dtype=torch.int8, device="cuda", generator=g)
+    b = torch.randint(-127, 128, (n, k), dtype=torch.int8, device="cuda", generator=g)
+    c = torch.empty((m, n), dtype=torch.int32, device="cuda")
+    lib.gemm_nt(a, b, c, L.I8, L.I32)
+    col, row = checksums(a, b)
+    c64 = c.double()
+    assert torch.equal(c64.sum(0), col)
+    assert torch.equal(c64.sum(1), row)
+    # one row recomputed directly
+    i = 12345 % m
+    assert torch.equal(c[i].double(), b.double() @ a[i].double())
+
+
+def test_fp8_product_at_the_size_of_the_dense_model(L):
+    """config[2]: the FFN dX product 32768 x 2048 x 8192 in e4m3 with fp32 accumulation; checksums within 1e-4 of the largest one"""
+    print("case fp8 full size", flush=True)
+    lib = L.load()
+    m, n, k = 32768, 2048, 8192
+    g = torch.Generator(device="cuda").manual_seed(3)
+    a = (torch.randn((m, k), device="cuda", generator=g) * 4).to(torch.float8_e4m3fn)
+    b = (torch.randn((n, k), device="cuda", generator=g) * 4).to(torch.float8_e4m3fn)
+    c = torch.empty((m, n), dtype=torch.float32, device="cuda")
+    lib.gemm_nt(a.view(torch.uint8), b.view(torch.uint8), c, L.E4M3, L.F32)
+    col, row = checksums(a.float(), b.float())
+    c64 = c.double()
+    # a checksum adds m (or n) results whose rounding errors (about 4e-5 of the row's largest partial sum each) are independent
+    scale = c64.abs().max().item()
+    assert (c64.sum(0) - col).abs().max().item() <= 1e-4 * scale * np.sqrt(m)
+    assert (c64.sum(1) - row).abs().max().item() <= 1e-4 * scale * np.sqrt(n)
+    i = 777
+    ref = b.double() @ a[i].double()
+    assert (c[i].double() - ref).abs().max().item() <= 2e-4 * ref.abs().max().item()
+
+
+def test_attention_at_full_size_treats_the_sequences_of_a_batch_independently(L):
+    """config[3]: 16 sequences x 2048 tokens, 16 heads.  Forward, dQ, dK and dV of one sequence taken from the batch run equal, bit
+    for bit, the run of that sequence alone (same tiles, same order of operations); dK/dV are linear in dO."""
+    print("case attention full size", flush=True)
+    B, S, H = 16, 2048, 16
+    n = B * S
+    i16 = torch.int16
+    g = torch.Generator(device="cuda").manual_seed(9)
+    q, k, v, do = [torch.randn((n, H * 128), device="cuda", generator=g).bfloat16() for _ in range(4)]
+    sc = 0.0637
+
+    def run(q, k, v, do, n, slope):
+        t = torch.arange(n, device="cuda", dtype=torch.int32)
+        start = ((t // S) * S).int().contiguous()
+        finish = torch.where(t - 1 >= start, t - 1, torch.full_like(t, -1)).int().contiguous()
+        val = torch.empty_like(q)
+        swl = torch.empty((H, n), device="cuda")
+        rl = torch.zeros(n // 128, dtype=torch.int32, device="cuda")
+        rh = torch.zeros_like(rl)
+        L.call("ts2_att_build_rev", n, n, start, finish, rl, rh)
+        L.att_forward(n, H, q.view(i16), k.view(i16), v.view(i16), start, finish, sc, slope, val.view(i16), swl)
+        ds = (val.float() * do.float()).view(n, H, 128).sum(-1).t().contiguous()
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+        L.att_backward(n, H, q.view(i16), k.view(i16), v.view(i16), do.view(i16), start, finish, rl, rh, sc, slope, swl, ds, dq.view(i16), dk.view(i16),
+                       dv.view(i16), L.BF16, 3)
+        return val, swl, dq, dk, dv, ds, (start, finish, rl, rh)
+
+    slope = 0.01
+    val, swl, dq, dk, dv, ds, aux = run(q, k, v, do, n, slope)
+    for t in (val, dq, dk, dv):
+        assert torch.isfinite(t.float()).all()
+    s = 5
+    sl = slice(s * S, (s + 1) * S)
+    val1, swl1, dq1, dk1, dv1, _, _ = run(q[sl].contiguous(), k[sl].contiguous(), v[sl].contiguous(), do[sl].contiguous(), S, slope)
+    assert torch.equal(val[sl].view(i16), val1.view(i16))
+    assert torch.equal(swl[:, sl], swl1)
+    assert torch.equal(dq[sl].view(i16), dq1.view(i16))
+    assert torch.equal(dk[sl].view(i16), dk1.view(i16))
+    assert torch.equal(dv[sl].view(i16), dv1.view(i16))
+    # the first token of a sequence sees nothing: output 0, statistics of the sink alone, no gradient to its query
+    assert (val[s * S].float() == 0).all() and (swl[:, s * S] == 0).all() and (dq[s * S].float() == 0).all()
+    # the last key of a sequence is seen by no query: no gradient
+    assert (dk[(s + 1) * S - 1].float() == 0).all() and (dv[(s + 1) * S - 1].float() == 0).all()
+    # dV is linear in dO (for fixed probabilities): dV(2 dO) = 2 dV(dO) exactly in bf16, since scaling by two is exact
+    start, finish, rl, rh = aux
+    do2 = (do.float() * 2).bfloat16()
+    dq2, dk2, dv2 = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+    L.att_backward(n, H, q.view(i16), k.view(i16), v.view(i16), do2.view(i16), start, finish, rl, rh, sc, slope, swl, (ds * 2).contiguous(), dq2.view(i16),
+                   dk2.view(i16), dv2.view(i16), L.BF16, 3)
+    assert torch.equal(dv2.float(), dv.float() * 2)
+    assert torch.equal(dk2.float(), dk.float() * 2)
+    assert torch.equal(dq2.float(), dq.float() * 2)
