@@ -83,7 +83,9 @@ def bench_linear_i8(args):
     w_scale = w.abs().amax(dim=1) / 127
     w8 = torch.clamp(torch.round(w / w_scale[:, None]), -128, 127).to(torch.int8)
     dy16 = dy.bfloat16()
-    bufs = L.MatMulBuffers(L.I8, len_, src_dim, grad_dim, k_tile=k_tile)
+    # the 4096 x 1024 delta has too few tiles for 256 CUs: two stored slices of the token axis on 256x128 tiles, packed from their sum
+    splits = args.delta_splits
+    bufs = L.MatMulBuffers(L.I8, len_, src_dim, grad_dim, k_tile=k_tile, splits=splits, share_row_max=True)
     dx = torch.empty((len_, src_dim), dtype=torch.float32, device="cuda")
     dyv = dy16.view(torch.int16)
 
@@ -116,7 +118,12 @@ def bench_linear_i8(args):
     lib = L.load()
 
     def dw():
-        lib.gemm_nt(gt, st, bufs.delta, L.I8, L.I8, k_tile_scale=tsc, k_tile=k_tile, epilogue=L.EPI_ROW_TILE_MAXNORM, tile_scale=bufs.delta_tile_scale)
+        if splits > 1:
+            part = bufs.t["partial"]
+            lib.gemm_nt(gt, st, part, L.I8, L.F32, k_tile_scale=tsc, k_tile=k_tile, split_k=splits, split_slab_bytes=grad_dim * src_dim * 4,
+                        tile_config=3, m=grad_dim)
+        else:
+            lib.gemm_nt(gt, st, bufs.delta, L.I8, L.I8, k_tile_scale=tsc, k_tile=k_tile, epilogue=L.EPI_ROW_TILE_MAXNORM, tile_scale=bufs.delta_tile_scale)
     ms_dw = event_time_ms(dw, 20)
     avg_ms = (ms_dx + ms_dw) / 2
     roof = {"bound": "mfma", "achieved": gemm_ops / (avg_ms * 1e-3) / 1e12, "peak": PEAK_INT8 / 1e12, "unit": "TFLOP/s",
@@ -363,6 +370,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="linear_i8_bwd", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--delta-splits", type=int, default=2, help="linear_i8_bwd: slices of the token axis in the delta product (1 = single pass)")
     ap.add_argument("--small", action="store_true", help="step_fp8 / moe_fp8: a reduced model for quick checks (not a valid benchmark figure)")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -85,7 +85,7 @@ typedef struct ts2_gemm_args {
     int32_t epilogue;
     ts2_mat tileScale; /* ROW_TILE_MAXNORM: fp32 [n/128][m] */
     int32_t splitK;
-    int32_t tileConfig; /* 0 = choose; 1 = 256x256 workgroup tile; 2 = 128x128 */
+    int32_t tileConfig; /* 0 = choose; 1 = 256x256 workgroup tile; 2 = 128x128; 3 = 256x128 (int8 with kTileScale, fp32 result) */
     /* Expert-grouped products (TMoeMatMulKernelCall / TMoeDeltaMatMulKernelCall, src/gpt/compute/moe_matmul.cuh:47-215):
      * tileGroup [m/128] (device): rows of A and C are grouped by expert in 128-row tiles; tile i multiplies the B slab
      *           b + tileGroup[i]*bSlabBytes (n rows each); tiles with group -1 are skipped (XpTileExpertId).
@@ -98,6 +98,9 @@ typedef struct ts2_gemm_args {
     int32_t groups;
     int64_t cSlabBytes;
     int64_t tileScaleSlabBytes;
+    /* splitK > 1 with splitSlabBytes != 0: slice i of the contraction is STORED to c + i*splitSlabBytes (fp32, TS2_EPI_STORE; slices
+     * are whole k-tiles) instead of being added atomically: deterministic, the caller sums the slices (ts2_pack_delta does). */
+    int64_t splitSlabBytes;
     /* TS2_EPI_ROW_TILE_NORM */
     int32_t normalize;
     float vecScale;
@@ -157,6 +160,12 @@ int ts2_backprop_lolu_dscale(int32_t len, int32_t lenRound, const ts2_mat *gate,
 int ts2_normalize_vecs_row_max(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, const float *colScale,
     const ts2_mat *dst, float *rowScale, void *stream);
 
+/* the same, also writing rowAbsMax[t] = abs-max of row t before the column scales (NULL: not wanted); ts2_tile_max_from_rows turns
+ * those into the k-tile maxima tileMax[t/kTile] = max_t rowAbsMax[t]*|rowMult[t]| without another pass over the matrix */
+int ts2_normalize_vecs_row_max2(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, const float *colScale,
+    const ts2_mat *dst, float *rowScale, float *rowAbsMax, void *stream);
+int ts2_tile_max_from_rows(int32_t len, const float *rowAbsMax, const float *rowMult, int32_t kTile, float *tileMax, void *stream);
+
 /* Per-k-tile abs-max of a [len][dim] matrix (optionally times rowMult[t]): tileMax[t/kTile] = max |src|, the first half of
  * ShuffleMaxScaleTransposeKernel (src/gpt/compute/matmul_fwdbwd.cuh:209-231) without the sort.  tileMax must be zeroed by the
  * caller or with clear=1. */
@@ -170,6 +179,12 @@ int ts2_tile_absmax(int32_t len, const ts2_mat *src, int32_t srcType, const floa
  * rowIndex (optional, [lenRound], -1 = zero row) gathers source rows first (MoeGroupSamples, moe_kernels.cuh:89-143). */
 int ts2_transpose_quant(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, const float *rowMult, const float *tileMax,
     int32_t kTile, const int32_t *rowIndex, const ts2_mat *dstT, int32_t dstType, float *tileScale, void *stream);
+
+/* Compress (src/gpt/matrix/delta.cpp:155-179) of a sum of fp32 partial products: delta = packed(alpha * (*alphaPtr) * sum_i partial_i),
+ * partial_i = fp32 [rows][cols] at partial->ptr + i*slabBytes; the same arithmetic as TS2_EPI_ROW_TILE_MAXNORM.  Used with the stored
+ * split-K products of ts2_gemm_nt (splitSlabBytes). */
+int ts2_pack_delta(const ts2_mat *partial, int32_t splits, int64_t slabBytes, int32_t rows, int32_t cols, float alpha, const float *alphaPtr,
+    const ts2_mat *delta, const ts2_mat *deltaTileScale, void *stream);
 
 /* ------------------------------------------------------------------------------------------------------------------------
  * Linear-layer backward operator = TMatMulBuffers::{BackpropMulti, BackpropDelta} + Backprop()
@@ -192,6 +207,15 @@ typedef struct ts2_matmul_bwd_buffers {
     float *tileMax;
     float *tileScale;
     ts2_mat transformT;
+    /* optional: fp32 [splits*gradDim][srcDim].  When present (ptr != NULL, splits > 1) BackpropDelta runs the product as `splits`
+     * deterministic slices of the token axis on the large tile and packs their sum (ts2_pack_delta): faster when gradDim x srcDim
+     * has too few tiles to fill the device; the fp32 sum is then associated per slice (slices are whole k-tiles). */
+    ts2_mat partial;
+    int32_t splits;
+    /* optional (I8): [lenRound] abs-max of every row of the gradient, written by BackpropMulti.  BackpropDelta reads it instead of
+     * scanning the gradient again when gradRowAbsMaxValid != 0: the caller sets that when both calls get the same gradient tensor. */
+    float *gradRowAbsMax;
+    int32_t gradRowAbsMaxValid;
 } ts2_matmul_bwd_buffers;
 
 /* BackpropMulti (prep of dX): I8: quantise grad (TS2_BF16 | TS2_F32, optionally times gradColScale[gradDim]) per row to

@@ -144,3 +144,71 @@ def test_fp8_linear_backward(L, orc):
     err = np.abs(got_delta - ref_delta).max() / np.abs(ref_delta).max()
     print("fp8 delta rel err", err)
     assert err <= 5e-3
+
+
+@pytest.mark.parametrize("mode", ["i8", "e4m3"])
+def test_delta_as_stored_slices_plus_pack_matches_the_single_pass(L, orc, mode):
+    """BackpropDelta with a `partial` workspace: the token axis is cut into slices whose products are stored in fp32 and packed from
+    their sum.  Same quantised operands and the same exact int32 sums per k-tile; only the association of the fp32 additions differs
+    (per slice, then across slices), so packed bytes may differ from the single-pass result by one unit in rare places."""
+    print("case delta split slices", mode, flush=True)
+    len_, src_dim, grad_dim, kt, splits = 2048, 256, 512, 256, 4
+    r = np.random.default_rng(21)
+    dy = (r.standard_normal((len_, grad_dim)) * (0.2 + r.random((len_, 1)))).astype(np.float32)
+    x = orc.normalize_state(r.standard_normal((len_, src_dim)).astype(np.float32), src_dim // 128)
+    if mode == "i8":
+        m = L.I8
+        xs = torch.from_numpy(orc.convert_i8(x, 24.0)).cuda()
+        g = torch.from_numpy(dy).bfloat16().cuda().view(torch.int16)
+        gt = L.BF16
+    else:
+        m = L.E4M3
+        xs = (torch.from_numpy(x).cuda() * 24).to(torch.float8_e4m3fn).view(torch.uint8)
+        g = (torch.from_numpy(dy).cuda() * 64).to(torch.float8_e4m3fn).view(torch.uint8)
+        gt = L.E4M3
+    one = L.MatMulBuffers(m, len_, src_dim, grad_dim, k_tile=kt)
+    cut = L.MatMulBuffers(m, len_, src_dim, grad_dim, k_tile=kt, splits=splits)
+    cut.delta.fill_(55)
+    one.backprop_delta(len_, xs, None, g, gt, alpha=0.5)
+    cut.backprop_delta(len_, xs, None, g, gt, alpha=0.5)
+    torch.cuda.synchronize()
+    a, b = one.delta_fp32().cpu().numpy(), cut.delta_fp32().cpu().numpy()
+    np.testing.assert_allclose(cut.delta_tile_scale.cpu().numpy(), one.delta_tile_scale.cpu().numpy(), rtol=3e-6)
+    dd = np.abs(cut.delta.cpu().numpy().astype(np.int32) - one.delta.cpu().numpy())
+    assert dd.max() <= 1 and (dd != 0).mean() < 2e-3
+    assert np.abs(a - b).max() <= np.abs(a).max() / 127 * 1.01
+    if mode == "i8":
+        # the slices themselves: partial i equals the k-tile sum over its own token range (exact int32 per k-tile; the fp32 additions
+        # of the tiles are fused multiply-adds on the device, separate operations in the oracle)
+        part = cut.t["partial"].cpu().numpy().reshape(splits, grad_dim, src_dim)
+        qk = cut.t["gradT"].cpu().numpy().T.copy(); x8 = cut.t["srcT"].cpu().numpy().T.copy(); tsc = cut.t["tileScale"].cpu().numpy()
+        import ctypes as C
+        per = len_ // splits
+        for i in range(splits):
+            acc = np.zeros((grad_dim, src_dim), np.float32)
+            orc.lib.orc_gemm_i8_nt_ktile(_ptr(np.ascontiguousarray(qk[i * per:(i + 1) * per].T)), _ptr(np.ascontiguousarray(x8[i * per:(i + 1) * per].T)),
+                                         _ptr(np.ascontiguousarray(tsc[i * per // kt:(i + 1) * per // kt])), kt, C.c_float(1.0), _ptr(acc), grad_dim, src_dim, per)
+            assert np.abs(part[i] - acc).max() <= 2e-7 * np.abs(acc).max() * (per // kt)
+
+
+def test_delta_from_shared_row_maxima_is_identical(L, orc):
+    """BackpropMulti can leave the abs-max of every gradient row behind; BackpropDelta then builds its k-tile scales from those instead
+    of reading the gradient again.  Same maxima, same scales: the packed delta is identical."""
+    print("case shared row maxima", flush=True)
+    len_, len_round, src_dim, grad_dim, kt = 900, 1024, 256, 384, 256
+    r = np.random.default_rng(31)
+    dy = torch.from_numpy((r.standard_normal((len_, grad_dim)) * (0.2 + r.random((len_, 1)))).astype(np.float32)).bfloat16().cuda().view(torch.int16)
+    x8 = torch.zeros((len_round, src_dim), dtype=torch.int8, device="cuda")
+    x8[:len_] = torch.from_numpy(orc.convert_i8(orc.normalize_state(r.standard_normal((len_, src_dim)).astype(np.float32), 2), 24.0)).cuda()
+    w8 = torch.randint(-100, 100, (grad_dim, src_dim), dtype=torch.int8, device="cuda")
+    col = torch.rand(grad_dim, device="cuda") + 0.5
+    xs = torch.rand(len_round, device="cuda") + 0.5
+    res = []
+    for share in (False, True):
+        b = L.MatMulBuffers(L.I8, len_round, src_dim, grad_dim, k_tile=kt, share_row_max=share)
+        b.backprop_multi(len_, w8, dy, L.BF16, col)
+        b.backprop_delta(len_, x8, xs, dy, L.BF16)
+        torch.cuda.synchronize()
+        res.append((b.delta.cpu().numpy(), b.delta_tile_scale.cpu().numpy(), b.t["tileScale"].cpu().numpy()))
+    for a, c in zip(*res):
+        np.testing.assert_array_equal(a, c)

@@ -283,83 +283,109 @@ __global__ void __launch_bounds__(256) BackpropLoLU(int len, int lenRound, int t
     }
 }
 
-// One workgroup per row; the row stays in registers between the abs-max pass and the quantise pass when it has at most 4096
-// elements (REG), otherwise it is read twice (the second read is served by L2).
+// Workgroups walk rows with a grid stride; a row stays in registers between the abs-max pass and the quantise pass when it has at
+// most 4096 elements (REG) and the next row is fetched before the current one is reduced, so a workgroup always has loads in
+// flight.  Longer rows are read twice (the second read is served by L2).
 template <class TSrc, bool REG>
-__global__ void __launch_bounds__(256) NormalizeVecsRowMax(int len, int dim, Mat src, const float *colScale, Mat dst, float *rowScale)
+__global__ void __launch_bounds__(256) NormalizeVecsRowMax(int len, int lenRound, int dim, Mat src, const float *colScale, Mat dst, float *rowScale,
+    float *rowAbsMax)
 {
-    __shared__ float red[4];
-    int t = blockIdx.x;
-    int tid = threadIdx.x;
-    if (t >= len) {
-        for (int col = tid * 4; col < dim; col += 1024) {
-            *(uint32_t *)At<TI8>(dst, t, col) = 0;
-        }
-        if (tid == 0) {
-            rowScale[t] = 0;
-        }
-        return;
-    }
-    float mx = 0;
-    F4 keep[4];
-    if (REG) {
+    __shared__ float red[2][4], redPlain[2][4];
+    const int tid = threadIdx.x;
+    F4 next[4];
+    auto fetch = [&](int t) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             int col = tid * 4 + i * 1024;
-            keep[i] = col < dim ? Load4<TSrc>(At<TSrc>(src, t, col)) : ZeroF4();
+            next[i] = (REG && t < len && col < dim) ? Load4<TSrc>(At<TSrc>(src, t, col)) : ZeroF4();
         }
-        if (colScale) {
+    };
+    fetch(blockIdx.x);
+    int phase = 0;
+    for (int t = blockIdx.x; t < lenRound; t += gridDim.x, phase ^= 1) {
+        if (t >= len) {
+            for (int col = tid * 4; col < dim; col += 1024) {
+                *(uint32_t *)At<TI8>(dst, t, col) = 0;
+            }
+            if (tid == 0) {
+                rowScale[t] = 0;
+                if (rowAbsMax) {
+                    rowAbsMax[t] = 0;
+                }
+            }
+            continue;
+        }
+        float mx = 0, plain = 0; // plain: abs-max of the row before the column scales (what the delta's k-tile scale is built from)
+        F4 keep[4];
+        if (REG) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                keep[i] = next[i];
+            }
+            fetch(t + gridDim.x);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                plain = fmaxf(plain, HMaxAbs(keep[i]));
+            }
+            if (colScale) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    int col = tid * 4 + i * 1024;
+                    if (col < dim) {
+                        keep[i] = keep[i] * Load4<TF32>(colScale + col);
+                    }
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                mx = fmaxf(mx, HMaxAbs(keep[i]));
+            }
+        } else {
+            for (int col = tid * 4; col < dim; col += 1024) {
+                F4 v = Load4<TSrc>(At<TSrc>(src, t, col));
+                plain = fmaxf(plain, HMaxAbs(v));
+                if (colScale) {
+                    v = v * Load4<TF32>(colScale + col);
+                }
+                mx = fmaxf(mx, HMaxAbs(v));
+            }
+        }
+        mx = WaveMax(mx);
+        plain = WaveMax(plain);
+        if ((tid & 63) == 0) {
+            red[phase][tid >> 6] = mx;
+            redPlain[phase][tid >> 6] = plain;
+        }
+        __syncthreads(); // the two phases of the exchange arrays make one barrier per row enough
+        mx = fmaxf(fmaxf(red[phase][0], red[phase][1]), fmaxf(red[phase][2], red[phase][3]));
+        if (tid == 0 && rowAbsMax) {
+            rowAbsMax[t] = fmaxf(fmaxf(redPlain[phase][0], redPlain[phase][1]), fmaxf(redPlain[phase][2], redPlain[phase][3]));
+        }
+        float discr = 0, mult = 0;
+        if (mx > 0) {
+            discr = mx / 127;
+            mult = 1 / discr;
+        }
+        if (REG) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 int col = tid * 4 + i * 1024;
                 if (col < dim) {
-                    keep[i] = keep[i] * Load4<TF32>(colScale + col);
+                    Store4<TI8>(At<TI8>(dst, t, col), keep[i] * mult);
                 }
             }
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            mx = fmaxf(mx, HMaxAbs(keep[i]));
-        }
-    } else {
-        for (int col = tid * 4; col < dim; col += 1024) {
-            F4 v = Load4<TSrc>(At<TSrc>(src, t, col));
-            if (colScale) {
-                v = v * Load4<TF32>(colScale + col);
-            }
-            mx = fmaxf(mx, HMaxAbs(v));
-        }
-    }
-    mx = WaveMax(mx);
-    if ((tid & 63) == 0) {
-        red[tid >> 6] = mx;
-    }
-    __syncthreads();
-    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    float discr = 0, mult = 0;
-    if (mx > 0) {
-        discr = mx / 127;
-        mult = 1 / discr;
-    }
-    if (REG) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            int col = tid * 4 + i * 1024;
-            if (col < dim) {
-                Store4<TI8>(At<TI8>(dst, t, col), keep[i] * mult);
+        } else {
+            for (int col = tid * 4; col < dim; col += 1024) {
+                F4 v = Load4<TSrc>(At<TSrc>(src, t, col));
+                if (colScale) {
+                    v = v * Load4<TF32>(colScale + col);
+                }
+                Store4<TI8>(At<TI8>(dst, t, col), v * mult);
             }
         }
-    } else {
-        for (int col = tid * 4; col < dim; col += 1024) {
-            F4 v = Load4<TSrc>(At<TSrc>(src, t, col));
-            if (colScale) {
-                v = v * Load4<TF32>(colScale + col);
-            }
-            Store4<TI8>(At<TI8>(dst, t, col), v * mult);
+        if (tid == 0) {
+            rowScale[t] = discr;
         }
-    }
-    if (tid == 0) {
-        rowScale[t] = discr;
     }
 }
 
@@ -368,6 +394,29 @@ __global__ void FillFloats(float *p, int n, float v)
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) {
         p[i] = v;
+    }
+}
+
+// tileMax[kt] = max over the k-tile's rows of rowAbsMax[t] * |rowMult[t]|: the k-tile abs-max when the row maxima are already known
+__global__ void __launch_bounds__(256) TileMaxFromRows(int len, const float *rowAbsMax, const float *rowMult, int kTile, float *tileMax)
+{
+    __shared__ float red[4];
+    int t0 = blockIdx.x * kTile;
+    float mx = 0;
+    for (int t = t0 + threadIdx.x; t < t0 + kTile && t < len; t += 256) {
+        float m = rowAbsMax[t];
+        if (rowMult) {
+            m *= fabsf(rowMult[t]);
+        }
+        mx = fmaxf(mx, m);
+    }
+    mx = WaveMax(mx);
+    if ((threadIdx.x & 63) == 0) {
+        red[threadIdx.x >> 6] = mx;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        tileMax[blockIdx.x] = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
     }
 }
 
@@ -628,6 +677,50 @@ __global__ void __launch_bounds__(256) BackpropRowTileNormalizeRope(int len, int
     }
 }
 
+// sum of `splits` fp32 partial products (slabs of [rows][cols]) -> packed delta: per row and 128-column tile scale = maxabs/127,
+// bytes = sat_i8(rne(v/scale)), TileScale[tile][row] = scale: the arithmetic of the GEMM's ROW_TILE_MAXNORM epilogue applied to the sum
+__global__ void __launch_bounds__(256) PackDelta(int rows, int tiles, int splits, const uint8_t *partial, int64_t ldPartial, int64_t slab, float alpha,
+    const float *alphaPtr, Mat delta, Mat tileScale)
+{
+    int t0, tile, h;
+    if (!Unit(rows, tiles, &t0, &tile, &h)) {
+        return;
+    }
+    float scale = alpha;
+    if (alphaPtr) {
+        scale *= *alphaPtr;
+    }
+    int col = tile * TILE + h * 4;
+    F4 v[U];
+    float discr[U];
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+        v[k] = ZeroF4();
+    }
+    for (int sIdx = 0; sIdx < splits; ++sIdx) {
+#pragma unroll
+        for (int k = 0; k < U; ++k) {
+            if (t0 + k < rows) {
+                v[k] = v[k] + Load4<TF32>(partial + sIdx * slab + (int64_t)(t0 + k) * ldPartial + (int64_t)col * 4);
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+        float mx = Half32Max(HMaxAbs(v[k])) * fabsf(scale);
+        discr[k] = 0;
+        float mult = 0;
+        if (mx > 0) {
+            discr[k] = mx / 127;
+            mult = 1 / discr[k];
+        }
+        if (t0 + k < rows) {
+            Store4<TI8>(At<TI8>(delta, t0 + k, col), v[k] * scale * mult);
+        }
+    }
+    StoreScales(tileScale, tile, t0, rows, h, discr);
+}
+
 bool MatOk(const ts2_mat *m, int rows, int cols, int elemSize)
 {
     return m && m->ptr && m->y >= rows && m->x >= cols && (m->strideBytes % 4) == 0 && m->strideBytes >= (int64_t)cols * elemSize;
@@ -829,8 +922,30 @@ extern "C" int ts2_backprop_lolu_dscale(int32_t len, int32_t lenRound, const ts2
         dScale, stream);
 }
 
+extern "C" int ts2_tile_max_from_rows(int32_t len, const float *rowAbsMax, const float *rowMult, int32_t kTile, float *tileMax, void *stream)
+{
+    if (!rowAbsMax || !tileMax) {
+        return TS2_ERR_NULL;
+    }
+    if (kTile <= 0 || kTile % 128 || len <= 0) {
+        return TS2_ERR_SHAPE;
+    }
+    hipLaunchKernelGGL(TileMaxFromRows, dim3((len + kTile - 1) / kTile), dim3(256), 0, STREAM, len, rowAbsMax, rowMult, kTile, tileMax);
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
+extern "C" int ts2_normalize_vecs_row_max2(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, const float *colScale,
+    const ts2_mat *dst, float *rowScale, float *rowAbsMax, void *stream);
+
 extern "C" int ts2_normalize_vecs_row_max(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, const float *colScale,
     const ts2_mat *dst, float *rowScale, void *stream)
+{
+    return ts2_normalize_vecs_row_max2(len, lenRound, src, srcType, colScale, dst, rowScale, nullptr, stream);
+}
+
+extern "C" int ts2_normalize_vecs_row_max2(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, const float *colScale,
+    const ts2_mat *dst, float *rowScale, float *rowAbsMax, void *stream)
 {
     if (!src || !dst || !rowScale) {
         return TS2_ERR_NULL;
@@ -840,7 +955,7 @@ extern "C" int ts2_normalize_vecs_row_max(int32_t len, int32_t lenRound, const t
         return TS2_ERR_SHAPE;
     }
     const bool reg = dim <= 4096;
-#define LAUNCH_RM(TS, REG) hipLaunchKernelGGL((NormalizeVecsRowMax<TS, REG>), dim3(lenRound), dim3(256), 0, STREAM, len, dim, M(*src), colScale, M(*dst), rowScale)
+#define LAUNCH_RM(TS, REG) hipLaunchKernelGGL((NormalizeVecsRowMax<TS, REG>), dim3(lenRound < 4096 ? lenRound : 4096), dim3(256), 0, STREAM, len, lenRound, dim, M(*src), colScale, M(*dst), rowScale, rowAbsMax)
     if (srcType == TS2_BF16) {
         if (reg) {
             LAUNCH_RM(TBF16, true);
@@ -981,6 +1096,23 @@ extern "C" int ts2_backprop_row_tile_normalize_rope(int32_t len, int32_t lenRoun
         TS2_DISPATCH_TYPE(dstType, TD, LAUNCH_BR(TBF16, TD));
     }
 #undef LAUNCH_BR
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
+extern "C" int ts2_pack_delta(const ts2_mat *partial, int32_t splits, int64_t slabBytes, int32_t rows, int32_t cols, float alpha, const float *alphaPtr,
+    const ts2_mat *delta, const ts2_mat *deltaTileScale, void *stream)
+{
+    if (!partial || !delta || !deltaTileScale) {
+        return TS2_ERR_NULL;
+    }
+    if (cols % TILE || splits < 1 || !MatOk(partial, rows, cols, 4) || !MatOk(delta, rows, cols, 1) || !MatOk(deltaTileScale, cols / TILE, rows, 4) ||
+        (slabBytes & 15) || (partial->strideBytes & 15) || ((uintptr_t)partial->ptr & 15)) {
+        return TS2_ERR_SHAPE;
+    }
+    int tiles = cols / TILE;
+    hipLaunchKernelGGL(PackDelta, GridFor(rows, tiles), dim3(256), 0, STREAM, rows, tiles, splits, (const uint8_t *)partial->ptr, partial->strideBytes,
+        slabBytes, alpha, alphaPtr, M(*delta), M(*deltaTileScale));
     TS2_CHECK_LAUNCH();
     return TS2_OK;
 }

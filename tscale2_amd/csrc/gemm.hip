@@ -40,6 +40,8 @@ struct GemmP {
     int64_t tileScaleSlab;   // floats
     int splitK_groups;       // number of groups when groupOffsets is set
     int direct;              // 1: direct global->LDS loader
+    int splits;              // >1 with splitSlab: blockIdx.y = slice of the contraction, partial product stored to c + y * splitSlab
+    int64_t splitSlab;       // bytes
     // row-tile normalise / rope epilogue (C_BF16NORM)
     int normalize;
     float vecScale;
@@ -612,6 +614,15 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN) / 4) GemmNTDirect(Gemm
         }
     }
 
+    if (p.splits > 1) {
+        // deterministic split of the contraction: slice y of p.splits, partial product to its own slab of C
+        int per = (kSteps + p.splits - 1) / p.splits;
+        kBeg = blockIdx.y * per;
+        kSteps = kSteps - kBeg < per ? kSteps - kBeg : per;
+        kSteps = kSteps < 0 ? 0 : kSteps;
+        p.c += (int64_t)blockIdx.y * p.splitSlab;
+    }
+
     // loader: wave w fills the 8-row blocks w, w+4, w+8, ... of each operand tile; inside a block lane -> (row = lane/8, slot = lane%8)
     // and the slot holds chunk slot ^ ((row >> 1) & 7) of the row.  All blocks of one wave have the same parity, so the chunk is fixed.
     const int lrow = wave * 8 + (lane >> 3);
@@ -776,7 +787,8 @@ template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT> int Launch(const
     }
     int nb = q.tilesM * q.tilesN * (p.splitK > 1 ? p.splitK : 1);
     if (p.direct && p.splitK <= 1) {
-        hipLaunchKernelGGL((GemmNTDirect<TYPE, WTM, WTN, CT, EPI, KT>), dim3(nb, p.groupOffsets ? p.splitK_groups : 1), dim3(256), 0, stream, q);
+        int gy = p.groupOffsets ? p.splitK_groups : (p.splits > 1 ? p.splits : 1);
+        hipLaunchKernelGGL((GemmNTDirect<TYPE, WTM, WTN, CT, EPI, KT>), dim3(nb, gy), dim3(256), 0, stream, q);
         TS2_CHECK_LAUNCH();
         return TS2_OK;
     }
@@ -822,7 +834,7 @@ template <int TYPE, int WTM, int WTN> int DispatchEpi(const ts2_gemm_args *a, co
         return TS2_ERR_UNSUPPORTED;
     }
     if (kt) {
-        if constexpr (TYPE == T_I8 && WTM == 2) {
+        if constexpr (TYPE == T_I8 && (WTM == 2 || (WTM == 4 && WTN == 2))) {
             if (a->cType == TS2_F32) {
                 return epi == TS2_EPI_ADD ? Launch<TYPE, WTM, WTN, C_F32, TS2_EPI_ADD, true>(p, stream)
                                           : Launch<TYPE, WTM, WTN, C_F32, TS2_EPI_STORE, true>(p, stream);
@@ -838,7 +850,7 @@ template <int TYPE, int WTM, int WTN> int DispatchEpi(const ts2_gemm_args *a, co
         }
         return TS2_ERR_UNSUPPORTED;
     }
-    const bool eight = WTM == 4 && (a->tileConfig & 8) && p.splitK <= 1;
+    const bool eight = WTM == 4 && WTN == 4 && (a->tileConfig & 8) && p.splitK <= 1;
     if (a->cType == TS2_F32) {
         if (eight) {
             return epi == TS2_EPI_ADD ? Launch8<TYPE, C_F32, TS2_EPI_ADD>(p, stream) : Launch8<TYPE, C_F32, TS2_EPI_STORE>(p, stream);
@@ -867,6 +879,15 @@ template <int TYPE> int DispatchTile(const ts2_gemm_args *a, const GemmP &p, hip
     // the 256x256 kernel needs full tiles and has no room for the second accumulator set of the k-tile-scaled variant
     if (cfg == 1 && !a->kTileScale && !p.tileGroup && (p.m % 256) == 0 && (p.n % 256) == 0) {
         return DispatchEpi<TYPE, 4, 4>(a, p, stream);
+    }
+    // 256x128: the large tile that still holds both accumulator sets (int8 with k-tile scales, fp32 result)
+    if (cfg == 3) {
+        if constexpr (TYPE == T_I8) {
+            if (a->kTileScale && a->cType == TS2_F32 && !p.tileGroup && (p.m % 256) == 0) {
+                return DispatchEpi<TYPE, 4, 2>(a, p, stream);
+            }
+        }
+        return TS2_ERR_UNSUPPORTED;
     }
     return DispatchEpi<TYPE, 2, 2>(a, p, stream);
 }
@@ -942,6 +963,21 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
             (a->rope.ptr && (a->rope.y < (a->mLive > 0 ? a->mLive : a->m) || a->rope.x < 128 || (a->rope.strideBytes & 7) || ((uintptr_t)a->rope.ptr & 7)))) {
             return TS2_ERR_SHAPE;
         }
+    }
+    p.splits = 1;
+    p.splitSlab = 0;
+    if (a->splitSlabBytes) {
+        // stored (not atomically added) partial products: needs the direct kernel, fp32 results and slices of whole k-tiles
+        int kStepsAll = (int)(((int64_t)a->k * esz) / BKB);
+        int per = (kStepsAll + splitK - 1) / splitK;
+        if (splitK <= 1 || a->cType != TS2_F32 || a->epilogue != TS2_EPI_STORE || a->tileGroup || a->groupOffsets || (a->tileConfig & 4) ||
+            (a->kTileScale && (per * BKB) % (a->kTile * esz)) || (a->splitSlabBytes & 7)) {
+            return TS2_ERR_UNSUPPORTED;
+        }
+        p.splits = splitK;
+        p.splitSlab = a->splitSlabBytes;
+        splitK = 1;
+        p.splitK = 1;
     }
     p.direct = (a->tileConfig & 4) ? 0 : 1; // bit 2 of tileConfig selects the register-staged loader (kept for comparison)
     if ((a->tileGroup || a->groupOffsets) && splitK > 1) {

@@ -26,7 +26,7 @@ extern "C" int ts2_matmul_backprop_multi(int32_t mode, int32_t len, int32_t lenR
         if (!grad || !buf->grad8RowScale) {
             return TS2_ERR_NULL;
         }
-        int rc = ts2_normalize_vecs_row_max(len, lenRound, grad, gradType, gradColScale, &buf->grad8, buf->grad8RowScale, stream);
+        int rc = ts2_normalize_vecs_row_max2(len, lenRound, grad, gradType, gradColScale, &buf->grad8, buf->grad8RowScale, buf->gradRowAbsMax, stream);
         if (rc) {
             return rc;
         }
@@ -85,7 +85,11 @@ extern "C" int ts2_matmul_backprop_delta(int32_t mode, int32_t len, int32_t lenR
         if (kTile <= 0 || kTile % 128 || lenRound % kTile || !buf->tileMax || !buf->tileScale) {
             return TS2_ERR_SHAPE;
         }
-        rc = ts2_tile_absmax(len, grad, gradType, srcRowScale, kTile, buf->tileMax, 1, stream);
+        if (buf->gradRowAbsMax && buf->gradRowAbsMaxValid) {
+            rc = ts2_tile_max_from_rows(len, buf->gradRowAbsMax, srcRowScale, kTile, buf->tileMax, stream);
+        } else {
+            rc = ts2_tile_absmax(len, grad, gradType, srcRowScale, kTile, buf->tileMax, 1, stream);
+        }
         if (rc) {
             return rc;
         }
@@ -110,12 +114,35 @@ extern "C" int ts2_matmul_backprop_delta(int32_t mode, int32_t len, int32_t lenR
     }
     g.a = buf->gradT;
     g.b = buf->srcT;
-    g.c = *delta;
     g.abType = mode;
-    g.cType = TS2_I8;
     g.m = gradDim;
     g.n = srcDim;
     g.k = lenRound;
+    const int splits = buf->partial.ptr ? buf->splits : 1;
+    if (splits > 1) {
+        // few output tiles: slices of the token axis as separate stored products on the large tile, then pack their sum
+        int esz = 1;
+        int64_t sliceBytes = ((int64_t)lenRound * esz / 128 + splits - 1) / splits * 128;
+        bool ok = buf->partial.y >= splits * gradDim && buf->partial.x >= srcDim && (mode != TS2_I8 || sliceBytes % kTile == 0);
+        if (!ok) {
+            return TS2_ERR_SHAPE;
+        }
+        g.c = buf->partial;
+        g.c.y = gradDim;
+        g.cType = TS2_F32;
+        g.alpha = 1.f;
+        g.epilogue = TS2_EPI_STORE;
+        g.splitK = splits;
+        g.splitSlabBytes = (int64_t)gradDim * buf->partial.strideBytes;
+        g.tileConfig = mode == TS2_I8 ? ((gradDim % 256) == 0 ? 3 : 2) : (((gradDim % 256) == 0 && (srcDim % 256) == 0) ? 1 : 2);
+        rc = ts2_gemm_nt(&g, stream);
+        if (rc) {
+            return rc;
+        }
+        return ts2_pack_delta(&buf->partial, splits, g.splitSlabBytes, gradDim, srcDim, alpha, gradScale, delta, deltaTileScale, stream);
+    }
+    g.c = *delta;
+    g.cType = TS2_I8;
     g.alpha = alpha;
     g.alphaPtr = gradScale;
     g.epilogue = TS2_EPI_ROW_TILE_MAXNORM;

@@ -19,7 +19,7 @@ class GemmArgs(C.Structure):
                 ("k", C.c_int32), ("mLive", C.c_int32), ("rowScale", C.c_void_p), ("kTileScale", C.c_void_p), ("kTile", C.c_int32),
                 ("alpha", C.c_float), ("alphaPtr", C.c_void_p), ("epilogue", C.c_int32), ("tileScale", Mat), ("splitK", C.c_int32),
                 ("tileConfig", C.c_int32), ("tileGroup", C.c_void_p), ("bSlabBytes", C.c_int64), ("groupOffsets", C.c_void_p),
-                ("groups", C.c_int32), ("cSlabBytes", C.c_int64), ("tileScaleSlabBytes", C.c_int64), ("normalize", C.c_int32),
+                ("groups", C.c_int32), ("cSlabBytes", C.c_int64), ("tileScaleSlabBytes", C.c_int64), ("splitSlabBytes", C.c_int64), ("normalize", C.c_int32),
                 ("vecScale", C.c_float), ("rope", Mat)]
 
 
@@ -57,7 +57,7 @@ class Lib:
     def gemm_nt(self, a, b, c, ab_type, c_type, row_scale=None, k_tile_scale=None, k_tile=0, alpha=1.0, alpha_ptr=None,
                 epilogue=EPI_STORE, tile_scale=None, split_k=1, m_live=0, tile_config=0, k=None, check=True, m=None, n=None,
                 tile_group=None, b_slab_bytes=0, group_offsets=None, groups=0, c_slab_bytes=0, tile_scale_slab_bytes=0,
-                normalize=False, vec_scale=1.0, rope=None):
+                normalize=False, vec_scale=1.0, rope=None, split_slab_bytes=0):
         args = GemmArgs()
         args.a, args.b, args.c = mat(a), mat(b), mat(c)
         args.abType, args.cType = ab_type, c_type
@@ -77,6 +77,7 @@ class Lib:
         args.splitK = split_k
         args.tileConfig = tile_config
         args.normalize, args.vecScale, args.rope = int(normalize), vec_scale, mat(rope)
+        args.splitSlabBytes = split_slab_bytes
         rc = self.dll.ts2_gemm_nt(C.byref(args), self.stream())
         if check:
             self.check(rc, "ts2_gemm_nt")
@@ -148,14 +149,15 @@ def probe_copy_rate(nbytes=1 << 30):
 
 class BwdBuffers(C.Structure):
     _fields_ = [("grad8", Mat), ("grad8RowScale", C.c_void_p), ("gradT", Mat), ("srcT", Mat), ("tileMax", C.c_void_p), ("tileScale", C.c_void_p),
-                ("transformT", Mat)]
+                ("transformT", Mat), ("partial", Mat), ("splits", C.c_int32), ("gradRowAbsMax", C.c_void_p),
+                ("gradRowAbsMaxValid", C.c_int32)]
 
 
 class MatMulBuffers:
     """Scratch of one linear layer's backward, allocated with torch (the reference allocates the same members from its pools,
     src/gpt/compute/matmul_fwdbwd.cuh:283-311).  mode: I8 or E4M3."""
 
-    def __init__(self, mode, len_round, src_dim, grad_dim, k_tile=512):
+    def __init__(self, mode, len_round, src_dim, grad_dim, k_tile=512, splits=1, share_row_max=False):
         import torch
         self.mode, self.len_round, self.src_dim, self.grad_dim, self.k_tile = mode, len_round, src_dim, grad_dim, k_tile
         bt = torch.int8 if mode == I8 else torch.uint8
@@ -173,6 +175,15 @@ class MatMulBuffers:
         self.c = BwdBuffers()
         for k, v in self.t.items():
             setattr(self.c, k, mat(v) if v.dim() == 2 else v.data_ptr())
+        if share_row_max and mode == I8:
+            # backprop_multi and backprop_delta will be given the same gradient tensor: the delta reuses the row maxima of the first
+            self.t["gradRowAbsMax"] = torch.empty(len_round, dtype=torch.float32, device=dev)
+            self.c.gradRowAbsMax = self.t["gradRowAbsMax"].data_ptr()
+            self.c.gradRowAbsMaxValid = 1
+        if splits > 1:
+            self.t["partial"] = torch.empty((splits * grad_dim, src_dim), dtype=torch.float32, device=dev)
+            self.c.partial = mat(self.t["partial"])
+            self.c.splits = splits
         self.delta = torch.empty((grad_dim, src_dim), dtype=torch.int8, device=dev)
         self.delta_tile_scale = torch.empty((src_dim // 128, grad_dim), dtype=torch.float32, device=dev)
 
