@@ -14,12 +14,12 @@
 //         S = Q K^T,  dP = dO V^T,  dV^T += dO^T P,  dK^T += Q^T dS             (lane = key)
 //     The probability / score-gradient tiles never leave registers: an MFMA result register block is fed back as the B operand of
 //     the next product (the contraction index order of an MFMA is free as long as A and B agree).
-//   * products that contract over token rows need the streamed tile with rows along the contraction: each tile is written to LDS
-//     row-major with coalesced 16-byte loads and then re-written transposed (two rows packed per dword with v_perm_b32, padded
-//     pitches chosen so the 8-byte operand reads are bank-conflict free).
+//   * products that contract over token rows need the streamed tile with rows along the contraction: the tile is fetched one tile
+//     ahead into registers and written to LDS row-major and/or transposed (two rows packed per dword with v_perm_b32, pitches chosen
+//     so that operand reads and transposed writes are bank-conflict free); the wave's own rows are parked in LDS in fragment order.
 //   * spans are one inclusive key range per query (every causal window / document-start pattern of
-//     src/gpt/att/sliding_window.cpp:111-118,226-240); masking is evaluated per element from those ranges, tiles outside the
-//     workgroup's range are never loaded.
+//     src/gpt/att/sliding_window.cpp:111-118,226-240); masking is one unsigned compare per element, tiles outside a wave's range are
+//     skipped, tiles outside the workgroup's range are never loaded.
 #include "common.h"
 
 namespace
