@@ -196,7 +196,8 @@ def test_eight_wave_configuration_is_bit_exact(lib, orc):
 @pytest.mark.parametrize("normalize,use_rope", [(True, True), (True, False), (False, True)])
 def test_fused_row_tile_normalize_rope_epilogue_matches_the_two_pass_path(ab, normalize, use_rope):
     """TS2_EPI_ROW_TILE_NORM against the same product stored in fp32 followed by ts2_row_tile_normalize_rope: same arithmetic except
-    for the order of the 128 squares in the tile sum, so the bf16 results may differ by one unit in the last place at most."""
+    for the order of the 128 squares in the tile sum, so the bf16 results differ by one unit in the last place at most (or by fp32
+    rounding of the tile's largest values where the rotation cancels)."""
     print("case fused norm/rope epilogue", ab, normalize, use_rope, flush=True)
     from tscale2_amd import lib as L
     lib = L.load()
@@ -229,7 +230,10 @@ def test_fused_row_tile_normalize_rope_epilogue_matches_the_two_pass_path(ab, no
     torch.cuda.synchronize()
     gf, wf = got.view(torch.bfloat16).float(), want.view(torch.bfloat16).float()
     assert (gf[m_live:] == 0).all() and (gf[300:310] == 0).all()
-    tol = wf.abs() * 2.0 ** -7 + 1e-30                               # one bf16 ulp
+    # one bf16 ulp, plus a few fp32 ulps of the rotation's operands: own*cos - other*sin can cancel to far below either product, and
+    # the two paths round the tile sum (hence the products) differently in the last fp32 bit
+    tile_max = wf.abs().view(m, n // 128, 128).amax(2, keepdim=True).expand(m, n // 128, 128).reshape(m, n)
+    tol = wf.abs() * 2.0 ** -7 + tile_max * 2.0 ** -21 + 1e-30
     assert ((gf - wf).abs() <= tol).all()
     assert (gf == wf).float().mean() > 0.99
     if normalize:

@@ -177,11 +177,8 @@ __device__ __forceinline__ void BlockKeyRange(int start, int finish, int tid, in
 {
     int s = finish >= start ? start : 0x7fffffff;
     int f = finish >= start ? finish : -1;
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        s = min(s, __shfl_xor(s, o, 64));
-        f = max(f, __shfl_xor(f, o, 64));
-    }
+    s = WaveMinInt(s);
+    f = WaveMaxInt(f);
     if ((tid & 63) == 0) {
         red[(tid >> 6) * 2] = s;
         red[(tid >> 6) * 2 + 1] = f;
@@ -206,13 +203,10 @@ __device__ __forceinline__ TRowSpan MakeRowSpan(int start, int finish)
     r.start = some ? start : 0x7fffffff;
     r.len = some ? (unsigned)(finish - start) : 0u;
     int a = r.start, b = some ? finish : -1, c = r.start, d = b;
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        a = max(a, __shfl_xor(a, o, 64));
-        b = min(b, __shfl_xor(b, o, 64));
-        c = min(c, __shfl_xor(c, o, 64));
-        d = max(d, __shfl_xor(d, o, 64));
-    }
+    a = WaveMaxInt(a);
+    b = WaveMinInt(b);
+    c = WaveMinInt(c);
+    d = WaveMaxInt(d);
     r.waveMaxStart = a;
     r.waveMinFinish = b;
     r.waveMinStart = c;
@@ -312,7 +306,11 @@ __global__ void __launch_bounds__(256, 2) AttForward(AttP p)
                 }
             }
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        {
+            float lo, hi;
+            LaneSwap32(mx, &lo, &hi);
+            mx = fmaxf(lo, hi);
+        }
         float alpha = __builtin_amdgcn_exp2f(m - mx);
         const bool rescale = __any(mx != m);
         m = mx;
@@ -325,7 +323,11 @@ __global__ void __launch_bounds__(256, 2) AttForward(AttP p)
                 ps += sv[kb][e];
             }
         }
-        ps += __shfl_xor(ps, 32, 64);
+        {
+            float lo, hi;
+            LaneSwap32(ps, &lo, &hi);
+            ps = lo + hi;
+        }
         sum = sum * alpha + ps;
         if (rescale) { // wave-uniform: the maximum of no row moved in most tiles
 #pragma unroll
@@ -514,13 +516,10 @@ template <bool F32> __global__ void __launch_bounds__(256) AttGradKV(AttP p)
             stS[tid] = preS;
             stF[tid] = (int)(preF >= preS ? (unsigned)(preF - preS) : 0u); // span length
             int a = preS, b = preF, c = preS, d = preF;
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) {
-                a = max(a, __shfl_xor(a, o, 64));
-                b = min(b, __shfl_xor(b, o, 64));
-                c = min(c, __shfl_xor(c, o, 64));
-                d = max(d, __shfl_xor(d, o, 64));
-            }
+            a = WaveMaxInt(a);
+            b = WaveMinInt(b);
+            c = WaveMinInt(c);
+            d = WaveMaxInt(d);
             if (tid == 0) {
                 stT[0] = a; // latest span start of the tile's queries
                 stT[1] = b; // earliest finish

@@ -62,42 +62,118 @@ __device__ __forceinline__ float E4m3ToFloat(uint32_t byte)
     return __builtin_amdgcn_cvt_f32_fp8((int)byte, 0);
 }
 
-// wave-wide reductions (DPP/ds_swizzle generated by the compiler from __shfl_xor)
-__device__ __forceinline__ float WaveSum(float v)
+// Cross-lane exchange without the LDS crossbar: DPP modifiers inside a row of 16 lanes (they fold into the consuming VALU
+// instruction), v_permlane16_swap / v_permlane32_swap of gfx950 across rows.  A butterfly reduction over 1, 2, 4, 8 uses
+// quad_perm, quad_perm, row_half_mirror and row_mirror: once the quads (the 8-lane halves) hold one value each, the mirrored lane
+// supplies the other quad's (half's) value, so every lane ends with the same bits as with xor-shuffles.
+enum { DPP_XOR1 = 0xB1, DPP_XOR2 = 0x4E, DPP_HALF_MIRROR = 0x141, DPP_MIRROR = 0x140 };
+
+template <int CTRL> __device__ __forceinline__ float LaneDpp(float v)
 {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        v += __shfl_xor(v, o, 64);
-    }
-    return v;
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
 }
 
-__device__ __forceinline__ float WaveMax(float v)
+template <int CTRL> __device__ __forceinline__ int LaneDpp(int v)
 {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        v = fmaxf(v, __shfl_xor(v, o, 64));
-    }
-    return v;
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, true);
+}
+
+// value of lane ^ 1
+__device__ __forceinline__ float LaneXor1(float v)
+{
+    return LaneDpp<DPP_XOR1>(v);
+}
+
+// (a, b): lanes of rows 0,2 get (own, row+1's), lanes of rows 1,3 get (row-1's, own) -- any symmetric combination of a and b is
+// the xor-16 butterfly step
+__device__ __forceinline__ void LaneSwap16(float v, float *a, float *b)
+{
+    const unsigned u = __float_as_uint(v);
+    auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    const unsigned r0 = r[0], r1 = r[1]; // through scalars: a bit_cast applied to r[1] directly reads element 0
+    *a = __uint_as_float(r0);
+    *b = __uint_as_float(r1);
+}
+
+__device__ __forceinline__ void LaneSwap32(float v, float *a, float *b)
+{
+    const unsigned u = __float_as_uint(v);
+    auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const unsigned r0 = r[0], r1 = r[1]; // through scalars: a bit_cast applied to r[1] directly reads element 0
+    *a = __uint_as_float(r0);
+    *b = __uint_as_float(r1);
 }
 
 // reductions inside each aligned group of 32 lanes (one 128-wide tile held as 4 floats per lane)
 __device__ __forceinline__ float Half32Sum(float v)
 {
-#pragma unroll
-    for (int o = 16; o > 0; o >>= 1) {
-        v += __shfl_xor(v, o, 64);
-    }
-    return v;
+    v += LaneDpp<DPP_XOR1>(v);
+    v += LaneDpp<DPP_XOR2>(v);
+    v += LaneDpp<DPP_HALF_MIRROR>(v);
+    v += LaneDpp<DPP_MIRROR>(v);
+    float a, b;
+    LaneSwap16(v, &a, &b);
+    return a + b;
 }
 
 __device__ __forceinline__ float Half32Max(float v)
 {
-#pragma unroll
-    for (int o = 16; o > 0; o >>= 1) {
-        v = fmaxf(v, __shfl_xor(v, o, 64));
-    }
-    return v;
+    v = fmaxf(v, LaneDpp<DPP_XOR1>(v));
+    v = fmaxf(v, LaneDpp<DPP_XOR2>(v));
+    v = fmaxf(v, LaneDpp<DPP_HALF_MIRROR>(v));
+    v = fmaxf(v, LaneDpp<DPP_MIRROR>(v));
+    float a, b;
+    LaneSwap16(v, &a, &b);
+    return fmaxf(a, b);
+}
+
+// wave-wide reductions
+__device__ __forceinline__ float WaveSum(float v)
+{
+    v = Half32Sum(v);
+    float a, b;
+    LaneSwap32(v, &a, &b);
+    return a + b;
+}
+
+__device__ __forceinline__ float WaveMax(float v)
+{
+    v = Half32Max(v);
+    float a, b;
+    LaneSwap32(v, &a, &b);
+    return fmaxf(a, b);
+}
+
+__device__ __forceinline__ void LaneSwap16(int v, int *a, int *b)
+{
+    auto r = __builtin_amdgcn_permlane16_swap((unsigned)v, (unsigned)v, false, false);
+    *a = (int)r[0];
+    *b = (int)r[1];
+}
+
+__device__ __forceinline__ void LaneSwap32(int v, int *a, int *b)
+{
+    auto r = __builtin_amdgcn_permlane32_swap((unsigned)v, (unsigned)v, false, false);
+    *a = (int)r[0];
+    *b = (int)r[1];
+}
+
+__device__ __forceinline__ int WaveMaxInt(int v)
+{
+    v = max(v, LaneDpp<DPP_XOR1>(v));
+    v = max(v, LaneDpp<DPP_XOR2>(v));
+    v = max(v, LaneDpp<DPP_HALF_MIRROR>(v));
+    v = max(v, LaneDpp<DPP_MIRROR>(v));
+    int a, b;
+    LaneSwap16(v, &a, &b);
+    v = max(a, b);
+    LaneSwap32(v, &a, &b);
+    return max(a, b);
+}
+
+__device__ __forceinline__ int WaveMinInt(int v)
+{
+    return -WaveMaxInt(-v); // callers keep away from INT_MIN
 }
 
 static inline bool Aligned16(const void *p, int64_t stride)

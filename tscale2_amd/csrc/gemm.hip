@@ -99,7 +99,7 @@ __device__ __forceinline__ void StoreBlockBf16(uint8_t *c, int64_t ldc, int col,
     for (int e = 0; e < 16; e += 2) {
         // rows e and e+1 are consecutive rows of the block (e%4 = 0,1 or 2,3)
         float give = odd ? v[e] : v[e + 1];
-        float got = __shfl_xor(give, 1, 64);
+        float got = LaneXor1(give);
         float lo = odd ? got : v[e];
         float hi = odd ? v[e + 1] : got;
         int row = rowOf(odd ? e + 1 : e);
@@ -136,7 +136,10 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
         const int tile = (colBase + wn * (32 * WTN)) / TILE;
 #pragma unroll
         for (int i = 0; i < WTM; ++i) {
+            // phase by phase over the 16 rows of the block row, so that the cross-lane steps and the loads of the rope table of
+            // different rows are independent instructions in flight together
             float out[WTN][16];
+            float sum2[16];
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const int row = rowBase + rowLocal(i, e);
@@ -144,39 +147,75 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
                 if (p.rowScale) {
                     rs *= p.rowScale[row];
                 }
-                float v[WTN];
-                float sum2 = 0;
+                sum2[e] = 0;
 #pragma unroll
                 for (int j = 0; j < WTN; ++j) {
-                    v[j] = accVal(i, j, e) * rs;
-                    sum2 += v[j] * v[j];
+                    out[j][e] = accVal(i, j, e) * rs;
+                    sum2[e] += out[j][e] * out[j][e];
                 }
-                float discr = 0;
-                if (p.normalize) {
-                    sum2 = Half32Sum(sum2);
-                    if (sum2 > 0 && row < mLive) {
-                        discr = sqrtf(sum2 / TILE) * p.vecScale;
+            }
+            if (p.normalize) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    sum2[e] += LaneDpp<DPP_XOR1>(sum2[e]);
+                }
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    sum2[e] += LaneDpp<DPP_XOR2>(sum2[e]);
+                }
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    sum2[e] += LaneDpp<DPP_HALF_MIRROR>(sum2[e]);
+                }
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    sum2[e] += LaneDpp<DPP_MIRROR>(sum2[e]);
+                }
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    float a, b;
+                    LaneSwap16(sum2[e], &a, &b);
+                    sum2[e] = a + b;
+                }
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int row = rowBase + rowLocal(i, e);
+                    float discr = 0;
+                    if (sum2[e] > 0 && row < mLive) {
+                        discr = sqrtf(sum2[e] / TILE) * p.vecScale;
                         float inv = 1 / discr;
 #pragma unroll
                         for (int j = 0; j < WTN; ++j) {
-                            v[j] *= inv;
+                            out[j][e] *= inv;
                         }
                     }
                     if (l32 == 0) {
                         p.tileScale[(int64_t)tile * p.ldTileScale + row] = discr;
                     }
                 }
-                if (p.rope) {
+            }
+            if (p.rope) {
 #pragma unroll
-                    for (int j = 0; j < WTN; ++j) {
-                        float2 cs = *(const float2 *)(p.rope + (int64_t)row * p.ldRope + ((j * 32 + l32) & ~1));
-                        float other = __shfl_xor(v[j], 1, 64);
-                        v[j] = (l32 & 1) ? other * cs.y + v[j] * cs.x : v[j] * cs.x - other * cs.y;
+                for (int eq = 0; eq < 4; ++eq) {
+                    float2 cs[4][WTN];
+#pragma unroll
+                    for (int ee = 0; ee < 4; ++ee) {
+                        const int row = rowBase + rowLocal(i, eq * 4 + ee);
+#pragma unroll
+                        for (int j = 0; j < WTN; ++j) {
+                            cs[ee][j] = *(const float2 *)(p.rope + (int64_t)row * p.ldRope + ((j * 32 + l32) & ~1));
+                        }
                     }
-                }
 #pragma unroll
-                for (int j = 0; j < WTN; ++j) {
-                    out[j][e] = v[j];
+                    for (int ee = 0; ee < 4; ++ee) {
+                        const int e = eq * 4 + ee;
+#pragma unroll
+                        for (int j = 0; j < WTN; ++j) {
+                            float own = out[j][e];
+                            float other = LaneXor1(own);
+                            out[j][e] = (l32 & 1) ? other * cs[ee][j].y + own * cs[ee][j].x : own * cs[ee][j].x - other * cs[ee][j].y;
+                        }
+                    }
                 }
             }
 #pragma unroll
@@ -190,19 +229,48 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
         // sat_i8(rne(v/scale)), TileScale[tile][row] = scale.  A 128-column tile is 4 MFMA blocks: inside one wave when WTN == 4,
         // shared by the two waves along N when WTN == 2 (row maxima exchanged through LDS, which the main loop no longer uses).
         float *xch = (float *)lds;
+        // row maxima of a block row, all 16 rows a step at a time (independent cross-lane instructions)
+        auto blockRowMax = [&](int i, float (&mx)[16]) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                mx[e] = 0;
+#pragma unroll
+                for (int j = 0; j < WTN; ++j) {
+                    mx[e] = fmaxf(mx[e], fabsf(accVal(i, j, e)));
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                mx[e] = fmaxf(mx[e], LaneDpp<DPP_XOR1>(mx[e]));
+            }
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                mx[e] = fmaxf(mx[e], LaneDpp<DPP_XOR2>(mx[e]));
+            }
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                mx[e] = fmaxf(mx[e], LaneDpp<DPP_HALF_MIRROR>(mx[e]));
+            }
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                mx[e] = fmaxf(mx[e], LaneDpp<DPP_MIRROR>(mx[e]));
+            }
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                float a, b;
+                LaneSwap16(mx[e], &a, &b);
+                mx[e] = fmaxf(a, b);
+            }
+        };
         if (WTN == 2) {
 #pragma unroll
             for (int i = 0; i < WTM; ++i) {
+                float mx[16];
+                blockRowMax(i, mx);
+                if (l32 == 0) {
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    float mx = 0;
-#pragma unroll
-                    for (int j = 0; j < WTN; ++j) {
-                        mx = fmaxf(mx, fabsf(accVal(i, j, e)));
-                    }
-                    mx = Half32Max(mx);
-                    if (l32 == 0) {
-                        xch[rowLocal(i, e) * 2 + wn] = mx;
+                    for (int e = 0; e < 16; ++e) {
+                        xch[rowLocal(i, e) * 2 + wn] = mx[e];
                     }
                 }
             }
@@ -210,6 +278,16 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
         }
 #pragma unroll
         for (int i = 0; i < WTM; ++i) {
+            float mxs[16];
+            if (WTN == 2) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int rl = rowLocal(i, e);
+                    mxs[e] = fmaxf(xch[rl * 2], xch[rl * 2 + 1]);
+                }
+            } else {
+                blockRowMax(i, mxs);
+            }
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const int rl = rowLocal(i, e);
@@ -218,24 +296,13 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
                 if (p.rowScale) {
                     rs *= p.rowScale[row];
                 }
-                rs = fabsf(rs);
-                float mx = 0;
-                if (WTN == 2) {
-                    mx = fmaxf(xch[rl * 2], xch[rl * 2 + 1]);
-                } else {
-#pragma unroll
-                    for (int j = 0; j < WTN; ++j) {
-                        mx = fmaxf(mx, fabsf(accVal(i, j, e)));
-                    }
-                    mx = Half32Max(mx);
-                }
-                mx *= rs;
+                float mx = mxs[e] * fabsf(rs);
                 float discr = 0, mult = 0;
                 if (mx > 0 && row < mLive) {
                     discr = mx / 127;
                     mult = 1 / discr;
                 }
-                float sgnScale = (p.rowScale ? p.rowScale[row] : 1.f) * scale;
+                float sgnScale = rs;
 #pragma unroll
                 for (int j = 0; j < WTN; ++j) {
                     int col = colBase + wn * (32 * WTN) + j * 32 + l32;
