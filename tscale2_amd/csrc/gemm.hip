@@ -45,6 +45,7 @@ struct GemmP {
     int64_t tileScaleSlab;   // floats
     int splitK_groups;       // number of groups when groupOffsets is set
     int direct;              // 1: direct global->LDS loader
+    int noRing;              // 1: keep the two-stage loop for the 256x256 tile (comparison)
     int splits;              // >1 with splitSlab: blockIdx.y = slice of the contraction, partial product stored to c + y * splitSlab
     int64_t splitSlab;       // bytes
     // row-tile normalise / rope epilogue (C_BF16NORM)
@@ -842,6 +843,215 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN) / 4) GemmNTDirect(Gemm
     Epilogue<TYPE, WTM, WTN, CT, EPI, KT>(p, acc, facc, sA0, rowBase, colBase, wm, wn, half, l32);
 }
 
+// ---------------------------------------------------------------------------------------------------------------------------
+// 256x256 tile, 4 waves, with the operand stages as a ring: three 32 KB stages of A (the M side: tokens, streamed once from HBM) and
+// two of B (the N side: the smaller, cache-resident operand) = all 160 KB of LDS.  The loads of step S are B of step S+1 and A of
+// step S+2, so an A line has two full steps to arrive and a B line one; they are issued one at a time between the MFMAs (a burst of
+// sixteen 1 KB loads blocks the wave's instruction issue for about as long as the transfer takes).  Loads complete in order, so
+// "all but the newest LA" (vmcnt) at the end of a step means A(S+1) and B(S+1) have landed.  Steps past the end of K reload the last
+// step (harmless: the target stage is free) so that the loop body has no branches.  The stage arrays are separate static arrays
+// (the compiler then knows that operand reads do not alias the loads in flight), hence six steps per loop iteration.
+template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(256, 1) GemmNTRing(GemmP p)
+{
+    typedef typename AccT<TYPE>::type TAcc;
+    constexpr int WTM = 4, WTN = 4, WN = 2, NW = 4, BM = 256, BN = 256;
+    __shared__ __attribute__((aligned(1024))) uint8_t sA0[BM * BKB];
+    __shared__ __attribute__((aligned(1024))) uint8_t sA1[BM * BKB];
+    __shared__ __attribute__((aligned(1024))) uint8_t sA2[BM * BKB];
+    __shared__ __attribute__((aligned(1024))) uint8_t sB0[BN * BKB];
+    __shared__ __attribute__((aligned(1024))) uint8_t sB1[BN * BKB];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // wave-uniform: LDS targets and tile rows of the loader stay scalar
+    const int wm = wave / WN;
+    const int wn = wave % WN;
+    int tm, tn;
+    MapTile(blockIdx.x, p.tilesM * p.tilesN, p.tilesM, p.tilesN, &tm, &tn);
+    const int rowBase = tm * BM;
+    const int colBase = tn * BN;
+    int kSteps = p.kBytes / BKB;
+    int kBeg = 0;
+    if (p.groupOffsets) {
+        int g = blockIdx.y;
+        kBeg = p.groupOffsets[g] * (TYPE == T_BF16 ? 2 : 1) / BKB;
+        kSteps = p.groupOffsets[g + 1] * (TYPE == T_BF16 ? 2 : 1) / BKB - kBeg;
+        p.c += (int64_t)g * p.cSlab;
+        if (p.tileScale) {
+            p.tileScale += (int64_t)g * p.tileScaleSlab;
+        }
+    }
+    if (p.splits > 1) {
+        int per = (kSteps + p.splits - 1) / p.splits;
+        kBeg = blockIdx.y * per;
+        kSteps = kSteps - kBeg < per ? kSteps - kBeg : per;
+        kSteps = kSteps < 0 ? 0 : kSteps;
+        p.c += (int64_t)blockIdx.y * p.splitSlab;
+    }
+    const int lrow = wave * 8 + (lane >> 3);
+    const int lchunk = (lane & 7) ^ ((lrow >> 1) & 7);
+    const uint8_t *gaTile = p.a + (int64_t)rowBase * p.lda + (int64_t)kBeg * BKB;
+    const uint8_t *gbTile = p.b + (int64_t)colBase * p.ldb + (int64_t)kBeg * BKB;
+    const uint32_t gaLane = (uint32_t)(lrow * (int)p.lda + lchunk * 16);
+    const uint32_t gbLane = (uint32_t)(lrow * (int)p.ldb + lchunk * 16);
+    constexpr int LA = BM / (8 * NW);
+    constexpr int LB = BN / (8 * NW);
+    const int lastStep = kSteps - 1;
+#define RING_LOAD(GT, LD, GL, SBUF, STEP, I0, I1)                                                                                          \
+    do {                                                                                                                                   \
+        const int st_ = (STEP) < lastStep ? (STEP) : lastStep;                                                                             \
+        _Pragma("unroll") for (int i = I0; i < I1; ++i) __builtin_amdgcn_global_load_lds(                                                  \
+            TS2_GLB_PTR(GT + ((int64_t)i * (8 * NW) * LD + (int64_t)st_ * BKB) + GL), TS2_LDS_PTR(SBUF + (wave + NW * i) * 1024), 16, 0, 0); \
+    } while (0)
+#define RING_LOAD_A(SBUF, STEP, I0, I1) RING_LOAD(gaTile, p.lda, gaLane, SBUF, STEP, I0, I1)
+#define RING_LOAD_B(SBUF, STEP, I0, I1) RING_LOAD(gbTile, p.ldb, gbLane, SBUF, STEP, I0, I1)
+
+    TAcc acc[WTM][WTN];
+    v16f facc[1][1];
+#pragma unroll
+    for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+        for (int j = 0; j < WTN; ++j) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                acc[i][j][e] = 0;
+            }
+        }
+    }
+    const int half = lane >> 5;
+    const int l32 = lane & 31;
+    const int aRow0 = wm * (32 * WTM) + l32;
+    const int bRow0 = wn * (32 * WTN) + l32;
+    constexpr int NS = TYPE == T_FP8 ? 2 : 4;
+    constexpr int ND = (WTM + WTN) * (TYPE == T_FP8 ? 2 : 1); // ds_read_b128 per fragment set
+    typedef typename std::conditional<TYPE == T_FP8, v8i, v4i>::type TFrag;
+    TFrag fa[2][WTM], fb[2][WTN];
+    auto loadOne = [&](const uint8_t *base, int row, int sl) -> TFrag {
+        if constexpr (TYPE == T_FP8) {
+            int ch = sl * 4 + half * 2;
+            v4i lo = *(const v4i *)(base + SwizzleOffset(row, ch));
+            v4i hi = *(const v4i *)(base + SwizzleOffset(row, ch + 1));
+            return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        } else {
+            return *(const v4i *)(base + SwizzleOffset(row, sl * 2 + half));
+        }
+    };
+    auto mfma = [&](TFrag a, TFrag b, TAcc c) -> TAcc {
+        if constexpr (TYPE == T_I8) {
+            return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+        } else if constexpr (TYPE == T_FP8) {
+            return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+        } else {
+            return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+        }
+    };
+#define LOAD_FRAGS(SET, SA, SB, SL)                                                                                                        \
+    do {                                                                                                                                   \
+        _Pragma("unroll") for (int i = 0; i < WTM; ++i) fa[SET][i] = loadOne(SA, aRow0 + 32 * i, SL);                                      \
+        _Pragma("unroll") for (int j = 0; j < WTN; ++j) fb[SET][j] = loadOne(SB, bRow0 + 32 * j, SL);                                      \
+    } while (0)
+#define MFMA_ROWS(SET, I0, I1)                                                                                                             \
+    do {                                                                                                                                   \
+        _Pragma("unroll") for (int i = I0; i < I1; ++i) _Pragma("unroll") for (int j = 0; j < WTN; ++j) acc[i][j] =                        \
+            mfma(fa[SET][i], fb[SET][j], acc[i][j]);                                                                                       \
+    } while (0)
+    // pin the order inside a region: REP groups of (NM MFMAs, NG global loads, NDS LDS reads)
+#define INTERLEAVE(REP, NM, NG, NDS)                                                                                                       \
+    do {                                                                                                                                   \
+        _Pragma("unroll") for (int q = 0; q < REP; ++q)                                                                                    \
+        {                                                                                                                                  \
+            __builtin_amdgcn_sched_group_barrier(0x008, NM, 0);                                                                            \
+            if (NG) __builtin_amdgcn_sched_group_barrier(0x020, NG, 0);                                                                    \
+            if (NDS) __builtin_amdgcn_sched_group_barrier(0x100, NDS, 0);                                                                  \
+        }                                                                                                                                  \
+    } while (0)
+    // one K step on stage (CA, CB); (NA1, NB) is the stage of step S+1, NA2 the A stage of step S+2
+#define STEP(CA, CB, NA1, NB, NA2, S)                                                                                                      \
+    do {                                                                                                                                   \
+        /* slice 0: B of step S+1, one load per two MFMAs */                                                                               \
+        RING_LOAD_B(NB, (S) + 1, 0, LB);                                                                                                   \
+        if constexpr (NS == 2) {                                                                                                           \
+            RING_LOAD_A(NA2, (S) + 2, 0, LA);                                                                                              \
+        }                                                                                                                                  \
+        LOAD_FRAGS(1, CA, CB, 1);                                                                                                          \
+        MFMA_ROWS(0, 0, WTM);                                                                                                              \
+        if constexpr (NS == 2) {                                                                                                           \
+            INTERLEAVE(16, 1, 1, ND / 16);                                                                                                 \
+        } else {                                                                                                                           \
+            INTERLEAVE(8, 2, 1, ND / 8);                                                                                                   \
+        }                                                                                                                                  \
+        __builtin_amdgcn_sched_barrier(0);                                                                                                 \
+        if constexpr (NS == 4) {                                                                                                           \
+            RING_LOAD_A(NA2, (S) + 2, 0, LA / 2);                                                                                          \
+            LOAD_FRAGS(0, CA, CB, 2);                                                                                                      \
+            MFMA_ROWS(1, 0, WTM);                                                                                                          \
+            INTERLEAVE(4, 4, 1, ND / 4);                                                                                                   \
+            __builtin_amdgcn_sched_barrier(0);                                                                                             \
+            RING_LOAD_A(NA2, (S) + 2, LA / 2, LA);                                                                                         \
+            LOAD_FRAGS(1, CA, CB, 3);                                                                                                      \
+            MFMA_ROWS(0, 0, WTM);                                                                                                          \
+            INTERLEAVE(4, 4, 1, ND / 4);                                                                                                   \
+            __builtin_amdgcn_sched_barrier(0);                                                                                             \
+            MFMA_ROWS(1, 0, WTM / 2);                                                                                                      \
+        } else {                                                                                                                           \
+            MFMA_ROWS(1, 0, WTM / 2);                                                                                                      \
+        }                                                                                                                                  \
+        __builtin_amdgcn_sched_barrier(0);                                                                                                 \
+        __builtin_amdgcn_s_waitcnt(0x0F70 | LA); /* vmcnt(LA): everything but A of step S+2 has landed */                                  \
+        __syncthreads();                                                                                                                   \
+        LOAD_FRAGS(0, NA1, NB, 0);                                                                                                         \
+        __builtin_amdgcn_sched_barrier(0);                                                                                                 \
+        MFMA_ROWS(1, WTM / 2, WTM);                                                                                                        \
+    } while (0)
+
+    static_assert(LA == 8 && LB == 8, "vmcnt immediate below assumes eight loads per operand stage");
+    if (kSteps > 0) {
+        RING_LOAD_A(sA0, 0, 0, LA);
+        RING_LOAD_B(sB0, 0, 0, LB);
+        RING_LOAD_A(sA1, 1, 0, LA);
+        __builtin_amdgcn_s_waitcnt(0x0F70 | LA);
+        __syncthreads();
+        LOAD_FRAGS(0, sA0, sB0, 0);
+        int s = 0;
+        for (; s + 6 <= kSteps; s += 6) {
+            STEP(sA0, sB0, sA1, sB1, sA2, s);
+            STEP(sA1, sB1, sA2, sB0, sA0, s + 1);
+            STEP(sA2, sB0, sA0, sB1, sA1, s + 2);
+            STEP(sA0, sB1, sA1, sB0, sA2, s + 3);
+            STEP(sA1, sB0, sA2, sB1, sA0, s + 4);
+            STEP(sA2, sB1, sA0, sB0, sA1, s + 5);
+        }
+        // up to five steps left: the stages continue in the same rotation
+        const int rem = kSteps - s;
+        // (separate conditionals, not nested ones: every join then has two predecessors and the accumulators stay in place)
+        if (rem > 0) {
+            STEP(sA0, sB0, sA1, sB1, sA2, s);
+        }
+        if (rem > 1) {
+            STEP(sA1, sB1, sA2, sB0, sA0, s + 1);
+        }
+        if (rem > 2) {
+            STEP(sA2, sB0, sA0, sB1, sA1, s + 2);
+        }
+        if (rem > 3) {
+            STEP(sA0, sB1, sA1, sB0, sA2, s + 3);
+        }
+        if (rem > 4) {
+            STEP(sA1, sB0, sA2, sB1, sA0, s + 4);
+        }
+    }
+#undef STEP
+#undef INTERLEAVE
+#undef LOAD_FRAGS
+#undef MFMA_ROWS
+#undef RING_LOAD_A
+#undef RING_LOAD_B
+#undef RING_LOAD
+    __builtin_amdgcn_s_waitcnt(0x0F70); // the redundant loads of the last steps
+    __syncthreads();
+    Epilogue<TYPE, WTM, WTN, CT, EPI, false>(p, acc, facc, sA0, rowBase, colBase, wm, wn, half, l32);
+}
+
 template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT> int Launch(const GemmP &p, hipStream_t stream)
 {
     constexpr int BM = 64 * WTM, BN = 64 * WTN;
@@ -860,6 +1070,13 @@ template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT> int Launch(const
     int nb = q.tilesM * q.tilesN * (p.splitK > 1 ? p.splitK : 1);
     if (p.direct && p.splitK <= 1) {
         int gy = p.groupOffsets ? p.splitK_groups : (p.splits > 1 ? p.splits : 1);
+        if constexpr (WTM == 4 && WTN == 4 && !KT) {
+            if (!p.tileGroup && !p.noRing) {
+                hipLaunchKernelGGL((GemmNTRing<TYPE, CT, EPI>), dim3(nb, gy), dim3(256), 0, stream, q);
+                TS2_CHECK_LAUNCH();
+                return TS2_OK;
+            }
+        }
         hipLaunchKernelGGL((GemmNTDirect<TYPE, WTM, WTN, CT, EPI, KT>), dim3(nb, gy), dim3(256), 0, stream, q);
         TS2_CHECK_LAUNCH();
         return TS2_OK;
@@ -1052,6 +1269,7 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
         p.splitK = 1;
     }
     p.direct = (a->tileConfig & 4) ? 0 : 1; // bit 2 of tileConfig selects the register-staged loader (kept for comparison)
+    p.noRing = (a->tileConfig & 16) ? 1 : 0; // bit 4: two-stage loop instead of the ring for the 256x256 tile (comparison)
     if ((a->tileGroup || a->groupOffsets) && splitK > 1) {
         return TS2_ERR_UNSUPPORTED;
     }
