@@ -46,6 +46,7 @@ struct GemmP {
     int splitK_groups;       // number of groups when groupOffsets is set
     int direct;              // 1: direct global->LDS loader
     int noRing;              // 1: keep the two-stage loop for the 256x256 tile (comparison)
+    int mapGroup;            // M tiles per group of the tile order (an XCD's share of the tiles should be about square)
     int splits;              // >1 with splitSlab: blockIdx.y = slice of the contraction, partial product stored to c + y * splitSlab
     int64_t splitSlab;       // bytes
     // row-tile normalise / rope epilogue (C_BF16NORM)
@@ -73,13 +74,12 @@ __device__ __forceinline__ int SwizzleOffset(int row, int chunk)
 }
 
 // tile id -> (tileM, tileN): XCD-aware, then grouped along M
-__device__ __forceinline__ void MapTile(int bid, int nb, int tilesM, int tilesN, int *tm, int *tn)
+__device__ __forceinline__ void MapTile(int bid, int nb, int tilesM, int tilesN, int *tm, int *tn, int GROUP = 8)
 {
     int id = bid;
     if ((nb & 7) == 0) {
         id = (bid & 7) * (nb >> 3) + (bid >> 3);
     }
-    constexpr int GROUP = 8;
     int perGroup = GROUP * tilesN;
     int g = id / perGroup;
     int first = g * GROUP;
@@ -427,7 +427,7 @@ __global__ void __launch_bounds__(256, 1) GemmNT(GemmP p)
         split = bid / tilesMN;
         bid -= split * tilesMN;
     }
-    MapTile(bid, tilesMN, p.tilesM, p.tilesN, &tm, &tn);
+    MapTile(bid, tilesMN, p.tilesM, p.tilesN, &tm, &tn, p.mapGroup ? p.mapGroup : 8);
     const int rowBase = tm * BM;
     const int colBase = tn * BN;
 
@@ -665,7 +665,7 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN) / 4) GemmNTDirect(Gemm
     int tm, tn;
     const int tilesMN = p.tilesM * p.tilesN;
     int bid = blockIdx.x;
-    MapTile(bid, tilesMN, p.tilesM, p.tilesN, &tm, &tn);
+    MapTile(bid, tilesMN, p.tilesM, p.tilesN, &tm, &tn, p.mapGroup ? p.mapGroup : 8);
     const int rowBase = tm * BM;
     const int colBase = tn * BN;
     int kSteps = p.kBytes / BKB;
@@ -867,7 +867,7 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(256, 1) G
     const int wm = wave / WN;
     const int wn = wave % WN;
     int tm, tn;
-    MapTile(blockIdx.x, p.tilesM * p.tilesN, p.tilesM, p.tilesN, &tm, &tn);
+    MapTile(blockIdx.x, p.tilesM * p.tilesN, p.tilesM, p.tilesN, &tm, &tn, p.mapGroup ? p.mapGroup : 8);
     const int rowBase = tm * BM;
     const int colBase = tn * BN;
     int kSteps = p.kBytes / BKB;
@@ -1070,6 +1070,11 @@ template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT> int Launch(const
     int nb = q.tilesM * q.tilesN * (p.splitK > 1 ? p.splitK : 1);
     if (p.direct && p.splitK <= 1) {
         int gy = p.groupOffsets ? p.splitK_groups : (p.splits > 1 ? p.splits : 1);
+        // an XCD runs nb/8 consecutive tiles: group the order so that they cover about as many rows of A as of B
+        {
+            int chunk = (nb % 8) == 0 ? nb / 8 : nb;
+            q.mapGroup = p.mapGroup ? p.mapGroup : chunk >= 64 ? 8 : chunk >= 8 ? 4 : 2;
+        }
         if constexpr (WTM == 4 && WTN == 4 && !KT) {
             if (!p.tileGroup && !p.noRing) {
                 hipLaunchKernelGGL((GemmNTRing<TYPE, CT, EPI>), dim3(nb, gy), dim3(256), 0, stream, q);
@@ -1269,6 +1274,7 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
         p.splitK = 1;
     }
     p.direct = (a->tileConfig & 4) ? 0 : 1; // bit 2 of tileConfig selects the register-staged loader (kept for comparison)
+    p.mapGroup = ((a->tileConfig >> 5) & 3) == 1 ? 8 : ((a->tileConfig >> 5) & 3) == 2 ? 4 : ((a->tileConfig >> 5) & 3) == 3 ? 2 : 0;
     p.noRing = (a->tileConfig & 16) ? 1 : 0; // bit 4: two-stage loop instead of the ring for the 256x256 tile (comparison)
     if ((a->tileGroup || a->groupOffsets) && splitK > 1) {
         return TS2_ERR_UNSUPPORTED;
