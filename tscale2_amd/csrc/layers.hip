@@ -133,6 +133,8 @@ struct ts2_model {
     Arr logits, gradV, gradVT, fnT, wfT;
     // linear backward scratch
     uint8_t *sGrad8 = 0, *sGradT = 0, *sSrcT = 0, *sWT = 0;
+    float *sPartial = 0;                     // fp32 slices of a delta product with few output tiles
+    size_t sPartialFloats = 0;
     float *sRowScale = 0, *sTileMax = 0, *sTileScale = 0;
     int maxW = 0, RP = 0; // RP = rows of the row-indexed scratch (max(R, lenMoe))
 
@@ -224,10 +226,34 @@ int BackpropDX(ts2_model *M, TMatrix &W, const Arr &gradFast, float alpha, bool 
         srcGrad.type, add, s);
 }
 
+// slices of the token axis for a delta product [dstDim x srcDim]: enough to give every CU a 256x256 tile, each slice a whole number of
+// k-tiles and at least 4096 tokens long
+int DeltaSplits(ts2_model *M, int srcDim, int dstDim)
+{
+    if (M->mode != TS2_E4M3 || (srcDim % 256) || (dstDim % 256)) {
+        return 1;
+    }
+    int tiles = (srcDim / 256) * (dstDim / 256);
+    if (tiles >= 192) {
+        return 1;
+    }
+    int splits = 1;
+    while (splits < 8 && tiles * splits < 192 && M->R % (splits * 2 * 128) == 0 && M->R / (splits * 2) >= 4096) {
+        splits *= 2;
+    }
+    return splits;
+}
+
 // delta = alpha * gradScale * gradFast^T * src8   (TMatMulBuffers::BackpropDelta)
 int BackpropDelta(ts2_model *M, TMatrix &W, const Arr &src8, const Arr &gradFast, float alpha, const float *gradScale, void *s)
 {
     ts2_matmul_bwd_buffers b = Scratch(M, M->R, W.srcDim, W.dstDim);
+    // a delta with fewer large tiles than the chip has CUs runs as slices of the token axis on the large tile, packed afterwards
+    int splits = DeltaSplits(M, W.srcDim, W.dstDim);
+    if (splits > 1 && (size_t)splits * W.dstDim * W.srcDim <= M->sPartialFloats) {
+        b.partial = Flat(M->sPartial, splits * W.dstDim, W.srcDim, TS2_F32).m;
+        b.splits = splits;
+    }
     return ts2_matmul_backprop_delta(M->mode, M->len, M->R, W.srcDim, W.dstDim, src8.P(), nullptr, gradFast.P(), gradFast.type, alpha, gradScale,
         M->kTile, &b, W.delta.P(), W.deltaTileScale.P(), s);
 }
@@ -781,6 +807,8 @@ extern "C" ts2_model *ts2_model_create(const ts2_model_config *cfg)
     M->sGradT = (uint8_t *)M->Dev((size_t)RP * maxW);
     M->sSrcT = (uint8_t *)M->Dev((size_t)RP * maxW);
     M->sWT = (uint8_t *)M->Dev((size_t)maxW * maxW);
+    M->sPartialFloats = (size_t)8 * 2048 * 2048; // eight slices of a 2048 x 2048 delta, four of a 4096 x 2048 one
+    M->sPartial = (float *)M->Dev(M->sPartialFloats * 4);
     M->sRowScale = (float *)M->Dev((size_t)RP * 4);
     M->sTileMax = (float *)M->Dev((size_t)(RP / 128 + 1) * 4);
     M->sTileScale = (float *)M->Dev((size_t)(RP / 128 + 1) * 4);
@@ -802,7 +830,7 @@ extern "C" ts2_model *ts2_model_create(const ts2_model_config *cfg)
     }
     ok &= M->Alloc(&M->logits, R, V, TS2_F32) && M->Alloc(&M->gradV, R, V, TS2_BF16) && M->Alloc(&M->gradVT, V, R, TS2_BF16) &&
           M->Alloc(&M->fnT, D, R, TS2_BF16) && M->Alloc(&M->wfT, D, V, TS2_BF16);
-    if (!ok || !M->sGrad8 || !M->sGradT || !M->sSrcT || !M->sWT) {
+    if (!ok || !M->sGrad8 || !M->sGradT || !M->sSrcT || !M->sWT || !M->sPartial) {
         delete M;
         return nullptr;
     }
