@@ -316,6 +316,60 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
             }
         }
     } else {
+        if constexpr (EPI == TS2_EPI_ADD && (CT == C_F32 || CT == C_BF16)) {
+            if (p.splitK <= 1) {
+                // C += product: the old values of eight rows (two e-quads) across the wave's width are one batch of loads, and the
+                // batch after the one being added and stored is already in flight, so the read latency of C is paid once per tile
+                constexpr int NCH = WTM * 2;
+                float old[2][8][WTN];
+                auto rowOf = [&](int ch, int r) { return rowBase + rowLocal(ch >> 1, (ch & 1) * 8 + r); };
+                auto fetch = [&](int ch, float (&o)[8][WTN]) {
+#pragma unroll
+                    for (int r = 0; r < 8; ++r) {
+                        const int row = rowOf(ch, r);
+                        const uint8_t *src = p.c + (int64_t)row * p.ldc;
+#pragma unroll
+                        for (int j = 0; j < WTN; ++j) {
+                            const int col = colBase + wn * (32 * WTN) + j * 32 + l32;
+                            if (CT == C_F32) {
+                                o[r][j] = row < mLive ? ((const float *)src)[col] : 0.f;
+                            } else {
+                                o[r][j] = row < mLive ? Bf16ToFloat(((const bf16_t *)src)[col]) : 0.f;
+                            }
+                        }
+                    }
+                };
+                fetch(0, old[0]);
+#pragma unroll
+                for (int ch = 0; ch < NCH; ++ch) {
+                    if (ch + 1 < NCH) {
+                        fetch(ch + 1, old[(ch + 1) & 1]);
+                    }
+#pragma unroll
+                    for (int r = 0; r < 8; ++r) {
+                        const int row = rowOf(ch, r);
+                        if (row < mLive) {
+                            uint8_t *dst = p.c + (int64_t)row * p.ldc;
+                            float rs = scale;
+                            if (p.rowScale) {
+                                rs *= p.rowScale[row];
+                            }
+#pragma unroll
+                            for (int j = 0; j < WTN; ++j) {
+                                const int col = colBase + wn * (32 * WTN) + j * 32 + l32;
+                                float v = old[ch & 1][r][j] + accVal(ch >> 1, j, (ch & 1) * 8 + r) * rs;
+                                if constexpr (CT == C_F32) {
+                                    ((float *)dst)[col] = v;
+                                } else {
+                                    ((bf16_t *)dst)[col] = FloatToBf16(v);
+                                }
+                            }
+                        }
+                    }
+                }
+                return;
+            }
+        }
         // four consecutive rows (one e-quad) across the wave's whole width at a time: a row's WTN 128-byte segments are written back
         // to back, and for the accumulate epilogues the 4 x WTN old values are all fetched before the first store
 #pragma unroll
