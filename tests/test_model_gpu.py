@@ -93,6 +93,15 @@ def test_tiny_dense_fp8_step():
     check_model(h, tol_state=5e-2, tol_grad=1.5e-1, tol_delta=2e-1)
 
 
+def test_vocabulary_padded_to_the_large_tile_fp8_step():
+    """A vocabulary of 4224 = 33 x 128 entries: the driver pads the final matrix to 4352 zero-filled rows so that the logits, the
+    state-gradient and the delta products of the final layer run on 256x256 tiles; loss, gradient and the 4224 delta rows must agree
+    with the oracle like in the unpadded case."""
+    print("case padded vocabulary fp8", flush=True)
+    h = Harness(E4M3, dim=256, heads=2, ffn_tiles=4, depth=1, vocab=4224, frag_count=4, frag_len=64, wide_window=64, seed=6)
+    check_model(h, tol_state=5e-2, tol_grad=1.5e-1, tol_delta=2e-1)
+
+
 def test_moe_layer_fp8_step():
     """attention + MoE (8 experts, top-2, expert width 128): exercises routing, grouping, grouped GEMMs, combine and routing backward"""
     print("case moe fp8", flush=True)

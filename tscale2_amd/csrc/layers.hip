@@ -97,6 +97,8 @@ struct ts2_model {
     std::vector<void *> allocs;
     int mode = TS2_I8, fastGradType = TS2_BF16;
     int R = 0; // lenRound capacity
+    int VP = 0; // vocabulary rows of the final matrix and columns of the logits as allocated: a large vocabulary is padded with zero
+                // rows to a multiple of 256 so that its three products run on the 256x256 tile
     int len = 0;
     int lenMoe = 0;
     int kTile = 512;
@@ -598,12 +600,13 @@ int FinalLogits(ts2_model *M, void *s)
 
 int FinalBackward(ts2_model *M, void *s)
 {
-    int D = M->cfg.dim, V = M->cfg.vocab, depth = (int)M->layers.size(), R = M->R;
+    int D = M->cfg.dim, V = M->cfg.vocab, VP = M->VP, depth = (int)M->layers.size(), R = M->R;
     CK(FinalLogits(M, s));
     CK(Ts2ZeroRows(Flat(M->lossSum, 1, 1, TS2_F32).P(), 1, 4, s));
     CK(Ts2FinalSoftmaxGrad(R, V, M->logits.P(), M->bias, M->target, 1.f, M->gradV.P(), M->lossSum, 0, s));
     // dfn = grad * Wf / sqrt(D): bf16 product, the 8-bit weights converted exactly
-    CK(Ts2TransposeToBf16(V, V, D, M->finalW.fast.P(), M->mode, M->wfT.P(), s));
+    // (columns V..VP of the logits are products with zero rows, the same columns of the gradient stay zero: the softmax pass covers V)
+    CK(Ts2TransposeToBf16(VP, VP, D, M->finalW.fast.P(), M->mode, M->wfT.P(), s));
     ts2_gemm_args g = {};
     g.a = M->gradV.m;
     g.b = M->wfT.m;
@@ -612,7 +615,7 @@ int FinalBackward(ts2_model *M, void *s)
     g.cType = TS2_F32;
     g.m = R;
     g.n = D;
-    g.k = V;
+    g.k = VP;
     g.mLive = M->len;
     g.alpha = DISCR * Dot(D);
     g.alphaPtr = M->finalW.scale;
@@ -620,7 +623,7 @@ int FinalBackward(ts2_model *M, void *s)
     g.splitK = 1;
     CK(ts2_gemm_nt(&g, s));
     // delta_final[v][d] = sum_t grad[t][v] * fn[t][d]
-    CK(Ts2TransposeToBf16(M->len, R, V, M->gradV.P(), TS2_BF16, M->gradVT.P(), s));
+    CK(Ts2TransposeToBf16(M->len, R, VP, M->gradV.P(), TS2_BF16, M->gradVT.P(), s));
     CK(Ts2TransposeToBf16(M->len, R, D, M->normState[depth].P(), M->mode, M->fnT.P(), s));
     ts2_gemm_args h = {};
     h.a = M->gradVT.m;
@@ -628,7 +631,7 @@ int FinalBackward(ts2_model *M, void *s)
     h.c = M->finalW.delta.m;
     h.abType = TS2_BF16;
     h.cType = TS2_I8;
-    h.m = V;
+    h.m = VP;
     h.n = D;
     h.k = R;
     h.alpha = VEC;
@@ -704,7 +707,9 @@ extern "C" ts2_model *ts2_model_create(const ts2_model_config *cfg)
     bool ok = true;
     ok &= InitMatrix(M, &M->embed, D, cfg->labelCount, 1) == 0; // delta storage reused as fp32 [labelCount][D]: allocate separately below
     ok &= M->Alloc(&M->embed.delta, cfg->labelCount, D, TS2_F32);
-    ok &= InitMatrix(M, &M->finalW, D, V, 1) == 0;
+    M->VP = (V >= 4096 && V % 256) ? RoundUp(V, 256) : V;
+    const int VP = M->VP;
+    ok &= InitMatrix(M, &M->finalW, D, VP, 1) == 0;
     M->bias = (float *)M->Dev((size_t)V * 4);
     M->layers.resize(cfg->depth);
     for (int d = 0; d < cfg->depth && ok; ++d) {
@@ -828,8 +833,8 @@ extern "C" ts2_model *ts2_model_create(const ts2_model_config *cfg)
         int wtRows = E * (X > D ? X : D), wtCols = X > D ? X : D;
         ok &= M->Alloc(&M->wT, wtRows, wtCols, M->mode);
     }
-    ok &= M->Alloc(&M->logits, R, V, TS2_F32) && M->Alloc(&M->gradV, R, V, TS2_BF16) && M->Alloc(&M->gradVT, V, R, TS2_BF16) &&
-          M->Alloc(&M->fnT, D, R, TS2_BF16) && M->Alloc(&M->wfT, D, V, TS2_BF16);
+    ok &= M->Alloc(&M->logits, R, VP, TS2_F32) && M->Alloc(&M->gradV, R, VP, TS2_BF16) && M->Alloc(&M->gradVT, VP, R, TS2_BF16) &&
+          M->Alloc(&M->fnT, D, R, TS2_BF16) && M->Alloc(&M->wfT, D, VP, TS2_BF16);
     if (!ok || !M->sGrad8 || !M->sGradT || !M->sSrcT || !M->sWT || !M->sPartial) {
         delete M;
         return nullptr;
