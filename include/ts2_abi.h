@@ -216,6 +216,9 @@ typedef struct ts2_matmul_bwd_buffers {
      * scanning the gradient again when gradRowAbsMaxValid != 0: the caller sets that when both calls get the same gradient tensor. */
     float *gradRowAbsMax;
     int32_t gradRowAbsMaxValid;
+    /* != 0: srcT already holds the transpose of the `src` given to BackpropDelta (an earlier BackpropDelta call with the same buffers
+     * and the same source tensor left it there, as for the matrices of one layer that share their input); the transpose is skipped. */
+    int32_t srcTValid;
 } ts2_matmul_bwd_buffers;
 
 /* BackpropMulti (prep of dX): I8: quantise grad (TS2_BF16 | TS2_F32, optionally times gradColScale[gradDim]) per row to

@@ -247,9 +247,11 @@ int DeltaSplits(ts2_model *M, int srcDim, int dstDim)
 }
 
 // delta = alpha * gradScale * gradFast^T * src8   (TMatMulBuffers::BackpropDelta)
-int BackpropDelta(ts2_model *M, TMatrix &W, const Arr &src8, const Arr &gradFast, float alpha, const float *gradScale, void *s)
+int BackpropDelta(ts2_model *M, TMatrix &W, const Arr &src8, const Arr &gradFast, float alpha, const float *gradScale, void *s,
+    bool sameSrcAsLastCall = false)
 {
     ts2_matmul_bwd_buffers b = Scratch(M, M->R, W.srcDim, W.dstDim);
+    b.srcTValid = sameSrcAsLastCall; // the matrices of a layer that share their input transpose it once
     // a delta with fewer large tiles than the chip has CUs runs as slices of the token axis on the large tile, packed afterwards
     int splits = DeltaSplits(M, W.srcDim, W.dstDim);
     if (splits > 1 && (size_t)splits * W.dstDim * W.srcDim <= M->sPartialFloats) {
@@ -301,7 +303,7 @@ int FfnBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
     // deltas (sources are stored in 1/24 units)
     CK(BackpropDelta(M, L.w[2], rg8, M->stateGradFast, VEC, gradScale, s));
     CK(BackpropDelta(M, L.w[0], norm8, dwide, VEC, gradScale, s));
-    return BackpropDelta(M, L.w[1], norm8, dgate, VEC, gradScale, s);
+    return BackpropDelta(M, L.w[1], norm8, dgate, VEC, gradScale, s, true);
 }
 
 // ---------------------------------------------------------------------------------------------------------------------------
@@ -399,9 +401,9 @@ int AttBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
     CK(BackpropDX(M, L.w[2], dVf, a, true, M->dNormState, true, s));
     CK(BackpropDX(M, L.w[3], dGate, a, false, M->dNormState, true, s));
     CK(BackpropDelta(M, L.w[0], norm8, dQf, VEC, gradScale, s));
-    CK(BackpropDelta(M, L.w[1], norm8, dKf, VEC, gradScale, s));
-    CK(BackpropDelta(M, L.w[2], norm8, dVf, VEC, gradScale, s));
-    return BackpropDelta(M, L.w[3], norm8, dGate, VEC, gradScale, s);
+    CK(BackpropDelta(M, L.w[1], norm8, dKf, VEC, gradScale, s, true));
+    CK(BackpropDelta(M, L.w[2], norm8, dVf, VEC, gradScale, s, true));
+    return BackpropDelta(M, L.w[3], norm8, dGate, VEC, gradScale, s, true);
 }
 
 // ---------------------------------------------------------------------------------------------------------------------------

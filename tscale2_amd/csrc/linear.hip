@@ -108,9 +108,11 @@ extern "C" int ts2_matmul_backprop_delta(int32_t mode, int32_t len, int32_t lenR
             return rc;
         }
     }
-    rc = ts2_transpose_quant(len, lenRound, src, mode, nullptr, nullptr, 0, nullptr, &buf->srcT, mode, nullptr, stream);
-    if (rc) {
-        return rc;
+    if (!buf->srcTValid) {
+        rc = ts2_transpose_quant(len, lenRound, src, mode, nullptr, nullptr, 0, nullptr, &buf->srcT, mode, nullptr, stream);
+        if (rc) {
+            return rc;
+        }
     }
     g.a = buf->gradT;
     g.b = buf->srcT;
