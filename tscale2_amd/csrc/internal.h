@@ -10,3 +10,4 @@ int Ts2FinalSoftmaxGrad(int rows, int vocab, const ts2_mat *logits, const float 
     float *lossSum, int keepProb, void *stream);
 int Ts2TransposeToBf16(int rows, int rowsRound, int cols, const ts2_mat *src, int srcType, const ts2_mat *dst, void *stream);
 int Ts2ZeroRows(const ts2_mat *m, int rows, int rowBytes, void *stream);
+int Ts2FillFloats(float *p, int n, float v, void *stream);

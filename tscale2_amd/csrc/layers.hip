@@ -651,6 +651,7 @@ int ModelBackprop(ts2_model *M, void *s)
     int D = M->cfg.dim, depth = (int)M->layers.size();
     CK(ModelForward(M, s));
     CK(Ts2ZeroRows(Flat(M->gradMaxNorm, 1, depth + 2, TS2_F32).P(), 1, (depth + 2) * 4, s));
+    CK(Ts2FillFloats(M->gradMult, 1, 1.f, s)); // the multiplier the final normalisation applies to the fast gradient
     CK(FinalBackward(M, s));
     M->useKept = M->keep;
     struct TReset {
@@ -661,8 +662,9 @@ int ModelBackprop(ts2_model *M, void *s)
     for (int d = depth - 1; d >= 0; --d, ++stepId) {
         float *prevMax = M->gradMaxNorm + stepId, *nextMax = M->gradMaxNorm + stepId + 1;
         float *gradScale = M->gradScale + stepId + 1, *gradMult = M->gradMult + stepId + 1;
-        // the fast gradient is rewritten unconditionally: its multiplier history does not survive between steps here
-        CK(ts2_scale_grad(prevMax, nullptr, M->stateGrad.P(), M->stateGradFast.P(), M->fastGradType, M->len, gradScale, gradMult, s));
+        // the fast gradient is rewritten only when its power-of-two multiplier differs from the one its producer applied (the final
+        // normalisation: 1, kept in gradMult[0]; a layer's normalisation backward: that layer's multiplier)
+        CK(ts2_scale_grad(prevMax, M->gradMult + stepId, M->stateGrad.P(), M->stateGradFast.P(), M->fastGradType, M->len, gradScale, gradMult, s));
         CK(LayerBackward(M, d, gradScale, s));
         CK(ts2_backprop_layer_normalize(M->normState[d].P(), M->mode, M->stateScale[d].P(), M->dNormState.P(), nullptr, gradScale, gradMult,
             M->stateGrad.P(), M->stateGradFast.P(), M->fastGradType, nextMax, M->len, s));

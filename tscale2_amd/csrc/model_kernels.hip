@@ -276,6 +276,21 @@ int Ts2TransposeToBf16(int rows, int rowsRound, int cols, const ts2_mat *src, in
     return TS2_OK;
 }
 
+__global__ void FillFloatsKernel(float *p, int n, float v)
+{
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        p[i] = v;
+    }
+}
+
+int Ts2FillFloats(float *p, int n, float v, void *stream)
+{
+    hipLaunchKernelGGL(FillFloatsKernel, dim3((n + 255) / 256), dim3(256), 0, STREAM, p, n, v);
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
 int Ts2ZeroRows(const ts2_mat *m, int rows, int rowBytes, void *stream)
 {
     hipLaunchKernelGGL(ZeroBytes, dim3(rows), dim3(256), 0, STREAM, (uint8_t *)m->ptr, m->strideBytes, rowBytes);
