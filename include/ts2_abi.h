@@ -105,6 +105,19 @@ typedef struct ts2_gemm_args {
     int32_t normalize;
     float vecScale;
     ts2_mat rope;
+    /* extraSegments > 0 (at most 3): C (+)= sum over the 1 + extraSegments products alpha_i * (*alphaPtr_i) * A_i * B_i^T with the same
+     * m, n, k, operand type and operand strides; a, b, alpha, alphaPtr above describe product 0, segment[i-1] product i.  One launch
+     * and one pass over C instead of one read-modify-write of C per product: the gradient of a layer input that feeds several
+     * matrices (Backprop of Q, K, V and gate in src/gpt/compute/layer_att.cu:236-260 adds four products into the same array).
+     * 256x256-tile kernel only (m, n multiples of 256), TS2_E4M3 or TS2_BF16 operands, fp32 or bf16 C, TS2_EPI_STORE or TS2_EPI_ADD,
+     * no rowScale, kTileScale, groups or splitK; the fp32 sums of the products are rescaled in registers between products. */
+    int32_t extraSegments;
+    struct {
+        const void *a;
+        const void *b;
+        float alpha;
+        const float *alphaPtr;
+    } segment[3];
 } ts2_gemm_args;
 
 int ts2_gemm_nt(const ts2_gemm_args *args, void *stream);
@@ -231,6 +244,15 @@ int ts2_matmul_backprop_multi(int32_t mode, int32_t len, int32_t lenRound, int32
 int ts2_matmul_backprop(int32_t mode, int32_t len, int32_t lenRound, int32_t srcDim, int32_t gradDim, const ts2_mat *grad,
     const ts2_matmul_bwd_buffers *buf, float alpha, const float *alphaPtr, const ts2_mat *srcGrad, int32_t srcGradType, int32_t add,
     void *stream);
+
+/* Backprop() of `count` (2..4) matrices that share their input (Q, K, V and gate of an attention layer,
+ * src/gpt/compute/layer_att.cu:236-260; wide and gate of an FFN layer, layer_ffn.cu): srcGrad (+)= sum_i alpha[i] * (*alphaPtr[i]) *
+ * grad[i] * W_i, where the reference adds one product after the other into the same array.  Every bufs[i] must have been prepared by
+ * ts2_matmul_backprop_multi for its matrix; all matrices are [gradDim][srcDim].  TS2_E4M3 with srcDim and lenRound multiples of 256
+ * runs as one launch (one pass over srcGrad); otherwise the products are launched one after the other as the reference does. */
+int ts2_matmul_backprop_group(int32_t mode, int32_t len, int32_t lenRound, int32_t srcDim, int32_t gradDim, int32_t count,
+    const ts2_mat *const *grad, const ts2_matmul_bwd_buffers *const *bufs, const float *alpha, const float *const *alphaPtr,
+    const ts2_mat *srcGrad, int32_t srcGradType, int32_t add, void *stream);
 
 /* BackpropDelta: delta[gradDim][srcDim] = alpha * (*gradScale) * sum_t grad[t][k]*src[t][x] as the packed delta (i8 + tileScale
  * [srcDim/128][gradDim], TCudaPackedDeltaMatrix, src/gpt/matrix/delta_cuda.h:9-38).  src is the 8-bit layer input

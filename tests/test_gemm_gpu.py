@@ -242,3 +242,45 @@ def test_fused_row_tile_normalize_rope_epilogue_matches_the_two_pass_path(ab, no
     # unsupported with 128x128 tiles: the caller falls back to the two-pass path
     assert lib.gemm_nt(a, b, got, t, L.BF16, tile_config=2, epilogue=L.EPI_ROW_TILE_NORM, normalize=True, vec_scale=1.0, tile_scale=got_sc,
                        check=False) == -3
+
+
+@pytest.mark.parametrize("ab,add", [("e4m3", False), ("e4m3", True), ("bf16", True)])
+def test_several_products_into_one_result(ab, add):
+    """extraSegments: C (+)= sum_i alpha_i * s_i * A_i B_i^T in one launch against the same products launched one after the other
+    (store, then accumulate).  The sums are the same fp32 MFMA sums; the one-launch form rescales them in registers between products
+    and rounds the total once, so the results agree to a few fp32 ulps of the largest partial sum."""
+    print("case several products", ab, add, flush=True)
+    from tscale2_amd import lib as L
+    lib = L.load()
+    m, n, k, nseg = 512, 768, 384, 4
+    g = torch.Generator(device="cuda").manual_seed(11)
+    As, Bs, alphas, ptrs = [], [], [], []
+    for i in range(nseg):
+        if ab == "e4m3":
+            a = (torch.randn((m, k), device="cuda", generator=g) * 6).to(torch.float8_e4m3fn).view(torch.uint8)
+            b = (torch.randn((n, k), device="cuda", generator=g) * 6).to(torch.float8_e4m3fn).view(torch.uint8)
+            t = L.E4M3
+        else:
+            a = torch.randn((m, k), device="cuda", generator=g).bfloat16().view(torch.int16)
+            b = torch.randn((n, k), device="cuda", generator=g).bfloat16().view(torch.int16)
+            t = L.BF16
+        As.append(a); Bs.append(b)
+        alphas.append(0.25 * (i + 1))
+        ptrs.append(None if i == 2 else torch.full((1,), 0.5 + 0.37 * i, device="cuda"))
+    c0 = torch.randn((m, n), device="cuda", generator=g)
+    want = c0.clone() if add else torch.empty_like(c0)
+    for i in range(nseg):
+        lib.gemm_nt(As[i], Bs[i], want, t, L.F32, alpha=alphas[i], alpha_ptr=ptrs[i], tile_config=1,
+                    epilogue=L.EPI_ADD if (add or i > 0) else L.EPI_STORE, m_live=500)
+    got = c0.clone() if add else torch.full_like(c0, 3.0)
+    lib.gemm_nt(As[0], Bs[0], got, t, L.F32, alpha=alphas[0], alpha_ptr=ptrs[0], epilogue=L.EPI_ADD if add else L.EPI_STORE, m_live=500,
+                segments=[(As[i], Bs[i], alphas[i], ptrs[i]) for i in range(1, nseg)])
+    torch.cuda.synchronize()
+    scale = want[:500].abs().max().item()
+    assert (got[:500] - want[:500]).abs().max().item() <= 4e-6 * scale
+    if not add:
+        assert (got[500:] == 0).all()
+    # not available off the 256x256 tile or for int8 operands
+    a8 = torch.zeros((m, k), dtype=torch.int8, device="cuda"); b8 = torch.zeros((n, k), dtype=torch.int8, device="cuda")
+    assert lib.gemm_nt(a8, b8, got, L.I8, L.F32, segments=[(a8, b8, 1.0, None)], check=False) == -3
+    assert lib.gemm_nt(As[0], Bs[0], got, t, L.F32, tile_config=2, segments=[(As[1], Bs[1], 1.0, None)], check=False) == -3

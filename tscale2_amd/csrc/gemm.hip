@@ -54,6 +54,11 @@ struct GemmP {
     float vecScale;
     const float *rope; // [m][128] (cos, sin) pairs, may be null
     int64_t ldRope;    // floats
+    // further products added into the same accumulators (ring kernel): product i+1 = segA[i] * segB[i]^T * segAlpha[i] * *segAlphaPtr[i]
+    int nSeg; // 1 + number of further products
+    const uint8_t *segA[3], *segB[3];
+    float segAlpha[3];
+    const float *segAlphaPtr[3];
 };
 
 enum { T_I8 = 0, T_FP8 = 1, T_BF16 = 2 };
@@ -944,8 +949,10 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(256, 1) G
     }
     const int lrow = wave * 8 + (lane >> 3);
     const int lchunk = (lane & 7) ^ ((lrow >> 1) & 7);
-    const uint8_t *gaTile = p.a + (int64_t)rowBase * p.lda + (int64_t)kBeg * BKB;
-    const uint8_t *gbTile = p.b + (int64_t)colBase * p.ldb + (int64_t)kBeg * BKB;
+    const int64_t aTileOff = (int64_t)rowBase * p.lda + (int64_t)kBeg * BKB;
+    const int64_t bTileOff = (int64_t)colBase * p.ldb + (int64_t)kBeg * BKB;
+    const uint8_t *gaTile = p.a + aTileOff;
+    const uint8_t *gbTile = p.b + bTileOff;
     const uint32_t gaLane = (uint32_t)(lrow * (int)p.lda + lchunk * 16);
     const uint32_t gbLane = (uint32_t)(lrow * (int)p.ldb + lchunk * 16);
     constexpr int LA = BM / (8 * NW);
@@ -1059,6 +1066,14 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(256, 1) G
     } while (0)
 
     static_assert(LA == 8 && LB == 8, "vmcnt immediate below assumes eight loads per operand stage");
+    // several products into the same accumulators: one pass of the pipeline per product (the stage rotation restarts), the fp32 sums
+    // rescaled in between so that the epilogue's single factor, the last product's, is right for all of them
+    for (int seg = 0; seg < p.nSeg; ++seg) {
+    if (seg > 0) {
+        // (constant subscripts only: a variable one would move the whole parameter block to private memory)
+        gaTile = (seg == 1 ? p.segA[0] : seg == 2 ? p.segA[1] : p.segA[2]) + aTileOff;
+        gbTile = (seg == 1 ? p.segB[0] : seg == 2 ? p.segB[1] : p.segB[2]) + bTileOff;
+    }
     if (kSteps > 0) {
         RING_LOAD_A(sA0, 0, 0, LA);
         RING_LOAD_B(sB0, 0, 0, LB);
@@ -1094,6 +1109,40 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(256, 1) G
             STEP(sA1, sB0, sA2, sB1, sA0, s + 4);
         }
     }
+    __builtin_amdgcn_s_waitcnt(0x0F70); // the redundant loads of the last steps
+    __syncthreads();
+    if constexpr (TYPE != T_I8) {
+        if (seg + 1 < p.nSeg) {
+            float cur = seg == 0 ? p.alpha : seg == 1 ? p.segAlpha[0] : p.segAlpha[1];
+            const float *curPtr = seg == 0 ? p.alphaPtr : seg == 1 ? p.segAlphaPtr[0] : p.segAlphaPtr[1];
+            float nxt = seg == 0 ? p.segAlpha[0] : seg == 1 ? p.segAlpha[1] : p.segAlpha[2];
+            const float *nxtPtr = seg == 0 ? p.segAlphaPtr[0] : seg == 1 ? p.segAlphaPtr[1] : p.segAlphaPtr[2];
+            if (curPtr) {
+                cur *= *curPtr;
+            }
+            if (nxtPtr) {
+                nxt *= *nxtPtr;
+            }
+            const float ratio = cur / nxt;
+#pragma unroll
+            for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+                for (int j = 0; j < WTN; ++j) {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        acc[i][j][e] *= ratio;
+                    }
+                }
+            }
+        }
+    }
+    } // products
+    if (p.nSeg > 1) {
+        const float lastAlpha = p.nSeg == 2 ? p.segAlpha[0] : p.nSeg == 3 ? p.segAlpha[1] : p.segAlpha[2];
+        const float *lastPtr = p.nSeg == 2 ? p.segAlphaPtr[0] : p.nSeg == 3 ? p.segAlphaPtr[1] : p.segAlphaPtr[2];
+        p.alpha = lastAlpha;
+        p.alphaPtr = lastPtr;
+    }
 #undef STEP
 #undef INTERLEAVE
 #undef LOAD_FRAGS
@@ -1101,8 +1150,6 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(256, 1) G
 #undef RING_LOAD_A
 #undef RING_LOAD_B
 #undef RING_LOAD
-    __builtin_amdgcn_s_waitcnt(0x0F70); // the redundant loads of the last steps
-    __syncthreads();
     Epilogue<TYPE, WTM, WTN, CT, EPI, false>(p, acc, facc, sA0, rowBase, colBase, wm, wn, half, l32);
 }
 
@@ -1136,9 +1183,15 @@ template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT> int Launch(const
                 return TS2_OK;
             }
         }
+        if (p.nSeg > 1) {
+            return TS2_ERR_UNSUPPORTED; // several products per launch: ring kernel only
+        }
         hipLaunchKernelGGL((GemmNTDirect<TYPE, WTM, WTN, CT, EPI, KT>), dim3(nb, gy), dim3(256), 0, stream, q);
         TS2_CHECK_LAUNCH();
         return TS2_OK;
+    }
+    if (p.nSeg > 1) {
+        return TS2_ERR_UNSUPPORTED;
     }
     hipLaunchKernelGGL(kern, dim3(nb, p.groupOffsets ? p.splitK_groups : 1), dim3(256), ldsBytes, stream, q);
     TS2_CHECK_LAUNCH();
@@ -1222,7 +1275,7 @@ template <int TYPE> int DispatchTile(const ts2_gemm_args *a, const GemmP &p, hip
     if (cfg == 0) {
         // 256x256 tiles only when they still fill the chip; the k-tile-scaled kernel keeps a second accumulator set and needs 128x128
         long tilesL = (long)(p.m / 256) * (p.n / 256) * (p.splitK > 1 ? p.splitK : 1);
-        cfg = tilesL >= 192 ? 1 : 2;
+        cfg = (tilesL >= 192 || p.nSeg > 1) ? 1 : 2;
     }
     // the 256x256 kernel needs full tiles and has no room for the second accumulator set of the k-tile-scaled variant
     if (cfg == 1 && !a->kTileScale && !p.tileGroup && (p.m % 256) == 0 && (p.n % 256) == 0) {
@@ -1311,6 +1364,28 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
             (a->rope.ptr && (a->rope.y < (a->mLive > 0 ? a->mLive : a->m) || a->rope.x < 128 || (a->rope.strideBytes & 7) || ((uintptr_t)a->rope.ptr & 7)))) {
             return TS2_ERR_SHAPE;
         }
+    }
+    p.nSeg = 1;
+    if (a->extraSegments) {
+        const bool bigTile = (a->m % 256) == 0 && (a->n % 256) == 0 && (a->tileConfig & 3) <= 1 && !(a->tileConfig & (4 | 8 | 16));
+        if (a->extraSegments < 0 || a->extraSegments > 3 || !bigTile || a->abType == TS2_I8 || a->rowScale || a->kTileScale || a->tileGroup ||
+            a->groupOffsets || splitK > 1 || (a->cType != TS2_F32 && a->cType != TS2_BF16) ||
+            (a->epilogue != TS2_EPI_STORE && a->epilogue != TS2_EPI_ADD)) {
+            return TS2_ERR_UNSUPPORTED;
+        }
+        for (int i = 0; i < a->extraSegments; ++i) {
+            if (!a->segment[i].a || !a->segment[i].b) {
+                return TS2_ERR_NULL;
+            }
+            if ((((uintptr_t)a->segment[i].a) & 15) || (((uintptr_t)a->segment[i].b) & 15)) {
+                return TS2_ERR_ALIGN;
+            }
+            p.segA[i] = (const uint8_t *)a->segment[i].a;
+            p.segB[i] = (const uint8_t *)a->segment[i].b;
+            p.segAlpha[i] = a->segment[i].alpha;
+            p.segAlphaPtr[i] = a->segment[i].alphaPtr;
+        }
+        p.nSeg = 1 + a->extraSegments;
     }
     p.splits = 1;
     p.splitSlab = 0;

@@ -228,6 +228,42 @@ int BackpropDX(ts2_model *M, TMatrix &W, const Arr &gradFast, float alpha, bool 
         srcGrad.type, add, s);
 }
 
+// srcGrad (+)= sum_i alpha [* scale_i] * grad_i * W_i for the matrices of a layer that share their input: every weight is transposed
+// into its own part of the transpose scratch, then one grouped Backprop
+int BackpropDXGroup(ts2_model *M, int count, TMatrix *const *W, const Arr *const *grad, float alpha, const bool *useScale, const Arr &srcGrad,
+    bool add, void *s)
+{
+    ts2_matmul_bwd_buffers b[4];
+    const ts2_matmul_bwd_buffers *bp[4];
+    const ts2_mat *gp[4];
+    float al[4];
+    const float *ap[4];
+    const int srcDim = W[0]->srcDim, dstDim = W[0]->dstDim;
+    if (M->mode != TS2_E4M3) {
+        // int8: the row-quantised gradient lives in the one shared scratch, so the products go one after the other
+        for (int i = 0; i < count; ++i) {
+            CK(BackpropDX(M, *W[i], *grad[i], alpha, useScale[i], srcGrad, add || i > 0, s));
+        }
+        return 0;
+    }
+    for (int i = 0; i < count; ++i) {
+        if (W[i]->srcDim != srcDim || W[i]->dstDim != dstDim) {
+            return TS2_ERR_SHAPE;
+        }
+        if ((size_t)(i + 1) * srcDim * dstDim > (size_t)4 * M->maxW * M->maxW) {
+            return TS2_ERR_SHAPE;
+        }
+        b[i] = Scratch(M, M->R, srcDim, dstDim);
+        b[i].transformT = Flat(M->sWT + (size_t)i * srcDim * dstDim, srcDim, dstDim, M->mode).m;
+        CK(ts2_matmul_backprop_multi(M->mode, M->len, M->R, srcDim, dstDim, W[i]->fast.P(), grad[i]->P(), grad[i]->type, nullptr, &b[i], s));
+        bp[i] = &b[i];
+        gp[i] = grad[i]->P();
+        al[i] = alpha;
+        ap[i] = useScale[i] ? W[i]->scale : nullptr;
+    }
+    return ts2_matmul_backprop_group(M->mode, M->len, M->R, srcDim, dstDim, count, gp, bp, al, ap, srcGrad.P(), srcGrad.type, add, s);
+}
+
 // slices of the token axis for a delta product [dstDim x srcDim]: enough to give every CU a 256x256 tile, each slice a whole number of
 // k-tiles and at least 4096 tokens long
 int DeltaSplits(ts2_model *M, int srcDim, int dstDim)
@@ -298,8 +334,12 @@ int FfnBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
     CK(BackpropDX(M, L.w[2], M->stateGradFast, DISCR * Dot(F), true, drg, false, s));
     CK(ts2_backprop_row_tile_normalize_lolu(len, R, gate16.P(), wide16.P(), VEC, wideScale.P(), drg.P(), TS2_BF16, dgate.P(), dwide.P(),
         M->fastGradType, s));
-    CK(BackpropDX(M, L.w[0], dwide, DISCR * Dot(D), true, M->dNormState, false, s));
-    CK(BackpropDX(M, L.w[1], dgate, DISCR * Dot(D), false, M->dNormState, true, s));
+    {
+        TMatrix *const ws[2] = {&L.w[0], &L.w[1]};
+        const Arr *const gs[2] = {&dwide, &dgate};
+        const bool us[2] = {true, false};
+        CK(BackpropDXGroup(M, 2, ws, gs, DISCR * Dot(D), us, M->dNormState, false, s));
+    }
     // deltas (sources are stored in 1/24 units)
     CK(BackpropDelta(M, L.w[2], rg8, M->stateGradFast, VEC, gradScale, s));
     CK(BackpropDelta(M, L.w[0], norm8, dwide, VEC, gradScale, s));
@@ -396,10 +436,12 @@ int AttBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
     CK(ts2_backprop_row_tile_normalize_rope(len, R, dK.P(), TS2_BF16, 1.f, nullptr, nullptr, M->rope.P(), dKf.P(), M->fastGradType, s));
     CK(ts2_backprop_row_tile_normalize_rope(len, R, dV.P(), TS2_BF16, 1.f, v16.P(), vScale.P(), nullptr, dVf.P(), M->fastGradType, s));
     float a = DISCR * Dot(D);
-    CK(BackpropDX(M, L.w[0], dQf, a, true, M->dNormState, false, s));
-    CK(BackpropDX(M, L.w[1], dKf, a, true, M->dNormState, true, s));
-    CK(BackpropDX(M, L.w[2], dVf, a, true, M->dNormState, true, s));
-    CK(BackpropDX(M, L.w[3], dGate, a, false, M->dNormState, true, s));
+    {
+        TMatrix *const ws[4] = {&L.w[0], &L.w[1], &L.w[2], &L.w[3]};
+        const Arr *const gs[4] = {&dQf, &dKf, &dVf, &dGate};
+        const bool us[4] = {true, true, true, false};
+        CK(BackpropDXGroup(M, 4, ws, gs, a, us, M->dNormState, false, s));
+    }
     CK(BackpropDelta(M, L.w[0], norm8, dQf, VEC, gradScale, s));
     CK(BackpropDelta(M, L.w[1], norm8, dKf, VEC, gradScale, s, true));
     CK(BackpropDelta(M, L.w[2], norm8, dVf, VEC, gradScale, s, true));
@@ -815,7 +857,7 @@ extern "C" ts2_model *ts2_model_create(const ts2_model_config *cfg)
     M->sGrad8 = (uint8_t *)M->Dev((size_t)RP * maxW);
     M->sGradT = (uint8_t *)M->Dev((size_t)RP * maxW);
     M->sSrcT = (uint8_t *)M->Dev((size_t)RP * maxW);
-    M->sWT = (uint8_t *)M->Dev((size_t)maxW * maxW);
+    M->sWT = (uint8_t *)M->Dev((size_t)4 * maxW * maxW); // up to four transposed weights side by side (BackpropDXGroup)
     M->sPartialFloats = (size_t)8 * 2048 * 2048; // eight slices of a 2048 x 2048 delta, four of a 4096 x 2048 one
     M->sPartial = (float *)M->Dev(M->sPartialFloats * 4);
     M->sRowScale = (float *)M->Dev((size_t)RP * 4);

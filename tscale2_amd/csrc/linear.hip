@@ -69,6 +69,56 @@ extern "C" int ts2_matmul_backprop(int32_t mode, int32_t len, int32_t lenRound, 
     return ts2_gemm_nt(&g, stream);
 }
 
+extern "C" int ts2_matmul_backprop_group(int32_t mode, int32_t len, int32_t lenRound, int32_t srcDim, int32_t gradDim, int32_t count,
+    const ts2_mat *const *grad, const ts2_matmul_bwd_buffers *const *bufs, const float *alpha, const float *const *alphaPtr,
+    const ts2_mat *srcGrad, int32_t srcGradType, int32_t add, void *stream)
+{
+    if (!grad || !bufs || !alpha || !srcGrad || count < 1 || count > 4) {
+        return TS2_ERR_NULL;
+    }
+    for (int i = 0; i < count; ++i) {
+        if (!bufs[i] || (mode != TS2_I8 && !grad[i])) {
+            return TS2_ERR_NULL;
+        }
+    }
+    bool one = mode == TS2_E4M3 && count > 1 && (lenRound % 256) == 0 && (srcDim % 256) == 0 && (srcGradType == TS2_F32 || srcGradType == TS2_BF16);
+    for (int i = 1; i < count && one; ++i) {
+        one = grad[i]->strideBytes == grad[0]->strideBytes && bufs[i]->transformT.strideBytes == bufs[0]->transformT.strideBytes;
+    }
+    if (!one) {
+        for (int i = 0; i < count; ++i) {
+            int rc = ts2_matmul_backprop(mode, len, lenRound, srcDim, gradDim, grad[i], bufs[i], alpha[i], alphaPtr ? alphaPtr[i] : nullptr, srcGrad,
+                srcGradType, add || i > 0, stream);
+            if (rc) {
+                return rc;
+            }
+        }
+        return TS2_OK;
+    }
+    ts2_gemm_args g = {};
+    g.a = *grad[0];
+    g.b = bufs[0]->transformT;
+    g.c = *srcGrad;
+    g.abType = mode;
+    g.cType = srcGradType;
+    g.m = lenRound;
+    g.n = srcDim;
+    g.k = gradDim;
+    g.mLive = len;
+    g.alpha = alpha[0];
+    g.alphaPtr = alphaPtr ? alphaPtr[0] : nullptr;
+    g.epilogue = add ? TS2_EPI_ADD : TS2_EPI_STORE;
+    g.splitK = 1;
+    g.extraSegments = count - 1;
+    for (int i = 1; i < count; ++i) {
+        g.segment[i - 1].a = grad[i]->ptr;
+        g.segment[i - 1].b = bufs[i]->transformT.ptr;
+        g.segment[i - 1].alpha = alpha[i];
+        g.segment[i - 1].alphaPtr = alphaPtr ? alphaPtr[i] : nullptr;
+    }
+    return ts2_gemm_nt(&g, stream);
+}
+
 extern "C" int ts2_matmul_backprop_delta(int32_t mode, int32_t len, int32_t lenRound, int32_t srcDim, int32_t gradDim, const ts2_mat *src,
     const float *srcRowScale, const ts2_mat *grad, int32_t gradType, float alpha, const float *gradScale, int32_t kTile, const ts2_matmul_bwd_buffers *buf,
     const ts2_mat *delta, const ts2_mat *deltaTileScale, void *stream)

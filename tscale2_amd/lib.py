@@ -14,13 +14,17 @@ class Mat(C.Structure):
     _fields_ = [("ptr", C.c_void_p), ("strideBytes", C.c_int64), ("x", C.c_int32), ("y", C.c_int32)]
 
 
+class GemmSegment(C.Structure):
+    _fields_ = [("a", C.c_void_p), ("b", C.c_void_p), ("alpha", C.c_float), ("alphaPtr", C.c_void_p)]
+
+
 class GemmArgs(C.Structure):
     _fields_ = [("a", Mat), ("b", Mat), ("c", Mat), ("abType", C.c_int32), ("cType", C.c_int32), ("m", C.c_int32), ("n", C.c_int32),
                 ("k", C.c_int32), ("mLive", C.c_int32), ("rowScale", C.c_void_p), ("kTileScale", C.c_void_p), ("kTile", C.c_int32),
                 ("alpha", C.c_float), ("alphaPtr", C.c_void_p), ("epilogue", C.c_int32), ("tileScale", Mat), ("splitK", C.c_int32),
                 ("tileConfig", C.c_int32), ("tileGroup", C.c_void_p), ("bSlabBytes", C.c_int64), ("groupOffsets", C.c_void_p),
                 ("groups", C.c_int32), ("cSlabBytes", C.c_int64), ("tileScaleSlabBytes", C.c_int64), ("splitSlabBytes", C.c_int64), ("normalize", C.c_int32),
-                ("vecScale", C.c_float), ("rope", Mat)]
+                ("vecScale", C.c_float), ("rope", Mat), ("extraSegments", C.c_int32), ("segment", GemmSegment * 3)]
 
 
 def mat(t):
@@ -57,7 +61,8 @@ class Lib:
     def gemm_nt(self, a, b, c, ab_type, c_type, row_scale=None, k_tile_scale=None, k_tile=0, alpha=1.0, alpha_ptr=None,
                 epilogue=EPI_STORE, tile_scale=None, split_k=1, m_live=0, tile_config=0, k=None, check=True, m=None, n=None,
                 tile_group=None, b_slab_bytes=0, group_offsets=None, groups=0, c_slab_bytes=0, tile_scale_slab_bytes=0,
-                normalize=False, vec_scale=1.0, rope=None, split_slab_bytes=0):
+                normalize=False, vec_scale=1.0, rope=None, split_slab_bytes=0, segments=()):
+        """segments: up to three further products (a_i, b_i, alpha_i, alpha_ptr_i) added into the same C in the same launch"""
         args = GemmArgs()
         args.a, args.b, args.c = mat(a), mat(b), mat(c)
         args.abType, args.cType = ab_type, c_type
@@ -78,6 +83,10 @@ class Lib:
         args.tileConfig = tile_config
         args.normalize, args.vecScale, args.rope = int(normalize), vec_scale, mat(rope)
         args.splitSlabBytes = split_slab_bytes
+        args.extraSegments = len(segments)
+        for i, (sa, sb, sal, sp) in enumerate(segments):
+            assert sa.stride(0) == a.stride(0) and sb.stride(0) == b.stride(0)
+            args.segment[i].a, args.segment[i].b, args.segment[i].alpha, args.segment[i].alphaPtr = sa.data_ptr(), sb.data_ptr(), sal, ptr(sp)
         rc = self.dll.ts2_gemm_nt(C.byref(args), self.stream())
         if check:
             self.check(rc, "ts2_gemm_nt")
