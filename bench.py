@@ -121,7 +121,7 @@ def bench_linear_i8(args):
         if splits > 1:
             part = bufs.t["partial"]
             lib.gemm_nt(gt, st, part, L.I8, L.F32, k_tile_scale=tsc, k_tile=k_tile, split_k=splits, split_slab_bytes=grad_dim * src_dim * 4,
-                        tile_config=3, m=grad_dim)
+                        tile_config=3 | 8, m=grad_dim)  # the configuration BackpropDelta launches: 256x128 tile, eight waves
         else:
             lib.gemm_nt(gt, st, bufs.delta, L.I8, L.I8, k_tile_scale=tsc, k_tile=k_tile, epilogue=L.EPI_ROW_TILE_MAXNORM, tile_scale=bufs.delta_tile_scale)
     ms_dw = event_time_ms(dw, 20)

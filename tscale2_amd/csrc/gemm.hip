@@ -1235,6 +1235,22 @@ template <int TYPE, int WTM, int WTN> int DispatchEpi(const ts2_gemm_args *a, co
         return TS2_ERR_UNSUPPORTED;
     }
     if (kt) {
+        if constexpr (TYPE == T_I8 && WTM == 4 && WTN == 2) {
+            if (a->cType == TS2_F32 && epi == TS2_EPI_STORE && (a->tileConfig & 8) && p.splitK <= 1 && !p.groupOffsets) {
+                // the same 256x128 tile with eight waves of 64x64: two waves per SIMD, so that one wave's conversion of a finished
+                // k-tile (VALU) runs under the other's MFMAs
+                GemmP q = p;
+                q.tilesM = p.m / 256;
+                q.tilesN = (p.n + 127) / 128;
+                int nb = q.tilesM * q.tilesN;
+                int chunk = (nb % 8) == 0 ? nb / 8 : nb;
+                q.mapGroup = p.mapGroup ? p.mapGroup : chunk >= 64 ? 8 : chunk >= 8 ? 4 : 2;
+                hipLaunchKernelGGL((GemmNTDirect<TYPE, 2, 2, C_F32, TS2_EPI_STORE, true, 4, 2>), dim3(nb, p.splits > 1 ? p.splits : 1), dim3(512), 0,
+                    stream, q);
+                TS2_CHECK_LAUNCH();
+                return TS2_OK;
+            }
+        }
         if constexpr (TYPE == T_I8 && (WTM == 2 || (WTM == 4 && WTN == 2))) {
             if (a->cType == TS2_F32) {
                 return epi == TS2_EPI_ADD ? Launch<TYPE, WTM, WTN, C_F32, TS2_EPI_ADD, true>(p, stream)

@@ -186,7 +186,8 @@ extern "C" int ts2_matmul_backprop_delta(int32_t mode, int32_t len, int32_t lenR
         g.epilogue = TS2_EPI_STORE;
         g.splitK = splits;
         g.splitSlabBytes = (int64_t)gradDim * buf->partial.strideBytes;
-        g.tileConfig = mode == TS2_I8 ? ((gradDim % 256) == 0 ? 3 : 2) : (((gradDim % 256) == 0 && (srcDim % 256) == 0) ? 1 : 2);
+        // int8: 256x128 tile with eight waves (the k-tile conversions of one wave run under the other's MFMAs)
+        g.tileConfig = mode == TS2_I8 ? ((gradDim % 256) == 0 ? (3 | 8) : 2) : (((gradDim % 256) == 0 && (srcDim % 256) == 0) ? 1 : 2);
         rc = ts2_gemm_nt(&g, stream);
         if (rc) {
             return rc;
