@@ -389,6 +389,77 @@ __global__ void __launch_bounds__(256) NormalizeVecsRowMax(int len, int lenRound
     }
 }
 
+// The same quantiser with one wave per row for bf16 rows of NCH * 512 elements (at most 4096): a lane holds NCH chunks of 8
+// consecutive elements (16-byte loads, 8-byte stores, each instruction of the wave covering 1 KB / 512 B of the row), the row
+// maxima are wave reductions, and no workgroup barrier or LDS exchange is left.  Same arithmetic per element as NormalizeVecsRowMax.
+template <int NCH>
+__global__ void __launch_bounds__(256) NormalizeRowsWave(int len, int lenRound, Mat src, const float *colScale, Mat dst, float *rowScale, float *rowAbsMax)
+{
+    const int lane = threadIdx.x & 63;
+    const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= lenRound) {
+        return;
+    }
+    uint8_t *out = dst.p + (int64_t)t * dst.ld;
+    if (t >= len) {
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            *(uint2 *)(out + (i * 64 + lane) * 8) = make_uint2(0u, 0u);
+        }
+        if (lane == 0) {
+            rowScale[t] = 0;
+            if (rowAbsMax) {
+                rowAbsMax[t] = 0;
+            }
+        }
+        return;
+    }
+    const uint8_t *in = src.p + (int64_t)t * src.ld;
+    uint4 raw[NCH];
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        raw[i] = *(const uint4 *)(in + (i * 64 + lane) * 16);
+    }
+    F4 v[NCH][2];
+    float mx = 0, plain = 0;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        v[i][0] = MakeF4(__uint_as_float(raw[i].x << 16), __uint_as_float(raw[i].x & 0xffff0000u), __uint_as_float(raw[i].y << 16),
+            __uint_as_float(raw[i].y & 0xffff0000u));
+        v[i][1] = MakeF4(__uint_as_float(raw[i].z << 16), __uint_as_float(raw[i].z & 0xffff0000u), __uint_as_float(raw[i].w << 16),
+            __uint_as_float(raw[i].w & 0xffff0000u));
+        plain = fmaxf(plain, fmaxf(HMaxAbs(v[i][0]), HMaxAbs(v[i][1])));
+        if (colScale) {
+            const float *cs = colScale + (i * 64 + lane) * 8;
+            v[i][0] = v[i][0] * Load4<TF32>(cs);
+            v[i][1] = v[i][1] * Load4<TF32>(cs + 4);
+        }
+        mx = fmaxf(mx, fmaxf(HMaxAbs(v[i][0]), HMaxAbs(v[i][1])));
+    }
+    mx = WaveMax(mx);
+    plain = WaveMax(plain);
+    float discr = 0, mult = 0;
+    if (mx > 0) {
+        discr = mx / 127;
+        mult = 1 / discr;
+    }
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        F4 a = v[i][0] * mult, b = v[i][1] * mult;
+        uint32_t lo = (uint32_t)(CvtToI8(a.x) & 0xff) | ((uint32_t)(CvtToI8(a.y) & 0xff) << 8) | ((uint32_t)(CvtToI8(a.z) & 0xff) << 16) |
+                      ((uint32_t)(CvtToI8(a.w) & 0xff) << 24);
+        uint32_t hi = (uint32_t)(CvtToI8(b.x) & 0xff) | ((uint32_t)(CvtToI8(b.y) & 0xff) << 8) | ((uint32_t)(CvtToI8(b.z) & 0xff) << 16) |
+                      ((uint32_t)(CvtToI8(b.w) & 0xff) << 24);
+        *(uint2 *)(out + (i * 64 + lane) * 8) = make_uint2(lo, hi);
+    }
+    if (lane == 0) {
+        rowScale[t] = discr;
+        if (rowAbsMax) {
+            rowAbsMax[t] = plain;
+        }
+    }
+}
+
 __global__ void FillFloats(float *p, int n, float v)
 {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -955,6 +1026,24 @@ extern "C" int ts2_normalize_vecs_row_max2(int32_t len, int32_t lenRound, const 
         return TS2_ERR_SHAPE;
     }
     const bool reg = dim <= 4096;
+    if (srcType == TS2_BF16 && dim % 512 == 0 && dim <= 4096 && Aligned16(src->ptr, src->strideBytes) && (((uintptr_t)dst->ptr | dst->strideBytes) & 7) == 0 &&
+        (!colScale || ((uintptr_t)colScale & 15) == 0)) {
+        const dim3 grid((lenRound + 3) / 4);
+#define LAUNCH_RW(N) hipLaunchKernelGGL((NormalizeRowsWave<N>), grid, dim3(256), 0, STREAM, len, lenRound, M(*src), colScale, M(*dst), rowScale, rowAbsMax)
+        switch (dim / 512) {
+        case 1: LAUNCH_RW(1); break;
+        case 2: LAUNCH_RW(2); break;
+        case 3: LAUNCH_RW(3); break;
+        case 4: LAUNCH_RW(4); break;
+        case 5: LAUNCH_RW(5); break;
+        case 6: LAUNCH_RW(6); break;
+        case 7: LAUNCH_RW(7); break;
+        default: LAUNCH_RW(8); break;
+        }
+#undef LAUNCH_RW
+        TS2_CHECK_LAUNCH();
+        return TS2_OK;
+    }
 #define LAUNCH_RM(TS, REG) hipLaunchKernelGGL((NormalizeVecsRowMax<TS, REG>), dim3(lenRound < 4096 ? lenRound : 4096), dim3(256), 0, STREAM, len, lenRound, dim, M(*src), colScale, M(*dst), rowScale, rowAbsMax)
     if (srcType == TS2_BF16) {
         if (reg) {
