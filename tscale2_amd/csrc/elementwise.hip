@@ -396,66 +396,73 @@ template <int NCH>
 __global__ void __launch_bounds__(256) NormalizeRowsWave(int len, int lenRound, Mat src, const float *colScale, Mat dst, float *rowScale, float *rowAbsMax)
 {
     const int lane = threadIdx.x & 63;
-    const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (t >= lenRound) {
-        return;
-    }
-    uint8_t *out = dst.p + (int64_t)t * dst.ld;
-    if (t >= len) {
+    const int nWaves = gridDim.x * 4;
+    // the column scales of the lane's chunks stay in registers for all the rows the wave walks
+    F4 cs[NCH][2];
+    if (colScale) {
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
-            *(uint2 *)(out + (i * 64 + lane) * 8) = make_uint2(0u, 0u);
+            cs[i][0] = Load4<TF32>(colScale + (i * 64 + lane) * 8);
+            cs[i][1] = Load4<TF32>(colScale + (i * 64 + lane) * 8 + 4);
+        }
+    }
+    for (int t = blockIdx.x * 4 + (threadIdx.x >> 6); t < lenRound; t += nWaves) {
+        uint8_t *out = dst.p + (int64_t)t * dst.ld;
+        if (t >= len) {
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) {
+                *(uint2 *)(out + (i * 64 + lane) * 8) = make_uint2(0u, 0u);
+            }
+            if (lane == 0) {
+                rowScale[t] = 0;
+                if (rowAbsMax) {
+                    rowAbsMax[t] = 0;
+                }
+            }
+            continue;
+        }
+        const uint8_t *in = src.p + (int64_t)t * src.ld;
+        uint4 raw[NCH];
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            raw[i] = *(const uint4 *)(in + (i * 64 + lane) * 16);
+        }
+        F4 v[NCH][2];
+        float mx = 0, plain = 0;
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            v[i][0] = MakeF4(__uint_as_float(raw[i].x << 16), __uint_as_float(raw[i].x & 0xffff0000u), __uint_as_float(raw[i].y << 16),
+                __uint_as_float(raw[i].y & 0xffff0000u));
+            v[i][1] = MakeF4(__uint_as_float(raw[i].z << 16), __uint_as_float(raw[i].z & 0xffff0000u), __uint_as_float(raw[i].w << 16),
+                __uint_as_float(raw[i].w & 0xffff0000u));
+            plain = fmaxf(plain, fmaxf(HMaxAbs(v[i][0]), HMaxAbs(v[i][1])));
+            if (colScale) {
+                v[i][0] = v[i][0] * cs[i][0];
+                v[i][1] = v[i][1] * cs[i][1];
+            }
+            mx = fmaxf(mx, fmaxf(HMaxAbs(v[i][0]), HMaxAbs(v[i][1])));
+        }
+        mx = WaveMax(mx);
+        plain = WaveMax(plain);
+        float discr = 0, mult = 0;
+        if (mx > 0) {
+            discr = mx / 127;
+            mult = 1 / discr;
+        }
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            F4 a = v[i][0] * mult, b = v[i][1] * mult;
+            uint32_t lo = (uint32_t)(CvtToI8(a.x) & 0xff) | ((uint32_t)(CvtToI8(a.y) & 0xff) << 8) | ((uint32_t)(CvtToI8(a.z) & 0xff) << 16) |
+                          ((uint32_t)(CvtToI8(a.w) & 0xff) << 24);
+            uint32_t hi = (uint32_t)(CvtToI8(b.x) & 0xff) | ((uint32_t)(CvtToI8(b.y) & 0xff) << 8) | ((uint32_t)(CvtToI8(b.z) & 0xff) << 16) |
+                          ((uint32_t)(CvtToI8(b.w) & 0xff) << 24);
+            *(uint2 *)(out + (i * 64 + lane) * 8) = make_uint2(lo, hi);
         }
         if (lane == 0) {
-            rowScale[t] = 0;
+            rowScale[t] = discr;
             if (rowAbsMax) {
-                rowAbsMax[t] = 0;
+                rowAbsMax[t] = plain;
             }
-        }
-        return;
-    }
-    const uint8_t *in = src.p + (int64_t)t * src.ld;
-    uint4 raw[NCH];
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-        raw[i] = *(const uint4 *)(in + (i * 64 + lane) * 16);
-    }
-    F4 v[NCH][2];
-    float mx = 0, plain = 0;
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-        v[i][0] = MakeF4(__uint_as_float(raw[i].x << 16), __uint_as_float(raw[i].x & 0xffff0000u), __uint_as_float(raw[i].y << 16),
-            __uint_as_float(raw[i].y & 0xffff0000u));
-        v[i][1] = MakeF4(__uint_as_float(raw[i].z << 16), __uint_as_float(raw[i].z & 0xffff0000u), __uint_as_float(raw[i].w << 16),
-            __uint_as_float(raw[i].w & 0xffff0000u));
-        plain = fmaxf(plain, fmaxf(HMaxAbs(v[i][0]), HMaxAbs(v[i][1])));
-        if (colScale) {
-            const float *cs = colScale + (i * 64 + lane) * 8;
-            v[i][0] = v[i][0] * Load4<TF32>(cs);
-            v[i][1] = v[i][1] * Load4<TF32>(cs + 4);
-        }
-        mx = fmaxf(mx, fmaxf(HMaxAbs(v[i][0]), HMaxAbs(v[i][1])));
-    }
-    mx = WaveMax(mx);
-    plain = WaveMax(plain);
-    float discr = 0, mult = 0;
-    if (mx > 0) {
-        discr = mx / 127;
-        mult = 1 / discr;
-    }
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-        F4 a = v[i][0] * mult, b = v[i][1] * mult;
-        uint32_t lo = (uint32_t)(CvtToI8(a.x) & 0xff) | ((uint32_t)(CvtToI8(a.y) & 0xff) << 8) | ((uint32_t)(CvtToI8(a.z) & 0xff) << 16) |
-                      ((uint32_t)(CvtToI8(a.w) & 0xff) << 24);
-        uint32_t hi = (uint32_t)(CvtToI8(b.x) & 0xff) | ((uint32_t)(CvtToI8(b.y) & 0xff) << 8) | ((uint32_t)(CvtToI8(b.z) & 0xff) << 16) |
-                      ((uint32_t)(CvtToI8(b.w) & 0xff) << 24);
-        *(uint2 *)(out + (i * 64 + lane) * 8) = make_uint2(lo, hi);
-    }
-    if (lane == 0) {
-        rowScale[t] = discr;
-        if (rowAbsMax) {
-            rowAbsMax[t] = plain;
         }
     }
 }
@@ -1028,7 +1035,9 @@ extern "C" int ts2_normalize_vecs_row_max2(int32_t len, int32_t lenRound, const 
     const bool reg = dim <= 4096;
     if (srcType == TS2_BF16 && dim % 512 == 0 && dim <= 4096 && Aligned16(src->ptr, src->strideBytes) && (((uintptr_t)dst->ptr | dst->strideBytes) & 7) == 0 &&
         (!colScale || ((uintptr_t)colScale & 15) == 0)) {
-        const dim3 grid((lenRound + 3) / 4);
+        // with column scales a wave walks several rows (the scales stay in registers), else one row per wave
+        const int wgs = (lenRound + 3) / 4;
+        const dim3 grid(colScale && wgs > 2048 ? 2048 : wgs);
 #define LAUNCH_RW(N) hipLaunchKernelGGL((NormalizeRowsWave<N>), grid, dim3(256), 0, STREAM, len, lenRound, M(*src), colScale, M(*dst), rowScale, rowAbsMax)
         switch (dim / 512) {
         case 1: LAUNCH_RW(1); break;
