@@ -129,8 +129,8 @@ def bench_linear_i8(args):
     roof = {"bound": "mfma", "achieved": gemm_ops / (avg_ms * 1e-3) / 1e12, "peak": PEAK_INT8 / 1e12, "unit": "TFLOP/s",
             "frac": gemm_ops / (avg_ms * 1e-3) / PEAK_INT8,
             # HBM bytes per GEMM launch (mean of the dX and the delta launch) from rocprofv3 FETCH_SIZE / WRITE_SIZE, calibrated against the
-            # copy probe (factors 2.0 and 1.0): dX 96.7 + 64.0 MiB, delta 192.7 + 4.1 MiB; algorithmic 132.1 and 84.1 MiB
-            "traffic": 0.5 * (160.7 + 196.8) * 2 ** 20, "traffic_algorithmic": 0.5 * (132.1 + 84.1) * 2 ** 20,
+            # copy probe (factors 2.0 and 1.0): dX 96.8 + 64.0 MiB, delta 192.3 + 32.0 MiB (two fp32 slices); algorithmic 132.1 and 112.0 MiB
+            "traffic": 0.5 * (160.8 + 224.3) * 2 ** 20, "traffic_algorithmic": 0.5 * (132.1 + 112.0) * 2 ** 20,
             "kernel": "GemmNT<int8> (dX launch %.1f us, delta launch %.1f us; 137.44 GOP per launch)" % (ms_dx * 1e3, ms_dw * 1e3)}
     out = {"metric": "fwd+bwd tokens/sec on 1 MI355X; bwd GEMM TFLOPS as % of MFMA peak", "value": len_ / (ms_per_step * 1e-3), "unit": "tokens/s",
            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
