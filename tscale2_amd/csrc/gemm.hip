@@ -5,17 +5,20 @@
 //   * a workgroup = 4 wavefronts (2x2), each wave owns a (32*WTM) x (32*WTN) block of C as WTM x WTN MFMA 32x32 accumulators
 //     (WTM = WTN = 4 -> 256x256 workgroup tile, 256 accumulator registers per lane; 2 -> 128x128; 4x2 -> 256x128 for the
 //     k-tile-scaled int8 product, which carries a second, fp32 accumulator set); an 8-wave 256x256 variant puts two waves on a SIMD;
-//   * K advances 128 bytes per step.  GemmNTDirect (the default) moves A and B tiles global -> LDS with global_load_lds_dwordx4, no
-//     staging registers and no ds_write; the two LDS stages are separate arrays so that operand reads of one stage never wait for the
-//     loads into the other.  GemmNT (tileConfig bit 2, and the atomically accumulated split-K) stages through registers.  In both,
-//     16-byte chunks are XOR-swizzled by (row/2)%8: loader writes and ds_read_b128 operand fetches are bank-conflict free;
+//   * K advances 128 bytes per step; A and B tiles go global -> LDS with global_load_lds_dwordx4, no staging registers and no
+//     ds_write.  GemmNTRing (the 256x256 tile) keeps three stages of A and two of B (all 160 KB of LDS): A is loaded two steps
+//     ahead, B one, one load at a time between the MFMAs.  GemmNTDirect (the other tiles, k-tile scales, expert groups) has two
+//     stages.  Stages are separate static arrays so that operand reads of one never wait for the loads into another.  GemmNT
+//     (tileConfig bit 2, and the atomically accumulated split-K) stages through registers.  In all of them 16-byte chunks are
+//     XOR-swizzled by (row/2)%8: loader writes and ds_read_b128 operand fetches are bank-conflict free;
 //   * operand fragments are read one K-slice ahead of the MFMAs that use them (two fragment sets), one barrier per step;
 //   * MFMA: v_mfma_i32_32x32x32_i8, v_mfma_f32_32x32x64_f8f6f4 (fp8 x fp8), v_mfma_f32_32x32x16_bf16;
 //   * workgroup ids are remapped so that each of the 8 XCDs (which receive ids round-robin) works on a compact band of C tiles
 //     and its L2 sees every A/B panel only a few times;
 //   * epilogues are fused: per-row scale, alpha, device scalar, store/accumulate in fp32/bf16, raw i32, packed int8 delta (row-tile
 //     max-normalise), row-tile normalise + RoPE to bf16, per-k-tile scales (exact int32 per tile, fp32 across tiles); the contraction
-//     can be cut into stored slices (deterministic split-K) or expert groups (MoE).
+//     can be cut into stored slices (deterministic split-K) or expert groups (MoE), and several products can be added into one
+//     result in one launch.
 #include "common.h"
 #include <type_traits>
 
