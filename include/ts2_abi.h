@@ -33,7 +33,8 @@ enum ts2_dtype {
     TS2_E4M3 = 1, /* OCP e4m3fn, the format of src/util/fp8.h:4-21 */
     TS2_BF16 = 2, /* 16-bit activations; the reference uses IEEE half here */
     TS2_F32 = 3,
-    TS2_I32 = 4
+    TS2_I32 = 4,
+    TS2_F16 = 5 /* IEEE half: result type of ts2_gemm_nt / ts2_matmul_forward only (the final layer's logits, as in the reference) */
 };
 
 /* row-major 2-D view: TCuda2DPtr<T>{Data, StrideInBytes} + debug sizes, src/lib/cuda/cuda_arrays.h:217-253 */
@@ -63,7 +64,8 @@ enum ts2_epilogue {
  *   Int8MatMulKernel / Int8MatMulKernelRowScale / Int8MatMulYScaleKernel  src/lib/cuda/cuda_i8.cuh:157-320
  *   GenericMatMulKernel (fp8, fp16)                                        src/lib/cuda/cuda_matmul.cuh:396-416
  * abType: TS2_I8 (int32 accumulate, exact), TS2_E4M3 or TS2_BF16 (fp32 accumulate).
- * cType : TS2_F32, TS2_BF16, TS2_I32 (raw accumulator, TS2_I8 inputs and TS2_EPI_STORE only) or TS2_I8 (ROW_TILE_MAXNORM).
+ * cType : TS2_F32, TS2_BF16, TS2_F16 (TS2_EPI_STORE only), TS2_I32 (raw accumulator, TS2_I8 inputs and TS2_EPI_STORE only) or TS2_I8
+ *         (ROW_TILE_MAXNORM).
  * rowScale  (optional, [m])  : per-row scale of A applied to the accumulator before the epilogue (the dX kernel).
  * kTileScale (optional, [k/kTile], TS2_I8 only): one scale per kTile contraction rows; each tile's int32 sum is exact and
  *             tiles are added in fp32 in tile order (the dW kernel).  kTile must be a multiple of 128.

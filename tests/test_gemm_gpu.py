@@ -284,3 +284,30 @@ def test_several_products_into_one_result(ab, add):
     a8 = torch.zeros((m, k), dtype=torch.int8, device="cuda"); b8 = torch.zeros((n, k), dtype=torch.int8, device="cuda")
     assert lib.gemm_nt(a8, b8, got, L.I8, L.F32, segments=[(a8, b8, 1.0, None)], check=False) == -3
     assert lib.gemm_nt(As[0], Bs[0], got, t, L.F32, tile_config=2, segments=[(As[1], Bs[1], 1.0, None)], check=False) == -3
+
+
+@pytest.mark.parametrize("ab,tile", [("e4m3", 1), ("i8", 1), ("e4m3", 2)])
+def test_half_results_are_the_rounded_fp32_results(ab, tile):
+    """cType TS2_F16 (the final layer's logits): every element is the fp32 result of the same launch configuration rounded to the
+    nearest IEEE half; rows >= mLive are zero."""
+    print("case half results", ab, tile, flush=True)
+    from tscale2_amd import lib as L
+    lib = L.load()
+    m, n, k = 512, 768, 256
+    g = torch.Generator(device="cuda").manual_seed(17)
+    if ab == "i8":
+        a = torch.randint(-100, 100, (m, k), dtype=torch.int8, device="cuda", generator=g)
+        b = torch.randint(-100, 100, (n, k), dtype=torch.int8, device="cuda", generator=g)
+        t = L.I8
+    else:
+        a = (torch.randn((m, k), device="cuda", generator=g) * 6).to(torch.float8_e4m3fn).view(torch.uint8)
+        b = (torch.randn((n, k), device="cuda", generator=g) * 6).to(torch.float8_e4m3fn).view(torch.uint8)
+        t = L.E4M3
+    c32 = torch.empty((m, n), dtype=torch.float32, device="cuda")
+    c16 = torch.full((m, n), 7, dtype=torch.int16, device="cuda")
+    lib.gemm_nt(a, b, c32, t, L.F32, alpha=3e-3, tile_config=tile, m_live=500)
+    lib.gemm_nt(a, b, c16, t, L.F16, alpha=3e-3, tile_config=tile, m_live=500)
+    torch.cuda.synchronize()
+    assert torch.equal(c16.view(torch.float16), c32.half())
+    assert (c16[500:] == 0).all()
+    assert lib.gemm_nt(a, b, c16, t, L.F16, epilogue=L.EPI_ADD, check=False) == -3

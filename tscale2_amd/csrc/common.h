@@ -36,6 +36,15 @@ __device__ __forceinline__ uint32_t PackBf16x2(float lo, float hi)
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, v2bf));
 }
 
+// two fp32 -> packed IEEE half, round to nearest even
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t PackF16x2(float lo, float hi)
+{
+    v2f f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, v2h));
+}
+
 __device__ __forceinline__ bf16_t FloatToBf16(float x)
 {
     return (bf16_t)(PackBf16x2(x, 0.f) & 0xffffu);

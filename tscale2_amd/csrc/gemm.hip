@@ -65,7 +65,7 @@ struct GemmP {
 };
 
 enum { T_I8 = 0, T_FP8 = 1, T_BF16 = 2 };
-enum { C_F32 = 0, C_BF16 = 1, C_I32 = 2, C_I8PACK = 3, C_BF16NORM = 4 };
+enum { C_F32 = 0, C_BF16 = 1, C_I32 = 2, C_I8PACK = 3, C_BF16NORM = 4, C_F16 = 5 };
 
 constexpr int BKB = 128; // bytes of K per step
 
@@ -100,7 +100,7 @@ __device__ __forceinline__ void MapTile(int bid, int nb, int tilesM, int tilesN,
 // bf16 store of one 32x32 block held as v[e] (lane = column, e -> row): neighbouring lanes swap one value so that even lanes store
 // columns (c, c+1) of the even row of a row pair and odd lanes those of the odd row: 4-byte stores instead of 2-byte ones.
 // rowOf(e) gives the global row; rows >= mLive are written as zeros.
-template <class TRow>
+template <bool F16 = false, class TRow>
 __device__ __forceinline__ void StoreBlockBf16(uint8_t *c, int64_t ldc, int col, int l32, int mLive, const float (&v)[16], TRow rowOf)
 {
     const bool odd = l32 & 1;
@@ -112,7 +112,7 @@ __device__ __forceinline__ void StoreBlockBf16(uint8_t *c, int64_t ldc, int col,
         float lo = odd ? got : v[e];
         float hi = odd ? v[e + 1] : got;
         int row = rowOf(odd ? e + 1 : e);
-        uint32_t packed = row < mLive ? PackBf16x2(lo, hi) : 0u;
+        uint32_t packed = row < mLive ? (F16 ? PackF16x2(lo, hi) : PackBf16x2(lo, hi)) : 0u;
         *(uint32_t *)(c + (int64_t)row * ldc + (int64_t)(col & ~1) * 2) = packed;
     }
 }
@@ -382,7 +382,7 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
         // to back, and for the accumulate epilogues the 4 x WTN old values are all fetched before the first store
 #pragma unroll
         for (int i = 0; i < WTM; ++i) {
-            if constexpr (CT == C_BF16 && EPI == TS2_EPI_STORE) {
+            if constexpr ((CT == C_BF16 || CT == C_F16) && EPI == TS2_EPI_STORE) {
 #pragma unroll
                 for (int j = 0; j < WTN; ++j) {
                     const int col = colBase + wn * (32 * WTN) + j * 32 + l32;
@@ -395,7 +395,7 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
                         }
                         v[e] = accVal(i, j, e) * rs;
                     }
-                    StoreBlockBf16(p.c, p.ldc, col, l32, mLive, v, [&](int e) { return rowBase + rowLocal(i, e); });
+                    StoreBlockBf16<CT == C_F16>(p.c, p.ldc, col, l32, mLive, v, [&](int e) { return rowBase + rowLocal(i, e); });
                 }
             } else {
 #pragma unroll
@@ -1278,6 +1278,14 @@ template <int TYPE, int WTM, int WTN> int DispatchEpi(const ts2_gemm_args *a, co
         return epi == TS2_EPI_ADD ? Launch<TYPE, WTM, WTN, C_F32, TS2_EPI_ADD, false>(p, stream)
                                   : Launch<TYPE, WTM, WTN, C_F32, TS2_EPI_STORE, false>(p, stream);
     }
+    if (a->cType == TS2_F16) {
+        if constexpr (WTM == WTN) {
+            if (epi == TS2_EPI_STORE && p.splitK <= 1) {
+                return Launch<TYPE, WTM, WTN, C_F16, TS2_EPI_STORE, false>(p, stream);
+            }
+        }
+        return TS2_ERR_UNSUPPORTED;
+    }
     if (a->cType == TS2_BF16) {
         if (eight) {
             return epi == TS2_EPI_ADD ? Launch8<TYPE, C_BF16, TS2_EPI_ADD>(p, stream) : Launch8<TYPE, C_BF16, TS2_EPI_STORE>(p, stream);
@@ -1335,7 +1343,7 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
     if (a->kTileScale && (a->abType != TS2_I8 || a->kTile <= 0 || (a->kTile % 128) || (a->k % a->kTile))) {
         return TS2_ERR_SHAPE;
     }
-    if (a->cType == TS2_BF16 && (a->c.strideBytes & 3)) {
+    if ((a->cType == TS2_BF16 || a->cType == TS2_F16) && (a->c.strideBytes & 3)) {
         return TS2_ERR_ALIGN; // bf16 results are stored two columns at a time
     }
     int splitK = a->splitK > 1 ? a->splitK : 1;

@@ -40,7 +40,7 @@ hipError_t Copy2D(void *dst, size_t dpitch, const void *src, size_t spitch, size
 
 int ElemSz(int type)
 {
-    return (type == TS2_F32 || type == TS2_I32) ? 4 : (type == TS2_BF16 ? 2 : 1);
+    return (type == TS2_F32 || type == TS2_I32) ? 4 : ((type == TS2_BF16 || type == TS2_F16) ? 2 : 1);
 }
 
 struct Arr {
@@ -133,6 +133,7 @@ struct ts2_model {
     Arr wT;                                  // transposed expert weights scratch
     // final layer
     Arr logits, gradV, gradVT, fnT, wfT;
+    Arr logits16;                            // IEEE-half logits of the backward pass (the fp32 ones serve ts2_model_forward)
     // linear backward scratch
     uint8_t *sGrad8 = 0, *sGradT = 0, *sSrcT = 0, *sWT = 0;
     float *sPartial = 0;                     // fp32 slices of a delta product with few output tiles
@@ -636,18 +637,19 @@ int ModelForward(ts2_model *M, void *s)
 }
 
 // final layer: src/gpt/compute/gpu_final.cuh:223-296 / cpu_transformer.cpp:119-172
-int FinalLogits(ts2_model *M, void *s)
+int FinalLogits(ts2_model *M, const Arr &logits, void *s)
 {
     int D = M->cfg.dim, depth = (int)M->layers.size();
-    return Forward(M, M->finalW, M->normState[depth], VEC * DISCR * Dot(D) / LN2F, true, M->logits, false, s);
+    return Forward(M, M->finalW, M->normState[depth], VEC * DISCR * Dot(D) / LN2F, true, logits, false, s);
 }
 
 int FinalBackward(ts2_model *M, void *s)
 {
     int D = M->cfg.dim, V = M->cfg.vocab, VP = M->VP, depth = (int)M->layers.size(), R = M->R;
-    CK(FinalLogits(M, s));
+    // logits in IEEE half like the reference's logit window: a third of the traffic of fp32 logits written once and read twice
+    CK(FinalLogits(M, M->logits16, s));
     CK(Ts2ZeroRows(Flat(M->lossSum, 1, 1, TS2_F32).P(), 1, 4, s));
-    CK(Ts2FinalSoftmaxGrad(R, V, M->logits.P(), M->bias, M->target, 1.f, M->gradV.P(), M->lossSum, 0, s));
+    CK(Ts2FinalSoftmaxGradHalf(R, V, M->logits16.P(), M->bias, M->target, 1.f, M->gradV.P(), M->lossSum, s));
     // dfn = grad * Wf / sqrt(D): bf16 product, the 8-bit weights converted exactly
     // (columns V..VP of the logits are products with zero rows, the same columns of the gradient stay zero: the softmax pass covers V)
     CK(Ts2TransposeToBf16(VP, VP, D, M->finalW.fast.P(), M->mode, M->wfT.P(), s));
@@ -879,7 +881,7 @@ extern "C" ts2_model *ts2_model_create(const ts2_model_config *cfg)
         int wtRows = E * (X > D ? X : D), wtCols = X > D ? X : D;
         ok &= M->Alloc(&M->wT, wtRows, wtCols, M->mode);
     }
-    ok &= M->Alloc(&M->logits, R, VP, TS2_F32) && M->Alloc(&M->gradV, R, VP, TS2_BF16) && M->Alloc(&M->gradVT, VP, R, TS2_BF16) &&
+    ok &= M->Alloc(&M->logits, R, VP, TS2_F32) && M->Alloc(&M->logits16, R, VP, TS2_F16) && M->Alloc(&M->gradV, R, VP, TS2_BF16) && M->Alloc(&M->gradVT, VP, R, TS2_BF16) &&
           M->Alloc(&M->fnT, D, R, TS2_BF16) && M->Alloc(&M->wfT, D, VP, TS2_BF16);
     if (!ok || !M->sGrad8 || !M->sGradT || !M->sSrcT || !M->sWT || !M->sPartial) {
         delete M;
@@ -971,7 +973,7 @@ extern "C" int ts2_model_forward(ts2_model *M, void *stream)
         return TS2_ERR_NULL;
     }
     CK(ModelForward(M, stream));
-    CK(FinalLogits(M, stream));
+    CK(FinalLogits(M, M->logits, stream));
     // probabilities in place of the logits; the gradient buffer is scratch here
     return Ts2FinalSoftmaxGrad(M->R, M->cfg.vocab, M->logits.P(), M->bias, M->target, 1.f, M->gradV.P(), nullptr, 1, stream);
 }

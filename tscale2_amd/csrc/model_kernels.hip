@@ -213,6 +213,87 @@ __global__ void ZeroBytes(uint8_t *p, int64_t ld, int rowBytes)
         *(uint32_t *)(row + x) = 0;
     }
 }
+// The same for IEEE-half logits (the reference keeps its logit window in half, src/gpt/compute/gpu_final.cuh:173-189): eight values
+// per 16-byte load, no probabilities kept
+__global__ void __launch_bounds__(256) FinalSoftmaxGradHalf(int vocab, const _Float16 *logits, int64_t ldLogits, const float *bias, const int *target,
+    float gradMult, bf16_t *grad, int64_t ldGrad, float *lossSum)
+{
+    typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+    __shared__ float redM[4], redS[4];
+    int t = blockIdx.x;
+    int tid = threadIdx.x;
+    const _Float16 *row = (const _Float16 *)((const uint8_t *)logits + (int64_t)t * ldLogits);
+    bf16_t *grow = (bf16_t *)((uint8_t *)grad + (int64_t)t * ldGrad);
+    int tg = target[t];
+    if (tg < 0) {
+        for (int k = tid * 8; k < vocab; k += 2048) {
+            *(uint4 *)(grow + k) = make_uint4(0, 0, 0, 0);
+        }
+        return;
+    }
+    float m = 0, sum = 0;
+    for (int k0 = tid * 8; k0 < vocab; k0 += 4096) {
+        float x[2][8], bv[2][8];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            int k = k0 + i * 2048;
+            bool in = k < vocab;
+            v8h h = in ? *(const v8h *)(row + k) : (v8h)(_Float16)-60000.f;
+            float4 b0 = in ? *(const float4 *)(bias + k) : make_float4(0, 0, 0, 0);
+            float4 b1 = in ? *(const float4 *)(bias + k + 4) : make_float4(0, 0, 0, 0);
+            const float bb[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                x[i][e] = (float)h[e];
+                bv[i][e] = bb[e];
+            }
+        }
+        float mNew = m;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                mNew = fmaxf(mNew, x[i][e]);
+            }
+        }
+        sum *= exp2f(m - mNew);
+        m = mNew;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                sum += exp2f(x[i][e] + bv[i][e] - m);
+            }
+        }
+    }
+    float mx = WaveMax(m);
+    if ((tid & 63) == 0) {
+        redM[tid >> 6] = mx;
+    }
+    __syncthreads();
+    mx = fmaxf(fmaxf(redM[0], redM[1]), fmaxf(redM[2], redM[3]));
+    sum = WaveSum(sum * exp2f(m - mx));
+    if ((tid & 63) == 0) {
+        redS[tid >> 6] = sum;
+    }
+    __syncthreads();
+    float scale = 1 / ((redS[0] + redS[1]) + (redS[2] + redS[3]));
+    for (int k = tid * 8; k < vocab; k += 2048) {
+        v8h h = *(const v8h *)(row + k); // second read of the row: served by L2
+        float4 b0 = *(const float4 *)(bias + k), b1 = *(const float4 *)(bias + k + 4);
+        const float bb[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+        float g[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            float pr = exp2f((float)h[e] + bb[e] - mx) * scale;
+            g[e] = ((k + e == tg ? 1.f : 0.f) - pr) * gradMult;
+            if (k + e == tg && lossSum) {
+                atomicAdd(lossSum, logf(pr));
+            }
+        }
+        *(uint4 *)(grow + k) = make_uint4(PackBf16x2(g[0], g[1]), PackBf16x2(g[2], g[3]), PackBf16x2(g[4], g[5]), PackBf16x2(g[6], g[7]));
+    }
+}
 } // namespace
 
 #define STREAM ((hipStream_t)stream)
@@ -240,6 +321,19 @@ int Ts2EmbedBackward(int len, int dim, const int *labelPtr, const uint32_t *labe
     TS2_CHECK_LAUNCH();
     hipLaunchKernelGGL(EmbedBackward, dim3(len), dim3(256), 0, STREAM, len, dim, labelPtr, labels, (const float *)grad->ptr, grad->strideBytes,
         (float *)delta->ptr, delta->strideBytes);
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
+int Ts2FinalSoftmaxGradHalf(int rows, int vocab, const ts2_mat *logits, const float *bias, const int *target, float gradMult, const ts2_mat *grad,
+    float *lossSum, void *stream)
+{
+    if (vocab % 8 || (logits->strideBytes & 15) || (grad->strideBytes & 15) || ((uintptr_t)logits->ptr & 15) || ((uintptr_t)grad->ptr & 15) ||
+        ((uintptr_t)bias & 15)) {
+        return TS2_ERR_ALIGN;
+    }
+    hipLaunchKernelGGL(FinalSoftmaxGradHalf, dim3(rows), dim3(256), 0, STREAM, vocab, (const _Float16 *)logits->ptr, logits->strideBytes, bias, target,
+        gradMult, (bf16_t *)grad->ptr, grad->strideBytes, lossSum);
     TS2_CHECK_LAUNCH();
     return TS2_OK;
 }

@@ -6,7 +6,7 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 SO = os.path.join(HERE, "libts2amd.so")
 
-I8, E4M3, BF16, F32, I32 = 0, 1, 2, 3, 4
+I8, E4M3, BF16, F32, I32, F16 = 0, 1, 2, 3, 4, 5
 EPI_STORE, EPI_ADD, EPI_ROW_TILE_MAXNORM, EPI_ROW_TILE_NORM = 0, 1, 2, 3
 
 
