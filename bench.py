@@ -141,7 +141,7 @@ def bench_linear_i8(args):
            "roofline": roof}
     roof["device_sustained"] = sustained(L.I8)
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline_linear(len_, src_dim, grad_dim, 2048)
+        out["cpu_baseline"] = cpu_baseline_linear(len_, src_dim, grad_dim, 4096)
     return out
 
 
