@@ -1029,6 +1029,17 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(256, 1) G
             if (NDS) __builtin_amdgcn_sched_group_barrier(0x100, NDS, 0);                                                                  \
         }                                                                                                                                  \
     } while (0)
+    // End of a step: this wave's loads except the newest LA (A of step S+2) have landed and its LDS reads have returned
+    // (vmcnt(LA) lgkmcnt(0)), then the workgroup barrier.  Not __syncthreads(): its fence makes the compiler drain every load in
+    // flight (vmcnt(0)) before the barrier, which would shorten the lookahead of A to one step.  The empty statements that
+    // clobber memory keep the compiler from moving LDS accesses across the barrier.
+#define RING_BARRIER()                                                                                                                     \
+    do {                                                                                                                                   \
+        __builtin_amdgcn_s_waitcnt(0x0070 | LA);                                                                                           \
+        asm volatile("" ::: "memory");                                                                                                     \
+        __builtin_amdgcn_s_barrier();                                                                                                      \
+        asm volatile("" ::: "memory");                                                                                                     \
+    } while (0)
     // one K step on stage (CA, CB); (NA1, NB) is the stage of step S+1, NA2 the A stage of step S+2
 #define STEP(CA, CB, NA1, NB, NA2, S)                                                                                                      \
     do {                                                                                                                                   \
@@ -1061,8 +1072,7 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(256, 1) G
             MFMA_ROWS(1, 0, WTM / 2);                                                                                                      \
         }                                                                                                                                  \
         __builtin_amdgcn_sched_barrier(0);                                                                                                 \
-        __builtin_amdgcn_s_waitcnt(0x0F70 | LA); /* vmcnt(LA): everything but A of step S+2 has landed */                                  \
-        __syncthreads();                                                                                                                   \
+        RING_BARRIER(); /* everything but A of step S+2 has landed, in every wave */                                                      \
         LOAD_FRAGS(0, NA1, NB, 0);                                                                                                         \
         __builtin_amdgcn_sched_barrier(0);                                                                                                 \
         MFMA_ROWS(1, WTM / 2, WTM);                                                                                                        \
@@ -1081,8 +1091,7 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(256, 1) G
         RING_LOAD_A(sA0, 0, 0, LA);
         RING_LOAD_B(sB0, 0, 0, LB);
         RING_LOAD_A(sA1, 1, 0, LA);
-        __builtin_amdgcn_s_waitcnt(0x0F70 | LA);
-        __syncthreads();
+        RING_BARRIER();
         LOAD_FRAGS(0, sA0, sB0, 0);
         int s = 0;
         for (; s + 6 <= kSteps; s += 6) {
@@ -1147,6 +1156,7 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(256, 1) G
         p.alphaPtr = lastPtr;
     }
 #undef STEP
+#undef RING_BARRIER
 #undef INTERLEAVE
 #undef LOAD_FRAGS
 #undef MFMA_ROWS
