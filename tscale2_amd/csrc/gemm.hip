@@ -1166,6 +1166,215 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(256, 1) G
     Epilogue<TYPE, WTM, WTN, CT, EPI, false>(p, acc, facc, sA0, rowBase, colBase, wm, wn, half, l32);
 }
 
+// ---------------------------------------------------------------------------------------------------------------------------
+// Three stages of both operands for the tiles that leave room for them (256x128: 144 KB): the loads issued during step S are those
+// of step S+2, one at a time between the MFMAs, and "all but the newest LA+LB" at the end of a step means step S+1 has landed.  Same
+// conventions as GemmNTRing (plain barrier with explicit waits, steps past the end reload the last one, separate static stage
+// arrays, three steps per loop iteration).  Carries the k-tile-scaled second accumulator set like GemmNTDirect; WM x WN waves.
+template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT, int WM, int WN>
+__global__ void __launch_bounds__(64 * WM * WN, (WM * WN) / 4) GemmNTRing3(GemmP p)
+{
+    typedef typename AccT<TYPE>::type TAcc;
+    constexpr int NW = WM * WN;
+    constexpr int BM = 32 * WTM * WM, BN = 32 * WTN * WN;
+    __shared__ __attribute__((aligned(1024))) uint8_t sA0[BM * BKB];
+    __shared__ __attribute__((aligned(1024))) uint8_t sA1[BM * BKB];
+    __shared__ __attribute__((aligned(1024))) uint8_t sA2[BM * BKB];
+    __shared__ __attribute__((aligned(1024))) uint8_t sB0[BN * BKB];
+    __shared__ __attribute__((aligned(1024))) uint8_t sB1[BN * BKB];
+    __shared__ __attribute__((aligned(1024))) uint8_t sB2[BN * BKB];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN;
+    const int wn = wave % WN;
+    int tm, tn;
+    MapTile(blockIdx.x, p.tilesM * p.tilesN, p.tilesM, p.tilesN, &tm, &tn, p.mapGroup ? p.mapGroup : 8);
+    const int rowBase = tm * BM;
+    const int colBase = tn * BN;
+    int kSteps = p.kBytes / BKB;
+    int kBeg = 0;
+    if (p.splits > 1) {
+        int per = (kSteps + p.splits - 1) / p.splits;
+        kBeg = blockIdx.y * per;
+        kSteps = kSteps - kBeg < per ? kSteps - kBeg : per;
+        kSteps = kSteps < 0 ? 0 : kSteps;
+        p.c += (int64_t)blockIdx.y * p.splitSlab;
+    }
+    const int lrow = wave * 8 + (lane >> 3);
+    const int lchunk = (lane & 7) ^ ((lrow >> 1) & 7);
+    const uint8_t *gaTile = p.a + (int64_t)rowBase * p.lda + (int64_t)kBeg * BKB;
+    const uint8_t *gbTile = p.b + (int64_t)colBase * p.ldb + (int64_t)kBeg * BKB;
+    const uint32_t gaLane = (uint32_t)(lrow * (int)p.lda + lchunk * 16);
+    const uint32_t gbLane = (uint32_t)(lrow * (int)p.ldb + lchunk * 16);
+    constexpr int LA = BM / (8 * NW);
+    constexpr int LB = BN / (8 * NW);
+    constexpr int LT = LA + LB;
+    const int lastStep = kSteps - 1;
+    // loads I0..I1-1 of the LT loads of a step: the first LA fill the A stage, the others the B stage
+#define RING_LOADS(SA, SB, STEP, I0, I1)                                                                                                   \
+    do {                                                                                                                                   \
+        const int st_ = (STEP) < lastStep ? (STEP) : lastStep;                                                                             \
+        _Pragma("unroll") for (int i = I0; i < (I1 < LT ? I1 : LT); ++i)                                                                   \
+        {                                                                                                                                  \
+            if (i < LA) {                                                                                                                  \
+                __builtin_amdgcn_global_load_lds(TS2_GLB_PTR(gaTile + ((int64_t)i * (8 * NW) * p.lda + (int64_t)st_ * BKB) + gaLane),      \
+                    TS2_LDS_PTR(SA + (wave + NW * i) * 1024), 16, 0, 0);                                                                   \
+            } else {                                                                                                                       \
+                __builtin_amdgcn_global_load_lds(TS2_GLB_PTR(gbTile + ((int64_t)(i - LA) * (8 * NW) * p.ldb + (int64_t)st_ * BKB) + gbLane), \
+                    TS2_LDS_PTR(SB + (wave + NW * (i - LA)) * 1024), 16, 0, 0);                                                            \
+            }                                                                                                                              \
+        }                                                                                                                                  \
+    } while (0)
+
+    TAcc acc[WTM][WTN];
+    v16f facc[KT ? WTM : 1][KT ? WTN : 1];
+#pragma unroll
+    for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+        for (int j = 0; j < WTN; ++j) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                acc[i][j][e] = 0;
+            }
+        }
+    }
+    if (KT) {
+#pragma unroll
+        for (int i = 0; i < (KT ? WTM : 1); ++i) {
+#pragma unroll
+            for (int j = 0; j < (KT ? WTN : 1); ++j) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    facc[i][j][e] = 0;
+                }
+            }
+        }
+    }
+    const int half = lane >> 5;
+    const int l32 = lane & 31;
+    const int aRow0 = wm * (32 * WTM) + l32;
+    const int bRow0 = wn * (32 * WTN) + l32;
+    constexpr int NS = TYPE == T_FP8 ? 2 : 4;
+    constexpr int ND = (WTM + WTN) * (TYPE == T_FP8 ? 2 : 1); // ds_read_b128 per fragment set
+    constexpr int NM = WTM * WTN;                             // MFMAs per K slice
+    constexpr int PER = (LT + NS - 2) / (NS - 1);             // loads issued per K slice (all but the last slice carry loads)
+    typedef typename std::conditional<TYPE == T_FP8, v8i, v4i>::type TFrag;
+    TFrag fa[2][WTM], fb[2][WTN];
+    auto loadOne = [&](const uint8_t *base, int row, int sl) -> TFrag {
+        if constexpr (TYPE == T_FP8) {
+            int ch = sl * 4 + half * 2;
+            v4i lo = *(const v4i *)(base + SwizzleOffset(row, ch));
+            v4i hi = *(const v4i *)(base + SwizzleOffset(row, ch + 1));
+            return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        } else {
+            return *(const v4i *)(base + SwizzleOffset(row, sl * 2 + half));
+        }
+    };
+    auto mfma = [&](TFrag a, TFrag b, TAcc c) -> TAcc {
+        if constexpr (TYPE == T_I8) {
+            return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+        } else if constexpr (TYPE == T_FP8) {
+            return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+        } else {
+            return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+        }
+    };
+#define LOAD_FRAGS(SET, SA, SB, SL)                                                                                                        \
+    do {                                                                                                                                   \
+        _Pragma("unroll") for (int i = 0; i < WTM; ++i) fa[SET][i] = loadOne(SA, aRow0 + 32 * i, SL);                                      \
+        _Pragma("unroll") for (int j = 0; j < WTN; ++j) fb[SET][j] = loadOne(SB, bRow0 + 32 * j, SL);                                      \
+    } while (0)
+#define MFMA_ROWS(SET, I0, I1)                                                                                                             \
+    do {                                                                                                                                   \
+        _Pragma("unroll") for (int i = I0; i < I1; ++i) _Pragma("unroll") for (int j = 0; j < WTN; ++j) acc[i][j] =                        \
+            mfma(fa[SET][i], fb[SET][j], acc[i][j]);                                                                                       \
+    } while (0)
+    // PER groups of (MFMAs, one load, LDS reads)
+#define INTERLEAVE()                                                                                                                       \
+    do {                                                                                                                                   \
+        _Pragma("unroll") for (int q = 0; q < PER; ++q)                                                                                    \
+        {                                                                                                                                  \
+            __builtin_amdgcn_sched_group_barrier(0x008, (NM + PER - 1) / PER, 0);                                                          \
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                                                                             \
+            __builtin_amdgcn_sched_group_barrier(0x100, (ND + PER - 1) / PER, 0);                                                          \
+        }                                                                                                                                  \
+    } while (0)
+#define RING_BARRIER()                                                                                                                     \
+    do {                                                                                                                                   \
+        __builtin_amdgcn_s_waitcnt(0x0070 | LT); /* vmcnt(LT) lgkmcnt(0): everything but step S+2 has landed */                            \
+        asm volatile("" ::: "memory");                                                                                                     \
+        __builtin_amdgcn_s_barrier();                                                                                                      \
+        asm volatile("" ::: "memory");                                                                                                     \
+    } while (0)
+    const int tileSteps = KT ? p.kTileBytes / BKB : 0;
+    // one K step on stage (CA, CB); (NA, NB) is the stage of step S+1, (FA, FB) the one that receives step S+2
+#define STEP(CA, CB, NA, NB, FA, FB, S)                                                                                                    \
+    do {                                                                                                                                   \
+        _Pragma("unroll") for (int sl = 0; sl < NS - 1; ++sl)                                                                              \
+        {                                                                                                                                  \
+            RING_LOADS(FA, FB, (S) + 2, sl * PER, (sl + 1) * PER);                                                                         \
+            if ((sl & 1) == 0) {                                                                                                           \
+                LOAD_FRAGS(1, CA, CB, sl + 1);                                                                                             \
+                MFMA_ROWS(0, 0, WTM);                                                                                                      \
+            } else {                                                                                                                       \
+                LOAD_FRAGS(0, CA, CB, sl + 1);                                                                                             \
+                MFMA_ROWS(1, 0, WTM);                                                                                                      \
+            }                                                                                                                              \
+            INTERLEAVE();                                                                                                                  \
+            __builtin_amdgcn_sched_barrier(0);                                                                                             \
+        }                                                                                                                                  \
+        MFMA_ROWS(1, 0, WTM / 2);                                                                                                          \
+        __builtin_amdgcn_sched_barrier(0);                                                                                                 \
+        RING_BARRIER();                                                                                                                    \
+        LOAD_FRAGS(0, NA, NB, 0);                                                                                                          \
+        __builtin_amdgcn_sched_barrier(0);                                                                                                 \
+        MFMA_ROWS(1, WTM / 2, WTM);                                                                                                        \
+        if (KT) {                                                                                                                          \
+            if ((kBeg + (S) + 1) % tileSteps == 0 || (S) + 1 == kSteps) {                                                                  \
+                float sc = p.kTileScale[(kBeg + (S)) / tileSteps];                                                                         \
+                _Pragma("unroll") for (int i = 0; i < (KT ? WTM : 1); ++i) _Pragma("unroll") for (int j = 0; j < (KT ? WTN : 1); ++j)      \
+                    _Pragma("unroll") for (int e = 0; e < 16; ++e)                                                                         \
+                {                                                                                                                          \
+                    facc[i][j][e] += sc * (float)acc[i][j][e];                                                                             \
+                    acc[i][j][e] = 0;                                                                                                      \
+                }                                                                                                                          \
+            }                                                                                                                              \
+        }                                                                                                                                  \
+    } while (0)
+
+    static_assert(LT <= 15, "vmcnt immediate");
+    if (kSteps > 0) {
+        RING_LOADS(sA0, sB0, 0, 0, LT);
+        RING_LOADS(sA1, sB1, 1, 0, LT);
+        RING_BARRIER();
+        LOAD_FRAGS(0, sA0, sB0, 0);
+        int s = 0;
+        for (; s + 3 <= kSteps; s += 3) {
+            STEP(sA0, sB0, sA1, sB1, sA2, sB2, s);
+            STEP(sA1, sB1, sA2, sB2, sA0, sB0, s + 1);
+            STEP(sA2, sB2, sA0, sB0, sA1, sB1, s + 2);
+        }
+        const int rem = kSteps - s;
+        if (rem > 0) {
+            STEP(sA0, sB0, sA1, sB1, sA2, sB2, s);
+        }
+        if (rem > 1) {
+            STEP(sA1, sB1, sA2, sB2, sA0, sB0, s + 1);
+        }
+    }
+#undef STEP
+#undef RING_BARRIER
+#undef INTERLEAVE
+#undef LOAD_FRAGS
+#undef MFMA_ROWS
+#undef RING_LOADS
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    Epilogue<TYPE, WTM, WTN, CT, EPI, KT>(p, acc, facc, sA0, rowBase, colBase, wm, wn, half, l32);
+}
+
 template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT> int Launch(const GemmP &p, hipStream_t stream)
 {
     constexpr int BM = 64 * WTM, BN = 64 * WTN;
@@ -1258,8 +1467,13 @@ template <int TYPE, int WTM, int WTN> int DispatchEpi(const ts2_gemm_args *a, co
                 int nb = q.tilesM * q.tilesN;
                 int chunk = (nb % 8) == 0 ? nb / 8 : nb;
                 q.mapGroup = p.mapGroup ? p.mapGroup : chunk >= 64 ? 8 : chunk >= 8 ? 4 : 2;
-                hipLaunchKernelGGL((GemmNTDirect<TYPE, 2, 2, C_F32, TS2_EPI_STORE, true, 4, 2>), dim3(nb, p.splits > 1 ? p.splits : 1), dim3(512), 0,
-                    stream, q);
+                if (p.noRing) {
+                    hipLaunchKernelGGL((GemmNTDirect<TYPE, 2, 2, C_F32, TS2_EPI_STORE, true, 4, 2>), dim3(nb, p.splits > 1 ? p.splits : 1), dim3(512),
+                        0, stream, q);
+                } else {
+                    hipLaunchKernelGGL((GemmNTRing3<TYPE, 2, 2, C_F32, TS2_EPI_STORE, true, 4, 2>), dim3(nb, p.splits > 1 ? p.splits : 1), dim3(512),
+                        0, stream, q);
+                }
                 TS2_CHECK_LAUNCH();
                 return TS2_OK;
             }
