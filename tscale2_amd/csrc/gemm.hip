@@ -191,8 +191,10 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
                     const int row = rowBase + rowLocal(i, e);
                     float discr = 0;
                     if (sum2[e] > 0 && row < mLive) {
-                        discr = sqrtf(sum2[e] / TILE) * p.vecScale;
-                        float inv = 1 / discr;
+                        // hardware square root and reciprocal (1 ulp each): every lane of the group repeats this per row, and the
+                        // correctly rounded sequences were most of the epilogue's instructions
+                        discr = __builtin_amdgcn_sqrtf(sum2[e] * (1.f / TILE)) * p.vecScale;
+                        float inv = __builtin_amdgcn_rcpf(discr);
 #pragma unroll
                         for (int j = 0; j < WTN; ++j) {
                             out[j][e] *= inv;
