@@ -191,6 +191,31 @@ def test_row_max_quantise(L, orc):
     np.testing.assert_array_equal(dst.cpu().numpy()[:len_], want)
 
 
+@pytest.mark.parametrize("dim,col_scale", [(512, False), (1536, True), (4096, True)])
+def test_row_max_quantise_of_bf16_rows_by_one_wave_per_row(L, orc, dim, col_scale):
+    """bf16 rows whose length is a multiple of 512 (up to 4096) take the wave-per-row kernel: bytes, row scales and row maxima must
+    equal the oracle's on the same bf16 values, with and without column scales; pad rows are cleared."""
+    print("case rowmax bf16 wave", dim, col_scale, flush=True)
+    r = np.random.default_rng(dim)
+    len_, len_round = 9000, 9216                       # more rows than waves in the launch: with column scales a wave walks several rows
+    x16 = torch.from_numpy((r.standard_normal((len_, dim)) * r.random((len_, 1)) * 5).astype(np.float32)).bfloat16()
+    x16[11] = 0
+    cs = (r.random(dim) + 0.5).astype(np.float32) if col_scale else None
+    x = x16.float().numpy()
+    xs = x * cs[None, :] if col_scale else x
+    want = np.zeros((len_, dim), np.int8); wscale = np.zeros(len_, np.float32)
+    orc.lib.orc_quant_rowmax_i8(_ptr(np.ascontiguousarray(xs)), _ptr(want), _ptr(wscale), len_, dim)
+    dst = torch.full((len_round, dim), 3, dtype=torch.int8, device="cuda")
+    rs = torch.full((len_round,), -1.0, device="cuda")
+    rmax = torch.full((len_round,), -1.0, device="cuda")
+    L.call("ts2_normalize_vecs_row_max2", len_, len_round, x16.cuda().view(torch.int16), L.BF16, dev(cs) if col_scale else None, dst, rs, rmax)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(rs.cpu().numpy()[:len_], wscale)
+    np.testing.assert_array_equal(dst.cpu().numpy()[:len_], want)
+    np.testing.assert_array_equal(rmax.cpu().numpy()[:len_], np.abs(x).max(1))
+    assert np.all(rs.cpu().numpy()[len_:] == 0) and np.all(dst.cpu().numpy()[len_:] == 0) and np.all(rmax.cpu().numpy()[len_:] == 0)
+
+
 def test_transpose_and_ktile_quant(L, orc):
     print("case transpose", flush=True)
     r = np.random.default_rng(6)
