@@ -212,3 +212,47 @@ def test_delta_from_shared_row_maxima_is_identical(L, orc):
         res.append((b.delta.cpu().numpy(), b.delta_tile_scale.cpu().numpy(), b.t["tileScale"].cpu().numpy()))
     for a, c in zip(*res):
         np.testing.assert_array_equal(a, c)
+
+
+@pytest.mark.parametrize("mode", ["e4m3", "i8"])
+def test_grouped_backprop_equals_the_products_added_one_after_the_other(L, orc, mode):
+    """ts2_matmul_backprop_group over four matrices that share their input against four Backprop() calls (store, then accumulate).
+    fp8 on the 256 grid runs as one launch (same fp32 MFMA sums, rescaled between products, one rounding of the total: a few ulps of
+    the largest partial sum); int8 falls back to the sequence itself and must be identical."""
+    print("case grouped dX", mode, flush=True)
+    from tscale2_amd import lib as LL
+    len_, src_dim, grad_dim, n = 700, 512, 256, 4
+    len_round = 768
+    r = np.random.default_rng(31)
+    m = L.E4M3 if mode == "e4m3" else L.I8
+    bufs, grads, scales = [], [], []
+    for i in range(n):
+        w = (r.standard_normal((grad_dim, src_dim)) * 20).astype(np.float32)
+        dy = (r.standard_normal((len_round, grad_dim)) * (0.3 + r.random((len_round, 1)))).astype(np.float32)
+        dy[len_:] = 0
+        if mode == "e4m3":
+            wf = (torch.from_numpy(w).cuda()).to(torch.float8_e4m3fn).view(torch.uint8)
+            g = (torch.from_numpy(dy).cuda() * 16).to(torch.float8_e4m3fn).view(torch.uint8)
+            gt = L.E4M3
+        else:
+            wf = torch.from_numpy(np.clip(np.rint(w), -127, 127).astype(np.int8)).cuda()
+            g = torch.from_numpy(dy).bfloat16().cuda().view(torch.int16)
+            gt = L.BF16
+        b = L.MatMulBuffers(m, len_round, src_dim, grad_dim)
+        b.backprop_multi(len_, wf, g, gt)
+        bufs.append(b); grads.append(g)
+        scales.append(None if i == 3 else torch.full((1,), 0.6 + 0.3 * i, device="cuda"))
+    alphas = [0.01 * (i + 1) for i in range(n)]
+    c0 = torch.randn((len_round, src_dim), device="cuda")
+    for add in (False, True):
+        want = c0.clone()
+        for i in range(n):
+            bufs[i].backprop(len_, grads[i] if mode == "e4m3" else None, alphas[i], scales[i], want, L.F32, add=add or i > 0)
+        got = c0.clone()
+        LL.matmul_backprop_group(bufs, len_, grads if mode == "e4m3" else [None] * n, alphas, scales, got, L.F32, add=add)
+        torch.cuda.synchronize()
+        if mode == "i8":
+            assert torch.equal(got, want)
+        else:
+            scale = want[:len_].abs().max().item()
+            assert (got[:len_] - want[:len_]).abs().max().item() <= 4e-6 * scale

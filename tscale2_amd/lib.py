@@ -214,6 +214,24 @@ class MatMulBuffers:
         return self.delta.float() * sc
 
 
+def matmul_backprop_group(bufs, len_, grads, alphas, alpha_ptrs, src_grad, src_grad_type, add=False, check=True):
+    """ts2_matmul_backprop_group over MatMulBuffers objects of equal shape whose backprop_multi has run: src_grad (+)= sum of the products"""
+    lib = load()
+    n = len(bufs)
+    b0 = bufs[0]
+    gm = [mat(g) if g is not None else Mat(None, 0, 0, 0) for g in grads]
+    gp = (C.POINTER(Mat) * n)(*[C.pointer(m) for m in gm])
+    bp = (C.POINTER(BwdBuffers) * n)(*[C.pointer(b.c) for b in bufs])
+    al = (C.c_float * n)(*[float(a) for a in alphas])
+    ap = (C.c_void_p * n)(*[None if p is None else p.data_ptr() for p in alpha_ptrs])
+    sg = mat(src_grad)
+    rc = lib.dll.ts2_matmul_backprop_group(C.c_int32(b0.mode), C.c_int32(len_), C.c_int32(b0.len_round), C.c_int32(b0.src_dim), C.c_int32(b0.grad_dim),
+                                           C.c_int32(n), gp, bp, al, ap, C.byref(sg), C.c_int32(src_grad_type), C.c_int32(int(add)), lib.stream())
+    if check:
+        lib.check(rc, "ts2_matmul_backprop_group")
+    return rc
+
+
 class AttArgs(C.Structure):
     _fields_ = [("len", C.c_int32), ("lenRound", C.c_int32), ("heads", C.c_int32), ("q", Mat), ("k", Mat), ("v", Mat),
                 ("spanStart", C.c_void_p), ("spanFinish", C.c_void_p), ("attDotScale", C.c_float), ("alibiSlope", C.c_float),
