@@ -135,6 +135,23 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
         }
     };
     auto rowLocal = [&](int i, int e) { return wm * (32 * WTM) + i * 32 + (e >> 2) * 8 + half * 4 + (e & 3); };
+    // scale of every row of the wave's tile, fetched up front (four consecutive rows per load): one dependent load per row inside
+    // the store loops cost the row-scaled product about 10 us per launch
+    float rsAll[WTM][16];
+#pragma unroll
+    for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            float4 r = make_float4(1.f, 1.f, 1.f, 1.f);
+            if (p.rowScale) {
+                r = *(const float4 *)(p.rowScale + rowBase + rowLocal(i, q * 4));
+            }
+            rsAll[i][q * 4 + 0] = scale * r.x;
+            rsAll[i][q * 4 + 1] = scale * r.y;
+            rsAll[i][q * 4 + 2] = scale * r.z;
+            rsAll[i][q * 4 + 3] = scale * r.w;
+        }
+    }
 
     if constexpr (CT == C_BF16NORM) {
         // TStoreRowTileNormalize / TStoreRowTileNormalizeRope (src/lib/cuda/cuda_matmul.cuh:495-525, src/gpt/compute/gpu_rope.cuh:25-60):
@@ -152,10 +169,7 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const int row = rowBase + rowLocal(i, e);
-                float rs = scale;
-                if (p.rowScale) {
-                    rs *= p.rowScale[row];
-                }
+                float rs = rsAll[i][e];
                 sum2[e] = 0;
 #pragma unroll
                 for (int j = 0; j < WTN; ++j) {
@@ -303,10 +317,7 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
             for (int e = 0; e < 16; ++e) {
                 const int rl = rowLocal(i, e);
                 const int row = rowBase + rl;
-                float rs = scale;
-                if (p.rowScale) {
-                    rs *= p.rowScale[row];
-                }
+                float rs = rsAll[i][e];
                 float mx = mxs[e] * fabsf(rs);
                 float discr = 0, mult = 0;
                 if (mx > 0 && row < mLive) {
@@ -360,10 +371,7 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
                         const int row = rowOf(ch, r);
                         if (row < mLive) {
                             uint8_t *dst = p.c + (int64_t)row * p.ldc;
-                            float rs = scale;
-                            if (p.rowScale) {
-                                rs *= p.rowScale[row];
-                            }
+                            const float rs = rsAll[ch >> 1][(ch & 1) * 8 + r];
 #pragma unroll
                             for (int j = 0; j < WTN; ++j) {
                                 const int col = colBase + wn * (32 * WTN) + j * 32 + l32;
@@ -391,11 +399,7 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
                     float v[16];
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
-                        float rs = scale;
-                        if (p.rowScale) {
-                            rs *= p.rowScale[rowBase + rowLocal(i, e)];
-                        }
-                        v[e] = accVal(i, j, e) * rs;
+                        v[e] = accVal(i, j, e) * rsAll[i][e];
                     }
                     StoreBlockBf16<CT == C_F16>(p.c, p.ldc, col, l32, mLive, v, [&](int e) { return rowBase + rowLocal(i, e); });
                 }
@@ -425,10 +429,7 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
                         const int row = rowBase + rowLocal(i, e);
                         const bool live = row < mLive;
                         uint8_t *dst = p.c + (int64_t)row * p.ldc;
-                        float rs = scale;
-                        if (p.rowScale) {
-                            rs *= p.rowScale[row];
-                        }
+                        float rs = rsAll[i][e];
 #pragma unroll
                         for (int j = 0; j < WTN; ++j) {
                             const int col = colBase + wn * (32 * WTN) + j * 32 + l32;
@@ -1565,6 +1566,9 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
     }
     if (a->a.y < a->m || a->b.y < a->n || a->a.x < a->k || a->b.x < a->k || a->c.y < a->m || a->c.x < a->n) {
         return TS2_ERR_SHAPE;
+    }
+    if (a->rowScale && (((uintptr_t)a->rowScale) & 15)) {
+        return TS2_ERR_ALIGN; // row scales are fetched four at a time
     }
     if (a->kTileScale && (a->abType != TS2_I8 || a->kTile <= 0 || (a->kTile % 128) || (a->k % a->kTile))) {
         return TS2_ERR_SHAPE;
