@@ -233,6 +233,43 @@ __global__ void __launch_bounds__(256) MatrixLoLU(int len, int lenRound, int til
     }
 }
 
+// The e4m3 result from bf16 inputs with eight elements per lane (16-byte loads, 8-byte stores; no reduction in this kernel, so the
+// tile structure does not matter): the form the model's FFN and attention forward use.  Two row segments per lane in flight.
+__global__ void __launch_bounds__(256) MatrixLoLU8(int len, int lenRound, int dim8, Mat gate, Mat vals, float resMult, Mat res)
+{
+    const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    const long total = (long)lenRound * dim8;
+    const long stride = (long)gridDim.x * 256;
+    uint4 g[2], v[2];
+    long id[2];
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        id[k] = idx + k * stride;
+        const int t = (int)(id[k] / dim8), c = (int)(id[k] - (long)t * dim8) * 8;
+        const bool live = id[k] < total && t < len;
+        g[k] = live ? *(const uint4 *)At<TBF16>(gate, t, c) : make_uint4(0, 0, 0, 0);
+        v[k] = live ? *(const uint4 *)At<TBF16>(vals, t, c) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        if (id[k] >= total) {
+            continue;
+        }
+        const int t = (int)(id[k] / dim8), c = (int)(id[k] - (long)t * dim8) * 8;
+        const uint32_t gw[4] = {g[k].x, g[k].y, g[k].z, g[k].w}, vw[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+        uint32_t out[2] = {0, 0};
+        if (t < len) {
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                float g0 = __uint_as_float(gw[w] << 16), g1 = __uint_as_float(gw[w] & 0xffff0000u);
+                float v0 = __uint_as_float(vw[w] << 16), v1 = __uint_as_float(vw[w] & 0xffff0000u);
+                out[w >> 1] |= CvtPkE4m3(v0 * LoLU1(g0) * resMult, v1 * LoLU1(g1) * resMult) << ((w & 1) * 16);
+            }
+        }
+        *(uint2 *)At<TE4M3>(res, t, c) = make_uint2(out[0], out[1]);
+    }
+}
+
 // MODE 0: FFN (tile-norm backward of vals fused); MODE 1: attention (dScale fused)
 template <class TGrad, class TOutG, class TOutV, int MODE>
 __global__ void __launch_bounds__(256) BackpropLoLU(int len, int lenRound, int tiles, Mat gate, Mat vals, float valsScale, Mat valsSrcTileScale,
@@ -927,6 +964,14 @@ extern "C" int ts2_matrix_lolu(int32_t len, int32_t lenRound, const ts2_mat *gat
         return TS2_ERR_SHAPE;
     }
     int tiles = dim / TILE;
+    if (resType == TS2_E4M3 && Aligned16(gate->ptr, gate->strideBytes) && Aligned16(vals->ptr, vals->strideBytes) &&
+        (((uintptr_t)res->ptr | res->strideBytes) & 7) == 0) {
+        const long lanes = ((long)lenRound * (dim / 8) + 1) / 2;
+        hipLaunchKernelGGL(MatrixLoLU8, dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, STREAM, len, lenRound, dim / 8, M(*gate), M(*vals),
+            resMult, M(*res));
+        TS2_CHECK_LAUNCH();
+        return TS2_OK;
+    }
     TS2_DISPATCH_TYPE(resType, TD,
         hipLaunchKernelGGL((MatrixLoLU<TD>), GridFor(lenRound, tiles), dim3(256), 0, STREAM, len, lenRound, tiles, M(*gate), M(*vals), resMult,
             M(*res)));
