@@ -174,6 +174,48 @@ def test_lolu_forward_backward(L, orc):
     assert np.all(ds.cpu().numpy()[:, len_:] == 0)
 
 
+def test_ffn_lolu_backward_and_forward_with_eight_elements_per_lane(L, orc):
+    """bf16 gradient in, e4m3 gradients out (the model's fp8 FFN backward) and the e4m3 forward take the kernels with eight elements
+    per lane: compared with the oracle on the same bf16 inputs, within the e4m3 rounding (2^-4 relative, half a denormal step
+    absolute), pad rows zero; odd row counts and a tile count that leaves half-filled waves."""
+    print("case lolu e4m3 8-wide", flush=True)
+    r = np.random.default_rng(14)
+    len_, len_round, dim = 301, 384, 384
+    gate = torch.from_numpy((r.standard_normal((len_, dim)) * 2).astype(np.float32)).bfloat16()
+    vals = torch.from_numpy((r.standard_normal((len_, dim)) * 24).astype(np.float32)).bfloat16()
+    grad = torch.from_numpy((r.standard_normal((len_, dim)) * 8).astype(np.float32)).bfloat16()
+    gnp, vnp, dnp = gate.float().numpy(), vals.float().numpy(), grad.float().numpy()
+    vs = 1 / 24.0
+    tsc = (r.random((dim // 128, len_)) + 0.5).astype(np.float32) * np.float32(vs)
+    tsc[1, 7] = 0                                                     # a zero tile: zero source, zero gradient
+    vnp_z = vnp.copy(); vnp_z[7, 128:256] = 0
+    vals = torch.from_numpy(vnp_z).bfloat16()
+    wide_norm = vnp_z * np.float32(vs)
+    wide = vnp_z * np.repeat(tsc.T, 128, axis=1)
+    dgate, dvals = orc.backprop_lolu(gnp, wide_norm, dnp)
+    dwide = orc.normalize_state_backward(wide, dvals, dim // 128)
+    gg = torch.full((len_round, dim), 9, dtype=torch.uint8, device="cuda")
+    gv = torch.full((len_round, dim), 9, dtype=torch.uint8, device="cuda")
+    L.call("ts2_backprop_row_tile_normalize_lolu", len_, len_round, gate.cuda().view(torch.int16), vals.cuda().view(torch.int16), vs, dev(tsc),
+           grad.cuda().view(torch.int16), L.BF16, gg, gv, L.E4M3)
+    torch.cuda.synchronize()
+    got_g, got_v = gg.view(torch.float8_e4m3fn).float().cpu().numpy(), gv.view(torch.float8_e4m3fn).float().cpu().numpy()
+    for name, got, want in (("dgate", got_g, dgate), ("dwide", got_v, dwide)):
+        assert np.all(got[len_:] == 0)
+        excess = np.abs(got[:len_] - np.clip(want, -448, 448)) - (np.abs(want) * 2.0 ** -4 + 2.0 ** -10 * 1.01)
+        i = np.unravel_index(np.argmax(excess), excess.shape)
+        assert excess[i] <= 0, (name, i, got[:len_][i], want[i])
+    assert np.all(got_v[7, 128:256] == 0)
+    # forward with the e4m3 result
+    res = torch.full((len_round, dim), 9, dtype=torch.uint8, device="cuda")
+    L.call("ts2_matrix_lolu", len_, len_round, gate.cuda().view(torch.int16), vals.cuda().view(torch.int16), 0.5, res, L.E4M3)
+    torch.cuda.synchronize()
+    want = orc.lolu(gnp, vnp_z) * 0.5
+    got = res.view(torch.float8_e4m3fn).float().cpu().numpy()
+    assert np.all(got[len_:] == 0)
+    assert np.all(np.abs(got[:len_] - np.clip(want, -448, 448)) <= np.abs(want) * 2.0 ** -4 + 2.0 ** -10 * 1.01)
+
+
 def test_row_max_quantise(L, orc):
     print("case rowmax", flush=True)
     r = np.random.default_rng(5)

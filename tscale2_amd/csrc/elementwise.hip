@@ -320,6 +320,90 @@ __global__ void __launch_bounds__(256) BackpropLoLU(int len, int lenRound, int t
     }
 }
 
+// The FFN flavour (MODE 0) for bf16 gradients and e4m3 results with eight elements per lane: a 128-wide tile is 16 lanes, so a wave
+// holds four (row, tile) units, the tile sums are four DPP steps inside a row of 16 lanes, loads are 16 bytes and stores 8.  Two
+// units per lane in flight.  Same arithmetic per element as BackpropLoLU<.., 0>.
+__device__ __forceinline__ float Row16Sum(float v)
+{
+    v += LaneDpp<DPP_XOR1>(v);
+    v += LaneDpp<DPP_XOR2>(v);
+    v += LaneDpp<DPP_HALF_MIRROR>(v);
+    v += LaneDpp<DPP_MIRROR>(v);
+    return v;
+}
+
+__global__ void __launch_bounds__(256) BackpropLoLU8(int len, int lenRound, int tiles, Mat gate, Mat vals, float valsScale, Mat valsSrcTileScale,
+    Mat gradArr, Mat gradGate, Mat gradVals)
+{
+    constexpr int UU = 2;
+    const int l16 = threadIdx.x & 15;
+    const long unit0 = ((long)blockIdx.x * 256 + threadIdx.x) >> 4; // (row, tile) units; consecutive units = consecutive tiles of a row
+    const long units = (long)lenRound * tiles;
+    const long stride = ((long)gridDim.x * 256) >> 4;
+    uint4 g[UU], v[UU], gr[UU];
+    float ts[UU];
+    int row[UU], col[UU];
+    bool any[UU], live[UU];
+#pragma unroll
+    for (int k = 0; k < UU; ++k) {
+        long u = unit0 + k * stride;
+        any[k] = u < units;
+        row[k] = any[k] ? (int)(u / tiles) : 0;
+        int tile = any[k] ? (int)(u - (long)row[k] * tiles) : 0;
+        col[k] = tile * TILE + l16 * 8;
+        live[k] = any[k] && row[k] < len;
+        g[k] = live[k] ? *(const uint4 *)At<TBF16>(gate, row[k], col[k]) : make_uint4(0, 0, 0, 0);
+        v[k] = live[k] ? *(const uint4 *)At<TBF16>(vals, row[k], col[k]) : make_uint4(0, 0, 0, 0);
+        gr[k] = live[k] ? *(const uint4 *)At<TBF16>(gradArr, row[k], col[k]) : make_uint4(0, 0, 0, 0);
+        ts[k] = live[k] ? ScaleAt(valsSrcTileScale, tile, row[k]) : 0.f;
+    }
+#pragma unroll
+    for (int k = 0; k < UU; ++k) {
+        const uint32_t gw[4] = {g[k].x, g[k].y, g[k].z, g[k].w}, vw[4] = {v[k].x, v[k].y, v[k].z, v[k].w}, rw[4] = {gr[k].x, gr[k].y, gr[k].z, gr[k].w};
+        float resGate[8], resVals[8], src[8];
+        float sum2 = 0, dp = 0;
+        const float srcMult = ts[k] / valsScale;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const uint32_t sh = (e & 1) ? 0xffff0000u : 0u;
+            float ge = (e & 1) ? __uint_as_float(gw[e >> 1] & sh) : __uint_as_float(gw[e >> 1] << 16);
+            float ve = (e & 1) ? __uint_as_float(vw[e >> 1] & sh) : __uint_as_float(vw[e >> 1] << 16);
+            float de = (e & 1) ? __uint_as_float(rw[e >> 1] & sh) : __uint_as_float(rw[e >> 1] << 16);
+            float vv = ve * valsScale;
+            float mult = LoLU1(ge);
+            resGate[e] = de * vv * (mult * (1 - mult) * 2.f);
+            resVals[e] = de * mult;
+            // un-normalised source = normalised * (tile scale / valsScale)
+            src[e] = vv * srcMult;
+            sum2 += src[e] * src[e];
+            dp += src[e] * resVals[e];
+        }
+        sum2 = Row16Sum(sum2);
+        dp = Row16Sum(dp);
+        if (!any[k]) {
+            continue;
+        }
+        uint32_t og[2] = {0, 0}, ov[2] = {0, 0};
+        if (live[k]) {
+            float sigma = 0, scale = 0;
+            if (sum2 != 0) {
+                float inv = 1 / sum2;
+                sigma = dp * inv;
+                scale = sqrtf(TILE * inv);
+            }
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                float a0 = sum2 != 0 ? (resVals[2 * w] - src[2 * w] * sigma) * scale : 0.f;
+                float a1 = sum2 != 0 ? (resVals[2 * w + 1] - src[2 * w + 1] * sigma) * scale : 0.f;
+                ov[w >> 1] |= CvtPkE4m3(a0, a1) << ((w & 1) * 16);
+                og[w >> 1] |= CvtPkE4m3(resGate[2 * w], resGate[2 * w + 1]) << ((w & 1) * 16);
+            }
+        }
+        *(uint2 *)At<TE4M3>(gradGate, row[k], col[k]) = make_uint2(og[0], og[1]);
+        *(uint2 *)At<TE4M3>(gradVals, row[k], col[k]) = make_uint2(ov[0], ov[1]);
+    }
+}
+
 // Workgroups walk rows with a grid stride; a row stays in registers between the abs-max pass and the quantise pass when it has at
 // most 4096 elements (REG) and the next row is fetched before the current one is reduced, so a workgroup always has loads in
 // flight.  Longer rows are read twice (the second read is served by L2).
@@ -999,6 +1083,15 @@ static int BackpropLoluImpl(int len, int lenRound, const ts2_mat *gate, const ts
     Mat ds = MODE == 1 ? M(*dScale) : Mat{nullptr, 0};
     if ((gradType != TS2_BF16 && gradType != TS2_F32) || (ggType != TS2_BF16 && ggType != TS2_E4M3) || (gvType != TS2_BF16 && gvType != TS2_E4M3)) {
         return TS2_ERR_UNSUPPORTED;
+    }
+    if (MODE == 0 && gradType == TS2_BF16 && ggType == TS2_E4M3 && gvType == TS2_E4M3 && Aligned16(gate->ptr, gate->strideBytes) &&
+        Aligned16(vals->ptr, vals->strideBytes) && Aligned16(grad->ptr, grad->strideBytes) &&
+        (((uintptr_t)gradGate->ptr | gradGate->strideBytes | (uintptr_t)gradVals->ptr | gradVals->strideBytes) & 7) == 0) {
+        const long lanes = ((long)lenRound * tiles * 16 + 1) / 2;
+        hipLaunchKernelGGL(BackpropLoLU8, dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, STREAM, len, lenRound, tiles, M(*gate), M(*vals), valsScale,
+            ts, M(*grad), M(*gradGate), M(*gradVals));
+        TS2_CHECK_LAUNCH();
+        return TS2_OK;
     }
 #define LAUNCH_BL(TG, TOG, TOV)                                                                                                            \
     hipLaunchKernelGGL((BackpropLoLU<TG, TOG, TOV, MODE>), GridFor(lenRound, tiles), dim3(256), 0, STREAM, len, lenRound, tiles, M(*gate),  \
