@@ -130,3 +130,30 @@ def test_rope_and_head_norm_passes(L, orc):
     torch.cuda.synchronize()
     # the stored normalised vector is bf16: 2^-8 relative on the source enters the projection
     assert np.abs(out.cpu().numpy()[:n] - want_g).max() <= 1e-2 * np.abs(want_g).max()
+
+
+@pytest.mark.parametrize("with_norm,with_rope", [(True, True), (False, True), (True, False)])
+def test_gradient_epilogue_with_eight_elements_per_lane_equals_the_four_wide_kernel(L, orc, with_norm, with_rope):
+    """bf16 gradient -> e4m3 (the model's attention backward) takes the kernel with eight elements per lane; the same values given
+    as fp32 take the four-wide kernel.  Same arithmetic except the order of the two tile sums: the e4m3 codes agree except for
+    rare neighbours, pad rows are zero; 3 heads leave half-filled waves."""
+    print("case gradient epilogue 8-wide", with_norm, with_rope, flush=True)
+    r = np.random.default_rng(41)
+    n, n_round, heads = 333, 384, 3
+    g16 = torch.from_numpy(r.standard_normal((n, heads * 128)).astype(np.float32) * 4).bfloat16().cuda()
+    sn = torch.from_numpy(r.standard_normal((n, heads * 128)).astype(np.float32)).bfloat16().cuda()
+    sn[5, 128:256] = 0
+    sc = (torch.rand((heads, n), device="cuda") + 0.5).contiguous()
+    rope = torch.from_numpy(orc.fill_rope_buf(128, n_round)).cuda()
+    a = torch.full((n_round, heads * 128), 9, dtype=torch.uint8, device="cuda")
+    b = torch.full((n_round, heads * 128), 9, dtype=torch.uint8, device="cuda")
+    args = (sn.view(torch.int16) if with_norm else None, sc if with_norm else None, rope if with_rope else None)
+    L.call("ts2_backprop_row_tile_normalize_rope", n, n_round, g16.view(torch.int16), L.BF16, 0.75, *args, a, L.E4M3)
+    L.call("ts2_backprop_row_tile_normalize_rope", n, n_round, g16.float().contiguous(), L.F32, 0.75, *args, b, L.E4M3)
+    torch.cuda.synchronize()
+    fa, fb = a.view(torch.float8_e4m3fn).float(), b.view(torch.float8_e4m3fn).float()
+    assert (fa[n:] == 0).all() and (fb[n:] == 0).all()
+    assert (a != b).float().mean().item() < 2e-3
+    assert ((fa - fb).abs() <= fb.abs() * 2.0 ** -3 + 2.0 ** -9).all()
+    if with_norm:
+        assert (fa[5, 128:256] == 0).all()

@@ -876,6 +876,85 @@ __global__ void __launch_bounds__(256) BackpropRowTileNormalizeRope(int len, int
     }
 }
 
+// bf16 gradient -> e4m3 with eight elements per lane (a tile = 16 lanes, the tile sums are four DPP steps, the rotated pairs sit in
+// one lane): the form the model's attention backward uses.  Same arithmetic per element as BackpropRowTileNormalizeRope.
+__global__ void __launch_bounds__(256) BackpropRowTileNormalizeRope8(int len, int lenRound, int tiles, Mat grad, float gradMult, Mat srcNorm,
+    Mat srcTileScale, Mat rope, Mat dst)
+{
+    constexpr int UU = 2;
+    const int l16 = threadIdx.x & 15;
+    const long unit0 = ((long)blockIdx.x * 256 + threadIdx.x) >> 4;
+    const long units = (long)lenRound * tiles;
+    const long stride = ((long)gridDim.x * 256) >> 4;
+    uint4 g[UU], sn[UU];
+    F4 rp[UU][2];
+    float sc[UU];
+    int row[UU], col[UU];
+    bool any[UU], live[UU];
+#pragma unroll
+    for (int k = 0; k < UU; ++k) {
+        long u = unit0 + k * stride;
+        any[k] = u < units;
+        row[k] = any[k] ? (int)(u / tiles) : 0;
+        int tile = any[k] ? (int)(u - (long)row[k] * tiles) : 0;
+        col[k] = tile * TILE + l16 * 8;
+        live[k] = any[k] && row[k] < len;
+        g[k] = live[k] ? *(const uint4 *)At<TBF16>(grad, row[k], col[k]) : make_uint4(0, 0, 0, 0);
+        sn[k] = (live[k] && srcNorm.p) ? *(const uint4 *)At<TBF16>(srcNorm, row[k], col[k]) : make_uint4(0, 0, 0, 0);
+        sc[k] = (live[k] && srcNorm.p) ? ScaleAt(srcTileScale, tile, row[k]) : 0.f;
+        rp[k][0] = (live[k] && rope.p) ? Load4<TF32>(At<TF32>(rope, row[k], l16 * 8)) : ZeroF4();
+        rp[k][1] = (live[k] && rope.p) ? Load4<TF32>(At<TF32>(rope, row[k], l16 * 8 + 4)) : ZeroF4();
+    }
+#pragma unroll
+    for (int k = 0; k < UU; ++k) {
+        const uint32_t gw[4] = {g[k].x, g[k].y, g[k].z, g[k].w}, sw[4] = {sn[k].x, sn[k].y, sn[k].z, sn[k].w};
+        float x[8], src[8];
+        float sum2 = 0, dp = 0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            float ge = (e & 1) ? __uint_as_float(gw[e >> 1] & 0xffff0000u) : __uint_as_float(gw[e >> 1] << 16);
+            float se = (e & 1) ? __uint_as_float(sw[e >> 1] & 0xffff0000u) : __uint_as_float(sw[e >> 1] << 16);
+            x[e] = ge * gradMult;
+            src[e] = se * sc[k];
+            sum2 += src[e] * src[e];
+            dp += src[e] * x[e];
+        }
+        if (srcNorm.p) { // uniform
+            sum2 = Row16Sum(sum2);
+            dp = Row16Sum(dp);
+        }
+        if (!any[k]) {
+            continue;
+        }
+        uint32_t out[2] = {0, 0};
+        if (live[k]) {
+            if (srcNorm.p) {
+                float sigma = 0, scale = 0;
+                if (sum2 != 0) {
+                    float inv = 1 / sum2;
+                    sigma = dp * inv;
+                    scale = sqrtf(TILE * inv);
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    x[e] = sum2 != 0 ? (x[e] - src[e] * sigma) * scale : 0.f;
+                }
+            }
+            if (rope.p) {
+                F4 lo = ApplyRope4(MakeF4(x[0], x[1], x[2], x[3]), rp[k][0], -1.f);
+                F4 hi = ApplyRope4(MakeF4(x[4], x[5], x[6], x[7]), rp[k][1], -1.f);
+                x[0] = lo.x; x[1] = lo.y; x[2] = lo.z; x[3] = lo.w;
+                x[4] = hi.x; x[5] = hi.y; x[6] = hi.z; x[7] = hi.w;
+            }
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                out[w >> 1] |= CvtPkE4m3(x[2 * w], x[2 * w + 1]) << ((w & 1) * 16);
+            }
+        }
+        *(uint2 *)At<TE4M3>(dst, row[k], col[k]) = make_uint2(out[0], out[1]);
+    }
+}
+
 // sum of `splits` fp32 partial products (slabs of [rows][cols]) -> packed delta: per row and 128-column tile scale = maxabs/127,
 // bytes = sat_i8(rne(v/scale)), TileScale[tile][row] = scale: the arithmetic of the GEMM's ROW_TILE_MAXNORM epilogue applied to the sum
 __global__ void __launch_bounds__(256) PackDelta(int rows, int tiles, int splits, const uint8_t *partial, int64_t ldPartial, int64_t slab, float alpha,
@@ -1322,6 +1401,14 @@ extern "C" int ts2_backprop_row_tile_normalize_rope(int32_t len, int32_t lenRoun
     Mat st = srcNorm ? M(*srcTileScale) : Mat{nullptr, 0};
     if (gradType != TS2_F32 && gradType != TS2_BF16) {
         return TS2_ERR_UNSUPPORTED;
+    }
+    if (gradType == TS2_BF16 && dstType == TS2_E4M3 && Aligned16(grad->ptr, grad->strideBytes) && (!srcNorm || Aligned16(srcNorm->ptr, srcNorm->strideBytes)) &&
+        (!ropeBuf || Aligned16(ropeBuf->ptr, ropeBuf->strideBytes)) && (((uintptr_t)dst->ptr | dst->strideBytes) & 7) == 0) {
+        const long lanes = ((long)lenRound * tiles * 16 + 1) / 2;
+        hipLaunchKernelGGL(BackpropRowTileNormalizeRope8, dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, STREAM, len, lenRound, tiles, M(*grad),
+            gradMult, sn, st, rope, M(*dst));
+        TS2_CHECK_LAUNCH();
+        return TS2_OK;
     }
 #define LAUNCH_BR(TG, TD)                                                                                                                  \
     hipLaunchKernelGGL((BackpropRowTileNormalizeRope<TG, TD>), GridFor(lenRound, tiles), dim3(256), 0, STREAM, len, lenRound, tiles, M(*grad), \
