@@ -167,6 +167,97 @@ __global__ void __launch_bounds__(256) BackpropLayerNormalize(int len, int rows,
     }
 }
 
+// e4m3 norm state and e4m3 fast gradient with eight elements per lane (a tile = 16 lanes, 16-byte accesses to the fp32 arrays): the
+// form the fp8 model runs.  Same arithmetic per element as BackpropLayerNormalize; Row16Sum is defined with the 8-wide LoLU kernel.
+__device__ __forceinline__ float Row16SumFwd(float v);
+
+template <bool FINAL>
+__global__ void __launch_bounds__(256) BackpropLayerNormalize8(int len, int rows, int tiles, Mat normState, Mat stateScale, Mat dNormState,
+    const float *combinerScale, const float *gradScale, const float *gradMult, Mat stateGrad, Mat stateGradFast, float *nextMaxNorm)
+{
+    __shared__ float red[4];
+    const int l16 = threadIdx.x & 15;
+    const long units = (long)rows * tiles;
+    float s = 1;
+    if (!FINAL) {
+        if (combinerScale) {
+            s *= *combinerScale;
+        }
+        if (gradScale) {
+            s *= *gradScale;
+        }
+    }
+    const float gm = (!FINAL && gradMult) ? *gradMult : 1.f;
+    float gmax = 0;
+    // every lane of a wave takes part in every iteration (the reductions are cross-lane): the loop bound is wave-uniform
+    const long unitFirst = ((long)blockIdx.x * 256 + (threadIdx.x & ~63)) >> 4;
+    for (long ub = unitFirst; ub < units; ub += (long)gridDim.x * 16) {
+        const long u = ub + ((threadIdx.x & 63) >> 4);
+        const bool any = u < units;
+        const int t = any ? (int)(u / tiles) : 0;
+        const int tile = any ? (int)(u - (long)t * tiles) : 0;
+        const int col = tile * TILE + l16 * 8;
+        const bool live = any && t < len;
+        uint2 nv = live ? *(const uint2 *)At<TE4M3>(normState, t, col) : make_uint2(0, 0);
+        F4 g0 = live ? Load4<TF32>(At<TF32>(dNormState, t, col)) : ZeroF4();
+        F4 g1 = live ? Load4<TF32>(At<TF32>(dNormState, t, col + 4)) : ZeroF4();
+        F4 p0 = (live && !FINAL) ? Load4<TF32>(At<TF32>(stateGrad, t, col)) : ZeroF4();
+        F4 p1 = (live && !FINAL) ? Load4<TF32>(At<TF32>(stateGrad, t, col + 4)) : ZeroF4();
+        const float sc = live ? ScaleAt(stateScale, tile, t) : 0.f;
+        float src[8], g[8];
+        const float nf[8] = {__builtin_amdgcn_cvt_f32_fp8((int)nv.x, 0), __builtin_amdgcn_cvt_f32_fp8((int)nv.x, 1), __builtin_amdgcn_cvt_f32_fp8((int)nv.x, 2),
+            __builtin_amdgcn_cvt_f32_fp8((int)nv.x, 3), __builtin_amdgcn_cvt_f32_fp8((int)nv.y, 0), __builtin_amdgcn_cvt_f32_fp8((int)nv.y, 1),
+            __builtin_amdgcn_cvt_f32_fp8((int)nv.y, 2), __builtin_amdgcn_cvt_f32_fp8((int)nv.y, 3)};
+        const float gin[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+        const float prev[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
+        float sum2 = 0, dp = 0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            src[e] = nf[e] * sc;
+            g[e] = FINAL ? gin[e] : gin[e] * s;
+            sum2 += src[e] * src[e];
+            dp += src[e] * g[e];
+        }
+        sum2 = Row16SumFwd(sum2);
+        dp = Row16SumFwd(dp);
+        if (!any) {
+            continue;
+        }
+        float sigma = 0, scale = 0;
+        if (sum2 != 0) {
+            float inv = 1 / sum2;
+            sigma = dp * inv;
+            scale = sqrtf(TILE * inv);
+        }
+        float out[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            float x = 0;
+            if (live) {
+                x = sum2 != 0 ? (g[e] - src[e] * sigma) * scale : 0.f;
+                if (!FINAL) {
+                    x += prev[e];
+                }
+                gmax = fmaxf(gmax, fabsf(x));
+            }
+            out[e] = x;
+        }
+        Store4<TF32>(At<TF32>(stateGrad, t, col), MakeF4(out[0], out[1], out[2], out[3]));
+        Store4<TF32>(At<TF32>(stateGrad, t, col + 4), MakeF4(out[4], out[5], out[6], out[7]));
+        uint32_t lo = CvtPkE4m3(out[0] * gm, out[1] * gm) | (CvtPkE4m3(out[2] * gm, out[3] * gm) << 16);
+        uint32_t hi = CvtPkE4m3(out[4] * gm, out[5] * gm) | (CvtPkE4m3(out[6] * gm, out[7] * gm) << 16);
+        *(uint2 *)At<TE4M3>(stateGradFast, t, col) = make_uint2(lo, hi);
+    }
+    gmax = WaveMax(gmax);
+    if ((threadIdx.x & 63) == 0) {
+        red[threadIdx.x >> 6] = gmax;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0 && nextMaxNorm) {
+        AtomicMaxPos(nextMaxNorm, fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])));
+    }
+}
+
 __device__ __forceinline__ float ComputeGradMult(float gradMaxNorm)
 {
     if (gradMaxNorm == 0) {
@@ -323,6 +414,12 @@ __global__ void __launch_bounds__(256) BackpropLoLU(int len, int lenRound, int t
 // The FFN flavour (MODE 0) for bf16 gradients and e4m3 results with eight elements per lane: a 128-wide tile is 16 lanes, so a wave
 // holds four (row, tile) units, the tile sums are four DPP steps inside a row of 16 lanes, loads are 16 bytes and stores 8.  Two
 // units per lane in flight.  Same arithmetic per element as BackpropLoLU<.., 0>.
+__device__ __forceinline__ float Row16Sum(float v);
+__device__ __forceinline__ float Row16SumFwd(float v)
+{
+    return Row16Sum(v);
+}
+
 __device__ __forceinline__ float Row16Sum(float v)
 {
     v += LaneDpp<DPP_XOR1>(v);
@@ -1057,6 +1154,20 @@ static int BackpropNormImpl(bool final, int len, int rows, const ts2_mat *normSt
     int tiles = dim / TILE;
     long nUnits = (long)rows * tiles;
     dim3 bnGrid((unsigned)((nUnits + 7) / 8 < 4096 ? (nUnits + 7) / 8 : 4096));
+    if (normType == TS2_E4M3 && fastType == TS2_E4M3 && (((uintptr_t)normState->ptr | normState->strideBytes | (uintptr_t)stateGradFast->ptr |
+                                                         stateGradFast->strideBytes) & 7) == 0 &&
+        Aligned16(dNormState->ptr, dNormState->strideBytes) && Aligned16(stateGrad->ptr, stateGrad->strideBytes)) {
+        dim3 grid8((unsigned)((nUnits + 15) / 16 < 8192 ? (nUnits + 15) / 16 : 8192));
+        if (final) {
+            hipLaunchKernelGGL((BackpropLayerNormalize8<true>), grid8, dim3(256), 0, STREAM, len, rows, tiles, M(*normState), M(*stateScale),
+                M(*dNormState), combinerScale, gradScale, gradMult, M(*stateGrad), M(*stateGradFast), nextMaxNorm);
+        } else {
+            hipLaunchKernelGGL((BackpropLayerNormalize8<false>), grid8, dim3(256), 0, STREAM, len, rows, tiles, M(*normState), M(*stateScale),
+                M(*dNormState), combinerScale, gradScale, gradMult, M(*stateGrad), M(*stateGradFast), nextMaxNorm);
+        }
+        TS2_CHECK_LAUNCH();
+        return TS2_OK;
+    }
 #define LAUNCH_BN(TN, TFA)                                                                                                                 \
     if (final)                                                                                                                             \
         hipLaunchKernelGGL((BackpropLayerNormalize<TN, TFA, true>), bnGrid, dim3(256), 0, STREAM, len, rows, tiles,         \
