@@ -27,6 +27,9 @@ namespace
 constexpr int HD = 128;          // Q_DIM = TT_DIM (src/gpt/compute/cfg_precision.h:79-80)
 constexpr int WROWS = 32;        // rows owned by one wave
 constexpr int BROWS = 128;       // rows owned by one workgroup
+#define TS2_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
+#define TS2_GLB_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
+
 constexpr int TR = 64;           // rows of a streamed tile
 constexpr int RP = HD * 2 + 16;  // row-major tile pitch (bytes)
 constexpr int TP = TR * 2 + 8;   // transposed tile pitch (bytes): 34 dwords -> 8-byte reads of 32 consecutive d hit all 64 banks
@@ -361,7 +364,7 @@ __global__ void __launch_bounds__(256, 2) AttForward(AttP p)
 
 // ---------------------------------------------------------------------------------------------------------------------------
 // dQ: grid (lenRound/128, heads)
-template <bool F32> __global__ void __launch_bounds__(256, 2) AttGradQ(AttP p)
+template <bool F32> __global__ void __launch_bounds__(256) AttGradQ(AttP p)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     uint8_t *kRm = lds, *vRm = lds + RM_BYTES, *kT = lds + 2 * RM_BYTES, *ownQ = lds + 2 * RM_BYTES + T_BYTES, *ownDO = ownQ + OWN_BYTES;
@@ -383,10 +386,13 @@ template <bool F32> __global__ void __launch_bounds__(256, 2) AttGradQ(AttP p)
 
     ParkOwnFrags(ownQ, p.q + (int64_t)(myRow - l32) * p.ldq + hoff, p.ldq, wave, lane);
     ParkOwnFrags(ownDO, p.dO + (int64_t)(myRow - l32) * p.lddo + hoff, p.lddo, wave, lane);
-    const float L = p.sumWeightLog[(int64_t)head * p.ldStat + myRow];
-    const float dScale = p.dScale[(int64_t)head * p.ldStat + myRow];
+    float L = p.sumWeightLog[(int64_t)head * p.ldStat + myRow];
+    float dScale = p.dScale[(int64_t)head * p.ldStat + myRow];
     const float gmul = p.attDotScale * LN2;
     const TRowSpan sp = MakeRowSpan(start, finish);
+    // L and dScale are used here, once, so that their loads are waited for before the loop: a first use inside the loop would
+    // put a wait for every outstanding load (the tile prefetch included) into each iteration
+    asm volatile("" : "+v"(L), "+v"(dScale));
     v16f acc[4];
 #pragma unroll
     for (int db = 0; db < 4; ++db) {
@@ -417,16 +423,44 @@ template <bool F32> __global__ void __launch_bounds__(256, 2) AttGradQ(AttP p)
                 dp[kb][e] = 0;
             }
         }
-        // phase 1: S^T and dP^T of the whole tile, four independent accumulator chains
+        // phase 1: S^T and dP^T of the whole tile, four independent accumulator chains.  One wave per SIMD (the workgroup's LDS
+        // leaves room for one workgroup per CU): the operands of step ds + 1 are requested before the products of step ds are issued
+        v8bf fq[2], fo[2], fk[2][NB], fv[2][NB];
+#define Q_LOAD1(DS)                                                                                                                        \
+    do {                                                                                                                                   \
+        fq[(DS) & 1] = OwnFrag(ownQ, wave, DS, lane);                                                                                      \
+        fo[(DS) & 1] = OwnFrag(ownDO, wave, DS, lane);                                                                                     \
+        _Pragma("unroll") for (int kb = 0; kb < NB; ++kb) {                                                                                \
+            fk[(DS) & 1][kb] = FragRM(kRm, kb, DS, l32, half);                                                                             \
+            fv[(DS) & 1][kb] = FragRM(vRm, kb, DS, l32, half);                                                                             \
+        }                                                                                                                                  \
+    } while (0)
+        Q_LOAD1(0);
 #pragma unroll
         for (int ds = 0; ds < 8; ++ds) {
-            v8bf qf = OwnFrag(ownQ, wave, ds, lane), dof = OwnFrag(ownDO, wave, ds, lane);
+            if (ds + 1 < 8) {
+                Q_LOAD1(ds + 1);
+            }
 #pragma unroll
             for (int kb = 0; kb < NB; ++kb) {
-                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(kRm, kb, ds, l32, half), qf, s[kb], 0, 0, 0);
-                dp[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(vRm, kb, ds, l32, half), dof, dp[kb], 0, 0, 0);
+                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fk[ds & 1][kb], fq[ds & 1], s[kb], 0, 0, 0);
+                dp[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fv[ds & 1][kb], fo[ds & 1], dp[kb], 0, 0, 0);
             }
         }
+#undef Q_LOAD1
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 + 2 * NB, 0);
+#pragma unroll
+        for (int ds = 0; ds < 7; ++ds) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 2 + 2 * NB, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 2 * NB, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 2 * NB, 0);
+        // the first operands of phase 3 are requested before the arithmetic of phase 2
+        v8bf ft[2][4];
+#define Q_LOAD3(KS)                                                                                                                        \
+    _Pragma("unroll") for (int db = 0; db < 4; ++db) ft[(KS) & 1][db] = FragT(kT, db, KS, l32, half)
+        Q_LOAD3(0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
         // phase 2: dS
         v8bf sb[NB][2];
         const float kc = p.slope * (float)(t0 + half * 4 - myRow) - L; // logit - L in one fma chain
@@ -444,14 +478,24 @@ template <bool F32> __global__ void __launch_bounds__(256, 2) AttGradQ(AttP p)
             sb[kb][0] = PackB(dsv, 0);
             sb[kb][1] = PackB(dsv, 1);
         }
-        // phase 3: dQ^T += K^T dS^T
+        // phase 3: dQ^T += K^T dS^T, operands one step (four products) ahead
 #pragma unroll
         for (int ks = 0; ks < 2 * NB; ++ks) {
+            if (ks + 1 < 2 * NB) {
+                Q_LOAD3(ks + 1);
+            }
 #pragma unroll
             for (int db = 0; db < 4; ++db) {
-                acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(kT, db, ks, l32, half), sb[ks >> 1][ks & 1], acc[db], 0, 0, 0);
+                acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ft[ks & 1][db], sb[ks >> 1][ks & 1], acc[db], 0, 0, 0);
             }
         }
+#undef Q_LOAD3
+#pragma unroll
+        for (int ks = 0; ks < 2 * NB - 1; ++ks) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
     }
     StoreOwnRows<F32>(p.out0 + (int64_t)(myRow - l32) * p.ldo0, p.ldo0, head * HD, acc, 1.f, l32, half);
 }
@@ -460,14 +504,13 @@ template <bool F32> __global__ void __launch_bounds__(256, 2) AttGradQ(AttP p)
 // dK, dV: grid (lenRound/128, heads); the workgroup owns 128 key rows and streams the query rows that reach them
 template <bool F32> __global__ void __launch_bounds__(256) AttGradKV(AttP p)
 {
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    uint8_t *qRm = lds, *doRm = lds + RM_BYTES, *qT = lds + 2 * RM_BYTES, *doT = lds + 2 * RM_BYTES + T_BYTES;
-    float *stL = (float *)(lds + 2 * RM_BYTES + 2 * T_BYTES); // [TR] each: L, dScale, start, finish
-    float *stD = stL + TR;
-    int *stS = (int *)(stD + TR);
-    int *stF = stS + TR;
-    int *stT = stF + TR; // [4] bounds over the tile's queries
-    uint8_t *ownK = (uint8_t *)(stT + 4), *ownV = ownK + OWN_BYTES;
+    // Static arrays, one per buffer: the compiler then knows that the operand reads do not touch the buffer that the direct
+    // global -> LDS loads below fill, and does not make them wait for those loads.
+    __shared__ __attribute__((aligned(16))) uint8_t qRm[RM_BYTES], doRm[RM_BYTES], qT[T_BYTES], doT[T_BYTES];
+    __shared__ __attribute__((aligned(16))) uint8_t ownK[OWN_BYTES], ownV[OWN_BYTES];
+    __shared__ __attribute__((aligned(16))) float stL[TR], stD[TR]; // per query of the tile: L, dScale
+    __shared__ __attribute__((aligned(16))) int stS[TR], stF[TR];   // span start, span length
+    __shared__ int stT[4];                                          // bounds over the tile's queries
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
     const int head = blockIdx.y;
     const int myRow = blockIdx.x * BROWS + wave * WROWS + l32; // my key
@@ -475,23 +518,24 @@ template <bool F32> __global__ void __launch_bounds__(256) AttGradKV(AttP p)
     const int qLo = p.revLo[blockIdx.x], qHi = p.revHi[blockIdx.x];
     const int tFirst = qHi >= qLo ? (qLo / TR) * TR : 1;
     TilePref pq, pdo;
-    float preL = 0, preD = 0;
-    int preS = 0x7fffffff, preF = -1;
+    // The per-query statistics of the next tile go global -> LDS without passing through registers: a register that a pending load
+    // writes is a register the compiler may move (the kernel runs at its register limit), and the move waits for every load issued
+    // before it, the tile prefetch included.  Two slots, used in turn; wave 0 issues the loads and, one tile later, reads them back.
+    __shared__ float rawStat[2][4][TR]; // [slot][L, dScale, span start, span finish][query]
     const int keyBase = blockIdx.x * BROWS;
-    auto prefetch = [&](int t0) {
+    auto prefetch = [&](int t0, int slot) {
+        if (wave == 0) {
+            const int64_t so = (int64_t)head * p.ldStat + t0 + lane;
+            __builtin_amdgcn_global_load_lds(TS2_GLB_PTR(p.sumWeightLog + so), TS2_LDS_PTR(&rawStat[slot][0][0]), 4, 0, 0);
+            __builtin_amdgcn_global_load_lds(TS2_GLB_PTR(p.dScale + so), TS2_LDS_PTR(&rawStat[slot][1][0]), 4, 0, 0);
+            __builtin_amdgcn_global_load_lds(TS2_GLB_PTR(p.spanStart + t0 + lane), TS2_LDS_PTR(&rawStat[slot][2][0]), 4, 0, 0);
+            __builtin_amdgcn_global_load_lds(TS2_GLB_PTR(p.spanFinish + t0 + lane), TS2_LDS_PTR(&rawStat[slot][3][0]), 4, 0, 0);
+        }
         PrefetchTile(pq, p.q + (int64_t)t0 * p.ldq + hoff, p.ldq, tid);
         PrefetchTile(pdo, p.dO + (int64_t)t0 * p.lddo + hoff, p.lddo, tid);
-        if (tid < TR) {
-            // per query: -L - slope * (query - first key of the workgroup), dScale, span start (0x7fffffff if empty) and finish
-            preL = -p.sumWeightLog[(int64_t)head * p.ldStat + t0 + tid] - p.slope * (float)(t0 + tid - keyBase);
-            preD = p.dScale[(int64_t)head * p.ldStat + t0 + tid];
-            int st = p.spanStart[t0 + tid], fi = p.spanFinish[t0 + tid];
-            preS = fi >= st ? st : 0x7fffffff;
-            preF = fi >= st ? fi : -1;
-        }
     };
     if (tFirst <= qHi) {
-        prefetch(tFirst);
+        prefetch(tFirst, 0);
     }
 
     ParkOwnFrags(ownK, p.k + (int64_t)(myRow - l32) * p.ldk + hoff, p.ldk, wave, lane);
@@ -506,13 +550,22 @@ template <bool F32> __global__ void __launch_bounds__(256) AttGradKV(AttP p)
             dv[db][e] = 0;
         }
     }
-    for (int t0 = tFirst; t0 <= qHi; t0 += TR) {
+    int slot = 0;
+    for (int t0 = tFirst; t0 <= qHi; t0 += TR, slot ^= 1) {
         __syncthreads();
         StoreTile<true, true>(pq, qRm, qT, tid);
         StoreTile<true, true>(pdo, doRm, doT, tid);
-        if (tid < TR) { // wave 0
-            stL[tid] = preL;
-            stD[tid] = preD;
+        if (tid < TR) { // wave 0; the tile stores above have waited for its loads, which were issued after the statistics'
+            __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0)
+            asm volatile("" ::: "memory");
+            // per query: -L - slope * (query - first key of the workgroup), dScale, span start (0x7fffffff if empty) and length
+            const float rawL = rawStat[slot][0][tid];
+            int preS = __float_as_int(rawStat[slot][2][tid]), preF = __float_as_int(rawStat[slot][3][tid]);
+            const bool some = preF >= preS;
+            preS = some ? preS : 0x7fffffff;
+            preF = some ? preF : -1;
+            stL[tid] = -rawL - p.slope * (float)(t0 + tid - keyBase);
+            stD[tid] = rawStat[slot][1][tid];
             stS[tid] = preS;
             stF[tid] = (int)(preF >= preS ? (unsigned)(preF - preS) : 0u); // span length
             int a = preS, b = preF, c = preS, d = preF;
@@ -529,7 +582,7 @@ template <bool F32> __global__ void __launch_bounds__(256) AttGradKV(AttP p)
         }
         __syncthreads();
         if (t0 + TR <= qHi) {
-            prefetch(t0 + TR);
+            prefetch(t0 + TR, slot ^ 1);
         }
         const int kw0 = myRow - l32; // first key of this wave
         if (stT[3] < kw0 || stT[2] > kw0 + 31) {
@@ -545,12 +598,45 @@ template <bool F32> __global__ void __launch_bounds__(256) AttGradKV(AttP p)
                 s[e] = 0;
                 dp[e] = 0;
             }
-            // phase 1: S and dP
+            // phase 1: S and dP.  One wave per SIMD: nothing else hides the LDS latency, so the operands of step ds + 2 are requested
+            // before the products of step ds are issued (three sets of operand registers in rotation)
+            v8bf fq[3], fk[3], fo[3], fv[3];
+#define KV_LOAD1(DS)                                                                                                                       \
+    do {                                                                                                                                   \
+        fq[(DS) % 3] = FragRM(qRm, qb, DS, l32, half);                                                                                     \
+        fk[(DS) % 3] = OwnFrag(ownK, wave, DS, lane);                                                                                      \
+        fo[(DS) % 3] = FragRM(doRm, qb, DS, l32, half);                                                                                    \
+        fv[(DS) % 3] = OwnFrag(ownV, wave, DS, lane);                                                                                      \
+    } while (0)
+            KV_LOAD1(0);
+            KV_LOAD1(1);
 #pragma unroll
             for (int ds = 0; ds < 8; ++ds) {
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(qRm, qb, ds, l32, half), OwnFrag(ownK, wave, ds, lane), s, 0, 0, 0);
-                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(doRm, qb, ds, l32, half), OwnFrag(ownV, wave, ds, lane), dp, 0, 0, 0);
+                if (ds + 2 < 8) {
+                    KV_LOAD1(ds + 2);
+                }
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fq[ds % 3], fk[ds % 3], s, 0, 0, 0);
+                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fo[ds % 3], fv[ds % 3], dp, 0, 0, 0);
             }
+#undef KV_LOAD1
+            __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+            for (int ds = 0; ds < 6; ++ds) {
+                __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+            // the first operands of phase 3 are requested before the arithmetic of phase 2, which covers their latency
+            v8bf to[3], tq[3];
+#define KV_LOAD3(ST)                                                                                                                       \
+    do {                                                                                                                                   \
+        to[(ST) % 3] = FragT(doT, (ST) & 3, qb * 2 + ((ST) >> 2), l32, half);                                                              \
+        tq[(ST) % 3] = FragT(qT, (ST) & 3, qb * 2 + ((ST) >> 2), l32, half);                                                               \
+    } while (0)
+            KV_LOAD3(0);
+            KV_LOAD3(1);
+            __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);  // (a transposed operand is one ds_read2_b64)
+            __builtin_amdgcn_sched_group_barrier(0x100, 16, 0); // the statistics of phase 2
             // phase 2: P and dS from the per-query statistics of the tile
             float pv[16], dsv[16];
 #pragma unroll
@@ -574,15 +660,22 @@ template <bool F32> __global__ void __launch_bounds__(256) AttGradKV(AttP p)
                 }
             }
             v8bf pb[2] = {PackB(pv, 0), PackB(pv, 1)}, sb[2] = {PackB(dsv, 0), PackB(dsv, 1)};
-            // phase 3: dV^T += dO^T P, dK^T += Q^T dS; eight accumulators in turn
+            // phase 3: dV^T += dO^T P, dK^T += Q^T dS; eight accumulators in turn, operands two steps ahead
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-#pragma unroll
-                for (int db = 0; db < 4; ++db) {
-                    dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(doT, db, qb * 2 + j, l32, half), pb[j], dv[db], 0, 0, 0);
-                    dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(qT, db, qb * 2 + j, l32, half), sb[j], dk[db], 0, 0, 0);
+            for (int st = 0; st < 8; ++st) {
+                if (st + 2 < 8) {
+                    KV_LOAD3(st + 2);
                 }
+                dv[st & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(to[st % 3], pb[st >> 2], dv[st & 3], 0, 0, 0);
+                dk[st & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tq[st % 3], sb[st >> 2], dk[st & 3], 0, 0, 0);
             }
+#undef KV_LOAD3
+#pragma unroll
+            for (int st = 0; st < 6; ++st) {
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
         }
     }
     StoreOwnRows<F32>(p.out0 + (int64_t)(myRow - l32) * p.ldo0, p.ldo0, head * HD, dk, 1.f, l32, half);
@@ -721,11 +814,9 @@ extern "C" int ts2_att_backward(const ts2_att_grad_args *a, void *stream)
     p.lenRound = a->lenRound;
     dim3 grid(a->lenRound / BROWS, a->heads);
     int ldsQ = 2 * RM_BYTES + T_BYTES + 2 * OWN_BYTES;
-    int ldsKV = 2 * RM_BYTES + 2 * T_BYTES + 4 * TR * 4 + 16 + 2 * OWN_BYTES;
     static bool done = false;
     if (!done) {
-        if (SetAttr((const void *)AttGradQ<true>, ldsQ) || SetAttr((const void *)AttGradQ<false>, ldsQ) ||
-            SetAttr((const void *)AttGradKV<true>, ldsKV) || SetAttr((const void *)AttGradKV<false>, ldsKV)) {
+        if (SetAttr((const void *)AttGradQ<true>, ldsQ) || SetAttr((const void *)AttGradQ<false>, ldsQ)) {
             return TS2_ERR_LAUNCH;
         }
         done = true;
@@ -746,9 +837,9 @@ extern "C" int ts2_att_backward(const ts2_att_grad_args *a, void *stream)
         p.out1 = (uint8_t *)a->dV.ptr;
         p.ldo1 = a->dV.strideBytes;
         if (f32) {
-            hipLaunchKernelGGL(AttGradKV<true>, grid, dim3(256), ldsKV, (hipStream_t)stream, p);
+            hipLaunchKernelGGL(AttGradKV<true>, grid, dim3(256), 0, (hipStream_t)stream, p); // its LDS is static
         } else {
-            hipLaunchKernelGGL(AttGradKV<false>, grid, dim3(256), ldsKV, (hipStream_t)stream, p);
+            hipLaunchKernelGGL(AttGradKV<false>, grid, dim3(256), 0, (hipStream_t)stream, p);
         }
         TS2_CHECK_LAUNCH();
     }
