@@ -17,6 +17,9 @@
 //   * products that contract over token rows need the streamed tile with rows along the contraction: the tile is fetched one tile
 //     ahead into registers and written to LDS row-major and/or transposed (two rows packed per dword with v_perm_b32, pitches chosen
 //     so that operand reads and transposed writes are bank-conflict free); the wave's own rows are parked in LDS in fragment order.
+//   * the backward kernels run one wave per SIMD (their LDS leaves room for one workgroup per CU), so latency is hidden by the
+//     instruction order alone: operand reads are issued one or two steps ahead of their products, and nothing inside the tile loop
+//     may wait on a load younger than the tile prefetch (vmcnt counts in order).
 //   * spans are one inclusive key range per query (every causal window / document-start pattern of
 //     src/gpt/att/sliding_window.cpp:111-118,226-240); masking is one unsigned compare per element, tiles outside a wave's range are
 //     skipped, tiles outside the workgroup's range are never loaded.
@@ -465,18 +468,35 @@ template <bool F32> __global__ void __launch_bounds__(256) AttGradQ(AttP p)
         v8bf sb[NB][2];
         const float kc = p.slope * (float)(t0 + half * 4 - myRow) - L; // logit - L in one fma chain
         const int rel0 = t0 + half * 4 - sp.start;
+        // tiles that every row of the wave sees completely skip the span tests
+        const bool full = t0 >= sp.waveMaxStart && t0 + TR - 1 <= sp.waveMinFinish;
+        if (full) {
 #pragma unroll
-        for (int kb = 0; kb < NB; ++kb) {
-            float dsv[16];
+            for (int kb = 0; kb < NB; ++kb) {
+                float dsv[16];
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                float x = fmaf(s[kb][e], p.attDotScale, fmaf(p.slope, (float)(kb * 32 + BlkRow(e, 0)), kc));
-                float w = __builtin_amdgcn_exp2f(x);
-                w = (unsigned)(rel0 + kb * 32 + BlkRow(e, 0)) <= sp.len ? w : 0.f;
-                dsv[e] = w * (dp[kb][e] - dScale) * gmul;
+                for (int e = 0; e < 16; ++e) {
+                    float x = fmaf(s[kb][e], p.attDotScale, fmaf(p.slope, (float)(kb * 32 + BlkRow(e, 0)), kc));
+                    float w = __builtin_amdgcn_exp2f(x);
+                    dsv[e] = w * (dp[kb][e] - dScale) * gmul;
+                }
+                sb[kb][0] = PackB(dsv, 0);
+                sb[kb][1] = PackB(dsv, 1);
             }
-            sb[kb][0] = PackB(dsv, 0);
-            sb[kb][1] = PackB(dsv, 1);
+        } else {
+#pragma unroll
+            for (int kb = 0; kb < NB; ++kb) {
+                float dsv[16];
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    float x = fmaf(s[kb][e], p.attDotScale, fmaf(p.slope, (float)(kb * 32 + BlkRow(e, 0)), kc));
+                    float w = __builtin_amdgcn_exp2f(x);
+                    w = (unsigned)(rel0 + kb * 32 + BlkRow(e, 0)) <= sp.len ? w : 0.f;
+                    dsv[e] = w * (dp[kb][e] - dScale) * gmul;
+                }
+                sb[kb][0] = PackB(dsv, 0);
+                sb[kb][1] = PackB(dsv, 1);
+            }
         }
         // phase 3: dQ^T += K^T dS^T, operands one step (four products) ahead
 #pragma unroll
@@ -513,16 +533,17 @@ template <bool F32> __global__ void __launch_bounds__(256) AttGradKV(AttP p)
     __shared__ int stT[4];                                          // bounds over the tile's queries
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
     const int head = blockIdx.y;
-    const int myRow = blockIdx.x * BROWS + wave * WROWS + l32; // my key
+    const int block = blockIdx.x;
+    const int myRow = block * BROWS + wave * WROWS + l32; // my key
     const int64_t hoff = (int64_t)head * HD * 2;
-    const int qLo = p.revLo[blockIdx.x], qHi = p.revHi[blockIdx.x];
+    const int qLo = p.revLo[block], qHi = p.revHi[block];
     const int tFirst = qHi >= qLo ? (qLo / TR) * TR : 1;
     TilePref pq, pdo;
     // The per-query statistics of the next tile go global -> LDS without passing through registers: a register that a pending load
     // writes is a register the compiler may move (the kernel runs at its register limit), and the move waits for every load issued
     // before it, the tile prefetch included.  Two slots, used in turn; wave 0 issues the loads and, one tile later, reads them back.
     __shared__ float rawStat[2][4][TR]; // [slot][L, dScale, span start, span finish][query]
-    const int keyBase = blockIdx.x * BROWS;
+    const int keyBase = block * BROWS;
     auto prefetch = [&](int t0, int slot) {
         if (wave == 0) {
             const int64_t so = (int64_t)head * p.ldStat + t0 + lane;
@@ -589,6 +610,7 @@ template <bool F32> __global__ void __launch_bounds__(256) AttGradKV(AttP p)
             continue; // no query of the tile sees a key of this wave (wave-uniform)
         }
         const float ck = p.slope * (float)(myRow - keyBase);
+        const bool full = stT[0] <= kw0 && stT[1] >= kw0 + 31; // latest span start and earliest finish of the tile's queries
         // 32 queries at a time: with both halves of the tile in flight the kernel does not fit into 256 registers
 #pragma unroll
         for (int qb = 0; qb < TR / 32; ++qb) {
@@ -636,27 +658,44 @@ template <bool F32> __global__ void __launch_bounds__(256) AttGradKV(AttP p)
             KV_LOAD3(0);
             KV_LOAD3(1);
             __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);  // (a transposed operand is one ds_read2_b64)
-            __builtin_amdgcn_sched_group_barrier(0x100, 16, 0); // the statistics of phase 2
             // phase 2: P and dS from the per-query statistics of the tile
             float pv[16], dsv[16];
+            if (full) { // every query of the tile sees every key of the wave: no span tests
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                int qi = qb * 32 + g * 8 + half * 4;
-                float4 L4 = *(const float4 *)(stL + qi);
-                float4 D4 = *(const float4 *)(stD + qi);
-                int4 S4 = *(const int4 *)(stS + qi);
-                int4 N4 = *(const int4 *)(stF + qi);
-                const float Ls[4] = {L4.x, L4.y, L4.z, L4.w};
-                const float Ds[4] = {D4.x, D4.y, D4.z, D4.w};
-                const int Ss[4] = {S4.x, S4.y, S4.z, S4.w};
-                const unsigned Ns[4] = {(unsigned)N4.x, (unsigned)N4.y, (unsigned)N4.z, (unsigned)N4.w};
+                for (int g = 0; g < 4; ++g) {
+                    int qi = qb * 32 + g * 8 + half * 4;
+                    float4 L4 = *(const float4 *)(stL + qi);
+                    float4 D4 = *(const float4 *)(stD + qi);
+                    const float Ls[4] = {L4.x, L4.y, L4.z, L4.w};
+                    const float Ds[4] = {D4.x, D4.y, D4.z, D4.w};
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    int e = g * 4 + j;
-                    float w = __builtin_amdgcn_exp2f(fmaf(s[e], p.attDotScale, Ls[j] + ck));
-                    w = (unsigned)(myRow - Ss[j]) <= Ns[j] ? w : 0.f;
-                    pv[e] = w;
-                    dsv[e] = w * (dp[e] - Ds[j]) * gmul;
+                    for (int j = 0; j < 4; ++j) {
+                        int e = g * 4 + j;
+                        float w = __builtin_amdgcn_exp2f(fmaf(s[e], p.attDotScale, Ls[j] + ck));
+                        pv[e] = w;
+                        dsv[e] = w * (dp[e] - Ds[j]) * gmul;
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    int qi = qb * 32 + g * 8 + half * 4;
+                    float4 L4 = *(const float4 *)(stL + qi);
+                    float4 D4 = *(const float4 *)(stD + qi);
+                    int4 S4 = *(const int4 *)(stS + qi);
+                    int4 N4 = *(const int4 *)(stF + qi);
+                    const float Ls[4] = {L4.x, L4.y, L4.z, L4.w};
+                    const float Ds[4] = {D4.x, D4.y, D4.z, D4.w};
+                    const int Ss[4] = {S4.x, S4.y, S4.z, S4.w};
+                    const unsigned Ns[4] = {(unsigned)N4.x, (unsigned)N4.y, (unsigned)N4.z, (unsigned)N4.w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        int e = g * 4 + j;
+                        float w = __builtin_amdgcn_exp2f(fmaf(s[e], p.attDotScale, Ls[j] + ck));
+                        w = (unsigned)(myRow - Ss[j]) <= Ns[j] ? w : 0.f;
+                        pv[e] = w;
+                        dsv[e] = w * (dp[e] - Ds[j]) * gmul;
+                    }
                 }
             }
             v8bf pb[2] = {PackB(pv, 0), PackB(pv, 1)}, sb[2] = {PackB(dsv, 0), PackB(dsv, 1)};
