@@ -53,7 +53,7 @@ class QMatrix:
 
 class Harness:
     def __init__(self, mode, dim, heads, ffn_tiles, depth, vocab, frag_count, frag_len, wide_window=64, experts=0, selected=2, xp=128, seed=1,
-                 std=0.02, k_std=None):
+                 std=0.02, k_std=None, bias_std=0.0):
         self.orc = Oracle()
         self.mode, self.dim, self.heads, self.ffn = mode, dim, heads, ffn_tiles * 128
         self.experts, self.selected, self.xp = experts, selected, xp
@@ -70,7 +70,8 @@ class Harness:
             self.layers.append(mats)
         self.embed = QMatrix(self.orc, r.standard_normal((self.label_count, dim)) * std, mode, False)
         self.final = QMatrix(self.orc, r.standard_normal((vocab, dim)) * std, mode, False)
-        self.bias = np.zeros(vocab, np.float32)
+        # final-layer bias (log2 units); drawn from its own generator so that the other draws do not depend on it
+        self.bias = (np.random.default_rng(seed + 1000).standard_normal(vocab) * bias_std).astype(np.float32)
         # batch: uniform random tokens, target = next token of the fragment, label = 1 + token (noise labels disabled)
         self.n = frag_count * frag_len
         tokens = r.integers(0, vocab, (frag_count, frag_len))

@@ -294,6 +294,141 @@ __global__ void __launch_bounds__(256) FinalSoftmaxGradHalf(int vocab, const _Fl
         *(uint4 *)(grow + k) = make_uint4(PackBf16x2(g[0], g[1]), PackBf16x2(g[2], g[3]), PackBf16x2(g[4], g[5]), PackBf16x2(g[6], g[7]));
     }
 }
+// The same for rows of at most ROW_ROUNDS * 8192 logits, with the row read once and one exponential per logit: a workgroup of 1024
+// threads walks rows with a grid stride and a thread keeps its logits in registers.  It takes its own maximum first (packed half
+// max), replaces every logit by 2^(logit + bias - own reference) as a half (a number in [0, 1] with 11 significant bits, more than
+// the bf16 gradient keeps) while summing in fp32, and after the workgroup reduction the gradient is that half times one per-thread
+// factor.  The next row's loads are in flight during all of this.  Arithmetic per logit: two conversions, two adds, one v_exp_f32,
+// one sum, one multiply - the two-pass kernel above is bound by its VALU work (two exponentials per logit), not by memory.
+constexpr int ROW_ROUNDS = 7; // up to 57344 logits; 2 x 28 registers of row data per thread
+
+__global__ void __launch_bounds__(1024) FinalSoftmaxGradHalfRow(int rows, int vocab, const _Float16 *logits, int64_t ldLogits, const float *bias,
+    const int *target, float gradMult, bf16_t *grad, int64_t ldGrad, float *lossSum)
+{
+    typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+    __shared__ float redM[16], redS[16];
+    const int tid = threadIdx.x;
+    v8h cur[ROW_ROUNDS], nxt[ROW_ROUNDS];
+    auto prefetch = [&](int t) {
+        const _Float16 *row = (const _Float16 *)((const uint8_t *)logits + (int64_t)t * ldLogits);
+#pragma unroll
+        for (int i = 0; i < ROW_ROUNDS; ++i) {
+            int k = tid * 8 + i * 8192;
+            nxt[i] = k < vocab ? *(const v8h *)(row + k) : (v8h)(_Float16)-60000.f;
+        }
+    };
+    int t = blockIdx.x;
+    if (t < rows) {
+        prefetch(t);
+    }
+    // a thread meets the same columns in every row: the largest bias among them, added to its reference, keeps the halves in [0, 1]
+    float biasTop = 0;
+#pragma unroll
+    for (int i = 0; i < ROW_ROUNDS; ++i) {
+        int k = tid * 8 + i * 8192;
+        if (k < vocab) {
+            float4 b0 = *(const float4 *)(bias + k), b1 = *(const float4 *)(bias + k + 4);
+            biasTop = fmaxf(fmaxf(fmaxf(biasTop, fmaxf(b0.x, b0.y)), fmaxf(b0.z, b0.w)), fmaxf(fmaxf(b1.x, b1.y), fmaxf(b1.z, b1.w)));
+        }
+    }
+    for (; t < rows; t += gridDim.x) {
+#pragma unroll
+        for (int i = 0; i < ROW_ROUNDS; ++i) {
+            cur[i] = nxt[i];
+        }
+        if (t + (int)gridDim.x < rows) {
+            prefetch(t + gridDim.x);
+        }
+        bf16_t *grow = (bf16_t *)((uint8_t *)grad + (int64_t)t * ldGrad);
+        const int tg = target[t];
+        if (tg < 0) { // (workgroup-uniform) no label: zero gradient
+            for (int k = tid * 8; k < vocab; k += 8192) {
+                *(uint4 *)(grow + k) = make_uint4(0, 0, 0, 0);
+            }
+            continue;
+        }
+        // own reference: the largest logit (not below 0, as in the two-pass kernel) plus the largest bias of the thread's columns
+        v8h hm = cur[0];
+#pragma unroll
+        for (int i = 1; i < ROW_ROUNDS; ++i) {
+            hm = __builtin_elementwise_max(hm, cur[i]);
+        }
+        float m = 0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            m = fmaxf(m, (float)hm[e]);
+        }
+        m += biasTop;
+        float sum = 0;
+#pragma unroll
+        for (int i = 0; i < ROW_ROUNDS; ++i) {
+            int k = tid * 8 + i * 8192;
+            if (k < vocab) {
+                float4 b0 = *(const float4 *)(bias + k), b1 = *(const float4 *)(bias + k + 4);
+                const float bb[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+                v8h ex;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    float w = __builtin_amdgcn_exp2f((float)cur[i][e] + (bb[e] - m)); // hardware exp2: below 2^-126 flushed to zero
+                    sum += w;
+                    ex[e] = (_Float16)w;
+                }
+                cur[i] = ex;
+            }
+        }
+        float mx = WaveMax(m);
+        if ((tid & 63) == 0) {
+            redM[tid >> 6] = mx;
+        }
+        __syncthreads();
+        mx = redM[0];
+#pragma unroll
+        for (int w = 1; w < 16; ++w) {
+            mx = fmaxf(mx, redM[w]);
+        }
+        const float own = __builtin_amdgcn_exp2f(m - mx); // own reference -> row reference
+        sum = WaveSum(sum * own);
+        if ((tid & 63) == 0) {
+            redS[tid >> 6] = sum;
+        }
+        __syncthreads();
+        float total = 0;
+#pragma unroll
+        for (int w = 0; w < 16; ++w) {
+            total += redS[w];
+        }
+        const float scale = own / total;       // half -> probability
+        const float negScale = -scale * gradMult; // half -> gradient of a logit that is not the label
+#pragma unroll
+        for (int i = 0; i < ROW_ROUNDS; ++i) {
+            int k = tid * 8 + i * 8192;
+            if (k < vocab) {
+                float g[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    g[e] = (float)cur[i][e] * negScale;
+                }
+                if ((unsigned)(tg - k) < 8u) { // the label's chunk (one thread of the workgroup)
+                    float pr = 0;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        pr = e == tg - k ? (float)cur[i][e] * scale : pr;
+                    }
+                    const float gt = (1.f - pr) * gradMult;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        g[e] = e == tg - k ? gt : g[e];
+                    }
+                    if (lossSum) {
+                        atomicAdd(lossSum, logf(pr));
+                    }
+                }
+                *(uint4 *)(grow + k) = make_uint4(PackBf16x2(g[0], g[1]), PackBf16x2(g[2], g[3]), PackBf16x2(g[4], g[5]), PackBf16x2(g[6], g[7]));
+            }
+        }
+        __syncthreads(); // the reduction slots are free again
+    }
+}
 } // namespace
 
 #define STREAM ((hipStream_t)stream)
@@ -332,8 +467,14 @@ int Ts2FinalSoftmaxGradHalf(int rows, int vocab, const ts2_mat *logits, const fl
         ((uintptr_t)bias & 15)) {
         return TS2_ERR_ALIGN;
     }
-    hipLaunchKernelGGL(FinalSoftmaxGradHalf, dim3(rows), dim3(256), 0, STREAM, vocab, (const _Float16 *)logits->ptr, logits->strideBytes, bias, target,
-        gradMult, (bf16_t *)grad->ptr, grad->strideBytes, lossSum);
+    if (vocab >= 2048 && vocab <= ROW_ROUNDS * 8192) {
+        const int wgs = rows < 512 ? rows : 512; // one workgroup of 16 waves per CU is resident (registers); two per CU in the queue
+        hipLaunchKernelGGL(FinalSoftmaxGradHalfRow, dim3(wgs), dim3(1024), 0, STREAM, rows, vocab, (const _Float16 *)logits->ptr,
+            logits->strideBytes, bias, target, gradMult, (bf16_t *)grad->ptr, grad->strideBytes, lossSum);
+    } else {
+        hipLaunchKernelGGL(FinalSoftmaxGradHalf, dim3(rows), dim3(256), 0, STREAM, vocab, (const _Float16 *)logits->ptr, logits->strideBytes, bias,
+            target, gradMult, (bf16_t *)grad->ptr, grad->strideBytes, lossSum);
+    }
     TS2_CHECK_LAUNCH();
     return TS2_OK;
 }
