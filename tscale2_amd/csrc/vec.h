@@ -158,12 +158,12 @@ __device__ __forceinline__ F4 TileNormBackprop(F4 src, F4 grad)
 // logistic gate of the reference (ComputeLoLU, src/gpt/compute/gpu_lolu.cuh:11-22): sigmoid(2x) with the +-20 clamps
 __device__ __forceinline__ float LoLU1(float x)
 {
-    float arg = x * 2.f;
-    // hardware exp2 and reciprocal (about 1 ulp each): these kernels are otherwise bound by the expf/division instruction count
-    float w = __builtin_amdgcn_exp2f(arg * 1.44269504088896341f);
-    float r = w * __builtin_amdgcn_rcpf(1 + w);
-    r = arg > 20 ? 1.f : r;
-    return arg < -20 ? 0.f : r;
+    // 1 / (1 + e^-2x) with the hardware exp2 and reciprocal (about 1 ulp each): these kernels are otherwise bound by their VALU
+    // instruction count.  Above the upper clamp (2x > 20) e^-2x < 2^-24 and the result is exactly 1 without a test; for large
+    // negative x the exponential overflows to +inf, whose reciprocal is 0, so no intermediate can be NaN.
+    float w = __builtin_amdgcn_exp2f(x * -2.88539008177792681f);
+    float r = __builtin_amdgcn_rcpf(1 + w);
+    return x < -10.f ? 0.f : r;
 }
 
 __device__ __forceinline__ F4 LoLU4(F4 g)
