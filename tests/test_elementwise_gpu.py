@@ -216,6 +216,37 @@ def test_ffn_lolu_backward_and_forward_with_eight_elements_per_lane(L, orc):
     assert np.all(np.abs(got[:len_] - np.clip(want, -448, 448)) <= np.abs(want) * 2.0 ** -4 + 2.0 ** -10 * 1.01)
 
 
+def test_attention_lolu_backward_with_eight_elements_per_lane(L, orc):
+    """bf16 gradient in, e4m3 gate gradient and bf16 value gradient out (the model's fp8 attention backward) takes the kernel with
+    eight elements per lane: gate gradient within the e4m3 rounding of the oracle's, value gradient within the bf16 rounding, the
+    per-(head, row) sums <values, value gradient> within fp32 summation error, pad rows zero."""
+    print("case attention lolu 8-wide", flush=True)
+    r = np.random.default_rng(15)
+    len_, len_round, dim = 301, 384, 384
+    gate = torch.from_numpy((r.standard_normal((len_, dim)) * 2).astype(np.float32)).bfloat16()
+    vals = torch.from_numpy((r.standard_normal((len_, dim)) * 24).astype(np.float32)).bfloat16()
+    grad = torch.from_numpy((r.standard_normal((len_, dim)) * 8).astype(np.float32)).bfloat16()
+    gnp, vnp, dnp = gate.float().numpy(), vals.float().numpy(), grad.float().numpy()
+    vs = 1 / 24.0
+    vals_scaled = vnp * np.float32(vs)
+    dgate, dvals = orc.backprop_lolu(gnp, vals_scaled, dnp)
+    want_ds = np.zeros((dim // 128, len_), np.float32)
+    orc.lib.orc_compute_dscale(len_, dim // 128, 128, _ptr(vals_scaled), _ptr(dvals), _ptr(want_ds))
+    gg = torch.full((len_round, dim), 9, dtype=torch.uint8, device="cuda")
+    gv = torch.full((len_round, dim), 9, dtype=torch.bfloat16, device="cuda")
+    ds = torch.full((dim // 128, len_round), -1.0, device="cuda")
+    L.call("ts2_backprop_lolu_dscale", len_, len_round, gate.cuda().view(torch.int16), vals.cuda().view(torch.int16), vs,
+           grad.cuda().view(torch.int16), L.BF16, gg, L.E4M3, gv.view(torch.int16), L.BF16, ds)
+    torch.cuda.synchronize()
+    got_g = gg.view(torch.float8_e4m3fn).float().cpu().numpy()
+    got_v = gv.float().cpu().numpy()
+    assert np.all(got_g[len_:] == 0) and np.all(got_v[len_:] == 0)
+    assert np.all(np.abs(got_g[:len_] - np.clip(dgate, -448, 448)) <= np.abs(dgate) * 2.0 ** -4 + 2.0 ** -10 * 1.01)
+    np.testing.assert_allclose(got_v[:len_], dvals, rtol=2 ** -7, atol=1e-5)
+    np.testing.assert_allclose(ds.cpu().numpy()[:, :len_], want_ds, rtol=1e-4, atol=2e-4)
+    assert np.all(ds.cpu().numpy()[:, len_:] == 0)
+
+
 def test_row_max_quantise(L, orc):
     print("case rowmax", flush=True)
     r = np.random.default_rng(5)

@@ -501,6 +501,67 @@ __global__ void __launch_bounds__(256) BackpropLoLU8(int len, int lenRound, int 
     }
 }
 
+// The attention flavour (MODE 1) with eight elements per lane: bf16 gate, values and gradient in, e4m3 gate gradient and bf16 value
+// gradient out, and the per-(head, row) sum <values, value gradient> that the attention backward subtracts (dScale).
+__global__ void __launch_bounds__(256) BackpropLoLUAtt8(int len, int lenRound, int tiles, Mat gate, Mat vals, float valsScale, Mat gradArr,
+    Mat gradGate, Mat gradVals, Mat dScale)
+{
+    constexpr int UU = 2;
+    const int l16 = threadIdx.x & 15;
+    const long unit0 = ((long)blockIdx.x * 256 + threadIdx.x) >> 4; // (row, tile) units; consecutive units = consecutive tiles of a row
+    const long units = (long)lenRound * tiles;
+    const long stride = ((long)gridDim.x * 256) >> 4;
+    uint4 g[UU], v[UU], gr[UU];
+    int row[UU], tile[UU];
+    bool any[UU], live[UU];
+#pragma unroll
+    for (int k = 0; k < UU; ++k) {
+        long u = unit0 + k * stride;
+        any[k] = u < units;
+        row[k] = any[k] ? (int)(u / tiles) : 0;
+        tile[k] = any[k] ? (int)(u - (long)row[k] * tiles) : 0;
+        const int col = tile[k] * TILE + l16 * 8;
+        live[k] = any[k] && row[k] < len;
+        g[k] = live[k] ? *(const uint4 *)At<TBF16>(gate, row[k], col) : make_uint4(0, 0, 0, 0);
+        v[k] = live[k] ? *(const uint4 *)At<TBF16>(vals, row[k], col) : make_uint4(0, 0, 0, 0);
+        gr[k] = live[k] ? *(const uint4 *)At<TBF16>(gradArr, row[k], col) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int k = 0; k < UU; ++k) {
+        const uint32_t gw[4] = {g[k].x, g[k].y, g[k].z, g[k].w}, vw[4] = {v[k].x, v[k].y, v[k].z, v[k].w}, rw[4] = {gr[k].x, gr[k].y, gr[k].z, gr[k].w};
+        float resGate[8], resVals[8];
+        float dp = 0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const uint32_t sh = 0xffff0000u;
+            float ge = (e & 1) ? __uint_as_float(gw[e >> 1] & sh) : __uint_as_float(gw[e >> 1] << 16);
+            float ve = (e & 1) ? __uint_as_float(vw[e >> 1] & sh) : __uint_as_float(vw[e >> 1] << 16);
+            float de = (e & 1) ? __uint_as_float(rw[e >> 1] & sh) : __uint_as_float(rw[e >> 1] << 16);
+            float vv = ve * valsScale;
+            float mult = LoLU1(ge);
+            resGate[e] = de * vv * (mult * (1 - mult) * 2.f);
+            resVals[e] = de * mult;
+            dp += vv * resVals[e];
+        }
+        dp = Row16Sum(dp); // zero for rows past len: their inputs were read as zero
+        if (!any[k]) {
+            continue;
+        }
+        const int col = tile[k] * TILE + l16 * 8;
+        uint32_t og[2] = {0, 0}, ov[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            og[w >> 1] |= CvtPkE4m3(resGate[2 * w], resGate[2 * w + 1]) << ((w & 1) * 16);
+            ov[w] = PackBf16x2(resVals[2 * w], resVals[2 * w + 1]);
+        }
+        *(uint2 *)At<TE4M3>(gradGate, row[k], col) = make_uint2(og[0], og[1]);
+        *(uint4 *)At<TBF16>(gradVals, row[k], col) = make_uint4(ov[0], ov[1], ov[2], ov[3]);
+        if (l16 == 0) {
+            ScaleAt(dScale, tile[k], row[k]) = dp;
+        }
+    }
+}
+
 // Workgroups walk rows with a grid stride; a row stays in registers between the abs-max pass and the quantise pass when it has at
 // most 4096 elements (REG) and the next row is fetched before the current one is reduced, so a workgroup always has loads in
 // flight.  Longer rows are read twice (the second read is served by L2).
@@ -1280,6 +1341,15 @@ static int BackpropLoluImpl(int len, int lenRound, const ts2_mat *gate, const ts
         const long lanes = ((long)lenRound * tiles * 16 + 1) / 2;
         hipLaunchKernelGGL(BackpropLoLU8, dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, STREAM, len, lenRound, tiles, M(*gate), M(*vals), valsScale,
             ts, M(*grad), M(*gradGate), M(*gradVals));
+        TS2_CHECK_LAUNCH();
+        return TS2_OK;
+    }
+    if (MODE == 1 && gradType == TS2_BF16 && ggType == TS2_E4M3 && gvType == TS2_BF16 && Aligned16(gate->ptr, gate->strideBytes) &&
+        Aligned16(vals->ptr, vals->strideBytes) && Aligned16(grad->ptr, grad->strideBytes) && Aligned16(gradVals->ptr, gradVals->strideBytes) &&
+        (((uintptr_t)gradGate->ptr | gradGate->strideBytes) & 7) == 0) {
+        const long lanes = ((long)lenRound * tiles * 16 + 1) / 2;
+        hipLaunchKernelGGL(BackpropLoLUAtt8, dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, STREAM, len, lenRound, tiles, M(*gate), M(*vals),
+            valsScale, M(*grad), M(*gradGate), M(*gradVals), ds);
         TS2_CHECK_LAUNCH();
         return TS2_OK;
     }
