@@ -214,6 +214,11 @@ def test_ffn_lolu_backward_and_forward_with_eight_elements_per_lane(L, orc):
     got = res.view(torch.float8_e4m3fn).float().cpu().numpy()
     assert np.all(got[len_:] == 0)
     assert np.all(np.abs(got[:len_] - np.clip(want, -448, 448)) <= np.abs(want) * 2.0 ** -4 + 2.0 ** -10 * 1.01)
+    # a result whose rows start 8 bytes off a 16-byte boundary takes the kernel with eight elements per lane: same bytes
+    wide_res = torch.full((len_round, dim + 8), 9, dtype=torch.uint8, device="cuda")
+    L.call("ts2_matrix_lolu", len_, len_round, gate.cuda().view(torch.int16), vals.cuda().view(torch.int16), 0.5, wide_res[:, 8:], L.E4M3)
+    torch.cuda.synchronize()
+    assert torch.equal(wide_res[:, 8:], res) and torch.all(wide_res[:, :8] == 9)
 
 
 def test_attention_lolu_backward_with_eight_elements_per_lane(L, orc):

@@ -361,6 +361,30 @@ __global__ void __launch_bounds__(256) MatrixLoLU8(int len, int lenRound, int di
     }
 }
 
+// Sixteen elements per lane: two 16-byte loads per input (the second is served by the line the first brought in) and one 16-byte store
+__global__ void __launch_bounds__(256) MatrixLoLU16(int len, int lenRound, int dim16, Mat gate, Mat vals, float resMult, Mat res)
+{
+    const long id = (long)blockIdx.x * 256 + threadIdx.x;
+    const long total = (long)lenRound * dim16;
+    if (id >= total) {
+        return;
+    }
+    const int t = (int)(id / dim16), c = (int)(id - (long)t * dim16) * 16;
+    uint32_t out[4] = {0, 0, 0, 0};
+    if (t < len) {
+        const uint4 g0 = *(const uint4 *)At<TBF16>(gate, t, c), g1 = *(const uint4 *)At<TBF16>(gate, t, c + 8);
+        const uint4 v0 = *(const uint4 *)At<TBF16>(vals, t, c), v1 = *(const uint4 *)At<TBF16>(vals, t, c + 8);
+        const uint32_t gw[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w}, vw[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+        for (int w = 0; w < 8; ++w) {
+            float ga = __uint_as_float(gw[w] << 16), gb = __uint_as_float(gw[w] & 0xffff0000u);
+            float va = __uint_as_float(vw[w] << 16), vb = __uint_as_float(vw[w] & 0xffff0000u);
+            out[w >> 1] |= CvtPkE4m3(va * LoLU1(ga) * resMult, vb * LoLU1(gb) * resMult) << ((w & 1) * 16);
+        }
+    }
+    *(uint4 *)At<TE4M3>(res, t, c) = make_uint4(out[0], out[1], out[2], out[3]);
+}
+
 // MODE 0: FFN (tile-norm backward of vals fused); MODE 1: attention (dScale fused)
 template <class TGrad, class TOutG, class TOutV, int MODE>
 __global__ void __launch_bounds__(256) BackpropLoLU(int len, int lenRound, int tiles, Mat gate, Mat vals, float valsScale, Mat valsSrcTileScale,
@@ -1299,6 +1323,14 @@ extern "C" int ts2_matrix_lolu(int32_t len, int32_t lenRound, const ts2_mat *gat
         return TS2_ERR_SHAPE;
     }
     int tiles = dim / TILE;
+    if (resType == TS2_E4M3 && Aligned16(gate->ptr, gate->strideBytes) && Aligned16(vals->ptr, vals->strideBytes) &&
+        Aligned16(res->ptr, res->strideBytes)) {
+        const long lanes = (long)lenRound * (dim / 16);
+        hipLaunchKernelGGL(MatrixLoLU16, dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, STREAM, len, lenRound, dim / 16, M(*gate), M(*vals),
+            resMult, M(*res));
+        TS2_CHECK_LAUNCH();
+        return TS2_OK;
+    }
     if (resType == TS2_E4M3 && Aligned16(gate->ptr, gate->strideBytes) && Aligned16(vals->ptr, vals->strideBytes) &&
         (((uintptr_t)res->ptr | res->strideBytes) & 7) == 0) {
         const long lanes = ((long)lenRound * (dim / 8) + 1) / 2;
