@@ -7,6 +7,7 @@
 // thousands of workgroups on the 256 CUs; consecutive 32-lane groups walk consecutive tiles of a row, i.e. HBM accesses are fully
 // coalesced 512-byte (fp32) runs.  The reference launches one 32-thread block per (tile, row) (src/lib/cuda/cuda_graph.cuh:359-365).
 #include "vec.h"
+#include "internal.h"
 
 namespace
 {
@@ -860,7 +861,7 @@ __global__ void __launch_bounds__(256) TileAbsMax(int len, int dim, Mat src, con
 // lanes cover the 128 bytes of one destination row.
 template <class TSrc, bool QUANT>
 __global__ void __launch_bounds__(256) TransposeQuant(int len, int lenRound, Mat src, const float *rowMult, const float *tileMax, int kTile,
-    const int *rowIndex, Mat dst, float *tileScale)
+    const int *rowIndex, Mat dst, float *tileScale, const float *rowAbsMax)
 {
     constexpr int PITCH = 132;
     __shared__ __attribute__((aligned(16))) uint8_t buf[128 * PITCH];
@@ -872,9 +873,29 @@ __global__ void __launch_bounds__(256) TransposeQuant(int len, int lenRound, Mat
     constexpr int RPP = 256 / LPR;                 // rows per pass
     constexpr int EPL = 16 / SB;                   // elements per lane
     const int lr = tid / LPR, lc = tid % LPR;
-    float mult = 0;
+    float mult = 0, tm = 0;
     if (QUANT) {
-        float tm = tileMax[tBlock / kTile];          // one 128-row block lies inside one k-tile (kTile is a multiple of 128)
+        if (rowAbsMax) {
+            // the k-tile's abs-max from the row maxima (max over its rows of rowAbsMax[t] * |rowMult[t]|), as TileMaxFromRows forms it
+            __shared__ float redT[4];
+            const int k0 = (tBlock / kTile) * kTile;
+            float mx = 0;
+            for (int t = k0 + tid; t < k0 + kTile && t < len; t += 256) {
+                float m = rowAbsMax[t];
+                if (rowMult) {
+                    m *= fabsf(rowMult[t]);
+                }
+                mx = fmaxf(mx, m);
+            }
+            mx = WaveMax(mx);
+            if ((tid & 63) == 0) {
+                redT[tid >> 6] = mx;
+            }
+            __syncthreads();
+            tm = fmaxf(fmaxf(redT[0], redT[1]), fmaxf(redT[2], redT[3]));
+        } else {
+            tm = tileMax[tBlock / kTile];            // one 128-row block lies inside one k-tile (kTile is a multiple of 128)
+        }
         mult = tm > 0 ? 1 / (tm / 127) : 0.f;        // same two roundings as scale = max/127, mult = 1/scale
     }
     for (int r0 = 0; r0 < 128; r0 += RPP * 4) {
@@ -963,7 +984,6 @@ __global__ void __launch_bounds__(256) TransposeQuant(int len, int lenRound, Mat
         *(uint4 *)(dst.p + (int64_t)(x + i) * dst.ld + tcol) = make_uint4(out[i][0], out[i][1], out[i][2], out[i][3]);
     }
     if (QUANT && tileScale && blockIdx.x == 0 && tid == 0) {
-        float tm = tileMax[tBlock / kTile];
         tileScale[tBlock / kTile] = tm > 0 ? tm / 127 : 1.f;
     }
 }
@@ -1536,6 +1556,14 @@ extern "C" int ts2_tile_absmax(int32_t len, const ts2_mat *src, int32_t srcType,
 extern "C" int ts2_transpose_quant(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, const float *rowMult, const float *tileMax,
     int32_t kTile, const int32_t *rowIndex, const ts2_mat *dstT, int32_t dstType, float *tileScale, void *stream)
 {
+    return Ts2TransposeQuantRows(len, lenRound, src, srcType, rowMult, tileMax, nullptr, kTile, rowIndex, dstT, dstType, tileScale, stream);
+}
+
+// ts2_transpose_quant whose k-tile maxima may come from the row maxima instead (rowAbsMax, with tileMax null and no row index): the
+// kernel then forms each k-tile's maximum itself and the separate ts2_tile_max_from_rows launch is not needed
+int Ts2TransposeQuantRows(int len, int lenRound, const ts2_mat *src, int srcType, const float *rowMult, const float *tileMax, const float *rowAbsMax,
+    int kTile, const int *rowIndex, const ts2_mat *dstT, int dstType, float *tileScale, void *stream)
+{
     if (!src || !dstT) {
         return TS2_ERR_NULL;
     }
@@ -1550,19 +1578,22 @@ extern "C" int ts2_transpose_quant(int32_t len, int32_t lenRound, const ts2_mat 
     dim3 grid(dim / 128, lenRound / 128);
     bool quant = dstType == TS2_I8 && (srcType == TS2_BF16 || srcType == TS2_F32);
     if (quant) {
-        if (!tileMax || kTile <= 0 || kTile % 128) {
+        if ((!tileMax && !rowAbsMax) || (rowAbsMax && rowIndex) || kTile <= 0 || kTile % 128) {
             return TS2_ERR_SHAPE;
+        }
+        if (tileMax) {
+            rowAbsMax = nullptr;
         }
         if (srcType == TS2_BF16) {
             hipLaunchKernelGGL((TransposeQuant<TBF16, true>), grid, dim3(256), 0, STREAM, len, lenRound, M(*src), rowMult, tileMax, kTile, rowIndex,
-                M(*dstT), tileScale);
+                M(*dstT), tileScale, rowAbsMax);
         } else {
             hipLaunchKernelGGL((TransposeQuant<TF32, true>), grid, dim3(256), 0, STREAM, len, lenRound, M(*src), rowMult, tileMax, kTile, rowIndex,
-                M(*dstT), tileScale);
+                M(*dstT), tileScale, rowAbsMax);
         }
     } else if (ElemSize(srcType) == 1 && dstType == srcType) {
         hipLaunchKernelGGL((TransposeQuant<TI8, false>), grid, dim3(256), 0, STREAM, len, lenRound, M(*src), nullptr, nullptr, 128, rowIndex,
-            M(*dstT), nullptr);
+            M(*dstT), nullptr, nullptr);
     } else {
         return TS2_ERR_UNSUPPORTED;
     }

@@ -1,6 +1,7 @@
 // Linear-layer backward operator: the call sequences of TMatMulBuffers (src/gpt/compute/layer_cuda_base.cuh:153-250) expressed
 // over the kernels of this library.  Host code only; every step is enqueued on the caller's stream.
 #include "common.h"
+#include "internal.h"
 
 namespace
 {
@@ -136,14 +137,17 @@ extern "C" int ts2_matmul_backprop_delta(int32_t mode, int32_t len, int32_t lenR
             return TS2_ERR_SHAPE;
         }
         if (buf->gradRowAbsMax && buf->gradRowAbsMaxValid) {
-            rc = ts2_tile_max_from_rows(len, buf->gradRowAbsMax, srcRowScale, kTile, buf->tileMax, stream);
+            // the k-tile maxima follow from the row maxima of the dX pass: the transposing quantiser forms them itself
+            rc = Ts2TransposeQuantRows(len, lenRound, grad, gradType, srcRowScale, nullptr, buf->gradRowAbsMax, kTile, nullptr, &buf->gradT, TS2_I8,
+                buf->tileScale, stream);
         } else {
             rc = ts2_tile_absmax(len, grad, gradType, srcRowScale, kTile, buf->tileMax, 1, stream);
+            if (rc) {
+                return rc;
+            }
+            rc = ts2_transpose_quant(len, lenRound, grad, gradType, srcRowScale, buf->tileMax, kTile, nullptr, &buf->gradT, TS2_I8, buf->tileScale,
+                stream);
         }
-        if (rc) {
-            return rc;
-        }
-        rc = ts2_transpose_quant(len, lenRound, grad, gradType, srcRowScale, buf->tileMax, kTile, nullptr, &buf->gradT, TS2_I8, buf->tileScale, stream);
         if (rc) {
             return rc;
         }
