@@ -311,3 +311,50 @@ def test_half_results_are_the_rounded_fp32_results(ab, tile):
     assert torch.equal(c16.view(torch.float16), c32.half())
     assert (c16[500:] == 0).all()
     assert lib.gemm_nt(a, b, c16, t, L.F16, epilogue=L.EPI_ADD, check=False) == -3
+
+
+@pytest.mark.parametrize("cfg", [0, 1, 2])
+def test_products_per_group_of_contraction_rows_are_bit_exact(lib, orc, cfg):
+    """The per-expert delta mode: one product per group g over the contraction range groupOffsets[g] .. groupOffsets[g+1], written
+    to its own slab of C.  int8 operands with the int32 result must equal the oracle's product over that range, on the 128x128 and on
+    the 256x256 tile (cfg 0 lets the library choose: with the groups counted, 256x256 here); an empty group gives a zero slab."""
+    print(f"case grouped contraction cfg={cfg}", flush=True)
+    from tscale2_amd import lib as L
+    r = np.random.default_rng(40 + cfg)
+    m, n, k = 256, 512, 1792
+    offs = np.array([0, 384, 384, 1280, 1792], np.int32)          # group 1 is empty
+    groups = len(offs) - 1
+    a = r.integers(-128, 128, (m, k), dtype=np.int8)
+    b = r.integers(-128, 128, (n, k), dtype=np.int8)
+    tc = torch.full((groups * m, n), -7, dtype=torch.int32, device="cuda")
+    lib.gemm_nt(torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(), tc, L.I8, L.I32, tile_config=cfg, m=m,
+                group_offsets=torch.from_numpy(offs).cuda(), groups=groups, c_slab_bytes=m * n * 4)
+    torch.cuda.synchronize()
+    got = tc.cpu().numpy().reshape(groups, m, n)
+    for g in range(groups):
+        lo, hi = int(offs[g]), int(offs[g + 1])
+        want = orc_gemm_i8(orc, np.ascontiguousarray(a[:, lo:hi]), np.ascontiguousarray(b[:, lo:hi])) if hi > lo else np.zeros((m, n), np.int32)
+        assert np.array_equal(got[g], want), g
+
+
+def test_weight_slab_chosen_per_row_tile_is_bit_exact(lib, orc):
+    """The expert-grouped forward / dX mode: every 128-row tile of A multiplies the B slab its tileGroup entry names; tiles with -1
+    are skipped and leave C alone."""
+    print("case slab per row tile", flush=True)
+    from tscale2_amd import lib as L
+    r = np.random.default_rng(44)
+    m, n, k, slabs = 640, 256, 512, 3
+    tg = np.array([2, 0, -1, 1, 2], np.int32)
+    a = r.integers(-128, 128, (m, k), dtype=np.int8)
+    b = r.integers(-128, 128, (slabs * n, k), dtype=np.int8)
+    tc = torch.full((m, n), -7, dtype=torch.int32, device="cuda")
+    lib.gemm_nt(torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(), tc, L.I8, L.I32, n=n,
+                tile_group=torch.from_numpy(tg).cuda(), b_slab_bytes=n * k)
+    torch.cuda.synchronize()
+    got = tc.cpu().numpy()
+    for t, g in enumerate(tg):
+        rows = slice(t * 128, (t + 1) * 128)
+        if g < 0:
+            assert np.all(got[rows] == -7)
+        else:
+            assert np.array_equal(got[rows], orc_gemm_i8(orc, np.ascontiguousarray(a[rows]), np.ascontiguousarray(b[g * n:(g + 1) * n])))

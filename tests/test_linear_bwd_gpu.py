@@ -146,13 +146,14 @@ def test_fp8_linear_backward(L, orc):
     assert err <= 5e-3
 
 
+@pytest.mark.parametrize("dims", [(256, 512), (384, 128)])
 @pytest.mark.parametrize("mode", ["i8", "e4m3"])
-def test_delta_as_stored_slices_plus_pack_matches_the_single_pass(L, orc, mode):
+def test_delta_as_stored_slices_plus_pack_matches_the_single_pass(L, orc, mode, dims):
     """BackpropDelta with a `partial` workspace: the token axis is cut into slices whose products are stored in fp32 and packed from
     their sum.  Same quantised operands and the same exact int32 sums per k-tile; only the association of the fp32 additions differs
     (per slice, then across slices), so packed bytes may differ from the single-pass result by one unit in rare places."""
-    print("case delta split slices", mode, flush=True)
-    len_, src_dim, grad_dim, kt, splits = 2048, 256, 512, 256, 4
+    print("case delta split slices", mode, dims, flush=True)
+    (src_dim, grad_dim), len_, kt, splits = dims, 2048, 256, 4   # (384, 128): 128x128 tiles, as for the select matrix of a MoE layer
     r = np.random.default_rng(21)
     dy = (r.standard_normal((len_, grad_dim)) * (0.2 + r.random((len_, 1)))).astype(np.float32)
     x = orc.normalize_state(r.standard_normal((len_, src_dim)).astype(np.float32), src_dim // 128)

@@ -1528,7 +1528,7 @@ template <int TYPE> int DispatchTile(const ts2_gemm_args *a, const GemmP &p, hip
     int cfg = a->tileConfig & 3;
     if (cfg == 0) {
         // 256x256 tiles only when they still fill the chip; the k-tile-scaled kernel keeps a second accumulator set and needs 128x128
-        long tilesL = (long)(p.m / 256) * (p.n / 256) * (p.splitK > 1 ? p.splitK : 1);
+        long tilesL = (long)(p.m / 256) * (p.n / 256) * (p.splitK > 1 ? p.splitK : 1) * (p.groupOffsets ? p.splitK_groups : 1);
         cfg = (tilesL >= 192 || p.nSeg > 1) ? 1 : 2;
     }
     // the 256x256 kernel needs full tiles and has no room for the second accumulator set of the k-tile-scaled variant

@@ -269,8 +269,16 @@ int BackpropDXGroup(ts2_model *M, int count, TMatrix *const *W, const Arr *const
 // k-tiles and at least 4096 tokens long
 int DeltaSplits(ts2_model *M, int srcDim, int dstDim)
 {
-    if (M->mode != TS2_E4M3 || (srcDim % 256) || (dstDim % 256)) {
+    if (M->mode != TS2_E4M3) {
         return 1;
+    }
+    if ((srcDim % 256) || (dstDim % 256)) {
+        // 128x128 tiles (the select matrix of a MoE layer: 128 x dim): two workgroups per CU, slices of at least 2048 tokens
+        int tiles = (srcDim / 128) * (dstDim / 128), splits = 1;
+        while (splits < 32 && tiles * splits < 512 && M->R % (splits * 2 * 128) == 0 && M->R / (splits * 2) >= 2048) {
+            splits *= 2;
+        }
+        return splits;
     }
     int tiles = (srcDim / 256) * (dstDim / 256);
     if (tiles >= 192) {
