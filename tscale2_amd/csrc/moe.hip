@@ -119,12 +119,24 @@ __global__ void __launch_bounds__(RB) MoeLocalRank(int total, int experts, const
 }
 
 // step 2 (one workgroup): per expert exclusive prefix over blocks, padded expert offsets, tile -> expert table.  The blocks are cut
-// into 256/experts chunks (experts <= 256) that are summed by different threads, so no thread walks a long chain of dependent loads.
-__global__ void __launch_bounds__(256) MoeOffsets(int nBlocks, int experts, int lenMoe, int *blockCounts, int *expertOffset, int *xpTileExpertId)
+// into 1024/experts chunks (experts <= 256) that are summed by different threads, so no thread walks a long chain of dependent loads.
+// (the two serial passes over a thread's blocks are chains of dependent global accesses: with useLds the table is staged in LDS,
+// scanned there and written back, all with coalesced accesses - 48 -> a few microseconds for 256 blocks x 64 experts)
+__global__ void __launch_bounds__(1024) MoeOffsets(int nBlocks, int experts, int lenMoe, int *blockCountsGlobal, int *expertOffset, int *xpTileExpertId,
+    int useLds)
 {
-    __shared__ int chunkSum[256];
-    __shared__ int counts[256];
-    const int chunks = 256 / experts > 0 ? 256 / experts : 1;
+    extern __shared__ int stage[];
+    constexpr int NT = 1024; // threads: experts x chunks of blocks; the passes over a chunk are serial, so many short chunks
+    __shared__ int chunkSum[NT];
+    __shared__ int counts[NT];
+    int *blockCounts = useLds ? stage : blockCountsGlobal;
+    if (useLds) {
+        for (int i = threadIdx.x; i < nBlocks * experts; i += NT) {
+            stage[i] = blockCountsGlobal[i];
+        }
+        __syncthreads();
+    }
+    const int chunks = NT / experts > 0 ? NT / experts : 1;
     const int e = threadIdx.x % experts, ch = threadIdx.x / experts;
     const int per = (nBlocks + chunks - 1) / chunks;
     const int b0 = ch * per, b1 = min(nBlocks, b0 + per);
@@ -163,7 +175,12 @@ __global__ void __launch_bounds__(256) MoeOffsets(int nBlocks, int experts, int 
         expertOffset[experts + 1] = lenMoe;
     }
     __syncthreads();
-    for (int x = threadIdx.x; x <= experts; x += 256) {
+    if (useLds) {
+        for (int i = threadIdx.x; i < nBlocks * experts; i += NT) {
+            blockCountsGlobal[i] = stage[i];
+        }
+    }
+    for (int x = threadIdx.x; x <= experts; x += NT) {
         int kStart = expertOffset[x] / TILE, kFinish = expertOffset[x + 1] / TILE;
         int res = x == experts ? -1 : x;
         for (int k = kStart; k < kFinish; ++k) {
@@ -407,7 +424,17 @@ extern "C" int ts2_moe_route(int32_t len, int32_t lenMoe, int32_t experts, int32
     int nBlocks = (total + RB - 1) / RB;
     hipLaunchKernelGGL(MoeLocalRank, dim3(nBlocks), dim3(RB), 0, STREAM, total, experts, tb->sampleExpertIds, tb->sampleExpertOffset, tb->blockCounts);
     TS2_CHECK_LAUNCH();
-    hipLaunchKernelGGL(MoeOffsets, dim3(1), dim3(256), 0, STREAM, nBlocks, experts, lenMoe, tb->blockCounts, tb->expertOffset, tb->xpTileExpertId);
+    const size_t tableBytes = (size_t)nBlocks * experts * 4;
+    const int useLds = tableBytes <= 150 * 1024;
+    static bool attrDone = false;
+    if (!attrDone) {
+        if (hipFuncSetAttribute((const void *)MoeOffsets, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) != hipSuccess) {
+            return TS2_ERR_LAUNCH;
+        }
+        attrDone = true;
+    }
+    hipLaunchKernelGGL(MoeOffsets, dim3(1), dim3(1024), useLds ? tableBytes : 0, STREAM, nBlocks, experts, lenMoe, tb->blockCounts, tb->expertOffset,
+        tb->xpTileExpertId, useLds);
     TS2_CHECK_LAUNCH();
     hipLaunchKernelGGL(MoeInitXp, dim3((lenMoe + 255) / 256), dim3(256), 0, STREAM, lenMoe, tb->xpSampleId, tb->xpSampleWeight);
     TS2_CHECK_LAUNCH();
