@@ -168,6 +168,14 @@ int ts2_backprop_row_tile_normalize_lolu(int32_t len, int32_t lenRound, const ts
     const ts2_mat *valsSrcTileScale, const ts2_mat *grad, int32_t gradType, const ts2_mat *gradGate, const ts2_mat *gradVals,
     int32_t gradOutType, void *stream);
 
+/* The same for TS2_BF16 gradients and TS2_E4M3 results, leaving also the transposed copies gradGateT, gradValsT [dim][lenRound] that
+ * the delta products of the two matrices contract over (the reference's producers can save a transposed copy the same way: saveTransposed
+ * of ComputeRG, src/gpt/compute/layer_moe.cu:117, and the transposing MoeGroupSamples, moe_kernels.cuh:89-143).  BackpropDelta is then
+ * called with gradT pointing at the copy and gradTValid set.  lenRound must be a multiple of 128. */
+int ts2_backprop_row_tile_normalize_lolu_t(int32_t len, int32_t lenRound, const ts2_mat *gate, const ts2_mat *vals, float valsScale,
+    const ts2_mat *valsSrcTileScale, const ts2_mat *grad, const ts2_mat *gradGate, const ts2_mat *gradVals, const ts2_mat *gradGateT,
+    const ts2_mat *gradValsT, void *stream);
+
 /* BackpropLoLUdScale, src/gpt/compute/gpu_lolu.cuh:141-173 (attention): gate backward plus dScale[head][t] = <vals*valsScale,
  * gradVals> per 128-wide head. */
 int ts2_backprop_lolu_dscale(int32_t len, int32_t lenRound, const ts2_mat *gate, const ts2_mat *vals, float valsScale, const ts2_mat *grad,
@@ -238,6 +246,9 @@ typedef struct ts2_matmul_bwd_buffers {
     /* != 0: srcT already holds the transpose of the `src` given to BackpropDelta (an earlier BackpropDelta call with the same buffers
      * and the same source tensor left it there, as for the matrices of one layer that share their input); the transpose is skipped. */
     int32_t srcTValid;
+    /* != 0 (E4M3): gradT already holds the transpose of the `grad` given to BackpropDelta (its producer wrote it, e.g.
+     * ts2_backprop_row_tile_normalize_lolu_t); the transpose is skipped. */
+    int32_t gradTValid;
 } ts2_matmul_bwd_buffers;
 
 /* BackpropMulti (prep of dX): I8: quantise grad (TS2_BF16 | TS2_F32, optionally times gradColScale[gradDim]) per row to

@@ -221,6 +221,34 @@ def test_ffn_lolu_backward_and_forward_with_eight_elements_per_lane(L, orc):
     assert torch.equal(wide_res[:, 8:], res) and torch.all(wide_res[:, :8] == 9)
 
 
+def test_ffn_lolu_backward_that_also_writes_the_transposed_gradients(L, orc):
+    """ts2_backprop_row_tile_normalize_lolu_t: same bytes as ts2_backprop_row_tile_normalize_lolu for bf16 gradients and e4m3 results
+    (itself checked against the oracle above), and the two transposed copies are exactly those bytes transposed, pad rows (columns of
+    the copies) zero."""
+    print("case lolu e4m3 with transposed copies", flush=True)
+    r = np.random.default_rng(16)
+    len_, len_round, dim = 301, 384, 384
+    gate = torch.from_numpy((r.standard_normal((len_, dim)) * 2).astype(np.float32)).bfloat16().cuda().view(torch.int16)
+    vnp = (r.standard_normal((len_, dim)) * 24).astype(np.float32)
+    vnp[7, 128:256] = 0
+    vals = torch.from_numpy(vnp).bfloat16().cuda().view(torch.int16)
+    grad = torch.from_numpy((r.standard_normal((len_, dim)) * 8).astype(np.float32)).bfloat16().cuda().view(torch.int16)
+    vs = 1 / 24.0
+    tsc = (r.random((dim // 128, len_)) + 0.5).astype(np.float32) * np.float32(vs)
+    tsc[1, 7] = 0
+    gg = torch.full((len_round, dim), 9, dtype=torch.uint8, device="cuda")
+    gv = torch.full((len_round, dim), 9, dtype=torch.uint8, device="cuda")
+    L.call("ts2_backprop_row_tile_normalize_lolu", len_, len_round, gate, vals, vs, dev(tsc), grad, L.BF16, gg, gv, L.E4M3)
+    gg2, gv2 = torch.full_like(gg, 5), torch.full_like(gv, 5)
+    ggT = torch.full((dim, len_round), 5, dtype=torch.uint8, device="cuda")
+    gvT = torch.full((dim, len_round), 5, dtype=torch.uint8, device="cuda")
+    L.call("ts2_backprop_row_tile_normalize_lolu_t", len_, len_round, gate, vals, vs, dev(tsc), grad, gg2, gv2, ggT, gvT)
+    torch.cuda.synchronize()
+    assert torch.equal(gg2, gg) and torch.equal(gv2, gv)
+    assert torch.equal(ggT, gg.T.contiguous()) and torch.equal(gvT, gv.T.contiguous())
+    assert torch.all(gg2[len_:] == 0) and torch.all(gvT[:, len_:] == 0)
+
+
 def test_attention_lolu_backward_with_eight_elements_per_lane(L, orc):
     """bf16 gradient in, e4m3 gate gradient and bf16 value gradient out (the model's fp8 attention backward) takes the kernel with
     eight elements per lane: gate gradient within the e4m3 rounding of the oracle's, value gradient within the bf16 rounding, the

@@ -526,6 +526,113 @@ __global__ void __launch_bounds__(256) BackpropLoLU8(int len, int lenRound, int 
     }
 }
 
+// A 128 x 128 block of bytes staged in LDS as [t][x] (pitch PITCH) goes out transposed: dst[x][t], 16 bytes (16 t) per store.
+// thread -> (tq = block of 16 t, xq = x quad)
+template <int PITCH> __device__ __forceinline__ void TransposeOut128(const uint8_t *buf, const Mat &dst, int xBlock, int tBlock, int tid)
+{
+    const int tq = tid & 7, xq = tid >> 3;
+    uint32_t out[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint8_t *b = buf + (tq * 16 + j * 4) * PITCH + xq * 4;
+        uint32_t r0 = *(const uint32_t *)(b);
+        uint32_t r1 = *(const uint32_t *)(b + PITCH);
+        uint32_t r2 = *(const uint32_t *)(b + 2 * PITCH);
+        uint32_t r3 = *(const uint32_t *)(b + 3 * PITCH);
+        // 4x4 byte transpose.  __builtin_amdgcn_perm(hi, lo, sel): result byte i = byte sel[i] of {hi:lo} (lo = bytes 0-3)
+        uint32_t a = __builtin_amdgcn_perm(r1, r0, 0x05010400); // r0.b0 r1.b0 r0.b1 r1.b1
+        uint32_t bb = __builtin_amdgcn_perm(r1, r0, 0x07030602); // r0.b2 r1.b2 r0.b3 r1.b3
+        uint32_t c = __builtin_amdgcn_perm(r3, r2, 0x05010400);
+        uint32_t d = __builtin_amdgcn_perm(r3, r2, 0x07030602);
+        out[0][j] = __builtin_amdgcn_perm(c, a, 0x05040100); // column 0: r0.b0 r1.b0 r2.b0 r3.b0
+        out[1][j] = __builtin_amdgcn_perm(c, a, 0x07060302);
+        out[2][j] = __builtin_amdgcn_perm(d, bb, 0x05040100);
+        out[3][j] = __builtin_amdgcn_perm(d, bb, 0x07060302);
+    }
+    int x = xBlock + xq * 4;
+    int tcol = tBlock + tq * 16;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        *(uint4 *)(dst.p + (int64_t)(x + i) * dst.ld + tcol) = make_uint4(out[i][0], out[i][1], out[i][2], out[i][3]);
+    }
+}
+
+// BackpropLoLU8 that also leaves the transposed copies of both results (gradGateT, gradValsT: [dim][lenRound]) which the delta
+// products of the two matrices contract over: a workgroup takes a block of 128 rows x one tile, computes it 16 rows at a time with
+// the arithmetic of BackpropLoLU8, stores the row-major bytes and stages them in LDS for the transposed stores.  Saves reading both
+// results back for their transposes.
+__global__ void __launch_bounds__(256) BackpropLoLU8T(int len, int lenRound, Mat gate, Mat vals, float valsScale, Mat valsSrcTileScale, Mat gradArr,
+    Mat gradGate, Mat gradVals, Mat gradGateT, Mat gradValsT)
+{
+    constexpr int PITCH = 132;
+    __shared__ __attribute__((aligned(16))) uint8_t bufG[128 * PITCH], bufV[128 * PITCH];
+    const int tid = threadIdx.x, l16 = tid & 15, lr = tid >> 4;
+    const int tile = blockIdx.x, tBlock = blockIdx.y * 128;
+    const int col = tile * TILE + l16 * 8;
+    for (int r0 = 0; r0 < 128; r0 += 64) {
+        uint4 g[4], v[4], gr[4];
+        float ts[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int row = tBlock + r0 + k * 16 + lr;
+            const bool live = row < len;
+            g[k] = live ? *(const uint4 *)At<TBF16>(gate, row, col) : make_uint4(0, 0, 0, 0);
+            v[k] = live ? *(const uint4 *)At<TBF16>(vals, row, col) : make_uint4(0, 0, 0, 0);
+            gr[k] = live ? *(const uint4 *)At<TBF16>(gradArr, row, col) : make_uint4(0, 0, 0, 0);
+            ts[k] = live ? ScaleAt(valsSrcTileScale, tile, row) : 0.f;
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int r = r0 + k * 16 + lr, row = tBlock + r;
+            const uint32_t gw[4] = {g[k].x, g[k].y, g[k].z, g[k].w}, vw[4] = {v[k].x, v[k].y, v[k].z, v[k].w}, rw[4] = {gr[k].x, gr[k].y, gr[k].z, gr[k].w};
+            float resGate[8], resVals[8], src[8];
+            float sum2 = 0, dp = 0;
+            const float srcMult = ts[k] / valsScale;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t sh = 0xffff0000u;
+                float ge = (e & 1) ? __uint_as_float(gw[e >> 1] & sh) : __uint_as_float(gw[e >> 1] << 16);
+                float ve = (e & 1) ? __uint_as_float(vw[e >> 1] & sh) : __uint_as_float(vw[e >> 1] << 16);
+                float de = (e & 1) ? __uint_as_float(rw[e >> 1] & sh) : __uint_as_float(rw[e >> 1] << 16);
+                float vv = ve * valsScale;
+                float mult = LoLU1(ge);
+                resGate[e] = de * vv * (mult * (1 - mult) * 2.f);
+                resVals[e] = de * mult;
+                src[e] = vv * srcMult;
+                sum2 += src[e] * src[e];
+                dp += src[e] * resVals[e];
+            }
+            sum2 = Row16Sum(sum2);
+            dp = Row16Sum(dp);
+            uint32_t og[2] = {0, 0}, ov[2] = {0, 0};
+            if (row < len) {
+                float sigma = 0, scale = 0;
+                if (sum2 != 0) {
+                    float inv = 1 / sum2;
+                    sigma = dp * inv;
+                    scale = sqrtf(TILE * inv);
+                }
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    float a0 = sum2 != 0 ? (resVals[2 * w] - src[2 * w] * sigma) * scale : 0.f;
+                    float a1 = sum2 != 0 ? (resVals[2 * w + 1] - src[2 * w + 1] * sigma) * scale : 0.f;
+                    ov[w >> 1] |= CvtPkE4m3(a0, a1) << ((w & 1) * 16);
+                    og[w >> 1] |= CvtPkE4m3(resGate[2 * w], resGate[2 * w + 1]) << ((w & 1) * 16);
+                }
+            }
+            *(uint2 *)At<TE4M3>(gradGate, row, col) = make_uint2(og[0], og[1]);
+            *(uint2 *)At<TE4M3>(gradVals, row, col) = make_uint2(ov[0], ov[1]);
+            *(uint32_t *)(bufG + r * PITCH + l16 * 8) = og[0];
+            *(uint32_t *)(bufG + r * PITCH + l16 * 8 + 4) = og[1];
+            *(uint32_t *)(bufV + r * PITCH + l16 * 8) = ov[0];
+            *(uint32_t *)(bufV + r * PITCH + l16 * 8 + 4) = ov[1];
+        }
+    }
+    __syncthreads();
+    TransposeOut128<PITCH>(bufG, gradGateT, tile * TILE, tBlock, tid);
+    TransposeOut128<PITCH>(bufV, gradValsT, tile * TILE, tBlock, tid);
+}
+
 // The attention flavour (MODE 1) with eight elements per lane: bf16 gate, values and gradient in, e4m3 gate gradient and bf16 value
 // gradient out, and the per-(head, row) sum <values, value gradient> that the attention backward subtracts (dScale).
 __global__ void __launch_bounds__(256) BackpropLoLUAtt8(int len, int lenRound, int tiles, Mat gate, Mat vals, float valsScale, Mat gradArr,
@@ -957,32 +1064,7 @@ __global__ void __launch_bounds__(256) TransposeQuant(int len, int lenRound, Mat
         }
     }
     __syncthreads();
-    // transpose: thread -> (tq = block of 16 t, xq = x quad)
-    const int tq = tid & 7, xq = tid >> 3;
-    uint32_t out[4][4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const uint8_t *b = buf + (tq * 16 + j * 4) * PITCH + xq * 4;
-        uint32_t r0 = *(const uint32_t *)(b);
-        uint32_t r1 = *(const uint32_t *)(b + PITCH);
-        uint32_t r2 = *(const uint32_t *)(b + 2 * PITCH);
-        uint32_t r3 = *(const uint32_t *)(b + 3 * PITCH);
-        // 4x4 byte transpose.  __builtin_amdgcn_perm(hi, lo, sel): result byte i = byte sel[i] of {hi:lo} (lo = bytes 0-3)
-        uint32_t a = __builtin_amdgcn_perm(r1, r0, 0x05010400); // r0.b0 r1.b0 r0.b1 r1.b1
-        uint32_t bb = __builtin_amdgcn_perm(r1, r0, 0x07030602); // r0.b2 r1.b2 r0.b3 r1.b3
-        uint32_t c = __builtin_amdgcn_perm(r3, r2, 0x05010400);
-        uint32_t d = __builtin_amdgcn_perm(r3, r2, 0x07030602);
-        out[0][j] = __builtin_amdgcn_perm(c, a, 0x05040100); // column 0: r0.b0 r1.b0 r2.b0 r3.b0
-        out[1][j] = __builtin_amdgcn_perm(c, a, 0x07060302);
-        out[2][j] = __builtin_amdgcn_perm(d, bb, 0x05040100);
-        out[3][j] = __builtin_amdgcn_perm(d, bb, 0x07060302);
-    }
-    int x = xBlock + xq * 4;
-    int tcol = tBlock + tq * 16;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        *(uint4 *)(dst.p + (int64_t)(x + i) * dst.ld + tcol) = make_uint4(out[i][0], out[i][1], out[i][2], out[i][3]);
-    }
+    TransposeOut128<PITCH>(buf, dst, xBlock, tBlock, tid);
     if (QUANT && tileScale && blockIdx.x == 0 && tid == 0) {
         tileScale[tBlock / kTile] = tm > 0 ? tm / 127 : 1.f;
     }
@@ -1680,6 +1762,30 @@ extern "C" int ts2_pack_delta(const ts2_mat *partial, int32_t splits, int64_t sl
     int tiles = cols / TILE;
     hipLaunchKernelGGL(PackDelta, GridFor(rows, tiles), dim3(256), 0, STREAM, rows, tiles, splits, (const uint8_t *)partial->ptr, partial->strideBytes,
         slabBytes, alpha, alphaPtr, M(*delta), M(*deltaTileScale));
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
+extern "C" int ts2_backprop_row_tile_normalize_lolu_t(int32_t len, int32_t lenRound, const ts2_mat *gate, const ts2_mat *vals, float valsScale,
+    const ts2_mat *valsSrcTileScale, const ts2_mat *grad, const ts2_mat *gradGate, const ts2_mat *gradVals, const ts2_mat *gradGateT,
+    const ts2_mat *gradValsT, void *stream)
+{
+    if (!gate || !vals || !valsSrcTileScale || !grad || !gradGate || !gradVals || !gradGateT || !gradValsT) {
+        return TS2_ERR_NULL;
+    }
+    int dim = grad->x;
+    if (dim % TILE || lenRound % 128 || lenRound < len || !MatOk(gate, len, dim, 2) || !MatOk(vals, len, dim, 2) || !MatOk(grad, len, dim, 2) ||
+        !MatOk(gradGate, lenRound, dim, 1) || !MatOk(gradVals, lenRound, dim, 1) || !MatOk(gradGateT, dim, lenRound, 1) ||
+        !MatOk(gradValsT, dim, lenRound, 1) || !MatOk(valsSrcTileScale, dim / TILE, len, 4)) {
+        return TS2_ERR_SHAPE;
+    }
+    if (!Aligned16(gate->ptr, gate->strideBytes) || !Aligned16(vals->ptr, vals->strideBytes) || !Aligned16(grad->ptr, grad->strideBytes) ||
+        !Aligned16(gradGateT->ptr, gradGateT->strideBytes) || !Aligned16(gradValsT->ptr, gradValsT->strideBytes) ||
+        (((uintptr_t)gradGate->ptr | gradGate->strideBytes | (uintptr_t)gradVals->ptr | gradVals->strideBytes) & 7)) {
+        return TS2_ERR_ALIGN;
+    }
+    hipLaunchKernelGGL(BackpropLoLU8T, dim3(dim / TILE, lenRound / 128), dim3(256), 0, STREAM, len, lenRound, M(*gate), M(*vals), valsScale,
+        M(*valsSrcTileScale), M(*grad), M(*gradGate), M(*gradVals), M(*gradGateT), M(*gradValsT));
     TS2_CHECK_LAUNCH();
     return TS2_OK;
 }

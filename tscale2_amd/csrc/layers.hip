@@ -136,6 +136,7 @@ struct ts2_model {
     Arr logits16;                            // IEEE-half logits of the backward pass (the fp32 ones serve ts2_model_forward)
     // linear backward scratch
     uint8_t *sGrad8 = 0, *sGradT = 0, *sSrcT = 0, *sWT = 0;
+    uint8_t *sGradTa = 0, *sGradTb = 0; // transposed gradients written by their producer (fp8 FFN backward)
     float *sPartial = 0;                     // fp32 slices of a delta product with few output tiles
     size_t sPartialFloats = 0;
     float *sRowScale = 0, *sTileMax = 0, *sTileScale = 0;
@@ -293,10 +294,14 @@ int DeltaSplits(ts2_model *M, int srcDim, int dstDim)
 
 // delta = alpha * gradScale * gradFast^T * src8   (TMatMulBuffers::BackpropDelta)
 int BackpropDelta(ts2_model *M, TMatrix &W, const Arr &src8, const Arr &gradFast, float alpha, const float *gradScale, void *s,
-    bool sameSrcAsLastCall = false)
+    bool sameSrcAsLastCall = false, const Arr *gradTReady = nullptr)
 {
     ts2_matmul_bwd_buffers b = Scratch(M, M->R, W.srcDim, W.dstDim);
     b.srcTValid = sameSrcAsLastCall; // the matrices of a layer that share their input transpose it once
+    if (gradTReady) { // the producer of the gradient left its transpose
+        b.gradT = gradTReady->m;
+        b.gradTValid = 1;
+    }
     // a delta with fewer large tiles than the chip has CUs runs as slices of the token axis on the large tile, packed afterwards
     int splits = DeltaSplits(M, W.srcDim, W.dstDim);
     if (splits > 1 && (size_t)splits * W.dstDim * W.srcDim <= M->sPartialFloats) {
@@ -341,8 +346,16 @@ int FfnBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
     }
     // contract backward
     CK(BackpropDX(M, L.w[2], M->stateGradFast, DISCR * Dot(F), true, drg, false, s));
-    CK(ts2_backprop_row_tile_normalize_lolu(len, R, gate16.P(), wide16.P(), VEC, wideScale.P(), drg.P(), TS2_BF16, dgate.P(), dwide.P(),
-        M->fastGradType, s));
+    // fp8: the gate/norm backward also writes the transposed gradients that the two delta products contract over
+    const bool fusedT = M->mode == TS2_E4M3 && M->fastGradType == TS2_E4M3 && M->sGradTa && (R % 128) == 0;
+    Arr dwideT = Flat(M->sGradTa, F, R, TS2_E4M3), dgateT = Flat(M->sGradTb, F, R, TS2_E4M3);
+    if (fusedT) {
+        CK(ts2_backprop_row_tile_normalize_lolu_t(len, R, gate16.P(), wide16.P(), VEC, wideScale.P(), drg.P(), dgate.P(), dwide.P(), dgateT.P(),
+            dwideT.P(), s));
+    } else {
+        CK(ts2_backprop_row_tile_normalize_lolu(len, R, gate16.P(), wide16.P(), VEC, wideScale.P(), drg.P(), TS2_BF16, dgate.P(), dwide.P(),
+            M->fastGradType, s));
+    }
     {
         TMatrix *const ws[2] = {&L.w[0], &L.w[1]};
         const Arr *const gs[2] = {&dwide, &dgate};
@@ -351,8 +364,8 @@ int FfnBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
     }
     // deltas (sources are stored in 1/24 units)
     CK(BackpropDelta(M, L.w[2], rg8, M->stateGradFast, VEC, gradScale, s));
-    CK(BackpropDelta(M, L.w[0], norm8, dwide, VEC, gradScale, s));
-    return BackpropDelta(M, L.w[1], norm8, dgate, VEC, gradScale, s, true);
+    CK(BackpropDelta(M, L.w[0], norm8, dwide, VEC, gradScale, s, false, fusedT ? &dwideT : nullptr));
+    return BackpropDelta(M, L.w[1], norm8, dgate, VEC, gradScale, s, true, fusedT ? &dgateT : nullptr);
 }
 
 // ---------------------------------------------------------------------------------------------------------------------------
@@ -866,6 +879,11 @@ extern "C" ts2_model *ts2_model_create(const ts2_model_config *cfg)
     // keep the two statistics arrays on one stride
     M->sGrad8 = (uint8_t *)M->Dev((size_t)RP * maxW);
     M->sGradT = (uint8_t *)M->Dev((size_t)RP * maxW);
+    if (M->mode == TS2_E4M3) {
+        M->sGradTa = (uint8_t *)M->Dev((size_t)RP * maxW);
+        M->sGradTb = (uint8_t *)M->Dev((size_t)RP * maxW);
+        ok &= M->sGradTa && M->sGradTb;
+    }
     M->sSrcT = (uint8_t *)M->Dev((size_t)RP * maxW);
     M->sWT = (uint8_t *)M->Dev((size_t)4 * maxW * maxW); // up to four transposed weights side by side (BackpropDXGroup)
     M->sPartialFloats = (size_t)8 * 2048 * 2048; // eight slices of a 2048 x 2048 delta, four of a 4096 x 2048 one

@@ -157,9 +157,11 @@ extern "C" int ts2_matmul_backprop_delta(int32_t mode, int32_t len, int32_t lenR
         if (gradType != TS2_E4M3) {
             return TS2_ERR_UNSUPPORTED;
         }
-        rc = ts2_transpose_quant(len, lenRound, grad, TS2_E4M3, nullptr, nullptr, 0, nullptr, &buf->gradT, TS2_E4M3, nullptr, stream);
-        if (rc) {
-            return rc;
+        if (!buf->gradTValid) {
+            rc = ts2_transpose_quant(len, lenRound, grad, TS2_E4M3, nullptr, nullptr, 0, nullptr, &buf->gradT, TS2_E4M3, nullptr, stream);
+            if (rc) {
+                return rc;
+            }
         }
     }
     if (!buf->srcTValid) {
