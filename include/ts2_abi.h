@@ -162,12 +162,6 @@ int ts2_scale_grad(const float *gradMaxNorm, const float *prevGradMult, const ts
 int ts2_matrix_lolu(int32_t len, int32_t lenRound, const ts2_mat *gate, const ts2_mat *vals, float resMult, const ts2_mat *res,
     int32_t resType, void *stream);
 
-/* The same for a TS2_E4M3 result, leaving also its transposed copy resT [dim][lenRound]: res is the source of the next matrix and its
- * delta product contracts over the token axis (BackpropDelta is then called with srcT pointing at the copy and srcTValid set; the
- * reference's ComputeRG has the same option, saveTransposed, src/gpt/compute/layer_moe.cu:117).  lenRound a multiple of 128. */
-int ts2_matrix_lolu_t(int32_t len, int32_t lenRound, const ts2_mat *gate, const ts2_mat *vals, float resMult, const ts2_mat *res,
-    const ts2_mat *resT, void *stream);
-
 /* BackpropRowTileNormalizeLoLU, src/gpt/compute/gpu_lolu.cuh:107-137 (FFN): vals*valsScale is the normalised "wide"; gradGate =
  * grad*vals*m(1-m)*2, gradVals = tile-norm backward of (grad*m) against vals*valsSrcTileScale; outputs as gradOutType. */
 int ts2_backprop_row_tile_normalize_lolu(int32_t len, int32_t lenRound, const ts2_mat *gate, const ts2_mat *vals, float valsScale,

@@ -219,12 +219,6 @@ def test_ffn_lolu_backward_and_forward_with_eight_elements_per_lane(L, orc):
     L.call("ts2_matrix_lolu", len_, len_round, gate.cuda().view(torch.int16), vals.cuda().view(torch.int16), 0.5, wide_res[:, 8:], L.E4M3)
     torch.cuda.synchronize()
     assert torch.equal(wide_res[:, 8:], res) and torch.all(wide_res[:, :8] == 9)
-    # the variant that also leaves the transposed copy: same bytes, and the copy is their transpose
-    res2 = torch.full((len_round, dim), 5, dtype=torch.uint8, device="cuda")
-    res_t = torch.full((dim, len_round), 5, dtype=torch.uint8, device="cuda")
-    L.call("ts2_matrix_lolu_t", len_, len_round, gate.cuda().view(torch.int16), vals.cuda().view(torch.int16), 0.5, res2, res_t)
-    torch.cuda.synchronize()
-    assert torch.equal(res2, res) and torch.equal(res_t, res.T.contiguous())
 
 
 def test_ffn_lolu_backward_that_also_writes_the_transposed_gradients(L, orc):

@@ -386,84 +386,6 @@ __global__ void __launch_bounds__(256) MatrixLoLU16(int len, int lenRound, int d
     *(uint4 *)At<TE4M3>(res, t, c) = make_uint4(out[0], out[1], out[2], out[3]);
 }
 
-// A 128 x 128 block of bytes staged in LDS as [t][x] (pitch PITCH) goes out transposed: dst[x][t], 16 bytes (16 t) per store.
-// thread -> (tq = block of 16 t, xq = x quad)
-template <int PITCH> __device__ __forceinline__ void TransposeOut128(const uint8_t *buf, const Mat &dst, int xBlock, int tBlock, int tid)
-{
-    const int tq = tid & 7, xq = tid >> 3;
-    uint32_t out[4][4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const uint8_t *b = buf + (tq * 16 + j * 4) * PITCH + xq * 4;
-        uint32_t r0 = *(const uint32_t *)(b);
-        uint32_t r1 = *(const uint32_t *)(b + PITCH);
-        uint32_t r2 = *(const uint32_t *)(b + 2 * PITCH);
-        uint32_t r3 = *(const uint32_t *)(b + 3 * PITCH);
-        // 4x4 byte transpose.  __builtin_amdgcn_perm(hi, lo, sel): result byte i = byte sel[i] of {hi:lo} (lo = bytes 0-3)
-        uint32_t a = __builtin_amdgcn_perm(r1, r0, 0x05010400); // r0.b0 r1.b0 r0.b1 r1.b1
-        uint32_t bb = __builtin_amdgcn_perm(r1, r0, 0x07030602); // r0.b2 r1.b2 r0.b3 r1.b3
-        uint32_t c = __builtin_amdgcn_perm(r3, r2, 0x05010400);
-        uint32_t d = __builtin_amdgcn_perm(r3, r2, 0x07030602);
-        out[0][j] = __builtin_amdgcn_perm(c, a, 0x05040100); // column 0: r0.b0 r1.b0 r2.b0 r3.b0
-        out[1][j] = __builtin_amdgcn_perm(c, a, 0x07060302);
-        out[2][j] = __builtin_amdgcn_perm(d, bb, 0x05040100);
-        out[3][j] = __builtin_amdgcn_perm(d, bb, 0x07060302);
-    }
-    int x = xBlock + xq * 4;
-    int tcol = tBlock + tq * 16;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        *(uint4 *)(dst.p + (int64_t)(x + i) * dst.ld + tcol) = make_uint4(out[i][0], out[i][1], out[i][2], out[i][3]);
-    }
-}
-
-// MatrixLoLU16 that also leaves the transposed copy resT [dim][lenRound], which the delta product of the next matrix contracts over
-// (it is that product's source): a workgroup takes 128 rows x 128 columns, 32 rows at a time, stores the row-major bytes and stages
-// them in LDS for the transposed stores.
-__global__ void __launch_bounds__(256) MatrixLoLU16T(int len, int lenRound, Mat gate, Mat vals, float resMult, Mat res, Mat resT)
-{
-    constexpr int PITCH = 132;
-    __shared__ __attribute__((aligned(16))) uint8_t buf[128 * PITCH];
-    const int tid = threadIdx.x, l8 = tid & 7, lr = tid >> 3;
-    const int xBlock = blockIdx.x * 128, tBlock = blockIdx.y * 128;
-    const int c = xBlock + l8 * 16;
-    for (int r0 = 0; r0 < 128; r0 += 64) {
-        uint4 g[2][2], v[2][2];
-#pragma unroll
-        for (int k = 0; k < 2; ++k) {
-            const int t = tBlock + r0 + k * 32 + lr;
-            const bool live = t < len;
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                g[k][h] = live ? *(const uint4 *)At<TBF16>(gate, t, c + 8 * h) : make_uint4(0, 0, 0, 0);
-                v[k][h] = live ? *(const uint4 *)At<TBF16>(vals, t, c + 8 * h) : make_uint4(0, 0, 0, 0);
-            }
-        }
-#pragma unroll
-        for (int k = 0; k < 2; ++k) {
-            const int r = r0 + k * 32 + lr, t = tBlock + r;
-            const uint32_t gw[8] = {g[k][0].x, g[k][0].y, g[k][0].z, g[k][0].w, g[k][1].x, g[k][1].y, g[k][1].z, g[k][1].w};
-            const uint32_t vw[8] = {v[k][0].x, v[k][0].y, v[k][0].z, v[k][0].w, v[k][1].x, v[k][1].y, v[k][1].z, v[k][1].w};
-            uint32_t out[4] = {0, 0, 0, 0};
-            if (t < len) {
-#pragma unroll
-                for (int w = 0; w < 8; ++w) {
-                    float ga = __uint_as_float(gw[w] << 16), gb = __uint_as_float(gw[w] & 0xffff0000u);
-                    float va = __uint_as_float(vw[w] << 16), vb = __uint_as_float(vw[w] & 0xffff0000u);
-                    out[w >> 1] |= CvtPkE4m3(va * LoLU1(ga) * resMult, vb * LoLU1(gb) * resMult) << ((w & 1) * 16);
-                }
-            }
-            *(uint4 *)At<TE4M3>(res, t, c) = make_uint4(out[0], out[1], out[2], out[3]);
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                *(uint32_t *)(buf + r * PITCH + l8 * 16 + 4 * q) = out[q];
-            }
-        }
-    }
-    __syncthreads();
-    TransposeOut128<PITCH>(buf, resT, xBlock, tBlock, tid);
-}
-
 // MODE 0: FFN (tile-norm backward of vals fused); MODE 1: attention (dScale fused)
 template <class TGrad, class TOutG, class TOutV, int MODE>
 __global__ void __launch_bounds__(256) BackpropLoLU(int len, int lenRound, int tiles, Mat gate, Mat vals, float valsScale, Mat valsSrcTileScale,
@@ -601,6 +523,37 @@ __global__ void __launch_bounds__(256) BackpropLoLU8(int len, int lenRound, int 
         }
         *(uint2 *)At<TE4M3>(gradGate, row[k], col[k]) = make_uint2(og[0], og[1]);
         *(uint2 *)At<TE4M3>(gradVals, row[k], col[k]) = make_uint2(ov[0], ov[1]);
+    }
+}
+
+// A 128 x 128 block of bytes staged in LDS as [t][x] (pitch PITCH) goes out transposed: dst[x][t], 16 bytes (16 t) per store.
+// thread -> (tq = block of 16 t, xq = x quad)
+template <int PITCH> __device__ __forceinline__ void TransposeOut128(const uint8_t *buf, const Mat &dst, int xBlock, int tBlock, int tid)
+{
+    const int tq = tid & 7, xq = tid >> 3;
+    uint32_t out[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint8_t *b = buf + (tq * 16 + j * 4) * PITCH + xq * 4;
+        uint32_t r0 = *(const uint32_t *)(b);
+        uint32_t r1 = *(const uint32_t *)(b + PITCH);
+        uint32_t r2 = *(const uint32_t *)(b + 2 * PITCH);
+        uint32_t r3 = *(const uint32_t *)(b + 3 * PITCH);
+        // 4x4 byte transpose.  __builtin_amdgcn_perm(hi, lo, sel): result byte i = byte sel[i] of {hi:lo} (lo = bytes 0-3)
+        uint32_t a = __builtin_amdgcn_perm(r1, r0, 0x05010400); // r0.b0 r1.b0 r0.b1 r1.b1
+        uint32_t bb = __builtin_amdgcn_perm(r1, r0, 0x07030602); // r0.b2 r1.b2 r0.b3 r1.b3
+        uint32_t c = __builtin_amdgcn_perm(r3, r2, 0x05010400);
+        uint32_t d = __builtin_amdgcn_perm(r3, r2, 0x07030602);
+        out[0][j] = __builtin_amdgcn_perm(c, a, 0x05040100); // column 0: r0.b0 r1.b0 r2.b0 r3.b0
+        out[1][j] = __builtin_amdgcn_perm(c, a, 0x07060302);
+        out[2][j] = __builtin_amdgcn_perm(d, bb, 0x05040100);
+        out[3][j] = __builtin_amdgcn_perm(d, bb, 0x07060302);
+    }
+    int x = xBlock + xq * 4;
+    int tcol = tBlock + tq * 16;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        *(uint4 *)(dst.p + (int64_t)(x + i) * dst.ld + tcol) = make_uint4(out[i][0], out[i][1], out[i][2], out[i][3]);
     }
 }
 
@@ -1833,27 +1786,6 @@ extern "C" int ts2_backprop_row_tile_normalize_lolu_t(int32_t len, int32_t lenRo
     }
     hipLaunchKernelGGL(BackpropLoLU8T, dim3(dim / TILE, lenRound / 128), dim3(256), 0, STREAM, len, lenRound, M(*gate), M(*vals), valsScale,
         M(*valsSrcTileScale), M(*grad), M(*gradGate), M(*gradVals), M(*gradGateT), M(*gradValsT));
-    TS2_CHECK_LAUNCH();
-    return TS2_OK;
-}
-
-extern "C" int ts2_matrix_lolu_t(int32_t len, int32_t lenRound, const ts2_mat *gate, const ts2_mat *vals, float resMult, const ts2_mat *res,
-    const ts2_mat *resT, void *stream)
-{
-    if (!gate || !vals || !res || !resT) {
-        return TS2_ERR_NULL;
-    }
-    int dim = res->x;
-    if (dim % TILE || lenRound % 128 || lenRound < len || !MatOk(gate, len, dim, 2) || !MatOk(vals, len, dim, 2) || !MatOk(res, lenRound, dim, 1) ||
-        !MatOk(resT, dim, lenRound, 1)) {
-        return TS2_ERR_SHAPE;
-    }
-    if (!Aligned16(gate->ptr, gate->strideBytes) || !Aligned16(vals->ptr, vals->strideBytes) || !Aligned16(res->ptr, res->strideBytes) ||
-        !Aligned16(resT->ptr, resT->strideBytes)) {
-        return TS2_ERR_ALIGN;
-    }
-    hipLaunchKernelGGL(MatrixLoLU16T, dim3(dim / 128, lenRound / 128), dim3(256), 0, STREAM, len, lenRound, M(*gate), M(*vals), resMult, M(*res),
-        M(*resT));
     TS2_CHECK_LAUNCH();
     return TS2_OK;
 }

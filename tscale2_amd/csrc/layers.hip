@@ -83,7 +83,6 @@ struct TActs {
     Arr a16[4]; // bf16: wide/q, gate, k, v
     Arr tsc[2]; // fp32 tile scales: wide/q, v
     Arr rg8;    // 8-bit rg / vlg
-    Arr rg8T;   // fp8 FFN: rg transposed, written by the forward (the source of the contract matrix's delta product)
     Arr val16;  // bf16 attention output (its storage is reused for dQ by the backward)
     Arr swl;    // fp32 [heads][R] softmax statistics
     bool valid = false;
@@ -295,14 +294,10 @@ int DeltaSplits(ts2_model *M, int srcDim, int dstDim)
 
 // delta = alpha * gradScale * gradFast^T * src8   (TMatMulBuffers::BackpropDelta)
 int BackpropDelta(ts2_model *M, TMatrix &W, const Arr &src8, const Arr &gradFast, float alpha, const float *gradScale, void *s,
-    bool sameSrcAsLastCall = false, const Arr *gradTReady = nullptr, const Arr *srcTReady = nullptr)
+    bool sameSrcAsLastCall = false, const Arr *gradTReady = nullptr)
 {
     ts2_matmul_bwd_buffers b = Scratch(M, M->R, W.srcDim, W.dstDim);
     b.srcTValid = sameSrcAsLastCall; // the matrices of a layer that share their input transpose it once
-    if (srcTReady) { // the producer of the source left its transpose
-        b.srcT = srcTReady->m;
-        b.srcTValid = 1;
-    }
     if (gradTReady) { // the producer of the gradient left its transpose
         b.gradT = gradTReady->m;
         b.gradTValid = 1;
@@ -329,9 +324,6 @@ int FfnComputeRG(ts2_model *M, TLayer &L, const Arr &norm8, void *s)
     CK(ForwardNormRope(M, L.w[0], norm8, VEC * DISCR * Dot(D), true, true, VEC, nullptr, wide16, &wideScale, s));
     // gate uses the matrix without its scale (GetDataNoScale)
     CK(Forward(M, L.w[1], norm8, VEC * DISCR * Dot(D), false, gate16, false, s));
-    if (A.rg8T.m.ptr) {
-        return ts2_matrix_lolu_t(len, R, gate16.P(), wide16.P(), 1.f, rg8.P(), View(A.rg8T, F, R).P(), s);
-    }
     return ts2_matrix_lolu(len, R, gate16.P(), wide16.P(), 1.f, rg8.P(), M->mode, s);
 }
 
@@ -371,8 +363,7 @@ int FfnBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
         CK(BackpropDXGroup(M, 2, ws, gs, DISCR * Dot(D), us, M->dNormState, false, s));
     }
     // deltas (sources are stored in 1/24 units)
-    Arr rg8T = View(A.rg8T, F, R);
-    CK(BackpropDelta(M, L.w[2], rg8, M->stateGradFast, VEC, gradScale, s, false, nullptr, A.rg8T.m.ptr ? &rg8T : nullptr));
+    CK(BackpropDelta(M, L.w[2], rg8, M->stateGradFast, VEC, gradScale, s));
     CK(BackpropDelta(M, L.w[0], norm8, dwide, VEC, gradScale, s, false, fusedT ? &dwideT : nullptr));
     return BackpropDelta(M, L.w[1], norm8, dgate, VEC, gradScale, s, true, fusedT ? &dgateT : nullptr);
 }
@@ -840,10 +831,6 @@ extern "C" ts2_model *ts2_model_create(const ts2_model_config *cfg)
     // layer scratch
     int RP = M->RP;
     ok &= M->Alloc(&M->raw, RP, maxW, TS2_F32) && M->Alloc(&M->g32, RP, maxW, TS2_F32) && M->Alloc(&M->shared.rg8, RP, maxW, M->mode);
-    const bool keepRgT = M->mode == TS2_E4M3 && (M->R % 128) == 0 && cfg->ffnDim > 0; // fp8: the FFN forward leaves rg transposed as well
-    if (keepRgT) {
-        ok &= M->Alloc(&M->shared.rg8T, cfg->ffnDim, RP, M->mode);
-    }
     for (int k = 0; k < 4; ++k) {
         ok &= M->Alloc(&M->shared.a16[k], RP, maxW, TS2_BF16) && M->Alloc(&M->g16[k], RP, maxW, TS2_BF16) &&
               M->Alloc(&M->gf[k], RP, maxW, M->fastGradType);
@@ -878,7 +865,7 @@ extern "C" ts2_model *ts2_model_create(const ts2_model_config *cfg)
             L.acts = &A;
             if (L.type == LT_FFN) {
                 ok &= M->Alloc(&A.a16[0], R, F, TS2_BF16) && M->Alloc(&A.a16[1], R, F, TS2_BF16) && M->Alloc(&A.tsc[0], F / 128, R, TS2_F32) &&
-                      M->Alloc(&A.rg8, R, F, M->mode) && (!keepRgT || M->Alloc(&A.rg8T, F, R, M->mode));
+                      M->Alloc(&A.rg8, R, F, M->mode);
             } else {
                 int Q = H * 128;
                 for (int k = 0; k < 4; ++k) {
