@@ -249,6 +249,9 @@ typedef struct ts2_matmul_bwd_buffers {
     /* != 0 (E4M3): gradT already holds the transpose of the `grad` given to BackpropDelta (its producer wrote it, e.g.
      * ts2_backprop_row_tile_normalize_lolu_t); the transpose is skipped. */
     int32_t gradTValid;
+    /* != 0: transformT already holds the transpose of the `transformFast` given to BackpropMulti (the matrix has not changed since an
+     * earlier call left it there: weights change once per optimiser step, not per micro-batch); the transpose is skipped. */
+    int32_t transformTValid;
 } ts2_matmul_bwd_buffers;
 
 /* BackpropMulti (prep of dX): I8: quantise grad (TS2_BF16 | TS2_F32, optionally times gradColScale[gradDim]) per row to

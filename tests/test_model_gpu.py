@@ -74,6 +74,47 @@ def test_kept_activations_give_the_same_deltas_as_recomputation(mode):
         assert np.array_equal(a, b)
 
 
+@pytest.mark.parametrize("mode", [I8, E4M3])
+def test_new_weights_replace_the_kept_transposes(mode):
+    """The driver keeps the transposed copy of every matrix from one backward to the next (weights change once per optimiser step).
+    Setting a matrix must drop that copy: a model that has stepped with old weights and is then given new ones must produce exactly
+    what a fresh model with the new weights produces."""
+    print("case weights replaced between steps", mode, flush=True)
+    from tscale2_amd import lib as L
+    old = Harness(mode, dim=256, heads=2, ffn_tiles=4, depth=2, vocab=256, frag_count=4, frag_len=64, wide_window=64, seed=9)
+    new = Harness(mode, dim=256, heads=2, ffn_tiles=4, depth=2, vocab=256, frag_count=4, frag_len=64, wide_window=64, seed=9)
+    for mats in new.layers:  # same batch, other weights: every matrix with its rows in reverse order
+        for q in mats:
+            q.fast = np.ascontiguousarray(q.fast[::-1])
+    assert any(not np.array_equal(a.fast, b.fast) for la, lb in zip(old.layers, new.layers) for a, b in zip(la, lb))
+
+    def results(m):
+        torch.cuda.synchronize()
+        return [m.get_delta(d, i, *q.fast.shape) for d in range(new.depth) for i, q in enumerate(new.layers[d])] + \
+               [m.array("stateGrad").float().cpu().numpy()]
+
+    m = old.device_model()
+    try:
+        m.backprop()
+        for d in range(new.depth):
+            for i, q in enumerate(new.layers[d]):
+                m.set_matrix(d, i, q.fast, q.scale)
+        m.set_matrix(L.LAYER_EMBED, 0, new.embed.fast, new.embed.scale)
+        m.set_matrix(L.LAYER_FINAL, 0, new.final.fast, new.final.scale)
+        m.backprop()
+        got = results(m)
+    finally:
+        m.close()
+    m = new.device_model()
+    try:
+        m.backprop()
+        want = results(m)
+    finally:
+        m.close()
+    for a, b in zip(got, want):
+        assert np.array_equal(a, b)
+
+
 def test_tiny_dense_int8_step():
     """BASELINE config[0]: e256 h2 d4 ffn8 w64 (8 layers), byte vocab, 8 fragments of 64 tokens, weights N(0, 0.02)"""
     print("case tiny dense int8", flush=True)

@@ -58,6 +58,8 @@ struct Arr {
 
 struct TMatrix {
     Arr fast;           // [dst][src] 8-bit ([slabs*dst][src] for expert matrices)
+    Arr fastT;          // [src][dst]: the transpose the dX products contract over, kept until the matrix is set again (not for slabs)
+    bool fastTValid = false;
     float *scale = 0;   // device: matrix scale (rms of the fp32 master weights)
     Arr delta;          // i8 packed delta, same shape
     Arr deltaTileScale; // fp32 [src/128][rows]
@@ -225,7 +227,12 @@ int ForwardNormRope(ts2_model *M, TMatrix &W, const Arr &src8, float alpha, bool
 int BackpropDX(ts2_model *M, TMatrix &W, const Arr &gradFast, float alpha, bool useScale, const Arr &srcGrad, bool add, void *s)
 {
     ts2_matmul_bwd_buffers b = Scratch(M, M->R, W.srcDim, W.dstDim);
+    if (W.fastT.m.ptr) {
+        b.transformT = W.fastT.m;
+        b.transformTValid = W.fastTValid;
+    }
     CK(ts2_matmul_backprop_multi(M->mode, M->len, M->R, W.srcDim, W.dstDim, W.fast.P(), gradFast.P(), gradFast.type, nullptr, &b, s));
+    W.fastTValid = W.fastT.m.ptr != nullptr;
     return ts2_matmul_backprop(M->mode, M->len, M->R, W.srcDim, W.dstDim, gradFast.P(), &b, alpha, useScale ? W.scale : nullptr, srcGrad.P(),
         srcGrad.type, add, s);
 }
@@ -257,7 +264,12 @@ int BackpropDXGroup(ts2_model *M, int count, TMatrix *const *W, const Arr *const
         }
         b[i] = Scratch(M, M->R, srcDim, dstDim);
         b[i].transformT = Flat(M->sWT + (size_t)i * srcDim * dstDim, srcDim, dstDim, M->mode).m;
+        if (W[i]->fastT.m.ptr) {
+            b[i].transformT = W[i]->fastT.m;
+            b[i].transformTValid = W[i]->fastTValid;
+        }
         CK(ts2_matmul_backprop_multi(M->mode, M->len, M->R, srcDim, dstDim, W[i]->fast.P(), grad[i]->P(), grad[i]->type, nullptr, &b[i], s));
+        W[i]->fastTValid = W[i]->fastT.m.ptr != nullptr;
         bp[i] = &b[i];
         gp[i] = grad[i]->P();
         al[i] = alpha;
@@ -595,13 +607,16 @@ int MoeBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
 // step driver
 namespace
 {
-int InitMatrix(ts2_model *M, TMatrix *W, int srcDim, int dstDim, int slabs)
+int InitMatrix(ts2_model *M, TMatrix *W, int srcDim, int dstDim, int slabs, bool keepT = true)
 {
     W->srcDim = srcDim;
     W->dstDim = dstDim;
     W->slabs = slabs;
     if (!M->Alloc(&W->fast, dstDim * slabs, srcDim, M->mode) || !M->Alloc(&W->delta, dstDim * slabs, srcDim, TS2_I8) ||
         !M->Alloc(&W->deltaTileScale, srcDim / 128, dstDim * slabs, TS2_F32)) {
+        return TS2_ERR_LAUNCH;
+    }
+    if (slabs == 1 && keepT && !M->Alloc(&W->fastT, srcDim, dstDim, M->mode)) {
         return TS2_ERR_LAUNCH;
     }
     W->scale = (float *)M->Dev(4);
@@ -774,11 +789,11 @@ extern "C" ts2_model *ts2_model_create(const ts2_model_config *cfg)
     }
     M->maxW = maxW;
     bool ok = true;
-    ok &= InitMatrix(M, &M->embed, D, cfg->labelCount, 1) == 0; // delta storage reused as fp32 [labelCount][D]: allocate separately below
+    ok &= InitMatrix(M, &M->embed, D, cfg->labelCount, 1, false) == 0; // delta storage reused as fp32 [labelCount][D]: allocate separately below
     ok &= M->Alloc(&M->embed.delta, cfg->labelCount, D, TS2_F32);
     M->VP = (V >= 4096 && V % 256) ? RoundUp(V, 256) : V;
     const int VP = M->VP;
-    ok &= InitMatrix(M, &M->finalW, D, VP, 1) == 0;
+    ok &= InitMatrix(M, &M->finalW, D, VP, 1, false) == 0;
     M->bias = (float *)M->Dev((size_t)V * 4);
     M->layers.resize(cfg->depth);
     for (int d = 0; d < cfg->depth && ok; ++d) {
@@ -948,6 +963,7 @@ extern "C" int ts2_model_set_matrix(ts2_model *M, int32_t layer, int32_t matrixI
         hipMemcpy(W->scale, &scale, 4, hipMemcpyHostToDevice) != hipSuccess) {
         return TS2_ERR_LAUNCH;
     }
+    W->fastTValid = false; // the kept transpose belongs to the old weights
     return 0;
 }
 

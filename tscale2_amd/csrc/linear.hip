@@ -33,6 +33,9 @@ extern "C" int ts2_matmul_backprop_multi(int32_t mode, int32_t len, int32_t lenR
         }
     }
     // W [gradDim][srcDim] -> W^T [srcDim][gradDim] so that the dX GEMM contracts over contiguous bytes
+    if (buf->transformTValid) {
+        return TS2_OK;
+    }
     return ts2_transpose_quant(gradDim, gradDim, transformFast, mode, nullptr, nullptr, 0, nullptr, &buf->transformT, mode, nullptr, stream);
 }
 

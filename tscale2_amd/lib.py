@@ -159,7 +159,7 @@ def probe_copy_rate(nbytes=1 << 30):
 class BwdBuffers(C.Structure):
     _fields_ = [("grad8", Mat), ("grad8RowScale", C.c_void_p), ("gradT", Mat), ("srcT", Mat), ("tileMax", C.c_void_p), ("tileScale", C.c_void_p),
                 ("transformT", Mat), ("partial", Mat), ("splits", C.c_int32), ("gradRowAbsMax", C.c_void_p),
-                ("gradRowAbsMaxValid", C.c_int32), ("srcTValid", C.c_int32), ("gradTValid", C.c_int32)]
+                ("gradRowAbsMaxValid", C.c_int32), ("srcTValid", C.c_int32), ("gradTValid", C.c_int32), ("transformTValid", C.c_int32)]
 
 
 class MatMulBuffers:
