@@ -115,8 +115,10 @@ typedef struct ts2_gemm_args {
      * m, n, k, operand type and operand strides; a, b, alpha, alphaPtr above describe product 0, segment[i-1] product i.  One launch
      * and one pass over C instead of one read-modify-write of C per product: the gradient of a layer input that feeds several
      * matrices (Backprop of Q, K, V and gate in src/gpt/compute/layer_att.cu:236-260 adds four products into the same array).
-     * 256x256-tile kernel only (m, n multiples of 256), TS2_E4M3 or TS2_BF16 operands, fp32 or bf16 C, TS2_EPI_STORE or TS2_EPI_ADD,
-     * no rowScale, kTileScale, groups or splitK; the fp32 sums of the products are rescaled in registers between products. */
+     * 256x256-tile kernel (m, n multiples of 256), or one further product on the 128x128 tile (tileConfig 2, or with tileGroup: the
+     * expert-grouped dX of wide and gate, src/gpt/compute/layer_moe.cu:236-250, where every B_i takes the tile's slab); TS2_E4M3 or
+     * TS2_BF16 operands, fp32 or bf16 C, TS2_EPI_STORE or TS2_EPI_ADD, no rowScale, kTileScale, groupOffsets or splitK; the fp32 sums
+     * of the products are rescaled in registers between products. */
     int32_t extraSegments;
     struct {
         const void *a;

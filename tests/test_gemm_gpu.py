@@ -280,10 +280,46 @@ def test_several_products_into_one_result(ab, add):
     assert (got[:500] - want[:500]).abs().max().item() <= 4e-6 * scale
     if not add:
         assert (got[500:] == 0).all()
-    # not available off the 256x256 tile or for int8 operands
+    # not available for int8 operands; the 128x128 tile takes one further product, not two
     a8 = torch.zeros((m, k), dtype=torch.int8, device="cuda"); b8 = torch.zeros((n, k), dtype=torch.int8, device="cuda")
     assert lib.gemm_nt(a8, b8, got, L.I8, L.F32, segments=[(a8, b8, 1.0, None)], check=False) == -3
-    assert lib.gemm_nt(As[0], Bs[0], got, t, L.F32, tile_config=2, segments=[(As[1], Bs[1], 1.0, None)], check=False) == -3
+    assert lib.gemm_nt(As[0], Bs[0], got, t, L.F32, tile_config=2, segments=[(As[1], Bs[1], 1.0, None), (As[2], Bs[2], 1.0, None)],
+                       check=False) == -3
+
+
+@pytest.mark.parametrize("grouped", [False, True])
+@pytest.mark.parametrize("c_type", ["f32", "bf16"])
+def test_two_products_into_one_result_on_the_small_tile(grouped, c_type):
+    """One further product on the 128x128 tile, plain and with a weight slab per 128-row tile (the expert-grouped dX of two matrices
+    that share their rows): against the two products launched one after the other (store, then accumulate).  Same MFMA sums; the
+    one-launch form rescales the first in registers and rounds the total once."""
+    print("case two products small tile", grouped, c_type, flush=True)
+    from tscale2_amd import lib as L
+    lib = L.load()
+    m, n, k, slabs = 640, 384, 256, 3
+    g = torch.Generator(device="cuda").manual_seed(12)
+    mk = lambda r, c: (torch.randn((r, c), device="cuda", generator=g) * 6).to(torch.float8_e4m3fn).view(torch.uint8)
+    a0, a1 = mk(m, k), mk(m, k)
+    b0, b1 = mk(n * (slabs if grouped else 1), k), mk(n * (slabs if grouped else 1), k)
+    p0 = torch.full((1,), 0.7, device="cuda")
+    kw = dict(n=n)
+    if grouped:
+        kw.update(tile_group=torch.tensor([2, 0, -1, 1, 2], dtype=torch.int32, device="cuda"), b_slab_bytes=n * k)
+    else:
+        kw.update(tile_config=2)
+    ct, dt = (L.F32, torch.float32) if c_type == "f32" else (L.BF16, torch.bfloat16)
+    view = (lambda x: x) if c_type == "f32" else (lambda x: x.view(torch.int16))
+    want = torch.full((m, n), 3.0, dtype=torch.float32, device="cuda")
+    lib.gemm_nt(a0, b0, want, L.E4M3, L.F32, alpha=0.25, alpha_ptr=p0, **kw)
+    lib.gemm_nt(a1, b1, want, L.E4M3, L.F32, alpha=0.5, epilogue=L.EPI_ADD, **kw)
+    got = torch.full((m, n), 3.0, dtype=dt, device="cuda")
+    lib.gemm_nt(a0, b0, view(got), L.E4M3, ct, alpha=0.25, alpha_ptr=p0, segments=[(a1, b1, 0.5, None)], **kw)
+    torch.cuda.synchronize()
+    scale = want.abs().max().item()
+    tol = 4e-6 * scale if c_type == "f32" else 2.0 ** -8 * scale
+    assert (got.float() - want).abs().max().item() <= tol
+    if grouped:
+        assert (got[256:384].float() == 3.0).all()   # the skipped tile is left alone
 
 
 @pytest.mark.parametrize("ab,tile", [("e4m3", 1), ("i8", 1), ("e4m3", 2)])

@@ -709,7 +709,9 @@ __global__ void ZeroRows(uint8_t *c, int64_t ldc, int rowBytes)
 #define TS2_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 #define TS2_GLB_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
 
-template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT, int WM = 2, int WN = 2>
+// SEG: two products into the same accumulators (C = alpha0 A0 B0^T + alpha1 A1 B1^T with the same k), the second operand pair and its
+// factors in segA[0], segB[0], segAlpha[0], segAlphaPtr[0]; with tileGroup both B operands take the tile's slab.
+template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT, int WM = 2, int WN = 2, bool SEG = false>
 __global__ void __launch_bounds__(64 * WM * WN, (WM * WN) / 4) GemmNTDirect(GemmP p)
 {
     typedef typename AccT<TYPE>::type TAcc;
@@ -741,6 +743,9 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN) / 4) GemmNTDirect(Gemm
             return;
         }
         p.b += (int64_t)g * p.bSlab;
+        if (SEG) {
+            p.segB[0] += (int64_t)g * p.bSlab;
+        }
     }
     if (p.groupOffsets) {
         int g = blockIdx.y;
@@ -766,8 +771,9 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN) / 4) GemmNTDirect(Gemm
     const int lrow = wave * 8 + (lane >> 3);
     const int lchunk = (lane & 7) ^ ((lrow >> 1) & 7);
     // address = wave-uniform base (scalar registers) + one 32-bit per-lane offset per operand
-    const uint8_t *gaTile = p.a + (int64_t)rowBase * p.lda + (int64_t)kBeg * BKB;
-    const uint8_t *gbTile = p.b + (int64_t)colBase * p.ldb + (int64_t)kBeg * BKB;
+    const int64_t aTileOff = (int64_t)rowBase * p.lda + (int64_t)kBeg * BKB, bTileOff = (int64_t)colBase * p.ldb + (int64_t)kBeg * BKB;
+    const uint8_t *gaTile = p.a + aTileOff;
+    const uint8_t *gbTile = p.b + bTileOff;
     const uint32_t gaLane = (uint32_t)(lrow * (int)p.lda + lchunk * 16);
     const uint32_t gbLane = (uint32_t)(lrow * (int)p.ldb + lchunk * 16);
     constexpr int LA = BM / (8 * NW);
@@ -882,6 +888,11 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN) / 4) GemmNTDirect(Gemm
         }                                                                                                                                  \
     } while (0)
 
+    for (int seg = 0; seg < (SEG ? 2 : 1); ++seg) {
+    if (SEG && seg == 1) {
+        gaTile = p.segA[0] + aTileOff;
+        gbTile = p.segB[0] + bTileOff;
+    }
     if (kSteps > 0) {
         DIRECT_LOAD(sA0, sB0, 0);
     }
@@ -898,6 +909,35 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN) / 4) GemmNTDirect(Gemm
     }
     if (s < kSteps) {
         STEP(sA0, sB0, sA1, sB1, s);
+    }
+    if constexpr (SEG && TYPE != T_I8) {
+        if (seg == 0) {
+            // the epilogue applies the second product's factor to the sum: bring the first product to that scale
+            float cur = p.alpha, nxt = p.segAlpha[0];
+            if (p.alphaPtr) {
+                cur *= *p.alphaPtr;
+            }
+            if (p.segAlphaPtr[0]) {
+                nxt *= *p.segAlphaPtr[0];
+            }
+            const float ratio = cur / nxt;
+#pragma unroll
+            for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+                for (int j = 0; j < WTN; ++j) {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        acc[i][j][e] *= ratio;
+                    }
+                }
+            }
+            __syncthreads(); // every wave has read its last operands of this product before the stages are refilled
+        }
+    }
+    } // products
+    if (SEG) {
+        p.alpha = p.segAlpha[0];
+        p.alphaPtr = p.segAlphaPtr[0];
     }
 #undef STEP
 #undef LOAD_FRAGS
@@ -1409,7 +1449,15 @@ template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT> int Launch(const
             }
         }
         if (p.nSeg > 1) {
-            return TS2_ERR_UNSUPPORTED; // several products per launch: ring kernel only
+            // several products per launch: the ring kernel, or two products on the 128x128 tile (fp32 / bf16 results)
+            if constexpr (WTM == 2 && WTN == 2 && !KT && TYPE != T_I8 && (CT == C_F32 || CT == C_BF16)) {
+                if (p.nSeg == 2 && !p.groupOffsets && p.splits <= 1) {
+                    hipLaunchKernelGGL((GemmNTDirect<TYPE, WTM, WTN, CT, EPI, KT, 2, 2, true>), dim3(nb, gy), dim3(256), 0, stream, q);
+                    TS2_CHECK_LAUNCH();
+                    return TS2_OK;
+                }
+            }
+            return TS2_ERR_UNSUPPORTED;
         }
         hipLaunchKernelGGL((GemmNTDirect<TYPE, WTM, WTN, CT, EPI, KT>), dim3(nb, gy), dim3(256), 0, stream, q);
         TS2_CHECK_LAUNCH();
@@ -1624,8 +1672,11 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
     }
     p.nSeg = 1;
     if (a->extraSegments) {
-        const bool bigTile = (a->m % 256) == 0 && (a->n % 256) == 0 && (a->tileConfig & 3) <= 1 && !(a->tileConfig & (4 | 8 | 16));
-        if (a->extraSegments < 0 || a->extraSegments > 3 || !bigTile || a->abType == TS2_I8 || a->rowScale || a->kTileScale || a->tileGroup ||
+        const bool bigTile = (a->m % 256) == 0 && (a->n % 256) == 0 && (a->tileConfig & 3) <= 1 && !(a->tileConfig & (4 | 8 | 16)) && !a->tileGroup;
+        // the 128x128 tile (chosen with tileConfig 2, or implied by tileGroup) takes one further product
+        const bool smallTile = a->extraSegments == 1 && ((a->tileConfig & 3) == 2 || a->tileGroup) && !(a->tileConfig & (4 | 8 | 16)) &&
+            !a->splitSlabBytes;
+        if (a->extraSegments < 0 || a->extraSegments > 3 || !(bigTile || smallTile) || a->abType == TS2_I8 || a->rowScale || a->kTileScale ||
             a->groupOffsets || splitK > 1 || (a->cType != TS2_F32 && a->cType != TS2_BF16) ||
             (a->epilogue != TS2_EPI_STORE && a->epilogue != TS2_EPI_ADD)) {
             return TS2_ERR_UNSUPPORTED;

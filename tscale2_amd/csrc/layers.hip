@@ -485,7 +485,7 @@ int AttBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
 // ---------------------------------------------------------------------------------------------------------------------------
 // MoE: src/gpt/compute/layer_moe.cu:117-272 with the CPU path's factors (layer_moe.cu:458-537).  fp8 operands only.
 int GroupedGemm(ts2_model *M, const Arr &a, const Arr &bSlabs, int slabRows, int n, int k, const Arr &c, float alpha, const float *alphaPtr, bool add,
-    void *s)
+    void *s, const Arr *a2 = nullptr, const Arr *bSlabs2 = nullptr, const float *alphaPtr2 = nullptr)
 {
     ts2_gemm_args g = {};
     g.a = a.m;
@@ -503,6 +503,16 @@ int GroupedGemm(ts2_model *M, const Arr &a, const Arr &bSlabs, int slabRows, int
     g.splitK = 1;
     g.tileGroup = M->moe.xpTileExpertId;
     g.bSlabBytes = (int64_t)slabRows * bSlabs.m.strideBytes;
+    if (a2) { // a second product with the same shapes and strides into the same result (its factor: alpha * *alphaPtr2)
+        if (a2->m.strideBytes != a.m.strideBytes || bSlabs2->m.strideBytes != bSlabs.m.strideBytes) {
+            return TS2_ERR_SHAPE;
+        }
+        g.extraSegments = 1;
+        g.segment[0].a = a2->m.ptr;
+        g.segment[0].b = bSlabs2->m.ptr;
+        g.segment[0].alpha = alpha;
+        g.segment[0].alphaPtr = alphaPtr2;
+    }
     return ts2_gemm_nt(&g, s);
 }
 
@@ -587,10 +597,12 @@ int MoeBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
     Arr sgFull = View(M->raw, RM, D);
     CK(ts2_transpose_u8_batched(E, X, D, L.w[0].fast.m.ptr, L.w[0].fast.m.strideBytes, (int64_t)X * L.w[0].fast.m.strideBytes, weT.m.ptr,
         weT.m.strideBytes, (int64_t)D * weT.m.strideBytes, s));
-    CK(GroupedGemm(M, dwide, weT, D, D, X, sgFull, DISCR * Dot(D), L.w[0].scale, false, s));
-    CK(ts2_transpose_u8_batched(E, X, D, L.w[1].fast.m.ptr, L.w[1].fast.m.strideBytes, (int64_t)X * L.w[1].fast.m.strideBytes, weT.m.ptr,
-        weT.m.strideBytes, (int64_t)D * weT.m.strideBytes, s));
-    CK(GroupedGemm(M, dgate, weT, D, D, X, sgFull, DISCR * Dot(D), nullptr, true, s));
+    // the gate matrix transposed next to the expand matrix; both products in one launch (one pass over the result)
+    Arr wgT = Flat((uint8_t *)M->wT.m.ptr + (size_t)E * D * weT.m.strideBytes, E * D, X, M->mode);
+    wgT.m.strideBytes = weT.m.strideBytes;
+    CK(ts2_transpose_u8_batched(E, X, D, L.w[1].fast.m.ptr, L.w[1].fast.m.strideBytes, (int64_t)X * L.w[1].fast.m.strideBytes, wgT.m.ptr,
+        wgT.m.strideBytes, (int64_t)D * wgT.m.strideBytes, s));
+    CK(GroupedGemm(M, dwide, weT, D, D, X, sgFull, DISCR * Dot(D), L.w[0].scale, false, s, &dgate, &wgT, nullptr));
     CK(ts2_combine_experts(len, K, sgFull.P(), TS2_F32, &M->moe, 1.f, nullptr, M->dNormState.P(), 0, s));
     // select matrix: dNormState += dMoe * Wsel / sqrt(D) and its delta through the same 8-bit operator as every other matrix (the
     // reference uses its fp16 kernels here, MatmulSelect.BackpropFp16, layer_moe.cu:264); rows >= experts of the matrix are zero
@@ -919,7 +931,7 @@ extern "C" ts2_model *ts2_model_create(const ts2_model_config *cfg)
         M->dExpertWeight = (float *)M->Dev((size_t)M->lenMoe * 4);
         ok &= M->Alloc(&M->normMoe, M->lenMoe, D, M->mode) && M->Alloc(&M->sgMoe, M->lenMoe, D, M->fastGradType) &&
               M->Alloc(&M->moeSel, R, SelectDim, TS2_F32) && M->Alloc(&M->dMoeSel, R, SelectDim, M->fastGradType);
-        int wtRows = E * (X > D ? X : D), wtCols = X > D ? X : D;
+        int wtRows = 2 * E * (X > D ? X : D), wtCols = X > D ? X : D; // two transposed expert matrices side by side (expand and gate)
         ok &= M->Alloc(&M->wT, wtRows, wtCols, M->mode);
     }
     ok &= M->Alloc(&M->logits, R, VP, TS2_F32) && M->Alloc(&M->logits16, R, VP, TS2_F16) && M->Alloc(&M->gradV, R, VP, TS2_BF16) && M->Alloc(&M->gradVT, VP, R, TS2_BF16) &&
