@@ -517,12 +517,15 @@ int GroupedGemm(ts2_model *M, const Arr &a, const Arr &bSlabs, int slabRows, int
 }
 
 // per-expert delta: delta_e[gradDim][srcDim] = alpha * gradScale * sum over the expert's rows of grad^T src
-int GroupedDelta(ts2_model *M, TMatrix &W, const Arr &src8, const Arr &gradFast, float alpha, const float *gradScale, void *s)
+int GroupedDelta(ts2_model *M, TMatrix &W, const Arr &src8, const Arr &gradFast, float alpha, const float *gradScale, void *s,
+    bool sameSrcAsLastCall = false)
 {
     int E = M->cfg.expertCount, rows = M->lenMoe;
     Arr gradT = Flat(M->sGradT, W.dstDim, rows, M->mode), srcT = Flat(M->sSrcT, W.srcDim, rows, M->mode);
     CK(ts2_transpose_quant(rows, rows, gradFast.P(), M->mode, nullptr, nullptr, 0, nullptr, gradT.P(), M->mode, nullptr, s));
-    CK(ts2_transpose_quant(rows, rows, src8.P(), M->mode, nullptr, nullptr, 0, nullptr, srcT.P(), M->mode, nullptr, s));
+    if (!sameSrcAsLastCall) { // (the expand and gate matrices share their source: one transpose)
+        CK(ts2_transpose_quant(rows, rows, src8.P(), M->mode, nullptr, nullptr, 0, nullptr, srcT.P(), M->mode, nullptr, s));
+    }
     ts2_gemm_args g = {};
     g.a = gradT.m;
     g.b = srcT.m;
@@ -611,7 +614,7 @@ int MoeBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
     // expert deltas
     CK(GroupedDelta(M, L.w[2], rg8, M->sgMoe, VEC, gradScale, s));
     CK(GroupedDelta(M, L.w[0], M->normMoe, dwide, VEC, gradScale, s));
-    return GroupedDelta(M, L.w[1], M->normMoe, dgate, VEC, gradScale, s);
+    return GroupedDelta(M, L.w[1], M->normMoe, dgate, VEC, gradScale, s, true);
 }
 } // namespace
 
