@@ -124,6 +124,7 @@ struct ts2_model {
     std::vector<TActs> acts;                 // per layer; entries of kept layers own storage, the others alias `shared`
     bool keep = false;      // FFN and attention layers own activation sets
     bool useKept = false;   // inside ModelBackprop: the backward of a layer starts from what its forward left
+    int sharedOwner = -1;   // the MoE layer whose forward filled the shared set, its gathered input and the routing tables last
     Arr g32;                                 // fp32 [R'][maxW] gradient scratch (drg / dvlg)
     Arr gf[4];                               // fast-gradient type [R'][maxW]: dwide/dq, dgate, dk, dv
     Arr g16[4];                              // bf16 [R'][maxW]: -, dVal, dK, dV
@@ -575,10 +576,12 @@ int MoeForward(ts2_model *M, TLayer &L, const Arr &norm8, void *s)
     return ts2_combine_experts(M->len, M->cfg.moeSelected, contract.P(), TS2_F32, &M->moe, 1.f, nullptr, M->state.P(), 1, s);
 }
 
-int MoeBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScale, void *s)
+int MoeBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScale, bool kept, void *s)
 {
     int D = M->cfg.dim, X = M->cfg.expertDim, E = M->cfg.expertCount, K = M->cfg.moeSelected, len = M->len, R = M->R, RM = M->lenMoe;
-    CK(MoeComputeRG(M, L, norm8, s));
+    if (!kept) {
+        CK(MoeComputeRG(M, L, norm8, s));
+    }
     TActs &A = M->shared;
     Arr wide16 = View(A.a16[0], RM, X), gate16 = View(A.a16[1], RM, X), wideScale = View(A.tsc[0], X / 128, RM), rg8 = View(A.rg8, RM, X);
     // state gradient into expert order
@@ -652,7 +655,12 @@ int LayerForward(ts2_model *M, int d, void *s)
     } else if (L.type == LT_ATT) {
         CK(AttForward(M, L, n8, s));
     } else if (L.type == LT_MOE) {
-        return MoeForward(M, L, n8, s);
+        // MoE layers work in the shared set; in keep mode nothing else touches it (nor the routing tables and the gathered input), so
+        // what the last MoE layer's forward left is still there when its backward runs
+        CK(MoeForward(M, L, n8, s));
+        M->shared.valid = M->keep;
+        M->sharedOwner = d;
+        return 0;
     } else {
         return TS2_ERR_UNSUPPORTED;
     }
@@ -669,7 +677,9 @@ int LayerBackward(ts2_model *M, int d, const float *gradScale, void *s)
     } else if (L.type == LT_ATT) {
         return AttBackward(M, L, n8, gradScale, s);
     } else if (L.type == LT_MOE) {
-        return MoeBackward(M, L, n8, gradScale, s);
+        const bool kept = M->useKept && M->shared.valid && M->sharedOwner == d;
+        M->shared.valid = false;
+        return MoeBackward(M, L, n8, gradScale, kept, s);
     }
     return TS2_ERR_UNSUPPORTED;
 }
