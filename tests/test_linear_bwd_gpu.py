@@ -257,3 +257,46 @@ def test_grouped_backprop_equals_the_products_added_one_after_the_other(L, orc, 
         else:
             scale = want[:len_].abs().max().item()
             assert (got[:len_] - want[:len_]).abs().max().item() <= 4e-6 * scale
+
+
+def test_transposes_left_by_the_caller_are_used_as_they_are(L, orc):
+    """transformTValid: BackpropMulti does not transpose the matrix again, so the product uses whatever transformT holds (here the
+    transpose of the first matrix although another one is passed); gradTValid: BackpropDelta contracts over the gradT it is given (here
+    the transposed gradient placed there by the caller, while the gradient argument holds other values).  With the flags cleared the
+    arguments count again."""
+    print("case caller-provided transposes", flush=True)
+    len_, src_dim, grad_dim = 512, 256, 384
+    g = torch.Generator(device="cuda").manual_seed(5)
+    f8 = lambda r, c, s: (torch.randn((r, c), device="cuda", generator=g) * s).to(torch.float8_e4m3fn).view(torch.uint8)
+    w1, w2 = f8(grad_dim, src_dim, 8), f8(grad_dim, src_dim, 8)
+    grad, other = f8(len_, grad_dim, 16), f8(len_, grad_dim, 16)
+    x = f8(len_, src_dim, 8)
+    b = L.MatMulBuffers(L.E4M3, len_, src_dim, grad_dim)
+
+    def dx(w):
+        out = torch.zeros((len_, src_dim), device="cuda")
+        b.backprop_multi(len_, w, grad, L.E4M3)
+        b.backprop(len_, grad, 0.01, None, out, L.F32)
+        torch.cuda.synchronize()
+        return out
+    first, second = dx(w1), dx(w2)
+    assert not torch.equal(first, second)
+    b.c.transformTValid = 1                       # transformT holds w2^T
+    assert torch.equal(dx(w1), second)
+    b.c.transformTValid = 0
+    assert torch.equal(dx(w1), first)
+
+    def delta(gr):
+        b.backprop_delta(len_, x, None, gr, L.E4M3, alpha=0.5)
+        torch.cuda.synchronize()
+        return b.delta.clone(), b.delta_tile_scale.clone()
+    d1, s1 = delta(grad)
+    d2, s2 = delta(other)
+    assert not torch.equal(d1, d2)
+    b.t["gradT"].copy_(grad.T)                    # the producer's transposed copy
+    b.c.gradTValid = 1
+    d3, s3 = delta(other)
+    assert torch.equal(d3, d1) and torch.equal(s3, s1)
+    b.c.gradTValid = 0
+    d4, s4 = delta(other)
+    assert torch.equal(d4, d2) and torch.equal(s4, s2)
