@@ -73,6 +73,10 @@ struct TLayer {
     int attId = 0;
     TMatrix w[5];
     TActs *acts = nullptr;
+    // fp8 attention layers: the packed deltas of Q, K, V and gate are row blocks of one [4Q][dim] array (and column blocks of one
+    // tile-scale array), so that one delta product over the four stacked transposed gradients fills them all
+    TMatrix qkvg;
+    bool fusedDelta = false;
 };
 
 enum { LT_ATT = 0, LT_FFN = 2, LT_MOE = 3 };
@@ -477,6 +481,19 @@ int AttBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
         const bool us[4] = {true, true, true, false};
         CK(BackpropDXGroup(M, 4, ws, gs, a, us, M->dNormState, false, s));
     }
+    if (L.fusedDelta) {
+        // the four transposed gradients stacked as row blocks of one [4Q][R] array, then one delta product [4Q x D]: 256 large tiles
+        // instead of four products of 64 that each need token-axis slices and a pack pass
+        Arr gT = Flat(M->sGradT, 4 * Q, R, M->mode);
+        const Arr *const gs4[4] = {&dQf, &dKf, &dVf, &dGate};
+        for (int k = 0; k < 4; ++k) {
+            Arr blk = gT;
+            blk.m.ptr = (uint8_t *)gT.m.ptr + (size_t)k * Q * gT.m.strideBytes;
+            blk.m.y = Q;
+            CK(ts2_transpose_quant(len, R, gs4[k]->P(), M->mode, nullptr, nullptr, 0, nullptr, blk.P(), M->mode, nullptr, s));
+        }
+        return BackpropDelta(M, L.qkvg, norm8, dQf, VEC, gradScale, s, false, &gT);
+    }
     CK(BackpropDelta(M, L.w[0], norm8, dQf, VEC, gradScale, s));
     CK(BackpropDelta(M, L.w[1], norm8, dKf, VEC, gradScale, s, true));
     CK(BackpropDelta(M, L.w[2], norm8, dVf, VEC, gradScale, s, true));
@@ -831,6 +848,21 @@ extern "C" ts2_model *ts2_model_create(const ts2_model_config *cfg)
                 ok &= InitMatrix(M, &L.w[k], D, H * 128, 1) == 0;
             }
             ok &= InitMatrix(M, &L.w[4], H * 128, D, 1) == 0;
+            const int Q = H * 128;
+            if (ok && M->mode == TS2_E4M3 && 4 * Q <= maxW && (Q % 256) == 0 && (D % 256) == 0) {
+                L.qkvg.srcDim = D;
+                L.qkvg.dstDim = 4 * Q;
+                ok &= M->Alloc(&L.qkvg.delta, 4 * Q, D, TS2_I8) && M->Alloc(&L.qkvg.deltaTileScale, D / 128, 4 * Q, TS2_F32);
+                for (int k = 0; k < 4 && ok; ++k) {
+                    L.w[k].delta = L.qkvg.delta;
+                    L.w[k].delta.m.ptr = (uint8_t *)L.qkvg.delta.m.ptr + (size_t)k * Q * L.qkvg.delta.m.strideBytes;
+                    L.w[k].delta.m.y = Q;
+                    L.w[k].deltaTileScale = L.qkvg.deltaTileScale;
+                    L.w[k].deltaTileScale.m.ptr = (uint8_t *)L.qkvg.deltaTileScale.m.ptr + (size_t)k * Q * 4;
+                    L.w[k].deltaTileScale.m.x = Q;
+                }
+                L.fusedDelta = ok;
+            }
         } else if (L.type == LT_FFN) {
             ok &= InitMatrix(M, &L.w[0], D, F, 1) == 0;
             ok &= InitMatrix(M, &L.w[1], D, F, 1) == 0;
