@@ -256,6 +256,12 @@ typedef struct ts2_matmul_bwd_buffers {
     int32_t transformTValid;
 } ts2_matmul_bwd_buffers;
 
+/* Bytes of every scratch member of ts2_matmul_bwd_buffers for one matrix, the sizes TInt8MatMulBwdBuffers / TFp8MatMulBwdBuffers allocate
+ * from the reference's pools (src/gpt/compute/matmul_fwdbwd.cuh:108-125,283-311): out[0] grad8, [1] grad8RowScale, [2] gradT, [3] srcT,
+ * [4] tileMax, [5] tileScale, [6] transformT, [7] partial (splits slices), [8] gradRowAbsMax; members the mode does not use are 0.
+ * Rows are dense (stride = row bytes).  Returns TS2_ERR_SHAPE for sizes the operator refuses. */
+int ts2_matmul_bwd_scratch_bytes(int32_t mode, int32_t lenRound, int32_t srcDim, int32_t gradDim, int32_t kTile, int32_t splits, int64_t out[9]);
+
 /* BackpropMulti (prep of dX): I8: quantise grad (TS2_BF16 | TS2_F32, optionally times gradColScale[gradDim]) per row to
  * grad8/grad8RowScale and transpose the weight; E4M3: transpose the weight.  transformFast is [gradDim][srcDim]. */
 int ts2_matmul_backprop_multi(int32_t mode, int32_t len, int32_t lenRound, int32_t srcDim, int32_t gradDim, const ts2_mat *transformFast,
@@ -447,6 +453,15 @@ int ts2_model_set_bias(ts2_model *m, const float *biasHost);
  * row and attention type, RoPE table [len][128]; host arrays */
 int ts2_model_set_batch(ts2_model *m, int32_t len, const int32_t *labelPtr, const uint32_t *labels, const int32_t *targetPerRow,
     const int32_t *const *spanStart, const int32_t *const *spanFinish, const float *ropeBuf, void *stream);
+/* The checks ts2_model_set_batch makes before it copies anything, as a host-only function (no device access): label CSR monotone from 0
+ * and within labelCap, label ids (low 31 bits; bit 31 is the sign of the embedding term, src/gpt/compute/cpu_transformer.cpp:76-100) below
+ * labelCount, -1 <= target < vocab, and for every attention type and row 0 <= start <= len, finish < len, finish >= start - 1.  The
+ * reference trusts its own node builder (InitLabelData, src/gpt/att/sliding_window.cpp:269-306); a caller-supplied batch that breaks one
+ * of these would be an out-of-bounds access on the device, so it is refused with TS2_ERR_SHAPE / TS2_ERR_NULL instead.
+ * ts2_model_set_batch, ts2_model_set_matrix and ts2_model_set_bias copy with blocking copies on the null stream; set_batch waits for
+ * `stream` first, so a step still running there cannot see a half-written batch. */
+int ts2_validate_batch(int32_t len, int32_t labelCap, int32_t labelCount, int32_t vocab, int32_t attTypeCount, const int32_t *labelPtr,
+    const uint32_t *labels, const int32_t *targetPerRow, const int32_t *const *spanStart, const int32_t *const *spanFinish);
 int ts2_model_forward(ts2_model *m, void *stream);  /* states + predictions ("prediction" array holds probabilities) */
 int ts2_model_backprop(ts2_model *m, void *stream); /* forward, loss gradient, backward through all layers, every delta */
 /* one layer in isolation on the model's buffers ("state" in, "state" out / "stateGrad" in-out) */
@@ -464,14 +479,6 @@ int ts2_model_scalars(ts2_model *m, float *lossSumHost, int32_t *lenRound, int32
 /* peak dense MFMA rate the library prices its kernels against, in T(FL)OP/s, and the CU count it tiles for */
 int ts2_device_info(int *cuCount, int *clockMHz);
 
-/* Machine probes (no counterpart in the reference; they exist so that the benchmark can price kernels against what the device
- * sustains, beside the published peaks).
- * ts2_probe_mfma_rate: runs nothing but MFMAs of the given operand type (TS2_I8 / TS2_E4M3 / TS2_BF16) on every CU, iters x 4 per wave,
- *   with constant operands (randomData = 0) or per-lane hashed bit patterns (1), and returns the sustained rate in T(FL)OP/s.
- *   scratch: device buffer of at least 256 ints per CU.
- * ts2_probe_copy_rate: streaming copy, four 16-byte loads in flight per lane, of `bytes` bytes (a multiple of 16); returns read+write GB/s. */
-int ts2_probe_mfma_rate(int32_t abType, int32_t randomData, int32_t iters, int32_t *scratch, int64_t scratchInts, double *topsOut, void *stream);
-int ts2_probe_copy_rate(const void *src, void *dst, int64_t bytes, double *gbPerSecOut, void *stream);
 const char *ts2_version(void);
 
 #ifdef __cplusplus

@@ -1,0 +1,25 @@
+/*
+ * ts2_probe.h - machine probes of the benchmark (libts2probe.so).  Not part of the product ABI: nothing in libts2amd.so depends on them.
+ */
+#ifndef TS2_PROBE_H
+#define TS2_PROBE_H
+#include <stdint.h>
+#include "ts2_abi.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Machine probes (no counterpart in the reference; they exist so that the benchmark can price kernels against what the device
+ * sustains, beside the published peaks).
+ * ts2_probe_mfma_rate: runs nothing but MFMAs of the given operand type (TS2_I8 / TS2_E4M3 / TS2_BF16) on every CU, iters x 4 per wave,
+ *   with constant operands (randomData = 0) or per-lane hashed bit patterns (1), and returns the sustained rate in T(FL)OP/s.
+ *   scratch: device buffer of at least 256 ints per CU.
+ * ts2_probe_copy_rate: streaming copy, four 16-byte loads in flight per lane, of `bytes` bytes (a multiple of 16); returns read+write GB/s. */
+int ts2_probe_mfma_rate(int32_t abType, int32_t randomData, int32_t iters, int32_t *scratch, int64_t scratchInts, double *topsOut, void *stream);
+int ts2_probe_copy_rate(const void *src, void *dst, int64_t bytes, double *gbPerSecOut, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -752,10 +752,6 @@ bool ActOk(const ts2_mat *m, int rows, int cols)
     return m && m->ptr && m->y >= rows && m->x >= cols && Aligned16(m->ptr, m->strideBytes);
 }
 
-int SetAttr(const void *fn, int bytes)
-{
-    return hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess ? 0 : TS2_ERR_LAUNCH;
-}
 } // namespace
 
 extern "C" int ts2_att_build_rev(int32_t len, int32_t lenRound, const int32_t *spanStart, const int32_t *spanFinish, int32_t *revLo, int32_t *revHi,
@@ -803,12 +799,9 @@ extern "C" int ts2_att_forward(const ts2_att_args *a, void *stream)
     p.ldo0 = a->valLookup.strideBytes;
     p.lenRound = a->lenRound;
     int ldsBytes = RM_BYTES + T_BYTES + OWN_BYTES;
-    static bool done = false;
-    if (!done) {
-        if (SetAttr((const void *)AttForward, ldsBytes)) {
-            return TS2_ERR_LAUNCH;
-        }
-        done = true;
+    static std::atomic<bool> done{false};
+    if (!Ts2SetDynamicLds(done, (const void *)AttForward, ldsBytes)) {
+        return TS2_ERR_LAUNCH;
     }
     hipLaunchKernelGGL(AttForward, dim3(a->lenRound / BROWS, a->heads), dim3(256), ldsBytes, (hipStream_t)stream, p);
     TS2_CHECK_LAUNCH();
@@ -853,12 +846,9 @@ extern "C" int ts2_att_backward(const ts2_att_grad_args *a, void *stream)
     p.lenRound = a->lenRound;
     dim3 grid(a->lenRound / BROWS, a->heads);
     int ldsQ = 2 * RM_BYTES + T_BYTES + 2 * OWN_BYTES;
-    static bool done = false;
-    if (!done) {
-        if (SetAttr((const void *)AttGradQ<true>, ldsQ) || SetAttr((const void *)AttGradQ<false>, ldsQ)) {
-            return TS2_ERR_LAUNCH;
-        }
-        done = true;
+    static std::atomic<bool> doneQ0{false}, doneQ1{false};
+    if (!Ts2SetDynamicLds(doneQ1, (const void *)AttGradQ<true>, ldsQ) || !Ts2SetDynamicLds(doneQ0, (const void *)AttGradQ<false>, ldsQ)) {
+        return TS2_ERR_LAUNCH;
     }
     if (a->which & 1) {
         p.out0 = (uint8_t *)a->dQ.ptr;

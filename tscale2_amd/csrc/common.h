@@ -1,6 +1,7 @@
 // Shared device/host helpers for the gfx950 kernels.  64-wide wavefronts throughout.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <stdint.h>
 #include "../../include/ts2_abi.h"
 
@@ -20,6 +21,20 @@ constexpr int TILE = 128; // STATE_NORM_TILE / MM_TILE of the reference (model_d
         if (hipGetLastError() != hipSuccess)                                                                                               \
             return TS2_ERR_LAUNCH;                                                                                                         \
     } while (0)
+
+// Raises a kernel's dynamic-LDS limit once per call site.  `done` is the call site's own flag; the attribute call is idempotent, so two
+// host threads that both find the flag clear simply both set it.
+inline bool Ts2SetDynamicLds(std::atomic<bool> &done, const void *kernel, int bytes)
+{
+    if (done.load(std::memory_order_acquire)) {
+        return true;
+    }
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
+        return false;
+    }
+    done.store(true, std::memory_order_release);
+    return true;
+}
 
 __device__ __forceinline__ float Bf16ToFloat(bf16_t x)
 {

@@ -1426,12 +1426,9 @@ template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT> int Launch(const
     q.tilesN = (p.n + BN - 1) / BN;
     int ldsBytes = 2 * (BM + BN) * BKB;
     auto kern = GemmNT<TYPE, WTM, WTN, CT, EPI, KT>;
-    static bool attrDone = false; // per instantiation
-    if (!attrDone) {
-        if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes) != hipSuccess) {
-            return TS2_ERR_LAUNCH;
-        }
-        attrDone = true;
+    static std::atomic<bool> attrDone{false}; // per instantiation
+    if (!Ts2SetDynamicLds(attrDone, (const void *)kern, ldsBytes)) {
+        return TS2_ERR_LAUNCH;
     }
     int nb = q.tilesM * q.tilesN * (p.splitK > 1 ? p.splitK : 1);
     if (p.direct && p.splitK <= 1) {

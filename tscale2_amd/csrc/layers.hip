@@ -993,6 +993,42 @@ extern "C" void ts2_model_destroy(ts2_model *M)
     delete M;
 }
 
+static int Ts2ValidateBatch(int len, int labelCap, int labelCount, int vocab, int attTypeCount, const int32_t *labelPtr, const uint32_t *labels,
+    const int32_t *targetPerRow, const int32_t *const *spanStart, const int32_t *const *spanFinish)
+{
+    if (!labelPtr || !labels || !targetPerRow || (attTypeCount > 0 && (!spanStart || !spanFinish))) {
+        return TS2_ERR_NULL;
+    }
+    if (len <= 0 || labelPtr[0] != 0) {
+        return TS2_ERR_SHAPE;
+    }
+    for (int t = 0; t < len; ++t) {
+        if (labelPtr[t + 1] < labelPtr[t] || labelPtr[t + 1] > labelCap) {
+            return TS2_ERR_SHAPE;
+        }
+        if (targetPerRow[t] < -1 || targetPerRow[t] >= vocab) {
+            return TS2_ERR_SHAPE;
+        }
+    }
+    for (int i = 0, n = labelPtr[len]; i < n; ++i) {
+        if ((labels[i] & 0x7fffffffu) >= (uint32_t)labelCount) {
+            return TS2_ERR_SHAPE;
+        }
+    }
+    for (int a = 0; a < attTypeCount; ++a) {
+        if (!spanStart[a] || !spanFinish[a]) {
+            return TS2_ERR_NULL;
+        }
+        for (int t = 0; t < len; ++t) {
+            const int st = spanStart[a][t], fi = spanFinish[a][t];
+            if (st < 0 || st > len || fi >= len || fi < st - 1) {
+                return TS2_ERR_SHAPE;
+            }
+        }
+    }
+    return 0;
+}
+
 static TMatrix *FindMatrix(ts2_model *M, int layer, int matrixId)
 {
     if (layer == TS2_LAYER_EMBED) {
@@ -1032,14 +1068,33 @@ extern "C" int ts2_model_set_bias(ts2_model *M, const float *biasHost)
     return hipMemcpy(M->bias, biasHost, (size_t)M->cfg.vocab * 4, hipMemcpyHostToDevice) == hipSuccess ? 0 : TS2_ERR_LAUNCH;
 }
 
+// Host-side check of a batch (no device access): label CSR monotone and within capacity, label ids (low 31 bits; the top bit is the
+// sign of the embedding term) below labelCount, targets in [-1, vocab), every span inside [0, len) with finish >= start - 1.
+extern "C" int ts2_validate_batch(int32_t len, int32_t labelCap, int32_t labelCount, int32_t vocab, int32_t attTypeCount, const int32_t *labelPtr,
+    const uint32_t *labels, const int32_t *targetPerRow, const int32_t *const *spanStart, const int32_t *const *spanFinish)
+{
+    return Ts2ValidateBatch(len, labelCap, labelCount, vocab, attTypeCount, labelPtr, labels, targetPerRow, spanStart, spanFinish);
+}
+
 extern "C" int ts2_model_set_batch(ts2_model *M, int32_t len, const int32_t *labelPtr, const uint32_t *labels, const int32_t *targetPerRow,
     const int32_t *const *spanStart, const int32_t *const *spanFinish, const float *ropeBuf, void *stream)
 {
     if (!M || !labelPtr || !labels || !targetPerRow || !ropeBuf) {
         return TS2_ERR_NULL;
     }
-    if (len <= 0 || len > M->cfg.maxLen || labelPtr[len] > M->labelCap) {
+    if (len <= 0 || len > M->cfg.maxLen) {
         return TS2_ERR_SHAPE;
+    }
+    // every index the kernels follow is checked here, before anything is copied: a label, a target or a span outside its range would
+    // be an out-of-bounds access on the device (embedding rows, logit columns, key rows of the attention)
+    int rcBatch = Ts2ValidateBatch(len, M->labelCap, M->cfg.labelCount, M->cfg.vocab, M->cfg.attTypeCount, labelPtr, labels, targetPerRow,
+        spanStart, spanFinish);
+    if (rcBatch != 0) {
+        return rcBatch;
+    }
+    // the uploads below are blocking copies on the null stream; the step they feed must not still be running on a non-blocking stream
+    if (stream && hipStreamSynchronize((hipStream_t)stream) != hipSuccess) {
+        return TS2_ERR_LAUNCH;
     }
     M->len = len;
     int R = M->R;

@@ -11,6 +11,36 @@ bool Is8(int mode)
 }
 } // namespace
 
+extern "C" int ts2_matmul_bwd_scratch_bytes(int32_t mode, int32_t lenRound, int32_t srcDim, int32_t gradDim, int32_t kTile, int32_t splits,
+    int64_t out[9])
+{
+    if (!out) {
+        return TS2_ERR_NULL;
+    }
+    if (!Is8(mode)) {
+        return TS2_ERR_UNSUPPORTED;
+    }
+    if (kTile <= 0) {
+        kTile = 512;
+    }
+    if (srcDim <= 0 || gradDim <= 0 || lenRound <= 0 || srcDim % 128 || gradDim % 128 || lenRound % 128 || kTile % 128 || splits < 0 ||
+        (mode == TS2_I8 && lenRound % kTile)) {
+        return TS2_ERR_SHAPE;
+    }
+    const int64_t L = lenRound, S = srcDim, G = gradDim, nTiles = (L + kTile - 1) / kTile;
+    const bool i8 = mode == TS2_I8;
+    out[0] = i8 ? L * G : 0;         // grad8
+    out[1] = i8 ? L * 4 : 0;         // grad8RowScale
+    out[2] = G * L;                  // gradT
+    out[3] = S * L;                  // srcT
+    out[4] = i8 ? nTiles * 4 : 0;    // tileMax
+    out[5] = i8 ? nTiles * 4 : 0;    // tileScale
+    out[6] = S * G;                  // transformT
+    out[7] = splits > 1 ? (int64_t)splits * G * S * 4 : 0; // partial
+    out[8] = i8 ? L * 4 : 0;         // gradRowAbsMax (optional)
+    return TS2_OK;
+}
+
 extern "C" int ts2_matmul_backprop_multi(int32_t mode, int32_t len, int32_t lenRound, int32_t srcDim, int32_t gradDim,
     const ts2_mat *transformFast, const ts2_mat *grad, int32_t gradType, const float *gradColScale, const ts2_matmul_bwd_buffers *buf, void *stream)
 {

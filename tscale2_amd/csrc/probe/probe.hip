@@ -2,7 +2,8 @@
 // The published MFMA peak assumes the boost clock; with operands that toggle like real data the chip is power limited well below it,
 // so a kernel's distance from "what the MFMA pipe sustains with nothing else running" is reported next to its fraction of the
 // published peak.  These entry points have no counterpart in the reference.
-#include "common.h"
+#include "../common.h"
+#include "../../../include/ts2_probe.h"
 
 namespace {
 
@@ -108,15 +109,23 @@ template <class TLaunch> int TimeIt(hipStream_t stream, float *ms, const TLaunch
     return rc;
 }
 
+int CuCount()
+{
+    int dev = 0, cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+        return 0;
+    }
+    return cu;
+}
+
 } // namespace
 
 extern "C" int ts2_probe_mfma_rate(int32_t abType, int32_t randomData, int32_t iters, int32_t *scratch, int64_t scratchInts, double *topsOut,
     void *streamV)
 {
     hipStream_t stream = (hipStream_t)streamV;
-    int cu = 0, mhz = 0;
-    ts2_device_info(&cu, &mhz);
-    if (iters <= 0 || !scratch || !topsOut || scratchInts < (int64_t)cu * 256) {
+    const int cu = CuCount();
+    if (cu <= 0 || iters <= 0 || !scratch || !topsOut || scratchInts < (int64_t)cu * 256) {
         return TS2_ERR_SHAPE;
     }
     float ms = 0;
@@ -144,11 +153,10 @@ extern "C" int ts2_probe_mfma_rate(int32_t abType, int32_t randomData, int32_t i
 extern "C" int ts2_probe_copy_rate(const void *src, void *dst, int64_t bytes, double *gbPerSecOut, void *streamV)
 {
     hipStream_t stream = (hipStream_t)streamV;
-    if (bytes <= 0 || bytes % 16 || !src || !dst || !gbPerSecOut) {
+    const int cu = CuCount();
+    if (cu <= 0 || bytes <= 0 || bytes % 16 || !src || !dst || !gbPerSecOut) {
         return TS2_ERR_SHAPE;
     }
-    int cu = 0, mhz = 0;
-    ts2_device_info(&cu, &mhz);
     float ms = 0;
     int rc = TimeIt(stream, &ms, [&] { hipLaunchKernelGGL(CopyRate, dim3(cu * 128), dim3(256), 0, stream, (const v4i *)src, (v4i *)dst, bytes / 16); });
     if (rc != TS2_OK) {

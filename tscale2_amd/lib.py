@@ -5,6 +5,7 @@ import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SO = os.path.join(HERE, "libts2amd.so")
+PROBE_SO = os.path.join(HERE, "libts2probe.so")  # the benchmark's machine probes (include/ts2_probe.h), not part of the product ABI
 
 I8, E4M3, BF16, F32, I32, F16 = 0, 1, 2, 3, 4, 5
 EPI_STORE, EPI_ADD, EPI_ROW_TILE_MAXNORM, EPI_ROW_TILE_NORM = 0, 1, 2, 3
@@ -134,13 +135,25 @@ def call(name, *args, check=True):
     return rc
 
 
+_probe = None
+
+
+def _probe_lib():
+    global _probe
+    if _probe is None:
+        if not os.path.exists(PROBE_SO):
+            raise RuntimeError(f"{PROBE_SO} is missing: build it with `python -m tscale2_amd.build`")
+        _probe = C.CDLL(PROBE_SO)
+    return _probe
+
+
 def probe_mfma_rate(ab_type, random_data, iters=20000):
     """Sustained rate, in T(FL)OP/s, of a kernel that issues nothing but MFMAs of the given operand type on every CU."""
     import torch
     lib = load()
     scratch = torch.empty(1024 * 256, dtype=torch.int32, device="cuda")
     out = C.c_double(0)
-    lib.check(lib.dll.ts2_probe_mfma_rate(C.c_int32(ab_type), C.c_int32(int(random_data)), C.c_int32(iters), ptr(scratch),
+    lib.check(_probe_lib().ts2_probe_mfma_rate(C.c_int32(ab_type), C.c_int32(int(random_data)), C.c_int32(iters), ptr(scratch),
                                           C.c_int64(scratch.numel()), C.byref(out), lib.stream()), "ts2_probe_mfma_rate")
     return out.value
 
@@ -152,7 +165,7 @@ def probe_copy_rate(nbytes=1 << 30):
     src = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
     dst = torch.empty_like(src)
     out = C.c_double(0)
-    lib.check(lib.dll.ts2_probe_copy_rate(ptr(src), ptr(dst), C.c_int64(nbytes), C.byref(out), lib.stream()), "ts2_probe_copy_rate")
+    lib.check(_probe_lib().ts2_probe_copy_rate(ptr(src), ptr(dst), C.c_int64(nbytes), C.byref(out), lib.stream()), "ts2_probe_copy_rate")
     return out.value
 
 
