@@ -386,6 +386,17 @@ typedef struct ts2_moe_tables {
 int ts2_moe_route(int32_t len, int32_t lenMoe, int32_t experts, int32_t selected, const ts2_mat *select, int32_t selectType,
     const ts2_moe_tables *tables, void *stream);
 
+/* ts2_moe_route for callers that cannot allocate and have no workspace to hand over (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same tables and same results as ts2_moe_route; the
+ * counting sort's scratch (tables->blockCounts there, ignored here and may be NULL) is a fixed device array inside the library:
+ * TS2_MOE_ROUTE_STATIC_INTS ints (512 KiB) held by every GPU the library runs on until the process ends.  A call needs
+ * ceil(len*selected/256) * experts <= TS2_MOE_ROUTE_STATIC_INTS (e.g. 65536 tokens, top-2, 64 experts: 32768) and returns TS2_ERR_SHAPE
+ * beyond that.  The call allocates and frees nothing.  All calls on one GPU share that GPU's array: calls that may overlap on one GPU
+ * (different streams, different host threads) race and must be ordered by the caller. */
+#define TS2_MOE_ROUTE_STATIC_INTS 131072
+int ts2_moe_route_static(int32_t len, int32_t lenMoe, int32_t experts, int32_t selected, const ts2_mat *select, int32_t selectType,
+    const ts2_moe_tables *tables, void *stream);
+
 /* MoeGroupSamples (moe_kernels.cuh:89-143): dst[row] = src[xpSampleId[row]] (zeros for padding) for row < lenMoe; elemSize 1 or 2
  * bytes.  The transposed copy the reference can emit is ts2_transpose_quant with rowIndex = xpSampleId. */
 int ts2_moe_group_samples(int32_t lenMoe, int32_t elemSize, const ts2_mat *src, const int32_t *xpSampleId, const ts2_mat *dst, void *stream);

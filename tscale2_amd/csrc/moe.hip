@@ -400,16 +400,11 @@ bool TablesOk(const ts2_moe_tables *t)
 
 #define STREAM ((hipStream_t)stream)
 
-extern "C" int ts2_moe_route(int32_t len, int32_t lenMoe, int32_t experts, int32_t selected, const ts2_mat *select, int32_t selectType,
-    const ts2_moe_tables *tb, void *stream)
+// Routing tables from the select logits; blockCounts is the counting sort's scratch: [ceil(len*selected/RB)][experts] ints, every entry in
+// use written by MoeLocalRank before it is read, so it needs no clearing between calls.
+static int MoeRoute(int32_t len, int32_t lenMoe, int32_t experts, int32_t selected, const ts2_mat *select, int32_t selectType,
+    const ts2_moe_tables *tb, int *blockCounts, void *stream)
 {
-    if (!select || !TablesOk(tb) || !tb->blockCounts) {
-        return TS2_ERR_NULL;
-    }
-    if (experts <= 0 || experts > 256 || selected <= 0 || selected > experts || selected > 64 || lenMoe % TILE ||
-        lenMoe < len * selected + TILE * experts || select->x < experts || select->y < len) {
-        return TS2_ERR_SHAPE;
-    }
     if (selectType == TS2_F32) {
         hipLaunchKernelGGL((MoeCalcSampleExpertLists<TF32>), dim3((len + 3) / 4), dim3(256), 0, STREAM, len, experts, selected, M(*select),
             tb->sampleExpertIds, tb->sampleExpertWeights);
@@ -422,26 +417,92 @@ extern "C" int ts2_moe_route(int32_t len, int32_t lenMoe, int32_t experts, int32
     TS2_CHECK_LAUNCH();
     int total = len * selected;
     int nBlocks = (total + RB - 1) / RB;
-    hipLaunchKernelGGL(MoeLocalRank, dim3(nBlocks), dim3(RB), 0, STREAM, total, experts, tb->sampleExpertIds, tb->sampleExpertOffset, tb->blockCounts);
+    hipLaunchKernelGGL(MoeLocalRank, dim3(nBlocks), dim3(RB), 0, STREAM, total, experts, tb->sampleExpertIds, tb->sampleExpertOffset, blockCounts);
     TS2_CHECK_LAUNCH();
     const size_t tableBytes = (size_t)nBlocks * experts * 4;
     const int useLds = tableBytes <= 150 * 1024;
-    static bool attrDone = false;
-    if (!attrDone) {
-        if (hipFuncSetAttribute((const void *)MoeOffsets, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) != hipSuccess) {
-            return TS2_ERR_LAUNCH;
-        }
-        attrDone = true;
+    static std::atomic<bool> attrDone{false};
+    if (!Ts2SetDynamicLds(attrDone, (const void *)MoeOffsets, 150 * 1024)) {
+        return TS2_ERR_LAUNCH;
     }
-    hipLaunchKernelGGL(MoeOffsets, dim3(1), dim3(1024), useLds ? tableBytes : 0, STREAM, nBlocks, experts, lenMoe, tb->blockCounts, tb->expertOffset,
+    hipLaunchKernelGGL(MoeOffsets, dim3(1), dim3(1024), useLds ? tableBytes : 0, STREAM, nBlocks, experts, lenMoe, blockCounts, tb->expertOffset,
         tb->xpTileExpertId, useLds);
     TS2_CHECK_LAUNCH();
     hipLaunchKernelGGL(MoeInitXp, dim3((lenMoe + 255) / 256), dim3(256), 0, STREAM, lenMoe, tb->xpSampleId, tb->xpSampleWeight);
     TS2_CHECK_LAUNCH();
     hipLaunchKernelGGL(MoeFillXp, dim3(nBlocks), dim3(RB), 0, STREAM, total, experts, selected, tb->sampleExpertIds, tb->sampleExpertWeights,
-        tb->sampleExpertOffset, tb->blockCounts, tb->expertOffset, tb->xpSampleId, tb->xpSampleWeight);
+        tb->sampleExpertOffset, blockCounts, tb->expertOffset, tb->xpSampleId, tb->xpSampleWeight);
     TS2_CHECK_LAUNCH();
     return TS2_OK;
+}
+
+static int MoeRouteShapeOk(int32_t len, int32_t lenMoe, int32_t experts, int32_t selected, const ts2_mat *select)
+{
+    return !(len <= 0 || experts <= 0 || experts > 256 || selected <= 0 || selected > experts || selected > 64 || lenMoe % TILE ||
+             (int64_t)lenMoe < (int64_t)len * selected + (int64_t)TILE * experts || select->x < experts || select->y < len);
+}
+
+extern "C" int ts2_moe_route(int32_t len, int32_t lenMoe, int32_t experts, int32_t selected, const ts2_mat *select, int32_t selectType,
+    const ts2_moe_tables *tb, void *stream)
+{
+    if (!select || !TablesOk(tb) || !tb->blockCounts) {
+        return TS2_ERR_NULL;
+    }
+    if (!MoeRouteShapeOk(len, lenMoe, experts, selected, select)) {
+        return TS2_ERR_SHAPE;
+    }
+    return MoeRoute(len, lenMoe, experts, selected, select, selectType, tb, tb->blockCounts, stream);
+}
+
+// ---- the routing entry point that allocates nothing and takes no workspace: the counting sort's scratch is a file-scope device array.
+// Every device the library runs on holds its own copy of the array at its own address (until the process ends); the name below is only
+// the host-side handle of the symbol, never a device address: host code uses the per-device pointer hipGetSymbolAddress returns.
+static __device__ __align__(256) int g_moeRouteScratch[TS2_MOE_ROUTE_STATIC_INTS];
+
+namespace
+{
+constexpr int MAX_DEVICES = 64;
+std::atomic<int *> g_moeRouteScratchPtr[MAX_DEVICES]; // zero-initialised (static storage)
+
+// device address of this device's copy of the scratch array (resolved once per device, with that device current)
+int *MoeRouteScratch()
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+        return nullptr;
+    }
+    int *p = g_moeRouteScratchPtr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        void *sym = nullptr;
+        if (hipGetSymbolAddress(&sym, HIP_SYMBOL(g_moeRouteScratch)) != hipSuccess || !sym) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        p = (int *)sym;
+        g_moeRouteScratchPtr[dev].store(p, std::memory_order_release); // two threads racing here store the same address
+    }
+    return p;
+}
+} // namespace
+
+extern "C" int ts2_moe_route_static(int32_t len, int32_t lenMoe, int32_t experts, int32_t selected, const ts2_mat *select, int32_t selectType,
+    const ts2_moe_tables *tb, void *stream)
+{
+    if (!select || !TablesOk(tb)) {
+        return TS2_ERR_NULL;
+    }
+    if (!MoeRouteShapeOk(len, lenMoe, experts, selected, select)) {
+        return TS2_ERR_SHAPE;
+    }
+    const int64_t nBlocks = ((int64_t)len * selected + RB - 1) / RB;
+    if (nBlocks * experts > TS2_MOE_ROUTE_STATIC_INTS) {
+        return TS2_ERR_SHAPE; // beyond the fixed scratch: use ts2_moe_route with a caller-owned blockCounts
+    }
+    int *scratch = MoeRouteScratch();
+    if (!scratch) {
+        return TS2_ERR_LAUNCH;
+    }
+    return MoeRoute(len, lenMoe, experts, selected, select, selectType, tb, scratch, stream);
 }
 
 extern "C" int ts2_moe_group_samples(int32_t lenMoe, int32_t elemSize, const ts2_mat *src, const int32_t *xpSampleId, const ts2_mat *dst, void *stream)
