@@ -4,12 +4,20 @@
  * reference's fp32 CPU path (file:line given at each definition).  All matrices are dense row-major float arrays
  * [rows][cols]; "len" is the number of token rows.
  *
- * Pinning status (what each function is checked against in tests/):
- *   linalg / norm / lolu / rope / attention / span graph / i8 + e4m3 converters / model schedule / label data
- *       -> bit-exact against the reference's own sources compiled into oracle/_ref/libts2ref.so, plus closed forms.
- *   delta compress, per-matrix quantiser, MoE routing, layer glue (FFN/attention/MoE layers, head, embedding)
- *       -> the reference files holding them need cuda_runtime.h and cannot be compiled here; pinned by closed forms,
- *          brute force, finite differences in fp64 and adjoint identities.
+ * Pinning status (what each function is checked against in tests/; "ref" = the reference's own sources compiled into
+ * oracle/_ref/libts2ref.so and the committed vectors they produced, tests/golden/ref_golden.npz):
+ *   mul_forward, mul_backward_accum, sum_rank_one, normalize_state(+backward), lolu, backprop_lolu, fill_rope_buf, apply_rope,
+ *   attention_forward, compute_dscale, attention_grad_q, attention_grad_k, transpose_attention, convert_i8, convert_e4m3,
+ *   e4m3_to_float, cvt_i8, cvt_e4m3, model_schedule, make_causal_spans (+ the harness's labels and targets)
+ *       -> bit-exact against ref (tests/test_oracle_vs_reference.py over tests/golden_cases.py).
+ *   cvt_e4m3_rne, compress_delta, quantize_matrix_i8/e4m3, grad_mult, cpu_moe, cpu_backprop_moe, scale_experts,
+ *   backprop_scale_experts, fwd/bwd_contract_matrix, layer_forward, layer_backward, final_backward, model_step
+ *       -> their reference sources need cuda_runtime.h and cannot be compiled here; pinned by brute force over the code table,
+ *          invariants, bilinear / adjoint identities and fp64 finite differences (tests/test_oracle_closed_forms.py).
+ *   quant_rowmax_i8, quant_ktile_i8, gemm_i8_nt, gemm_i8_nt_rowscale, gemm_i8_nt_ktile, gemm_f32_nt, dequant_i8/e4m3, bf16_round,
+ *   softmax2, embedding_forward/backward, and the same-contract layer functions (orc_sc_*)
+ *       -> this library's own contracts and helpers: closed forms against numpy round-half-even and int64 products, torch's bfloat16
+ *          conversion, scipy's softmax, adjoint identities (tests/test_oracle_own_contract.py, tests/test_same_contract_cpu.py).
  */
 #ifndef TS2_ORACLE_H
 #define TS2_ORACLE_H

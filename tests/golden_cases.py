@@ -92,5 +92,54 @@ def case_convert(o):
     return {"i8": o.convert_i8(x, 1.0), "i8s": o.convert_i8(x, 0.37), "e4": o.convert_e4m3(y, 1.0), "e4s": o.convert_e4m3(y, 7.3), "tab": tab}
 
 
+MODEL_STRINGS = ["e256h2d4ffn8w64", "e2048h16d12ffn64w1024", "e512h4d1ffn16w256", "e1024xp512moe64moes2h8d1w128", "e512xp256moe8moes2h4d26w512"]
+
+
+def case_model_schedule(o):
+    """layer schedule of a model string (InitAlibi, src/gpt/model_params/model_dim.cpp:82-158): the oracle builds it from the numbers
+    the test harness reads out of the string; the reference build parses the string itself and also reports those numbers"""
+    from model_harness import parse_model_descr
+    out = {}
+    for i, descr in enumerate(MODEL_STRINGS):
+        dims, wide = parse_model_descr(descr)
+        r = o.model_schedule(descr, int(dims[9]), int(dims[6]), wide)
+        out[f"{i}_dims"] = r.get("dims", dims)
+        for k in ("layer_type", "layer_att_id", "layer_slope", "att_width"):
+            out[f"{i}_{k}"] = r[k]
+    return out
+
+
+def case_label_data(o):
+    """nodes of a batch (InitLabelData with noise labels disabled, src/gpt/att/sliding_window.cpp:269-306): labels, targets and the
+    causal spans of every attention type, as the test harness builds them"""
+    from model_harness import make_batch, parse_model_descr
+    out = {}
+    for i, (descr, vocab, fc, fl) in enumerate([("e256h2d4ffn8w64", 256, 3, 70), ("e256h2d1ffn8w16", 50, 2, 40), ("e256h2d4ffn8w1024", 1000, 2, 150)]):
+        tokens = _rng(200 + i).integers(0, vocab, (fc, fl)).astype(np.int32)
+        dims, wide = parse_model_descr(descr)
+        widths = o.model_schedule(descr, int(dims[9]), int(dims[6]), wide)["att_width"]
+        if o.use_ref:
+            tg = np.full((fc, fl), -1, np.int32)
+            tg[:, :-1] = tokens[:, 1:]
+            for a in range(len(widths)):
+                r = o.ref_label_data(descr, vocab, tokens, tg, a)
+                for k in ("label_count", "label_ptr", "labels", "target_pairs"):
+                    out[f"{i}_{k}"] = r[k]
+                out[f"{i}_span_ptr{a}"] = r["span_ptr"]
+                out[f"{i}_spans{a}"] = r["spans"].reshape(-1, 2)
+        else:
+            b = make_batch(o, vocab, tokens, widths)
+            out[f"{i}_label_count"] = np.array([b["label_count"]], np.int32)
+            out[f"{i}_label_ptr"] = b["label_ptr"]
+            out[f"{i}_labels"] = b["labels"]
+            rows = np.nonzero(b["target"] >= 0)[0]
+            out[f"{i}_target_pairs"] = np.stack([rows, b["target"][rows]], 1).astype(np.int32)
+            for a, (sp, ss) in enumerate(b["spans"]):
+                out[f"{i}_span_ptr{a}"] = sp
+                out[f"{i}_spans{a}"] = np.asarray(ss, np.int32).reshape(-1, 2)
+    return out
+
+
 def build_cases():
-    return {"linalg": case_linalg, "norm_lolu": case_norm_lolu, "rope": case_rope, "attention": case_attention, "convert": case_convert}
+    return {"linalg": case_linalg, "norm_lolu": case_norm_lolu, "rope": case_rope, "attention": case_attention, "convert": case_convert,
+            "model_schedule": case_model_schedule, "label_data": case_label_data}

@@ -13,11 +13,34 @@ I8, E4M3 = 0, 1
 
 
 def schedule(orc, depth, experts, wide_window):
-    lt = np.zeros(256, np.int32); la = np.zeros(256, np.int32); ls = np.zeros(256, np.float32)
-    aw = np.zeros(4, np.int32); ac = C.c_int(0)
-    n = orc.lib.orc_model_schedule(depth, experts, wide_window, _ptr(lt), _ptr(la), _ptr(ls), 256, _ptr(aw), C.byref(ac))
-    assert n > 0
-    return lt[:n].copy(), la[:n].copy(), ls[:n].copy(), aw[:ac.value].copy()
+    r = orc.model_schedule(None, depth, experts, wide_window)
+    return r["layer_type"], r["layer_att_id"], r["layer_slope"], r["att_width"]
+
+
+def parse_model_descr(descr):
+    """The numbers a reference model string stands for (TModelDescrString, src/gpt/model_params/model_dim.cpp:17-58), in the order
+    {Dim, QDim, TTDim, ExpertDim, HeadCount, FfnTiles, MoeExpertCount, MoeSelected, KVrep, Depth} + the wide attention window.
+    Fields that a string does not name keep the reference's defaults."""
+    import re
+    f = {k: float(v) for k, v in re.findall(r"([a-z]+)([0-9.]+)", descr)}
+    dims = [int(f.get("e", 256)), 128, 128, int(f.get("xp", 128)), int(f.get("h", 1)), int(f.get("ffn", 1)), int(f.get("moe", 0)),
+            int(f.get("moes", 2)), int(f.get("rep", 16)), int(f.get("d", 60))]
+    return np.array(dims, np.int32), int(f.get("w", 64))
+
+
+def make_batch(orc, vocab, tokens, att_widths):
+    """Nodes of a batch of equal-length fragments as InitLabelData builds them with noise labels disabled
+    (src/gpt/att/sliding_window.cpp:269-306): one label 1 + token per node, target = next token of the fragment (none for the last),
+    one causal span [max(fragment start, t - width), t - 1] per node and attention type."""
+    tokens = np.asarray(tokens)
+    frag_count, frag_len = tokens.shape
+    n = frag_count * frag_len
+    label_ptr = np.arange(n + 1, dtype=np.int32)
+    labels = (1 + tokens).astype(np.uint32).ravel()
+    tg = np.full((frag_count, frag_len), -1, np.int32)
+    tg[:, :-1] = tokens[:, 1:]
+    spans = [orc.make_causal_spans(frag_count, frag_len, int(w)) for w in att_widths]
+    return {"label_count": vocab + 1, "label_ptr": label_ptr, "labels": labels, "target": tg.ravel(), "spans": spans}
 
 
 def layer_shapes(ltype, dim, heads, ffn, xp, experts):
@@ -75,12 +98,9 @@ class Harness:
         # batch: uniform random tokens, target = next token of the fragment, label = 1 + token (noise labels disabled)
         self.n = frag_count * frag_len
         tokens = r.integers(0, vocab, (frag_count, frag_len))
-        self.label_ptr = np.arange(self.n + 1, dtype=np.int32)
-        self.labels = (1 + tokens).astype(np.uint32).ravel()
-        tg = np.full((frag_count, frag_len), -1, np.int32)
-        tg[:, :-1] = tokens[:, 1:]
-        self.target = tg.ravel()
-        self.spans = [self.orc.make_causal_spans(frag_count, frag_len, int(w)) for w in self.att_width]
+        b = make_batch(self.orc, vocab, tokens, self.att_width)
+        assert b["label_count"] == self.label_count
+        self.label_ptr, self.labels, self.target, self.spans = b["label_ptr"], b["labels"], b["target"], b["spans"]
         self.rev = [self.orc.transpose_attention(sp, ss) for sp, ss in self.spans]
         self.rope = self.orc.fill_rope_buf(128, self.n)
 

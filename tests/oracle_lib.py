@@ -182,6 +182,37 @@ class Oracle:
         self.lib.orc_make_causal_spans(frag_count, frag_len, window, _ptr(sp), _ptr(spans), C.byref(cnt))
         return sp, spans[:cnt.value].copy()
 
+    # ---- model schedule / batch nodes
+    def model_schedule(self, descr, depth, experts, wide_window):
+        """layer schedule {type, attention type id, slope} and attention widths.  Reference side: parsed from the model string by
+        InitModelDescrImpl; oracle side: orc_model_schedule from the numbers the string stands for (the caller supplies both)."""
+        lt = np.zeros(256, np.int32); la = np.zeros(256, np.int32); ls = np.zeros(256, F32); aw = np.zeros(8, np.int32); ac = C.c_int(0)
+        out = {}
+        if self.use_ref:
+            dims = np.zeros(10, np.int32)
+            n = self.lib.ref_model_descr(descr.encode(), _ptr(dims), _ptr(lt), _ptr(la), _ptr(ls), 256, _ptr(aw), C.byref(ac))
+            out["dims"] = dims
+        else:
+            n = self.lib.orc_model_schedule(depth, experts, wide_window, _ptr(lt), _ptr(la), _ptr(ls), 256, _ptr(aw), C.byref(ac))
+        assert n > 0
+        out.update(layer_type=lt[:n].copy(), layer_att_id=la[:n].copy(), layer_slope=ls[:n].copy(), att_width=aw[:ac.value].copy())
+        return out
+
+    def ref_label_data(self, descr, vocab, tokens, targets, att_type):
+        """InitLabelData of the reference build (noise labels disabled) for equal-length fragments: tokens/targets [frag][len]"""
+        assert self.use_ref
+        tokens = np.ascontiguousarray(tokens, np.int32); targets = np.ascontiguousarray(targets, np.int32)
+        fc, fl = tokens.shape
+        n = fc * fl
+        lc = C.c_int(0); tc = C.c_int(0)
+        lp = np.zeros(n + 1, np.int32); lb = np.zeros(4 * n, np.uint32); tp = np.zeros((n, 2), np.int32)
+        sp = np.zeros(n + 1, np.int32); ss = np.zeros((4 * n, 2), np.int32)
+        got = self.lib.ref_init_label_data(descr.encode(), vocab, fc, fl, _ptr(tokens), _ptr(targets), C.byref(lc), _ptr(lp), _ptr(lb), C.byref(tc),
+                                           _ptr(tp), att_type, _ptr(sp), _ptr(ss))
+        assert got == n
+        return {"label_count": np.array([lc.value], np.int32), "label_ptr": lp, "labels": lb[:lp[n]].copy(), "target_pairs": tp[:tc.value].copy(),
+                "span_ptr": sp, "spans": ss[:sp[n]].copy()}
+
     # ---- converters
     def convert_i8(self, src, mult):
         s = np.ascontiguousarray(src, F32).ravel(); d = np.empty(s.size, np.int8)
