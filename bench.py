@@ -1,10 +1,13 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X backward path.  Prints ONE JSON line.
 
-Default workload ("linear_i8_bwd") = the int8 linear-layer backward of the reference's operator TMatMulBuffers
-(BackpropMulti + Backprop + BackpropDelta): X i8 [16384x1024] with per-row scales, dY bf16 [16384x4096], W i8 [4096x1024] with
-per-output-channel scales; one step = quantise dY per row, transpose W, dX GEMM, re-quantise dY per k-tile + transpose,
-transpose X, delta GEMM with the packed-delta epilogue.  All inputs are resident in HBM before the timed region.
+Default workload ("step_fp8") = the dense GPT forward + backward step the metric's tokens/s is quoted on: e2048 h16 d12 ffn64 w1024
+(24 layers), vocabulary 50304, 32 sequences x 1024 tokens, e4m3 matmuls with bf16 activations.  One step = forward, loss gradient,
+backward through every layer with every packed delta (no optimiser).  The same line carries the second half of the metric, the int8
+backward GEMMs of the linear-layer microbenchmark (`bwd_gemm_int8`: X i8 [16384x1024], dY [16384x4096], W i8 [4096x1024]) and the
+fused bandwidth kernels' GB/s (`bandwidth_kernels`).  All inputs are resident in HBM before a timed region starts.
+Other workloads: "linear_i8_bwd" (that microbenchmark as the step), "att_bwd", "moe_fp8", "gemm_fp8" (the dominant GEMM alone plus the
+copy probe: the command the HBM-traffic counters are collected on).
 
 python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
 """
@@ -46,32 +49,47 @@ def sustained(ab_type):
             "copy_read_plus_write_gbps": round(L.probe_copy_rate(1 << 30), 1)}
 
 
+def omp_threads(n):
+    """thread count of the oracle's OpenMP loops (liboracle.so links libgomp; this is the same runtime instance)"""
+    C.CDLL("libgomp.so.1").omp_set_num_threads(int(n))
+
+
+def host_cores():
+    return min(len(os.sched_getaffinity(0)), 16)
+
+
 def cpu_baseline_linear(len_full, src_dim, grad_dim, sample_rows):
-    """The oracle's restatement of the reference CPU path (MulBackwardWithAccum + SumRankOne, cpu_util.cpp:30-67), OpenMP over
-    independent output rows, on a row subsample; tokens/s = sample_rows / time."""
+    """The oracle's restatement of the reference CPU path (MulBackwardWithAccum + SumRankOne, cpu_util.cpp:30-67) on a row subsample:
+    as written (one thread, a quarter of the sample) and with OpenMP over independent output rows on the host's cores"""
     import numpy as np
     from oracle_lib import Oracle
     orc = Oracle()
-    cores = len(os.sched_getaffinity(0))
-    cores = min(cores, 16)
-    os.environ["OMP_NUM_THREADS"] = str(cores)
+    cores = host_cores()
     r = np.random.default_rng(0)
     w = (r.standard_normal((grad_dim, src_dim)) * 0.02).astype(np.float32)
     x = r.standard_normal((sample_rows, src_dim)).astype(np.float32)
     dy = r.standard_normal((sample_rows, grad_dim)).astype(np.float32)
-    t0 = time.perf_counter()
-    orc.mul_backward_accum(np.zeros((sample_rows, src_dim), np.float32), w, dy)
-    orc.sum_rank_one(x, dy)
-    dt = time.perf_counter() - t0
-    return {"value": sample_rows / dt, "unit": "tokens/s", "cores": cores, "kind": "port",
-            "sample": f"{sample_rows} of {len_full} rows (dX + delta, fp32 scalar loops of the reference CPU path, OpenMP over output rows), {dt:.1f} s"}
+
+    def run(rows):
+        t0 = time.perf_counter()
+        orc.mul_backward_accum(np.zeros((rows, src_dim), np.float32), w, dy[:rows])
+        orc.sum_rank_one(x[:rows], dy[:rows])
+        return time.perf_counter() - t0
+    omp_threads(cores)
+    dt = run(sample_rows)
+    omp_threads(1)
+    rows1 = max(sample_rows // 16, 64)
+    dt1 = run(rows1)
+    omp_threads(cores)
+    return {"value": sample_rows / dt, "unit": "rows/s", "cores": cores, "kind": "port",
+            "sample": f"{sample_rows} of {len_full} rows (dX + delta, fp32 scalar loops of the reference CPU path, OpenMP over output rows), {dt:.1f} s",
+            "single_thread": {"value": rows1 / dt1, "cores": 1, "sample": f"{rows1} rows, {dt1:.1f} s (the reference as written: no threading)"}}
 
 
-def bench_linear_i8(args):
-    import numpy as np
+def linear_i8_setup(delta_splits):
+    """BASELINE config[1]: tensors and operator buffers of the int8 linear-layer backward"""
     import torch
     from tscale2_amd import lib as L
-    L.load()
     len_, src_dim, grad_dim, k_tile = 16384, 1024, 4096, 512
     g = torch.Generator(device="cuda").manual_seed(1)
     x = torch.randn((len_, src_dim), device="cuda", generator=g)
@@ -83,9 +101,8 @@ def bench_linear_i8(args):
     w_scale = w.abs().amax(dim=1) / 127
     w8 = torch.clamp(torch.round(w / w_scale[:, None]), -128, 127).to(torch.int8)
     dy16 = dy.bfloat16()
-    # the 4096 x 1024 delta has too few tiles for 256 CUs: two stored slices of the token axis on 256x128 tiles, packed from their sum
-    splits = args.delta_splits
-    bufs = L.MatMulBuffers(L.I8, len_, src_dim, grad_dim, k_tile=k_tile, splits=splits, share_row_max=True)
+    # the 4096 x 1024 delta has too few tiles for 256 CUs: stored slices of the token axis on 256x128 tiles, packed from their sum
+    bufs = L.MatMulBuffers(L.I8, len_, src_dim, grad_dim, k_tile=k_tile, splits=delta_splits, share_row_max=True)
     dx = torch.empty((len_, src_dim), dtype=torch.float32, device="cuda")
     dyv = dy16.view(torch.int16)
 
@@ -95,25 +112,29 @@ def bench_linear_i8(args):
         bufs.backprop(len_, None, 1.0, None, dx, L.F32)
         # delta = sum_t (s_x[t] dY[t]) X8[t] : the row scale of X is folded into dY before k-tile quantisation
         bufs.backprop_delta(len_, x8, x_scale, dyv, L.BF16)
+    return {"len": len_, "src_dim": src_dim, "grad_dim": grad_dim, "k_tile": k_tile, "splits": delta_splits, "bufs": bufs, "dx": dx, "step": step,
+            "x8": x8, "x_scale": x_scale, "w8": w8, "w_scale": w_scale, "dy16": dy16}
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    ms_per_step = dt / args.steps * 1e3
 
-    # sanity of the result (not timed): against fp64 on a slice
-    ref_dx = (dy16[:256].double() * w_scale.double()[None, :]) @ w8.double()
+def linear_i8_check(c):
+    """sanity of both results (not timed): dX and the dequantised packed delta against fp64 products on slices"""
+    import torch
+    dx, bufs = c["dx"], c["bufs"]
+    ref_dx = (c["dy16"][:256].double() * c["w_scale"].double()[None, :]) @ c["w8"].double()
     err = ((dx[:256].double() - ref_dx).abs().max() / ref_dx.abs().max()).item()
     assert err < 3e-2, f"dX deviates from the fp64 product: {err}"
+    rows = slice(0, 64)
+    ref_dw = (c["dy16"].double()[:, rows] * c["x_scale"].double()[:, None]).t() @ c["x8"].double()
+    got = bufs.delta_fp32()[rows].double()
+    err = ((got - ref_dw).abs().max() / ref_dw.abs().max()).item()
+    assert err < 3e-2, f"the packed delta deviates from the fp64 product: {err}"
 
-    # dominant kernel, timed alone with events on the launch stream: the two int8 MFMA GEMMs (dX and delta), 137.44 GOP each
-    gemm_ops = 2.0 * len_ * src_dim * grad_dim
-    ms_dx = event_time_ms(lambda: bufs.backprop(len_, None, 1.0, None, dx, L.F32), 20)
+
+def linear_i8_gemm_times(c, iters=20):
+    """the two int8 MFMA GEMMs (dX and delta, 137.44 GOP each) timed alone with events on the launch stream"""
+    from tscale2_amd import lib as L
+    bufs, len_, src_dim, grad_dim, k_tile, splits = c["bufs"], c["len"], c["src_dim"], c["grad_dim"], c["k_tile"], c["splits"]
+    ms_dx = event_time_ms(lambda: bufs.backprop(len_, None, 1.0, None, c["dx"], L.F32), iters)
     tsc, gt, st = bufs.t["tileScale"], bufs.t["gradT"], bufs.t["srcT"]
     lib = L.load()
 
@@ -124,24 +145,55 @@ def bench_linear_i8(args):
                         tile_config=3 | 8, m=grad_dim)  # the configuration BackpropDelta launches: 256x128 tile, eight waves
         else:
             lib.gemm_nt(gt, st, bufs.delta, L.I8, L.I8, k_tile_scale=tsc, k_tile=k_tile, epilogue=L.EPI_ROW_TILE_MAXNORM, tile_scale=bufs.delta_tile_scale)
-    ms_dw = event_time_ms(dw, 20)
-    avg_ms = (ms_dx + ms_dw) / 2
-    roof = {"bound": "mfma", "achieved": gemm_ops / (avg_ms * 1e-3) / 1e12, "peak": PEAK_INT8 / 1e12, "unit": "TFLOP/s",
-            "frac": gemm_ops / (avg_ms * 1e-3) / PEAK_INT8,
-            # HBM bytes per GEMM launch (mean of the dX and the delta launch) from rocprofv3 FETCH_SIZE / WRITE_SIZE, calibrated against the
-            # copy probe (factors 2.0 and 1.0): dX 96.8 + 64.0 MiB, delta 192.3 + 32.0 MiB (two fp32 slices); algorithmic 132.1 and 112.0 MiB
-            "traffic": 0.5 * (160.8 + 224.3) * 2 ** 20, "traffic_algorithmic": 0.5 * (132.1 + 112.0) * 2 ** 20,
-            "kernel": "GemmNT<int8> (dX launch %.1f us, delta launch %.1f us; 137.44 GOP per launch)" % (ms_dx * 1e3, ms_dw * 1e3)}
-    out = {"metric": "fwd+bwd tokens/sec on 1 MI355X; bwd GEMM TFLOPS as % of MFMA peak", "value": len_ / (ms_per_step * 1e-3), "unit": "tokens/s",
-           "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
-           "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+    ms_dw = event_time_ms(dw, iters)
+    gemm_ops = 2.0 * len_ * src_dim * grad_dim
+    return {"shape": "dY[16384x4096] x W[4096x1024] and dY^T x X[16384x1024], int8 -> int32", "gop_per_launch": gemm_ops / 1e9,
+            "dx_us": ms_dx * 1e3, "delta_us": ms_dw * 1e3, "dx_tops": gemm_ops / (ms_dx * 1e-3) / 1e12, "delta_tops": gemm_ops / (ms_dw * 1e-3) / 1e12,
+            "tops": 2 * gemm_ops / ((ms_dx + ms_dw) * 1e-3) / 1e12, "frac_of_peak": 2 * gemm_ops / ((ms_dx + ms_dw) * 1e-3) / PEAK_INT8}
+
+
+def profile_traffic(name):
+    """HBM bytes per launch of the dominant kernel as the committed counter summary profiles/<name> states them (a line
+    `traffic_bytes_per_launch: N`, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs); None when there is no such summary"""
+    path = os.path.join(ROOT, "profiles", name)
+    if not os.path.exists(path):
+        return None
+    for line in open(path):
+        if line.startswith("traffic_bytes_per_launch:"):
+            return float(line.split(":")[1])
+    return None
+
+
+def bench_linear_i8(args):
+    import torch
+    from tscale2_amd import lib as L
+    L.load()
+    c = linear_i8_setup(args.delta_splits)
+    step, len_ = c["step"], c["len"]
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    linear_i8_check(c)
+    g = linear_i8_gemm_times(c)
+    gemm_ops = g["gop_per_launch"] * 1e9
+    roof = {"bound": "mfma", "achieved": g["tops"], "peak": PEAK_INT8 / 1e12, "unit": "TFLOP/s", "frac": g["frac_of_peak"],
+            "traffic": profile_traffic("linear_i8_bwd_hbm_traffic.txt"),
+            "kernel": "GemmNT<int8> (dX launch %.1f us, delta launch %.1f us; 137.44 GOP per launch)" % (g["dx_us"], g["delta_us"])}
+    out = {"metric": "int8 linear-layer backward rows/sec on 1 MI355X; bwd GEMM TOPS as % of MFMA peak", "value": len_ / (ms_per_step * 1e-3),
+           "unit": "rows/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
            "config": {"workload": "int8 linear-layer backward (dX + delta): X[16384x1024] i8 per-row scales, dY[16384x4096] bf16, W[4096x1024] i8 "
                                   "per-channel scales, k-tile 512", "tokens_per_step": len_, "gemm_gop_per_step": 2 * gemm_ops / 1e9},
-           "bwd_gemm_tflops": 2 * gemm_ops / ((ms_dx + ms_dw) * 1e-3) / 1e12, "bwd_gemm_pct_of_peak": 100 * roof["frac"],
-           "roofline": roof}
+           "bwd_gemm_tflops": g["tops"], "bwd_gemm_pct_of_peak": 100 * roof["frac"], "bwd_gemm_int8": g, "roofline": roof}
     roof["device_sustained"] = sustained(L.I8)
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline_linear(len_, src_dim, grad_dim, 4096)
+        out["cpu_baseline"] = cpu_baseline_linear(len_, c["src_dim"], c["grad_dim"], 4096)
     return out
 
 
@@ -151,6 +203,129 @@ def _fast_weights(torch, rows, cols, mode_e4m3, gen):
     if mode_e4m3:
         return w.to(torch.float8_e4m3fn).view(torch.uint8).cpu().numpy(), 0.02
     return torch.clamp(torch.round(w), -128, 127).to(torch.int8).cpu().numpy(), 0.02
+
+
+def bandwidth_kernels(iters=10):
+    """The fused bandwidth-bound kernels at the shapes of the dense fp8 step (32768 tokens, dim 2048, ffn 8192), of the int8
+    linear-layer microbenchmark (16384 x 4096) and of the MoE layer (65536 tokens, top-2 of 64, dim 1024): algorithmic bytes (live
+    elements x dtype size of every operand), event time, GB/s and the fraction of the 8 TB/s HBM peak.  Working sets are 0.2-2 GB,
+    far beyond the caches."""
+    import torch
+    from tscale2_amd import lib as L
+    dev = "cuda"
+    R, D, F = 32768, 2048, 8192
+    Q = D
+    f32, bf16, u8, i8 = torch.float32, torch.bfloat16, torch.uint8, torch.int8
+    res = []
+
+    def rnd(rows, cols, dt):
+        if dt in (u8,):
+            return torch.randint(0, 120, (rows, cols), dtype=u8, device=dev)   # positive finite e4m3 codes
+        if dt == i8:
+            return torch.randint(-127, 128, (rows, cols), dtype=i8, device=dev)
+        return torch.randn((rows, cols), device=dev, dtype=f32).to(dt)
+
+    def add(name, nbytes, fn):
+        fn()
+        torch.cuda.synchronize()
+        ms = event_time_ms(fn, iters)
+        res.append({"kernel": name, "mbytes": round(nbytes / 1e6, 1), "us": round(ms * 1e3, 1), "gbps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                    "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / PEAK_HBM, 3)})
+
+    one = torch.ones(4, device=dev)
+    # ---- residual state kernels [R][D]
+    state = rnd(R, D, f32); norm8 = rnd(R, D, u8); sscale = torch.rand((D // 128, R), device=dev) + 0.5
+    add("LayerNormalizeStateVecs f32->e4m3 [32768x2048]", R * D * 5 + R * D // 128 * 4,
+        lambda: L.call("ts2_layer_normalize_state_vecs", state, L.F32, R, R, 1 / 24, norm8, L.E4M3, sscale))
+    dnorm = rnd(R, D, f32); sgrad = rnd(R, D, f32); sfast = torch.empty((R, D), dtype=u8, device=dev); mx = torch.zeros(4, device=dev)
+    add("BackpropLayerNormalize e4m3 [32768x2048]", R * D * 14 + R * D // 128 * 4,
+        lambda: L.call("ts2_backprop_layer_normalize", norm8, L.E4M3, sscale, dnorm, None, one, one, sgrad, sfast, L.E4M3, mx, R))
+    mx.fill_(1.0)
+    add("ScaleGrad f32->e4m3 [32768x2048]", R * D * 5, lambda: L.call("ts2_scale_grad", mx, None, sgrad, sfast, L.E4M3, R, one[1:], one[2:]))
+    del state, dnorm, sgrad, sfast, norm8
+    # ---- FFN gate kernels [R][F]
+    gate = rnd(R, F, bf16); vals = rnd(R, F, bf16); rg = torch.empty((R, F), dtype=u8, device=dev)
+    add("MatrixLoLU bf16,bf16->e4m3 [32768x8192]", R * F * 5, lambda: L.call("ts2_matrix_lolu", R, R, gate, vals, 1.0, rg, L.E4M3))
+    grad = rnd(R, F, bf16); vts = torch.rand((F // 128, R), device=dev) + 0.5
+    gg = torch.empty((R, F), dtype=u8, device=dev); gv = torch.empty_like(gg); ggT = torch.empty((F, R), dtype=u8, device=dev); gvT = torch.empty_like(ggT)
+    add("BackpropRowTileNormalizeLoLU (+ transposed copies) bf16->e4m3 [32768x8192]", R * F * 10 + R * F // 128 * 4,
+        lambda: L.call("ts2_backprop_row_tile_normalize_lolu_t", R, R, gate, vals, 1 / 24, vts, grad, gg, gv, ggT, gvT))
+    add("TransposeQuant e4m3 byte transpose [32768x8192]", R * F * 2,
+        lambda: L.call("ts2_transpose_quant", R, R, gg, L.E4M3, None, None, 0, None, ggT, L.E4M3, None))
+    del gate, vals, rg, grad, gg, gv, ggT, gvT, vts
+    # ---- attention epilogue kernels [R][Q]
+    gate = rnd(R, Q, bf16); vals = rnd(R, Q, bf16); grad = rnd(R, Q, bf16)
+    dgate = torch.empty((R, Q), dtype=u8, device=dev); dval = torch.empty((R, Q), dtype=bf16, device=dev); dsc = torch.empty((Q // 128, R), device=dev)
+    add("BackpropLoLUdScale bf16 -> e4m3 + bf16 [32768x2048]", R * Q * 9 + R * Q // 128 * 4,
+        lambda: L.call("ts2_backprop_lolu_dscale", R, R, gate, vals, 1.0, grad, L.BF16, dgate, L.E4M3, dval, L.BF16, dsc))
+    rope = torch.randn((R, 128), device=dev); qsc = torch.rand((Q // 128, R), device=dev) + 0.5
+    add("BackpropRowTileNormalizeRope bf16->e4m3 (norm backward + inverse RoPE) [32768x2048]", R * Q * 5 + R * 128 * 4 + R * Q // 128 * 4,
+        lambda: L.call("ts2_backprop_row_tile_normalize_rope", R, R, grad, L.BF16, 1.0, vals, qsc, rope, dgate, L.E4M3))
+    raw = rnd(R, Q, f32)
+    add("RowTileNormalizeRope f32->bf16 [32768x2048]", R * Q * 6 + R * 128 * 4 + R * Q // 128 * 4,
+        lambda: L.call("ts2_row_tile_normalize_rope", R, R, raw, L.F32, 1.0, 1, 1.0, rope, dval, qsc))
+    del gate, vals, grad, dgate, dval, raw
+    # ---- int8 linear-layer preparation [16384][4096] bf16
+    R1, G1, KT = 16384, 4096, 512
+    dy = rnd(R1, G1, bf16); d8 = torch.empty((R1, G1), dtype=i8, device=dev); rs = torch.empty(R1, device=dev); ram = torch.empty(R1, device=dev)
+    add("NormalizeVecsRowMax bf16->i8 [16384x4096]", R1 * G1 * 3 + R1 * 8,
+        lambda: L.call("ts2_normalize_vecs_row_max2", R1, R1, dy, L.BF16, None, d8, rs, ram))
+    tmax = torch.zeros(R1 // KT, device=dev); tsc = torch.empty(R1 // KT, device=dev); d8T = torch.empty((G1, R1), dtype=i8, device=dev)
+    add("TileAbsMax bf16 [16384x4096]", R1 * G1 * 2, lambda: L.call("ts2_tile_absmax", R1, dy, L.BF16, None, KT, tmax, 1))
+    add("TransposeQuant bf16->i8 per k-tile [16384x4096]", R1 * G1 * 3,
+        lambda: L.call("ts2_transpose_quant", R1, R1, dy, L.BF16, None, tmax, KT, None, d8T, L.I8, tsc))
+    del dy, d8, d8T
+    # ---- MoE gradient movement: 65536 tokens, top-2 of 64 experts, dim 1024
+    N4, E4, K4, D4 = 65536, 64, 2, 1024
+    len_moe = N4 * K4 + 128 * E4
+    sel = torch.randn((N4, E4), device=dev)
+    tot = N4 * K4
+    t = {"ids": torch.zeros(tot, dtype=torch.int32, device=dev), "w": torch.zeros(tot, device=dev), "off": torch.zeros(tot, dtype=torch.int32, device=dev),
+         "eo": torch.zeros(E4 + 2, dtype=torch.int32, device=dev), "tile": torch.zeros(len_moe // 128, dtype=torch.int32, device=dev),
+         "sid": torch.zeros(len_moe, dtype=torch.int32, device=dev), "sw": torch.zeros(len_moe, device=dev),
+         "bc": torch.zeros(((tot + 255) // 256) * E4, dtype=torch.int32, device=dev)}
+
+    class Tables(C.Structure):
+        _fields_ = [(n, C.c_void_p) for n in ("ids", "w", "off", "eo", "tile", "sid", "sw", "bc")]
+    tb = Tables(*[t[n].data_ptr() for n in ("ids", "w", "off", "eo", "tile", "sid", "sw", "bc")])
+    L.call("ts2_moe_route", N4, len_moe, E4, K4, sel, L.F32, C.byref(tb))
+    src8 = rnd(N4, D4, u8); grp = torch.empty((len_moe, D4), dtype=u8, device=dev)
+    add("MoeGroupSamples 8-bit gather into expert order [131072 of 139264 rows x 1024]", tot * D4 * 2 + len_moe * 4,
+        lambda: L.call("ts2_moe_group_samples", len_moe, 1, src8, t["sid"], grp))
+    full = rnd(len_moe, D4, f32); comb = torch.empty((N4, D4), device=dev)
+    add("CombineExperts f32 2-way gather-sum [65536x1024]", tot * D4 * 4 + N4 * D4 * 4 + tot * 8,
+        lambda: L.call("ts2_combine_experts", N4, K4, full, L.F32, C.byref(tb), 1.0, None, comb, 0))
+    return res
+
+
+def fp8_backward_gemms(n, dim, ffn, iters=10):
+    """the e4m3 backward GEMM shapes of the dense step, each timed alone with events: dX of the FFN contract / expand matrices,
+    the FFN delta (packed-delta epilogue) and the attention-width dX"""
+    import torch
+    from tscale2_amd import lib as L
+    lib = L.load()
+    out = []
+
+    def run(name, m, nn, k, packed=False):
+        a = torch.randint(0, 120, (m, k), dtype=torch.uint8, device="cuda"); b = torch.randint(0, 120, (nn, k), dtype=torch.uint8, device="cuda")
+        if packed:
+            c = torch.empty((m, nn), dtype=torch.int8, device="cuda"); ts = torch.empty((nn // 128, m), device="cuda")
+            fn = lambda: lib.gemm_nt(a, b, c, L.E4M3, L.I8, epilogue=L.EPI_ROW_TILE_MAXNORM, tile_scale=ts)  # noqa: E731
+        else:
+            c = torch.empty((m, nn), dtype=torch.float32, device="cuda")
+            fn = lambda: lib.gemm_nt(a, b, c, L.E4M3, L.F32)  # noqa: E731
+        fn(); torch.cuda.synchronize()
+        ms = event_time_ms(fn, iters)
+        ops = 2.0 * m * nn * k
+        out.append({"product": name, "m": m, "n": nn, "k": k, "us": round(ms * 1e3, 1), "tflops": round(ops / (ms * 1e-3) / 1e12, 1),
+                    "frac_of_peak": round(ops / (ms * 1e-3) / PEAK_FP8, 3)})
+        return ms, ops
+    first = run("dX: dY[tokens x ffn] x W^T (FFN expand / gate), fp32 result", n, dim, ffn)
+    run("dX: dY[tokens x dim] x W^T (FFN contract), fp32 result", n, ffn, dim)
+    run("dX: dY[tokens x dim] x W^T (attention Q/K/V/gate/combiner), fp32 result", n, dim, dim)
+    run("delta: dY^T[ffn x tokens] x X^T (FFN expand / gate), packed i8 result", ffn, dim, n, packed=True)
+    run("delta: dY^T[dim x tokens] x X^T (FFN contract), packed i8 result", dim, ffn, n, packed=True)
+    return out, first
 
 
 def bench_step_fp8(args):
@@ -210,46 +385,111 @@ def bench_step_fp8(args):
             pairs = sum(min(i, w) for i in range(frag_len)) * frags
             att += 7 * 2.0 * pairs * 128 * heads
     flop = 6.0 * params * n + att
-    # dominant kernel: the e4m3 GEMM, timed alone on the biggest backward shape of the model (dX of the FFN expand: M=tokens, K=ffn, N=dim)
-    a = torch.randint(0, 120, (n, ffn), dtype=torch.uint8, device="cuda"); b = torch.randint(0, 120, (dim, ffn), dtype=torch.uint8, device="cuda")
-    c = torch.empty((n, dim), dtype=torch.float32, device="cuda")
-    lib = L.load()
-    ms_g = event_time_ms(lambda: lib.gemm_nt(a, b, c, L.E4M3, L.F32), 10)
-    gops = 2.0 * n * ffn * dim
+    # dominant kernel: the e4m3 GEMM, timed alone with events on the launch stream at the model's backward shapes; the roofline line is
+    # the biggest of them (dX of the FFN expand / gate matrices: M = tokens, K = ffn, N = dim)
+    gemms, (ms_g, gops) = fp8_backward_gemms(n, dim, ffn)
     roof = {"bound": "mfma", "achieved": gops / (ms_g * 1e-3) / 1e12, "peak": PEAK_FP8 / 1e12, "unit": "TFLOP/s",
-            "frac": gops / (ms_g * 1e-3) / PEAK_FP8, "traffic": None,
-            "kernel": "GemmNT<e4m3> %dx%dx%d (%.1f us per launch)" % (n, dim, ffn, ms_g * 1e3)}
+            "frac": gops / (ms_g * 1e-3) / PEAK_FP8, "traffic": None if args.small else profile_traffic("gemm_fp8_32768x2048x8192_hbm_traffic.txt"),
+            "kernel": "GemmNTRing<e4m3> %dx%dx%d (%.1f us per launch, %.2f GOP)" % (n, dim, ffn, ms_g * 1e3, gops / 1e9)}
     out = {"metric": "fwd+bwd tokens/sec on 1 MI355X; bwd GEMM TFLOPS as % of MFMA peak", "value": n / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1,
            "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": "fp8_e4m3", "data": "synthetic",
            "config": {"workload": "dense GPT fwd+bwd step, e%dh%dd%dffn%dw%d (%d layers), vocab %d, %d x %d tokens, e4m3 matmuls, bf16 activations"
                                   % (dim, heads, depth, ffn // 128, wide, len(lt), vocab, frags, frag_len),
                       "tokens_per_step": n, "matmul_params": params, "useful_tflop_per_step": flop / 1e12},
-           "step_tflops": flop / (ms * 1e-3) / 1e12, "bwd_gemm_pct_of_peak": 100 * roof["frac"], "loss": loss, "roofline": roof}
+           "step_tflops": flop / (ms * 1e-3) / 1e12, "bwd_gemm_pct_of_peak": 100 * roof["frac"], "loss": loss, "roofline": roof,
+           "bwd_gemm_fp8": gemms}
+    m.close()
+    del m
+    torch.cuda.empty_cache()
+    # the second half of the metric: the int8 backward GEMMs of the linear-layer microbenchmark, in the same run
+    c1 = linear_i8_setup(args.delta_splits)
+    c1["step"]()
+    torch.cuda.synchronize()
+    linear_i8_check(c1)
+    out["bwd_gemm_int8"] = linear_i8_gemm_times(c1)
+    del c1
+    torch.cuda.empty_cache()
+    out["bandwidth_kernels"] = bandwidth_kernels()
     roof["device_sustained"] = sustained(L.E4M3)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_step(orc, dim, heads, ffn, lt, la, ls, aw, vocab)
-    m.close()
     return out
 
 
 def cpu_baseline_step(orc, dim, heads, ffn, lt, la, ls, aw, vocab):
     """the oracle's full step (the reference's CPU ComputeBackprop restated) on a bounded sample of the same model: one layer pair
-    (attention + FFN) of the real width on 256 tokens, extrapolated per token and per layer"""
-    import numpy as np
+    (attention + FFN) of the real width on 256 tokens (16 for the single-thread figure), extrapolated per token and per layer"""
     from model_harness import Harness
-    cores = min(len(os.sched_getaffinity(0)), 16)
-    os.environ["OMP_NUM_THREADS"] = str(cores)
-    h = Harness(1, dim=dim, heads=heads, ffn_tiles=ffn // 128, depth=1, vocab=256, frag_count=2, frag_len=128, wide_window=128, seed=1)
-    t0 = time.perf_counter()
-    h.oracle_step()
-    dt = time.perf_counter() - t0
+    cores = host_cores()
     layers_full = len(lt)
+
+    def run(frag_len):
+        h = Harness(1, dim=dim, heads=heads, ffn_tiles=ffn // 128, depth=1, vocab=256, frag_count=2, frag_len=frag_len, wide_window=frag_len, seed=1)
+        t0 = time.perf_counter()
+        h.oracle_step()
+        return h.n, time.perf_counter() - t0
+    omp_threads(cores)
+    n, dt = run(128)
+    omp_threads(1)
+    n1, dt1 = run(8)
+    omp_threads(cores)
     # depth=1 schedule = 1 attention + 1 ffn layer; the full model has layers_full/2 such pairs; the head (vocab) is left out of the sample
-    tok_s = h.n / (dt * layers_full / 2)
-    return {"value": tok_s, "unit": "tokens/s", "cores": cores, "kind": "port",
+    return {"value": n / (dt * layers_full / 2), "unit": "tokens/s", "cores": cores, "kind": "port",
             "sample": "one attention+FFN layer pair of the full width on %d tokens (%.1f s), scaled by %d layer pairs; final layer excluded"
-                      % (h.n, dt, layers_full // 2)}
+                      % (n, dt, layers_full // 2),
+            "single_thread": {"value": n1 / (dt1 * layers_full / 2), "cores": 1,
+                              "sample": "the same pair on %d tokens (%.1f s): the reference as written, no threading" % (n1, dt1)}}
+
+
+def cpu_baseline_att(heads_full, seqs_full, seq_len):
+    """the oracle's attention backward (dScale, GradQ, GradK of layer_att_reference.h restated) on one head of one sequence"""
+    import numpy as np
+    from oracle_lib import Oracle
+    orc = Oracle()
+    cores = host_cores()
+    r = np.random.default_rng(5)
+
+    def run(s_len):
+        q, k, v, do = [r.standard_normal((s_len, 128)).astype(np.float32) for _ in range(4)]
+        sp, spans = orc.make_causal_spans(1, s_len, s_len)
+        t0 = time.perf_counter()
+        orc.attention(1, 128, 128, 0.0, sp, spans, q, k, v, do)
+        return time.perf_counter() - t0
+    omp_threads(cores)
+    dt = run(seq_len)
+    omp_threads(1)
+    dt1 = run(seq_len // 4)
+    omp_threads(cores)
+    scale = heads_full * seqs_full
+    return {"value": seq_len / (dt * heads_full), "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": "forward + backward of 1 head x 1 sequence of %d tokens (%.1f s), scaled by %d heads (x %d sequences = %d head-sequences in the "
+                      "workload)" % (seq_len, dt, heads_full, seqs_full, scale),
+            "single_thread": {"value": (seq_len // 4) / (dt1 * heads_full * 4), "cores": 1,
+                              "sample": "1 head x %d tokens (%.1f s), scaled quadratically to %d tokens per sequence" % (seq_len // 4, dt1, seq_len)}}
+
+
+def cpu_baseline_moe(dim, xp, experts, selected, tokens):
+    """the oracle's MoE layer step (the reference CPU path evaluates every expert densely, layer_moe.cu:458-537) on a token sample"""
+    from model_harness import Harness
+    cores = host_cores()
+
+    def run(n):
+        h = Harness(1, dim=dim, heads=1, ffn_tiles=1, depth=1, vocab=128, frag_count=1, frag_len=n, wide_window=1, experts=experts, selected=selected,
+                    xp=xp, seed=1)
+        t0 = time.perf_counter()
+        h.oracle_step()
+        return time.perf_counter() - t0
+    omp_threads(cores)
+    dt = run(tokens)
+    omp_threads(1)
+    n1 = max(tokens // 32, 8)
+    dt1 = run(n1)
+    omp_threads(cores)
+    return {"value": tokens / dt, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": "one attention (1 head, window 1) + MoE layer pair, %d experts of width %d evaluated densely, on %d tokens (%.1f s)"
+                      % (experts, xp, tokens, dt),
+            "single_thread": {"value": n1 / dt1, "cores": 1, "sample": "%d tokens (%.1f s)" % (n1, dt1)}}
 
 
 def bench_att_bwd(args):
@@ -284,10 +524,13 @@ def bench_att_bwd(args):
     flop5 = 5 * 2.0 * pairs * 128
     roof = {"bound": "mfma", "achieved": flop5 / (ms * 1e-3) / 1e12, "peak": PEAK_BF16 / 1e12, "unit": "TFLOP/s", "frac": flop5 / (ms * 1e-3) / PEAK_BF16,
             "traffic": None, "kernel": "AttGradQ + AttGradKV, 5-product causal count (7 products executed)"}
-    return {"metric": "fwd+bwd tokens/sec on 1 MI355X; bwd GEMM TFLOPS as % of MFMA peak", "value": n / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1,
-            "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-            "dtype": "bf16", "data": "synthetic", "config": {"workload": "causal attention backward, 16 x 2048 tokens, 16 heads x 128, bf16"},
-            "roofline": roof}
+    out = {"metric": "attention backward tokens/sec on 1 MI355X; TFLOPS as % of MFMA peak", "value": n / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1,
+           "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "bf16", "data": "synthetic", "config": {"workload": "causal attention backward, 16 x 2048 tokens, 16 heads x 128, bf16"},
+           "roofline": roof}
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline_att(H, B, S)
+    return out
 
 
 def bench_moe_fp8(args):
@@ -357,10 +600,38 @@ def bench_moe_fp8(args):
                       "rows_per_expert_min_mean_max": [int(per_expert.min()), float(per_expert.mean()), int(per_expert.max())]},
            "layer_tflops": flop / (ms * 1e-3) / 1e12, "roofline": roof}
     m.close()
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline_moe(dim, xp, experts, selected, 256)
     return out
 
 
-WORKLOADS = {"linear_i8_bwd": bench_linear_i8, "step_fp8": bench_step_fp8, "att_bwd": bench_att_bwd, "moe_fp8": bench_moe_fp8}
+def bench_gemm_fp8(args):
+    """the dominant kernel of the dense fp8 step alone (e4m3 32768 x 2048 x 8192, fp32 result) followed by the copy probe of 1 GiB: the
+    command the HBM-traffic counters (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) are collected on; the probe calibrates the counters"""
+    import torch
+    from tscale2_amd import lib as L
+    lib = L.load()
+    n, dim, ffn = 32768, 2048, 8192
+    a = torch.randint(0, 120, (n, ffn), dtype=torch.uint8, device="cuda"); b = torch.randint(0, 120, (dim, ffn), dtype=torch.uint8, device="cuda")
+    c = torch.empty((n, dim), dtype=torch.float32, device="cuda")
+    fn = lambda: lib.gemm_nt(a, b, c, L.E4M3, L.F32)  # noqa: E731
+    for _ in range(args.warmup):
+        fn()
+    torch.cuda.synchronize()
+    ms = event_time_ms(fn, args.steps)
+    gops = 2.0 * n * dim * ffn
+    copy = L.probe_copy_rate(1 << 30)
+    roof = {"bound": "mfma", "achieved": gops / (ms * 1e-3) / 1e12, "peak": PEAK_FP8 / 1e12, "unit": "TFLOP/s", "frac": gops / (ms * 1e-3) / PEAK_FP8,
+            "traffic": profile_traffic("gemm_fp8_32768x2048x8192_hbm_traffic.txt"), "traffic_algorithmic": n * ffn + dim * ffn + n * dim * 4,
+            "kernel": "GemmNTRing<e4m3> %dx%dx%d" % (n, dim, ffn)}
+    return {"metric": "e4m3 GEMM launches/sec on 1 MI355X; TFLOPS as % of MFMA peak", "value": 1e3 / ms, "unit": "launches/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "fp8_e4m3", "data": "synthetic", "config": {"workload": "e4m3 GEMM 32768 x 2048 x 8192 (dX of the FFN expand matrix), fp32 result"},
+            "copy_probe_gbps": copy, "roofline": roof}
+
+
+WORKLOADS = {"linear_i8_bwd": bench_linear_i8, "step_fp8": bench_step_fp8, "att_bwd": bench_att_bwd, "moe_fp8": bench_moe_fp8,
+             "gemm_fp8": bench_gemm_fp8}
 
 
 def main():
@@ -368,13 +639,13 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="linear_i8_bwd", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="step_fp8", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--delta-splits", type=int, default=2, help="linear_i8_bwd: slices of the token axis in the delta product (1 = single pass)")
     ap.add_argument("--small", action="store_true", help="step_fp8 / moe_fp8: a reduced model for quick checks (not a valid benchmark figure)")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build runs on one GPU only (the path has no multi-GPU leg); use --gpus 1", file=sys.stderr)
+        print("bench.py: this build measures one GPU only (no collective, sharding or rank code is part of it): run with --gpus 1", file=sys.stderr)
         sys.exit(2)
     out = WORKLOADS[args.workload](args)
     print(json.dumps(out))

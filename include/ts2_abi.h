@@ -466,7 +466,7 @@ int ts2_model_set_batch(ts2_model *m, int32_t len, const int32_t *labelPtr, cons
     const int32_t *const *spanStart, const int32_t *const *spanFinish, const float *ropeBuf, void *stream);
 /* The checks ts2_model_set_batch makes before it copies anything, as a host-only function (no device access): label CSR monotone from 0
  * and within labelCap, label ids (low 31 bits; bit 31 is the sign of the embedding term, src/gpt/compute/cpu_transformer.cpp:76-100) below
- * labelCount, -1 <= target < vocab, and for every attention type and row 0 <= start <= len, finish < len, finish >= start - 1.  The
+ * labelCount, -1 <= target < vocab, and for every attention type and row 0 <= start <= len and -1 <= finish < len (finish < start = empty).  The
  * reference trusts its own node builder (InitLabelData, src/gpt/att/sliding_window.cpp:269-306); a caller-supplied batch that breaks one
  * of these would be an out-of-bounds access on the device, so it is refused with TS2_ERR_SHAPE / TS2_ERR_NULL instead.
  * ts2_model_set_batch, ts2_model_set_matrix and ts2_model_set_bias copy with blocking copies on the null stream; set_batch waits for

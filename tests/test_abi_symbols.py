@@ -81,7 +81,9 @@ def test_batch_validation_rejects_out_of_range_indices():
     assert run(label_cap=5) == -1                                # more labels than the model holds
     assert run(start=[0, 0, 0, 0, 0, -1]) == -1                  # span starts before row 0
     assert run(finish=[-1, 0, 1, 2, 3, 6]) == -1                 # span ends beyond the batch
-    assert run(start=[0, 0, 0, 0, 0, 5], finish=[-1, 0, 1, 2, 3, 2]) == -1  # finish < start - 1
+    assert run(start=[0, 0, 0, 0, 0, 5], finish=[-1, 0, 1, 2, 3, 2]) == 0   # finish < start: an empty span
+    assert run(finish=[-2, 0, 1, 2, 3, 4]) == -1                 # finish below -1
+    assert run(start=[0, 0, 0, 0, 0, 7]) == -1                   # start beyond the batch
 
 
 def test_every_entry_point_cites_the_interface_it_replaces():

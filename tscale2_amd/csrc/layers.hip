@@ -1021,7 +1021,7 @@ static int Ts2ValidateBatch(int len, int labelCap, int labelCount, int vocab, in
         }
         for (int t = 0; t < len; ++t) {
             const int st = spanStart[a][t], fi = spanFinish[a][t];
-            if (st < 0 || st > len || fi >= len || fi < st - 1) {
+            if (st < 0 || st > len || fi >= len || fi < -1) {
                 return TS2_ERR_SHAPE;
             }
         }
@@ -1069,7 +1069,7 @@ extern "C" int ts2_model_set_bias(ts2_model *M, const float *biasHost)
 }
 
 // Host-side check of a batch (no device access): label CSR monotone and within capacity, label ids (low 31 bits; the top bit is the
-// sign of the embedding term) below labelCount, targets in [-1, vocab), every span inside [0, len) with finish >= start - 1.
+// sign of the embedding term) below labelCount, targets in [-1, vocab), every span with 0 <= start <= len and -1 <= finish < len (finish < start = empty).
 extern "C" int ts2_validate_batch(int32_t len, int32_t labelCap, int32_t labelCount, int32_t vocab, int32_t attTypeCount, const int32_t *labelPtr,
     const uint32_t *labels, const int32_t *targetPerRow, const int32_t *const *spanStart, const int32_t *const *spanFinish)
 {
