@@ -161,6 +161,13 @@ class Harness:
         return m
 
 
+def scale_fit(got, ref):
+    """least-squares scale of got on ref (1 = unbiased) and their correlation"""
+    g = got.astype(np.float64).ravel(); r = ref.astype(np.float64).ravel()
+    rr = (r * r).sum() + 1e-300
+    return float((g * r).sum() / rr), float((g * r).sum() / (np.sqrt((g * g).sum() * rr) + 1e-300))
+
+
 def rel_err(got, ref):
     d = got.astype(np.float64) - ref
     den = np.sqrt((ref.astype(np.float64) ** 2).mean()) + 1e-30

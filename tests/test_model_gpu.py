@@ -6,11 +6,20 @@ import pytest
 
 pytestmark = pytest.mark.gpu
 torch = pytest.importorskip("torch")
-from model_harness import E4M3, I8, Harness, rel_err  # noqa: E402
+from model_harness import E4M3, I8, Harness, rel_err, scale_fit  # noqa: E402
 
 
-def check_model(h, tol_state, tol_grad, tol_delta):
+def check_model(h, tol_state, tol_grad, tol_delta, tol_fit=5e-3, min_corr=0.99):
+    """per tensor: rms error relative to the tensor's rms (the 8-bit storage noise of states and gradients), and - what makes that noise
+    harmless - no bias: the least-squares scale of the device tensor on the oracle's within 1 +- tol_fit and a correlation of at least
+    min_corr.  A wrong constant factor, a dropped term or a transposed operand moves the fit or the correlation, not just the rms."""
     failures = []
+    fits = []
+
+    def expect_fit(got, ref, what):
+        fit, corr = scale_fit(got, ref)
+        fits.append((what, fit, corr))
+        expect(abs(fit - 1) <= tol_fit and corr >= min_corr, ('fit', what, round(fit, 5), round(corr, 5)))
 
     def expect(cond, what):
         if not cond:
@@ -28,6 +37,7 @@ def check_model(h, tol_state, tol_grad, tol_delta):
         rms, mx = rel_err(g0, h.ref_grad0)
         print("embedding-level state gradient rel err rms/max", rms, mx)
         expect(rms <= tol_grad, 'stateGrad')
+        expect_fit(g0, h.ref_grad0, 'stateGrad')
         loss = m.loss_sum() / (h.target >= 0).sum()
         print("loss", loss, h.ref_loss)
         expect(abs(loss - h.ref_loss) <= 2e-3 * abs(h.ref_loss), 'loss')
@@ -39,15 +49,21 @@ def check_model(h, tol_state, tol_grad, tol_delta):
                 worst = max(worst, rms)
                 print(f"layer {d} type {h.lt[d]} matrix {i}: delta rel err rms/max {rms:.4f} {mx:.4f}")
                 expect(rms <= tol_delta, ('delta', d, i))
+                expect_fit(got, h.ref_delta[d][i], ('delta', d, i))
         got = m.get_delta(-2, 0, h.vocab, h.dim)
         rms, mx = rel_err(got, h.ref_delta_final)
         print("final layer delta rel err", rms, mx)
         expect(rms <= tol_delta, 'final delta')
+        expect_fit(got, h.ref_delta_final, 'final delta')
         got = m.get_delta(-1, 0, h.label_count, h.dim)
         rms, mx = rel_err(got, h.ref_delta_embed)
         print("embedding delta rel err", rms, mx)
         expect(rms <= tol_grad, 'embed delta')
+        expect_fit(got, h.ref_delta_embed, 'embed delta')
         print("worst layer delta rms rel err", worst)
+        print("scale fits min/max", min(f[1] for f in fits), max(f[1] for f in fits), "min correlation", min(f[2] for f in fits))
+        for f in fits:
+            print("   fit", f)
         assert not failures, failures
     finally:
         m.close()
@@ -151,8 +167,10 @@ def test_moe_layer_fp8_step():
     h = Harness(E4M3, dim=256, heads=2, ffn_tiles=2, depth=1, vocab=256, frag_count=4, frag_len=96, wide_window=64, experts=8, selected=2, xp=128,
                 seed=6, std=0.05)
     # besides the fp8 storage noise, a few tokens whose 2nd/3rd select logits are nearly tied pick another expert than the fp32 CPU path
-    # (the logits come from 8-bit states): large but isolated row errors, visible in the max and not in the rms
-    check_model(h, tol_state=8e-2, tol_grad=1.5e-1, tol_delta=2e-1)
+    # (the logits come from 8-bit states): large but isolated row errors, visible in the max and not in the rms; a token that goes to
+    # another expert contributes to the deltas of both experts something the oracle's deltas do not hold, which pulls the least-squares
+    # scale below 1 (measured 0.990 - 0.998 with 384 tokens)
+    check_model(h, tol_state=8e-2, tol_grad=1.5e-1, tol_delta=2e-1, tol_fit=1.5e-2)
 
 
 def test_moe_routing_tables_match_cpu_moe():
