@@ -481,7 +481,14 @@ int ts2_layer_backward(ts2_model *m, int32_t layer, void *stream);
 /* dequantised delta of a matrix into hostOut [rows][cols] (synchronises the device) */
 int ts2_model_get_delta(ts2_model *m, int32_t layer, int32_t matrixId, float *hostOut, int32_t rows, int32_t cols);
 /* device view of an internal array: "state", "stateGrad", "stateGradFast", "dNormState", "prediction", "normState"[i], "stateScale"[i],
- * "expertOffset" (TS2_I32 [1][experts+2], MoE models: the routing of the last MoE layer that ran) */
+ * "expertOffset" (TS2_I32 [1][experts+2], MoE models: the routing of the last MoE layer that ran), "gradMaxNorm" (fp32 [1][depth+2]: the
+ * running maxima of |stateGrad|; ts2_layer_backward derives its gradient multiplier from element 0, which a caller that sets stateGrad
+ * itself must set to its abs-max), "finalGrad" (bf16 [lenRound][vocab]: the soft-max gradient of the last ts2_model_backprop).
+ * For tests that compare a layer's interior: "act.a0".."act.a3", "act.scale0", "act.scale1", "act.rg", "act.val", "act.swl" with index =
+ * layer: what that layer keeps from its forward pass (FFN: wide, gate, wide's tile scales, rg; attention: q, gate, k, v, q's and v's
+ * scales, the attention output - overwritten with dQ by the layer's backward -, vlg, the soft-max statistics); "scratch.g0".."scratch.g3",
+ * "scratch.f0".."scratch.f3", "scratch.dscale" with index = number of columns: the gradient scratch of the layer backward that ran last
+ * (bf16: drg / dvlg, dVal, dK, dV; fast-gradient type: dwide / dq, dgate, dk, dv). */
 int ts2_model_array(ts2_model *m, const char *name, int32_t index, ts2_mat *out, int32_t *type);
 /* host copy of the same arrays, rows packed ([y][x] elements); synchronises the device */
 int ts2_model_read(ts2_model *m, const char *name, int32_t index, void *hostOut, int64_t hostBytes);

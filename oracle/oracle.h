@@ -70,6 +70,7 @@ int8_t orc_cvt_i8(float x);
 void orc_convert_i8(int8_t *dst, const float *src, int n, float mult);
 uint8_t orc_cvt_e4m3(float x);
 uint8_t orc_cvt_e4m3_rne(float x);
+void orc_round_e4m3_rne(float *dst, const float *src, long n);
 void orc_convert_e4m3(uint8_t *dst, const float *src, int n, float mult);
 float orc_e4m3_to_float(int code);
 float orc_quantize_matrix_i8(const float *w, int8_t *fast, int ySize, int xSize);

@@ -145,6 +145,17 @@ uint8_t orc_cvt_e4m3_rne(float x)
     return sign | (uint8_t)((be << 3) | m);
 }
 
+/* the same rule over an array, result decoded back to fp32 (the value the device stores): used by the same-contract model of the tests */
+void orc_round_e4m3_rne(float *dst, const float *src, long n)
+{
+#pragma omp parallel for schedule(static)
+    for (long i = 0; i < n; ++i) {
+        uint8_t c = orc_cvt_e4m3_rne(src[i]);
+        float v = orc_e4m3_to_float(c & 0x7f);
+        dst[i] = (c & 0x80) ? -v : v;
+    }
+}
+
 /* src/gpt/matrix/quant.h:42-62 TQuantizedMatrix::Convert (i8): scale = rms of the matrix; fast = sat_i8(rne(w / (rms/32))).
  * Returns the matrix scale (rms).  The reference sums squares in 8 AVX lanes; the summation here is in double. */
 float orc_quantize_matrix_i8(const float *w, int8_t *fast, int ySize, int xSize)

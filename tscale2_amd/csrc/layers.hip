@@ -1205,6 +1205,48 @@ extern "C" int ts2_model_array(ts2_model *M, const char *name, int32_t index, ts
     if (!strcmp(name, "expertOffset") && M->moe.expertOffset) {
         tmp = Flat(M->moe.expertOffset, 1, M->cfg.expertCount + 2, TS2_I32); // first grouped row of each expert, rows in use, capacity
         a = &tmp;
+    } else if (!strncmp(name, "act.", 4) && index >= 0 && index < (int)M->layers.size() && M->layers[index].acts) {
+        // what layer `index` keeps from its forward pass (in recompute mode and for MoE layers: the shared set, valid for the layer that
+        // ran last).  FFN: wide, gate (bf16), wideScale, rg (8-bit); attention: q, gate, k, v (bf16), qScale, vScale, val (bf16; holds dQ
+        // after the layer's backward), vlg (8-bit), sumWeightLog
+        const TLayer &L = M->layers[index];
+        const TActs &A = *L.acts;
+        const int R = M->R, W = L.type == LT_FFN ? M->cfg.ffnDim : M->cfg.headCount * 128, T = W / 128;
+        const char *f = name + 4;
+        if (!strcmp(f, "a0") || !strcmp(f, "a1") || !strcmp(f, "a2") || !strcmp(f, "a3")) {
+            tmp = View(A.a16[f[1] - '0'], R, W);
+        } else if (!strcmp(f, "scale0") || !strcmp(f, "scale1")) {
+            tmp = View(A.tsc[f[5] - '0'], T, R);
+        } else if (!strcmp(f, "rg")) {
+            tmp = View(A.rg8, R, W);
+        } else if (!strcmp(f, "val")) {
+            tmp = View(A.val16, R, W);
+        } else if (!strcmp(f, "swl")) {
+            tmp = A.swl;
+        } else {
+            return TS2_ERR_UNSUPPORTED;
+        }
+        if (!tmp.m.ptr) {
+            return TS2_ERR_UNSUPPORTED;
+        }
+        a = &tmp;
+    } else if (!strncmp(name, "scratch.", 8) && index > 0) {
+        // gradient scratch of the layer backward that ran last, `index` columns wide: g0..g3 bf16 (drg / dvlg, dVal, dK, dV),
+        // f0..f3 fast-gradient type (dwide / dq, dgate, dk, dv), dscale fp32 [heads][lenRound]
+        const char *f = name + 8;
+        if ((f[0] == 'g' || f[0] == 'f') && f[1] >= '0' && f[1] <= '3' && !f[2] && index <= M->maxW) {
+            tmp = View(f[0] == 'g' ? M->g16[f[1] - '0'] : M->gf[f[1] - '0'], M->R, index);
+        } else if (!strcmp(f, "dscale")) {
+            tmp = M->dScale;
+        } else {
+            return TS2_ERR_UNSUPPORTED;
+        }
+        a = &tmp;
+    } else if (!strcmp(name, "gradMaxNorm")) {
+        tmp = Flat(M->gradMaxNorm, 1, (int)M->layers.size() + 2, TS2_F32); // running maxima of |stateGrad|: [0] feeds ts2_layer_backward
+        a = &tmp;
+    } else if (!strcmp(name, "finalGrad")) {
+        a = &M->gradV; // bf16 [lenRound][vocab]: the soft-max gradient of the last ts2_model_backprop
     } else if (!strcmp(name, "state")) {
         a = &M->state;
     } else if (!strcmp(name, "stateGrad")) {
