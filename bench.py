@@ -86,7 +86,7 @@ def cpu_baseline_linear(len_full, src_dim, grad_dim, sample_rows):
             "single_thread": {"value": rows1 / dt1, "cores": 1, "sample": f"{rows1} rows, {dt1:.1f} s (the reference as written: no threading)"}}
 
 
-def linear_i8_setup(delta_splits):
+def linear_i8_setup(delta_splits, sort_rows=False):
     """BASELINE config[1]: tensors and operator buffers of the int8 linear-layer backward"""
     import torch
     from tscale2_amd import lib as L
@@ -102,7 +102,7 @@ def linear_i8_setup(delta_splits):
     w8 = torch.clamp(torch.round(w / w_scale[:, None]), -128, 127).to(torch.int8)
     dy16 = dy.bfloat16()
     # the 4096 x 1024 delta has too few tiles for 256 CUs: stored slices of the token axis on 256x128 tiles, packed from their sum
-    bufs = L.MatMulBuffers(L.I8, len_, src_dim, grad_dim, k_tile=k_tile, splits=delta_splits, share_row_max=True)
+    bufs = L.MatMulBuffers(L.I8, len_, src_dim, grad_dim, k_tile=k_tile, splits=delta_splits, share_row_max=True, sort_rows=sort_rows)
     dx = torch.empty((len_, src_dim), dtype=torch.float32, device="cuda")
     dyv = dy16.view(torch.int16)
 
@@ -168,7 +168,7 @@ def bench_linear_i8(args):
     import torch
     from tscale2_amd import lib as L
     L.load()
-    c = linear_i8_setup(args.delta_splits)
+    c = linear_i8_setup(args.delta_splits, args.sort_rows)
     step, len_ = c["step"], c["len"]
     for _ in range(args.warmup):
         step()
@@ -189,7 +189,7 @@ def bench_linear_i8(args):
            "unit": "rows/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
            "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
            "config": {"workload": "int8 linear-layer backward (dX + delta): X[16384x1024] i8 per-row scales, dY[16384x4096] bf16, W[4096x1024] i8 "
-                                  "per-channel scales, k-tile 512", "tokens_per_step": len_, "gemm_gop_per_step": 2 * gemm_ops / 1e9},
+                                  "per-channel scales, k-tile 512" + (", rows sorted by scale" if args.sort_rows else ""), "tokens_per_step": len_, "gemm_gop_per_step": 2 * gemm_ops / 1e9},
            "bwd_gemm_tflops": g["tops"], "bwd_gemm_pct_of_peak": 100 * roof["frac"], "bwd_gemm_int8": g, "roofline": roof}
     roof["device_sustained"] = sustained(L.I8)
     if not args.no_cpu:
@@ -642,6 +642,7 @@ def main():
     ap.add_argument("--workload", default="step_fp8", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--delta-splits", type=int, default=2, help="linear_i8_bwd: slices of the token axis in the delta product (1 = single pass)")
+    ap.add_argument("--sort-rows", action="store_true", help="linear_i8_bwd: sort the gradient rows by scale before the delta product (the reference's order)")
     ap.add_argument("--small", action="store_true", help="step_fp8 / moe_fp8: a reduced model for quick checks (not a valid benchmark figure)")
     args = ap.parse_args()
     if args.gpus != 1:

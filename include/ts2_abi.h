@@ -195,6 +195,13 @@ int ts2_normalize_vecs_row_max2(int32_t len, int32_t lenRound, const ts2_mat *sr
     const ts2_mat *dst, float *rowScale, float *rowAbsMax, void *stream);
 int ts2_tile_max_from_rows(int32_t len, const float *rowAbsMax, const float *rowMult, int32_t kTile, float *tileMax, void *stream);
 
+/* HistSortFloatsStableKernel, src/lib/cuda/cuda_sort.cu:115-186 (SortPositiveFloatsApproxStable as BackpropMulti calls it on the row
+ * scales of the gradient, src/gpt/compute/matmul_fwdbwd.cuh:325): order[0..len) = the rows sorted ascending by the top 13 bits (sign,
+ * exponent, four mantissa bits) of key[t] = rowAbsMax[t] * |rowMult[t]| (rowMult optional); rows that share those bits come in
+ * descending row order, as in the reference (whose own test holds the hash of that order).  Deterministic.  tmp: len ints of scratch.
+ * (The reference sorts fewer than 500 values exactly instead; here every length takes the histogram order.) */
+int ts2_sort_rows_by_scale(int32_t len, const float *rowAbsMax, const float *rowMult, int32_t *order, int32_t *tmp, void *stream);
+
 /* Per-k-tile abs-max of a [len][dim] matrix (optionally times rowMult[t]): tileMax[t/kTile] = max |src|, the first half of
  * ShuffleMaxScaleTransposeKernel (src/gpt/compute/matmul_fwdbwd.cuh:209-231) without the sort.  tileMax must be zeroed by the
  * caller or with clear=1. */
@@ -226,8 +233,8 @@ int ts2_pack_delta(const ts2_mat *partial, int32_t splits, int64_t slabBytes, in
  *   srcT  [srcDim][lenRound] 8-bit                              (I8: Src8T;  E4M3: SrcE4T)
  *   tileMax, tileScale [lenRound/kTile] fp32                    (I8: SortedTileScale)
  *   transformT [srcDim][gradDim] 8-bit                          (TransformT)
- * Differences from the reference, by design: no random dither in the int8 quantisers, no sort of the rows (each kTile
- * consecutive tokens share the delta GEMM's scale) and exact int32 sums per k-tile added in fp32. */
+ * Differences from the reference, by design: no random dither in the int8 quantisers, the sort of the rows is optional (sortRows;
+ * without it each kTile consecutive tokens share the delta GEMM's scale) and exact int32 sums per k-tile added in fp32. */
 typedef struct ts2_matmul_bwd_buffers {
     ts2_mat grad8;
     float *grad8RowScale;
@@ -254,6 +261,14 @@ typedef struct ts2_matmul_bwd_buffers {
     /* != 0: transformT already holds the transpose of the `transformFast` given to BackpropMulti (the matrix has not changed since an
      * earlier call left it there: weights change once per optimiser step, not per micro-batch); the transpose is skipped. */
     int32_t transformTValid;
+    /* optional (I8): sortRows != 0 makes BackpropDelta contract over the rows in the order of ts2_sort_rows_by_scale (key = the gradient
+     * row's abs-max times |srcRowScale|), as the reference does (ShuffleMaxScaleTransposeKernel / ShuffleTransposeKernel gather the rows
+     * through the sorted list, matmul_fwdbwd.cuh:169-280): the rows of a k-tile then have like magnitudes and their common scale wastes
+     * few bits.  Needs gradRowAbsMax (valid) and rowOrder / rowOrderTmp [lenRound]; srcTValid is ignored (the source is gathered in this
+     * matrix's own order).  The delta itself does not depend on the order of the rows beyond the quantisation. */
+    int32_t *rowOrder;
+    int32_t *rowOrderTmp;
+    int32_t sortRows;
 } ts2_matmul_bwd_buffers;
 
 /* Bytes of every scratch member of ts2_matmul_bwd_buffers for one matrix, the sizes TInt8MatMulBwdBuffers / TFp8MatMulBwdBuffers allocate

@@ -10,6 +10,7 @@
  *   attention_forward, compute_dscale, attention_grad_q, attention_grad_k, transpose_attention, convert_i8, convert_e4m3,
  *   e4m3_to_float, cvt_i8, cvt_e4m3, model_schedule, make_causal_spans (+ the harness's labels and targets)
  *       -> bit-exact against ref (tests/test_oracle_vs_reference.py over tests/golden_cases.py).
+ *   hist_sort_stable -> the hash the reference's own sort test holds for its Mersenne-twister input (tests/test_oracle_own_contract.py).
  *   cvt_e4m3_rne, compress_delta, quantize_matrix_i8/e4m3, grad_mult, cpu_moe, cpu_backprop_moe, scale_experts,
  *   backprop_scale_experts, fwd/bwd_contract_matrix, layer_forward, layer_backward, final_backward, model_step
  *       -> their reference sources need cuda_runtime.h and cannot be compiled here; pinned by brute force over the code table,
@@ -82,6 +83,10 @@ void orc_quant_rowmax_i8(const float *src, int8_t *dst, float *rowScale, int len
 void orc_quant_ktile_i8(const float *src, int8_t *dst, float *tileScale, int len, int dim, int kTile);
 float orc_grad_mult(float maxNorm);
 float orc_bf16_round(float x);
+
+/* ---- sort.c ---- */
+void orc_hist_sort_stable(const float *val, int nodeCount, int *order, int forceHist);
+uint32_t orc_sort_result_hash(const int *order, int n);
 
 /* ---- moe.c ---- */
 void orc_cpu_moe(int len, int expertCount, int selectedCount, const float *moeSrc, float *res);

@@ -20,6 +20,7 @@
 #include <gpt/model_params/model_dim.h>
 #include <gpt/model_params/sse_utils.h>
 #include <util/fp8.h>
+#include <lib/random/mersenne.h>
 
 static void ToArr(TArray2D<float> *p, const float *src, yint ySize, yint xSize)
 {
@@ -274,6 +275,16 @@ int ref_init_label_data(const char *descr, int vocab, int fragCount, int fragLen
         spans[k * 2 + 1] = att.Spans[k].Finish;
     }
     return (int)n;
+}
+
+
+// the input of the reference's own sort test (TestCudaSort, src/lib/cuda/cuda_sort.cu:232-247): n draws of TMersenne<ui32>(seed).GenRandReal3()
+void ref_mersenne_real3(unsigned seed, int n, float *out)
+{
+    TMersenne<ui32> rng(seed);
+    for (int i = 0; i < n; ++i) {
+        out[i] = (float)rng.GenRandReal3();
+    }
 }
 
 }

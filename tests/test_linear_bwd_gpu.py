@@ -300,3 +300,105 @@ def test_transposes_left_by_the_caller_are_used_as_they_are(L, orc):
     b.c.gradTValid = 0
     d4, s4 = delta(other)
     assert torch.equal(d4, d2) and torch.equal(s4, s2)
+
+
+# ---- rows sorted by scale before the delta product (the reference's order) -----------------------------------------------------------
+
+def _sort_dev(L, key, mult=None):
+    n = key.size
+    order = torch.full((n,), -1, dtype=torch.int32, device="cuda"); tmp = torch.empty_like(order)
+    L.call("ts2_sort_rows_by_scale", n, torch.from_numpy(key).cuda(), None if mult is None else torch.from_numpy(mult).cuda(), order, tmp)
+    torch.cuda.synchronize()
+    return order.cpu().numpy()
+
+
+def test_row_sort_reproduces_the_reference_order(L, orc):
+    """ts2_sort_rows_by_scale on the input of the reference's own sort test: the hash of the order it holds (cuda_sort.cu:247), and the
+    oracle's order on other lengths and with a row multiplier"""
+    import ctypes as C
+    import os
+    print("case row sort", flush=True)
+    orc.lib.orc_sort_result_hash.restype = C.c_uint32
+    x = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_golden.npz"))["sort.mt1313_real3"]
+    got = _sort_dev(L, x)
+    assert orc.lib.orc_sort_result_hash(_ptr(np.ascontiguousarray(got)), x.size) == 1749808112
+    r = np.random.default_rng(31)
+    for n in (1, 63, 700, 5000, 32768, 70001):
+        key = np.exp(r.standard_normal(n) * 3).astype(np.float32)
+        key[r.random(n) < 0.05] = 0                                            # zero rows sort first
+        mult = (r.standard_normal(n) * 2).astype(np.float32) if n % 2 else None  # the key is |mult| * max
+        eff = key if mult is None else (key * np.abs(mult)).astype(np.float32)
+        want = np.zeros(n, np.int32)
+        orc.lib.orc_hist_sort_stable(_ptr(eff), n, _ptr(want), 1)
+        np.testing.assert_array_equal(_sort_dev(L, key, mult), want)
+
+
+@pytest.mark.parametrize("k_tile", [128, 512])
+def test_int8_delta_with_sorted_rows_same_contract(L, orc, k_tile):
+    """BackpropDelta with sortRows: the same contract on the CPU (the oracle's sort, rows gathered in that order, k-tile quantiser, exact
+    int32 sums per k-tile, packed delta) gives the same bytes; the row order and both transposed operands are checked on the way"""
+    import ctypes as C
+    print("case int8 delta, sorted rows", k_tile, flush=True)
+    len_, src_dim, grad_dim = 1500, 256, 384
+    len_round = (len_ + 511) // 512 * 512
+    r = np.random.default_rng(32)
+    x = orc.normalize_state(r.standard_normal((len_, src_dim)).astype(np.float32), src_dim // 128)
+    x8 = orc.convert_i8(x, 24.0)
+    dy16 = torch.from_numpy((r.standard_normal((len_, grad_dim)) * np.exp(r.standard_normal((len_, 1)) * 2)).astype(np.float32)).bfloat16()
+    dyf = dy16.float().numpy()
+    w8 = r.integers(-127, 128, (grad_dim, src_dim), dtype=np.int8)
+    bufs = L.MatMulBuffers(L.I8, len_round, src_dim, grad_dim, k_tile=k_tile, share_row_max=True, sort_rows=True)
+    x8d = torch.zeros((len_round, src_dim), dtype=torch.int8, device="cuda"); x8d[:len_] = torch.from_numpy(x8).cuda()
+    dyd = dy16.cuda().view(torch.int16)
+    bufs.backprop_multi(len_, torch.from_numpy(w8).cuda(), dyd, L.BF16)   # leaves the row maxima the sort keys come from
+    bufs.backprop_delta(len_, x8d, None, dyd, L.BF16)
+    torch.cuda.synchronize()
+    key = np.abs(dyf).max(1).astype(np.float32)
+    order = np.zeros(len_, np.int32)
+    orc.lib.orc_hist_sort_stable(_ptr(key), len_, _ptr(order), 1)
+    np.testing.assert_array_equal(bufs.t["rowOrder"].cpu().numpy()[:len_], order)
+    dys = np.zeros((len_round, grad_dim), np.float32); dys[:len_] = dyf[order]
+    xs = np.zeros((len_round, src_dim), np.int8); xs[:len_] = x8[order]
+    qk = np.zeros((len_round, grad_dim), np.int8); tsc = np.zeros(len_round // k_tile, np.float32)
+    orc.lib.orc_quant_ktile_i8(_ptr(dys), _ptr(qk), _ptr(tsc), len_round, grad_dim, k_tile)
+    np.testing.assert_array_equal(bufs.t["gradT"].cpu().numpy(), qk.T)
+    np.testing.assert_array_equal(bufs.t["srcT"].cpu().numpy(), xs.T)
+    acc = np.zeros((grad_dim, src_dim), np.float32)
+    orc.lib.orc_gemm_i8_nt_ktile(_ptr(np.ascontiguousarray(qk.T)), _ptr(np.ascontiguousarray(xs.T)), _ptr(tsc), k_tile, C.c_float(1.0), _ptr(acc),
+                                 grad_dim, src_dim, len_round)
+    want = np.zeros((grad_dim, src_dim), np.int8); want_ts = np.zeros((src_dim // 128, grad_dim), np.float32)
+    orc.lib.orc_compress_delta(_ptr(acc), _ptr(want), _ptr(want_ts), grad_dim, src_dim)
+    np.testing.assert_allclose(bufs.delta_tile_scale.cpu().numpy(), want_ts, rtol=2e-6)
+    dd = np.abs(bufs.delta.cpu().numpy().astype(np.int32) - want)
+    assert dd.max() <= 1 and (dd != 0).mean() < 1e-3
+
+
+def test_int8_delta_precision_on_heavy_tailed_rows(L, orc):
+    """What the common scale of a k-tile costs when the gradient rows differ in magnitude (log-normal row scales, sigma 0.5 and 3),
+    with consecutive rows and with rows sorted by scale, against the fp32 SumRankOne of the CPU path.  int8 with one scale per k-tile
+    keeps about two per cent of the delta's rms whatever the order; sorting helps where the spread is mild."""
+    print("case int8 delta, heavy-tailed rows", flush=True)
+    len_, src_dim, grad_dim = 4096, 256, 256
+    r = np.random.default_rng(33)
+    x8 = orc.convert_i8(orc.normalize_state(r.standard_normal((len_, src_dim)).astype(np.float32), src_dim // 128), 24.0)
+    x8d = torch.from_numpy(x8).cuda()
+    w8 = torch.from_numpy(r.integers(-127, 128, (grad_dim, src_dim), dtype=np.int8)).cuda()
+    res = {}
+    for sigma in (0.5, 3.0):
+        dy16 = torch.from_numpy((r.standard_normal((len_, grad_dim)) * np.exp(r.standard_normal((len_, 1)) * sigma)).astype(np.float32)).bfloat16()
+        ref = orc.sum_rank_one(x8.astype(np.float32), dy16.float().numpy())
+        for sort_rows in (False, True):
+            for kt in (128, 512):
+                bufs = L.MatMulBuffers(L.I8, len_, src_dim, grad_dim, k_tile=kt, share_row_max=True, sort_rows=sort_rows)
+                dyd = dy16.cuda().view(torch.int16)
+                bufs.backprop_multi(len_, w8, dyd, L.BF16)
+                bufs.backprop_delta(len_, x8d, None, dyd, L.BF16)
+                torch.cuda.synchronize()
+                d = bufs.delta_fp32().cpu().numpy() - ref
+                res[(sigma, sort_rows, kt)] = (float(np.sqrt((d ** 2).mean()) / np.sqrt((ref ** 2).mean())), float(np.abs(d).max() / np.abs(ref).max()))
+                print(f"sigma {sigma} sorted {sort_rows} kTile {kt}: rms {res[(sigma, sort_rows, kt)][0]:.4f} max/max {res[(sigma, sort_rows, kt)][1]:.4f}")
+    for k, (rms, mx) in res.items():
+        assert rms <= 0.10 and mx <= 0.08, (k, rms, mx)
+    # mild spread: rows of like scale share a tile once sorted, and the result is clearly closer
+    assert res[(0.5, True, 128)][0] <= 0.7 * res[(0.5, False, 128)][0]
+    assert res[(0.5, True, 512)][0] <= 0.8 * res[(0.5, False, 512)][0]

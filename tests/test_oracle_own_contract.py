@@ -174,3 +174,28 @@ def test_embedding_is_a_signed_gather_and_its_backward_the_scatter(orc):
         for k in range(label_ptr[t], label_ptr[t + 1]):
             wd[ids[k]] += grad[t] * (-1 if neg[k] else 1)
     np.testing.assert_allclose(delta, wd, rtol=1e-6, atol=1e-6)
+
+
+def test_hist_sort_reproduces_the_hash_of_the_reference_sort_test(orc):
+    """TestCudaSort (src/lib/cuda/cuda_sort.cu:232-250) sorts 16384 draws of TMersenne(1313).GenRandReal3() and checks the hash of the
+    node ids against 1749808112: the restated order (bins of the top 13 bits ascending, descending id inside a bin) must give it"""
+    import os
+    gold = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_golden.npz"))
+    x = gold["sort.mt1313_real3"]
+    # the same stream from numpy's Mersenne twister (init_genrand(1313), (u32 + 0.5) / 2^32): the fixture is what the reference draws
+    u = np.random.RandomState(1313).randint(0, 2 ** 32, x.size, dtype=np.uint64)
+    assert np.array_equal(((u.astype(np.float64) + 0.5) / 4294967296.0).astype(np.float32), x)
+    order = np.zeros(x.size, np.int32)
+    orc.lib.orc_hist_sort_stable(_ptr(x), x.size, _ptr(order), 0)
+    orc.lib.orc_sort_result_hash.restype = C.c_uint32
+    assert orc.lib.orc_sort_result_hash(_ptr(order), x.size) == 1749808112
+    assert sorted(order.tolist()) == list(range(x.size))
+    keys = x.view(np.uint32) >> 18
+    assert (np.diff(keys[order].astype(np.int64)) >= 0).all()
+    same = keys[order][1:] == keys[order][:-1]
+    assert (np.diff(order)[same] < 0).all()                              # descending id inside a bin
+    # below 500 values the reference sorts exactly, by (score, id)
+    y = np.round(x[:300] * 20) / 20
+    o2 = np.zeros(300, np.int32)
+    orc.lib.orc_hist_sort_stable(_ptr(y), 300, _ptr(o2), 0)
+    assert np.array_equal(o2, np.lexsort((np.arange(300), y)))

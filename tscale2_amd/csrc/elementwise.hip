@@ -988,9 +988,13 @@ __global__ void __launch_bounds__(256) TransposeQuant(int len, int lenRound, Mat
             const int k0 = (tBlock / kTile) * kTile;
             float mx = 0;
             for (int t = k0 + tid; t < k0 + kTile && t < len; t += 256) {
-                float m = rowAbsMax[t];
+                const int sr = rowIndex ? rowIndex[t] : t; // (a gathered tile: the maxima of the rows that land in it)
+                if (sr < 0) {
+                    continue;
+                }
+                float m = rowAbsMax[sr];
                 if (rowMult) {
-                    m *= fabsf(rowMult[t]);
+                    m *= fabsf(rowMult[sr]);
                 }
                 mx = fmaxf(mx, m);
             }
@@ -1641,8 +1645,9 @@ extern "C" int ts2_transpose_quant(int32_t len, int32_t lenRound, const ts2_mat 
     return Ts2TransposeQuantRows(len, lenRound, src, srcType, rowMult, tileMax, nullptr, kTile, rowIndex, dstT, dstType, tileScale, stream);
 }
 
-// ts2_transpose_quant whose k-tile maxima may come from the row maxima instead (rowAbsMax, with tileMax null and no row index): the
-// kernel then forms each k-tile's maximum itself and the separate ts2_tile_max_from_rows launch is not needed
+// ts2_transpose_quant whose k-tile maxima may come from the row maxima instead (rowAbsMax, with tileMax null; with a row index: the
+// maxima of the rows gathered into the tile): the kernel then forms each k-tile's maximum itself and the separate
+// ts2_tile_max_from_rows launch is not needed
 int Ts2TransposeQuantRows(int len, int lenRound, const ts2_mat *src, int srcType, const float *rowMult, const float *tileMax, const float *rowAbsMax,
     int kTile, const int *rowIndex, const ts2_mat *dstT, int dstType, float *tileScale, void *stream)
 {
@@ -1660,7 +1665,7 @@ int Ts2TransposeQuantRows(int len, int lenRound, const ts2_mat *src, int srcType
     dim3 grid(dim / 128, lenRound / 128);
     bool quant = dstType == TS2_I8 && (srcType == TS2_BF16 || srcType == TS2_F32);
     if (quant) {
-        if ((!tileMax && !rowAbsMax) || (rowAbsMax && rowIndex) || kTile <= 0 || kTile % 128) {
+        if ((!tileMax && !rowAbsMax) || kTile <= 0 || kTile % 128) {
             return TS2_ERR_SHAPE;
         }
         if (tileMax) {

@@ -169,7 +169,18 @@ extern "C" int ts2_matmul_backprop_delta(int32_t mode, int32_t len, int32_t lenR
         if (kTile <= 0 || kTile % 128 || lenRound % kTile || !buf->tileMax || !buf->tileScale) {
             return TS2_ERR_SHAPE;
         }
-        if (buf->gradRowAbsMax && buf->gradRowAbsMaxValid) {
+        if (buf->sortRows) {
+            // the reference's order: rows sorted by their scale, gathered through the sorted list by both transposing passes
+            if (!buf->gradRowAbsMax || !buf->gradRowAbsMaxValid || !buf->rowOrder || !buf->rowOrderTmp) {
+                return TS2_ERR_NULL;
+            }
+            rc = ts2_sort_rows_by_scale(len, buf->gradRowAbsMax, srcRowScale, buf->rowOrder, buf->rowOrderTmp, stream);
+            if (rc) {
+                return rc;
+            }
+            rc = Ts2TransposeQuantRows(len, lenRound, grad, gradType, srcRowScale, nullptr, buf->gradRowAbsMax, kTile, buf->rowOrder, &buf->gradT,
+                TS2_I8, buf->tileScale, stream);
+        } else if (buf->gradRowAbsMax && buf->gradRowAbsMaxValid) {
             // the k-tile maxima follow from the row maxima of the dX pass: the transposing quantiser forms them itself
             rc = Ts2TransposeQuantRows(len, lenRound, grad, gradType, srcRowScale, nullptr, buf->gradRowAbsMax, kTile, nullptr, &buf->gradT, TS2_I8,
                 buf->tileScale, stream);
@@ -197,8 +208,9 @@ extern "C" int ts2_matmul_backprop_delta(int32_t mode, int32_t len, int32_t lenR
             }
         }
     }
-    if (!buf->srcTValid) {
-        rc = ts2_transpose_quant(len, lenRound, src, mode, nullptr, nullptr, 0, nullptr, &buf->srcT, mode, nullptr, stream);
+    const int *rowOrder = (mode == TS2_I8 && buf->sortRows) ? buf->rowOrder : nullptr;
+    if (!buf->srcTValid || rowOrder) {
+        rc = ts2_transpose_quant(len, lenRound, src, mode, nullptr, nullptr, 0, rowOrder, &buf->srcT, mode, nullptr, stream);
         if (rc) {
             return rc;
         }

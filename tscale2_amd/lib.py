@@ -172,14 +172,15 @@ def probe_copy_rate(nbytes=1 << 30):
 class BwdBuffers(C.Structure):
     _fields_ = [("grad8", Mat), ("grad8RowScale", C.c_void_p), ("gradT", Mat), ("srcT", Mat), ("tileMax", C.c_void_p), ("tileScale", C.c_void_p),
                 ("transformT", Mat), ("partial", Mat), ("splits", C.c_int32), ("gradRowAbsMax", C.c_void_p),
-                ("gradRowAbsMaxValid", C.c_int32), ("srcTValid", C.c_int32), ("gradTValid", C.c_int32), ("transformTValid", C.c_int32)]
+                ("gradRowAbsMaxValid", C.c_int32), ("srcTValid", C.c_int32), ("gradTValid", C.c_int32), ("transformTValid", C.c_int32),
+                ("rowOrder", C.c_void_p), ("rowOrderTmp", C.c_void_p), ("sortRows", C.c_int32)]
 
 
 class MatMulBuffers:
     """Scratch of one linear layer's backward, allocated with torch (the reference allocates the same members from its pools,
     src/gpt/compute/matmul_fwdbwd.cuh:283-311).  mode: I8 or E4M3."""
 
-    def __init__(self, mode, len_round, src_dim, grad_dim, k_tile=512, splits=1, share_row_max=False):
+    def __init__(self, mode, len_round, src_dim, grad_dim, k_tile=512, splits=1, share_row_max=False, sort_rows=False):
         import torch
         self.mode, self.len_round, self.src_dim, self.grad_dim, self.k_tile = mode, len_round, src_dim, grad_dim, k_tile
         bt = torch.int8 if mode == I8 else torch.uint8
@@ -202,6 +203,11 @@ class MatMulBuffers:
             self.t["gradRowAbsMax"] = torch.empty(len_round, dtype=torch.float32, device=dev)
             self.c.gradRowAbsMax = self.t["gradRowAbsMax"].data_ptr()
             self.c.gradRowAbsMaxValid = 1
+        if sort_rows:
+            assert share_row_max and mode == I8, "the sorted delta needs the row maxima that backprop_multi leaves"
+            self.t["rowOrder"] = torch.empty(len_round, dtype=torch.int32, device=dev)
+            self.t["rowOrderTmp"] = torch.empty(len_round, dtype=torch.int32, device=dev)
+            self.c.rowOrder, self.c.rowOrderTmp, self.c.sortRows = self.t["rowOrder"].data_ptr(), self.t["rowOrderTmp"].data_ptr(), 1
         if splits > 1:
             self.t["partial"] = torch.empty((splits * grad_dim, src_dim), dtype=torch.float32, device=dev)
             self.c.partial = mat(self.t["partial"])
