@@ -442,6 +442,66 @@ int ts2_transpose_u8_batched(int32_t batch, int32_t rows, int32_t cols, const vo
     int64_t dstStride, int64_t dstSlabBytes, void *stream);
 
 /* ------------------------------------------------------------------------------------------------------------------------
+ * Optimiser apply on the device (src/gpt/matrix/agpu_cuda.cuh, agpu_cuda.cu; CPU twin THostModelMatrix::AddDelta,
+ * src/gpt/matrix/host_matrix.cpp:112-145): packed delta -> row-normalised moving average -> fp32 master weights -> fast weights.
+ * Matrices are [ySize = out][xSize = in], xSize a multiple of 128; every array is device-resident and caller-owned. */
+
+/* TAddGradientKernelParams (agpu_cuda.cuh:19-27), device-resident like the reference's CudaAGParams so that a captured sequence of launches
+ * follows a changing learning rate; stepMult = TTrainingStep::Rate (src/gpt/train_config/train_step.h:4-27). */
+typedef struct ts2_add_gradient_params {
+    float dispDecay, beta1, weight0, weight1, l2Reg, stepMult;
+} ts2_add_gradient_params;
+
+/* UnpackDeltaKernel<ADD_TO_TARGET>, agpu_cuda.cuh:35-49: dst[y][x] (+)= delta[y][x] * tileScale[x/128][y] */
+int ts2_unpack_delta(int32_t xSize, int32_t ySize, const ts2_mat *delta, const ts2_mat *tileScale, const ts2_mat *dst, int32_t addToTarget,
+    void *stream);
+/* MatrixRowSum2Kernel, agpu_cuda.cu:33-52: sum2arr[y] = sum_x matr[y][x]^2 */
+int ts2_matrix_row_sum2(int32_t xSize, int32_t ySize, const ts2_mat *matr, float *sum2arr, void *stream);
+/* the same row sums taken from a packed delta without expanding it (UnpackDeltaKernel<0> + MatrixRowSum2Kernel in one pass over the bytes) */
+int ts2_packed_delta_row_sum2(int32_t xSize, int32_t ySize, const ts2_mat *delta, const ts2_mat *tileScale, float *sum2arr, void *stream);
+/* UpdateGlobalRowDisp, agpu_cuda.cu:60-109: sumWeight = sumWeight * dispDecay + 1; per block of ySize / rowDispSize rows
+ * rowDisp = rowDisp * dispDecay + mean square of the block's delta; rowScale[y] = 1 / sqrt(rowDisp / sumWeight) (0 when that is 0) */
+int ts2_update_global_row_disp(int32_t xSize, int32_t ySize, int32_t rowDispSize, const float *deltaSum2arr, const ts2_add_gradient_params *params,
+    float *sumWeight, float *rowDisp, float *rowScale, void *stream);
+/* AddGradientKernel, agpu_cuda.cu:112-139: d = grad * rowScale[y]; avgGrad = avgGrad * beta1 + d * (1 - beta1);
+ * weights = weights * (1 - step * l2Reg) + (avgGrad * weight1 + d * weight0) * step with step = stepMult * sqrt(*sparsity);
+ * weightsRowSum2[y] = sum_x weights[y][x]^2 */
+int ts2_add_gradient(int32_t xSize, int32_t ySize, const ts2_mat *grad, const ts2_add_gradient_params *params, const float *rowScale,
+    const float *sparsity, const ts2_mat *avgGrad, const ts2_mat *weights, float *weightsRowSum2, void *stream);
+/* ConvertMatrixKernel, agpu_cuda.cuh:65-101: *matrixScale = sko = sqrt(sum(sum2arr[0..totalYSize)) / (totalXSize * totalYSize));
+ * fast = cvt(weights * 32 / sko) as fastType (TS2_I8 | TS2_E4M3 | TS2_BF16), all zero for a zero matrix; rows ySize .. yBufSize cleared.
+ * convertMult: one float of scratch. */
+int ts2_convert_matrix(int32_t xSize, int32_t ySize, int32_t yBufSize, int32_t totalXSize, int32_t totalYSize, const ts2_mat *weights,
+    const float *sum2arr, const ts2_mat *fast, int32_t fastType, float *matrixScale, float *convertMult, void *stream);
+
+/* device state of one matrix = the members of TAgpuCudaModelMatrix (agpu_cuda.cuh:343-360,431-470) on one device */
+typedef struct ts2_opt_matrix {
+    int32_t xSize, ySize, yBufSize; /* yBufSize: rows of `fast` (ySize rounded up to 128) */
+    int32_t rowDispSize;            /* divides ySize: rows per dispersion estimate = ySize / rowDispSize (GetRowDispSize) */
+    ts2_mat weights, avgGrad;       /* fp32 [ySize][xSize]: Weights, AvgGrad */
+    ts2_mat grad;                   /* fp32 [ySize][xSize]: Grad, the accumulator over micro-batches; may be empty when every delta is
+                                       applied at once (TS2_BM_GRAD_APPLY without TS2_BM_GRAD_ADD) */
+    float *gradRowSum2, *weightsRowSum2, *rowScale; /* [ySize] */
+    float *rowDisp;                 /* [rowDispSize] */
+    float *sumWeight, *sparsity;    /* [1] each */
+    ts2_mat fast;                   /* FastDevice [yBufSize][xSize] of fastType */
+    int32_t fastType;
+    float *matrixScale;             /* [1]: MatrixScale (GetScale) */
+    float *convertMult;             /* [1] scratch */
+} ts2_opt_matrix;
+
+enum { TS2_BM_GRAD_ADD = 1, TS2_BM_GRAD_APPLY = 2 }; /* EBackpropMode bits, src/gpt/matrix/base_cuda.cuh */
+
+/* TAgpuCudaModelMatrix::Convert, agpu_cuda.cuh:412-428 (after the master weights were set: CopyToDevice) */
+int ts2_opt_convert(const ts2_opt_matrix *m, void *stream);
+/* TAgpuCudaModelMatrix::AddDelta(TCudaPackedDeltaMatrix&, bm) with ApplyGradientImpl, agpu_cuda.cuh:484-590, on one device (its
+ * all-reduces over devices drop out): backpropMode = TS2_BM_GRAD_ADD adds the delta to `grad`, otherwise it replaces it;
+ * TS2_BM_GRAD_APPLY then updates the dispersion estimates, the moving average, the weights and the fast weights.  APPLY without ADD
+ * reads the packed bytes directly and leaves `grad` untouched. */
+int ts2_opt_add_delta(const ts2_opt_matrix *m, const ts2_mat *delta, const ts2_mat *tileScale, int32_t backpropMode,
+    const ts2_add_gradient_params *params, void *stream);
+
+/* ------------------------------------------------------------------------------------------------------------------------
  * Layer stack and one-GPU step driver: the counterpart of TCudaLayerBase::{AddForward, AddBackward}
  * (src/gpt/compute/layer_cuda_base.cuh:290-294) and of the executor's forward/backprop graphs
  * (src/gpt/compute/gpu_transformer.cu:260-471; IModelImpl::Backprop, src/gpt/compute/model.h:60-67).

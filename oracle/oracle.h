@@ -11,6 +11,8 @@
  *   e4m3_to_float, cvt_i8, cvt_e4m3, model_schedule, make_causal_spans (+ the harness's labels and targets)
  *       -> bit-exact against ref (tests/test_oracle_vs_reference.py over tests/golden_cases.py).
  *   hist_sort_stable -> the hash the reference's own sort test holds for its Mersenne-twister input (tests/test_oracle_own_contract.py).
+ *   unpack_delta, apply_delta -> closed forms of the update rule (tests/test_oracle_optim.py): unpack o compress = id within half a step,
+ *       unit step length per row, geometric moving average, weight decay, block dispersion = mean over the block's rows.
  *   cvt_e4m3_rne, compress_delta, quantize_matrix_i8/e4m3, grad_mult, cpu_moe, cpu_backprop_moe, scale_experts,
  *   backprop_scale_experts, fwd/bwd_contract_matrix, layer_forward, layer_backward, final_backward, model_step
  *       -> their reference sources need cuda_runtime.h and cannot be compiled here; pinned by brute force over the code table,
@@ -87,6 +89,14 @@ float orc_bf16_round(float x);
 /* ---- sort.c ---- */
 void orc_hist_sort_stable(const float *val, int nodeCount, int *order, int forceHist);
 uint32_t orc_sort_result_hash(const int *order, int n);
+
+/* ---- optim.c ---- */
+typedef struct {
+    float rate, l2Reg, beta1, weight0, weight1, dispDecay; /* TTrainingStep, src/gpt/train_config/train_step.h:4-27 */
+} orc_train_step;
+void orc_unpack_delta(const int8_t *delta, const float *tileScale, float *dst, int ySize, int xSize, int add);
+double orc_apply_delta(float *weights, float *avgGrad, const float *delta, int ySize, int xSize, int rowDispSize, float *rowDisp, float *sumWeight,
+    float sparsity, const orc_train_step *st, float *rowScaleOut);
 
 /* ---- moe.c ---- */
 void orc_cpu_moe(int len, int expertCount, int selectedCount, const float *moeSrc, float *res);
