@@ -535,6 +535,17 @@ void ts2_model_destroy(ts2_model *m);
  * (model_dim.h:65-80); fastHost is [rows][cols] bytes of the model's 8-bit type, scale the matrix scale. */
 int ts2_model_set_matrix(ts2_model *m, int32_t layer, int32_t matrixId, const void *fastHost, int32_t rows, int32_t cols, float scale);
 int ts2_model_set_bias(ts2_model *m, const float *biasHost);
+/* Optimiser state of the step driver (optional).  ts2_model_set_master gives a matrix fp32 master weights [rows][cols] (rows without the
+ * tile padding), a dispersion granularity (rowDispSize = rows: per row, 1: per matrix; SetSizesPerRowDisp / SetSizesPerMatrixDisp,
+ * src/gpt/model_params/model_matrix.h:116-127) and its sparsity factor, and derives the fast weights and the matrix scale from them on the
+ * device (CopyToDevice + Convert, src/gpt/matrix/agpu_cuda.cuh:412-428,473-482).  ts2_model_apply_deltas runs one optimiser step
+ * (ts2_opt_add_delta with TS2_BM_GRAD_APPLY) over every such matrix with the deltas of the last ts2_model_backprop; matrices without
+ * master weights keep theirs.  paramsHost is a host struct.  ts2_model_get_master / ts2_model_get_matrix read weights back. */
+int ts2_model_set_master(ts2_model *m, int32_t layer, int32_t matrixId, const float *weightsHost, int32_t rows, int32_t cols, int32_t rowDispSize,
+    float sparsity);
+int ts2_model_apply_deltas(ts2_model *m, const ts2_add_gradient_params *paramsHost, void *stream);
+int ts2_model_get_master(ts2_model *m, int32_t layer, int32_t matrixId, float *hostOut, int32_t rows, int32_t cols);
+int ts2_model_get_matrix(ts2_model *m, int32_t layer, int32_t matrixId, void *fastHostOut, int32_t rows, int32_t cols, float *scaleOut);
 /* nodes of one batch (TBatchNodes, src/gpt/att/nodes_batch.h:42-57): label CSR, target token per row (-1 = none), one span per
  * row and attention type, RoPE table [len][128]; host arrays */
 int ts2_model_set_batch(ts2_model *m, int32_t len, const int32_t *labelPtr, const uint32_t *labels, const int32_t *targetPerRow,

@@ -62,6 +62,7 @@ class QMatrix:
     def __init__(self, orc, w, mode, no_scale):
         rows, cols = w.shape
         w = np.ascontiguousarray(w, np.float32)
+        self.w = w  # the fp32 master weights the fast bytes were derived from
         if mode == I8:
             self.fast = np.zeros((rows, cols), np.int8)
             self.scale = float(orc.lib.orc_quantize_matrix_i8(_ptr(w), _ptr(self.fast), rows, cols))

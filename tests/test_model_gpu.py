@@ -217,3 +217,69 @@ def test_moe_routing_tables_match_cpu_moe():
         assert np.all(np.diff(live) >= 0)  # stable: token order inside an expert
         assert np.all(tile[eo[e] // 128:eo[e + 1] // 128] == e)
     assert np.all(tile[eo[E] // 128:] == -1)
+
+
+@pytest.mark.parametrize("mode", [I8, E4M3])
+def test_two_steps_with_a_real_optimiser_update(mode):
+    """backprop -> optimiser apply on the device -> backprop.  (1) master weights loaded with ts2_model_set_master give the fast bytes
+    and scale of the per-matrix quantiser; (2) the update equals the oracle's THostModelMatrix::AddDelta on the device's own deltas;
+    (3) the second step is exactly what a fresh model holding the updated fast weights computes - the transposed copies the driver keeps
+    between steps were dropped by the update; (4) the loss on the same batch went down."""
+    import ctypes as C
+    print("case two steps with optimiser update", mode, flush=True)
+    from oracle_lib import _ptr
+    from tscale2_amd import lib as L
+    h = Harness(mode, dim=256, heads=2, ffn_tiles=4, depth=2, vocab=256, frag_count=4, frag_len=64, wide_window=64, seed=9)
+    bdt = np.int8 if mode == I8 else np.uint8
+    mats = [(d, i, q) for d in range(h.depth) for i, q in enumerate(h.layers[d])] + [(L.LAYER_EMBED, 0, h.embed), (L.LAYER_FINAL, 0, h.final)]
+
+    class Step(C.Structure):
+        _fields_ = [(n, C.c_float) for n in ("rate", "l2Reg", "beta1", "weight0", "weight1", "dispDecay")]
+    st = Step(0.02, 0.0, 0.9, 1.0, 0.5, 0.9)
+    h.orc.lib.orc_apply_delta.restype = C.c_double
+    m = h.device_model()
+    try:
+        for d, i, q in mats:
+            m.set_master(d, i, q.w, q.w.shape[0])                             # per-row dispersion
+            fast, scale = m.get_matrix(d, i, *q.fast.shape, bdt)
+            assert abs(scale - q.scale) <= 3e-6 * q.scale
+            assert (fast != q.fast).mean() < 2e-3                             # the same bytes but for values within an ulp of a rounding tie
+        m.backprop()
+        torch.cuda.synchronize()
+        loss1 = m.loss_sum()
+        deltas1 = [m.get_delta(d, i, *q.fast.shape) for d, i, q in mats]
+        m.apply_deltas(st.rate, st.l2Reg, st.beta1, st.weight0, st.weight1, st.dispDecay)
+        torch.cuda.synchronize()
+        new_fast = []
+        for (d, i, q), delta in zip(mats, deltas1):
+            rows, cols = q.w.shape
+            w = q.w.copy(); ag = np.zeros_like(w); rd = np.zeros(rows, np.float32); sw = np.zeros(1, np.float32)
+            h.orc.lib.orc_apply_delta(_ptr(w), _ptr(ag), _ptr(np.ascontiguousarray(delta)), rows, cols, rows, _ptr(rd), _ptr(sw), C.c_float(1.0),
+                                      C.byref(st), None)
+            got = m.get_master(d, i, rows, cols)
+            np.testing.assert_allclose(got, w, rtol=2e-5, atol=2e-6 * np.abs(w).max())
+            assert np.abs(got - q.w).max() > 0                                # the weights did move
+            new_fast.append(m.get_matrix(d, i, rows, cols, bdt))
+        m.backprop()
+        torch.cuda.synchronize()
+        loss2 = m.loss_sum()
+        deltas2 = [m.get_delta(d, i, *q.fast.shape) for d, i, q in mats] + [m.array("stateGrad").float().cpu().numpy()]
+    finally:
+        m.close()
+    print("loss before / after the update", loss1, loss2)
+    assert loss2 > loss1                                                      # (the loss is the sum of log-probabilities: up is better)
+    m2 = h.device_model()
+    try:
+        for (d, i, q), (fast, scale) in zip(mats, new_fast):
+            m2.set_matrix(d, i, fast, scale)
+        m2.backprop()
+        torch.cuda.synchronize()
+        want = [m2.get_delta(d, i, *q.fast.shape) for d, i, q in mats] + [m2.array("stateGrad").float().cpu().numpy()]
+    finally:
+        m2.close()
+    names = [(d, i) for d, i, _ in mats] + ["stateGrad"]
+    for nm, a, b in zip(names, deltas2, want):
+        if nm == (L.LAYER_EMBED, 0):   # the embedding delta is summed with fp32 atomics: equal up to the order of the additions
+            np.testing.assert_allclose(a, b, rtol=0, atol=1e-6 * np.abs(b).max())
+        else:
+            assert np.array_equal(a, b), nm

@@ -64,6 +64,11 @@ struct TMatrix {
     Arr delta;          // i8 packed delta, same shape
     Arr deltaTileScale; // fp32 [src/128][rows]
     int srcDim = 0, dstDim = 0, slabs = 1;
+    // optimiser state (master weights, moving average, dispersion estimates), present once ts2_model_set_master has been called
+    ts2_opt_matrix opt = {};
+    Arr optWeights, optAvgGrad;
+    bool hasOpt = false;
+    int optRows = 0; // rows of the master matrix (the model's rows without tile padding)
 };
 
 struct TActs;
@@ -111,6 +116,7 @@ struct ts2_model {
     // model
     TMatrix embed, finalW;
     float *bias = 0;
+    ts2_add_gradient_params *optParams = 0; // device copy of the optimiser step parameters
     // batch
     int *labelPtr = 0;
     uint32_t *labels = 0;
@@ -1057,6 +1063,136 @@ extern "C" int ts2_model_set_matrix(ts2_model *M, int32_t layer, int32_t matrixI
         return TS2_ERR_LAUNCH;
     }
     W->fastTValid = false; // the kept transpose belongs to the old weights
+    return 0;
+}
+
+// master weights of a matrix: allocates its optimiser state on first use, uploads the fp32 weights and derives the fast weights and the
+// matrix scale from them on the device (TAgpuCudaModelMatrix::CopyToDevice, src/gpt/matrix/agpu_cuda.cuh:473-482)
+extern "C" int ts2_model_set_master(ts2_model *M, int32_t layer, int32_t matrixId, const float *weightsHost, int32_t rows, int32_t cols,
+    int32_t rowDispSize, float sparsity)
+{
+    TMatrix *W = M ? FindMatrix(M, layer, matrixId) : nullptr;
+    if (!W || !weightsHost) {
+        return TS2_ERR_NULL;
+    }
+    if (cols != W->srcDim || rows <= 0 || rows > W->dstDim * W->slabs || rowDispSize <= 0 || rows % rowDispSize) {
+        return TS2_ERR_SHAPE;
+    }
+    if (W->hasOpt && W->optRows != rows) {
+        return TS2_ERR_SHAPE;
+    }
+    if (!W->hasOpt) {
+        ts2_opt_matrix &o = W->opt;
+        bool ok = M->Alloc(&W->optWeights, rows, cols, TS2_F32) && M->Alloc(&W->optAvgGrad, rows, cols, TS2_F32);
+        o.gradRowSum2 = (float *)M->Dev((size_t)rows * 4);
+        o.weightsRowSum2 = (float *)M->Dev((size_t)rows * 4);
+        o.rowScale = (float *)M->Dev((size_t)rows * 4);
+        o.rowDisp = (float *)M->Dev((size_t)rows * 4); // room for any later rowDispSize
+        o.sumWeight = (float *)M->Dev(4);
+        o.sparsity = (float *)M->Dev(4);
+        o.convertMult = (float *)M->Dev(4);
+        if (!ok || !o.gradRowSum2 || !o.weightsRowSum2 || !o.rowScale || !o.rowDisp || !o.sumWeight || !o.sparsity || !o.convertMult) {
+            return TS2_ERR_LAUNCH;
+        }
+        o.xSize = cols;
+        o.ySize = rows;
+        o.yBufSize = W->fast.m.y; // the conversion also clears the padding rows of the fast matrix
+        o.weights = W->optWeights.m;
+        o.avgGrad = W->optAvgGrad.m;
+        o.fast = W->fast.m;
+        o.fastType = M->mode;
+        o.matrixScale = W->scale;
+        W->optRows = rows;
+        W->hasOpt = true;
+    }
+    W->opt.rowDispSize = rowDispSize;
+    if (Copy2D(W->optWeights.m.ptr, W->optWeights.m.strideBytes, weightsHost, (size_t)cols * 4, (size_t)cols * 4, rows, hipMemcpyHostToDevice) !=
+            hipSuccess ||
+        hipMemcpy(W->opt.sparsity, &sparsity, 4, hipMemcpyHostToDevice) != hipSuccess ||
+        hipMemset(W->optAvgGrad.m.ptr, 0, (size_t)W->optAvgGrad.m.strideBytes * rows) != hipSuccess ||
+        hipMemset(W->opt.rowDisp, 0, (size_t)rows * 4) != hipSuccess || hipMemset(W->opt.sumWeight, 0, 4) != hipSuccess) {
+        return TS2_ERR_LAUNCH;
+    }
+    W->fastTValid = false;
+    return ts2_opt_convert(&W->opt, nullptr);
+}
+
+// one optimiser step over every matrix that has master weights: the packed delta of the last ts2_model_backprop is applied
+// (TAgpuCudaModelMatrix::AddDelta with BM_GRAD_APPLY, agpu_cuda.cuh:564-590; the embedding's delta is fp32 and goes through the
+// unpacked sequence, :536-562), new fast weights and scales replace the old ones and the kept transposes are dropped
+extern "C" int ts2_model_apply_deltas(ts2_model *M, const ts2_add_gradient_params *paramsHost, void *stream)
+{
+    if (!M || !paramsHost) {
+        return TS2_ERR_NULL;
+    }
+    if (!M->optParams) {
+        M->optParams = (ts2_add_gradient_params *)M->Dev(sizeof(ts2_add_gradient_params));
+        if (!M->optParams) {
+            return TS2_ERR_LAUNCH;
+        }
+    }
+    if (hipMemcpyAsync(M->optParams, paramsHost, sizeof(ts2_add_gradient_params), hipMemcpyHostToDevice, (hipStream_t)stream) != hipSuccess) {
+        return TS2_ERR_LAUNCH;
+    }
+    auto apply = [&](TMatrix &W, bool packed) -> int {
+        if (!W.hasOpt) {
+            return 0;
+        }
+        W.fastTValid = false;
+        const ts2_opt_matrix &o = W.opt;
+        if (packed) {
+            return ts2_opt_add_delta(&o, W.delta.P(), W.deltaTileScale.P(), TS2_BM_GRAD_APPLY, M->optParams, stream);
+        }
+        CK(ts2_matrix_row_sum2(o.xSize, o.ySize, W.delta.P(), o.gradRowSum2, stream));
+        CK(ts2_update_global_row_disp(o.xSize, o.ySize, o.rowDispSize, o.gradRowSum2, M->optParams, o.sumWeight, o.rowDisp, o.rowScale, stream));
+        CK(ts2_add_gradient(o.xSize, o.ySize, W.delta.P(), M->optParams, o.rowScale, o.sparsity, &o.avgGrad, &o.weights, o.weightsRowSum2, stream));
+        return ts2_convert_matrix(o.xSize, o.ySize, o.yBufSize, o.xSize, o.ySize, &o.weights, o.weightsRowSum2, &o.fast, o.fastType, o.matrixScale,
+            o.convertMult, stream);
+    };
+    CK(apply(M->embed, false));
+    CK(apply(M->finalW, true));
+    for (TLayer &L : M->layers) {
+        for (int k = 0; k < 5; ++k) {
+            if (L.w[k].fast.m.ptr) {
+                CK(apply(L.w[k], true));
+            }
+        }
+    }
+    return 0;
+}
+
+// host copy of a matrix's master weights [rows][cols] (synchronises the device)
+extern "C" int ts2_model_get_master(ts2_model *M, int32_t layer, int32_t matrixId, float *hostOut, int32_t rows, int32_t cols)
+{
+    TMatrix *W = M ? FindMatrix(M, layer, matrixId) : nullptr;
+    if (!W || !hostOut) {
+        return TS2_ERR_NULL;
+    }
+    if (!W->hasOpt || rows != W->optRows || cols != W->srcDim) {
+        return TS2_ERR_SHAPE;
+    }
+    if (hipDeviceSynchronize() != hipSuccess ||
+        Copy2D(hostOut, (size_t)cols * 4, W->optWeights.m.ptr, W->optWeights.m.strideBytes, (size_t)cols * 4, rows, hipMemcpyDeviceToHost) != hipSuccess) {
+        return TS2_ERR_LAUNCH;
+    }
+    return 0;
+}
+
+// host copy of a matrix's fast weights [rows][cols] bytes and its scale (synchronises the device)
+extern "C" int ts2_model_get_matrix(ts2_model *M, int32_t layer, int32_t matrixId, void *fastHostOut, int32_t rows, int32_t cols, float *scaleOut)
+{
+    TMatrix *W = M ? FindMatrix(M, layer, matrixId) : nullptr;
+    if (!W || !fastHostOut || !scaleOut) {
+        return TS2_ERR_NULL;
+    }
+    if (cols != W->srcDim || rows > W->dstDim * W->slabs) {
+        return TS2_ERR_SHAPE;
+    }
+    if (hipDeviceSynchronize() != hipSuccess ||
+        Copy2D(fastHostOut, cols, W->fast.m.ptr, W->fast.m.strideBytes, cols, rows, hipMemcpyDeviceToHost) != hipSuccess ||
+        hipMemcpy(scaleOut, W->scale, 4, hipMemcpyDeviceToHost) != hipSuccess) {
+        return TS2_ERR_LAUNCH;
+    }
     return 0;
 }
 

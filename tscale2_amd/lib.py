@@ -287,6 +287,10 @@ class ModelConfig(C.Structure):
                 ("labelCount", C.c_int32), ("maxLen", C.c_int32), ("kTile", C.c_int32), ("recompute", C.c_int32)]
 
 
+class AddGradientParams(C.Structure):
+    _fields_ = [(n, C.c_float) for n in ("dispDecay", "beta1", "weight0", "weight1", "l2Reg", "stepMult")]
+
+
 LAYER_EMBED, LAYER_FINAL = -1, -2
 
 
@@ -324,6 +328,32 @@ class Model:
         fast = np.ascontiguousarray(fast)
         self._ck(self.lib.dll.ts2_model_set_matrix(self.h, layer, matrix_id, fast.ctypes.data_as(C.c_void_p), fast.shape[0], fast.shape[1],
                                                    C.c_float(scale)), "ts2_model_set_matrix")
+
+    def set_master(self, layer, matrix_id, weights, row_disp_size, sparsity=1.0):
+        """fp32 master weights of a matrix (optimiser state is created on first use); the fast weights are derived on the device"""
+        import numpy as np
+        w = np.ascontiguousarray(weights, np.float32)
+        self._ck(self.lib.dll.ts2_model_set_master(self.h, layer, matrix_id, w.ctypes.data_as(C.c_void_p), w.shape[0], w.shape[1], row_disp_size,
+                                                   C.c_float(sparsity)), "ts2_model_set_master")
+
+    def apply_deltas(self, rate, l2_reg=0.0, beta1=0.0, weight0=1.0, weight1=0.0, disp_decay=0.9):
+        """one optimiser step with the deltas of the last backprop (TTrainingStep fields)"""
+        p = AddGradientParams(disp_decay, beta1, weight0, weight1, l2_reg, rate)
+        self._ck(self.lib.dll.ts2_model_apply_deltas(self.h, C.byref(p), self.lib.stream()), "ts2_model_apply_deltas")
+
+    def get_master(self, layer, matrix_id, rows, cols):
+        import numpy as np
+        out = np.empty((rows, cols), np.float32)
+        self._ck(self.lib.dll.ts2_model_get_master(self.h, layer, matrix_id, out.ctypes.data_as(C.c_void_p), rows, cols), "ts2_model_get_master")
+        return out
+
+    def get_matrix(self, layer, matrix_id, rows, cols, dtype):
+        """fast weights (bytes of the model's 8-bit type) and the matrix scale"""
+        import numpy as np
+        out = np.empty((rows, cols), dtype)
+        sc = C.c_float(0)
+        self._ck(self.lib.dll.ts2_model_get_matrix(self.h, layer, matrix_id, out.ctypes.data_as(C.c_void_p), rows, cols, C.byref(sc)), "ts2_model_get_matrix")
+        return out, sc.value
 
     def set_bias(self, bias):
         import numpy as np
