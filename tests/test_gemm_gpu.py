@@ -394,3 +394,35 @@ def test_weight_slab_chosen_per_row_tile_is_bit_exact(lib, orc):
             assert np.all(got[rows] == -7)
         else:
             assert np.array_equal(got[rows], orc_gemm_i8(orc, np.ascontiguousarray(a[rows]), np.ascontiguousarray(b[g * n:(g + 1) * n])))
+
+
+@pytest.mark.parametrize("zero_at", [(0,), (1,), (3,), (1, 2), (0, 1, 2, 3)])
+def test_products_with_a_zero_factor_contribute_nothing(zero_at):
+    """a device-resident factor of zero (the scale of an all-zero matrix) on any of the products of a one-launch sum: the product is
+    skipped, the others keep their sum - no 0 * inf from rescaling to a zero factor"""
+    print("case several products, zero factors at", zero_at, flush=True)
+    from tscale2_amd import lib as L
+    lib = L.load()
+    m, n, k, nseg = 512, 512, 256, 4
+    g = torch.Generator(device="cuda").manual_seed(13)
+    mk = lambda r, c: (torch.randn((r, c), device="cuda", generator=g) * 6).to(torch.float8_e4m3fn).view(torch.uint8)
+    As = [mk(m, k) for _ in range(nseg)]; Bs = [mk(n, k) for _ in range(nseg)]
+    ptrs = [torch.full((1,), 0.0 if i in zero_at else 0.5 + 0.3 * i, device="cuda") for i in range(nseg)]
+    want = torch.zeros((m, n), device="cuda")
+    for i in range(nseg):
+        lib.gemm_nt(As[i], Bs[i], want, L.E4M3, L.F32, alpha=0.25, alpha_ptr=ptrs[i], tile_config=1, epilogue=L.EPI_ADD)
+    got = torch.full((m, n), 3.0, device="cuda")
+    lib.gemm_nt(As[0], Bs[0], got, L.E4M3, L.F32, alpha=0.25, alpha_ptr=ptrs[0], segments=[(As[i], Bs[i], 0.25, ptrs[i]) for i in range(1, nseg)])
+    torch.cuda.synchronize()
+    assert torch.isfinite(got).all()
+    assert (got - want).abs().max().item() <= 4e-6 * max(want.abs().max().item(), 1e-30)
+    # the 128x128 tile with one further product
+    for za in ((0,), (1,), (0, 1)):
+        p2 = [torch.full((1,), 0.0 if i in za else 0.7, device="cuda") for i in range(2)]
+        want2 = torch.zeros((m, n), device="cuda")
+        for i in range(2):
+            lib.gemm_nt(As[i], Bs[i], want2, L.E4M3, L.F32, alpha=0.5, alpha_ptr=p2[i], tile_config=2, epilogue=L.EPI_ADD)
+        got2 = torch.full((m, n), 3.0, device="cuda")
+        lib.gemm_nt(As[0], Bs[0], got2, L.E4M3, L.F32, alpha=0.5, alpha_ptr=p2[0], tile_config=2, segments=[(As[1], Bs[1], 0.5, p2[1])])
+        torch.cuda.synchronize()
+        assert torch.isfinite(got2).all() and (got2 - want2).abs().max().item() <= 4e-6 * max(want2.abs().max().item(), 1e-30), za

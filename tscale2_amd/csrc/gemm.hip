@@ -888,6 +888,7 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN) / 4) GemmNTDirect(Gemm
         }                                                                                                                                  \
     } while (0)
 
+    float segUnits = 0; // SEG: the one factor the epilogue applies
     for (int seg = 0; seg < (SEG ? 2 : 1); ++seg) {
     if (SEG && seg == 1) {
         gaTile = p.segA[0] + aTileOff;
@@ -912,7 +913,8 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN) / 4) GemmNTDirect(Gemm
     }
     if constexpr (SEG && TYPE != T_I8) {
         if (seg == 0) {
-            // the epilogue applies the second product's factor to the sum: bring the first product to that scale
+            // the epilogue applies one factor to the sum: the second product's, unless that is zero (an all-zero matrix has scale 0; the
+            // product then contributes nothing and is skipped, and the first product's factor stays)
             float cur = p.alpha, nxt = p.segAlpha[0];
             if (p.alphaPtr) {
                 cur *= *p.alphaPtr;
@@ -920,14 +922,22 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN) / 4) GemmNTDirect(Gemm
             if (p.segAlphaPtr[0]) {
                 nxt *= *p.segAlphaPtr[0];
             }
-            const float ratio = cur / nxt;
+            segUnits = cur;
+            if (nxt == 0) {
+                __syncthreads();
+                break;
+            }
+            segUnits = nxt;
+            if (cur != nxt) {
+                const float ratio = cur / nxt;
 #pragma unroll
-            for (int i = 0; i < WTM; ++i) {
+                for (int i = 0; i < WTM; ++i) {
 #pragma unroll
-                for (int j = 0; j < WTN; ++j) {
+                    for (int j = 0; j < WTN; ++j) {
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) {
-                        acc[i][j][e] *= ratio;
+                        for (int e = 0; e < 16; ++e) {
+                            acc[i][j][e] *= ratio;
+                        }
                     }
                 }
             }
@@ -935,9 +945,9 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN) / 4) GemmNTDirect(Gemm
         }
     }
     } // products
-    if (SEG) {
-        p.alpha = p.segAlpha[0];
-        p.alphaPtr = p.segAlphaPtr[0];
+    if constexpr (SEG && TYPE != T_I8) {
+        p.alpha = segUnits;
+        p.alphaPtr = nullptr;
     }
 #undef STEP
 #undef LOAD_FRAGS
@@ -1124,13 +1134,44 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(256, 1) G
     static_assert(LA == 8 && LB == 8, "vmcnt immediate below assumes eight loads per operand stage");
     // several products into the same accumulators: one pass of the pipeline per product (the stage rotation restarts), the fp32 sums
     // rescaled in between so that the epilogue's single factor, the last product's, is right for all of them
+    // `units`: the factor the accumulators have to be multiplied with in the end = the factor of the product that ran last.  A product
+    // whose factor is zero (an all-zero matrix has scale 0) contributes nothing and is skipped: rescaling the earlier sums to a zero
+    // factor would turn them into infinities.
+    float units = 0;
     for (int seg = 0; seg < p.nSeg; ++seg) {
     if (seg > 0) {
         // (constant subscripts only: a variable one would move the whole parameter block to private memory)
         gaTile = (seg == 1 ? p.segA[0] : seg == 2 ? p.segA[1] : p.segA[2]) + aTileOff;
         gbTile = (seg == 1 ? p.segB[0] : seg == 2 ? p.segB[1] : p.segB[2]) + bTileOff;
     }
-    if (kSteps > 0) {
+    bool skip = false;
+    if constexpr (TYPE != T_I8) {
+        if (p.nSeg > 1) {
+            float f = seg == 0 ? p.alpha : seg == 1 ? p.segAlpha[0] : seg == 2 ? p.segAlpha[1] : p.segAlpha[2];
+            const float *fPtr = seg == 0 ? p.alphaPtr : seg == 1 ? p.segAlphaPtr[0] : seg == 2 ? p.segAlphaPtr[1] : p.segAlphaPtr[2];
+            if (fPtr) {
+                f *= *fPtr;
+            }
+            skip = f == 0;
+            if (!skip) {
+                if (units != 0 && units != f) {
+                    const float ratio = units / f;
+#pragma unroll
+                    for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+                        for (int j = 0; j < WTN; ++j) {
+#pragma unroll
+                            for (int e = 0; e < 16; ++e) {
+                                acc[i][j][e] *= ratio;
+                            }
+                        }
+                    }
+                }
+                units = f;
+            }
+        }
+    }
+    if (kSteps > 0 && !skip) {
         RING_LOAD_A(sA0, 0, 0, LA);
         RING_LOAD_B(sB0, 0, 0, LB);
         RING_LOAD_A(sA1, 1, 0, LA);
@@ -1166,37 +1207,12 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(256, 1) G
     }
     __builtin_amdgcn_s_waitcnt(0x0F70); // the redundant loads of the last steps
     __syncthreads();
-    if constexpr (TYPE != T_I8) {
-        if (seg + 1 < p.nSeg) {
-            float cur = seg == 0 ? p.alpha : seg == 1 ? p.segAlpha[0] : p.segAlpha[1];
-            const float *curPtr = seg == 0 ? p.alphaPtr : seg == 1 ? p.segAlphaPtr[0] : p.segAlphaPtr[1];
-            float nxt = seg == 0 ? p.segAlpha[0] : seg == 1 ? p.segAlpha[1] : p.segAlpha[2];
-            const float *nxtPtr = seg == 0 ? p.segAlphaPtr[0] : seg == 1 ? p.segAlphaPtr[1] : p.segAlphaPtr[2];
-            if (curPtr) {
-                cur *= *curPtr;
-            }
-            if (nxtPtr) {
-                nxt *= *nxtPtr;
-            }
-            const float ratio = cur / nxt;
-#pragma unroll
-            for (int i = 0; i < WTM; ++i) {
-#pragma unroll
-                for (int j = 0; j < WTN; ++j) {
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) {
-                        acc[i][j][e] *= ratio;
-                    }
-                }
-            }
-        }
-    }
     } // products
-    if (p.nSeg > 1) {
-        const float lastAlpha = p.nSeg == 2 ? p.segAlpha[0] : p.nSeg == 3 ? p.segAlpha[1] : p.segAlpha[2];
-        const float *lastPtr = p.nSeg == 2 ? p.segAlphaPtr[0] : p.nSeg == 3 ? p.segAlphaPtr[1] : p.segAlphaPtr[2];
-        p.alpha = lastAlpha;
-        p.alphaPtr = lastPtr;
+    if constexpr (TYPE != T_I8) {
+        if (p.nSeg > 1) {
+            p.alpha = units;
+            p.alphaPtr = nullptr;
+        }
     }
 #undef STEP
 #undef RING_BARRIER
