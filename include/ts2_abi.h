@@ -580,6 +580,45 @@ int ts2_model_array(ts2_model *m, const char *name, int32_t index, ts2_mat *out,
 int ts2_model_read(ts2_model *m, const char *name, int32_t index, void *hostOut, int64_t hostBytes);
 int ts2_model_scalars(ts2_model *m, float *lossSumHost, int32_t *lenRound, int32_t *lenMoe);
 
+/* ------------------------------------------------------------------------------------------------------------------------
+ * Checkpoint and weight-exchange formats (host side; no device work).
+ * ts2_checkpoint_parse reads the bytes of a TModelParams as the reference's SAVELOAD writes them (src/gpt/model_params/model_params.h:7-18,
+ * model_matrix.h:61-70, model_dim.h:118-178 through src/util/bin_saver.h) and returns NULL when they do not parse exactly;
+ * ts2_checkpoint_write produces the same bytes again (returns the byte count, also when out is NULL or cap too small: nothing beyond
+ * cap is written).  Matrices: layer = -1 addresses the model-level ones (0 = embedding MP_MODEL_EMBED, 1 = final MP_MODEL_FINAL,
+ * model_dim.h:84-86), otherwise a layer's in the order of EnumLayerMatrices (model_dim.h:225-262).  The views point into the
+ * checkpoint object and live as long as it does; weights / avgGrad are [ySize][xSize] floats (Matr, Grad1), rowDispSize is 1 or ySize. */
+typedef struct ts2_checkpoint ts2_checkpoint;
+typedef struct ts2_checkpoint_info {
+    int32_t dim, qDim, ttDim, expertDim, headCount, ffnTiles, moeExpertCount, moeSelected, kvRep, depth; /* TModelDims */
+    int64_t labelCount, inputTokenCount, outputTokenCount;
+    int32_t attTypeCount, layerCount;
+    uint64_t flags, docStartToken;
+    int64_t fragLen;
+    int32_t biasCount;
+    const float *bias;
+} ts2_checkpoint_info;
+typedef struct ts2_checkpoint_matrix_view {
+    int32_t xSize, ySize;
+    const float *weights, *avgGrad;
+    float sumWeight;
+    const float *rowDisp;
+    int32_t rowDispSize;
+    float sparsity;
+} ts2_checkpoint_matrix_view;
+ts2_checkpoint *ts2_checkpoint_parse(const void *bytes, int64_t size);
+void ts2_checkpoint_free(ts2_checkpoint *c);
+int64_t ts2_checkpoint_write(const ts2_checkpoint *c, void *out, int64_t cap);
+int ts2_checkpoint_get_info(const ts2_checkpoint *c, ts2_checkpoint_info *out);
+int ts2_checkpoint_att_type(const ts2_checkpoint *c, int32_t id, int32_t *width, int32_t *type);
+int ts2_checkpoint_layer(const ts2_checkpoint *c, int32_t layer, int32_t *layerType, float *alibiSlope, int32_t *attTypeId, int32_t *matrixCount);
+int ts2_checkpoint_matrix(const ts2_checkpoint *c, int32_t layer, int32_t matrixId, ts2_checkpoint_matrix_view *out);
+/* PackMatrix / AddPackedMatrix, src/gpt/model_params/model_matrix.cpp:6-58: the fp16-row format in which weights travel between
+ * workers: per row a float rms, then (unless it is 0) xSize IEEE halves of row / rms; xSize a multiple of 16.
+ * ts2_pack_matrix_fp16 returns the byte count (also when out is NULL or cap too small); ts2_add_packed_matrix_fp16 adds scale * matrix. */
+int64_t ts2_pack_matrix_fp16(const float *matr, int32_t xSize, int32_t ySize, void *out, int64_t cap);
+int ts2_add_packed_matrix_fp16(float *matr, int32_t xSize, int32_t ySize, const void *in, int64_t size, float scale);
+
 /* peak dense MFMA rate the library prices its kernels against, in T(FL)OP/s, and the CU count it tiles for */
 int ts2_device_info(int *cuCount, int *clockMHz);
 

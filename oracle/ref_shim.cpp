@@ -21,6 +21,8 @@
 #include <gpt/model_params/sse_utils.h>
 #include <util/fp8.h>
 #include <lib/random/mersenne.h>
+#include <util/mem_io.h>
+#include <gpt/model_params/model_params.h>
 
 static void ToArr(TArray2D<float> *p, const float *src, yint ySize, yint xSize)
 {
@@ -285,6 +287,113 @@ void ref_mersenne_real3(unsigned seed, int n, float *out)
     for (int i = 0; i < n; ++i) {
         out[i] = (float)rng.GenRandReal3();
     }
+}
+
+
+// a checkpoint as the reference writes it: a TModelParams laid out like AllocateModel does (src/gpt/model_params/model_params.cpp:142-163)
+// for a model string, every matrix filled from a small deterministic generator (InitModel's threads are not needed for the format), the
+// optimiser state of one matrix set, serialised with SAVELOAD (TModelParams, model_params.h:7-18) into memory.
+// Returns the byte count (or -needed when cap is too small).
+static float CkValue(unsigned *state)
+{
+    *state = *state * 1664525u + 1013904223u;
+    return ((int)(*state >> 8) % 2001 - 1000) * (1.f / 1024);
+}
+
+static void CkFill(TModelMatrix *mm, unsigned *state)
+{
+    TArray2D<float> a, g;
+    a.SetSizes(mm->GetXSize(), mm->GetYSize());
+    g.SetSizes(mm->GetXSize(), mm->GetYSize());
+    for (yint y = 0; y < mm->GetYSize(); ++y) {
+        for (yint x = 0; x < mm->GetXSize(); ++x) {
+            a[y][x] = CkValue(state);
+            g[y][x] = CkValue(state) * 0.25f;
+        }
+    }
+    mm->SetMatrix(a);
+    mm->GetGrad1() = g;
+}
+
+long ref_make_checkpoint(const char *descr, int vocab, unsigned seed, char *out, long cap)
+{
+    TModelDescr md;
+    InitModelDescr(&md, descr, vocab, vocab, MPF_DISABLE_NOISE_LABELS);
+    TModelParams params;
+    params.ModelDescr = md;
+    yint dim = md.Dims.Dim;
+    params.MatrArr.resize(MP_MODEL_COUNT);
+    params.MatrArr[MP_MODEL_EMBED].SetSizesPerRowDisp(dim, md.LabelCount, 1);
+    params.MatrArr[MP_MODEL_FINAL].SetSizesPerRowDisp(dim, md.OutputTokenCount, 1);
+    yint depth = YSize(md.LayerArr);
+    params.LayerArr.resize(depth);
+    for (yint d = 0; d < depth; ++d) {
+        TModelParams::TAttentionMatrices &dst = params.LayerArr[d];
+        dst.MatrArr.resize(MP_MAX_COUNT);
+        yint ptr = 0;
+        md.EnumLayerMatrices(d, [&](yint xSize, yint ySize, float noise, float moeFraction) {
+            dst.MatrArr[ptr++].SetSizesPerMatrixDisp(xSize, ySize, moeFraction);
+        });
+        dst.MatrArr.resize(ptr);
+    }
+    unsigned state = seed;
+    params.ForEachModelMatrix([&](TModelMatrix &mm) { CkFill(&mm, &state); });
+    params.Bias.resize(vocab);
+    for (int k = 0; k < vocab; ++k) {
+        params.Bias[k] = 0.01f * k;
+    }
+    {
+        TVector<float> rd(params.MatrArr[MP_MODEL_FINAL].GetRowDisp().size(), 0.f);
+        for (yint k = 0; k < YSize(rd); ++k) {
+            rd[k] = 0.125f + k;
+        }
+        params.MatrArr[MP_MODEL_FINAL].SetRowDisp(2.5f, rd);
+        params.LayerArr[0].MatrArr[0].SetRowDisp(1.5f, TVector<float>(1, 0.75f));
+    }
+    TVector<char> data;
+    SerializeMem(IO_WRITE, &data, params);
+    if ((long)data.size() > cap) {
+        return -(long)data.size();
+    }
+    memcpy(out, data.data(), data.size());
+    return (long)data.size();
+}
+
+// PackMatrix / AddPackedMatrix (src/gpt/model_params/model_matrix.cpp:6-58): the fp16-row wire format
+long ref_pack_matrix(const float *matr, int xSize, int ySize, char *out, long cap)
+{
+    // (the AVX code of the reference reads and writes rows with aligned accesses)
+    float *m = (float *)aligned_alloc(64, sizeof(float) * xSize * ySize);
+    memcpy(m, matr, sizeof(float) * xSize * ySize);
+    TVector<char> data;
+    {
+        TMemStream f(&data);
+        {
+            TBufferedStream bufIO(IO_WRITE, f);
+            PackMatrix(bufIO, THost2DPtr<float>(m, xSize * sizeof(float), xSize, ySize));
+        }
+        f.Swap(&data);
+    }
+    free(m);
+    if ((long)data.size() > cap) {
+        return -(long)data.size();
+    }
+    memcpy(out, data.data(), data.size());
+    return (long)data.size();
+}
+
+void ref_add_packed_matrix(float *matr, int xSize, int ySize, const char *in, long size, float scale)
+{
+    float *m = (float *)aligned_alloc(64, sizeof(float) * xSize * ySize);
+    memcpy(m, matr, sizeof(float) * xSize * ySize);
+    TVector<char> data(in, in + size);
+    {
+        TMemStream f(&data);
+        TBufferedStream bufIO(IO_READ, f);
+        AddPackedMatrix(THost2DPtr<float>(m, xSize * sizeof(float), xSize, ySize), bufIO, scale);
+    }
+    memcpy(matr, m, sizeof(float) * xSize * ySize);
+    free(m);
 }
 
 }
