@@ -298,7 +298,7 @@ def bandwidth_kernels(iters=10):
     return res
 
 
-def fp8_backward_gemms(n, dim, ffn, iters=10):
+def fp8_backward_gemms(n, dim, ffn, iters=10, only_dominant=False):
     """the e4m3 backward GEMM shapes of the dense step, each timed alone with events: dX of the FFN contract / expand matrices,
     the FFN delta (packed-delta epilogue) and the attention-width dX"""
     import torch
@@ -321,6 +321,8 @@ def fp8_backward_gemms(n, dim, ffn, iters=10):
                     "frac_of_peak": round(ops / (ms * 1e-3) / PEAK_FP8, 3)})
         return ms, ops
     first = run("dX: dY[tokens x ffn] x W^T (FFN expand / gate), fp32 result", n, dim, ffn)
+    if only_dominant:
+        return out, first
     run("dX: dY[tokens x dim] x W^T (FFN contract), fp32 result", n, ffn, dim)
     run("dX: dY[tokens x dim] x W^T (attention Q/K/V/gate/combiner), fp32 result", n, dim, dim)
     run("delta: dY^T[ffn x tokens] x X^T (FFN expand / gate), packed i8 result", ffn, dim, n, packed=True)
@@ -387,7 +389,7 @@ def bench_step_fp8(args):
     flop = 6.0 * params * n + att
     # dominant kernel: the e4m3 GEMM, timed alone with events on the launch stream at the model's backward shapes; the roofline line is
     # the biggest of them (dX of the FFN expand / gate matrices: M = tokens, K = ffn, N = dim)
-    gemms, (ms_g, gops) = fp8_backward_gemms(n, dim, ffn)
+    gemms, (ms_g, gops) = fp8_backward_gemms(n, dim, ffn, only_dominant=args.no_extras)
     roof = {"bound": "mfma", "achieved": gops / (ms_g * 1e-3) / 1e12, "peak": PEAK_FP8 / 1e12, "unit": "TFLOP/s",
             "frac": gops / (ms_g * 1e-3) / PEAK_FP8, "traffic": None if args.small else profile_traffic("gemm_fp8_32768x2048x8192_hbm_traffic.txt"),
             "kernel": "GemmNTRing<e4m3> %dx%dx%d (%.1f us per launch, %.2f GOP)" % (n, dim, ffn, ms_g * 1e3, gops / 1e9)}
@@ -402,6 +404,8 @@ def bench_step_fp8(args):
     m.close()
     del m
     torch.cuda.empty_cache()
+    if args.no_extras:
+        return out
     # the second half of the metric: the int8 backward GEMMs of the linear-layer microbenchmark, in the same run
     c1 = linear_i8_setup(args.delta_splits)
     c1["step"]()
@@ -643,6 +647,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--delta-splits", type=int, default=2, help="linear_i8_bwd: slices of the token axis in the delta product (1 = single pass)")
     ap.add_argument("--sort-rows", action="store_true", help="linear_i8_bwd: sort the gradient rows by scale before the delta product (the reference's order)")
+    ap.add_argument("--no-extras", action="store_true", help="step_fp8: only the step and its dominant GEMM (no int8 GEMMs, bandwidth kernels, device "
+                                                              "probes or CPU leg): the command a kernel trace of the step is taken on")
     ap.add_argument("--small", action="store_true", help="step_fp8 / moe_fp8: a reduced model for quick checks (not a valid benchmark figure)")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -213,10 +213,11 @@ __device__ __forceinline__ TRowSpan MakeRowSpan(int start, int finish)
     b = WaveMinInt(b);
     c = WaveMinInt(c);
     d = WaveMaxInt(d);
-    r.waveMaxStart = a;
-    r.waveMinFinish = b;
-    r.waveMinStart = c;
-    r.waveMaxFinish = d;
+    // the same in every lane: held as scalars, so that the tests on them are uniform branches
+    r.waveMaxStart = __builtin_amdgcn_readfirstlane(a);
+    r.waveMinFinish = __builtin_amdgcn_readfirstlane(b);
+    r.waveMinStart = __builtin_amdgcn_readfirstlane(c);
+    r.waveMaxFinish = __builtin_amdgcn_readfirstlane(d);
     return r;
 }
 
@@ -605,7 +606,7 @@ template <bool F32> __global__ void __launch_bounds__(256) AttGradKV(AttP p)
         if (t0 + TR <= qHi) {
             prefetch(t0 + TR, slot ^ 1);
         }
-        const int kw0 = myRow - l32; // first key of this wave
+        const int kw0 = __builtin_amdgcn_readfirstlane(myRow - l32); // first key of this wave
         if (stT[3] < kw0 || stT[2] > kw0 + 31) {
             continue; // no query of the tile sees a key of this wave (wave-uniform)
         }
@@ -747,6 +748,565 @@ __global__ void RevBuild(const int *spanStart, const int *spanFinish, int len, i
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------------------
+// Backward kernels, two workgroups per CU.
+//
+// The streamed tiles (64 rows x 256 bytes) go global -> LDS with global_load_lds_dwordx4 into two buffers used in turn: no staging
+// registers, no ds_write, one barrier per tile.  Rows are unpadded; the 16-byte chunks of a row are XOR-swizzled by
+// Swz(row) = 4 * (row % 4) + (row / 4) % 4, which makes both kinds of operand fetch bank-conflict free:
+//   * row-major fragments (contraction over d): ds_read_b128, 16 consecutive rows at one chunk column -> 16 different chunks;
+//   * transposed fragments (contraction over the tile's rows): ds_read_b64_tr_b16 straight from the row-major tile.  Inside each group
+//     of 16 lanes the instruction hands lane j, element e the 16-bit value number j % 4 of the 8 bytes addressed by lane 4 * e + j / 4;
+//     with lane i pointing at row i / 4, columns 4 * (i % 4) .. + 3 of a 4 x 16 block, lane j receives column j of rows 0..3: the four
+//     contraction slots of an MFMA A operand.  A half wave touches 4 rows x 64 bytes, which the swizzle spreads over all 64 banks.
+// The wave's own rows (the B operands of the products that contract over d) stay in registers for the whole kernel, so every MFMA
+// costs one 1 KB operand fetch from LDS.  All of this fits 256 registers and 64-67 KB of LDS: two workgroups share a CU, and the
+// exponentials and conversions of one wave run under the products of the other.
+constexpr int ROWB = HD * 2;           // bytes of a tile row
+constexpr int TILE_BYTES = TR * ROWB;  // 16 KB
+
+typedef short v4s16 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ int Swz(int row)
+{
+    return ((row & 3) << 2) | ((row >> 2) & 3);
+}
+
+// the lane index, computed where it is asked for (the volatile asm keeps the computation, and everything derived from it, from
+// being moved out of a loop and held in registers across it)
+__device__ __forceinline__ int FreshLaneId()
+{
+    int lane;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane));
+    return lane;
+}
+
+// Direct tile load: a wave-level load fills 4 consecutive tile rows (1 KB); wave w issues the loads of row groups w, w + 4, w + 8,
+// w + 12, whose Swz depends on the lane and on w only.  Buffer addressing: the tile's first row is the base of a descriptor held
+// in scalar registers, a lane adds one 32-bit offset and the row group a scalar one, so a load costs no 64-bit vector arithmetic and
+// no address registers outlive it (the lane index is obtained on the spot for the same reason).  Reads past the 64 rows of the
+// descriptor would return zeros instead of touching memory.
+__device__ __forceinline__ void LoadTileDirect(uint8_t *tile, const uint8_t *g, int64_t ld, int wave)
+{
+    const int lane = FreshLaneId();
+    const int lrow = lane >> 4;
+    const int chunk = (lane & 15) ^ ((lrow << 2) | wave);
+    const int laneOff = lrow * (int)ld + chunk * 16;
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)g, 0, TR * (int)ld, 0x00020000);
+#pragma unroll
+    for (int i = 0; i < TR / 16; ++i) {
+        const int u = wave + 4 * i;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, TS2_LDS_PTR(tile + u * 1024), 16, laneOff, 4 * u * (int)ld, 0, 0);
+    }
+}
+
+// Operand fetches take (tile, compile-time offset) + a per-lane byte offset that is computed once per kernel and made opaque to the
+// optimiser: the tile address and the constant part then fold into the instruction's offset field, and a kernel keeps 8 + 8 address
+// registers for all of its fetches instead of one per (buffer, block, step).
+typedef const __attribute__((address_space(3))) uint8_t *TLdsBytes;
+
+struct TFragLane {
+    int row[4];   // FragRow, ds = 0..3: l32 * ROWB + (((2 * ds) ^ Swz(l32) ^ half) << 4)
+    int rowHi;    // ds = 4..7 flips bit 3 of the chunk: row[ds - 4] + rowHi, rowHi = +-128
+    int trLo[4];  // FragTr, slots 0..3 of column block db
+    int trHi;     // slots 4..7 (8 rows further down, chunk ^ 2): trLo[db] + trHi
+};
+
+__device__ __forceinline__ TFragLane MakeFragLane(int lane)
+{
+    const int l32 = lane & 31, half = lane >> 5;
+    const int swzLane = Swz(l32) ^ half;
+    TFragLane f;
+#pragma unroll
+    for (int ds = 0; ds < 4; ++ds) {
+        f.row[ds] = l32 * ROWB + (((2 * ds) ^ swzLane) << 4);
+        asm volatile("" : "+v"(f.row[ds]));
+    }
+    f.rowHi = (swzLane & 8) ? -128 : 128;
+    asm volatile("" : "+v"(f.rowHi));
+    // transposed fetch: inside a group of 16 lanes, lane i points at row i / 4, columns 4 * (i % 4) .. + 3 of the group's 4 x 16 block;
+    // the two groups of a half wave sit side by side (32 columns), the halves of the wave 4 rows apart
+    const int g = lane >> 4, i = lane & 15, h = g >> 1, dsub = g & 1, r = i >> 2, c4 = i & 3;
+    const int base = (4 * h + r) * ROWB + 8 * (c4 & 1);
+    const int cl = (2 * dsub + (c4 >> 1)) ^ h;
+#pragma unroll
+    for (int db = 0; db < 4; ++db) {
+        const int blk = (db ^ r) << 2;
+        f.trLo[db] = base + ((blk | cl) << 4);
+        asm volatile("" : "+v"(f.trLo[db]));
+    }
+    f.trHi = 8 * ROWB + (((cl ^ 2) - cl) << 4);
+    asm volatile("" : "+v"(f.trHi));
+    return f;
+}
+
+// A operand, contraction over d: lane row = rb * 32 + l32, d = ds * 16 + half * 8 .. + 7
+__device__ __forceinline__ v8bf FragRow(const uint8_t *tile, int rb, int ds, const TFragLane &f)
+{
+    TLdsBytes b = (TLdsBytes)TS2_LDS_PTR(tile) + rb * 32 * ROWB;
+    const int off = ds < 4 ? f.row[ds] : f.row[ds - 4] + f.rowHi;
+    return __builtin_bit_cast(v8bf, *(const __attribute__((address_space(3))) v4i *)(b + off));
+}
+
+// A operand, contraction over tile rows: lane row = d = db * 32 + l32; slots = tile rows rb * 32 + 16 * ks + 4 * half + {0..3} and + 8
+__device__ __forceinline__ v8bf FragTr(const uint8_t *tile, int rb, int ks, int db, const TFragLane &f)
+{
+    typedef __attribute__((address_space(3))) v4s16 *TTrPtr;
+    TLdsBytes b = (TLdsBytes)TS2_LDS_PTR(tile) + (rb * 32 + 16 * ks) * ROWB;
+    v4s16 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TTrPtr)(b + f.trLo[db]));
+    v4s16 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TTrPtr)(b + (f.trLo[db] + f.trHi)));
+    typedef short v8s16 __attribute__((ext_vector_type(8)));
+    v8s16 r = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return __builtin_bit_cast(v8bf, r);
+}
+
+// the wave's own rows as B operands: lane row = l32, d = ds * 16 + half * 8 .. + 7
+__device__ __forceinline__ void LoadOwnFrags(v8bf (&f)[8], const uint8_t *g, int64_t ld, int l32, int half)
+{
+#pragma unroll
+    for (int ds = 0; ds < 8; ++ds) {
+        f[ds] = __builtin_bit_cast(v8bf, *(const v4i *)(g + (int64_t)l32 * ld + (ds * 16 + half * 8) * 2));
+    }
+}
+
+// workgroup ids are handed to the 8 XCDs in turn: remap them so that an XCD works on consecutive blocks of one head (the rows they
+// stream overlap, and so stay in that XCD's L2)
+__device__ __forceinline__ void MapAttBlock(int *blk, int *head)
+{
+    const int nbx = gridDim.x, nb = nbx * gridDim.y, bid = blockIdx.x + blockIdx.y * nbx;
+    const int id = (nb & 7) == 0 ? (bid & 7) * (nb >> 3) + (bid >> 3) : bid;
+    *head = id / nbx;
+    *blk = id - *head * nbx;
+}
+
+// dQ: grid (lenRound/128, heads); a wave owns 32 query rows
+template <bool F32> __global__ void __launch_bounds__(256, 2) AttGradQ2(AttP p)
+{
+    __shared__ __attribute__((aligned(1024))) uint8_t kT0[TILE_BYTES], kT1[TILE_BYTES], vT0[TILE_BYTES], vT1[TILE_BYTES];
+    __shared__ int red[8];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l32 = lane & 31, half = lane >> 5;
+    int blk, head;
+    MapAttBlock(&blk, &head);
+    // later query blocks of a causal sequence see more keys: they start first so that the short ones fill the tail of the launch
+    const int myRow = (gridDim.x - 1 - blk) * BROWS + wave * WROWS + l32;
+    const int64_t hoff = (int64_t)head * HD * 2;
+    const int start = p.spanStart[myRow], finish = p.spanFinish[myRow];
+    int kLo, kHi;
+    BlockKeyRange(start, finish, tid, &kLo, &kHi, red);
+    kLo = __builtin_amdgcn_readfirstlane(kLo);
+    kHi = __builtin_amdgcn_readfirstlane(kHi);
+    const int tFirst = kHi >= kLo ? (kLo / TR) * TR : 1;
+    const uint8_t *gk = p.k + hoff, *gv = p.v + hoff;
+    if (tFirst <= kHi) {
+        LoadTileDirect(kT0, gk + (int64_t)tFirst * p.ldk, p.ldk, wave);
+        LoadTileDirect(vT0, gv + (int64_t)tFirst * p.ldv, p.ldv, wave);
+    }
+    v8bf qf[8], of[8];
+    LoadOwnFrags(qf, p.q + (int64_t)(myRow - l32) * p.ldq + hoff, p.ldq, l32, half);
+    LoadOwnFrags(of, p.dO + (int64_t)(myRow - l32) * p.lddo + hoff, p.lddo, l32, half);
+    const float L = p.sumWeightLog[(int64_t)head * p.ldStat + myRow];
+    const float dScale = p.dScale[(int64_t)head * p.ldStat + myRow];
+    const float gmul = p.attDotScale * LN2;
+    const TRowSpan sp = MakeRowSpan(start, finish);
+    const TFragLane fl = MakeFragLane(lane);
+    // cleared from a register the optimiser cannot see through: a constant zero vector would be kept alive across the tile loop as the
+    // source of every other zero in the kernel, sixteen registers wide
+    float zero = 0;
+    asm volatile("" : "+v"(zero));
+    v16f acc[4];
+#pragma unroll
+    for (int db = 0; db < 4; ++db) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            acc[db][e] = zero;
+        }
+    }
+    // one 64-key tile: the 32-key blocks that some row of the wave sees (a run of blocks, wave-uniform bounds)
+    auto tile = [&](const uint8_t *kt, const uint8_t *vt, int t0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int kb = 0; kb < TR / 32; ++kb) {
+            const int k0 = t0 + kb * 32;
+            const uint8_t *kt2 = kt + kb * 32 * ROWB, *vt2 = vt + kb * 32 * ROWB;
+            // A block is skipped by a loop of no trips rather than by a branch around it: the accumulators are then values carried by
+            // a loop, which stay in their registers, where the join after a branch made the compiler copy all 64 of them.  The trip
+            // count is opaque to the optimiser, or it would turn the loop back into that branch.
+            int trips = __builtin_amdgcn_readfirstlane((int)!(k0 > sp.waveMaxFinish || k0 + 31 < sp.waveMinStart));
+            asm volatile("" : "+s"(trips));
+#pragma unroll 1
+            for (int trip = 0; trip < trips; ++trip) {
+            v16f s, dp;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                s[e] = 0;
+                dp[e] = 0;
+            }
+            // phase 1: S^T = K Q^T and dP^T = V dO^T; the operands of step ds + 1 are requested before the products of step ds
+            v8bf fk[2], fv[2];
+            fk[0] = FragRow(kt2, 0, 0, fl);
+            fv[0] = FragRow(vt2, 0, 0, fl);
+#pragma unroll
+            for (int ds = 0; ds < 8; ++ds) {
+                if (ds + 1 < 8) {
+                    fk[(ds + 1) & 1] = FragRow(kt2, 0, ds + 1, fl);
+                    fv[(ds + 1) & 1] = FragRow(vt2, 0, ds + 1, fl);
+                }
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fk[ds & 1], qf[ds], s, 0, 0, 0);
+                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fv[ds & 1], of[ds], dp, 0, 0, 0);
+            }
+            // the first operands of phase 3 are requested before the arithmetic of phase 2, which covers their latency
+            v8bf ft[3];
+            ft[0] = FragTr(kt2, 0, 0, 0, fl);
+            ft[1] = FragTr(kt2, 0, 0, 1, fl);
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+#pragma unroll
+            for (int ds = 0; ds < 7; ++ds) {
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+            // phase 2: dS
+            const float kc = p.slope * (float)(k0 + half * 4 - myRow) - L; // logit - L in one fma chain
+            const int rel0 = k0 + half * 4 - sp.start;
+            const bool full = k0 >= sp.waveMaxStart && k0 + 31 <= sp.waveMinFinish;
+            float dsv[16];
+            if (full) { // every row of the wave sees every key of the block: no span tests
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    float x = fmaf(s[e], p.attDotScale, fmaf(p.slope, (float)BlkRow(e, 0), kc));
+                    float w = __builtin_amdgcn_exp2f(x);
+                    dsv[e] = w * (dp[e] - dScale) * gmul;
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    float x = fmaf(s[e], p.attDotScale, fmaf(p.slope, (float)BlkRow(e, 0), kc));
+                    float w = __builtin_amdgcn_exp2f(x);
+                    w = (unsigned)(rel0 + BlkRow(e, 0)) <= sp.len ? w : 0.f;
+                    dsv[e] = w * (dp[e] - dScale) * gmul;
+                }
+            }
+            const v8bf sb[2] = {PackB(dsv, 0), PackB(dsv, 1)};
+            // phase 3: dQ^T += K^T dS^T, operands two products ahead
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                if (i + 2 < 8) {
+                    ft[(i + 2) % 3] = FragTr(kt2, 0, (i + 2) >> 2, (i + 2) & 3, fl);
+                }
+                acc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ft[i % 3], sb[i >> 2], acc[i & 3], 0, 0, 0);
+            }
+#pragma unroll
+            for (int i = 0; i < 6; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            }
+        }
+    };
+    // two tiles per trip, one per buffer, in straight-line code: the accumulators live in one set of registers throughout, and the
+    // operand reads of one buffer are known not to touch the buffer that the loads in flight fill
+    for (int t0 = tFirst; t0 <= kHi;) {
+        __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): the tile of this step has landed
+        __syncthreads();                    // ... for every wave, and every wave is done with the other buffer
+        if (t0 + TR <= kHi) {
+            LoadTileDirect(kT1, gk + (int64_t)(t0 + TR) * p.ldk, p.ldk, wave);
+            LoadTileDirect(vT1, gv + (int64_t)(t0 + TR) * p.ldv, p.ldv, wave);
+        }
+        tile(kT0, vT0, t0);
+        t0 += TR;
+        if (t0 > kHi) {
+            break;
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+        if (t0 + TR <= kHi) {
+            LoadTileDirect(kT0, gk + (int64_t)(t0 + TR) * p.ldk, p.ldk, wave);
+            LoadTileDirect(vT0, gv + (int64_t)(t0 + TR) * p.ldv, p.ldv, wave);
+        }
+        tile(kT1, vT1, t0);
+        t0 += TR;
+    }
+    StoreOwnRows<F32>(p.out0 + (int64_t)(myRow - l32) * p.ldo0, p.ldo0, head * HD, acc, 1.f, l32, half);
+}
+
+__device__ __forceinline__ int Half32MaxInt(int v)
+{
+    v = max(v, LaneDpp<DPP_XOR1>(v));
+    v = max(v, LaneDpp<DPP_XOR2>(v));
+    v = max(v, LaneDpp<DPP_HALF_MIRROR>(v));
+    v = max(v, LaneDpp<DPP_MIRROR>(v));
+    int a, b;
+    LaneSwap16(v, &a, &b);
+    return max(a, b);
+}
+
+// dK, dV: grid (lenRound/64, heads).  The workgroup owns 64 key rows and streams the query rows that reach them; its four waves are
+// two key blocks x two roles: one wave of a block accumulates dV^T += dO^T P (it needs S only), the other dK^T += Q^T dS (S and dP).
+// Both accumulators of a key block in one wave would need 128 registers and leave room for one wave per SIMD only; split, the kernel
+// recomputes S once more but runs two workgroups per CU.
+constexpr int KVROWS = 64;
+
+template <bool F32> __global__ void __launch_bounds__(256, 2) AttGradKV2(AttP p)
+{
+    __shared__ __attribute__((aligned(1024))) uint8_t qT0[TILE_BYTES], qT1[TILE_BYTES], oT0[TILE_BYTES], oT1[TILE_BYTES];
+    __shared__ __attribute__((aligned(16))) float rawStat[2][4][TR];  // [slot][L, dScale, span start, span finish][query], as loaded
+    // [slot][-L - slope * (q - keyBase), dScale, span start (0x7fffffff if empty), span length][query]: one array, one address register
+    __shared__ __attribute__((aligned(16))) float st[2][4][TR];
+    __shared__ int stT[2][2][4];                                          // [slot][32-query block]: bounds over the block's queries
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l32 = lane & 31, half = lane >> 5;
+    int block, head;
+    MapAttBlock(&block, &head);
+    // co-resident workgroups get opposite role orders, so that a SIMD is not handed two waves of the longer role
+    const int role = (wave ^ (((blockIdx.x + blockIdx.y * gridDim.x) >> 8) & 1)) & 1; // 0: dV, 1: dK
+    const int keyBase = block * KVROWS;
+    const int myRow = keyBase + (wave >> 1) * WROWS + l32; // my key
+    const int64_t hoff = (int64_t)head * HD * 2;
+    const int qLo = p.revLo[block >> 1], qHi = p.revHi[block >> 1];
+    const int tFirst = qHi >= qLo ? (qLo / TR) * TR : 1;
+    const uint8_t *gq = p.q + hoff, *go = p.dO + hoff;
+    auto loadStats = [&](int t0, int slot) __attribute__((always_inline)) {
+        if (wave == 0) {
+            const int lane = FreshLaneId();
+            const int64_t so = (int64_t)head * p.ldStat + t0 + lane;
+            __builtin_amdgcn_global_load_lds(TS2_GLB_PTR(p.sumWeightLog + so), TS2_LDS_PTR(&rawStat[slot][0][0]), 4, 0, 0);
+            __builtin_amdgcn_global_load_lds(TS2_GLB_PTR(p.dScale + so), TS2_LDS_PTR(&rawStat[slot][1][0]), 4, 0, 0);
+            __builtin_amdgcn_global_load_lds(TS2_GLB_PTR(p.spanStart + t0 + lane), TS2_LDS_PTR(&rawStat[slot][2][0]), 4, 0, 0);
+            __builtin_amdgcn_global_load_lds(TS2_GLB_PTR(p.spanFinish + t0 + lane), TS2_LDS_PTR(&rawStat[slot][3][0]), 4, 0, 0);
+        }
+    };
+    // wave 0: raw statistics of the tile at t0 (slot) -> the form the products use
+    auto digestStats = [&](int t0, int slot) __attribute__((always_inline)) {
+        if (wave == 0) {
+            // the lane index is computed afresh: a value kept from the kernel's start would hold registers (or be spilled) across the
+            // tile loop for the sake of these few instructions
+            const int lane = FreshLaneId(), l32 = lane & 31, half = lane >> 5;
+            const float rawL = rawStat[slot][0][lane];
+            int preS = __float_as_int(rawStat[slot][2][lane]), preF = __float_as_int(rawStat[slot][3][lane]);
+            const bool some = preF >= preS;
+            preS = some ? preS : 0x7fffffff;
+            preF = some ? preF : -1;
+            float *dst = &st[slot][0][lane];
+            dst[0] = -rawL - p.slope * (float)(t0 + lane - keyBase);
+            dst[TR] = rawStat[slot][1][lane];
+            dst[2 * TR] = __int_as_float(preS);
+            dst[3 * TR] = __int_as_float(some ? preF - preS : 0);
+            const int a = Half32MaxInt(preS), b = -Half32MaxInt(-preF), c = -Half32MaxInt(-preS), d = Half32MaxInt(preF);
+            if (l32 == 0) {
+                stT[slot][half][0] = a; // latest span start of the block's queries
+                stT[slot][half][1] = b; // earliest finish
+                stT[slot][half][2] = c; // earliest start
+                stT[slot][half][3] = d; // latest finish
+            }
+        }
+    };
+    if (tFirst <= qHi) {
+        loadStats(tFirst, 0);
+        if (tFirst + TR <= qHi) {
+            loadStats(tFirst + TR, 1);
+        }
+        LoadTileDirect(qT0, gq + (int64_t)tFirst * p.ldq, p.ldq, wave);
+        LoadTileDirect(oT0, go + (int64_t)tFirst * p.lddo, p.lddo, wave);
+    }
+    const float gmul = p.attDotScale * LN2;
+    const TFragLane fl = MakeFragLane(lane);
+    const int kw0 = __builtin_amdgcn_readfirstlane(myRow - l32); // first key of this wave
+    const float ck = p.slope * (float)(myRow - keyBase);
+    // the whole tile loop once per role, as separate code: no value of one role's path meets a value of the other's, and every
+    // operand fetch names the LDS array it reads (a fetch through a selected pointer would have to wait for the loads in flight)
+    auto run = [&](auto roleTag) __attribute__((always_inline)) {
+        constexpr int ROLE = decltype(roleTag)::value;
+        v8bf kf[8], vf[ROLE ? 8 : 1];
+        LoadOwnFrags(kf, p.k + (int64_t)(myRow - l32) * p.ldk + hoff, p.ldk, l32, half);
+        if constexpr (ROLE) {
+            LoadOwnFrags(vf, p.v + (int64_t)(myRow - l32) * p.ldv + hoff, p.ldv, l32, half);
+        }
+        float zero = 0; // opaque, as in AttGradQ2
+        asm volatile("" : "+v"(zero));
+        v16f acc[4];
+#pragma unroll
+        for (int db = 0; db < 4; ++db) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                acc[db][e] = zero;
+            }
+        }
+        if (tFirst <= qHi) {
+            __builtin_amdgcn_s_waitcnt(0x0f70);
+            digestStats(tFirst, 0);
+        }
+        // one 64-query tile: the 32-query blocks of which some query sees a key of this wave
+        auto tile = [&](const uint8_t *qt, const uint8_t *ot, int slot) __attribute__((always_inline)) {
+            int bounds[2][4];
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    bounds[qb][j] = __builtin_amdgcn_readfirstlane(stT[slot][qb][j]);
+                }
+            }
+#pragma unroll
+            for (int qb = 0; qb < TR / 32; ++qb) {
+                const bool full = bounds[qb][0] <= kw0 && bounds[qb][1] >= kw0 + 31;
+                const uint8_t *qt2 = qt + qb * 32 * ROWB, *ot2 = ot + qb * 32 * ROWB;
+                // skipped by a loop of no trips, not by a branch (see AttGradQ2)
+                int trips = __builtin_amdgcn_readfirstlane((int)!(bounds[qb][3] < kw0 || bounds[qb][2] > kw0 + 31));
+                asm volatile("" : "+s"(trips));
+#pragma unroll 1
+                for (int trip = 0; trip < trips; ++trip) {
+                v16f s, dp;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    s[e] = 0;
+                    dp[e] = 0;
+                }
+                const uint8_t *tt = ROLE ? qt2 : ot2; // the tile whose transpose the last product takes
+                v8bf ft[3];
+                if constexpr (ROLE) {
+                    // S = Q K^T, dP = dO V^T; the operands of step ds + 1 are requested before the products of step ds (this role has
+                    // no registers left for a third set of operands)
+                    v8bf fq[2], fo[2];
+                    fq[0] = FragRow(qt2, 0, 0, fl);
+                    fo[0] = FragRow(ot2, 0, 0, fl);
+#pragma unroll
+                    for (int ds = 0; ds < 8; ++ds) {
+                        if (ds + 1 < 8) {
+                            fq[(ds + 1) & 1] = FragRow(qt2, 0, ds + 1, fl);
+                            fo[(ds + 1) & 1] = FragRow(ot2, 0, ds + 1, fl);
+                        }
+                        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fq[ds & 1], kf[ds], s, 0, 0, 0);
+                        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fo[ds & 1], vf[ds], dp, 0, 0, 0);
+                    }
+                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+#pragma unroll
+                    for (int ds = 0; ds < 7; ++ds) {
+                        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+                    }
+                    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+                } else {
+                    // S = Q K^T, operands three steps ahead (one product per step)
+                    v8bf fq[4];
+#pragma unroll
+                    for (int ds = 0; ds < 3; ++ds) {
+                        fq[ds] = FragRow(qt2, 0, ds, fl);
+                    }
+#pragma unroll
+                    for (int ds = 0; ds < 8; ++ds) {
+                        if (ds + 3 < 8) {
+                            fq[(ds + 3) & 3] = FragRow(qt2, 0, ds + 3, fl);
+                        }
+                        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fq[ds & 3], kf[ds], s, 0, 0, 0);
+                    }
+                    ft[0] = FragTr(tt, 0, 0, 0, fl);
+                    ft[1] = FragTr(tt, 0, 0, 1, fl);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+#pragma unroll
+                    for (int ds = 0; ds < 5; ++ds) {
+                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    }
+                    __builtin_amdgcn_sched_group_barrier(0x008, 3, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+                }
+                // P (dV role) or dS (dK role) from the per-query statistics of the tile
+                float wv[16];
+                const float *ps = &st[slot][0][qb * 32 + half * 4];
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const float4 L4 = *(const float4 *)(ps + g * 8);
+                    const float Ls[4] = {L4.x, L4.y, L4.z, L4.w};
+                    float Ds[4] = {0, 0, 0, 0};
+                    if constexpr (ROLE) {
+                        const float4 D4 = *(const float4 *)(ps + TR + g * 8);
+                        Ds[0] = D4.x; Ds[1] = D4.y; Ds[2] = D4.z; Ds[3] = D4.w;
+                    }
+                    int Ss[4] = {0, 0, 0, 0};
+                    unsigned Ns[4] = {0, 0, 0, 0};
+                    if (!full) {
+                        const int4 S4 = *(const int4 *)(ps + 2 * TR + g * 8);
+                        const int4 N4 = *(const int4 *)(ps + 3 * TR + g * 8);
+                        Ss[0] = S4.x; Ss[1] = S4.y; Ss[2] = S4.z; Ss[3] = S4.w;
+                        Ns[0] = (unsigned)N4.x; Ns[1] = (unsigned)N4.y; Ns[2] = (unsigned)N4.z; Ns[3] = (unsigned)N4.w;
+                    }
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const int e = g * 4 + j;
+                        float w = __builtin_amdgcn_exp2f(fmaf(s[e], p.attDotScale, Ls[j] + ck));
+                        if (!full) {
+                            w = (unsigned)(myRow - Ss[j]) <= Ns[j] ? w : 0.f;
+                        }
+                        wv[e] = ROLE ? w * (dp[e] - Ds[j]) * gmul : w;
+                    }
+                    // four queries at a time: without the fence the scheduler runs all sixteen side by side, and their temporaries
+                    // push the role that holds both K and V over its registers
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                const v8bf wb[2] = {PackB(wv, 0), PackB(wv, 1)};
+                // dV^T += dO^T P, or dK^T += Q^T dS, operands two products ahead
+                if constexpr (ROLE) { // this role had no registers to hold them through the arithmetic above
+                    ft[0] = FragTr(tt, 0, 0, 0, fl);
+                    ft[1] = FragTr(tt, 0, 0, 1, fl);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+                }
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    if (i + 2 < 8) {
+                        ft[(i + 2) % 3] = FragTr(tt, 0, (i + 2) >> 2, (i + 2) & 3, fl);
+                    }
+                    acc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ft[i % 3], wb[i >> 2], acc[i & 3], 0, 0, 0);
+                }
+#pragma unroll
+                for (int i = 0; i < 6; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                }
+                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+                }
+            }
+        };
+        // two tiles per trip, one per buffer, in straight-line code (as in AttGradQ2).  The raw statistics of the next tile are digested
+        // before any new load is in flight, so that their reads wait for nothing.
+        for (int t0 = tFirst; t0 <= qHi;) {
+            __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): the tile of this step and the raw statistics of the next have landed
+            __syncthreads();                    // ... for every wave; every wave is done with the other buffers; st*[0] is visible
+            if (t0 + TR <= qHi) {
+                digestStats(t0 + TR, 1);
+                LoadTileDirect(qT1, gq + (int64_t)(t0 + TR) * p.ldq, p.ldq, wave);
+                LoadTileDirect(oT1, go + (int64_t)(t0 + TR) * p.lddo, p.lddo, wave);
+            }
+            if (t0 + 2 * TR <= qHi) {
+                loadStats(t0 + 2 * TR, 0); // the slot of this step's raw statistics, digested one step ago
+            }
+            tile(qT0, oT0, 0);
+            t0 += TR;
+            if (t0 > qHi) {
+                break;
+            }
+            __builtin_amdgcn_s_waitcnt(0x0f70);
+            __syncthreads();
+            if (t0 + TR <= qHi) {
+                digestStats(t0 + TR, 0);
+                LoadTileDirect(qT0, gq + (int64_t)(t0 + TR) * p.ldq, p.ldq, wave);
+                LoadTileDirect(oT0, go + (int64_t)(t0 + TR) * p.lddo, p.lddo, wave);
+            }
+            if (t0 + 2 * TR <= qHi) {
+                loadStats(t0 + 2 * TR, 1);
+            }
+            tile(qT1, oT1, 1);
+            t0 += TR;
+        }
+        uint8_t *out = ROLE ? p.out0 : p.out1;
+        const int64_t ldo = ROLE ? p.ldo0 : p.ldo1;
+        StoreOwnRows<F32>(out + (int64_t)(myRow - l32) * ldo, ldo, head * HD, acc, 1.f, l32, half);
+    };
+    if (role) {
+        run(std::integral_constant<int, 1>{});
+    } else {
+        run(std::integral_constant<int, 0>{});
+    }
+}
+
 bool ActOk(const ts2_mat *m, int rows, int cols)
 {
     return m && m->ptr && m->y >= rows && m->x >= cols && Aligned16(m->ptr, m->strideBytes);
@@ -853,7 +1413,13 @@ extern "C" int ts2_att_backward(const ts2_att_grad_args *a, void *stream)
     if (a->which & 1) {
         p.out0 = (uint8_t *)a->dQ.ptr;
         p.ldo0 = a->dQ.strideBytes;
-        if (f32) {
+        if (!getenv("TS2_ATT_OLD")) {
+            if (f32) {
+                hipLaunchKernelGGL(AttGradQ2<true>, grid, dim3(256), 0, (hipStream_t)stream, p);
+            } else {
+                hipLaunchKernelGGL(AttGradQ2<false>, grid, dim3(256), 0, (hipStream_t)stream, p);
+            }
+        } else if (f32) {
             hipLaunchKernelGGL(AttGradQ<true>, grid, dim3(256), ldsQ, (hipStream_t)stream, p);
         } else {
             hipLaunchKernelGGL(AttGradQ<false>, grid, dim3(256), ldsQ, (hipStream_t)stream, p);
@@ -865,7 +1431,14 @@ extern "C" int ts2_att_backward(const ts2_att_grad_args *a, void *stream)
         p.ldo0 = a->dK.strideBytes;
         p.out1 = (uint8_t *)a->dV.ptr;
         p.ldo1 = a->dV.strideBytes;
-        if (f32) {
+        if (!getenv("TS2_ATT_OLD")) {
+            dim3 grid2(a->lenRound / KVROWS, a->heads);
+            if (f32) {
+                hipLaunchKernelGGL(AttGradKV2<true>, grid2, dim3(256), 0, (hipStream_t)stream, p);
+            } else {
+                hipLaunchKernelGGL(AttGradKV2<false>, grid2, dim3(256), 0, (hipStream_t)stream, p);
+            }
+        } else if (f32) {
             hipLaunchKernelGGL(AttGradKV<true>, grid, dim3(256), 0, (hipStream_t)stream, p); // its LDS is static
         } else {
             hipLaunchKernelGGL(AttGradKV<false>, grid, dim3(256), 0, (hipStream_t)stream, p);
