@@ -106,6 +106,13 @@ def test_attention_window_one(L, orc):
     run_case(L, orc, frag_count=2, frag_len=70, window=1, heads=1, slope=0.0, seed=23, grad_type=L.F32)
 
 
+def test_attention_remapped_block_order(L, orc):
+    """a launch whose workgroup count is a multiple of 8 (the block order is then remapped per XCD), several 128-row blocks per
+    sequence, a slope, key ranges that start inside a 64-row tile"""
+    print("case att remapped order", flush=True)
+    run_case(L, orc, frag_count=4, frag_len=256, window=200, heads=2, slope=0.25, seed=24, grad_type=L.BF16)
+
+
 def test_rope_and_head_norm_passes(L, orc):
     print("case rope/norm passes", flush=True)
     r = np.random.default_rng(24)

@@ -148,7 +148,10 @@ def test_tiny_dense_int8_step_sharp_attention():
 def test_tiny_dense_fp8_step():
     print("case tiny dense fp8", flush=True)
     h = Harness(E4M3, dim=256, heads=2, ffn_tiles=8, depth=4, vocab=256, frag_count=8, frag_len=64, wide_window=64, seed=5)
-    check_model(h, tol_state=5e-2, tol_grad=1.5e-1, tol_delta=2e-1)
+    # e4m3 gradients below the smallest subnormal round to zero, which shrinks the small-signal deltas (Q and K of the window-1 layers,
+    # whose only gradient path is w (1 - w) dP) by a few tenths of a percent; which of them vanish depends on the last bit of the
+    # attention arithmetic: fits between 0.9945 and 1.0008 over kernel revisions, against 0.9973 .. 1.0004 in int8 mode
+    check_model(h, tol_state=5e-2, tol_grad=1.5e-1, tol_delta=2e-1, tol_fit=1e-2)
 
 
 def test_vocabulary_padded_to_the_large_tile_fp8_step():

@@ -7,38 +7,50 @@
 //
 // Design for CDNA4 (replaces Fp16Att / Fp16AttGradQ / Fp16AttGradKV, src/gpt/compute/gpu_att_fp16.cuh:60-358, whose 16-key
 // mma.sync tiling does not map to MFMA):
-//   * a workgroup = 4 waves x 32 rows = 128 query rows (forward, dQ) or 128 key rows (dK/dV); the other side streams through LDS
-//     in 64-row tiles.  Every product is a v_mfma_f32_32x32x16_bf16 whose N index (the lane) is the wave's own row, so all
-//     softmax statistics are per lane and the running rescale of the accumulators needs no cross-lane traffic:
+//   * a wave owns 32 rows (queries in the forward and dQ kernels, keys in the dK/dV kernel); the other side streams through LDS in
+//     64-row tiles and is consumed 32 rows at a time.  Every product is a v_mfma_f32_32x32x16_bf16 whose N index (the lane) is the
+//     wave's own row, so all softmax statistics are per lane and the running rescale of the accumulators needs no cross-lane traffic:
 //         S^T = K Q^T,  O^T += V^T P^T,  dP^T = V dO^T,  dQ^T += K^T dS^T      (lane = query)
 //         S = Q K^T,  dP = dO V^T,  dV^T += dO^T P,  dK^T += Q^T dS             (lane = key)
-//     The probability / score-gradient tiles never leave registers: an MFMA result register block is fed back as the B operand of
-//     the next product (the contraction index order of an MFMA is free as long as A and B agree).
-//   * products that contract over token rows need the streamed tile with rows along the contraction: the tile is fetched one tile
-//     ahead into registers and written to LDS row-major and/or transposed (two rows packed per dword with v_perm_b32, pitches chosen
-//     so that operand reads and transposed writes are bank-conflict free); the wave's own rows are parked in LDS in fragment order.
-//   * the backward kernels run one wave per SIMD (their LDS leaves room for one workgroup per CU), so latency is hidden by the
-//     instruction order alone: operand reads are issued one or two steps ahead of their products, and nothing inside the tile loop
-//     may wait on a load younger than the tile prefetch (vmcnt counts in order).
+//     The probability / score-gradient blocks never leave registers: an MFMA result block, rounded to bf16, is the B operand of the
+//     next product (the contraction index order of an MFMA is free as long as A and B agree).
+//   * the streamed tiles go global -> LDS with buffer_load_dwordx4 ... lds into two buffers used in turn: no staging registers, no
+//     ds_write, one barrier per tile.  Rows are unpadded; the 16-byte chunks of a row are XOR-swizzled by
+//     Swz(row) = 4 * (row % 4) + (row / 4) % 4, which makes both kinds of operand fetch bank-conflict free:
+//       - row-major fragments (contraction over d): ds_read_b128, 16 consecutive rows at one chunk column -> 16 different chunks;
+//       - transposed fragments (contraction over the tile's rows): ds_read_b64_tr_b16 straight from the row-major tile.  Inside each
+//         group of 16 lanes the instruction hands lane j, element e the 16-bit value number j % 4 of the 8 bytes addressed by lane
+//         4 * e + j / 4; with lane i pointing at row i / 4, columns 4 * (i % 4) .. + 3 of a 4 x 16 block, lane j receives column j
+//         of rows 0..3: four contraction slots of an MFMA A operand.  A half wave touches 4 rows x 64 bytes, which the swizzle
+//         spreads over all 64 banks.
+//   * the wave's own rows (the B operands of the products that contract over d) stay in registers for the whole kernel, so every
+//     MFMA costs one 1 KB operand fetch from LDS.  With that every kernel fits 256 registers and 64-70 KB of LDS: two workgroups share
+//     a CU (the exponentials and conversions of one run between the products of the other), where one wave per SIMD waits out every
+//     LDS and MFMA latency itself.  The dK/dV kernel gets there by giving dK and dV to different waves.
+//   * the register budget shapes the control flow: blocks of 32 rows that a wave does not see are skipped by loops of no trips, not
+//     by branches (the join after a branch makes the compiler copy the 64 accumulator registers); the two tile buffers are two
+//     copies of the code in one loop body (an operand fetch names its LDS array, so it never waits for the loads in flight into the
+//     other array); values needed once per tile (lane offsets of the loads, the statistics pass) are recomputed from a lane index
+//     obtained on the spot instead of living across the loop.
+//   * workgroup ids are remapped so that an XCD works on consecutive blocks of one head, whose streamed rows overlap in its L2.
 //   * spans are one inclusive key range per query (every causal window / document-start pattern of
-//     src/gpt/att/sliding_window.cpp:111-118,226-240); masking is one unsigned compare per element, tiles outside a wave's range are
-//     skipped, tiles outside the workgroup's range are never loaded.
+//     src/gpt/att/sliding_window.cpp:111-118,226-240); masking is one unsigned compare per element, blocks outside a wave's range are
+//     skipped, tiles outside the workgroup's range are never loaded; kernels are specialised on whether there is a slope.
 #include "common.h"
+#include <type_traits>
 
 namespace
 {
 constexpr int HD = 128;          // Q_DIM = TT_DIM (src/gpt/compute/cfg_precision.h:79-80)
 constexpr int WROWS = 32;        // rows owned by one wave
-constexpr int BROWS = 128;       // rows owned by one workgroup
+constexpr int BROWS = 128;       // rows owned by one workgroup of the forward and dQ kernels, and of a reverse range
+constexpr int KVROWS = 64;       // key rows owned by one workgroup of the dK/dV kernel
+constexpr int TR = 64;           // rows of a streamed tile
+constexpr int ROWB = HD * 2;     // bytes of a tile row
+constexpr int TILE_BYTES = TR * ROWB;
+constexpr float LN2 = 0.693147f; // LOG2 of src/gpt/model_params/model_dim.h:16
 #define TS2_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 #define TS2_GLB_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
-
-constexpr int TR = 64;           // rows of a streamed tile
-constexpr int RP = HD * 2 + 16;  // row-major tile pitch (bytes)
-constexpr int TP = TR * 2 + 8;   // transposed tile pitch (bytes): 34 dwords -> 8-byte reads of 32 consecutive d hit all 64 banks
-constexpr int RM_BYTES = TR * RP;
-constexpr int T_BYTES = HD * TP;
-constexpr float LN2 = 0.693147f; // LOG2 of src/gpt/model_params/model_dim.h:16
 
 struct AttP {
     const uint8_t *q, *k, *v, *dO; // bf16 [lenRound][heads*128]
@@ -54,90 +66,7 @@ struct AttP {
     int lenRound;
 };
 
-// Streamed tiles are fetched one tile ahead into registers (the loads of tile i+1 are in flight while tile i is multiplied) and go
-// from there to LDS row-major and/or transposed, so a tile costs two workgroup barriers and no LDS-to-LDS pass.  A thread holds two
-// pairs of neighbouring rows (16 bytes of each): lane -> 64 contiguous bytes of a row per 4 lanes, 16 row pairs per wave; with
-// this mapping the dword writes of the transposed copy (two rows per dword) fall into 64 different banks.
-struct TilePref {
-    v4i a[2][2];
-};
-
-__device__ __forceinline__ void TileSlot(int tid, int i, int *r2, int *c)
-{
-    int lane = tid & 63, combo = (tid >> 6) + 4 * i;
-    *r2 = (combo & 1) * 16 + (lane >> 2);
-    *c = (combo >> 1) * 4 + (lane & 3);
-}
-
-__device__ __forceinline__ void PrefetchTile(TilePref &r, const uint8_t *g, int64_t ld, int tid)
-{
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        int r2, c;
-        TileSlot(tid, i, &r2, &c);
-        r.a[i][0] = *(const v4i *)(g + (int64_t)(2 * r2) * ld + c * 16);
-        r.a[i][1] = *(const v4i *)(g + (int64_t)(2 * r2 + 1) * ld + c * 16);
-    }
-}
-
-template <bool RM, bool T> __device__ __forceinline__ void StoreTile(const TilePref &r, uint8_t *rm, uint8_t *t, int tid)
-{
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        int r2, c;
-        TileSlot(tid, i, &r2, &c);
-        if (RM) {
-            *(v4i *)(rm + (2 * r2) * RP + c * 16) = r.a[i][0];
-            *(v4i *)(rm + (2 * r2 + 1) * RP + c * 16) = r.a[i][1];
-        }
-        if (T) {
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                uint32_t lo = __builtin_amdgcn_perm((uint32_t)r.a[i][1][w], (uint32_t)r.a[i][0][w], 0x05040100);
-                uint32_t hi = __builtin_amdgcn_perm((uint32_t)r.a[i][1][w], (uint32_t)r.a[i][0][w], 0x07060302);
-                *(uint32_t *)(t + (8 * c + 2 * w) * TP + 4 * r2) = lo;
-                *(uint32_t *)(t + (8 * c + 2 * w + 1) * TP + 4 * r2) = hi;
-            }
-        }
-    }
-}
-
-// A operand from a row-major tile: lane row = rb*32 + l32, 8 consecutive d at ds*16 + half*8
-__device__ __forceinline__ v8bf FragRM(const uint8_t *rm, int rb, int ds, int l32, int half)
-{
-    return __builtin_bit_cast(v8bf, *(const v4i *)(rm + (rb * 32 + l32) * RP + (ds * 16 + half * 8) * 2));
-}
-
-// A operand from a transposed tile: lane row = d = db*32 + l32; contraction slots = tile rows 16*ks + half*4 + {0..3} and +8
-__device__ __forceinline__ v8bf FragT(const uint8_t *t, int db, int ks, int l32, int half)
-{
-    const uint8_t *p = t + (db * 32 + l32) * TP + (16 * ks + half * 4) * 2;
-    uint2 lo = *(const uint2 *)p;
-    uint2 hi = *(const uint2 *)(p + 16);
-    v4i r = {(int)lo.x, (int)lo.y, (int)hi.x, (int)hi.y};
-    return __builtin_bit_cast(v8bf, r);
-}
-
-// The wave's own rows are a loop-invariant B operand.  Held in registers they cost 32 VGPRs per matrix for the whole kernel, which
-// pushes the kernels over the 256 VGPRs a wave can address directly and makes the compiler shuttle values through AGPRs in the
-// inner loop; parked in LDS in fragment order (lane-linear 16-byte slots: conflict-free ds_read_b128) they cost 8 reads per tile.
-constexpr int OWN_BYTES = 4 * 8 * 64 * 16; // 4 waves x 8 fragments x 64 lanes x 16 bytes
-
-__device__ __forceinline__ void ParkOwnFrags(uint8_t *own, const uint8_t *g, int64_t ld, int wave, int lane)
-{
-    int l32 = lane & 31, half = lane >> 5;
-#pragma unroll
-    for (int ds = 0; ds < 8; ++ds) {
-        *(v4i *)(own + (wave * 8 + ds) * 1024 + lane * 16) = *(const v4i *)(g + (int64_t)l32 * ld + (ds * 16 + half * 8) * 2);
-    }
-}
-
-__device__ __forceinline__ v8bf OwnFrag(const uint8_t *own, int wave, int ds, int lane)
-{
-    return __builtin_bit_cast(v8bf, *(const v4i *)(own + (wave * 8 + ds) * 1024 + lane * 16));
-}
-
-// result registers 8*s .. 8*s+7 of a 32x32 block -> bf16 B operand whose slots match FragT's row order
+// result registers 8*s .. 8*s+7 of a 32x32 block -> bf16 B operand whose slots match FragTr's row order
 __device__ __forceinline__ v8bf PackB(const float *x, int s)
 {
     v4i r;
@@ -221,507 +150,6 @@ __device__ __forceinline__ TRowSpan MakeRowSpan(int start, int finish)
     return r;
 }
 
-// ---------------------------------------------------------------------------------------------------------------------------
-// forward: grid (lenRound/128, heads)
-// two workgroups per CU (256 registers per wave, no AGPR form): their barriers and tile latencies overlap
-__global__ void __launch_bounds__(256, 2) AttForward(AttP p)
-{
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    uint8_t *kRm = lds, *vT = lds + RM_BYTES, *ownQ = lds + RM_BYTES + T_BYTES;
-    __shared__ int red[8];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
-    const int head = blockIdx.y;
-    // later query blocks of a causal sequence see more keys: they start first so that the short ones fill the tail of the launch
-    const int myRow = (gridDim.x - 1 - blockIdx.x) * BROWS + wave * WROWS + l32;
-    const int64_t hoff = (int64_t)head * HD * 2;
-    const int start = p.spanStart[myRow], finish = p.spanFinish[myRow];
-    int kLo, kHi;
-    BlockKeyRange(start, finish, tid, &kLo, &kHi, red);
-    const int tFirst = kHi >= kLo ? (kLo / TR) * TR : 1;
-    TilePref pk, pv;
-    if (tFirst <= kHi) {
-        PrefetchTile(pk, p.k + (int64_t)tFirst * p.ldk + hoff, p.ldk, tid);
-        PrefetchTile(pv, p.v + (int64_t)tFirst * p.ldv + hoff, p.ldv, tid);
-    }
-
-    ParkOwnFrags(ownQ, p.q + (int64_t)(myRow - l32) * p.ldq + hoff, p.ldq, wave, lane);
-    v16f oacc[4];
-#pragma unroll
-    for (int db = 0; db < 4; ++db) {
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            oacc[db][e] = 0;
-        }
-    }
-    float m = 0, sum = 1; // the sink: a zero vector with weight 2^-m
-    const TRowSpan sp = MakeRowSpan(start, finish);
-    for (int t0 = tFirst; t0 <= kHi; t0 += TR) {
-        __syncthreads();
-        StoreTile<true, false>(pk, kRm, nullptr, tid);
-        StoreTile<false, true>(pv, nullptr, vT, tid);
-        __syncthreads();
-        if (t0 + TR <= kHi) {
-            PrefetchTile(pk, p.k + (int64_t)(t0 + TR) * p.ldk + hoff, p.ldk, tid);
-            PrefetchTile(pv, p.v + (int64_t)(t0 + TR) * p.ldv + hoff, p.ldv, tid);
-        }
-        if (t0 > sp.waveMaxFinish || t0 + TR - 1 < sp.waveMinStart) {
-            continue; // no row of this wave sees a key of the tile (wave-uniform)
-        }
-        // phase 1: scores of all 64 keys of the tile (two independent accumulator chains)
-        constexpr int NB = TR / 32;
-        v16f s[NB];
-#pragma unroll
-        for (int kb = 0; kb < NB; ++kb) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                s[kb][e] = 0;
-            }
-        }
-#pragma unroll
-        for (int ds = 0; ds < 8; ++ds) {
-            v8bf qf = OwnFrag(ownQ, wave, ds, lane);
-#pragma unroll
-            for (int kb = 0; kb < NB; ++kb) {
-                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragRM(kRm, kb, ds, l32, half), qf, s[kb], 0, 0, 0);
-            }
-        }
-        // phase 2: one running-max update per tile.  logit = s*scale - slope*(row - key); tiles that every row of the wave sees
-        // completely skip the span tests
-        float sv[NB][16];
-        float mx = m;
-        const float kc = p.slope * (float)(t0 + half * 4 - myRow); // small exact integer times the slope
-        const bool full = t0 >= sp.waveMaxStart && t0 + TR - 1 <= sp.waveMinFinish;
-        if (full) {
-#pragma unroll
-            for (int kb = 0; kb < NB; ++kb) {
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    sv[kb][e] = fmaf(s[kb][e], p.attDotScale, fmaf(p.slope, (float)(kb * 32 + BlkRow(e, 0)), kc));
-                    mx = fmaxf(mx, sv[kb][e]);
-                }
-            }
-        } else {
-            const int rel0 = t0 + half * 4 - sp.start;
-#pragma unroll
-            for (int kb = 0; kb < NB; ++kb) {
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    bool valid = (unsigned)(rel0 + kb * 32 + BlkRow(e, 0)) <= sp.len;
-                    float x = fmaf(s[kb][e], p.attDotScale, fmaf(p.slope, (float)(kb * 32 + BlkRow(e, 0)), kc));
-                    sv[kb][e] = valid ? x : -INFINITY;
-                    mx = fmaxf(mx, sv[kb][e]);
-                }
-            }
-        }
-        {
-            float lo, hi;
-            LaneSwap32(mx, &lo, &hi);
-            mx = fmaxf(lo, hi);
-        }
-        float alpha = __builtin_amdgcn_exp2f(m - mx);
-        const bool rescale = __any(mx != m);
-        m = mx;
-        float ps = 0;
-#pragma unroll
-        for (int kb = 0; kb < NB; ++kb) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                sv[kb][e] = __builtin_amdgcn_exp2f(sv[kb][e] - m); // exp2(-inf) = 0 for masked keys
-                ps += sv[kb][e];
-            }
-        }
-        {
-            float lo, hi;
-            LaneSwap32(ps, &lo, &hi);
-            ps = lo + hi;
-        }
-        sum = sum * alpha + ps;
-        if (rescale) { // wave-uniform: the maximum of no row moved in most tiles
-#pragma unroll
-            for (int db = 0; db < 4; ++db) {
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    oacc[db][e] *= alpha;
-                }
-            }
-        }
-        // phase 3: O^T += V^T P^T, neighbouring MFMAs on different accumulators
-        v8bf pb[NB][2];
-#pragma unroll
-        for (int kb = 0; kb < NB; ++kb) {
-            pb[kb][0] = PackB(sv[kb], 0);
-            pb[kb][1] = PackB(sv[kb], 1);
-        }
-#pragma unroll
-        for (int ks = 0; ks < 2 * NB; ++ks) {
-#pragma unroll
-            for (int db = 0; db < 4; ++db) {
-                oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FragT(vT, db, ks, l32, half), pb[ks >> 1][ks & 1], oacc[db], 0, 0, 0);
-            }
-        }
-    }
-    StoreOwnRows<false>(p.out0 + (int64_t)(myRow - l32) * p.ldo0, p.ldo0, head * HD, oacc, 1 / sum, l32, half);
-    if (half == 0) {
-        p.sumWeightLog[(int64_t)head * p.ldStat + myRow] = m + log2f(sum);
-    }
-}
-
-// ---------------------------------------------------------------------------------------------------------------------------
-// dQ: grid (lenRound/128, heads)
-template <bool F32> __global__ void __launch_bounds__(256) AttGradQ(AttP p)
-{
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    uint8_t *kRm = lds, *vRm = lds + RM_BYTES, *kT = lds + 2 * RM_BYTES, *ownQ = lds + 2 * RM_BYTES + T_BYTES, *ownDO = ownQ + OWN_BYTES;
-    __shared__ int red[8];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
-    const int head = blockIdx.y;
-    // later query blocks of a causal sequence see more keys: they start first so that the short ones fill the tail of the launch
-    const int myRow = (gridDim.x - 1 - blockIdx.x) * BROWS + wave * WROWS + l32;
-    const int64_t hoff = (int64_t)head * HD * 2;
-    const int start = p.spanStart[myRow], finish = p.spanFinish[myRow];
-    int kLo, kHi;
-    BlockKeyRange(start, finish, tid, &kLo, &kHi, red);
-    const int tFirst = kHi >= kLo ? (kLo / TR) * TR : 1;
-    TilePref pk, pv;
-    if (tFirst <= kHi) {
-        PrefetchTile(pk, p.k + (int64_t)tFirst * p.ldk + hoff, p.ldk, tid);
-        PrefetchTile(pv, p.v + (int64_t)tFirst * p.ldv + hoff, p.ldv, tid);
-    }
-
-    ParkOwnFrags(ownQ, p.q + (int64_t)(myRow - l32) * p.ldq + hoff, p.ldq, wave, lane);
-    ParkOwnFrags(ownDO, p.dO + (int64_t)(myRow - l32) * p.lddo + hoff, p.lddo, wave, lane);
-    float L = p.sumWeightLog[(int64_t)head * p.ldStat + myRow];
-    float dScale = p.dScale[(int64_t)head * p.ldStat + myRow];
-    const float gmul = p.attDotScale * LN2;
-    const TRowSpan sp = MakeRowSpan(start, finish);
-    // L and dScale are used here, once, so that their loads are waited for before the loop: a first use inside the loop would
-    // put a wait for every outstanding load (the tile prefetch included) into each iteration
-    asm volatile("" : "+v"(L), "+v"(dScale));
-    v16f acc[4];
-#pragma unroll
-    for (int db = 0; db < 4; ++db) {
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            acc[db][e] = 0;
-        }
-    }
-    for (int t0 = tFirst; t0 <= kHi; t0 += TR) {
-        __syncthreads();
-        StoreTile<true, true>(pk, kRm, kT, tid);
-        StoreTile<true, false>(pv, vRm, nullptr, tid);
-        __syncthreads();
-        if (t0 + TR <= kHi) {
-            PrefetchTile(pk, p.k + (int64_t)(t0 + TR) * p.ldk + hoff, p.ldk, tid);
-            PrefetchTile(pv, p.v + (int64_t)(t0 + TR) * p.ldv + hoff, p.ldv, tid);
-        }
-        if (t0 > sp.waveMaxFinish || t0 + TR - 1 < sp.waveMinStart) {
-            continue; // no row of this wave sees a key of the tile (wave-uniform)
-        }
-        constexpr int NB = TR / 32;
-        v16f s[NB], dp[NB];
-#pragma unroll
-        for (int kb = 0; kb < NB; ++kb) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                s[kb][e] = 0;
-                dp[kb][e] = 0;
-            }
-        }
-        // phase 1: S^T and dP^T of the whole tile, four independent accumulator chains.  One wave per SIMD (the workgroup's LDS
-        // leaves room for one workgroup per CU): the operands of step ds + 1 are requested before the products of step ds are issued
-        v8bf fq[2], fo[2], fk[2][NB], fv[2][NB];
-#define Q_LOAD1(DS)                                                                                                                        \
-    do {                                                                                                                                   \
-        fq[(DS) & 1] = OwnFrag(ownQ, wave, DS, lane);                                                                                      \
-        fo[(DS) & 1] = OwnFrag(ownDO, wave, DS, lane);                                                                                     \
-        _Pragma("unroll") for (int kb = 0; kb < NB; ++kb) {                                                                                \
-            fk[(DS) & 1][kb] = FragRM(kRm, kb, DS, l32, half);                                                                             \
-            fv[(DS) & 1][kb] = FragRM(vRm, kb, DS, l32, half);                                                                             \
-        }                                                                                                                                  \
-    } while (0)
-        Q_LOAD1(0);
-#pragma unroll
-        for (int ds = 0; ds < 8; ++ds) {
-            if (ds + 1 < 8) {
-                Q_LOAD1(ds + 1);
-            }
-#pragma unroll
-            for (int kb = 0; kb < NB; ++kb) {
-                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fk[ds & 1][kb], fq[ds & 1], s[kb], 0, 0, 0);
-                dp[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fv[ds & 1][kb], fo[ds & 1], dp[kb], 0, 0, 0);
-            }
-        }
-#undef Q_LOAD1
-        __builtin_amdgcn_sched_group_barrier(0x100, 2 + 2 * NB, 0);
-#pragma unroll
-        for (int ds = 0; ds < 7; ++ds) {
-            __builtin_amdgcn_sched_group_barrier(0x100, 2 + 2 * NB, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, 2 * NB, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, 2 * NB, 0);
-        // the first operands of phase 3 are requested before the arithmetic of phase 2
-        v8bf ft[2][4];
-#define Q_LOAD3(KS)                                                                                                                        \
-    _Pragma("unroll") for (int db = 0; db < 4; ++db) ft[(KS) & 1][db] = FragT(kT, db, KS, l32, half)
-        Q_LOAD3(0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-        // phase 2: dS
-        v8bf sb[NB][2];
-        const float kc = p.slope * (float)(t0 + half * 4 - myRow) - L; // logit - L in one fma chain
-        const int rel0 = t0 + half * 4 - sp.start;
-        // tiles that every row of the wave sees completely skip the span tests
-        const bool full = t0 >= sp.waveMaxStart && t0 + TR - 1 <= sp.waveMinFinish;
-        if (full) {
-#pragma unroll
-            for (int kb = 0; kb < NB; ++kb) {
-                float dsv[16];
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    float x = fmaf(s[kb][e], p.attDotScale, fmaf(p.slope, (float)(kb * 32 + BlkRow(e, 0)), kc));
-                    float w = __builtin_amdgcn_exp2f(x);
-                    dsv[e] = w * (dp[kb][e] - dScale) * gmul;
-                }
-                sb[kb][0] = PackB(dsv, 0);
-                sb[kb][1] = PackB(dsv, 1);
-            }
-        } else {
-#pragma unroll
-            for (int kb = 0; kb < NB; ++kb) {
-                float dsv[16];
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    float x = fmaf(s[kb][e], p.attDotScale, fmaf(p.slope, (float)(kb * 32 + BlkRow(e, 0)), kc));
-                    float w = __builtin_amdgcn_exp2f(x);
-                    w = (unsigned)(rel0 + kb * 32 + BlkRow(e, 0)) <= sp.len ? w : 0.f;
-                    dsv[e] = w * (dp[kb][e] - dScale) * gmul;
-                }
-                sb[kb][0] = PackB(dsv, 0);
-                sb[kb][1] = PackB(dsv, 1);
-            }
-        }
-        // phase 3: dQ^T += K^T dS^T, operands one step (four products) ahead
-#pragma unroll
-        for (int ks = 0; ks < 2 * NB; ++ks) {
-            if (ks + 1 < 2 * NB) {
-                Q_LOAD3(ks + 1);
-            }
-#pragma unroll
-            for (int db = 0; db < 4; ++db) {
-                acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ft[ks & 1][db], sb[ks >> 1][ks & 1], acc[db], 0, 0, 0);
-            }
-        }
-#undef Q_LOAD3
-#pragma unroll
-        for (int ks = 0; ks < 2 * NB - 1; ++ks) {
-            __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
-    }
-    StoreOwnRows<F32>(p.out0 + (int64_t)(myRow - l32) * p.ldo0, p.ldo0, head * HD, acc, 1.f, l32, half);
-}
-
-// ---------------------------------------------------------------------------------------------------------------------------
-// dK, dV: grid (lenRound/128, heads); the workgroup owns 128 key rows and streams the query rows that reach them
-template <bool F32> __global__ void __launch_bounds__(256) AttGradKV(AttP p)
-{
-    // Static arrays, one per buffer: the compiler then knows that the operand reads do not touch the buffer that the direct
-    // global -> LDS loads below fill, and does not make them wait for those loads.
-    __shared__ __attribute__((aligned(16))) uint8_t qRm[RM_BYTES], doRm[RM_BYTES], qT[T_BYTES], doT[T_BYTES];
-    __shared__ __attribute__((aligned(16))) uint8_t ownK[OWN_BYTES], ownV[OWN_BYTES];
-    __shared__ __attribute__((aligned(16))) float stL[TR], stD[TR]; // per query of the tile: L, dScale
-    __shared__ __attribute__((aligned(16))) int stS[TR], stF[TR];   // span start, span length
-    __shared__ int stT[4];                                          // bounds over the tile's queries
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
-    const int head = blockIdx.y;
-    const int block = blockIdx.x;
-    const int myRow = block * BROWS + wave * WROWS + l32; // my key
-    const int64_t hoff = (int64_t)head * HD * 2;
-    const int qLo = p.revLo[block], qHi = p.revHi[block];
-    const int tFirst = qHi >= qLo ? (qLo / TR) * TR : 1;
-    TilePref pq, pdo;
-    // The per-query statistics of the next tile go global -> LDS without passing through registers: a register that a pending load
-    // writes is a register the compiler may move (the kernel runs at its register limit), and the move waits for every load issued
-    // before it, the tile prefetch included.  Two slots, used in turn; wave 0 issues the loads and, one tile later, reads them back.
-    __shared__ float rawStat[2][4][TR]; // [slot][L, dScale, span start, span finish][query]
-    const int keyBase = block * BROWS;
-    auto prefetch = [&](int t0, int slot) {
-        if (wave == 0) {
-            const int64_t so = (int64_t)head * p.ldStat + t0 + lane;
-            __builtin_amdgcn_global_load_lds(TS2_GLB_PTR(p.sumWeightLog + so), TS2_LDS_PTR(&rawStat[slot][0][0]), 4, 0, 0);
-            __builtin_amdgcn_global_load_lds(TS2_GLB_PTR(p.dScale + so), TS2_LDS_PTR(&rawStat[slot][1][0]), 4, 0, 0);
-            __builtin_amdgcn_global_load_lds(TS2_GLB_PTR(p.spanStart + t0 + lane), TS2_LDS_PTR(&rawStat[slot][2][0]), 4, 0, 0);
-            __builtin_amdgcn_global_load_lds(TS2_GLB_PTR(p.spanFinish + t0 + lane), TS2_LDS_PTR(&rawStat[slot][3][0]), 4, 0, 0);
-        }
-        PrefetchTile(pq, p.q + (int64_t)t0 * p.ldq + hoff, p.ldq, tid);
-        PrefetchTile(pdo, p.dO + (int64_t)t0 * p.lddo + hoff, p.lddo, tid);
-    };
-    if (tFirst <= qHi) {
-        prefetch(tFirst, 0);
-    }
-
-    ParkOwnFrags(ownK, p.k + (int64_t)(myRow - l32) * p.ldk + hoff, p.ldk, wave, lane);
-    ParkOwnFrags(ownV, p.v + (int64_t)(myRow - l32) * p.ldv + hoff, p.ldv, wave, lane);
-    const float gmul = p.attDotScale * LN2;
-    v16f dk[4], dv[4];
-#pragma unroll
-    for (int db = 0; db < 4; ++db) {
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            dk[db][e] = 0;
-            dv[db][e] = 0;
-        }
-    }
-    int slot = 0;
-    for (int t0 = tFirst; t0 <= qHi; t0 += TR, slot ^= 1) {
-        __syncthreads();
-        StoreTile<true, true>(pq, qRm, qT, tid);
-        StoreTile<true, true>(pdo, doRm, doT, tid);
-        if (tid < TR) { // wave 0; the tile stores above have waited for its loads, which were issued after the statistics'
-            __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0)
-            asm volatile("" ::: "memory");
-            // per query: -L - slope * (query - first key of the workgroup), dScale, span start (0x7fffffff if empty) and length
-            const float rawL = rawStat[slot][0][tid];
-            int preS = __float_as_int(rawStat[slot][2][tid]), preF = __float_as_int(rawStat[slot][3][tid]);
-            const bool some = preF >= preS;
-            preS = some ? preS : 0x7fffffff;
-            preF = some ? preF : -1;
-            stL[tid] = -rawL - p.slope * (float)(t0 + tid - keyBase);
-            stD[tid] = rawStat[slot][1][tid];
-            stS[tid] = preS;
-            stF[tid] = (int)(preF >= preS ? (unsigned)(preF - preS) : 0u); // span length
-            int a = preS, b = preF, c = preS, d = preF;
-            a = WaveMaxInt(a);
-            b = WaveMinInt(b);
-            c = WaveMinInt(c);
-            d = WaveMaxInt(d);
-            if (tid == 0) {
-                stT[0] = a; // latest span start of the tile's queries
-                stT[1] = b; // earliest finish
-                stT[2] = c; // earliest start
-                stT[3] = d; // latest finish
-            }
-        }
-        __syncthreads();
-        if (t0 + TR <= qHi) {
-            prefetch(t0 + TR, slot ^ 1);
-        }
-        const int kw0 = __builtin_amdgcn_readfirstlane(myRow - l32); // first key of this wave
-        if (stT[3] < kw0 || stT[2] > kw0 + 31) {
-            continue; // no query of the tile sees a key of this wave (wave-uniform)
-        }
-        const float ck = p.slope * (float)(myRow - keyBase);
-        const bool full = stT[0] <= kw0 && stT[1] >= kw0 + 31; // latest span start and earliest finish of the tile's queries
-        // 32 queries at a time: with both halves of the tile in flight the kernel does not fit into 256 registers
-#pragma unroll
-        for (int qb = 0; qb < TR / 32; ++qb) {
-            v16f s, dp;
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                s[e] = 0;
-                dp[e] = 0;
-            }
-            // phase 1: S and dP.  One wave per SIMD: nothing else hides the LDS latency, so the operands of step ds + 2 are requested
-            // before the products of step ds are issued (three sets of operand registers in rotation)
-            v8bf fq[3], fk[3], fo[3], fv[3];
-#define KV_LOAD1(DS)                                                                                                                       \
-    do {                                                                                                                                   \
-        fq[(DS) % 3] = FragRM(qRm, qb, DS, l32, half);                                                                                     \
-        fk[(DS) % 3] = OwnFrag(ownK, wave, DS, lane);                                                                                      \
-        fo[(DS) % 3] = FragRM(doRm, qb, DS, l32, half);                                                                                    \
-        fv[(DS) % 3] = OwnFrag(ownV, wave, DS, lane);                                                                                      \
-    } while (0)
-            KV_LOAD1(0);
-            KV_LOAD1(1);
-#pragma unroll
-            for (int ds = 0; ds < 8; ++ds) {
-                if (ds + 2 < 8) {
-                    KV_LOAD1(ds + 2);
-                }
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fq[ds % 3], fk[ds % 3], s, 0, 0, 0);
-                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fo[ds % 3], fv[ds % 3], dp, 0, 0, 0);
-            }
-#undef KV_LOAD1
-            __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
-#pragma unroll
-            for (int ds = 0; ds < 6; ++ds) {
-                __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-            }
-            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
-            // the first operands of phase 3 are requested before the arithmetic of phase 2, which covers their latency
-            v8bf to[3], tq[3];
-#define KV_LOAD3(ST)                                                                                                                       \
-    do {                                                                                                                                   \
-        to[(ST) % 3] = FragT(doT, (ST) & 3, qb * 2 + ((ST) >> 2), l32, half);                                                              \
-        tq[(ST) % 3] = FragT(qT, (ST) & 3, qb * 2 + ((ST) >> 2), l32, half);                                                               \
-    } while (0)
-            KV_LOAD3(0);
-            KV_LOAD3(1);
-            __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);  // (a transposed operand is one ds_read2_b64)
-            // phase 2: P and dS from the per-query statistics of the tile
-            float pv[16], dsv[16];
-            if (full) { // every query of the tile sees every key of the wave: no span tests
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    int qi = qb * 32 + g * 8 + half * 4;
-                    float4 L4 = *(const float4 *)(stL + qi);
-                    float4 D4 = *(const float4 *)(stD + qi);
-                    const float Ls[4] = {L4.x, L4.y, L4.z, L4.w};
-                    const float Ds[4] = {D4.x, D4.y, D4.z, D4.w};
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        int e = g * 4 + j;
-                        float w = __builtin_amdgcn_exp2f(fmaf(s[e], p.attDotScale, Ls[j] + ck));
-                        pv[e] = w;
-                        dsv[e] = w * (dp[e] - Ds[j]) * gmul;
-                    }
-                }
-            } else {
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    int qi = qb * 32 + g * 8 + half * 4;
-                    float4 L4 = *(const float4 *)(stL + qi);
-                    float4 D4 = *(const float4 *)(stD + qi);
-                    int4 S4 = *(const int4 *)(stS + qi);
-                    int4 N4 = *(const int4 *)(stF + qi);
-                    const float Ls[4] = {L4.x, L4.y, L4.z, L4.w};
-                    const float Ds[4] = {D4.x, D4.y, D4.z, D4.w};
-                    const int Ss[4] = {S4.x, S4.y, S4.z, S4.w};
-                    const unsigned Ns[4] = {(unsigned)N4.x, (unsigned)N4.y, (unsigned)N4.z, (unsigned)N4.w};
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        int e = g * 4 + j;
-                        float w = __builtin_amdgcn_exp2f(fmaf(s[e], p.attDotScale, Ls[j] + ck));
-                        w = (unsigned)(myRow - Ss[j]) <= Ns[j] ? w : 0.f;
-                        pv[e] = w;
-                        dsv[e] = w * (dp[e] - Ds[j]) * gmul;
-                    }
-                }
-            }
-            v8bf pb[2] = {PackB(pv, 0), PackB(pv, 1)}, sb[2] = {PackB(dsv, 0), PackB(dsv, 1)};
-            // phase 3: dV^T += dO^T P, dK^T += Q^T dS; eight accumulators in turn, operands two steps ahead
-#pragma unroll
-            for (int st = 0; st < 8; ++st) {
-                if (st + 2 < 8) {
-                    KV_LOAD3(st + 2);
-                }
-                dv[st & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(to[st % 3], pb[st >> 2], dv[st & 3], 0, 0, 0);
-                dk[st & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tq[st % 3], sb[st >> 2], dk[st & 3], 0, 0, 0);
-            }
-#undef KV_LOAD3
-#pragma unroll
-            for (int st = 0; st < 6; ++st) {
-                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-            }
-            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
-        }
-    }
-    StoreOwnRows<F32>(p.out0 + (int64_t)(myRow - l32) * p.ldo0, p.ldo0, head * HD, dk, 1.f, l32, half);
-    StoreOwnRows<F32>(p.out1 + (int64_t)(myRow - l32) * p.ldo1, p.ldo1, head * HD, dv, 1.f, l32, half);
-}
-
 // reverse ranges: for every 128-key block the first and last query row whose span touches it
 __global__ void RevInit(int *revLo, int *revHi, int n)
 {
@@ -748,25 +176,9 @@ __global__ void RevBuild(const int *spanStart, const int *spanFinish, int len, i
     }
 }
 
-// ---------------------------------------------------------------------------------------------------------------------------
-// Backward kernels, two workgroups per CU.
-//
-// The streamed tiles (64 rows x 256 bytes) go global -> LDS with global_load_lds_dwordx4 into two buffers used in turn: no staging
-// registers, no ds_write, one barrier per tile.  Rows are unpadded; the 16-byte chunks of a row are XOR-swizzled by
-// Swz(row) = 4 * (row % 4) + (row / 4) % 4, which makes both kinds of operand fetch bank-conflict free:
-//   * row-major fragments (contraction over d): ds_read_b128, 16 consecutive rows at one chunk column -> 16 different chunks;
-//   * transposed fragments (contraction over the tile's rows): ds_read_b64_tr_b16 straight from the row-major tile.  Inside each group
-//     of 16 lanes the instruction hands lane j, element e the 16-bit value number j % 4 of the 8 bytes addressed by lane 4 * e + j / 4;
-//     with lane i pointing at row i / 4, columns 4 * (i % 4) .. + 3 of a 4 x 16 block, lane j receives column j of rows 0..3: the four
-//     contraction slots of an MFMA A operand.  A half wave touches 4 rows x 64 bytes, which the swizzle spreads over all 64 banks.
-// The wave's own rows (the B operands of the products that contract over d) stay in registers for the whole kernel, so every MFMA
-// costs one 1 KB operand fetch from LDS.  All of this fits 256 registers and 64-67 KB of LDS: two workgroups share a CU, and the
-// exponentials and conversions of one wave run under the products of the other.
-constexpr int ROWB = HD * 2;           // bytes of a tile row
-constexpr int TILE_BYTES = TR * ROWB;  // 16 KB
-
 typedef short v4s16 __attribute__((ext_vector_type(4)));
 
+// chunk swizzle of a tile row (16 chunks of 16 bytes): a bijection of row % 16 whose upper two bits are row % 4
 __device__ __forceinline__ int Swz(int row)
 {
     return ((row & 3) << 2) | ((row >> 2) & 3);
@@ -801,7 +213,7 @@ __device__ __forceinline__ void LoadTileDirect(uint8_t *tile, const uint8_t *g, 
 }
 
 // Operand fetches take (tile, compile-time offset) + a per-lane byte offset that is computed once per kernel and made opaque to the
-// optimiser: the tile address and the constant part then fold into the instruction's offset field, and a kernel keeps 8 + 8 address
+// optimiser: the tile address and the constant part then fold into the instruction's offset field, and a kernel keeps ten address
 // registers for all of its fetches instead of one per (buffer, block, step).
 typedef const __attribute__((address_space(3))) uint8_t *TLdsBytes;
 
@@ -879,8 +291,182 @@ __device__ __forceinline__ void MapAttBlock(int *blk, int *head)
     *blk = id - *head * nbx;
 }
 
+// forward: grid (lenRound/128, heads); a wave owns 32 query rows
+template <bool ALIBI> __global__ void __launch_bounds__(256, 2) AttForward(AttP p)
+{
+    __shared__ __attribute__((aligned(1024))) uint8_t kT0[TILE_BYTES], kT1[TILE_BYTES], vT0[TILE_BYTES], vT1[TILE_BYTES];
+    __shared__ int red[8];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l32 = lane & 31, half = lane >> 5;
+    int blk, head;
+    MapAttBlock(&blk, &head);
+    // later query blocks of a causal sequence see more keys: they start first so that the short ones fill the tail of the launch
+    const int myRow = (gridDim.x - 1 - blk) * BROWS + wave * WROWS + l32;
+    const int64_t hoff = (int64_t)head * HD * 2;
+    const int start = p.spanStart[myRow], finish = p.spanFinish[myRow];
+    int kLo, kHi;
+    BlockKeyRange(start, finish, tid, &kLo, &kHi, red);
+    kLo = __builtin_amdgcn_readfirstlane(kLo);
+    kHi = __builtin_amdgcn_readfirstlane(kHi);
+    const int tFirst = kHi >= kLo ? (kLo / TR) * TR : 1;
+    const uint8_t *gk = p.k + hoff, *gv = p.v + hoff;
+    if (tFirst <= kHi) {
+        LoadTileDirect(kT0, gk + (int64_t)tFirst * p.ldk, p.ldk, wave);
+        LoadTileDirect(vT0, gv + (int64_t)tFirst * p.ldv, p.ldv, wave);
+    }
+    v8bf qf[8];
+    LoadOwnFrags(qf, p.q + (int64_t)(myRow - l32) * p.ldq + hoff, p.ldq, l32, half);
+    const TRowSpan sp = MakeRowSpan(start, finish);
+    const TFragLane fl = MakeFragLane(lane);
+    float zero = 0; // opaque, as in AttGradQ
+    asm volatile("" : "+v"(zero));
+    v16f oacc[4];
+#pragma unroll
+    for (int db = 0; db < 4; ++db) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            oacc[db][e] = zero;
+        }
+    }
+    float m = 0, sum = 1; // the sink: a zero vector with weight 2^-m
+    auto tile = [&](const uint8_t *kt, const uint8_t *vt, int t0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int kb = 0; kb < TR / 32; ++kb) {
+            const int k0 = t0 + kb * 32;
+            const uint8_t *kt2 = kt + kb * 32 * ROWB, *vt2 = vt + kb * 32 * ROWB;
+            int trips = __builtin_amdgcn_readfirstlane((int)!(k0 > sp.waveMaxFinish || k0 + 31 < sp.waveMinStart)); // (see AttGradQ)
+            asm volatile("" : "+s"(trips));
+#pragma unroll 1
+            for (int trip = 0; trip < trips; ++trip) {
+                v16f s;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    s[e] = 0;
+                }
+                // phase 1: S^T = K Q^T, operands three steps ahead (one product per step)
+                v8bf fk[4];
+#pragma unroll
+                for (int ds = 0; ds < 3; ++ds) {
+                    fk[ds] = FragRow(kt2, 0, ds, fl);
+                }
+#pragma unroll
+                for (int ds = 0; ds < 8; ++ds) {
+                    if (ds + 3 < 8) {
+                        fk[(ds + 3) & 3] = FragRow(kt2, 0, ds + 3, fl);
+                    }
+                    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fk[ds & 3], qf[ds], s, 0, 0, 0);
+                }
+                // the first operands of phase 3 are requested before the arithmetic of phase 2, which covers their latency
+                v8bf ft[3];
+                ft[0] = FragTr(vt2, 0, 0, 0, fl);
+                ft[1] = FragTr(vt2, 0, 0, 1, fl);
+                __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+#pragma unroll
+                for (int ds = 0; ds < 5; ++ds) {
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                }
+                __builtin_amdgcn_sched_group_barrier(0x008, 3, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+                // phase 2: running maximum and weights of the block's 32 keys.  logit = s * scale - slope * (row - key)
+                float sv[16];
+                float mx = m;
+                const float kc = ALIBI ? p.slope * (float)(k0 + half * 4 - myRow) : 0.f;
+                const bool full = k0 >= sp.waveMaxStart && k0 + 31 <= sp.waveMinFinish;
+                if (full) { // every row of the wave sees every key of the block: no span tests
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        sv[e] = ALIBI ? fmaf(s[e], p.attDotScale, fmaf(p.slope, (float)BlkRow(e, 0), kc)) : s[e] * p.attDotScale;
+                        mx = fmaxf(mx, sv[e]);
+                    }
+                } else {
+                    const int rel0 = k0 + half * 4 - sp.start;
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const float x = ALIBI ? fmaf(s[e], p.attDotScale, fmaf(p.slope, (float)BlkRow(e, 0), kc)) : s[e] * p.attDotScale;
+                        sv[e] = (unsigned)(rel0 + BlkRow(e, 0)) <= sp.len ? x : -INFINITY;
+                        mx = fmaxf(mx, sv[e]);
+                    }
+                }
+                {
+                    float lo, hi;
+                    LaneSwap32(mx, &lo, &hi);
+                    mx = fmaxf(lo, hi);
+                }
+                const float alpha = __builtin_amdgcn_exp2f(m - mx);
+                int rescale = __builtin_amdgcn_readfirstlane((int)(__any(mx != m) != 0));
+                asm volatile("" : "+s"(rescale));
+                m = mx;
+                float ps = 0;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    sv[e] = __builtin_amdgcn_exp2f(sv[e] - m); // exp2(-inf) = 0 for masked keys
+                    ps += sv[e];
+                }
+                {
+                    float lo, hi;
+                    LaneSwap32(ps, &lo, &hi);
+                    ps = lo + hi;
+                }
+                sum = sum * alpha + ps;
+                // the maximum of no row moved in most blocks; the rescaling is a loop of no trips then (not a branch, see AttGradQ)
+#pragma unroll 1
+                for (int r = 0; r < rescale; ++r) {
+#pragma unroll
+                    for (int db = 0; db < 4; ++db) {
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) {
+                            oacc[db][e] *= alpha;
+                        }
+                    }
+                }
+                const v8bf pb[2] = {PackB(sv, 0), PackB(sv, 1)};
+                // phase 3: O^T += V^T P^T, operands two products ahead
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    if (i + 2 < 8) {
+                        ft[(i + 2) % 3] = FragTr(vt2, 0, (i + 2) >> 2, (i + 2) & 3, fl);
+                    }
+                    oacc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ft[i % 3], pb[i >> 2], oacc[i & 3], 0, 0, 0);
+                }
+#pragma unroll
+                for (int i = 0; i < 6; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                }
+                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            }
+        }
+    };
+    // two tiles per trip, one per buffer, in straight-line code (see AttGradQ)
+    for (int t0 = tFirst; t0 <= kHi;) {
+        __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): the tile of this step has landed
+        __syncthreads();                    // ... for every wave, and every wave is done with the other buffer
+        if (t0 + TR <= kHi) {
+            LoadTileDirect(kT1, gk + (int64_t)(t0 + TR) * p.ldk, p.ldk, wave);
+            LoadTileDirect(vT1, gv + (int64_t)(t0 + TR) * p.ldv, p.ldv, wave);
+        }
+        tile(kT0, vT0, t0);
+        t0 += TR;
+        if (t0 > kHi) {
+            break;
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+        if (t0 + TR <= kHi) {
+            LoadTileDirect(kT0, gk + (int64_t)(t0 + TR) * p.ldk, p.ldk, wave);
+            LoadTileDirect(vT0, gv + (int64_t)(t0 + TR) * p.ldv, p.ldv, wave);
+        }
+        tile(kT1, vT1, t0);
+        t0 += TR;
+    }
+    StoreOwnRows<false>(p.out0 + (int64_t)(myRow - l32) * p.ldo0, p.ldo0, head * HD, oacc, 1 / sum, l32, half);
+    if (half == 0) {
+        p.sumWeightLog[(int64_t)head * p.ldStat + myRow] = m + log2f(sum);
+    }
+}
+
 // dQ: grid (lenRound/128, heads); a wave owns 32 query rows
-template <bool F32> __global__ void __launch_bounds__(256, 2) AttGradQ2(AttP p)
+template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGradQ(AttP p)
 {
     __shared__ __attribute__((aligned(1024))) uint8_t kT0[TILE_BYTES], kT1[TILE_BYTES], vT0[TILE_BYTES], vT1[TILE_BYTES];
     __shared__ int red[8];
@@ -905,8 +491,8 @@ template <bool F32> __global__ void __launch_bounds__(256, 2) AttGradQ2(AttP p)
     LoadOwnFrags(qf, p.q + (int64_t)(myRow - l32) * p.ldq + hoff, p.ldq, l32, half);
     LoadOwnFrags(of, p.dO + (int64_t)(myRow - l32) * p.lddo + hoff, p.lddo, l32, half);
     const float L = p.sumWeightLog[(int64_t)head * p.ldStat + myRow];
-    const float dScale = p.dScale[(int64_t)head * p.ldStat + myRow];
     const float gmul = p.attDotScale * LN2;
+    const float negDScale = -p.dScale[(int64_t)head * p.ldStat + myRow] * gmul;
     const TRowSpan sp = MakeRowSpan(start, finish);
     const TFragLane fl = MakeFragLane(lane);
     // cleared from a register the optimiser cannot see through: a constant zero vector would be kept alive across the tile loop as the
@@ -965,25 +551,26 @@ template <bool F32> __global__ void __launch_bounds__(256, 2) AttGradQ2(AttP p)
             }
             __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-            // phase 2: dS
-            const float kc = p.slope * (float)(k0 + half * 4 - myRow) - L; // logit - L in one fma chain
+            // phase 2: dS = w (dP - dScale) attDotScale ln2, w = 2^(logit - L): three instructions and the exponential per element
+            // (without a slope the position term drops out of the logit)
+            const float kc = ALIBI ? p.slope * (float)(k0 + half * 4 - myRow) - L : -L;
             const int rel0 = k0 + half * 4 - sp.start;
             const bool full = k0 >= sp.waveMaxStart && k0 + 31 <= sp.waveMinFinish;
             float dsv[16];
             if (full) { // every row of the wave sees every key of the block: no span tests
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    float x = fmaf(s[e], p.attDotScale, fmaf(p.slope, (float)BlkRow(e, 0), kc));
+                    float x = fmaf(s[e], p.attDotScale, ALIBI ? fmaf(p.slope, (float)BlkRow(e, 0), kc) : kc);
                     float w = __builtin_amdgcn_exp2f(x);
-                    dsv[e] = w * (dp[e] - dScale) * gmul;
+                    dsv[e] = w * fmaf(dp[e], gmul, negDScale);
                 }
             } else {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    float x = fmaf(s[e], p.attDotScale, fmaf(p.slope, (float)BlkRow(e, 0), kc));
+                    float x = fmaf(s[e], p.attDotScale, ALIBI ? fmaf(p.slope, (float)BlkRow(e, 0), kc) : kc);
                     float w = __builtin_amdgcn_exp2f(x);
                     w = (unsigned)(rel0 + BlkRow(e, 0)) <= sp.len ? w : 0.f;
-                    dsv[e] = w * (dp[e] - dScale) * gmul;
+                    dsv[e] = w * fmaf(dp[e], gmul, negDScale);
                 }
             }
             const v8bf sb[2] = {PackB(dsv, 0), PackB(dsv, 1)};
@@ -1045,13 +632,12 @@ __device__ __forceinline__ int Half32MaxInt(int v)
 // two key blocks x two roles: one wave of a block accumulates dV^T += dO^T P (it needs S only), the other dK^T += Q^T dS (S and dP).
 // Both accumulators of a key block in one wave would need 128 registers and leave room for one wave per SIMD only; split, the kernel
 // recomputes S once more but runs two workgroups per CU.
-constexpr int KVROWS = 64;
-
-template <bool F32> __global__ void __launch_bounds__(256, 2) AttGradKV2(AttP p)
+template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGradKV(AttP p)
 {
     __shared__ __attribute__((aligned(1024))) uint8_t qT0[TILE_BYTES], qT1[TILE_BYTES], oT0[TILE_BYTES], oT1[TILE_BYTES];
     __shared__ __attribute__((aligned(16))) float rawStat[2][4][TR];  // [slot][L, dScale, span start, span finish][query], as loaded
-    // [slot][-L - slope * (q - keyBase), dScale, span start (0x7fffffff if empty), span length][query]: one array, one address register
+    // [slot][-L - slope * (q - keyBase), -dScale * attDotScale * ln2, span start (0x7fffffff if empty), span length][query]: one array,
+    // one address register
     __shared__ __attribute__((aligned(16))) float st[2][4][TR];
     __shared__ int stT[2][2][4];                                          // [slot][32-query block]: bounds over the block's queries
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l32 = lane & 31, half = lane >> 5;
@@ -1088,7 +674,7 @@ template <bool F32> __global__ void __launch_bounds__(256, 2) AttGradKV2(AttP p)
             preF = some ? preF : -1;
             float *dst = &st[slot][0][lane];
             dst[0] = -rawL - p.slope * (float)(t0 + lane - keyBase);
-            dst[TR] = rawStat[slot][1][lane];
+            dst[TR] = -rawStat[slot][1][lane] * (p.attDotScale * LN2);
             dst[2 * TR] = __int_as_float(preS);
             dst[3 * TR] = __int_as_float(some ? preF - preS : 0);
             const int a = Half32MaxInt(preS), b = -Half32MaxInt(-preF), c = -Half32MaxInt(-preS), d = Half32MaxInt(preF);
@@ -1121,7 +707,7 @@ template <bool F32> __global__ void __launch_bounds__(256, 2) AttGradKV2(AttP p)
         if constexpr (ROLE) {
             LoadOwnFrags(vf, p.v + (int64_t)(myRow - l32) * p.ldv + hoff, p.ldv, l32, half);
         }
-        float zero = 0; // opaque, as in AttGradQ2
+        float zero = 0; // opaque, as in AttGradQ
         asm volatile("" : "+v"(zero));
         v16f acc[4];
 #pragma unroll
@@ -1149,7 +735,7 @@ template <bool F32> __global__ void __launch_bounds__(256, 2) AttGradKV2(AttP p)
             for (int qb = 0; qb < TR / 32; ++qb) {
                 const bool full = bounds[qb][0] <= kw0 && bounds[qb][1] >= kw0 + 31;
                 const uint8_t *qt2 = qt + qb * 32 * ROWB, *ot2 = ot + qb * 32 * ROWB;
-                // skipped by a loop of no trips, not by a branch (see AttGradQ2)
+                // skipped by a loop of no trips, not by a branch (see AttGradQ)
                 int trips = __builtin_amdgcn_readfirstlane((int)!(bounds[qb][3] < kw0 || bounds[qb][2] > kw0 + 31));
                 asm volatile("" : "+s"(trips));
 #pragma unroll 1
@@ -1232,11 +818,11 @@ template <bool F32> __global__ void __launch_bounds__(256, 2) AttGradKV2(AttP p)
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         const int e = g * 4 + j;
-                        float w = __builtin_amdgcn_exp2f(fmaf(s[e], p.attDotScale, Ls[j] + ck));
+                        float w = __builtin_amdgcn_exp2f(fmaf(s[e], p.attDotScale, ALIBI ? Ls[j] + ck : Ls[j]));
                         if (!full) {
                             w = (unsigned)(myRow - Ss[j]) <= Ns[j] ? w : 0.f;
                         }
-                        wv[e] = ROLE ? w * (dp[e] - Ds[j]) * gmul : w;
+                        wv[e] = ROLE ? w * fmaf(dp[e], gmul, Ds[j]) : w;
                     }
                     // four queries at a time: without the fence the scheduler runs all sixteen side by side, and their temporaries
                     // push the role that holds both K and V over its registers
@@ -1265,7 +851,7 @@ template <bool F32> __global__ void __launch_bounds__(256, 2) AttGradKV2(AttP p)
                 }
             }
         };
-        // two tiles per trip, one per buffer, in straight-line code (as in AttGradQ2).  The raw statistics of the next tile are digested
+        // two tiles per trip, one per buffer, in straight-line code (as in AttGradQ).  The raw statistics of the next tile are digested
         // before any new load is in flight, so that their reads wait for nothing.
         for (int t0 = tFirst; t0 <= qHi;) {
             __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): the tile of this step and the raw statistics of the next have landed
@@ -1309,7 +895,8 @@ template <bool F32> __global__ void __launch_bounds__(256, 2) AttGradKV2(AttP p)
 
 bool ActOk(const ts2_mat *m, int rows, int cols)
 {
-    return m && m->ptr && m->y >= rows && m->x >= cols && Aligned16(m->ptr, m->strideBytes);
+    // the tile loads address a row group of a tile with 32-bit offsets (64 rows of one stride)
+    return m && m->ptr && m->y >= rows && m->x >= cols && Aligned16(m->ptr, m->strideBytes) && m->strideBytes > 0 && m->strideBytes < (1 << 24);
 }
 
 } // namespace
@@ -1358,12 +945,9 @@ extern "C" int ts2_att_forward(const ts2_att_args *a, void *stream)
     p.out0 = (uint8_t *)a->valLookup.ptr;
     p.ldo0 = a->valLookup.strideBytes;
     p.lenRound = a->lenRound;
-    int ldsBytes = RM_BYTES + T_BYTES + OWN_BYTES;
-    static std::atomic<bool> done{false};
-    if (!Ts2SetDynamicLds(done, (const void *)AttForward, ldsBytes)) {
-        return TS2_ERR_LAUNCH;
-    }
-    hipLaunchKernelGGL(AttForward, dim3(a->lenRound / BROWS, a->heads), dim3(256), ldsBytes, (hipStream_t)stream, p);
+    // the kernels without a slope leave the position term out of every logit; all LDS is static (two workgroups per CU)
+    auto kernel = a->alibiSlope != 0 ? AttForward<true> : AttForward<false>;
+    hipLaunchKernelGGL(kernel, dim3(a->lenRound / BROWS, a->heads), dim3(256), 0, (hipStream_t)stream, p);
     TS2_CHECK_LAUNCH();
     return TS2_OK;
 }
@@ -1404,26 +988,12 @@ extern "C" int ts2_att_backward(const ts2_att_grad_args *a, void *stream)
     p.dScale = (const float *)a->dScale.ptr;
     p.ldStat = a->sumWeightLog.strideBytes / 4;
     p.lenRound = a->lenRound;
-    dim3 grid(a->lenRound / BROWS, a->heads);
-    int ldsQ = 2 * RM_BYTES + T_BYTES + 2 * OWN_BYTES;
-    static std::atomic<bool> doneQ0{false}, doneQ1{false};
-    if (!Ts2SetDynamicLds(doneQ1, (const void *)AttGradQ<true>, ldsQ) || !Ts2SetDynamicLds(doneQ0, (const void *)AttGradQ<false>, ldsQ)) {
-        return TS2_ERR_LAUNCH;
-    }
+    const bool alibi = a->alibiSlope != 0; // the kernels without a slope leave the position term out of every logit
     if (a->which & 1) {
         p.out0 = (uint8_t *)a->dQ.ptr;
         p.ldo0 = a->dQ.strideBytes;
-        if (!getenv("TS2_ATT_OLD")) {
-            if (f32) {
-                hipLaunchKernelGGL(AttGradQ2<true>, grid, dim3(256), 0, (hipStream_t)stream, p);
-            } else {
-                hipLaunchKernelGGL(AttGradQ2<false>, grid, dim3(256), 0, (hipStream_t)stream, p);
-            }
-        } else if (f32) {
-            hipLaunchKernelGGL(AttGradQ<true>, grid, dim3(256), ldsQ, (hipStream_t)stream, p);
-        } else {
-            hipLaunchKernelGGL(AttGradQ<false>, grid, dim3(256), ldsQ, (hipStream_t)stream, p);
-        }
+        auto kernel = f32 ? (alibi ? AttGradQ<true, true> : AttGradQ<true, false>) : (alibi ? AttGradQ<false, true> : AttGradQ<false, false>);
+        hipLaunchKernelGGL(kernel, dim3(a->lenRound / BROWS, a->heads), dim3(256), 0, (hipStream_t)stream, p);
         TS2_CHECK_LAUNCH();
     }
     if (a->which & 2) {
@@ -1431,18 +1001,8 @@ extern "C" int ts2_att_backward(const ts2_att_grad_args *a, void *stream)
         p.ldo0 = a->dK.strideBytes;
         p.out1 = (uint8_t *)a->dV.ptr;
         p.ldo1 = a->dV.strideBytes;
-        if (!getenv("TS2_ATT_OLD")) {
-            dim3 grid2(a->lenRound / KVROWS, a->heads);
-            if (f32) {
-                hipLaunchKernelGGL(AttGradKV2<true>, grid2, dim3(256), 0, (hipStream_t)stream, p);
-            } else {
-                hipLaunchKernelGGL(AttGradKV2<false>, grid2, dim3(256), 0, (hipStream_t)stream, p);
-            }
-        } else if (f32) {
-            hipLaunchKernelGGL(AttGradKV<true>, grid, dim3(256), 0, (hipStream_t)stream, p); // its LDS is static
-        } else {
-            hipLaunchKernelGGL(AttGradKV<false>, grid, dim3(256), 0, (hipStream_t)stream, p);
-        }
+        auto kernel = f32 ? (alibi ? AttGradKV<true, true> : AttGradKV<true, false>) : (alibi ? AttGradKV<false, true> : AttGradKV<false, false>);
+        hipLaunchKernelGGL(kernel, dim3(a->lenRound / KVROWS, a->heads), dim3(256), 0, (hipStream_t)stream, p);
         TS2_CHECK_LAUNCH();
     }
     return TS2_OK;
