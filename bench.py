@@ -298,9 +298,10 @@ def bandwidth_kernels(iters=10):
     return res
 
 
-def fp8_backward_gemms(n, dim, ffn, iters=10, only_dominant=False):
-    """the e4m3 backward GEMM shapes of the dense step, each timed alone with events: dX of the FFN contract / expand matrices,
-    the FFN delta (packed-delta epilogue) and the attention-width dX"""
+def fp8_backward_gemms(n, dim, ffn, iters=100, warm=20, only_dominant=False):
+    """the e4m3 backward GEMM shapes of the dense step, each timed alone with events over `iters` launches after `warm` untimed ones
+    (the device settles at its sustained clock within the first few milliseconds of such a run): dX of the FFN contract / expand
+    matrices, the FFN delta (packed-delta epilogue) and the attention-width dX"""
     import torch
     from tscale2_amd import lib as L
     lib = L.load()
@@ -314,7 +315,9 @@ def fp8_backward_gemms(n, dim, ffn, iters=10, only_dominant=False):
         else:
             c = torch.empty((m, nn), dtype=torch.float32, device="cuda")
             fn = lambda: lib.gemm_nt(a, b, c, L.E4M3, L.F32)  # noqa: E731
-        fn(); torch.cuda.synchronize()
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
         ms = event_time_ms(fn, iters)
         ops = 2.0 * m * nn * k
         out.append({"product": name, "m": m, "n": nn, "k": k, "us": round(ms * 1e3, 1), "tflops": round(ops / (ms * 1e-3) / 1e12, 1),
