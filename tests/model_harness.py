@@ -77,7 +77,7 @@ class QMatrix:
 
 class Harness:
     def __init__(self, mode, dim, heads, ffn_tiles, depth, vocab, frag_count, frag_len, wide_window=64, experts=0, selected=2, xp=128, seed=1,
-                 std=0.02, k_std=None, bias_std=0.0):
+                 std=0.02, k_std=None, bias_std=0.0, sel_std=None):
         self.orc = Oracle()
         self.mode, self.dim, self.heads, self.ffn = mode, dim, heads, ffn_tiles * 128
         self.experts, self.selected, self.xp = experts, selected, xp
@@ -90,6 +90,8 @@ class Harness:
             mats = []
             for i, (rows, cols) in enumerate(layer_shapes(self.lt[d], dim, heads, self.ffn, xp, experts)):
                 s = std if not (k_std and self.lt[d] == LT_ATT and i == 1) else k_std
+                if sel_std and self.lt[d] == LT_MOE and i == 3:
+                    s = sel_std  # the select matrix: wider logit gaps, fewer tokens whose top-k choice hangs on 8-bit noise
                 mats.append(QMatrix(self.orc, r.standard_normal((rows, cols)) * s, mode, i in NO_SCALE[int(self.lt[d])]))
             self.layers.append(mats)
         self.embed = QMatrix(self.orc, r.standard_normal((self.label_count, dim)) * std, mode, False)

@@ -8,12 +8,12 @@ sqrt and the rare roundings those flip: it is what the device results are compar
 It follows the call order of the library's step driver (embedding, per layer normalise + FFN / attention forward, final layer and loss
 gradient, backward loop with ScaleGrad / layer backward / normalisation backward, embedding delta), which is the order of the
 reference's AddForward / AddBackward (src/gpt/compute/layer_ffn.cu:56-113, layer_att.cu:108-226, gpu_transformer.cu:260-471) with the
-CPU path's factors.  Test infrastructure: dense FFN and attention layers, both 8-bit modes."""
+CPU path's factors.  Test infrastructure: FFN and attention layers in both 8-bit modes, MoE layers (layer_moe.cu:186-285) in e4m3 mode."""
 import ctypes as C
 
 import numpy as np
 
-from model_harness import E4M3, I8, LT_ATT, LT_FFN
+from model_harness import E4M3, I8, LT_ATT, LT_FFN, LT_MOE
 from oracle_lib import _ptr
 
 F32 = np.float32
@@ -270,10 +270,107 @@ class SameContract:
         self.delta[d] = [self.backprop_delta(norm8, g, grad_scale) for g in (dqf, dkf, dvf, dgate)] + [delta_comb]
         return dnorm
 
+    # ---- MoE layer: every (token, slot) pair is a row of its expert; the device groups those rows by expert, this model loops over experts
+    def moe_route(self, sel):
+        """MoeCalcSampleExpertLists: top-k by value with first-index ties, w = exp((s - max) / 2), scaled so that sum w^2 = experts"""
+        n, E = sel.shape
+        K = self.h.selected
+        v = sel.astype(F32).copy()
+        ids = np.zeros((n, K), np.int64); w = np.zeros((n, K), F32)
+        rows = np.arange(n)
+        for z in range(K):
+            ids[:, z] = np.argmax(v, 1)  # first index among equals
+            top = v[rows, ids[:, z]]
+            if z == 0:
+                mx = top.copy()
+            w[:, z] = np.exp(((top - mx) * F32(0.5)).astype(F32)).astype(F32)
+            v[rows, ids[:, z]] = F32(-1e10)
+        scale = (np.sqrt(F32(E)) * np.sqrt(F32(1) / (w * w).sum(1, dtype=F32))).astype(F32)
+        return ids, (w * scale[:, None]).astype(F32)
+
+    def moe_forward(self, d, norm8):
+        h = self.h
+        assert self.mode == E4M3
+        W = h.layers[d]
+        E, K, X, D, n = h.experts, h.selected, h.xp, h.dim, self.n
+        a = VEC * DISCR * dot(D)
+        sel = self.forward_mm(norm8, W[3], False, a)
+        ids, wts = self.moe_route(sel)
+        we, wg, wc = self.val(W[0]).reshape(E, X, D), self.val(W[1]).reshape(E, X, D), self.val(W[2]).reshape(E, D, X)
+        wide16 = np.zeros((n, K, X), F32); wscale = np.zeros((n, K, X // 128), F32); gate16 = np.zeros((n, K, X), F32)
+        rg8 = np.zeros((n, K, X), F32); contract = np.zeros((n, K, D), F32)
+        for k in range(K):
+            for e in range(E):
+                r = np.nonzero(ids[:, k] == e)[0]
+                if not len(r):
+                    continue
+                raw = (mm(norm8[r], we[e]) * (a * F32(W[0].scale))).astype(F32)
+                wide16[r, k], wscale[r, k] = self.norm_rope(raw, True, VEC, None)
+                gate16[r, k] = bf16((mm(norm8[r], wg[e]) * a).astype(F32))
+                rg8[r, k] = self.q8((wide16[r, k] * lolu(gate16[r, k])).astype(F32) * wts[r, k][:, None])
+                contract[r, k] = (mm(rg8[r, k], wc[e]) * (VEC * DISCR * dot(E * X) * F32(W[2].scale))).astype(F32)
+        self.acts[d] = (ids, wts, wide16, wscale, gate16, rg8)
+        out = contract[:, 0]
+        for k in range(1, K):
+            out = (out + contract[:, k]).astype(F32)
+        return out
+
+    def moe_backward(self, d, norm8, sg_fast, grad_scale):
+        h = self.h
+        W = h.layers[d]
+        E, K, X, D, n = h.experts, h.selected, h.xp, h.dim, self.n
+        ids, wts, wide16, wscale, gate16, rg8 = self.acts[d]
+        we, wg, wc = self.val(W[0]).reshape(E, X, D), self.val(W[1]).reshape(E, X, D), self.val(W[2]).reshape(E, D, X)
+        dwide = np.zeros((n, K, X), F32); dgate = np.zeros((n, K, X), F32); gm = np.zeros((n, K), F32)
+        full = np.zeros((n, K, D), F32)
+        f2 = DISCR * dot(E * X) * F32(W[2].scale)
+        f0 = DISCR * dot(D)
+        deltas = [np.zeros(W[i].fast.shape, F32) for i in range(3)]
+        for k in range(K):
+            for e in range(E):
+                r = np.nonzero(ids[:, k] == e)[0]
+                if not len(r):
+                    continue
+                drg = (mm(sg_fast[r], wc[e].T) * f2).astype(F32)
+                vv = (wide16[r, k] * VEC).astype(F32)
+                mult = lolu(gate16[r, k])
+                moe = wts[r, k][:, None]
+                gm[r, k] = (drg.astype(np.float64) * vv * mult).sum(1).astype(F32)
+                dgate[r, k] = self.qfast((drg * vv * (mult * (1 - mult) * 2)).astype(F32) * moe)
+                src = (vv * rep((wscale[r, k] / VEC).astype(F32))).astype(F32)
+                dwide[r, k] = self.qfast(tile_norm_backprop(src, ((drg * mult).astype(F32) * moe).astype(F32)))
+                # expand and gate products in one launch: the sums of the first are rescaled to the second's factor, one multiply at the end
+                full[r, k] = ((mm(dwide[r, k], we[e].T).astype(np.float64) * float(f0 * F32(W[0].scale)) +
+                               mm(dgate[r, k], wg[e].T).astype(np.float64) * float(f0))).astype(F32)
+        # the deltas of an expert contract over all its rows, whatever their slot
+        for e in range(E):
+            tk = np.nonzero(ids == e)
+            if not len(tk[0]):
+                continue
+            src = norm8[tk[0]]
+            g = F32(VEC * F32(grad_scale))
+            deltas[2][e * D:(e + 1) * D] = (mm(sg_fast[tk[0]].T, rg8[tk].T) * g).astype(F32)
+            deltas[0][e * X:(e + 1) * X] = (mm(dwide[tk].T, src.T) * g).astype(F32)
+            deltas[1][e * X:(e + 1) * X] = (mm(dgate[tk].T, src.T) * g).astype(F32)
+        # BackpropMoe (CpuBackpropMoe restricted to the selected experts)
+        ms = np.sqrt(F32(E))
+        w = (wts / ms).astype(F32); g = (gm * ms).astype(F32)
+        avrg = (w * g).sum(1, dtype=F32)[:, None]
+        dsel = np.zeros((n, E), F32)
+        dsel[np.arange(n)[:, None], ids] = self.qfast(((w * g - w * w * avrg) * F32(0.5)).astype(F32))
+        dnorm = full[:, 0]
+        for k in range(1, K):
+            dnorm = (dnorm + full[:, k]).astype(F32)
+        dnorm = (dnorm + self.backprop_dx(dsel, W[3], False, f0)).astype(F32)
+        self.core = {"dsel": dsel, "ids": ids, "wts": wts}
+        self.delta[d] = [self.pack(deltas[0]), self.pack(deltas[1]), self.pack(deltas[2]), self.backprop_delta(norm8, dsel, grad_scale)]
+        return dnorm
+
     # ---- one layer / the final layer on given inputs -------------------------------------------------------------------------------
     def layer_forward(self, d, norm8):
         """the layer's addition to the residual state from its 8-bit input"""
-        return self.ffn_forward(d, norm8) if self.h.lt[d] == LT_FFN else self.att_forward(d, norm8)
+        lt = int(self.h.lt[d])
+        return self.ffn_forward(d, norm8) if lt == LT_FFN else self.moe_forward(d, norm8) if lt == LT_MOE else self.att_forward(d, norm8)
 
     def layer_backward(self, d, norm8, scale, grad):
         """one step of the backward loop: ScaleGrad, the layer's backward (deltas to self.delta[d]), the normalisation backward with the
@@ -281,7 +378,9 @@ class SameContract:
         gm = F32(self.orc.lib.orc_grad_mult(float(np.abs(grad).max())))
         gs = F32(1) / gm
         sg_fast = self.qfast(grad * gm)
-        dn = self.ffn_backward(d, norm8, sg_fast, gs) if self.h.lt[d] == LT_FFN else self.att_backward(d, norm8, sg_fast, gs)
+        lt = int(self.h.lt[d])
+        back = self.ffn_backward if lt == LT_FFN else self.moe_backward if lt == LT_MOE else self.att_backward
+        dn = back(d, norm8, sg_fast, gs)
         return (tile_norm_backprop((norm8 * rep(scale)).astype(F32), (dn * gs).astype(F32)) + grad).astype(F32)
 
     def final_backward(self, fn8, scale):

@@ -176,6 +176,28 @@ def test_moe_layer_fp8_step():
     check_model(h, tol_state=8e-2, tol_grad=1.5e-1, tol_delta=2e-1, tol_fit=1.5e-2)
 
 
+def test_kept_activations_equal_recomputation_with_moe_layers():
+    """kept-versus-recomputed with MoE layers in a non-last and the last position (the MoE forward results live in buffers shared by all
+    MoE layers: only the layer that ran last may use them as they are), expert width 512, two steps"""
+    print("case kept vs recomputed activations, MoE", flush=True)
+    h = Harness(E4M3, dim=256, heads=2, ffn_tiles=2, depth=3, vocab=256, frag_count=4, frag_len=64, wide_window=64, experts=4, selected=2, xp=512,
+                seed=17, std=0.05)
+    assert [int(t) for t in h.lt].count(3) == 2
+    res = []
+    for recompute in (False, True):
+        m = h.device_model(recompute=recompute)
+        try:
+            for _ in range(2):
+                m.backprop()
+            torch.cuda.synchronize()
+            res.append([m.get_delta(d, i, *q.fast.shape) for d in range(len(h.layers)) for i, q in enumerate(h.layers[d])] +
+                       [m.array("stateGrad").float().cpu().numpy()])
+        finally:
+            m.close()
+    for a, b in zip(*res):
+        assert np.array_equal(a, b)
+
+
 def test_moe_routing_tables_match_cpu_moe():
     """ts2_moe_route against CpuMoe (layer_moe.cu:287-327): same experts, same weights, sum w^2 = E, stable grouping"""
     print("case moe route", flush=True)

@@ -42,3 +42,21 @@ def test_same_contract_step_is_the_oracle_step_plus_unbiased_storage_noise(mode)
         fit, corr = scale_fit(got, ref)
         # e4m3 fast gradients flush what lies more than 17 binary orders below their maximum: a slight shrink (measured down to 0.9936)
         assert rms <= 0.12 and abs(fit - 1) <= (6e-3 if mode == I8 else 1e-2) and corr >= 0.995, (what, rms, fit, corr)
+
+
+def test_same_contract_moe_step_follows_the_oracle_step():
+    """attention + MoE (e4m3): the model's MoE layer against the fp32 oracle's.  Looser than the dense case: besides the storage noise a
+    few per cent of the tokens pick another expert once their select logits come from 8-bit states"""
+    h = Harness(E4M3, dim=256, heads=2, ffn_tiles=2, depth=1, vocab=256, frag_count=4, frag_len=96, wide_window=64, experts=8, selected=2, xp=256,
+                seed=16, std=0.05)
+    h.oracle_step()
+    s = SameContract(h).run()
+    assert abs(s.loss - h.ref_loss) <= 2e-3 * abs(h.ref_loss)
+    pairs = [("state", s.state, h.states[-1]), ("stateGrad", s.state_grad, h.ref_grad0), ("final", s.delta_final, h.ref_delta_final)]
+    for d in range(h.depth):
+        for i in range(len(h.layers[d])):
+            pairs.append((("delta", d, i), s.delta[d][i], h.ref_delta[d][i]))
+    for what, got, ref in pairs:
+        rms, _ = rel_err(got, ref)
+        fit, corr = scale_fit(got, ref)
+        assert rms <= 0.25 and abs(fit - 1) <= 2e-2 and corr >= 0.97, (what, rms, fit, corr)

@@ -122,3 +122,14 @@ def test_layers_same_contract_large_tile_branches(mode):
     slices of the small deltas, the stacked Q/K/V/gate delta and the grouped dX products all run inside the layer backward here"""
     print("case same contract per layer: large-tile branches", mode, flush=True)
     check_layers(Harness(mode, dim=512, heads=4, ffn_tiles=16, depth=1, vocab=256, frag_count=16, frag_len=512, wide_window=512, seed=12))
+
+
+def test_layers_same_contract_moe():
+    """the reference's depth-3 schedule with experts (att ffn att ffn att moe att moe), expert width 256: each MoE layer alone on the
+    device's own stored input - routing, gather, grouped expand / gate / contract products, combine, the gate and norm backward over
+    grouped rows, routing backward, grouped dX products and the per-expert deltas - against the model that rounds where the device does.
+    Both sides route from the same 8-bit input, so they pick the same experts (the fp32 oracle does not: a few per cent of the tokens
+    change experts under 8-bit state noise, which is why the whole-step comparison of MoE models is loose)"""
+    print("case same contract per layer: MoE", flush=True)
+    check_layers(Harness(E4M3, dim=256, heads=2, ffn_tiles=2, depth=3, vocab=256, frag_count=4, frag_len=96, wide_window=64, experts=8,
+                         selected=2, xp=256, seed=16, std=0.05))
