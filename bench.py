@@ -87,7 +87,7 @@ def cpu_baseline_linear(len_full, src_dim, grad_dim, sample_rows):
 
 
 def linear_i8_setup(delta_splits, sort_rows=False):
-    """BASELINE config[1]: tensors and operator buffers of the int8 linear-layer backward"""
+    """int8 linear-layer workload: tensors and operator buffers of the int8 linear-layer backward"""
     import torch
     from tscale2_amd import lib as L
     len_, src_dim, grad_dim, k_tile = 16384, 1024, 4096, 512
@@ -334,7 +334,7 @@ def fp8_backward_gemms(n, dim, ffn, iters=100, warm=20, only_dominant=False):
 
 
 def bench_step_fp8(args):
-    """BASELINE config[2]: e2048 h16 d12 ffn64 w1024 (24 layers), vocab 50304, 32 sequences x 1024 tokens, e4m3 weights/states/gradients,
+    """dense fp8 step workload: e2048 h16 d12 ffn64 w1024 (24 layers), vocab 50304, 32 sequences x 1024 tokens, e4m3 weights/states/gradients,
     bf16 activations.  One step = forward + loss gradient + backward through all layers with every delta (no optimiser)."""
     import numpy as np
     import torch
@@ -500,7 +500,7 @@ def cpu_baseline_moe(dim, xp, experts, selected, tokens):
 
 
 def bench_att_bwd(args):
-    """BASELINE config[3]: causal attention backward alone, 16 sequences x 2048, 16 heads x 128, bf16"""
+    """attention workload: causal attention backward alone, 16 sequences x 2048, 16 heads x 128, bf16"""
     import torch
     from tscale2_amd import lib as L
     L.load()
@@ -541,7 +541,7 @@ def bench_att_bwd(args):
 
 
 def bench_moe_fp8(args):
-    """BASELINE config[4]: one MoE layer forward + backward: 64 experts, top-2, dim 1024, expert width 512, 65536 tokens, e4m3 expert
+    """MoE workload: one MoE layer forward + backward: 64 experts, top-2, dim 1024, expert width 512, 65536 tokens, e4m3 expert
     weights; the router logits come from a random select matrix on tile-normalised N(0,1) states (mildly imbalanced load).
     One step = ts2_layer_forward + ts2_layer_backward of that layer (routing, gather, grouped expand/gate/contract products, combine,
     routing backward, grouped dX products, grouped deltas, select-matrix backward)."""

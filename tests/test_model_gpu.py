@@ -132,7 +132,7 @@ def test_new_weights_replace_the_kept_transposes(mode):
 
 
 def test_tiny_dense_int8_step():
-    """BASELINE config[0]: e256 h2 d4 ffn8 w64 (8 layers), byte vocab, 8 fragments of 64 tokens, weights N(0, 0.02)"""
+    """the reference's own CPU-runnable configuration: e256 h2 d4 ffn8 w64 (8 layers), byte vocab, 8 fragments of 64 tokens, weights N(0, 0.02)"""
     print("case tiny dense int8", flush=True)
     h = Harness(I8, dim=256, heads=2, ffn_tiles=8, depth=4, vocab=256, frag_count=8, frag_len=64, wide_window=64, seed=3)
     check_model(h, tol_state=4e-2, tol_grad=5e-2, tol_delta=1e-1)
