@@ -126,6 +126,12 @@ typedef struct ts2_gemm_args {
         float alpha;
         const float *alphaPtr;
     } segment[3];
+    /* kMajor != 0: A is [k][m] and B is [k][n] - the rows of both operands are the contraction index, C[i][j] = sum_k A[k][i] * B[k][j].
+     * The form a delta product dW = dY^T X takes on the untransposed activations ([token][feature], src/gpt/compute/matmul_fwdbwd.cuh:314-391
+     * transposes both first): the operands are transposed by the LDS reads of the kernel instead.  TS2_E4M3 operands, m and n multiples
+     * of 256 (the 256x256 kernel; with tileConfig 0 the caller must make sure that (m/256)*(n/256)*slices >= 192 or pass tileConfig 1),
+     * fp32 TS2_EPI_STORE results (also as stored slices, splitSlabBytes) or TS2_EPI_ROW_TILE_MAXNORM; nothing else. */
+    int32_t kMajor;
 } ts2_gemm_args;
 
 int ts2_gemm_nt(const ts2_gemm_args *args, void *stream);
@@ -269,6 +275,11 @@ typedef struct ts2_matmul_bwd_buffers {
     int32_t *rowOrder;
     int32_t *rowOrderTmp;
     int32_t sortRows;
+    /* != 0 (E4M3): rows len .. lenRound of the `src` and `grad` given to BackpropDelta hold zeros (the producers of this library leave
+     * them so, like the reference's, src/lib/cuda/cuda_matmul.cuh:10).  With srcDim and gradDim on the 256 grid the delta product then
+     * reads both operands as they are - contraction-major, ts2_gemm_args.kMajor - and neither is transposed: gradT, srcT and their
+     * Valid flags are not used.  The result is bit-identical to the transposing sequence. */
+    int32_t padRowsZero;
 } ts2_matmul_bwd_buffers;
 
 /* Bytes of every scratch member of ts2_matmul_bwd_buffers for one matrix, the sizes TInt8MatMulBwdBuffers / TFp8MatMulBwdBuffers allocate

@@ -426,3 +426,58 @@ def test_products_with_a_zero_factor_contribute_nothing(zero_at):
         lib.gemm_nt(As[0], Bs[0], got2, L.E4M3, L.F32, alpha=0.5, alpha_ptr=p2[0], tile_config=2, segments=[(As[1], Bs[1], 0.5, p2[1])])
         torch.cuda.synchronize()
         assert torch.isfinite(got2).all() and (got2 - want2).abs().max().item() <= 4e-6 * max(want2.abs().max().item(), 1e-30), za
+
+
+def test_contraction_major_operands_equal_the_transposed_product(lib, orc):
+    """kMajor: A [k][m], B [k][n] (the untransposed activations of a delta product) against the same product on explicitly transposed
+    operands.  Both feed the MFMAs the same operand bytes in the same contraction slots, so fp32 results, stored slices and packed
+    deltas must be bit-identical; operands with live strides larger than the tile, a contraction of 9 steps (ring loop + tail)"""
+    print("case contraction-major operands", flush=True)
+    from tscale2_amd import lib as L
+    m, n, k = 512, 768, 1152
+    r = np.random.default_rng(31)
+
+    def codes(shape):  # e4m3 bytes without the NaN codes, both signs
+        return (r.integers(0, 120, shape) | (r.integers(0, 2, shape) << 7)).astype(np.uint8)
+    big_a, big_b = codes((k, m + 256)), codes((k, n + 512))
+    akm = torch.from_numpy(big_a).cuda()[:, 128:128 + m]   # [k][m] view with a larger row stride
+    bkn = torch.from_numpy(big_b).cuda()[:, 256:256 + n]
+    at, bt = akm.t().contiguous(), bkn.t().contiguous()    # [m][k], [n][k]
+    # fp32 store
+    c0 = torch.zeros((m, n), device="cuda"); c1 = torch.ones((m, n), device="cuda")
+    lib.gemm_nt(at, bt, c0, L.E4M3, L.F32, alpha=0.5, tile_config=1)
+    lib.gemm_nt(akm, bkn, c1, L.E4M3, L.F32, alpha=0.5, tile_config=1, m=m, n=n, k=k, k_major=True)
+    torch.cuda.synchronize()
+    assert torch.equal(c0, c1) and float(c0.abs().max()) > 0
+    tab = orc.e4m3_table(hw=True)
+    ref = (tab[big_a[:, 128:128 + m]].astype(np.float64).T @ tab[big_b[:, 256:256 + n]].astype(np.float64)) * 0.5
+    assert np.abs(c1.cpu().numpy() - ref).max() <= 2e-4 * np.abs(ref).max()
+    # packed delta
+    d0 = torch.zeros((m, n), dtype=torch.int8, device="cuda"); d1 = torch.ones_like(d0)
+    t0 = torch.zeros((n // 128, m), device="cuda"); t1 = torch.ones_like(t0)
+    lib.gemm_nt(at, bt, d0, L.E4M3, L.I8, epilogue=L.EPI_ROW_TILE_MAXNORM, tile_scale=t0, tile_config=1)
+    lib.gemm_nt(akm, bkn, d1, L.E4M3, L.I8, epilogue=L.EPI_ROW_TILE_MAXNORM, tile_scale=t1, tile_config=1, m=m, n=n, k=k, k_major=True)
+    torch.cuda.synchronize()
+    assert torch.equal(d0, d1) and torch.equal(t0, t1)
+    # three stored slices of the contraction
+    s0 = torch.zeros((3, m, n), device="cuda"); s1 = torch.ones_like(s0)
+    lib.gemm_nt(at, bt, s0.view(3 * m, n), L.E4M3, L.F32, split_k=3, split_slab_bytes=m * n * 4, tile_config=1, m=m, n=n, k=k)
+    lib.gemm_nt(akm, bkn, s1.view(3 * m, n), L.E4M3, L.F32, split_k=3, split_slab_bytes=m * n * 4, tile_config=1, m=m, n=n, k=k, k_major=True)
+    torch.cuda.synchronize()
+    assert torch.equal(s0, s1)
+    assert np.abs(s1.sum(0).cpu().numpy() - ref * 2).max() <= 2e-4 * np.abs(ref).max() * 2
+    # one packed delta per group of contraction rows (the per-expert deltas; group 1 is empty, group 0 a single step)
+    offs = torch.tensor([0, 128, 128, 768, 1152], dtype=torch.int32, device="cuda")
+    g0 = torch.zeros((4 * m, n), dtype=torch.int8, device="cuda"); g1 = torch.ones_like(g0)
+    u0 = torch.zeros((n // 128, 4 * m), device="cuda"); u1 = torch.ones_like(u0)
+    kw = dict(epilogue=L.EPI_ROW_TILE_MAXNORM, tile_config=1, m=m, n=n, k=k, group_offsets=offs, groups=4, c_slab_bytes=m * n,
+              tile_scale_slab_bytes=m * 4)
+    lib.gemm_nt(at, bt, g0, L.E4M3, L.I8, tile_scale=u0, **kw)
+    lib.gemm_nt(akm, bkn, g1, L.E4M3, L.I8, tile_scale=u1, k_major=True, **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(g0, g1) and torch.equal(u0, u1) and int(g1[:m].abs().max()) > 0 and int(g1[m:2 * m].abs().max()) == 0
+    # what the variant does not take
+    TS2_ERR_UNSUPPORTED = -3
+    ai = torch.zeros((k, m), dtype=torch.int8, device="cuda"); bi = torch.zeros((k, n), dtype=torch.int8, device="cuda")
+    ci = torch.zeros((m, n), dtype=torch.int32, device="cuda")
+    assert lib.gemm_nt(ai, bi, ci, L.I8, L.I32, m=m, n=n, k=k, k_major=True, check=False) == TS2_ERR_UNSUPPORTED

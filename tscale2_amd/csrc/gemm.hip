@@ -49,6 +49,7 @@ struct GemmP {
     int splitK_groups;       // number of groups when groupOffsets is set
     int direct;              // 1: direct global->LDS loader
     int noRing;              // 1: keep the two-stage loop for the 256x256 tile (comparison)
+    int kMajor;              // 1: A is [k][m], B is [k][n] (fp8, ring kernel): operands are transposed by the LDS reads
     int mapGroup;            // M tiles per group of the tile order (an XCD's share of the tiles should be about square)
     int splits;              // >1 with splitSlab: blockIdx.y = slice of the contraction, partial product stored to c + y * splitSlab
     int64_t splitSlab;       // bytes
@@ -966,7 +967,7 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN) / 4) GemmNTDirect(Gemm
 // "all but the newest LA" (vmcnt) at the end of a step means A(S+1) and B(S+1) have landed.  Steps past the end of K reload the last
 // step (harmless: the target stage is free) so that the loop body has no branches.  The stage arrays are separate static arrays
 // (the compiler then knows that operand reads do not alias the loads in flight), hence six steps per loop iteration.
-template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(256, 1) GemmNTRing(GemmP p)
+template <int TYPE, int CT, int EPI, bool TN = false> __global__ void __launch_bounds__(256, 1) GemmNTRing(GemmP p)
 {
     typedef typename AccT<TYPE>::type TAcc;
     constexpr int WTM = 4, WTN = 4, WN = 2, NW = 4, BM = 256, BN = 256;
@@ -1003,22 +1004,27 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(256, 1) G
         kSteps = kSteps < 0 ? 0 : kSteps;
         p.c += (int64_t)blockIdx.y * p.splitSlab;
     }
-    const int lrow = wave * 8 + (lane >> 3);
-    const int lchunk = (lane & 7) ^ ((lrow >> 1) & 7);
-    const int64_t aTileOff = (int64_t)rowBase * p.lda + (int64_t)kBeg * BKB;
-    const int64_t bTileOff = (int64_t)colBase * p.ldb + (int64_t)kBeg * BKB;
+    // NT: a wave-level load fills 8 tile rows of 128 K bytes, chunks swizzled by (row / 2) % 8.
+    // K-major operands (TN): a stage is 128 K rows of 256 tile-row bytes; a wave-level load fills 4 of them, and the 32-byte granules of
+    // a row are XOR-swizzled by (K row) % 8 so that the transposing reads below (8 K rows x 32 bytes per half wave) hit every bank once.
+    const int lrow = TN ? wave * 4 + (lane >> 4) : wave * 8 + (lane >> 3);
+    const int lchunk = TN ? (((((lane & 15) >> 1) ^ (((wave & 1) << 2) | (lane >> 4))) << 1) | (lane & 1)) : (lane & 7) ^ ((lrow >> 1) & 7);
+    const int64_t aTileOff = TN ? (int64_t)kBeg * BKB * p.lda + rowBase : (int64_t)rowBase * p.lda + (int64_t)kBeg * BKB;
+    const int64_t bTileOff = TN ? (int64_t)kBeg * BKB * p.ldb + colBase : (int64_t)colBase * p.ldb + (int64_t)kBeg * BKB;
     const uint8_t *gaTile = p.a + aTileOff;
     const uint8_t *gbTile = p.b + bTileOff;
     const uint32_t gaLane = (uint32_t)(lrow * (int)p.lda + lchunk * 16);
     const uint32_t gbLane = (uint32_t)(lrow * (int)p.ldb + lchunk * 16);
     constexpr int LA = BM / (8 * NW);
     constexpr int LB = BN / (8 * NW);
+    constexpr int IROWS = TN ? 4 * NW : 8 * NW; // operand rows between two loads of a wave
     const int lastStep = kSteps - 1;
 #define RING_LOAD(GT, LD, GL, SBUF, STEP, I0, I1)                                                                                          \
     do {                                                                                                                                   \
         const int st_ = (STEP) < lastStep ? (STEP) : lastStep;                                                                             \
         _Pragma("unroll") for (int i = I0; i < I1; ++i) __builtin_amdgcn_global_load_lds(                                                  \
-            TS2_GLB_PTR(GT + ((int64_t)i * (8 * NW) * LD + (int64_t)st_ * BKB) + GL), TS2_LDS_PTR(SBUF + (wave + NW * i) * 1024), 16, 0, 0); \
+            TS2_GLB_PTR(GT + ((int64_t)i * IROWS * LD + (int64_t)st_ * (TN ? (int64_t)BKB * LD : (int64_t)BKB)) + GL),                     \
+            TS2_LDS_PTR(SBUF + (wave + NW * i) * 1024), 16, 0, 0);                                                                         \
     } while (0)
 #define RING_LOAD_A(SBUF, STEP, I0, I1) RING_LOAD(gaTile, p.lda, gaLane, SBUF, STEP, I0, I1)
 #define RING_LOAD_B(SBUF, STEP, I0, I1) RING_LOAD(gbTile, p.ldb, gbLane, SBUF, STEP, I0, I1)
@@ -1040,7 +1046,7 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(256, 1) G
     const int aRow0 = wm * (32 * WTM) + l32;
     const int bRow0 = wn * (32 * WTN) + l32;
     constexpr int NS = TYPE == T_FP8 ? 2 : 4;
-    constexpr int ND = (WTM + WTN) * (TYPE == T_FP8 ? 2 : 1); // ds_read_b128 per fragment set
+    constexpr int ND = (WTM + WTN) * (TN ? 4 : TYPE == T_FP8 ? 2 : 1); // LDS reads per fragment set
     typedef typename std::conditional<TYPE == T_FP8, v8i, v4i>::type TFrag;
     TFrag fa[2][WTM], fb[2][WTN];
     auto loadOne = [&](const uint8_t *base, int row, int sl) -> TFrag {
@@ -1062,10 +1068,47 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(256, 1) G
             return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
         }
     };
+    // K-major operands: ds_read_b64_tr_b8.  Inside a group of 16 lanes the instruction hands lane j, byte e the byte number j % 8 of
+    // the 8 bytes addressed by lane 2 * e + j / 8: with the even lanes pointing at K rows 0..7 of one 8-byte column segment and the odd
+    // lanes at the same rows of the next segment, lane j receives column j of those 8 rows - eight consecutive K slots of an MFMA
+    // operand whose row is the lane.  Four such reads (K rows 32 * half + 8 * q ..) make the 32 bytes of a 32x32x64 operand.
+    int tnA[TN ? WTM : 1], tnB[TN ? WTN : 1];
+    if constexpr (TN) {
+        const int e8 = (lane & 15) >> 1, lanePart = (32 * half + e8) * 256 + 16 * ((lane >> 4) & 1) + 8 * (lane & 1);
+#pragma unroll
+        for (int i = 0; i < WTM; ++i) {
+            tnA[i] = lanePart + (((wm * WTM + i) ^ e8) << 5);
+            asm volatile("" : "+v"(tnA[i]));
+        }
+#pragma unroll
+        for (int j = 0; j < WTN; ++j) {
+            tnB[j] = lanePart + (((wn * WTN + j) ^ e8) << 5);
+            asm volatile("" : "+v"(tnB[j]));
+        }
+    }
+    auto loadOneT = [&](const uint8_t *base, int laneOff, int sl) -> TFrag {
+        if constexpr (TYPE == T_FP8) {
+            typedef int v2i_t __attribute__((ext_vector_type(2)));
+            typedef __attribute__((address_space(3))) v2i_t *TTr8;
+            const __attribute__((address_space(3))) uint8_t *q = (const __attribute__((address_space(3))) uint8_t *)TS2_LDS_PTR(base) + sl * 64 * 256;
+            v2i_t r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((TTr8)(q + laneOff));
+            v2i_t r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((TTr8)(q + laneOff + 8 * 256));
+            v2i_t r2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((TTr8)(q + laneOff + 16 * 256));
+            v2i_t r3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((TTr8)(q + laneOff + 24 * 256));
+            return TFrag{r0[0], r0[1], r1[0], r1[1], r2[0], r2[1], r3[0], r3[1]};
+        } else {
+            return TFrag{};
+        }
+    };
 #define LOAD_FRAGS(SET, SA, SB, SL)                                                                                                        \
     do {                                                                                                                                   \
-        _Pragma("unroll") for (int i = 0; i < WTM; ++i) fa[SET][i] = loadOne(SA, aRow0 + 32 * i, SL);                                      \
-        _Pragma("unroll") for (int j = 0; j < WTN; ++j) fb[SET][j] = loadOne(SB, bRow0 + 32 * j, SL);                                      \
+        if constexpr (TN) {                                                                                                                \
+            _Pragma("unroll") for (int i = 0; i < WTM; ++i) fa[SET][i] = loadOneT(SA, tnA[i], SL);                                         \
+            _Pragma("unroll") for (int j = 0; j < WTN; ++j) fb[SET][j] = loadOneT(SB, tnB[j], SL);                                         \
+        } else {                                                                                                                           \
+            _Pragma("unroll") for (int i = 0; i < WTM; ++i) fa[SET][i] = loadOne(SA, aRow0 + 32 * i, SL);                                  \
+            _Pragma("unroll") for (int j = 0; j < WTN; ++j) fb[SET][j] = loadOne(SB, bRow0 + 32 * j, SL);                                  \
+        }                                                                                                                                  \
     } while (0)
 #define MFMA_ROWS(SET, I0, I1)                                                                                                             \
     do {                                                                                                                                   \
@@ -1455,6 +1498,16 @@ template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT> int Launch(const
             q.mapGroup = p.mapGroup ? p.mapGroup : chunk >= 64 ? 8 : chunk >= 8 ? 4 : 2;
         }
         if constexpr (WTM == 4 && WTN == 4 && !KT) {
+            if (p.kMajor) {
+                if constexpr (TYPE == T_FP8 && (CT == C_F32 || CT == C_I8PACK) && EPI == TS2_EPI_STORE) {
+                    if (!p.tileGroup && p.nSeg == 1) {
+                        hipLaunchKernelGGL((GemmNTRing<TYPE, CT, EPI, true>), dim3(nb, gy), dim3(256), 0, stream, q);
+                        TS2_CHECK_LAUNCH();
+                        return TS2_OK;
+                    }
+                }
+                return TS2_ERR_UNSUPPORTED;
+            }
             if (!p.tileGroup && !p.noRing) {
                 hipLaunchKernelGGL((GemmNTRing<TYPE, CT, EPI>), dim3(nb, gy), dim3(256), 0, stream, q);
                 TS2_CHECK_LAUNCH();
@@ -1472,11 +1525,14 @@ template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT> int Launch(const
             }
             return TS2_ERR_UNSUPPORTED;
         }
+        if (p.kMajor) {
+            return TS2_ERR_UNSUPPORTED;
+        }
         hipLaunchKernelGGL((GemmNTDirect<TYPE, WTM, WTN, CT, EPI, KT>), dim3(nb, gy), dim3(256), 0, stream, q);
         TS2_CHECK_LAUNCH();
         return TS2_OK;
     }
-    if (p.nSeg > 1) {
+    if (p.nSeg > 1 || p.kMajor) {
         return TS2_ERR_UNSUPPORTED;
     }
     hipLaunchKernelGGL(kern, dim3(nb, p.groupOffsets ? p.splitK_groups : 1), dim3(256), ldsBytes, stream, q);
@@ -1592,6 +1648,12 @@ template <int TYPE> int DispatchTile(const ts2_gemm_args *a, const GemmP &p, hip
         long tilesL = (long)(p.m / 256) * (p.n / 256) * (p.splitK > 1 ? p.splitK : 1) * (p.groupOffsets ? p.splitK_groups : 1);
         cfg = (tilesL >= 192 || p.nSeg > 1) ? 1 : 2;
     }
+    if (p.kMajor) {
+        cfg = 1; // only the 256x256 ring kernel reads contraction-major operands
+        if (a->kTileScale || p.tileGroup || (p.m % 256) || (p.n % 256)) {
+            return TS2_ERR_UNSUPPORTED;
+        }
+    }
     // the 256x256 kernel needs full tiles and has no room for the second accumulator set of the k-tile-scaled variant
     if (cfg == 1 && !a->kTileScale && !p.tileGroup && (p.m % 256) == 0 && (p.n % 256) == 0) {
         return DispatchEpi<TYPE, 4, 4>(a, p, stream);
@@ -1625,7 +1687,17 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
     if (!Aligned16(a->a.ptr, a->a.strideBytes) || !Aligned16(a->b.ptr, a->b.strideBytes) || (((uintptr_t)a->c.ptr) & 3)) {
         return TS2_ERR_ALIGN;
     }
-    if (a->a.y < a->m || a->b.y < a->n || a->a.x < a->k || a->b.x < a->k || a->c.y < a->m || a->c.x < a->n) {
+    if (a->kMajor) {
+        // rows of A and B are the contraction index: e4m3 operands on the 256x256 ring kernel only
+        if (a->abType != TS2_E4M3 || (a->m % 256) || (a->n % 256) || a->rowScale || a->kTileScale || a->tileGroup || a->extraSegments ||
+            (a->tileConfig & (2 | 4 | 8 | 16)) || (a->splitK > 1 && !a->splitSlabBytes) ||
+            !((a->cType == TS2_F32 && a->epilogue == TS2_EPI_STORE) || a->epilogue == TS2_EPI_ROW_TILE_MAXNORM)) {
+            return TS2_ERR_UNSUPPORTED;
+        }
+        if (a->a.y < a->k || a->b.y < a->k || a->a.x < a->m || a->b.x < a->n || a->c.y < a->m || a->c.x < a->n) {
+            return TS2_ERR_SHAPE;
+        }
+    } else if (a->a.y < a->m || a->b.y < a->n || a->a.x < a->k || a->b.x < a->k || a->c.y < a->m || a->c.x < a->n) {
         return TS2_ERR_SHAPE;
     }
     if (a->rowScale && (((uintptr_t)a->rowScale) & 15)) {
@@ -1726,6 +1798,7 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
     p.direct = (a->tileConfig & 4) ? 0 : 1; // bit 2 of tileConfig selects the register-staged loader (kept for comparison)
     p.mapGroup = ((a->tileConfig >> 5) & 3) == 1 ? 8 : ((a->tileConfig >> 5) & 3) == 2 ? 4 : ((a->tileConfig >> 5) & 3) == 3 ? 2 : 0;
     p.noRing = (a->tileConfig & 16) ? 1 : 0; // bit 4: two-stage loop instead of the ring for the 256x256 tile (comparison)
+    p.kMajor = a->kMajor ? 1 : 0;
     if ((a->tileGroup || a->groupOffsets) && splitK > 1) {
         return TS2_ERR_UNSUPPORTED;
     }

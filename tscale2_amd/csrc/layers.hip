@@ -315,6 +315,22 @@ int DeltaSplits(ts2_model *M, int srcDim, int dstDim)
     return splits;
 }
 
+// fp8 operands, whole 128-row groups, both widths on the 256 grid: the delta product contracts over the rows of gradient and source as
+// they lie in memory (ts2_gemm_args.kMajor), so nobody has to leave or make a transpose of either
+bool DeltaReadsRows(ts2_model *M, int srcDim, int dstDim)
+{
+    return M->mode == TS2_E4M3 && M->fastGradType == TS2_E4M3 && M->len == M->R && (srcDim % 256) == 0 && (dstDim % 256) == 0;
+}
+
+// columns [k * cols, (k + 1) * cols) of a
+Arr ColBlock(const Arr &a, int k, int cols)
+{
+    Arr r = a;
+    r.m.ptr = (uint8_t *)a.m.ptr + (size_t)k * cols * ElemSz(a.type);
+    r.m.x = cols;
+    return r;
+}
+
 // delta = alpha * gradScale * gradFast^T * src8   (TMatMulBuffers::BackpropDelta)
 int BackpropDelta(ts2_model *M, TMatrix &W, const Arr &src8, const Arr &gradFast, float alpha, const float *gradScale, void *s,
     bool sameSrcAsLastCall = false, const Arr *gradTReady = nullptr)
@@ -370,7 +386,7 @@ int FfnBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
     // contract backward
     CK(BackpropDX(M, L.w[2], M->stateGradFast, DISCR * Dot(F), true, drg, false, s));
     // fp8: the gate/norm backward also writes the transposed gradients that the two delta products contract over
-    const bool fusedT = M->mode == TS2_E4M3 && M->fastGradType == TS2_E4M3 && M->sGradTa && (R % 128) == 0;
+    const bool fusedT = !DeltaReadsRows(M, D, F) && M->mode == TS2_E4M3 && M->fastGradType == TS2_E4M3 && M->sGradTa && (R % 128) == 0;
     Arr dwideT = Flat(M->sGradTa, F, R, TS2_E4M3), dgateT = Flat(M->sGradTb, F, R, TS2_E4M3);
     if (fusedT) {
         CK(ts2_backprop_row_tile_normalize_lolu_t(len, R, gate16.P(), wide16.P(), VEC, wideScale.P(), drg.P(), dgate.P(), dwide.P(), dgateT.P(),
@@ -441,6 +457,13 @@ int AttBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
     Arr q16 = View(A.a16[0], R, Q), gate16 = View(A.a16[1], R, Q), k16 = View(A.a16[2], R, Q), v16 = View(A.a16[3], R, Q);
     Arr qScale = View(A.tsc[0], H, R), vScale = View(A.tsc[1], H, R), val16 = View(A.val16, R, Q), vlg8 = View(A.rg8, R, Q);
     Arr dvlg = View(M->g16[0], R, Q), dGate = View(M->gf[1], R, Q), dVal16 = View(M->g16[1], R, Q);
+    // one delta product for the four matrices that read the layer input, contracting over rows: their gradients are written side by side
+    // as column blocks of one [R][4Q] array (the transpose scratch, which nothing else uses then)
+    const bool stacked = L.fusedDelta && DeltaReadsRows(M, D, 4 * Q);
+    Arr gStack = Flat(M->sGradT, R, 4 * Q, M->fastGradType);
+    if (stacked) {
+        dGate = ColBlock(gStack, 3, Q);
+    }
     if (!(M->useKept && A.valid)) {
         CK(AttComputeVLG(M, L, norm8, s));
     }
@@ -477,6 +500,11 @@ int AttBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
     CK(ts2_att_backward(&ag, s));
     // epilogues: norm backward against the stored rotated vector, then inverse rope (TStoreAttBack*, gpu_att_utils.cuh:280-352)
     Arr dQf = View(M->gf[0], R, Q), dKf = View(M->gf[2], R, Q), dVf = View(M->gf[3], R, Q);
+    if (stacked) {
+        dQf = ColBlock(gStack, 0, Q);
+        dKf = ColBlock(gStack, 1, Q);
+        dVf = ColBlock(gStack, 2, Q);
+    }
     CK(ts2_backprop_row_tile_normalize_rope(len, R, dQ.P(), TS2_BF16, 1.f, q16.P(), qScale.P(), M->rope.P(), dQf.P(), M->fastGradType, s));
     CK(ts2_backprop_row_tile_normalize_rope(len, R, dK.P(), TS2_BF16, 1.f, nullptr, nullptr, M->rope.P(), dKf.P(), M->fastGradType, s));
     CK(ts2_backprop_row_tile_normalize_rope(len, R, dV.P(), TS2_BF16, 1.f, v16.P(), vScale.P(), nullptr, dVf.P(), M->fastGradType, s));
@@ -486,6 +514,9 @@ int AttBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
         const Arr *const gs[4] = {&dQf, &dKf, &dVf, &dGate};
         const bool us[4] = {true, true, true, false};
         CK(BackpropDXGroup(M, 4, ws, gs, a, us, M->dNormState, false, s));
+    }
+    if (stacked) {
+        return BackpropDelta(M, L.qkvg, norm8, gStack, VEC, gradScale, s);
     }
     if (L.fusedDelta) {
         // the four transposed gradients stacked as row blocks of one [4Q][R] array, then one delta product [4Q x D]: 256 large tiles
@@ -545,14 +576,22 @@ int GroupedDelta(ts2_model *M, TMatrix &W, const Arr &src8, const Arr &gradFast,
     bool sameSrcAsLastCall = false)
 {
     int E = M->cfg.expertCount, rows = M->lenMoe;
-    Arr gradT = Flat(M->sGradT, W.dstDim, rows, M->mode), srcT = Flat(M->sSrcT, W.srcDim, rows, M->mode);
-    CK(ts2_transpose_quant(rows, rows, gradFast.P(), M->mode, nullptr, nullptr, 0, nullptr, gradT.P(), M->mode, nullptr, s));
-    if (!sameSrcAsLastCall) { // (the expand and gate matrices share their source: one transpose)
-        CK(ts2_transpose_quant(rows, rows, src8.P(), M->mode, nullptr, nullptr, 0, nullptr, srcT.P(), M->mode, nullptr, s));
-    }
     ts2_gemm_args g = {};
-    g.a = gradT.m;
-    g.b = srcT.m;
+    if (M->fastGradType == TS2_E4M3 && (W.srcDim % 256) == 0 && (W.dstDim % 256) == 0) {
+        // every row of the expert-ordered arrays is written (pad rows of an expert's group hold zeros): contract over them as they lie
+        g.a = gradFast.m;
+        g.b = src8.m;
+        g.kMajor = 1;
+        g.tileConfig = 1;
+    } else {
+        Arr gradT = Flat(M->sGradT, W.dstDim, rows, M->mode), srcT = Flat(M->sSrcT, W.srcDim, rows, M->mode);
+        CK(ts2_transpose_quant(rows, rows, gradFast.P(), M->mode, nullptr, nullptr, 0, nullptr, gradT.P(), M->mode, nullptr, s));
+        if (!sameSrcAsLastCall) { // (the expand and gate matrices share their source: one transpose)
+            CK(ts2_transpose_quant(rows, rows, src8.P(), M->mode, nullptr, nullptr, 0, nullptr, srcT.P(), M->mode, nullptr, s));
+        }
+        g.a = gradT.m;
+        g.b = srcT.m;
+    }
     g.c = W.delta.m;
     g.c.y = W.dstDim;
     g.abType = M->mode;

@@ -164,6 +164,7 @@ extern "C" int ts2_matmul_backprop_delta(int32_t mode, int32_t len, int32_t lenR
         return TS2_ERR_UNSUPPORTED;
     }
     int rc;
+    bool kMajor = false;
     ts2_gemm_args g = {};
     if (mode == TS2_I8) {
         if (kTile <= 0 || kTile % 128 || lenRound % kTile || !buf->tileMax || !buf->tileScale) {
@@ -201,7 +202,9 @@ extern "C" int ts2_matmul_backprop_delta(int32_t mode, int32_t len, int32_t lenR
         if (gradType != TS2_E4M3) {
             return TS2_ERR_UNSUPPORTED;
         }
-        if (!buf->gradTValid) {
+        // both operands as they lie in memory, [token][feature]: the kernel's LDS reads do the transposing
+        kMajor = (len == lenRound || buf->padRowsZero) && (gradDim % 256) == 0 && (srcDim % 256) == 0 && grad->y >= lenRound && src->y >= lenRound;
+        if (!kMajor && !buf->gradTValid) {
             rc = ts2_transpose_quant(len, lenRound, grad, TS2_E4M3, nullptr, nullptr, 0, nullptr, &buf->gradT, TS2_E4M3, nullptr, stream);
             if (rc) {
                 return rc;
@@ -209,14 +212,15 @@ extern "C" int ts2_matmul_backprop_delta(int32_t mode, int32_t len, int32_t lenR
         }
     }
     const int *rowOrder = (mode == TS2_I8 && buf->sortRows) ? buf->rowOrder : nullptr;
-    if (!buf->srcTValid || rowOrder) {
+    if (!kMajor && (!buf->srcTValid || rowOrder)) {
         rc = ts2_transpose_quant(len, lenRound, src, mode, nullptr, nullptr, 0, rowOrder, &buf->srcT, mode, nullptr, stream);
         if (rc) {
             return rc;
         }
     }
-    g.a = buf->gradT;
-    g.b = buf->srcT;
+    g.a = kMajor ? *grad : buf->gradT;
+    g.b = kMajor ? *src : buf->srcT;
+    g.kMajor = kMajor ? 1 : 0;
     g.abType = mode;
     g.m = gradDim;
     g.n = srcDim;

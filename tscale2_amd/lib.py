@@ -25,7 +25,7 @@ class GemmArgs(C.Structure):
                 ("alpha", C.c_float), ("alphaPtr", C.c_void_p), ("epilogue", C.c_int32), ("tileScale", Mat), ("splitK", C.c_int32),
                 ("tileConfig", C.c_int32), ("tileGroup", C.c_void_p), ("bSlabBytes", C.c_int64), ("groupOffsets", C.c_void_p),
                 ("groups", C.c_int32), ("cSlabBytes", C.c_int64), ("tileScaleSlabBytes", C.c_int64), ("splitSlabBytes", C.c_int64), ("normalize", C.c_int32),
-                ("vecScale", C.c_float), ("rope", Mat), ("extraSegments", C.c_int32), ("segment", GemmSegment * 3)]
+                ("vecScale", C.c_float), ("rope", Mat), ("extraSegments", C.c_int32), ("segment", GemmSegment * 3), ("kMajor", C.c_int32)]
 
 
 def mat(t):
@@ -62,8 +62,9 @@ class Lib:
     def gemm_nt(self, a, b, c, ab_type, c_type, row_scale=None, k_tile_scale=None, k_tile=0, alpha=1.0, alpha_ptr=None,
                 epilogue=EPI_STORE, tile_scale=None, split_k=1, m_live=0, tile_config=0, k=None, check=True, m=None, n=None,
                 tile_group=None, b_slab_bytes=0, group_offsets=None, groups=0, c_slab_bytes=0, tile_scale_slab_bytes=0,
-                normalize=False, vec_scale=1.0, rope=None, split_slab_bytes=0, segments=()):
-        """segments: up to three further products (a_i, b_i, alpha_i, alpha_ptr_i) added into the same C in the same launch"""
+                normalize=False, vec_scale=1.0, rope=None, split_slab_bytes=0, segments=(), k_major=False):
+        """segments: up to three further products (a_i, b_i, alpha_i, alpha_ptr_i) added into the same C in the same launch;
+        k_major: a is [k][m] and b is [k][n] (pass m, n, k)"""
         args = GemmArgs()
         args.a, args.b, args.c = mat(a), mat(b), mat(c)
         args.abType, args.cType = ab_type, c_type
@@ -85,6 +86,7 @@ class Lib:
         args.normalize, args.vecScale, args.rope = int(normalize), vec_scale, mat(rope)
         args.splitSlabBytes = split_slab_bytes
         args.extraSegments = len(segments)
+        args.kMajor = int(k_major)
         for i, (sa, sb, sal, sp) in enumerate(segments):
             assert sa.stride(0) == a.stride(0) and sb.stride(0) == b.stride(0)
             args.segment[i].a, args.segment[i].b, args.segment[i].alpha, args.segment[i].alphaPtr = sa.data_ptr(), sb.data_ptr(), sal, ptr(sp)
@@ -173,7 +175,7 @@ class BwdBuffers(C.Structure):
     _fields_ = [("grad8", Mat), ("grad8RowScale", C.c_void_p), ("gradT", Mat), ("srcT", Mat), ("tileMax", C.c_void_p), ("tileScale", C.c_void_p),
                 ("transformT", Mat), ("partial", Mat), ("splits", C.c_int32), ("gradRowAbsMax", C.c_void_p),
                 ("gradRowAbsMaxValid", C.c_int32), ("srcTValid", C.c_int32), ("gradTValid", C.c_int32), ("transformTValid", C.c_int32),
-                ("rowOrder", C.c_void_p), ("rowOrderTmp", C.c_void_p), ("sortRows", C.c_int32)]
+                ("rowOrder", C.c_void_p), ("rowOrderTmp", C.c_void_p), ("sortRows", C.c_int32), ("padRowsZero", C.c_int32)]
 
 
 class MatMulBuffers:
