@@ -53,8 +53,10 @@ enum ts2_epilogue {
     /* TStoreRowTileNormalize :495-525 and TStoreRowTileNormalizeRope (src/gpt/compute/gpu_rope.cuh:25-60): cType TS2_BF16;
      * v = alpha*acc; if normalize: tileScale[n/128][m] = rms over each 128-column tile * vecScale (0 for zero tiles), v /= it;
      * if rope.ptr: rotate (even, odd) column pairs of each 128-wide head by the row's (cos, sin) table fp32 [m][128].
-     * Only the 256x256-tile kernel carries it: m, n multiples of 256 and (m/256)*(n/256) >= 192 (or tileConfig 1), else
-     * TS2_ERR_UNSUPPORTED and the caller runs ts2_row_tile_normalize_rope on a plain product. */
+     * Carried by the 256x256-tile kernel (m, n multiples of 256 and (m/256)*(n/256) >= 192, or tileConfig 1) and, for TS2_E4M3 and
+     * TS2_BF16 operands, by the 128x128-tile kernel (tileConfig 2, or implied by tileGroup: the expert-grouped expand product,
+     * MatmulExpand.Forward<TStoreRowTileNormalize>, src/gpt/compute/layer_moe.cu:160-162); else TS2_ERR_UNSUPPORTED and the caller
+     * runs ts2_row_tile_normalize_rope on a plain product. */
     TS2_EPI_ROW_TILE_NORM = 3
 };
 

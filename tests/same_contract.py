@@ -308,7 +308,7 @@ class SameContract:
                 wide16[r, k], wscale[r, k] = self.norm_rope(raw, True, VEC, None)
                 gate16[r, k] = bf16((mm(norm8[r], wg[e]) * a).astype(F32))
                 rg8[r, k] = self.q8((wide16[r, k] * lolu(gate16[r, k])).astype(F32) * wts[r, k][:, None])
-                contract[r, k] = (mm(rg8[r, k], wc[e]) * (VEC * DISCR * dot(E * X) * F32(W[2].scale))).astype(F32)
+                contract[r, k] = bf16((mm(rg8[r, k], wc[e]) * (VEC * DISCR * dot(E * X) * F32(W[2].scale))).astype(F32))
         self.acts[d] = (ids, wts, wide16, wscale, gate16, rg8)
         out = contract[:, 0]
         for k in range(1, K):
@@ -331,7 +331,7 @@ class SameContract:
                 r = np.nonzero(ids[:, k] == e)[0]
                 if not len(r):
                     continue
-                drg = (mm(sg_fast[r], wc[e].T) * f2).astype(F32)
+                drg = bf16((mm(sg_fast[r], wc[e].T) * f2).astype(F32))
                 vv = (wide16[r, k] * VEC).astype(F32)
                 mult = lolu(gate16[r, k])
                 moe = wts[r, k][:, None]
@@ -340,8 +340,8 @@ class SameContract:
                 src = (vv * rep((wscale[r, k] / VEC).astype(F32))).astype(F32)
                 dwide[r, k] = self.qfast(tile_norm_backprop(src, ((drg * mult).astype(F32) * moe).astype(F32)))
                 # expand and gate products in one launch: the sums of the first are rescaled to the second's factor, one multiply at the end
-                full[r, k] = ((mm(dwide[r, k], we[e].T).astype(np.float64) * float(f0 * F32(W[0].scale)) +
-                               mm(dgate[r, k], wg[e].T).astype(np.float64) * float(f0))).astype(F32)
+                full[r, k] = bf16(((mm(dwide[r, k], we[e].T).astype(np.float64) * float(f0 * F32(W[0].scale)) +
+                                    mm(dgate[r, k], wg[e].T).astype(np.float64) * float(f0))).astype(F32))
         # the deltas of an expert contract over all its rows, whatever their slot
         for e in range(E):
             tk = np.nonzero(ids == e)

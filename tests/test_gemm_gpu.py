@@ -223,25 +223,31 @@ def test_fused_row_tile_normalize_rope_epilogue_matches_the_two_pass_path(ab, no
     want = torch.full((m, n), 7, dtype=torch.int16, device="cuda")
     want_sc = torch.full((n // 128, m), -1.0, device="cuda")
     L.call("ts2_row_tile_normalize_rope", m_live, m, raw, L.F32, 1.0, int(normalize), 1 / 24.0, rope, want, want_sc if normalize else None)
-    got = torch.full((m, n), 9, dtype=torch.int16, device="cuda")
-    got_sc = torch.full((n // 128, m), -2.0, device="cuda")
-    lib.gemm_nt(a, b, got, t, L.BF16, alpha=alpha, m_live=m_live, tile_config=1, epilogue=L.EPI_ROW_TILE_NORM, normalize=normalize,
-                vec_scale=1 / 24.0, rope=rope, tile_scale=got_sc if normalize else None)
-    torch.cuda.synchronize()
-    gf, wf = got.view(torch.bfloat16).float(), want.view(torch.bfloat16).float()
-    assert (gf[m_live:] == 0).all() and (gf[300:310] == 0).all()
+    wf = want.view(torch.bfloat16).float()
     # one bf16 ulp, plus a few fp32 ulps of the rotation's operands: own*cos - other*sin can cancel to far below either product, and
     # the two paths round the tile sum (hence the products) differently in the last fp32 bit
     tile_max = wf.abs().view(m, n // 128, 128).amax(2, keepdim=True).expand(m, n // 128, 128).reshape(m, n)
     tol = wf.abs() * 2.0 ** -7 + tile_max * 2.0 ** -21 + 1e-30
-    assert ((gf - wf).abs() <= tol).all()
-    assert (gf == wf).float().mean() > 0.99
-    if normalize:
-        assert torch.allclose(got_sc[:, :m_live], want_sc[:, :m_live], rtol=1e-6, atol=0)
-        assert (got_sc[:, 300:310] == 0).all()
-    # unsupported with 128x128 tiles: the caller falls back to the two-pass path
-    assert lib.gemm_nt(a, b, got, t, L.BF16, tile_config=2, epilogue=L.EPI_ROW_TILE_NORM, normalize=True, vec_scale=1.0, tile_scale=got_sc,
-                       check=False) == -3
+    # the 256x256 tile (a wave holds a whole 128-column tile); e4m3 also the 128x128 tile (two waves share a tile's sums), alone and as
+    # the expert-grouped product (here every row tile names the one slab)
+    one_slab = dict(tile_group=torch.zeros(m // 128, dtype=torch.int32, device="cuda"), b_slab_bytes=n * k)
+    for cfg, extra in ((1, {}),) + (((2, {}), (2, one_slab)) if ab != "i8" else ()):
+        got = torch.full((m, n), 9, dtype=torch.int16, device="cuda")
+        got_sc = torch.full((n // 128, m), -2.0, device="cuda")
+        lib.gemm_nt(a, b, got, t, L.BF16, alpha=alpha, m_live=m_live, tile_config=cfg, epilogue=L.EPI_ROW_TILE_NORM, normalize=normalize,
+                    vec_scale=1 / 24.0, rope=rope, tile_scale=got_sc if normalize else None, n=n, **extra)
+        torch.cuda.synchronize()
+        gf = got.view(torch.bfloat16).float()
+        assert (gf[m_live:] == 0).all() and (gf[300:310] == 0).all()
+        assert ((gf - wf).abs() <= tol).all(), cfg
+        assert (gf == wf).float().mean() > 0.99
+        if normalize:
+            assert torch.allclose(got_sc[:, :m_live], want_sc[:, :m_live], rtol=1e-6, atol=0)
+            assert (got_sc[:, 300:310] == 0).all()
+    # int8 operands: unsupported with 128x128 tiles, the caller falls back to the two-pass path
+    if ab == "i8":
+        assert lib.gemm_nt(a, b, got, t, L.BF16, tile_config=2, epilogue=L.EPI_ROW_TILE_NORM, normalize=True, vec_scale=1.0, tile_scale=got_sc,
+                           check=False) == -3
 
 
 @pytest.mark.parametrize("ab,add", [("e4m3", False), ("e4m3", True), ("bf16", True)])

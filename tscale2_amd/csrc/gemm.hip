@@ -159,17 +159,16 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
         // per row and 128-column tile v = acc*scale; scale_t = rms(v)*vecScale, v /= scale_t; rotate (even, odd) column pairs by the
         // row's (cos, sin) table; bf16.  The wave's 128 columns (WTN == 4) are exactly one tile, so the reduction stays inside the
         // 32-lane group.
-        static_assert(WTN == 4 || CT != C_BF16NORM, "the normalising epilogue needs the 128-column wave tile");
+        // With the 64-column wave tile (WTN == 2) a tile's columns lie in the two waves along N: they exchange their halves of every
+        // row's sum through LDS, which the main loop no longer uses, and add them in the same order.
+        static_assert(WTN == 4 || WTN == 2 || CT != C_BF16NORM, "the normalising epilogue needs a wave tile of 64 or 128 columns");
         const int tile = (colBase + wn * (32 * WTN)) / TILE;
-#pragma unroll
-        for (int i = 0; i < WTM; ++i) {
-            // phase by phase over the 16 rows of the block row, so that the cross-lane steps and the loads of the rope table of
-            // different rows are independent instructions in flight together
-            float out[WTN][16];
-            float sum2[16];
+        const int colInTile = (wn * (32 * WTN)) & (TILE - 1);
+        float *xch = (float *)lds;
+        // sums of squares of the 16 rows of block row i over the wave's columns
+        auto blockRowSum2 = [&](int i, float (&out)[WTN][16], float (&sum2)[16]) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const int row = rowBase + rowLocal(i, e);
                 float rs = rsAll[i][e];
                 sum2[e] = 0;
 #pragma unroll
@@ -201,6 +200,38 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
                     LaneSwap16(sum2[e], &a, &b);
                     sum2[e] = a + b;
                 }
+            }
+        };
+        if (WTN == 2 && p.normalize) {
+#pragma unroll
+            for (int i = 0; i < WTM; ++i) {
+                float out[WTN][16];
+                float sum2[16];
+                blockRowSum2(i, out, sum2);
+                if (l32 == 0) {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        xch[rowLocal(i, e) * 2 + wn] = sum2[e];
+                    }
+                }
+            }
+            __syncthreads();
+        }
+#pragma unroll
+        for (int i = 0; i < WTM; ++i) {
+            // phase by phase over the 16 rows of the block row, so that the cross-lane steps and the loads of the rope table of
+            // different rows are independent instructions in flight together
+            float out[WTN][16];
+            float sum2[16];
+            blockRowSum2(i, out, sum2);
+            if (p.normalize) {
+                if (WTN == 2) {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const int rl = rowLocal(i, e);
+                        sum2[e] = xch[rl * 2] + xch[rl * 2 + 1];
+                    }
+                }
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const int row = rowBase + rowLocal(i, e);
@@ -215,7 +246,7 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
                             out[j][e] *= inv;
                         }
                     }
-                    if (l32 == 0) {
+                    if (l32 == 0 && (WTN == 4 || wn == 0)) {
                         p.tileScale[(int64_t)tile * p.ldTileScale + row] = discr;
                     }
                 }
@@ -229,7 +260,7 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
                         const int row = rowBase + rowLocal(i, eq * 4 + ee);
 #pragma unroll
                         for (int j = 0; j < WTN; ++j) {
-                            cs[ee][j] = *(const float2 *)(p.rope + (int64_t)row * p.ldRope + ((j * 32 + l32) & ~1));
+                            cs[ee][j] = *(const float2 *)(p.rope + (int64_t)row * p.ldRope + ((colInTile + j * 32 + l32) & ~1));
                         }
                     }
 #pragma unroll
@@ -1607,7 +1638,7 @@ template <int TYPE, int WTM, int WTN> int DispatchEpi(const ts2_gemm_args *a, co
         return TS2_ERR_UNSUPPORTED;
     }
     if (epi == TS2_EPI_ROW_TILE_NORM) {
-        if constexpr (WTN == 4) {
+        if constexpr (WTN == 4 || (WTM == 2 && WTN == 2 && TYPE != T_I8)) {
             if (a->cType == TS2_BF16 && !kt && p.splitK <= 1) {
                 return Launch<TYPE, WTM, WTN, C_BF16NORM, TS2_EPI_STORE, false>(p, stream);
             }

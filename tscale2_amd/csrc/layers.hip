@@ -540,7 +540,8 @@ int AttBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
 // ---------------------------------------------------------------------------------------------------------------------------
 // MoE: src/gpt/compute/layer_moe.cu:117-272 with the CPU path's factors (layer_moe.cu:458-537).  fp8 operands only.
 int GroupedGemm(ts2_model *M, const Arr &a, const Arr &bSlabs, int slabRows, int n, int k, const Arr &c, float alpha, const float *alphaPtr, bool add,
-    void *s, const Arr *a2 = nullptr, const Arr *bSlabs2 = nullptr, const float *alphaPtr2 = nullptr)
+    void *s, const Arr *a2 = nullptr, const Arr *bSlabs2 = nullptr, const float *alphaPtr2 = nullptr, const Arr *normTileScale = nullptr,
+    float normVecScale = 1.f)
 {
     ts2_gemm_args g = {};
     g.a = a.m;
@@ -558,6 +559,12 @@ int GroupedGemm(ts2_model *M, const Arr &a, const Arr &bSlabs, int slabRows, int
     g.splitK = 1;
     g.tileGroup = M->moe.xpTileExpertId;
     g.bSlabBytes = (int64_t)slabRows * bSlabs.m.strideBytes;
+    if (normTileScale) { // Forward<TStoreRowTileNormalize>: the product leaves normalised 16-bit rows and their tile scales
+        g.epilogue = TS2_EPI_ROW_TILE_NORM;
+        g.normalize = 1;
+        g.vecScale = normVecScale;
+        g.tileScale = normTileScale->m;
+    }
     if (a2) { // a second product with the same shapes and strides into the same result (its factor: alpha * *alphaPtr2)
         if (a2->m.strideBytes != a.m.strideBytes || bSlabs2->m.strideBytes != bSlabs.m.strideBytes) {
             return TS2_ERR_SHAPE;
@@ -621,10 +628,9 @@ int MoeComputeRG(ts2_model *M, TLayer &L, const Arr &norm8, void *s)
     CK(ts2_moe_route(len, RM, E, K, M->moeSel.P(), TS2_F32, &M->moe, s));
     CK(ts2_moe_group_samples(RM, 1, norm8.P(), M->moe.xpSampleId, M->normMoe.P(), s));
     TActs &A = M->shared;
-    Arr wideRaw = View(M->raw, RM, X), wide16 = View(A.a16[0], RM, X), gate16 = View(A.a16[1], RM, X), wideScale = View(A.tsc[0], X / 128, RM);
+    Arr wide16 = View(A.a16[0], RM, X), gate16 = View(A.a16[1], RM, X), wideScale = View(A.tsc[0], X / 128, RM);
     Arr rg8 = View(A.rg8, RM, X);
-    CK(GroupedGemm(M, M->normMoe, L.w[0].fast, X, X, D, wideRaw, a, L.w[0].scale, false, s));
-    CK(ts2_row_tile_normalize_rope(RM, RM, wideRaw.P(), TS2_F32, 1.f, 1, VEC, nullptr, wide16.P(), wideScale.P(), s));
+    CK(GroupedGemm(M, M->normMoe, L.w[0].fast, X, X, D, wide16, a, L.w[0].scale, false, s, nullptr, nullptr, nullptr, &wideScale, VEC));
     CK(GroupedGemm(M, M->normMoe, L.w[1].fast, X, X, D, gate16, a, nullptr, false, s));
     return ts2_matrix_lolu_moe(RM, M->moe.xpSampleWeight, gate16.P(), wide16.P(), 1.f, rg8.P(), M->mode, s);
 }
@@ -633,9 +639,10 @@ int MoeForward(ts2_model *M, TLayer &L, const Arr &norm8, void *s)
 {
     int D = M->cfg.dim, X = M->cfg.expertDim, E = M->cfg.expertCount, RM = M->lenMoe;
     CK(MoeComputeRG(M, L, norm8, s));
-    Arr contract = View(M->g32, RM, D);
+    // the experts' results travel in 16 bits (the reference's ContractResult is half, layer_moe.cu:33)
+    Arr contract = View(M->g16[0], RM, D);
     CK(GroupedGemm(M, View(M->shared.rg8, RM, X), L.w[2].fast, D, D, X, contract, VEC * DISCR * Dot(E * X), L.w[2].scale, false, s));
-    return ts2_combine_experts(M->len, M->cfg.moeSelected, contract.P(), TS2_F32, &M->moe, 1.f, nullptr, M->state.P(), 1, s);
+    return ts2_combine_experts(M->len, M->cfg.moeSelected, contract.P(), TS2_BF16, &M->moe, 1.f, nullptr, M->state.P(), 1, s);
 }
 
 int MoeBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScale, bool kept, void *s)
@@ -652,17 +659,17 @@ int MoeBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
     Arr wcT = View(M->wT, E * X, D);
     CK(ts2_transpose_u8_batched(E, D, X, L.w[2].fast.m.ptr, L.w[2].fast.m.strideBytes, (int64_t)D * L.w[2].fast.m.strideBytes, wcT.m.ptr,
         wcT.m.strideBytes, (int64_t)X * wcT.m.strideBytes, s));
-    Arr drg = View(M->g32, RM, X);
+    Arr drg = View(M->g16[0], RM, X); // 16 bits like the reference's DRG and StateGradFull (layer_moe.cu:35,46)
     CK(GroupedGemm(M, M->sgMoe, wcT, X, X, D, drg, DISCR * Dot(E * X), L.w[2].scale, false, s));
     Arr dwide = View(M->gf[0], RM, X), dgate = View(M->gf[1], RM, X);
-    CK(ts2_backprop_row_tile_normalize_lolu_moe(RM, M->moe.xpSampleWeight, gate16.P(), wide16.P(), VEC, wideScale.P(), drg.P(), TS2_F32, 1.f,
+    CK(ts2_backprop_row_tile_normalize_lolu_moe(RM, M->moe.xpSampleWeight, gate16.P(), wide16.P(), VEC, wideScale.P(), drg.P(), TS2_BF16, 1.f,
         dgate.P(), dwide.P(), M->fastGradType, M->dExpertWeight, s));
     // dExpertWeight was computed against rg in 1/24 units of nothing: vals*valsScale is the true normalised wide, so it is in true
     // (scaled-gradient) units already
     CK(ts2_backprop_moe(len, R, E, K, &M->moe, M->dExpertWeight, M->dMoeSel.P(), M->fastGradType, s));
     // expand + gate backward into grouped rows, then back to token order
     Arr weT = View(M->wT, E * D, X);
-    Arr sgFull = View(M->raw, RM, D);
+    Arr sgFull = View(M->g16[1], RM, D);
     CK(ts2_transpose_u8_batched(E, X, D, L.w[0].fast.m.ptr, L.w[0].fast.m.strideBytes, (int64_t)X * L.w[0].fast.m.strideBytes, weT.m.ptr,
         weT.m.strideBytes, (int64_t)D * weT.m.strideBytes, s));
     // the gate matrix transposed next to the expand matrix; both products in one launch (one pass over the result)
@@ -671,7 +678,7 @@ int MoeBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
     CK(ts2_transpose_u8_batched(E, X, D, L.w[1].fast.m.ptr, L.w[1].fast.m.strideBytes, (int64_t)X * L.w[1].fast.m.strideBytes, wgT.m.ptr,
         wgT.m.strideBytes, (int64_t)D * wgT.m.strideBytes, s));
     CK(GroupedGemm(M, dwide, weT, D, D, X, sgFull, DISCR * Dot(D), L.w[0].scale, false, s, &dgate, &wgT, nullptr));
-    CK(ts2_combine_experts(len, K, sgFull.P(), TS2_F32, &M->moe, 1.f, nullptr, M->dNormState.P(), 0, s));
+    CK(ts2_combine_experts(len, K, sgFull.P(), TS2_BF16, &M->moe, 1.f, nullptr, M->dNormState.P(), 0, s));
     // select matrix: dNormState += dMoe * Wsel / sqrt(D) and its delta through the same 8-bit operator as every other matrix (the
     // reference uses its fp16 kernels here, MatmulSelect.BackpropFp16, layer_moe.cu:264); rows >= experts of the matrix are zero
     CK(BackpropDX(M, L.w[3], M->dMoeSel, DISCR * Dot(D), false, M->dNormState, true, s));
