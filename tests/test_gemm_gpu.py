@@ -434,6 +434,75 @@ def test_products_with_a_zero_factor_contribute_nothing(zero_at):
         assert torch.isfinite(got2).all() and (got2 - want2).abs().max().item() <= 4e-6 * max(want2.abs().max().item(), 1e-30), za
 
 
+def test_ring_pipeline_on_the_small_tile_equals_the_two_stage_loop(lib):
+    """The 128x128 tile has two kernels for e4m3 operands: the two-stage loop and the ring pipeline (three A and two B stages, two
+    workgroups per CU), chosen by the contraction length (tileConfig bit 7 / bit 4 force one or the other).  Both feed the MFMAs the
+    same operands in the same order, so every result type must come out bit-identical: fp32 stored and accumulated (contractions of
+    1 .. 16 steps, live rows short of m), bf16, the packed delta, the normalising epilogue, the expert-grouped product with a skipped
+    row tile, and two grouped products into one result."""
+    print("case small-tile ring", flush=True)
+    from tscale2_amd import lib as L
+    RING, LOOP = 2 | 128, 2 | 16
+    g = torch.Generator(device="cuda").manual_seed(3)
+
+    def codes(shape):  # e4m3 bytes without the NaN codes, both signs
+        return (torch.randint(0, 120, shape, device="cuda", generator=g) | (torch.randint(0, 2, shape, device="cuda", generator=g) << 7)).to(torch.uint8)
+
+    def both(fn, outs, skip_rows=None, loop=LOOP):
+        res = []
+        for cfg, fill in ((loop, 0), (RING, 1)):
+            for o in outs:
+                o.fill_(fill)
+            fn(cfg)
+            torch.cuda.synchronize()
+            res.append([o.clone() for o in outs])
+        for a, b in zip(*res):
+            if skip_rows is not None:   # rows of a skipped tile keep what the buffer held
+                a[skip_rows] = 0; b[skip_rows] = 0
+            assert torch.equal(a, b)
+        assert float(res[0][0].float().abs().max()) > 0
+    for k in (128, 256, 384, 768, 1152, 2048):
+        m, n = 384, 256
+        a, b = codes((m, k)), codes((n, k))
+        c = torch.zeros((m, n), device="cuda")
+        both(lambda cfg: lib.gemm_nt(a, b, c, L.E4M3, L.F32, alpha=0.25, tile_config=cfg, m_live=300), [c])
+    m, n, k = 640, 384, 896
+    a, b = codes((m, k)), codes((n, k))
+    c16 = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+    both(lambda cfg: lib.gemm_nt(a, b, c16, L.E4M3, L.BF16, alpha=0.25, tile_config=cfg), [c16])
+    cadd = torch.zeros((m, n), device="cuda")
+    start = torch.randn((m, n), device="cuda", generator=g)
+
+    def add(cfg):
+        cadd.copy_(start)
+        lib.gemm_nt(a, b, cadd, L.E4M3, L.F32, alpha=0.25, tile_config=cfg, epilogue=L.EPI_ADD)
+    both(add, [cadd])
+    d8 = torch.zeros((m, n), dtype=torch.int8, device="cuda"); ts = torch.zeros((n // 128, m), device="cuda")
+    both(lambda cfg: lib.gemm_nt(a, b, d8, L.E4M3, L.I8, tile_config=cfg, epilogue=L.EPI_ROW_TILE_MAXNORM, tile_scale=ts), [d8, ts])
+    cn = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda"); tn = torch.zeros((n // 128, m), device="cuda")
+    both(lambda cfg: lib.gemm_nt(a, b, cn, L.E4M3, L.BF16, alpha=0.3, tile_config=cfg, epilogue=L.EPI_ROW_TILE_NORM, normalize=True,
+                                 vec_scale=1 / 24.0, tile_scale=tn), [cn, tn])
+    slabs = 3
+    bs = codes((slabs * n, k))
+    tg = torch.tensor([2, 0, -1, 1, 2], dtype=torch.int32, device="cuda")
+    cg = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+    skipped = slice(256, 384)
+    both(lambda cfg: lib.gemm_nt(a, bs, cg, L.E4M3, L.BF16, n=n, tile_config=cfg, tile_group=tg, b_slab_bytes=n * k), [cg], skipped)
+    a2, bs2 = codes((m, k)), codes((slabs * n, k))
+    sc1 = torch.tensor([0.7], device="cuda"); sc2 = torch.tensor([1.9], device="cuda")
+    both(lambda cfg: lib.gemm_nt(a, bs, cg, L.E4M3, L.BF16, n=n, alpha=0.1, alpha_ptr=sc1, tile_config=cfg, tile_group=tg, b_slab_bytes=n * k,
+                                 segments=[(a2, bs2, 0.1, sc2)]), [cg], skipped, loop=2)  # (k < 1024: the loop is the library's choice)
+    # the grouped product against a plain product per row tile
+    want = torch.zeros((m, n), device="cuda")
+    for t, e in enumerate(tg.tolist()):
+        if e >= 0:
+            lib.gemm_nt(a[t * 128:(t + 1) * 128], bs[e * n:(e + 1) * n], want[t * 128:(t + 1) * 128], L.E4M3, L.F32, tile_config=LOOP)
+    got = torch.zeros((m, n), device="cuda")
+    lib.gemm_nt(a, bs, got, L.E4M3, L.F32, n=n, tile_config=RING, tile_group=tg, b_slab_bytes=n * k)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+
+
 def test_contraction_major_operands_equal_the_transposed_product(lib, orc):
     """kMajor: A [k][m], B [k][n] (the untransposed activations of a delta product) against the same product on explicitly transposed
     operands.  Both feed the MFMAs the same operand bytes in the same contraction slots, so fp32 results, stored slices and packed

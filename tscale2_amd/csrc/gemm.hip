@@ -50,6 +50,7 @@ struct GemmP {
     int direct;              // 1: direct global->LDS loader
     int noRing;              // 1: keep the two-stage loop for the 256x256 tile (comparison)
     int kMajor;              // 1: A is [k][m], B is [k][n] (fp8, ring kernel): operands are transposed by the LDS reads
+    int ring128;             // 128x128 tile: the ring pipeline (two workgroups per CU) instead of the two-stage loop
     int mapGroup;            // M tiles per group of the tile order (an XCD's share of the tiles should be about square)
     int splits;              // >1 with splitSlab: blockIdx.y = slice of the contraction, partial product stored to c + y * splitSlab
     int64_t splitSlab;       // bytes
@@ -998,10 +999,14 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN) / 4) GemmNTDirect(Gemm
 // "all but the newest LA" (vmcnt) at the end of a step means A(S+1) and B(S+1) have landed.  Steps past the end of K reload the last
 // step (harmless: the target stage is free) so that the loop body has no branches.  The stage arrays are separate static arrays
 // (the compiler then knows that operand reads do not alias the loads in flight), hence six steps per loop iteration.
-template <int TYPE, int CT, int EPI, bool TN = false> __global__ void __launch_bounds__(256, 1) GemmNTRing(GemmP p)
+// WT = 2 is the same pipeline on a 128x128 tile (wave tile 64x64): the stages are 16 KB, the ring 80 KB, and two workgroups share a
+// CU, so that one's start-up and stores fall into the other's main loop - for products whose workgroups are short (a contraction of
+// 512 .. 2048 bytes: the expert-grouped products, whose 128-row tiles each take their expert's slab of B, tileGroup).  e4m3 only.
+template <int TYPE, int CT, int EPI, bool TN = false, int WT = 4> __global__ void __launch_bounds__(256, WT == 4 ? 1 : 2) GemmNTRing(GemmP p)
 {
     typedef typename AccT<TYPE>::type TAcc;
-    constexpr int WTM = 4, WTN = 4, WN = 2, NW = 4, BM = 256, BN = 256;
+    constexpr int WTM = WT, WTN = WT, WN = 2, NW = 4, BM = 64 * WT, BN = 64 * WT;
+    static_assert(WT == 4 || (WT == 2 && TYPE == T_FP8 && !TN), "the 128x128 ring takes e4m3 operands with the contraction along the rows");
     __shared__ __attribute__((aligned(1024))) uint8_t sA0[BM * BKB];
     __shared__ __attribute__((aligned(1024))) uint8_t sA1[BM * BKB];
     __shared__ __attribute__((aligned(1024))) uint8_t sA2[BM * BKB];
@@ -1041,7 +1046,17 @@ template <int TYPE, int CT, int EPI, bool TN = false> __global__ void __launch_b
     const int lrow = TN ? wave * 4 + (lane >> 4) : wave * 8 + (lane >> 3);
     const int lchunk = TN ? (((((lane & 15) >> 1) ^ (((wave & 1) << 2) | (lane >> 4))) << 1) | (lane & 1)) : (lane & 7) ^ ((lrow >> 1) & 7);
     const int64_t aTileOff = TN ? (int64_t)kBeg * BKB * p.lda + rowBase : (int64_t)rowBase * p.lda + (int64_t)kBeg * BKB;
-    const int64_t bTileOff = TN ? (int64_t)kBeg * BKB * p.ldb + colBase : (int64_t)colBase * p.ldb + (int64_t)kBeg * BKB;
+    int64_t bTileOff = TN ? (int64_t)kBeg * BKB * p.ldb + colBase : (int64_t)colBase * p.ldb + (int64_t)kBeg * BKB;
+    if constexpr (WT == 2) {
+        if (p.tileGroup) {
+            // the rows of a 128-row tile belong to one group; every B operand of the launch is taken from that group's slab
+            const int g = p.tileGroup[rowBase / TILE];
+            if (g < 0) {
+                return;
+            }
+            bTileOff += (int64_t)g * p.bSlab;
+        }
+    }
     const uint8_t *gaTile = p.a + aTileOff;
     const uint8_t *gbTile = p.b + bTileOff;
     const uint32_t gaLane = (uint32_t)(lrow * (int)p.lda + lchunk * 16);
@@ -1178,7 +1193,7 @@ template <int TYPE, int CT, int EPI, bool TN = false> __global__ void __launch_b
         LOAD_FRAGS(1, CA, CB, 1);                                                                                                          \
         MFMA_ROWS(0, 0, WTM);                                                                                                              \
         if constexpr (NS == 2) {                                                                                                           \
-            INTERLEAVE(16, 1, 1, ND / 16);                                                                                                 \
+            INTERLEAVE(WTM * WTN, 1, (LA + LB) / (WTM * WTN), ND / (WTM * WTN));                                                           \
         } else {                                                                                                                           \
             INTERLEAVE(8, 2, 1, ND / 8);                                                                                                   \
         }                                                                                                                                  \
@@ -1205,7 +1220,7 @@ template <int TYPE, int CT, int EPI, bool TN = false> __global__ void __launch_b
         MFMA_ROWS(1, WTM / 2, WTM);                                                                                                        \
     } while (0)
 
-    static_assert(LA == 8 && LB == 8, "vmcnt immediate below assumes eight loads per operand stage");
+    static_assert(LA == 2 * WT && LB == 2 * WT, "the vmcnt immediate of the step barrier is the number of loads of an A stage");
     // several products into the same accumulators: one pass of the pipeline per product (the stage rotation restarts), the fp32 sums
     // rescaled in between so that the epilogue's single factor, the last product's, is right for all of them
     // `units`: the factor the accumulators have to be multiplied with in the end = the factor of the product that ran last.  A product
@@ -1545,6 +1560,13 @@ template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT> int Launch(const
                 return TS2_OK;
             }
         }
+        if constexpr (WTM == 2 && WTN == 2 && !KT && TYPE == T_FP8 && CT != C_I32) {
+            if (p.ring128 && !p.kMajor) {
+                hipLaunchKernelGGL((GemmNTRing<TYPE, CT, EPI, false, 2>), dim3(nb, gy), dim3(256), 0, stream, q);
+                TS2_CHECK_LAUNCH();
+                return TS2_OK;
+            }
+        }
         if (p.nSeg > 1) {
             // several products per launch: the ring kernel, or two products on the 128x128 tile (fp32 / bf16 results)
             if constexpr (WTM == 2 && WTN == 2 && !KT && TYPE != T_I8 && (CT == C_F32 || CT == C_BF16)) {
@@ -1830,6 +1852,9 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
     p.mapGroup = ((a->tileConfig >> 5) & 3) == 1 ? 8 : ((a->tileConfig >> 5) & 3) == 2 ? 4 : ((a->tileConfig >> 5) & 3) == 3 ? 2 : 0;
     p.noRing = (a->tileConfig & 16) ? 1 : 0; // bit 4: two-stage loop instead of the ring for the 256x256 tile (comparison)
     p.kMajor = a->kMajor ? 1 : 0;
+    // 128x128 tile, e4m3: the ring pipeline from a contraction of eight steps on (measured on the expert-grouped products: 136 -> 120 us
+    // at K = 1024, no gain at K = 512); bit 7 of tileConfig asks for it at any length, bit 4 for the two-stage loop
+    p.ring128 = !(a->tileConfig & 16) && ((a->tileConfig & 128) || (int64_t)a->k * esz >= 8 * BKB) ? 1 : 0;
     if ((a->tileGroup || a->groupOffsets) && splitK > 1) {
         return TS2_ERR_UNSUPPORTED;
     }
