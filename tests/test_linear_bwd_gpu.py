@@ -144,6 +144,24 @@ def test_fp8_linear_backward(L, orc):
     err = np.abs(got_delta - ref_delta).max() / np.abs(ref_delta).max()
     print("fp8 delta rel err", err)
     assert err <= 5e-3
+    # the caller's word that the pad rows hold zeros (they do: xd, dyd above): the delta product reads both arrays as they lie,
+    # transposes nothing (the transpose scratch keeps its marker bytes) and gives the same bytes and tile scales
+    rows = L.MatMulBuffers(L.E4M3, len_round, src_dim, grad_dim)
+    rows.c.padRowsZero = 1
+    rows.t["gradT"].fill_(0x5A); rows.t["srcT"].fill_(0x5A)
+    rows.delta.fill_(77); rows.delta_tile_scale.fill_(-1)
+    rows.backprop_delta(len_, xd, None, dyd, L.E4M3, gscale)
+    torch.cuda.synchronize()
+    assert torch.equal(rows.delta, bufs.delta) and torch.equal(rows.delta_tile_scale, bufs.delta_tile_scale)
+    assert (rows.t["gradT"] == 0x5A).all() and (rows.t["srcT"] == 0x5A).all()
+    assert not (bufs.t["gradT"] == 0x5A).all()            # the transposing sequence did write its scratch
+    # whole 128-row groups: the same without the flag
+    full = L.MatMulBuffers(L.E4M3, len_round, src_dim, grad_dim)
+    full.t["gradT"].fill_(0x5A)
+    full.backprop_delta(len_round, xd, None, dyd, L.E4M3, gscale)
+    torch.cuda.synchronize()
+    assert torch.equal(full.delta, bufs.delta) and torch.equal(full.delta_tile_scale, bufs.delta_tile_scale)
+    assert (full.t["gradT"] == 0x5A).all()
 
 
 @pytest.mark.parametrize("dims", [(256, 512), (384, 128)])
