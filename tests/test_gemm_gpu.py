@@ -434,6 +434,39 @@ def test_products_with_a_zero_factor_contribute_nothing(zero_at):
         assert torch.isfinite(got2).all() and (got2 - want2).abs().max().item() <= 4e-6 * max(want2.abs().max().item(), 1e-30), za
 
 
+def test_contraction_major_bf16_operands_equal_the_transposed_product(lib):
+    """kMajor with bf16 operands (the delta of the final layer: gradient [token][vocab] and final state [token][dim] as they lie, the
+    reference's Fp16MatMul<1, 1, TStoreDelta>, src/gpt/compute/gpu_final.cuh:265): bit-identical to the product of the explicitly
+    transposed operands, for the fp32 store, the packed delta and stored slices; strided views, 9 contraction steps."""
+    print("case contraction-major bf16 operands", flush=True)
+    from tscale2_amd import lib as L
+    m, n, k = 512, 768, 576
+    g = torch.Generator(device="cuda").manual_seed(32)
+    big_a = torch.randn((k, m + 256), device="cuda", generator=g).bfloat16()
+    big_b = torch.randn((k, n + 512), device="cuda", generator=g).bfloat16()
+    akm, bkn = big_a[:, 128:128 + m], big_b[:, 256:256 + n]      # [k][m], [k][n] views with larger row strides
+    at, bt = akm.t().contiguous(), bkn.t().contiguous()
+    c0 = torch.zeros((m, n), device="cuda"); c1 = torch.ones((m, n), device="cuda")
+    lib.gemm_nt(at, bt, c0, L.BF16, L.F32, alpha=0.5, tile_config=1)
+    lib.gemm_nt(akm, bkn, c1, L.BF16, L.F32, alpha=0.5, tile_config=1, m=m, n=n, k=k, k_major=True)
+    torch.cuda.synchronize()
+    assert torch.equal(c0, c1)
+    ref = (akm.double().t() @ bkn.double()) * 0.5
+    assert float((c1.double() - ref).abs().max()) <= 1e-5 * float(ref.abs().max())
+    d0 = torch.zeros((m, n), dtype=torch.int8, device="cuda"); d1 = torch.ones_like(d0)
+    t0 = torch.zeros((n // 128, m), device="cuda"); t1 = torch.ones_like(t0)
+    lib.gemm_nt(at, bt, d0, L.BF16, L.I8, epilogue=L.EPI_ROW_TILE_MAXNORM, tile_scale=t0, tile_config=1)
+    lib.gemm_nt(akm, bkn, d1, L.BF16, L.I8, epilogue=L.EPI_ROW_TILE_MAXNORM, tile_scale=t1, tile_config=1, m=m, n=n, k=k, k_major=True)
+    torch.cuda.synchronize()
+    assert torch.equal(d0, d1) and torch.equal(t0, t1) and int(d1.abs().max()) == 127
+    s0 = torch.zeros((3, m, n), device="cuda"); s1 = torch.ones_like(s0)
+    lib.gemm_nt(at, bt, s0.view(3 * m, n), L.BF16, L.F32, split_k=3, split_slab_bytes=m * n * 4, tile_config=1, m=m, n=n, k=k)
+    lib.gemm_nt(akm, bkn, s1.view(3 * m, n), L.BF16, L.F32, split_k=3, split_slab_bytes=m * n * 4, tile_config=1, m=m, n=n, k=k, k_major=True)
+    torch.cuda.synchronize()
+    assert torch.equal(s0, s1)
+    assert float((s1.sum(0).double() - ref * 2).abs().max()) <= 1e-5 * float(ref.abs().max()) * 2
+
+
 def test_ring_pipeline_on_the_small_tile_equals_the_two_stage_loop(lib):
     """The 128x128 tile has two kernels for e4m3 operands: the two-stage loop and the ring pipeline (three A and two B stages, two
     workgroups per CU), chosen by the contraction length (tileConfig bit 7 / bit 4 force one or the other).  Both feed the MFMAs the

@@ -1007,6 +1007,9 @@ template <int TYPE, int CT, int EPI, bool TN = false, int WT = 4> __global__ voi
     typedef typename AccT<TYPE>::type TAcc;
     constexpr int WTM = WT, WTN = WT, WN = 2, NW = 4, BM = 64 * WT, BN = 64 * WT;
     static_assert(WT == 4 || (WT == 2 && TYPE == T_FP8 && !TN), "the 128x128 ring takes e4m3 operands with the contraction along the rows");
+    static_assert(!TN || TYPE != T_I8, "contraction-major operands: e4m3 and bf16");
+    constexpr int ESZ = TYPE == T_BF16 ? 2 : 1;
+    constexpr int KR = BKB / ESZ; // contraction rows of a step (K-major operands)
     __shared__ __attribute__((aligned(1024))) uint8_t sA0[BM * BKB];
     __shared__ __attribute__((aligned(1024))) uint8_t sA1[BM * BKB];
     __shared__ __attribute__((aligned(1024))) uint8_t sA2[BM * BKB];
@@ -1041,12 +1044,16 @@ template <int TYPE, int CT, int EPI, bool TN = false, int WT = 4> __global__ voi
         p.c += (int64_t)blockIdx.y * p.splitSlab;
     }
     // NT: a wave-level load fills 8 tile rows of 128 K bytes, chunks swizzled by (row / 2) % 8.
-    // K-major operands (TN): a stage is 128 K rows of 256 tile-row bytes; a wave-level load fills 4 of them, and the 32-byte granules of
-    // a row are XOR-swizzled by (K row) % 8 so that the transposing reads below (8 K rows x 32 bytes per half wave) hit every bank once.
-    const int lrow = TN ? wave * 4 + (lane >> 4) : wave * 8 + (lane >> 3);
-    const int lchunk = TN ? (((((lane & 15) >> 1) ^ (((wave & 1) << 2) | (lane >> 4))) << 1) | (lane & 1)) : (lane & 7) ^ ((lrow >> 1) & 7);
-    const int64_t aTileOff = TN ? (int64_t)kBeg * BKB * p.lda + rowBase : (int64_t)rowBase * p.lda + (int64_t)kBeg * BKB;
-    int64_t bTileOff = TN ? (int64_t)kBeg * BKB * p.ldb + colBase : (int64_t)colBase * p.ldb + (int64_t)kBeg * BKB;
+    // K-major operands (TN), e4m3: a stage is 128 K rows of 256 tile-row bytes; a wave-level load fills 4 of them, and the 32-byte
+    // granules of a row are XOR-swizzled by (K row) % 8 so that the transposing reads below (8 K rows x 32 bytes per half wave) hit
+    // every bank once.  bf16: 64 K rows of 512 bytes, two per wave-level load; the 64-byte granules (32 tile rows) are XOR-swizzled by
+    // (K row) % 4: a half wave of the 16-bit transposing read takes 64 bytes from each of 4 consecutive K rows.
+    const int lrow = !TN ? wave * 8 + (lane >> 3) : TYPE == T_BF16 ? wave * 2 + (lane >> 5) : wave * 4 + (lane >> 4);
+    const int lchunk = !TN               ? (lane & 7) ^ ((lrow >> 1) & 7)
+                       : TYPE == T_BF16 ? (lane & 31) ^ ((lrow & 3) << 2)
+                                        : (((((lane & 15) >> 1) ^ (((wave & 1) << 2) | (lane >> 4))) << 1) | (lane & 1));
+    const int64_t aTileOff = TN ? (int64_t)kBeg * KR * p.lda + rowBase * ESZ : (int64_t)rowBase * p.lda + (int64_t)kBeg * BKB;
+    int64_t bTileOff = TN ? (int64_t)kBeg * KR * p.ldb + colBase * ESZ : (int64_t)colBase * p.ldb + (int64_t)kBeg * BKB;
     if constexpr (WT == 2) {
         if (p.tileGroup) {
             // the rows of a 128-row tile belong to one group; every B operand of the launch is taken from that group's slab
@@ -1063,13 +1070,13 @@ template <int TYPE, int CT, int EPI, bool TN = false, int WT = 4> __global__ voi
     const uint32_t gbLane = (uint32_t)(lrow * (int)p.ldb + lchunk * 16);
     constexpr int LA = BM / (8 * NW);
     constexpr int LB = BN / (8 * NW);
-    constexpr int IROWS = TN ? 4 * NW : 8 * NW; // operand rows between two loads of a wave
+    constexpr int IROWS = !TN ? 8 * NW : TYPE == T_BF16 ? 2 * NW : 4 * NW; // operand rows between two loads of a wave
     const int lastStep = kSteps - 1;
 #define RING_LOAD(GT, LD, GL, SBUF, STEP, I0, I1)                                                                                          \
     do {                                                                                                                                   \
         const int st_ = (STEP) < lastStep ? (STEP) : lastStep;                                                                             \
         _Pragma("unroll") for (int i = I0; i < I1; ++i) __builtin_amdgcn_global_load_lds(                                                  \
-            TS2_GLB_PTR(GT + ((int64_t)i * IROWS * LD + (int64_t)st_ * (TN ? (int64_t)BKB * LD : (int64_t)BKB)) + GL),                     \
+            TS2_GLB_PTR(GT + ((int64_t)i * IROWS * LD + (int64_t)st_ * (TN ? (int64_t)KR * LD : (int64_t)BKB)) + GL),                      \
             TS2_LDS_PTR(SBUF + (wave + NW * i) * 1024), 16, 0, 0);                                                                         \
     } while (0)
 #define RING_LOAD_A(SBUF, STEP, I0, I1) RING_LOAD(gaTile, p.lda, gaLane, SBUF, STEP, I0, I1)
@@ -1092,7 +1099,7 @@ template <int TYPE, int CT, int EPI, bool TN = false, int WT = 4> __global__ voi
     const int aRow0 = wm * (32 * WTM) + l32;
     const int bRow0 = wn * (32 * WTN) + l32;
     constexpr int NS = TYPE == T_FP8 ? 2 : 4;
-    constexpr int ND = (WTM + WTN) * (TN ? 4 : TYPE == T_FP8 ? 2 : 1); // LDS reads per fragment set
+    constexpr int ND = (WTM + WTN) * (TN ? (TYPE == T_FP8 ? 4 : 2) : TYPE == T_FP8 ? 2 : 1); // LDS reads per fragment set
     typedef typename std::conditional<TYPE == T_FP8, v8i, v4i>::type TFrag;
     TFrag fa[2][WTM], fb[2][WTN];
     auto loadOne = [&](const uint8_t *base, int row, int sl) -> TFrag {
@@ -1118,8 +1125,23 @@ template <int TYPE, int CT, int EPI, bool TN = false, int WT = 4> __global__ voi
     // the 8 bytes addressed by lane 2 * e + j / 8: with the even lanes pointing at K rows 0..7 of one 8-byte column segment and the odd
     // lanes at the same rows of the next segment, lane j receives column j of those 8 rows - eight consecutive K slots of an MFMA
     // operand whose row is the lane.  Four such reads (K rows 32 * half + 8 * q ..) make the 32 bytes of a 32x32x64 operand.
+    // bf16: ds_read_b64_tr_b16 hands lane j, element e the 16-bit value number j % 4 of the 8 bytes addressed by lane 4 * e + j / 4 of
+    // its group of 16: lanes 4e .. 4e+3 point at K row e, four tile rows each, and lane j receives tile row j of K rows 0..3; two reads
+    // (K rows 8 * half + 4 * r ..) make the eight contraction slots of a 32x32x16 operand.
     int tnA[TN ? WTM : 1], tnB[TN ? WTN : 1];
-    if constexpr (TN) {
+    if constexpr (TN && TYPE == T_BF16) {
+        const int e4 = (lane & 15) >> 2, lanePart = (8 * half + e4) * 512 + 32 * ((lane >> 4) & 1) + 8 * (lane & 3);
+#pragma unroll
+        for (int i = 0; i < WTM; ++i) {
+            tnA[i] = lanePart + (((wm * WTM + i) ^ e4) << 6);
+            asm volatile("" : "+v"(tnA[i]));
+        }
+#pragma unroll
+        for (int j = 0; j < WTN; ++j) {
+            tnB[j] = lanePart + (((wn * WTN + j) ^ e4) << 6);
+            asm volatile("" : "+v"(tnB[j]));
+        }
+    } else if constexpr (TN) {
         const int e8 = (lane & 15) >> 1, lanePart = (32 * half + e8) * 256 + 16 * ((lane >> 4) & 1) + 8 * (lane & 1);
 #pragma unroll
         for (int i = 0; i < WTM; ++i) {
@@ -1142,6 +1164,14 @@ template <int TYPE, int CT, int EPI, bool TN = false, int WT = 4> __global__ voi
             v2i_t r2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((TTr8)(q + laneOff + 16 * 256));
             v2i_t r3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((TTr8)(q + laneOff + 24 * 256));
             return TFrag{r0[0], r0[1], r1[0], r1[1], r2[0], r2[1], r3[0], r3[1]};
+        } else if constexpr (TYPE == T_BF16) {
+            typedef short v4s_t __attribute__((ext_vector_type(4)));
+            typedef int v2i_t __attribute__((ext_vector_type(2)));
+            typedef __attribute__((address_space(3))) v4s_t *TTr16;
+            const __attribute__((address_space(3))) uint8_t *q = (const __attribute__((address_space(3))) uint8_t *)TS2_LDS_PTR(base) + sl * 16 * 512;
+            v2i_t r0 = __builtin_bit_cast(v2i_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((TTr16)(q + laneOff)));
+            v2i_t r1 = __builtin_bit_cast(v2i_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((TTr16)(q + laneOff + 4 * 512)));
+            return TFrag{r0[0], r0[1], r1[0], r1[1]};
         } else {
             return TFrag{};
         }
@@ -1545,7 +1575,7 @@ template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT> int Launch(const
         }
         if constexpr (WTM == 4 && WTN == 4 && !KT) {
             if (p.kMajor) {
-                if constexpr (TYPE == T_FP8 && (CT == C_F32 || CT == C_I8PACK) && EPI == TS2_EPI_STORE) {
+                if constexpr ((TYPE == T_FP8 || TYPE == T_BF16) && (CT == C_F32 || CT == C_I8PACK) && EPI == TS2_EPI_STORE) {
                     if (!p.tileGroup && p.nSeg == 1) {
                         hipLaunchKernelGGL((GemmNTRing<TYPE, CT, EPI, true>), dim3(nb, gy), dim3(256), 0, stream, q);
                         TS2_CHECK_LAUNCH();
@@ -1741,8 +1771,8 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
         return TS2_ERR_ALIGN;
     }
     if (a->kMajor) {
-        // rows of A and B are the contraction index: e4m3 operands on the 256x256 ring kernel only
-        if (a->abType != TS2_E4M3 || (a->m % 256) || (a->n % 256) || a->rowScale || a->kTileScale || a->tileGroup || a->extraSegments ||
+        // rows of A and B are the contraction index: e4m3 or bf16 operands on the 256x256 ring kernel only
+        if ((a->abType != TS2_E4M3 && a->abType != TS2_BF16) || (a->m % 256) || (a->n % 256) || a->rowScale || a->kTileScale || a->tileGroup || a->extraSegments ||
             (a->tileConfig & (2 | 4 | 8 | 16)) || (a->splitK > 1 && !a->splitSlabBytes) ||
             !((a->cType == TS2_F32 && a->epilogue == TS2_EPI_STORE) || a->epilogue == TS2_EPI_ROW_TILE_MAXNORM)) {
             return TS2_ERR_UNSUPPORTED;

@@ -11,6 +11,7 @@ int Ts2FinalSoftmaxGrad(int rows, int vocab, const ts2_mat *logits, const float 
 int Ts2FinalSoftmaxGradHalf(int rows, int vocab, const ts2_mat *logits, const float *bias, const int *target, float gradMult, const ts2_mat *grad,
     float *lossSum, void *stream);
 int Ts2TransposeToBf16(int rows, int rowsRound, int cols, const ts2_mat *src, int srcType, const ts2_mat *dst, void *stream);
+int Ts2RowsToBf16(int rows, int rowsRound, int cols, const ts2_mat *src, int srcType, const ts2_mat *dst, void *stream);
 int Ts2ZeroRows(const ts2_mat *m, int rows, int rowBytes, void *stream);
 int Ts2FillFloats(float *p, int n, float v, void *stream);
 // ts2_transpose_quant with the k-tile maxima formed in the kernel from row maxima (rowAbsMax) when tileMax is null

@@ -782,7 +782,10 @@ int FinalBackward(ts2_model *M, void *s)
     CK(Ts2FinalSoftmaxGradHalf(R, V, M->logits16.P(), M->bias, M->target, 1.f, M->gradV.P(), M->lossSum, s));
     // dfn = grad * Wf / sqrt(D): bf16 product, the 8-bit weights converted exactly
     // (columns V..VP of the logits are products with zero rows, the same columns of the gradient stay zero: the softmax pass covers V)
-    CK(Ts2TransposeToBf16(VP, VP, D, M->finalW.fast.P(), M->mode, M->wfT.P(), s));
+    if (!M->finalW.fastTValid) { // kept until the matrix is set or updated, like the layer matrices' transposes
+        CK(Ts2TransposeToBf16(VP, VP, D, M->finalW.fast.P(), M->mode, M->wfT.P(), s));
+        M->finalW.fastTValid = true;
+    }
     ts2_gemm_args g = {};
     g.a = M->gradV.m;
     g.b = M->wfT.m;
@@ -799,11 +802,22 @@ int FinalBackward(ts2_model *M, void *s)
     g.splitK = 1;
     CK(ts2_gemm_nt(&g, s));
     // delta_final[v][d] = sum_t grad[t][v] * fn[t][d]
-    CK(Ts2TransposeToBf16(M->len, R, VP, M->gradV.P(), TS2_BF16, M->gradVT.P(), s));
-    CK(Ts2TransposeToBf16(M->len, R, D, M->normState[depth].P(), M->mode, M->fnT.P(), s));
     ts2_gemm_args h = {};
-    h.a = M->gradVT.m;
-    h.b = M->fnT.m;
+    if (M->len == R && (VP % 256) == 0 && (D % 256) == 0) {
+        // whole row groups: the product contracts over the rows of the gradient and of the final state as they lie
+        // (Fp16MatMul<1, 1, TStoreDelta>, gpu_final.cuh:265); the 8-bit state only changes its type
+        Arr fn16 = Flat(M->fnT.m.ptr, R, D, TS2_BF16);
+        CK(Ts2RowsToBf16(M->len, R, D, M->normState[depth].P(), M->mode, fn16.P(), s));
+        h.a = M->gradV.m;
+        h.b = fn16.m;
+        h.kMajor = 1;
+        h.tileConfig = 1;
+    } else {
+        CK(Ts2TransposeToBf16(M->len, R, VP, M->gradV.P(), TS2_BF16, M->gradVT.P(), s));
+        CK(Ts2TransposeToBf16(M->len, R, D, M->normState[depth].P(), M->mode, M->fnT.P(), s));
+        h.a = M->gradVT.m;
+        h.b = M->fnT.m;
+    }
     h.c = M->finalW.delta.m;
     h.abType = TS2_BF16;
     h.cType = TS2_I8;

@@ -488,6 +488,54 @@ int Ts2FinalSoftmaxGrad(int rows, int vocab, const ts2_mat *logits, const float 
     return TS2_OK;
 }
 
+// dst[t][x] = bf16(src[t][x]) for 8-bit src (exact), rows <= t < rowsRound zero; a lane converts 8 consecutive elements
+template <class TSrc>
+__global__ void __launch_bounds__(256) RowsToBf16(int rows, int rowsRound, int cols8, const uint8_t *src, int64_t ldSrc, uint8_t *dst, int64_t ldDst)
+{
+    const long total = (long)rowsRound * cols8;
+    for (long u = (long)blockIdx.x * 256 + threadIdx.x; u < total; u += (long)gridDim.x * 256) {
+        const int t = (int)(u / cols8), c = (int)(u % cols8);
+        uint32_t out[4] = {0, 0, 0, 0};
+        if (t < rows) {
+            const uint2 in = *(const uint2 *)(src + (int64_t)t * ldSrc + c * 8);
+            const uint32_t w[2] = {in.x, in.y};
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+                float lo, hi;
+                if (std::is_same<TSrc, TI8>::value) {
+                    lo = (float)(int8_t)(w[e >> 2] >> (8 * (e & 3)));
+                    hi = (float)(int8_t)(w[e >> 2] >> (8 * ((e + 1) & 3)));
+                } else {
+                    lo = (e & 3) == 0 ? __builtin_amdgcn_cvt_f32_fp8((int)w[e >> 2], 0) : __builtin_amdgcn_cvt_f32_fp8((int)w[e >> 2], 2);
+                    hi = (e & 3) == 0 ? __builtin_amdgcn_cvt_f32_fp8((int)w[e >> 2], 1) : __builtin_amdgcn_cvt_f32_fp8((int)w[e >> 2], 3);
+                }
+                out[e >> 1] = PackBf16x2(lo, hi);
+            }
+        }
+        *(uint4 *)(dst + (int64_t)t * ldDst + c * 16) = make_uint4(out[0], out[1], out[2], out[3]);
+    }
+}
+
+int Ts2RowsToBf16(int rows, int rowsRound, int cols, const ts2_mat *src, int srcType, const ts2_mat *dst, void *stream)
+{
+    if ((cols & 7) || (src->strideBytes & 7) || (dst->strideBytes & 15) || ((uintptr_t)src->ptr & 7) || ((uintptr_t)dst->ptr & 15)) {
+        return TS2_ERR_ALIGN;
+    }
+    const long total = (long)rowsRound * (cols / 8);
+    const dim3 grid((unsigned)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192));
+    if (srcType == TS2_I8) {
+        hipLaunchKernelGGL((RowsToBf16<TI8>), grid, dim3(256), 0, STREAM, rows, rowsRound, cols / 8, (const uint8_t *)src->ptr, src->strideBytes,
+            (uint8_t *)dst->ptr, dst->strideBytes);
+    } else if (srcType == TS2_E4M3) {
+        hipLaunchKernelGGL((RowsToBf16<TE4M3>), grid, dim3(256), 0, STREAM, rows, rowsRound, cols / 8, (const uint8_t *)src->ptr, src->strideBytes,
+            (uint8_t *)dst->ptr, dst->strideBytes);
+    } else {
+        return TS2_ERR_UNSUPPORTED;
+    }
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
 int Ts2TransposeToBf16(int rows, int rowsRound, int cols, const ts2_mat *src, int srcType, const ts2_mat *dst, void *stream)
 {
     dim3 grid((cols + 63) / 64, (rowsRound + 63) / 64);
