@@ -131,7 +131,8 @@ typedef struct ts2_gemm_args {
     } segment[3];
     /* kMajor != 0: A is [k][m] and B is [k][n] - the rows of both operands are the contraction index, C[i][j] = sum_k A[k][i] * B[k][j].
      * The form a delta product dW = dY^T X takes on the untransposed activations ([token][feature], src/gpt/compute/matmul_fwdbwd.cuh:314-391
-     * transposes both first): the operands are transposed by the LDS reads of the kernel instead.  TS2_E4M3 operands, m and n multiples
+     * transposes both first; the final layer's Fp16MatMul<1, 1, TStoreDelta>, src/gpt/compute/gpu_final.cuh:265, reads both transposed):
+     * the operands are transposed by the LDS reads of the kernel instead.  TS2_E4M3 or TS2_BF16 operands, m and n multiples
      * of 256 (the 256x256 kernel; with tileConfig 0 the caller must make sure that (m/256)*(n/256)*slices >= 192 or pass tileConfig 1),
      * fp32 TS2_EPI_STORE results (also as stored slices, splitSlabBytes) or TS2_EPI_ROW_TILE_MAXNORM; nothing else. */
     int32_t kMajor;
