@@ -119,6 +119,55 @@ __device__ __forceinline__ void StoreBlockBf16(uint8_t *c, int64_t ldc, int col,
     }
 }
 
+// The same store for a block whose 32 rows all lie below mLive, through a buffer descriptor that starts at the wave tile's first row:
+// the lane's part of the address (its column pair, and the row it owns inside a group of eight) is one register for the whole
+// epilogue and the block's part goes in as the scalar offset, so a store costs no vector arithmetic for its address.  The pair is
+// made from the lane's own packed (row e, row e+1) values and the neighbour's by one byte permute instead of three selects.
+struct TWaveStore {
+    __amdgpu_buffer_rsrc_t rsrc;
+    int laneOff;   // bytes: (row owned inside a group of eight) * ldc + column part
+    uint32_t sel;  // byte selector of the pair permute (16-bit results)
+    int ldc;
+};
+
+template <int WTM> __device__ __forceinline__ TWaveStore MakeWaveStore(uint8_t *c, int64_t ldc, int firstRow, int col, int elemBytes, int half, int l32)
+{
+    TWaveStore w;
+    w.rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(c + (int64_t)firstRow * ldc), 0, (int)(32 * WTM * ldc), 0x00020000);
+    const bool odd = l32 & 1;
+    w.ldc = (int)ldc;
+    if (elemBytes == 2) {
+        w.laneOff = (half * 4 + (odd ? 1 : 0)) * (int)ldc + (col & ~1) * 2;
+    } else {
+        w.laneOff = (half * 4) * (int)ldc + col * 4;
+    }
+    w.sel = odd ? 0x07060302u : 0x01000504u;
+    return w;
+}
+
+// v[e]: the 16 values of the lane's column in block row `blockRow` of the wave tile, block column offset colBytes
+template <bool F16> __device__ __forceinline__ void StoreBlock16Buf(const TWaveStore &w, int blockRow, int colBytes, const float (&v)[16])
+{
+#pragma unroll
+    for (int e = 0; e < 16; e += 2) {
+        const uint32_t own = F16 ? PackF16x2(v[e], v[e + 1]) : PackBf16x2(v[e], v[e + 1]);
+        const uint32_t other = (uint32_t)LaneDpp<DPP_XOR1>((int)own);
+        // even lanes: (own row e, neighbour's row e) = columns (c, c+1) of row e; odd lanes: (neighbour's row e+1, own row e+1)
+        const uint32_t packed = __builtin_amdgcn_perm(own, other, w.sel);
+        const int rowInTile = blockRow * 32 + (e >> 2) * 8 + (e & 2);
+        __builtin_amdgcn_raw_buffer_store_b32(packed, w.rsrc, w.laneOff, rowInTile * w.ldc + colBytes, 0);
+    }
+}
+
+__device__ __forceinline__ void StoreBlock32Buf(const TWaveStore &w, int blockRow, int colBytes, const float (&v)[16])
+{
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        const int rowInTile = blockRow * 32 + (e >> 2) * 8 + (e & 3);
+        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v[e]), w.rsrc, w.laneOff, rowInTile * w.ldc + colBytes, 0);
+    }
+}
+
 template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT, class TAcc, class TFAcc>
 __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], TFAcc &facc, uint8_t *lds, int rowBase, int colBase, int wm, int wn,
     int half, int l32)
@@ -415,6 +464,30 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
                                     ((bf16_t *)dst)[col] = FloatToBf16(v);
                                 }
                             }
+                        }
+                    }
+                }
+                return;
+            }
+        }
+        if constexpr ((CT == C_BF16 || CT == C_F16 || CT == C_F32) && EPI == TS2_EPI_STORE && !KT) {
+            // every row of the wave tile is live, no atomics, rows within the descriptor's reach: the stores with scalar addressing
+            const int firstRow = rowBase + wm * (32 * WTM);
+            if (p.splitK <= 1 && firstRow + 32 * WTM <= mLive && (int64_t)32 * WTM * p.ldc < ((int64_t)1 << 31)) {
+                const TWaveStore w = MakeWaveStore<WTM>(p.c, p.ldc, firstRow, colBase + wn * (32 * WTN) + l32, CT == C_F32 ? 4 : 2, half, l32);
+#pragma unroll
+                for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+                    for (int j = 0; j < WTN; ++j) {
+                        float v[16];
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) {
+                            v[e] = accVal(i, j, e) * rsAll[i][e];
+                        }
+                        if constexpr (CT == C_F32) {
+                            StoreBlock32Buf(w, i, j * 128, v);
+                        } else {
+                            StoreBlock16Buf<CT == C_F16>(w, i, j * 64, v);
                         }
                     }
                 }
