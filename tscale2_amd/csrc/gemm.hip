@@ -155,7 +155,7 @@ template <bool F16> __device__ __forceinline__ void StoreBlock16Buf(const TWaveS
         // even lanes: (own row e, neighbour's row e) = columns (c, c+1) of row e; odd lanes: (neighbour's row e+1, own row e+1)
         const uint32_t packed = __builtin_amdgcn_perm(own, other, w.sel);
         const int rowInTile = blockRow * 32 + (e >> 2) * 8 + (e & 2);
-        __builtin_amdgcn_raw_buffer_store_b32(packed, w.rsrc, w.laneOff, rowInTile * w.ldc + colBytes, 0);
+        __builtin_amdgcn_raw_buffer_store_b32(packed, w.rsrc, w.laneOff, rowInTile * w.ldc + colBytes, 2);
     }
 }
 
@@ -164,7 +164,7 @@ __device__ __forceinline__ void StoreBlock32Buf(const TWaveStore &w, int blockRo
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
         const int rowInTile = blockRow * 32 + (e >> 2) * 8 + (e & 3);
-        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v[e]), w.rsrc, w.laneOff, rowInTile * w.ldc + colBytes, 0);
+        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v[e]), w.rsrc, w.laneOff, rowInTile * w.ldc + colBytes, 2);
     }
 }
 
@@ -214,6 +214,10 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
         static_assert(WTN == 4 || WTN == 2 || CT != C_BF16NORM, "the normalising epilogue needs a wave tile of 64 or 128 columns");
         const int tile = (colBase + wn * (32 * WTN)) / TILE;
         const int colInTile = (wn * (32 * WTN)) & (TILE - 1);
+        // all rows of the wave tile live: the stores with scalar addressing
+        const int firstRow = rowBase + wm * (32 * WTM);
+        const bool wholeTileLive = firstRow + 32 * WTM <= mLive && (int64_t)32 * WTM * p.ldc < ((int64_t)1 << 31);
+        const TWaveStore waveStore = MakeWaveStore<WTM>(p.c, p.ldc, firstRow, colBase + wn * (32 * WTN) + l32, 2, half, l32);
         float *xch = (float *)lds;
         // sums of squares of the 16 rows of block row i over the wave's columns
         auto blockRowSum2 = [&](int i, float (&out)[WTN][16], float (&sum2)[16]) {
@@ -325,10 +329,17 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
                     }
                 }
             }
+            if (wholeTileLive) {
 #pragma unroll
-            for (int j = 0; j < WTN; ++j) {
-                StoreBlockBf16(p.c, p.ldc, colBase + wn * (32 * WTN) + j * 32 + l32, l32, mLive, out[j],
-                    [&](int e) { return rowBase + rowLocal(i, e); });
+                for (int j = 0; j < WTN; ++j) {
+                    StoreBlock16Buf<false>(waveStore, i, j * 64, out[j]);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < WTN; ++j) {
+                    StoreBlockBf16(p.c, p.ldc, colBase + wn * (32 * WTN) + j * 32 + l32, l32, mLive, out[j],
+                        [&](int e) { return rowBase + rowLocal(i, e); });
+                }
             }
         }
     } else if constexpr (CT == C_I8PACK) {
@@ -435,7 +446,7 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
                         for (int j = 0; j < WTN; ++j) {
                             const int col = colBase + wn * (32 * WTN) + j * 32 + l32;
                             if (CT == C_F32) {
-                                o[r][j] = row < mLive ? ((const float *)src)[col] : 0.f;
+                                o[r][j] = row < mLive ? __builtin_nontemporal_load((const float *)src + col) : 0.f;
                             } else {
                                 o[r][j] = row < mLive ? Bf16ToFloat(((const bf16_t *)src)[col]) : 0.f;
                             }
@@ -459,7 +470,7 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
                                 const int col = colBase + wn * (32 * WTN) + j * 32 + l32;
                                 float v = old[ch & 1][r][j] + accVal(ch >> 1, j, (ch & 1) * 8 + r) * rs;
                                 if constexpr (CT == C_F32) {
-                                    ((float *)dst)[col] = v;
+                                    __builtin_nontemporal_store(v, (float *)dst + col);
                                 } else {
                                     ((bf16_t *)dst)[col] = FloatToBf16(v);
                                 }
