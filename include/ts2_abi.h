@@ -93,7 +93,8 @@ typedef struct ts2_gemm_args {
      * Comparison switches, all off in normal use: bit 2 (4) register-staged loader; bit 3 (8) eight waves per workgroup (256x256
      * store/accumulate results; with tile 3: the form BackpropDelta launches); bit 4 (16) two LDS stages instead of the ring on the
      * 256x256 tile (and on the 128x128 tile with TS2_E4M3 operands, which takes the ring from k = 1024 on); bits 5-6 tile-order
-     * group 8 / 4 / 2 instead of the automatic choice; bit 7 (128) the ring on the 128x128 tile at any k. */
+     * group 8 / 4 / 2 instead of the automatic choice; bit 7 (128) the ring on the 128x128 tile at any k; bits 9 / 10 (512 / 1024)
+     * plain / non-temporal stores of C instead of the choice by k. */
     int32_t tileConfig;
     /* Expert-grouped products (TMoeMatMulKernelCall / TMoeDeltaMatMulKernelCall, src/gpt/compute/moe_matmul.cuh:47-215):
      * tileGroup [m/128] (device): rows of A and C are grouped by expert in 128-row tiles; tile i multiplies the B slab

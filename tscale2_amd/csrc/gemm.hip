@@ -50,6 +50,7 @@ struct GemmP {
     int direct;              // 1: direct global->LDS loader
     int noRing;              // 1: keep the two-stage loop for the 256x256 tile (comparison)
     int kMajor;              // 1: A is [k][m], B is [k][n] (fp8, ring kernel): operands are transposed by the LDS reads
+    int streamC;             // results stored with the non-temporal hint
     int ring128;             // 128x128 tile: the ring pipeline (two workgroups per CU) instead of the two-stage loop
     int mapGroup;            // M tiles per group of the tile order (an XCD's share of the tiles should be about square)
     int splits;              // >1 with splitSlab: blockIdx.y = slice of the contraction, partial product stored to c + y * splitSlab
@@ -146,7 +147,7 @@ template <int WTM> __device__ __forceinline__ TWaveStore MakeWaveStore(uint8_t *
 }
 
 // v[e]: the 16 values of the lane's column in block row `blockRow` of the wave tile, block column offset colBytes
-template <bool F16> __device__ __forceinline__ void StoreBlock16Buf(const TWaveStore &w, int blockRow, int colBytes, const float (&v)[16])
+template <bool F16, int AUX> __device__ __forceinline__ void StoreBlock16Buf(const TWaveStore &w, int blockRow, int colBytes, const float (&v)[16])
 {
 #pragma unroll
     for (int e = 0; e < 16; e += 2) {
@@ -155,16 +156,16 @@ template <bool F16> __device__ __forceinline__ void StoreBlock16Buf(const TWaveS
         // even lanes: (own row e, neighbour's row e) = columns (c, c+1) of row e; odd lanes: (neighbour's row e+1, own row e+1)
         const uint32_t packed = __builtin_amdgcn_perm(own, other, w.sel);
         const int rowInTile = blockRow * 32 + (e >> 2) * 8 + (e & 2);
-        __builtin_amdgcn_raw_buffer_store_b32(packed, w.rsrc, w.laneOff, rowInTile * w.ldc + colBytes, 2);
+        __builtin_amdgcn_raw_buffer_store_b32(packed, w.rsrc, w.laneOff, rowInTile * w.ldc + colBytes, AUX);
     }
 }
 
-__device__ __forceinline__ void StoreBlock32Buf(const TWaveStore &w, int blockRow, int colBytes, const float (&v)[16])
+template <int AUX> __device__ __forceinline__ void StoreBlock32Buf(const TWaveStore &w, int blockRow, int colBytes, const float (&v)[16])
 {
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
         const int rowInTile = blockRow * 32 + (e >> 2) * 8 + (e & 3);
-        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v[e]), w.rsrc, w.laneOff, rowInTile * w.ldc + colBytes, 2);
+        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v[e]), w.rsrc, w.laneOff, rowInTile * w.ldc + colBytes, AUX);
     }
 }
 
@@ -332,7 +333,11 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
             if (wholeTileLive) {
 #pragma unroll
                 for (int j = 0; j < WTN; ++j) {
-                    StoreBlock16Buf<false>(waveStore, i, j * 64, out[j]);
+                    if (p.streamC) {
+                        StoreBlock16Buf<false, 2>(waveStore, i, j * 64, out[j]);
+                    } else {
+                        StoreBlock16Buf<false, 0>(waveStore, i, j * 64, out[j]);
+                    }
                 }
             } else {
 #pragma unroll
@@ -496,9 +501,17 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
                             v[e] = accVal(i, j, e) * rsAll[i][e];
                         }
                         if constexpr (CT == C_F32) {
-                            StoreBlock32Buf(w, i, j * 128, v);
+                            if (p.streamC) {
+                                StoreBlock32Buf<2>(w, i, j * 128, v);
+                            } else {
+                                StoreBlock32Buf<0>(w, i, j * 128, v);
+                            }
                         } else {
-                            StoreBlock16Buf<CT == C_F16>(w, i, j * 64, v);
+                            if (p.streamC) {
+                                StoreBlock16Buf<CT == C_F16, 2>(w, i, j * 64, v);
+                            } else {
+                                StoreBlock16Buf<CT == C_F16, 0>(w, i, j * 64, v);
+                            }
                         }
                     }
                 }
@@ -1971,6 +1984,11 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
     p.mapGroup = ((a->tileConfig >> 5) & 3) == 1 ? 8 : ((a->tileConfig >> 5) & 3) == 2 ? 4 : ((a->tileConfig >> 5) & 3) == 3 ? 2 : 0;
     p.noRing = (a->tileConfig & 16) ? 1 : 0; // bit 4: two-stage loop instead of the ring for the 256x256 tile (comparison)
     p.kMajor = a->kMajor ? 1 : 0;
+    // The result is read by another kernel later: with a contraction of 2048 bytes or more its stores leave the L2 to the operands
+    // (the config of the dense fp8 step: 2.4 ms of 125 per step, all of it from the K = 2048 products); shorter products are mostly
+    // their stores, and inside a layer those measured the same or slower with the hint (bits 9 / 10 of tileConfig force one or the
+    // other, for comparison)
+    p.streamC = (a->tileConfig & 512) ? 0 : (a->tileConfig & 1024) ? 1 : ((int64_t)a->k * esz >= 2048 ? 1 : 0);
     // 128x128 tile, e4m3: the ring pipeline from a contraction of eight steps on (measured on the expert-grouped products: 136 -> 120 us
     // at K = 1024, no gain at K = 512); bit 7 of tileConfig asks for it at any length, bit 4 for the two-stage loop
     p.ring128 = !(a->tileConfig & 16) && ((a->tileConfig & 128) || (int64_t)a->k * esz >= 8 * BKB) ? 1 : 0;
