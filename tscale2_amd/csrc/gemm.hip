@@ -1984,11 +1984,11 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
     p.mapGroup = ((a->tileConfig >> 5) & 3) == 1 ? 8 : ((a->tileConfig >> 5) & 3) == 2 ? 4 : ((a->tileConfig >> 5) & 3) == 3 ? 2 : 0;
     p.noRing = (a->tileConfig & 16) ? 1 : 0; // bit 4: two-stage loop instead of the ring for the 256x256 tile (comparison)
     p.kMajor = a->kMajor ? 1 : 0;
-    // The result is read by another kernel later: with a contraction of 2048 bytes or more its stores leave the L2 to the operands
-    // (the config of the dense fp8 step: 2.4 ms of 125 per step, all of it from the K = 2048 products); shorter products are mostly
-    // their stores, and inside a layer those measured the same or slower with the hint (bits 9 / 10 of tileConfig force one or the
-    // other, for comparison)
-    p.streamC = (a->tileConfig & 512) ? 0 : (a->tileConfig & 1024) ? 1 : ((int64_t)a->k * esz >= 2048 ? 1 : 0);
+    // The result is read by another kernel later: with a contraction of 1024 bytes or more its stores leave the L2 to the operands
+    // (the dense fp8 step: 2.4 ms of 125 per step, all of it from the K = 2048 products; the expert-grouped products at K = 1024:
+    // 127 -> 112 us); shorter products are mostly their stores, and inside a layer those measured slower with the hint (K = 512:
+    // 167 -> 180 us).  Bits 9 / 10 of tileConfig force one or the other, for comparison.
+    p.streamC = (a->tileConfig & 512) ? 0 : (a->tileConfig & 1024) ? 1 : ((int64_t)a->k * esz >= 1024 ? 1 : 0);
     // 128x128 tile, e4m3: the ring pipeline from a contraction of eight steps on (measured on the expert-grouped products: 136 -> 120 us
     // at K = 1024, no gain at K = 512); bit 7 of tileConfig asks for it at any length, bit 4 for the two-stage loop
     p.ring128 = !(a->tileConfig & 16) && ((a->tileConfig & 128) || (int64_t)a->k * esz >= 8 * BKB) ? 1 : 0;

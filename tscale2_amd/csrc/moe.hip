@@ -360,6 +360,62 @@ __global__ void __launch_bounds__(256) CombineExperts(int len, int tiles, int se
     Store4<TF32>(At<TF32>(res, t, col), sum);
 }
 
+// 16-bit experts' results: a lane takes 8 consecutive elements (16-byte loads), a tile is 16 lanes, and the rows of all selected
+// experts are looked up before the first of them is read, so their loads are in flight together.  The sums are formed in the order
+// of the slots, like CombineExperts.
+__global__ void __launch_bounds__(256) CombineExperts8(int len, int tiles, int selected, Mat src, const int *sampleExpertIds,
+    const int *sampleExpertOffset, const int *expertOffset, float alpha, const float *alphaPtr, Mat res, int add)
+{
+    const long unit = ((long)blockIdx.x * 256 + threadIdx.x) >> 4;
+    const int l16 = threadIdx.x & 15;
+    if (unit >= (long)len * tiles) {
+        return;
+    }
+    const int t = (int)(unit / tiles), tile = (int)(unit - (long)t * tiles);
+    const int col = tile * TILE + l16 * 8;
+    float sum[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    F4 old0 = ZeroF4(), old1 = ZeroF4();
+    if (add) {
+        old0 = Load4<TF32>(At<TF32>(res, t, col));
+        old1 = Load4<TF32>(At<TF32>(res, t, col + 4));
+    }
+    constexpr int KB = 4; // slots per batch of loads
+    for (int k0 = 0; k0 < selected; k0 += KB) {
+        int row[KB];
+        uint4 v[KB];
+#pragma unroll
+        for (int k = 0; k < KB; ++k) {
+            const int idx = t * selected + (k0 + k < selected ? k0 + k : selected - 1);
+            row[k] = expertOffset[sampleExpertIds[idx]] + sampleExpertOffset[idx];
+        }
+#pragma unroll
+        for (int k = 0; k < KB; ++k) {
+            v[k] = *(const uint4 *)At<TBF16>(src, row[k], col);
+        }
+#pragma unroll
+        for (int k = 0; k < KB; ++k) {
+            if (k0 + k < selected) {
+                const uint32_t w[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    sum[e] += (e & 1) ? __uint_as_float(w[e >> 1] & 0xffff0000u) : __uint_as_float(w[e >> 1] << 16);
+                }
+            }
+        }
+    }
+    float s = alpha;
+    if (alphaPtr) {
+        s *= *alphaPtr;
+    }
+    F4 r0 = MakeF4(sum[0], sum[1], sum[2], sum[3]) * s, r1 = MakeF4(sum[4], sum[5], sum[6], sum[7]) * s;
+    if (add) {
+        r0 = r0 + old0;
+        r1 = r1 + old1;
+    }
+    Store4<TF32>(At<TF32>(res, t, col), r0);
+    Store4<TF32>(At<TF32>(res, t, col + 4), r1);
+}
+
 // 128x128 byte-tile transposes over a batch of slabs
 __global__ void __launch_bounds__(256) TransposeU8Batched(const uint8_t *src, int64_t srcStride, int64_t srcSlab, uint8_t *dst, int64_t dstStride,
     int64_t dstSlab)
@@ -610,7 +666,10 @@ extern "C" int ts2_combine_experts(int32_t len, int32_t selected, const ts2_mat 
     int tiles = dim / TILE;
     long units = (long)len * tiles;
     dim3 grid((unsigned)((units * 32 + 255) / 256));
-    if (srcType == TS2_BF16) {
+    if (srcType == TS2_BF16 && Aligned16(src->ptr, src->strideBytes) && Aligned16(res->ptr, res->strideBytes)) {
+        hipLaunchKernelGGL(CombineExperts8, dim3((unsigned)((units * 16 + 255) / 256)), dim3(256), 0, STREAM, len, tiles, selected, M(*src),
+            tb->sampleExpertIds, tb->sampleExpertOffset, tb->expertOffset, alpha, alphaPtr, M(*res), add);
+    } else if (srcType == TS2_BF16) {
         hipLaunchKernelGGL((CombineExperts<TBF16>), grid, dim3(256), 0, STREAM, len, tiles, selected, M(*src), tb->sampleExpertIds,
             tb->sampleExpertOffset, tb->expertOffset, alpha, alphaPtr, M(*res), add);
     } else if (srcType == TS2_F32) {
