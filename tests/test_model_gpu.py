@@ -198,6 +198,48 @@ def test_kept_activations_equal_recomputation_with_moe_layers():
         assert np.array_equal(a, b)
 
 
+def test_expert_matrices_set_again_drop_their_kept_transposes():
+    """The transposed copies of the expert matrices that the MoE dX products contract over are kept from one backward to the next;
+    setting a matrix again must drop its copy.  After a step, every expert matrix of the first MoE layer gets new weights: the next
+    step must be exactly what a fresh model holding the new weights computes."""
+    print("case kept expert transposes dropped by set_matrix", flush=True)
+    from model_harness import QMatrix
+    from tscale2_amd import lib as L
+    h = Harness(E4M3, dim=256, heads=2, ffn_tiles=2, depth=3, vocab=256, frag_count=4, frag_len=64, wide_window=64, experts=4, selected=2, xp=256,
+                seed=21, std=0.05)
+    d_moe = [d for d, t in enumerate(h.lt) if int(t) == 3][0]
+
+    def everything(m):
+        return [m.get_delta(d, i, *q.fast.shape) for d in range(len(h.layers)) for i, q in enumerate(h.layers[d])] + \
+               [m.array("stateGrad").float().cpu().numpy(), np.array([m.loss_sum()])]
+    m = h.device_model()
+    try:
+        m.backprop()
+        torch.cuda.synchronize()
+        before = everything(m)
+        r = np.random.default_rng(5)
+        for i in range(3):
+            q = h.layers[d_moe][i]
+            h.layers[d_moe][i] = QMatrix(h.orc, r.standard_normal(q.w.shape) * 0.05, E4M3, i == 1)
+            m.set_matrix(d_moe, i, h.layers[d_moe][i].fast, h.layers[d_moe][i].scale)
+        m.backprop()
+        torch.cuda.synchronize()
+        after = everything(m)
+    finally:
+        m.close()
+    fresh = h.device_model()
+    try:
+        fresh.backprop()
+        torch.cuda.synchronize()
+        want = everything(fresh)
+    finally:
+        fresh.close()
+    assert any(not np.array_equal(a, b) for a, b in zip(before, after))
+    for a, b in zip(after[:-1], want[:-1]):
+        assert np.array_equal(a, b)
+    assert abs(after[-1][0] - want[-1][0]) <= 1e-5 * abs(want[-1][0])      # (the loss is summed with float atomics: order varies)
+
+
 def test_moe_routing_tables_match_cpu_moe():
     """ts2_moe_route against CpuMoe (layer_moe.cu:287-327): same experts, same weights, sum w^2 = E, stable grouping"""
     print("case moe route", flush=True)

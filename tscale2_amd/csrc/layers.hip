@@ -143,7 +143,6 @@ struct ts2_model {
     ts2_moe_tables moe = {};
     Arr normMoe, sgMoe, moeSel, dMoeSel;     // grouped 8-bit input / gradient, select logits fp32, their gradient
     float *dExpertWeight = 0;
-    Arr wT;                                  // transposed expert weights scratch
     // final layer
     Arr logits, gradV, gradVT, fnT, wfT;
     Arr logits16;                            // IEEE-half logits of the backward pass (the fp32 ones serve ts2_model_forward)
@@ -656,9 +655,18 @@ int MoeBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
     // state gradient into expert order
     CK(ts2_moe_group_samples(RM, 1, M->stateGradFast.P(), M->moe.xpSampleId, M->sgMoe.P(), s));
     // contract backward: dRG[row][x] = sum_d sg[row][d] Wc_e[d][x]: needs Wc_e^T = [X][D] per expert
-    Arr wcT = View(M->wT, E * X, D);
-    CK(ts2_transpose_u8_batched(E, D, X, L.w[2].fast.m.ptr, L.w[2].fast.m.strideBytes, (int64_t)D * L.w[2].fast.m.strideBytes, wcT.m.ptr,
-        wcT.m.strideBytes, (int64_t)X * wcT.m.strideBytes, s));
+    // (the experts' transposed matrices are kept from one backward to the next like the dense layers', and redone when a matrix is set
+    // or updated)
+    auto keptT = [&](TMatrix &W, int rows, int cols) -> int { // slabs of [rows][cols] -> [cols][rows]
+        if (!W.fastTValid) {
+            CK(ts2_transpose_u8_batched(E, rows, cols, W.fast.m.ptr, W.fast.m.strideBytes, (int64_t)rows * W.fast.m.strideBytes, W.fastT.m.ptr,
+                W.fastT.m.strideBytes, (int64_t)cols * W.fastT.m.strideBytes, s));
+            W.fastTValid = true;
+        }
+        return 0;
+    };
+    CK(keptT(L.w[2], D, X));
+    Arr wcT = L.w[2].fastT;
     Arr drg = View(M->g16[0], RM, X); // 16 bits like the reference's DRG and StateGradFull (layer_moe.cu:35,46)
     CK(GroupedGemm(M, M->sgMoe, wcT, X, X, D, drg, DISCR * Dot(E * X), L.w[2].scale, false, s));
     Arr dwide = View(M->gf[0], RM, X), dgate = View(M->gf[1], RM, X);
@@ -668,15 +676,11 @@ int MoeBackward(ts2_model *M, TLayer &L, const Arr &norm8, const float *gradScal
     // (scaled-gradient) units already
     CK(ts2_backprop_moe(len, R, E, K, &M->moe, M->dExpertWeight, M->dMoeSel.P(), M->fastGradType, s));
     // expand + gate backward into grouped rows, then back to token order
-    Arr weT = View(M->wT, E * D, X);
     Arr sgFull = View(M->g16[1], RM, D);
-    CK(ts2_transpose_u8_batched(E, X, D, L.w[0].fast.m.ptr, L.w[0].fast.m.strideBytes, (int64_t)X * L.w[0].fast.m.strideBytes, weT.m.ptr,
-        weT.m.strideBytes, (int64_t)D * weT.m.strideBytes, s));
-    // the gate matrix transposed next to the expand matrix; both products in one launch (one pass over the result)
-    Arr wgT = Flat((uint8_t *)M->wT.m.ptr + (size_t)E * D * weT.m.strideBytes, E * D, X, M->mode);
-    wgT.m.strideBytes = weT.m.strideBytes;
-    CK(ts2_transpose_u8_batched(E, X, D, L.w[1].fast.m.ptr, L.w[1].fast.m.strideBytes, (int64_t)X * L.w[1].fast.m.strideBytes, wgT.m.ptr,
-        wgT.m.strideBytes, (int64_t)D * wgT.m.strideBytes, s));
+    CK(keptT(L.w[0], X, D));
+    CK(keptT(L.w[1], X, D));
+    // both products in one launch (one pass over the result)
+    Arr weT = L.w[0].fastT, wgT = L.w[1].fastT;
     CK(GroupedGemm(M, dwide, weT, D, D, X, sgFull, DISCR * Dot(D), L.w[0].scale, false, s, &dgate, &wgT, nullptr));
     CK(ts2_combine_experts(len, K, sgFull.P(), TS2_BF16, &M->moe, 1.f, nullptr, M->dNormState.P(), 0, s));
     // select matrix: dNormState += dMoe * Wsel / sqrt(D) and its delta through the same 8-bit operator as every other matrix (the
@@ -703,7 +707,8 @@ int InitMatrix(ts2_model *M, TMatrix *W, int srcDim, int dstDim, int slabs, bool
         !M->Alloc(&W->deltaTileScale, srcDim / 128, dstDim * slabs, TS2_F32)) {
         return TS2_ERR_LAUNCH;
     }
-    if (slabs == 1 && keepT && !M->Alloc(&W->fastT, srcDim, dstDim, M->mode)) {
+    // the transposed copy the dX products contract over, kept while the weights do not change (expert matrices: slab by slab)
+    if (keepT && !M->Alloc(&W->fastT, srcDim * slabs, dstDim, M->mode)) {
         return TS2_ERR_LAUNCH;
     }
     W->scale = (float *)M->Dev(4);
@@ -1042,8 +1047,6 @@ extern "C" ts2_model *ts2_model_create(const ts2_model_config *cfg)
         M->dExpertWeight = (float *)M->Dev((size_t)M->lenMoe * 4);
         ok &= M->Alloc(&M->normMoe, M->lenMoe, D, M->mode) && M->Alloc(&M->sgMoe, M->lenMoe, D, M->fastGradType) &&
               M->Alloc(&M->moeSel, R, SelectDim, TS2_F32) && M->Alloc(&M->dMoeSel, R, SelectDim, M->fastGradType);
-        int wtRows = 2 * E * (X > D ? X : D), wtCols = X > D ? X : D; // two transposed expert matrices side by side (expand and gate)
-        ok &= M->Alloc(&M->wT, wtRows, wtCols, M->mode);
     }
     ok &= M->Alloc(&M->logits, R, VP, TS2_F32) && M->Alloc(&M->logits16, R, VP, TS2_F16) && M->Alloc(&M->gradV, R, VP, TS2_BF16) && M->Alloc(&M->gradVT, VP, R, TS2_BF16) &&
           M->Alloc(&M->fnT, D, R, TS2_BF16) && M->Alloc(&M->wfT, D, VP, TS2_BF16);

@@ -251,6 +251,41 @@ __global__ void __launch_bounds__(256) MatrixLoLUmoe(int lenMoe, int tiles, cons
     Store4<TDst>(At<TDst>(res, t, col), v);
 }
 
+// sum over the 16 lanes of a row of the wave (one 128-wide tile at 8 elements per lane)
+__device__ __forceinline__ float Row16Sum(float v)
+{
+    v += LaneDpp<DPP_XOR1>(v);
+    v += LaneDpp<DPP_XOR2>(v);
+    v += LaneDpp<DPP_HALF_MIRROR>(v);
+    v += LaneDpp<DPP_MIRROR>(v);
+    return v;
+}
+
+// e4m3 results, sixteen elements per lane (two 16-byte loads per input, one 16-byte store): the arithmetic of MatrixLoLUmoe
+__global__ void __launch_bounds__(256) MatrixLoLUmoe16(int lenMoe, int dim16, const float *xpSampleWeight, Mat gate, Mat vals, float resMult, Mat res)
+{
+    const long id = (long)blockIdx.x * 256 + threadIdx.x;
+    if (id >= (long)lenMoe * dim16) {
+        return;
+    }
+    const int t = (int)(id / dim16), c = (int)(id - (long)t * dim16) * 16;
+    const float moe = xpSampleWeight[t];
+    uint32_t out[4] = {0, 0, 0, 0};
+    if (moe != 0) {
+        const uint4 g0 = *(const uint4 *)At<TBF16>(gate, t, c), g1 = *(const uint4 *)At<TBF16>(gate, t, c + 8);
+        const uint4 v0 = *(const uint4 *)At<TBF16>(vals, t, c), v1 = *(const uint4 *)At<TBF16>(vals, t, c + 8);
+        const uint32_t gw[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w}, vw[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+        const float f = moe * resMult;
+#pragma unroll
+        for (int w = 0; w < 8; ++w) {
+            float ga = __uint_as_float(gw[w] << 16), gb = __uint_as_float(gw[w] & 0xffff0000u);
+            float va = __uint_as_float(vw[w] << 16), vb = __uint_as_float(vw[w] & 0xffff0000u);
+            out[w >> 1] |= CvtPkE4m3(va * LoLU1(ga) * f, vb * LoLU1(gb) * f) << ((w & 1) * 16);
+        }
+    }
+    *(uint4 *)At<TE4M3>(res, t, c) = make_uint4(out[0], out[1], out[2], out[3]);
+}
+
 // one workgroup (8 x 32 lanes) per grouped row so that the routing-weight gradient is a plain block reduction
 template <class TGrad, class TOut>
 __global__ void __launch_bounds__(256) BackpropRowTileNormalizeLoLUmoe(int tiles, const float *xpSampleWeight, Mat gate, Mat vals, float valsScale,
@@ -285,6 +320,80 @@ __global__ void __launch_bounds__(256) BackpropRowTileNormalizeLoLUmoe(int tiles
     __syncthreads();
     if (threadIdx.x == 0) {
         dExpertWeight[t] = ((red[0] + red[1]) + (red[2] + red[3])) + ((red[4] + red[5]) + (red[6] + red[7]));
+    }
+}
+
+// The fp8 model's types (bf16 gradient in, e4m3 out): one wave per grouped row, a tile is 16 lanes of 8 elements (16-byte loads,
+// 8-byte stores), four tiles per pass, and the routing-weight gradient is a wave reduction: no LDS, no workgroup barrier, no idle
+// lanes at expert widths below 1024.  Per element the arithmetic of BackpropRowTileNormalizeLoLUmoe.
+__global__ void __launch_bounds__(256) BackpropRowTileNormalizeLoLUmoe8(int lenMoe, int tiles, const float *xpSampleWeight, Mat gate, Mat vals,
+    float valsScale, Mat valsSrcTileScale, Mat gradArr, float gradMult, Mat gradGate, Mat gradVals, float *dExpertWeight)
+{
+    const int t = blockIdx.x * 4 + (threadIdx.x >> 6); // wave-uniform
+    if (t >= lenMoe) {
+        return;
+    }
+    const int lane = threadIdx.x & 63, l16 = lane & 15, q = lane >> 4;
+    const float moe = xpSampleWeight[t];
+    float gm = 0;
+    for (int tile0 = 0; tile0 < tiles; tile0 += 4) {
+        const int tile = tile0 + q;
+        const bool any = tile < tiles;
+        const bool live = any && moe != 0;
+        const int col = (any ? tile : 0) * TILE + l16 * 8;
+        uint4 g = make_uint4(0, 0, 0, 0), v = g, gr = g;
+        float ts = 0;
+        if (live) {
+            g = *(const uint4 *)At<TBF16>(gate, t, col);
+            v = *(const uint4 *)At<TBF16>(vals, t, col);
+            gr = *(const uint4 *)At<TBF16>(gradArr, t, col);
+            ts = ScaleAt(valsSrcTileScale, tile, t);
+        }
+        const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, vw[4] = {v.x, v.y, v.z, v.w}, rw[4] = {gr.x, gr.y, gr.z, gr.w};
+        float resGate[8], resVals[8], src[8];
+        float sum2 = 0, dp = 0;
+        const float srcMult = ts / valsScale;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float ge = (e & 1) ? __uint_as_float(gw[e >> 1] & 0xffff0000u) : __uint_as_float(gw[e >> 1] << 16);
+            const float ve = (e & 1) ? __uint_as_float(vw[e >> 1] & 0xffff0000u) : __uint_as_float(vw[e >> 1] << 16);
+            const float de = ((e & 1) ? __uint_as_float(rw[e >> 1] & 0xffff0000u) : __uint_as_float(rw[e >> 1] << 16)) * gradMult;
+            const float vv = ve * valsScale;
+            const float mult = LoLU1(ge);
+            resGate[e] = de * vv * (mult * (1 - mult) * 2.f) * moe;
+            resVals[e] = de * mult * moe;
+            gm += de * vv * mult;
+            src[e] = vv * srcMult;
+            sum2 += src[e] * src[e];
+            dp += src[e] * resVals[e];
+        }
+        sum2 = Row16Sum(sum2);
+        dp = Row16Sum(dp);
+        if (!any) {
+            continue;
+        }
+        uint32_t og[2] = {0, 0}, ov[2] = {0, 0};
+        if (live) {
+            float sigma = 0, scale = 0;
+            if (sum2 != 0) {
+                const float inv = 1 / sum2;
+                sigma = dp * inv;
+                scale = sqrtf(TILE * inv);
+            }
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const float a0 = sum2 != 0 ? (resVals[2 * w] - src[2 * w] * sigma) * scale : 0.f;
+                const float a1 = sum2 != 0 ? (resVals[2 * w + 1] - src[2 * w + 1] * sigma) * scale : 0.f;
+                ov[w >> 1] |= CvtPkE4m3(a0, a1) << ((w & 1) * 16);
+                og[w >> 1] |= CvtPkE4m3(resGate[2 * w], resGate[2 * w + 1]) << ((w & 1) * 16);
+            }
+        }
+        *(uint2 *)At<TE4M3>(gradGate, t, col) = make_uint2(og[0], og[1]);
+        *(uint2 *)At<TE4M3>(gradVals, t, col) = make_uint2(ov[0], ov[1]);
+    }
+    gm = WaveSum(gm);
+    if (lane == 0) {
+        dExpertWeight[t] = gm;
     }
 }
 
@@ -588,6 +697,14 @@ extern "C" int ts2_matrix_lolu_moe(int32_t lenMoe, const float *xpSampleWeight, 
     }
     int tiles = dim / TILE;
     long units = (long)lenMoe * tiles;
+    if (resType == TS2_E4M3 && Aligned16(gate->ptr, gate->strideBytes) && Aligned16(vals->ptr, vals->strideBytes) &&
+        Aligned16(res->ptr, res->strideBytes)) {
+        const long lanes = (long)lenMoe * (dim / 16);
+        hipLaunchKernelGGL(MatrixLoLUmoe16, dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, STREAM, lenMoe, dim / 16, xpSampleWeight, M(*gate),
+            M(*vals), resMult, M(*res));
+        TS2_CHECK_LAUNCH();
+        return TS2_OK;
+    }
     dim3 grid((unsigned)((units * 32 + 255) / 256));
     TS2_DISPATCH_TYPE(resType, TD,
         hipLaunchKernelGGL((MatrixLoLUmoe<TD>), grid, dim3(256), 0, STREAM, lenMoe, tiles, xpSampleWeight, M(*gate), M(*vals), resMult, M(*res)));
@@ -611,7 +728,11 @@ extern "C" int ts2_backprop_row_tile_normalize_lolu_moe(int32_t lenMoe, const fl
 #define LAUNCH_M(TG, TO)                                                                                                                   \
     hipLaunchKernelGGL((BackpropRowTileNormalizeLoLUmoe<TG, TO>), dim3(lenMoe), dim3(256), 0, STREAM, tiles, xpSampleWeight, M(*gate), M(*vals), \
         valsScale, M(*valsSrcTileScale), M(*grad), gradMult, M(*gradGate), M(*gradVals), dExpertWeight)
-    if (gradType == TS2_BF16 && gradOutType == TS2_BF16) {
+    if (gradType == TS2_BF16 && gradOutType == TS2_E4M3 && Aligned16(gate->ptr, gate->strideBytes) && Aligned16(vals->ptr, vals->strideBytes) &&
+        Aligned16(grad->ptr, grad->strideBytes) && (((uintptr_t)gradGate->ptr | gradGate->strideBytes | (uintptr_t)gradVals->ptr | gradVals->strideBytes) & 7) == 0) {
+        hipLaunchKernelGGL(BackpropRowTileNormalizeLoLUmoe8, dim3((lenMoe + 3) / 4), dim3(256), 0, STREAM, lenMoe, tiles, xpSampleWeight, M(*gate),
+            M(*vals), valsScale, M(*valsSrcTileScale), M(*grad), gradMult, M(*gradGate), M(*gradVals), dExpertWeight);
+    } else if (gradType == TS2_BF16 && gradOutType == TS2_BF16) {
         LAUNCH_M(TBF16, TBF16);
     } else if (gradType == TS2_BF16 && gradOutType == TS2_E4M3) {
         LAUNCH_M(TBF16, TE4M3);
