@@ -486,7 +486,7 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
                 return;
             }
         }
-        if constexpr ((CT == C_BF16 || CT == C_F16 || CT == C_F32) && EPI == TS2_EPI_STORE && !KT) {
+        if constexpr ((CT == C_BF16 || CT == C_F16 || CT == C_F32) && EPI == TS2_EPI_STORE) {
             // every row of the wave tile is live, no atomics, rows within the descriptor's reach: the stores with scalar addressing
             const int firstRow = rowBase + wm * (32 * WTM);
             if (p.splitK <= 1 && firstRow + 32 * WTM <= mLive && (int64_t)32 * WTM * p.ldc < ((int64_t)1 << 31)) {
