@@ -64,6 +64,40 @@ def test_fp8_product_at_the_size_of_the_dense_model(L):
     assert (c[i].double() - ref).abs().max().item() <= 2e-4 * ref.abs().max().item()
 
 
+def test_fp8_delta_product_on_untransposed_operands_at_the_size_of_the_dense_model(L):
+    """config[2]: the delta of the FFN expand matrix, 8192 x 2048 over 32768 tokens, contracting over the rows of the gradient
+    [token][8192] and the layer input [token][2048] as they lie (kMajor).  fp32 store: checksums within 1e-4 of the largest result
+    times sqrt(count), one row recomputed directly; the packed delta (what the operator stores) dequantised within 1/254 of each
+    row tile's maximum of the fp32 result."""
+    print("case fp8 K-major delta full size", flush=True)
+    lib = L.load()
+    m, n, k = 8192, 2048, 32768
+    g = torch.Generator(device="cuda").manual_seed(4)
+    a = (torch.randn((k, m), device="cuda", generator=g) * 2).to(torch.float8_e4m3fn)     # gradient [token][m]
+    b = (torch.randn((k, n), device="cuda", generator=g) * 2).to(torch.float8_e4m3fn)     # input [token][n]
+    c = torch.empty((m, n), dtype=torch.float32, device="cuda")
+    lib.gemm_nt(a.view(torch.uint8), b.view(torch.uint8), c, L.E4M3, L.F32, m=m, n=n, k=k, k_major=True)
+    a64sum, b64sum = a.double().sum(1), b.double().sum(1)                                   # per token
+    col = (a64sum.unsqueeze(0) @ b.double()).ravel()                                        # sum_i C[i][j]
+    row = (a.double().t() @ b64sum.unsqueeze(1)).ravel()                                    # sum_j C[i][j]
+    c64 = c.double()
+    scale = c64.abs().max().item()
+    assert (c64.sum(0) - col).abs().max().item() <= 1e-4 * scale * np.sqrt(m)
+    assert (c64.sum(1) - row).abs().max().item() <= 1e-4 * scale * np.sqrt(n)
+    i = 4321
+    ref = a[:, i].double() @ b.double()
+    assert (c[i].double() - ref).abs().max().item() <= 2e-4 * ref.abs().max().item()
+    d8 = torch.empty((m, n), dtype=torch.int8, device="cuda")
+    ts = torch.empty((n // 128, m), device="cuda")
+    lib.gemm_nt(a.view(torch.uint8), b.view(torch.uint8), d8, L.E4M3, L.I8, epilogue=L.EPI_ROW_TILE_MAXNORM, tile_scale=ts, m=m, n=n, k=k,
+                k_major=True)
+    torch.cuda.synchronize()
+    deq = d8.float().view(m, n // 128, 128) * ts.t().unsqueeze(2)
+    tile_max = c.view(m, n // 128, 128).abs().amax(2, keepdim=True)
+    assert ((deq - c.view(m, n // 128, 128)).abs() <= tile_max / 254 * 1.0001 + 1e-30).all()
+    assert torch.allclose(ts.t(), tile_max.squeeze(2) / 127, rtol=1e-6)
+
+
 def test_attention_at_full_size_treats_the_sequences_of_a_batch_independently(L):
     """config[3]: 16 sequences x 2048 tokens, 16 heads.  Forward, dQ, dK and dV of one sequence taken from the batch run equal, bit
     for bit, the run of that sequence alone (same tiles, same order of operations); dK/dV are linear in dO."""
