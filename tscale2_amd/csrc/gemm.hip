@@ -597,6 +597,105 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
     }
 }
 
+// The normalising epilogue (TStoreRowTileNormalize / TStoreRowTileNormalizeRope) of the 256x256 ring kernel on accumulators that the
+// MFMAs produced transposed (operands swapped: a block holds C^T, so a lane owns one ROW of the block and its registers walk along the
+// columns, four consecutive ones per e-quad).  The sum of squares of a row's 128-column tile is then 64 in-lane terms plus one swap
+// with the other half wave, one square root and reciprocal per lane and block row, the rotated pairs of RoPE sit in one lane - against
+// five cross-lane steps for each of the 16 rows of a block row, and 16 square roots per lane, in the lane = column layout.  The bf16
+// rows go through the wave's own 32 KB of LDS (free after the main loop; 8-byte granules XOR-swizzled by the row so that the 32 rows
+// of a store hit different banks) and leave as 16-byte stores of whole 256-byte row segments.
+template <int TYPE, class TAcc>
+__device__ __forceinline__ void NormEpilogueRows(const GemmP &p, TAcc (&acc)[4][4], uint8_t *waveLds, int rowBase, int colBase, int wm, int wn,
+    int lane)
+{
+    const int half = lane >> 5, l32 = lane & 31;
+    float scale = p.alpha;
+    if (p.alphaPtr) {
+        scale *= *p.alphaPtr;
+    }
+    const int mLive = p.mLive > 0 ? p.mLive : p.m;
+    const int tile = (colBase + wn * 128) / TILE;
+    const int firstRow = rowBase + wm * 128;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = i * 32 + l32; // row inside the wave tile
+        const int row = firstRow + r;
+        const bool live = row < mLive;
+        float rs = scale;
+        if (p.rowScale) {
+            rs *= p.rowScale[row];
+        }
+        float v[4][16];
+        float sum2 = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                v[j][e] = live ? (float)acc[i][j][e] * rs : 0.f;
+                sum2 += v[j][e] * v[j][e];
+            }
+        }
+        if (p.normalize) {
+            float a, b;
+            LaneSwap32(sum2, &a, &b);
+            sum2 = a + b;
+            float discr = 0;
+            if (sum2 > 0) {
+                discr = __builtin_amdgcn_sqrtf(sum2 * (1.f / TILE)) * p.vecScale;
+                const float inv = __builtin_amdgcn_rcpf(discr);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        v[j][e] *= inv;
+                    }
+                }
+            }
+            if (half == 0) {
+                p.tileScale[(int64_t)tile * p.ldTileScale + row] = discr;
+            }
+        }
+        if (p.rope && live) {
+            const float *ropeRow = p.rope + (int64_t)row * p.ldRope;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                for (int e = 0; e < 16; e += 2) {
+                    const float2 cs = *(const float2 *)(ropeRow + j * 32 + (e >> 2) * 8 + half * 4 + (e & 3));
+                    const float x = v[j][e], y = v[j][e + 1];
+                    v[j][e] = x * cs.x - y * cs.y;
+                    v[j][e + 1] = y * cs.x + x * cs.y;
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int g = (j * 8 + q * 2 + half) ^ ((r & 15) << 1); // 8-byte granule of the row, swizzled
+                *(uint2 *)(waveLds + r * 256 + g * 8) = make_uint2(PackBf16x2(v[j][4 * q], v[j][4 * q + 1]), PackBf16x2(v[j][4 * q + 2], v[j][4 * q + 3]));
+            }
+        }
+    }
+    // rows back out: 16 lanes take one row's 256 bytes, four rows per store instruction
+    typedef unsigned v4u_t __attribute__((ext_vector_type(4)));
+    const int t = lane & 15, rsub = lane >> 4;
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(p.c + (int64_t)firstRow * p.ldc), 0, (int)(128 * p.ldc), 0x00020000);
+    const int ldc = (int)p.ldc;
+    const int laneOff = rsub * ldc + (colBase + wn * 128) * 2 + t * 16;
+#pragma unroll
+    for (int it = 0; it < 32; ++it) {
+        const int r = it * 4 + rsub;
+        const int g = (2 * t) ^ ((r & 15) << 1);
+        const uint4 d = *(const uint4 *)(waveLds + r * 256 + g * 8);
+        if (p.streamC) {
+            __builtin_amdgcn_raw_buffer_store_b128((v4u_t){d.x, d.y, d.z, d.w}, rsrc, laneOff, it * 4 * ldc, 2);
+        } else {
+            __builtin_amdgcn_raw_buffer_store_b128((v4u_t){d.x, d.y, d.z, d.w}, rsrc, laneOff, it * 4 * ldc, 0);
+        }
+    }
+}
+
 template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT>
 __global__ void __launch_bounds__(256, 1) GemmNT(GemmP p)
 {
@@ -1105,6 +1204,8 @@ template <int TYPE, int CT, int EPI, bool TN = false, int WT = 4> __global__ voi
     constexpr int WTM = WT, WTN = WT, WN = 2, NW = 4, BM = 64 * WT, BN = 64 * WT;
     static_assert(WT == 4 || (WT == 2 && TYPE == T_FP8 && !TN), "the 128x128 ring takes e4m3 operands with the contraction along the rows");
     static_assert(!TN || TYPE != T_I8, "contraction-major operands: e4m3 and bf16");
+    // the normalising epilogue of the large tile works on transposed blocks: the MFMAs take their operands the other way round
+    constexpr bool SWAPC = CT == C_BF16NORM && WT == 4 && !TN;
     constexpr int ESZ = TYPE == T_BF16 ? 2 : 1;
     constexpr int KR = BKB / ESZ; // contraction rows of a step (K-major operands)
     __shared__ __attribute__((aligned(1024))) uint8_t sA0[BM * BKB];
@@ -1286,7 +1387,7 @@ template <int TYPE, int CT, int EPI, bool TN = false, int WT = 4> __global__ voi
 #define MFMA_ROWS(SET, I0, I1)                                                                                                             \
     do {                                                                                                                                   \
         _Pragma("unroll") for (int i = I0; i < I1; ++i) _Pragma("unroll") for (int j = 0; j < WTN; ++j) acc[i][j] =                        \
-            mfma(fa[SET][i], fb[SET][j], acc[i][j]);                                                                                       \
+            mfma(SWAPC ? fb[SET][j] : fa[SET][i], SWAPC ? fa[SET][i] : fb[SET][j], acc[i][j]);                                             \
     } while (0)
     // pin the order inside a region: REP groups of (NM MFMAs, NG global loads, NDS LDS reads)
 #define INTERLEAVE(REP, NM, NG, NDS)                                                                                                       \
@@ -1438,7 +1539,13 @@ template <int TYPE, int CT, int EPI, bool TN = false, int WT = 4> __global__ voi
 #undef RING_LOAD_A
 #undef RING_LOAD_B
 #undef RING_LOAD
-    Epilogue<TYPE, WTM, WTN, CT, EPI, false>(p, acc, facc, sA0, rowBase, colBase, wm, wn, half, l32);
+    if constexpr (SWAPC) {
+        // every wave stages its rows in a stage array of its own
+        uint8_t *waveLds = wave == 0 ? sA0 : wave == 1 ? sA1 : wave == 2 ? sA2 : sB0;
+        NormEpilogueRows<TYPE>(p, acc, waveLds, rowBase, colBase, wm, wn, lane);
+    } else {
+        Epilogue<TYPE, WTM, WTN, CT, EPI, false>(p, acc, facc, sA0, rowBase, colBase, wm, wn, half, l32);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------------------------------------
@@ -1932,7 +2039,9 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
     p.rope = (const float *)a->rope.ptr;
     p.ldRope = a->rope.strideBytes / 4;
     if (a->epilogue == TS2_EPI_ROW_TILE_NORM) {
-        if (a->cType != TS2_BF16 || (a->c.strideBytes & 3)) {
+        // (the large tile stores rows of 16 bytes per lane through a buffer descriptor over 128 rows)
+        if (a->cType != TS2_BF16 || (a->c.strideBytes & 3) || (int64_t)128 * a->c.strideBytes >= ((int64_t)1 << 31) ||
+            ((a->m % 256) == 0 && (a->n % 256) == 0 && (((uintptr_t)a->c.ptr | a->c.strideBytes) & 15))) {
             return TS2_ERR_UNSUPPORTED;
         }
         if ((a->normalize && (!a->tileScale.ptr || a->tileScale.y < a->n / 128 || a->tileScale.x < a->m)) ||
