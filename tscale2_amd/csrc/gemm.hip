@@ -604,7 +604,8 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
 // five cross-lane steps for each of the 16 rows of a block row, and 16 square roots per lane, in the lane = column layout.  The bf16
 // rows go through the wave's own 32 KB of LDS (free after the main loop; 8-byte granules XOR-swizzled by the row so that the 32 rows
 // of a store hit different banks) and leave as 16-byte stores of whole 256-byte row segments.
-template <int TYPE, class TAcc>
+// NORM false: the plain 16-bit store (TStoreScaled) through the same staging; F16: IEEE half instead of bf16.
+template <int TYPE, bool NORM, bool F16, class TAcc>
 __device__ __forceinline__ void NormEpilogueRows(const GemmP &p, TAcc (&acc)[4][4], uint8_t *waveLds, int rowBase, int colBase, int wm, int wn,
     int lane)
 {
@@ -635,7 +636,7 @@ __device__ __forceinline__ void NormEpilogueRows(const GemmP &p, TAcc (&acc)[4][
                 sum2 += v[j][e] * v[j][e];
             }
         }
-        if (p.normalize) {
+        if (NORM && p.normalize) {
             float a, b;
             LaneSwap32(sum2, &a, &b);
             sum2 = a + b;
@@ -655,7 +656,7 @@ __device__ __forceinline__ void NormEpilogueRows(const GemmP &p, TAcc (&acc)[4][
                 p.tileScale[(int64_t)tile * p.ldTileScale + row] = discr;
             }
         }
-        if (p.rope && live) {
+        if (NORM && p.rope && live) {
             const float *ropeRow = p.rope + (int64_t)row * p.ldRope;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -673,7 +674,8 @@ __device__ __forceinline__ void NormEpilogueRows(const GemmP &p, TAcc (&acc)[4][
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const int g = (j * 8 + q * 2 + half) ^ ((r & 15) << 1); // 8-byte granule of the row, swizzled
-                *(uint2 *)(waveLds + r * 256 + g * 8) = make_uint2(PackBf16x2(v[j][4 * q], v[j][4 * q + 1]), PackBf16x2(v[j][4 * q + 2], v[j][4 * q + 3]));
+                *(uint2 *)(waveLds + r * 256 + g * 8) = F16 ? make_uint2(PackF16x2(v[j][4 * q], v[j][4 * q + 1]), PackF16x2(v[j][4 * q + 2], v[j][4 * q + 3]))
+                                                            : make_uint2(PackBf16x2(v[j][4 * q], v[j][4 * q + 1]), PackBf16x2(v[j][4 * q + 2], v[j][4 * q + 3]));
             }
         }
     }
@@ -683,12 +685,19 @@ __device__ __forceinline__ void NormEpilogueRows(const GemmP &p, TAcc (&acc)[4][
     const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(p.c + (int64_t)firstRow * p.ldc), 0, (int)(128 * p.ldc), 0x00020000);
     const int ldc = (int)p.ldc;
     const int laneOff = rsub * ldc + (colBase + wn * 128) * 2 + t * 16;
+    const bool aligned16 = (((uintptr_t)p.c | (uintptr_t)p.ldc) & 15) == 0;
 #pragma unroll
     for (int it = 0; it < 32; ++it) {
         const int r = it * 4 + rsub;
         const int g = (2 * t) ^ ((r & 15) << 1);
         const uint4 d = *(const uint4 *)(waveLds + r * 256 + g * 8);
-        if (p.streamC) {
+        if (!aligned16) {
+            // (a result whose rows do not start on 16 bytes: the same data in 4-byte stores)
+            __builtin_amdgcn_raw_buffer_store_b32(d.x, rsrc, laneOff, it * 4 * ldc, 0);
+            __builtin_amdgcn_raw_buffer_store_b32(d.y, rsrc, laneOff, it * 4 * ldc + 4, 0);
+            __builtin_amdgcn_raw_buffer_store_b32(d.z, rsrc, laneOff, it * 4 * ldc + 8, 0);
+            __builtin_amdgcn_raw_buffer_store_b32(d.w, rsrc, laneOff, it * 4 * ldc + 12, 0);
+        } else if (p.streamC) {
             __builtin_amdgcn_raw_buffer_store_b128((v4u_t){d.x, d.y, d.z, d.w}, rsrc, laneOff, it * 4 * ldc, 2);
         } else {
             __builtin_amdgcn_raw_buffer_store_b128((v4u_t){d.x, d.y, d.z, d.w}, rsrc, laneOff, it * 4 * ldc, 0);
@@ -1205,7 +1214,7 @@ template <int TYPE, int CT, int EPI, bool TN = false, int WT = 4> __global__ voi
     static_assert(WT == 4 || (WT == 2 && TYPE == T_FP8 && !TN), "the 128x128 ring takes e4m3 operands with the contraction along the rows");
     static_assert(!TN || TYPE != T_I8, "contraction-major operands: e4m3 and bf16");
     // the normalising epilogue of the large tile works on transposed blocks: the MFMAs take their operands the other way round
-    constexpr bool SWAPC = CT == C_BF16NORM && WT == 4 && !TN;
+    constexpr bool SWAPC = (CT == C_BF16NORM || ((CT == C_BF16 || CT == C_F16) && EPI == TS2_EPI_STORE)) && WT == 4 && !TN;
     constexpr int ESZ = TYPE == T_BF16 ? 2 : 1;
     constexpr int KR = BKB / ESZ; // contraction rows of a step (K-major operands)
     __shared__ __attribute__((aligned(1024))) uint8_t sA0[BM * BKB];
@@ -1542,7 +1551,7 @@ template <int TYPE, int CT, int EPI, bool TN = false, int WT = 4> __global__ voi
     if constexpr (SWAPC) {
         // every wave stages its rows in a stage array of its own
         uint8_t *waveLds = wave == 0 ? sA0 : wave == 1 ? sA1 : wave == 2 ? sA2 : sB0;
-        NormEpilogueRows<TYPE>(p, acc, waveLds, rowBase, colBase, wm, wn, lane);
+        NormEpilogueRows<TYPE, CT == C_BF16NORM, CT == C_F16>(p, acc, waveLds, rowBase, colBase, wm, wn, lane);
     } else {
         Epilogue<TYPE, WTM, WTN, CT, EPI, false>(p, acc, facc, sA0, rowBase, colBase, wm, wn, half, l32);
     }
@@ -2001,6 +2010,9 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
     if ((a->cType == TS2_BF16 || a->cType == TS2_F16) && (a->c.strideBytes & 3)) {
         return TS2_ERR_ALIGN; // bf16 results are stored two columns at a time
     }
+    if ((a->cType == TS2_BF16 || a->cType == TS2_F16) && (int64_t)128 * a->c.strideBytes >= ((int64_t)1 << 31)) {
+        return TS2_ERR_UNSUPPORTED; // the row stores address 128 rows of C from one 32-bit offset
+    }
     int splitK = a->splitK > 1 ? a->splitK : 1;
     if (splitK > 1 && (a->cType != TS2_F32 || a->epilogue == TS2_EPI_ROW_TILE_MAXNORM)) {
         return TS2_ERR_UNSUPPORTED;
@@ -2040,8 +2052,7 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
     p.ldRope = a->rope.strideBytes / 4;
     if (a->epilogue == TS2_EPI_ROW_TILE_NORM) {
         // (the large tile stores rows of 16 bytes per lane through a buffer descriptor over 128 rows)
-        if (a->cType != TS2_BF16 || (a->c.strideBytes & 3) || (int64_t)128 * a->c.strideBytes >= ((int64_t)1 << 31) ||
-            ((a->m % 256) == 0 && (a->n % 256) == 0 && (((uintptr_t)a->c.ptr | a->c.strideBytes) & 15))) {
+        if (a->cType != TS2_BF16 || (a->c.strideBytes & 3) || (int64_t)128 * a->c.strideBytes >= ((int64_t)1 << 31)) {
             return TS2_ERR_UNSUPPORTED;
         }
         if ((a->normalize && (!a->tileScale.ptr || a->tileScale.y < a->n / 128 || a->tileScale.x < a->m)) ||
