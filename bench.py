@@ -247,12 +247,10 @@ def bandwidth_kernels(iters=10):
     gate = rnd(R, F, bf16); vals = rnd(R, F, bf16); rg = torch.empty((R, F), dtype=u8, device=dev)
     add("MatrixLoLU bf16,bf16->e4m3 [32768x8192]", R * F * 5, lambda: L.call("ts2_matrix_lolu", R, R, gate, vals, 1.0, rg, L.E4M3))
     grad = rnd(R, F, bf16); vts = torch.rand((F // 128, R), device=dev) + 0.5
-    gg = torch.empty((R, F), dtype=u8, device=dev); gv = torch.empty_like(gg); ggT = torch.empty((F, R), dtype=u8, device=dev); gvT = torch.empty_like(ggT)
-    add("BackpropRowTileNormalizeLoLU (+ transposed copies) bf16->e4m3 [32768x8192]", R * F * 10 + R * F // 128 * 4,
-        lambda: L.call("ts2_backprop_row_tile_normalize_lolu_t", R, R, gate, vals, 1 / 24, vts, grad, gg, gv, ggT, gvT))
-    add("TransposeQuant e4m3 byte transpose [32768x8192]", R * F * 2,
-        lambda: L.call("ts2_transpose_quant", R, R, gg, L.E4M3, None, None, 0, None, ggT, L.E4M3, None))
-    del gate, vals, rg, grad, gg, gv, ggT, gvT, vts
+    gg = torch.empty((R, F), dtype=u8, device=dev); gv = torch.empty_like(gg)
+    add("BackpropRowTileNormalizeLoLU bf16,bf16,bf16->e4m3,e4m3 [32768x8192]", R * F * 8 + R * F // 128 * 4,
+        lambda: L.call("ts2_backprop_row_tile_normalize_lolu", R, R, gate, vals, 1 / 24, vts, grad, L.BF16, gg, gv, L.E4M3))
+    del gate, vals, rg, grad, gg, gv, vts
     # ---- attention epilogue kernels [R][Q]
     gate = rnd(R, Q, bf16); vals = rnd(R, Q, bf16); grad = rnd(R, Q, bf16)
     dgate = torch.empty((R, Q), dtype=u8, device=dev); dval = torch.empty((R, Q), dtype=bf16, device=dev); dsc = torch.empty((Q // 128, R), device=dev)
@@ -292,9 +290,9 @@ def bandwidth_kernels(iters=10):
     src8 = rnd(N4, D4, u8); grp = torch.empty((len_moe, D4), dtype=u8, device=dev)
     add("MoeGroupSamples 8-bit gather into expert order [131072 of 139264 rows x 1024]", tot * D4 * 2 + len_moe * 4,
         lambda: L.call("ts2_moe_group_samples", len_moe, 1, src8, t["sid"], grp))
-    full = rnd(len_moe, D4, f32); comb = torch.empty((N4, D4), device=dev)
-    add("CombineExperts f32 2-way gather-sum [65536x1024]", tot * D4 * 4 + N4 * D4 * 4 + tot * 8,
-        lambda: L.call("ts2_combine_experts", N4, K4, full, L.F32, C.byref(tb), 1.0, None, comb, 0))
+    full = rnd(len_moe, D4, bf16); comb = torch.empty((N4, D4), device=dev)
+    add("CombineExperts bf16 2-way gather-sum -> f32 [65536x1024]", tot * D4 * 2 + N4 * D4 * 4 + tot * 8,
+        lambda: L.call("ts2_combine_experts", N4, K4, full, L.BF16, C.byref(tb), 1.0, None, comb, 0))
     return res
 
 
