@@ -305,14 +305,16 @@ def fp8_backward_gemms(n, dim, ffn, iters=100, warm=20, only_dominant=False):
     lib = L.load()
     out = []
 
-    def run(name, m, nn, k, packed=False):
-        a = torch.randint(0, 120, (m, k), dtype=torch.uint8, device="cuda"); b = torch.randint(0, 120, (nn, k), dtype=torch.uint8, device="cuda")
+    def run(name, m, nn, k, packed=False, ctype=None):
         if packed:
+            # the delta products of the step contract over the rows of both operands as they lie in memory (K-major form)
+            a = torch.randint(0, 120, (k, m), dtype=torch.uint8, device="cuda"); b = torch.randint(0, 120, (k, nn), dtype=torch.uint8, device="cuda")
             c = torch.empty((m, nn), dtype=torch.int8, device="cuda"); ts = torch.empty((nn // 128, m), device="cuda")
-            fn = lambda: lib.gemm_nt(a, b, c, L.E4M3, L.I8, epilogue=L.EPI_ROW_TILE_MAXNORM, tile_scale=ts)  # noqa: E731
+            fn = lambda: lib.gemm_nt(a, b, c, L.E4M3, L.I8, epilogue=L.EPI_ROW_TILE_MAXNORM, tile_scale=ts, m=m, n=nn, k=k, k_major=True)  # noqa: E731
         else:
-            c = torch.empty((m, nn), dtype=torch.float32, device="cuda")
-            fn = lambda: lib.gemm_nt(a, b, c, L.E4M3, L.F32)  # noqa: E731
+            a = torch.randint(0, 120, (m, k), dtype=torch.uint8, device="cuda"); b = torch.randint(0, 120, (nn, k), dtype=torch.uint8, device="cuda")
+            c = torch.empty((m, nn), dtype=torch.bfloat16 if ctype == L.BF16 else torch.float32, device="cuda")
+            fn = lambda: lib.gemm_nt(a, b, c, L.E4M3, ctype or L.F32)  # noqa: E731
         for _ in range(warm):
             fn()
         torch.cuda.synchronize()
@@ -324,10 +326,10 @@ def fp8_backward_gemms(n, dim, ffn, iters=100, warm=20, only_dominant=False):
     first = run("dX: dY[tokens x ffn] x W^T (FFN expand / gate), fp32 result", n, dim, ffn)
     if only_dominant:
         return out, first
-    run("dX: dY[tokens x dim] x W^T (FFN contract), fp32 result", n, ffn, dim)
+    run("dX: dY[tokens x dim] x W^T (FFN contract), bf16 result", n, ffn, dim, ctype=L.BF16)
     run("dX: dY[tokens x dim] x W^T (attention Q/K/V/gate/combiner), fp32 result", n, dim, dim)
-    run("delta: dY^T[ffn x tokens] x X^T (FFN expand / gate), packed i8 result", ffn, dim, n, packed=True)
-    run("delta: dY^T[dim x tokens] x X^T (FFN contract), packed i8 result", dim, ffn, n, packed=True)
+    run("delta: dY^T[ffn x tokens] x X (FFN expand / gate), both operands token-major, packed i8 result", ffn, dim, n, packed=True)
+    run("delta: dY^T[dim x tokens] x X (FFN contract), both operands token-major, packed i8 result", dim, ffn, n, packed=True)
     return out, first
 
 

@@ -350,3 +350,31 @@ def test_two_steps_with_a_real_optimiser_update(mode):
             np.testing.assert_allclose(a, b, rtol=0, atol=1e-6 * np.abs(b).max())
         else:
             assert np.array_equal(a, b), nm
+
+
+def test_final_delta_of_a_vocabulary_with_a_partial_last_round_of_tiles():
+    """34048 x 512 final matrix, 16384 tokens: 133 x 2 large tiles.  The chip takes 256 at a time, so the driver runs the last five
+    256-row groups of the vocabulary as slices of the token axis (stored fp32 products, packed afterwards) beside the main product.
+    The packed delta is checked against an fp32 product of the device's own soft-max gradient and final state: every element within
+    half a step of its row tile's scale, in the main rows and in the sliced ones alike.  The oracle is not run at this size."""
+    print("case final delta with token-sliced tail rows", flush=True)
+    VEC_SCALE = 1 / 24.0  # STATE_VEC_SCALE, src/gpt/compute/cfg_precision.h:72-77: the delta product's factor
+    h = Harness(E4M3, dim=512, heads=4, ffn_tiles=4, depth=1, vocab=34048, frag_count=16, frag_len=1024, wide_window=64, seed=11)
+    m = h.device_model()
+    m.backprop()
+    torch.cuda.synchronize()
+    depth = h.depth
+    g = m.array("finalGrad").float()                                                   # [R][vocab]
+    fn = m.array("normState", depth).view(torch.float8_e4m3fn).float()                 # [R][dim], 8-bit codes as values
+    assert g.shape[0] == h.n and fn.shape[0] == h.n
+    want = (g.t() @ fn) * VEC_SCALE
+    got = torch.from_numpy(m.get_delta(-2, 0, h.vocab, h.dim)).cuda()
+    tile_max = want.view(h.vocab, h.dim // 128, 128).abs().amax(dim=2, keepdim=True)
+    err = ((got - want).view(h.vocab, h.dim // 128, 128).abs() / (tile_max / 127 + 1e-30)).amax(dim=(1, 2))
+    live = tile_max.amax(dim=(1, 2)) > 0
+    assert live.float().mean() > 0.3
+    print("worst error in steps of the tile scale: main rows", float(err[:32768][live[:32768]].max()), "sliced rows",
+          float(err[32768:][live[32768:]].max()), flush=True)
+    assert float(err[live].max()) <= 0.52
+    assert float(got[~live].abs().max() if (~live).any() else 0.0) == 0.0
+    m.close()

@@ -153,6 +153,7 @@ struct ts2_model {
     size_t sPartialFloats = 0;
     float *sRowScale = 0, *sTileMax = 0, *sTileScale = 0;
     int maxW = 0, RP = 0; // RP = rows of the row-indexed scratch (max(R, lenMoe))
+    int cuCount = 256;
 
     void *Dev(size_t bytes)
     {
@@ -160,8 +161,10 @@ struct ts2_model {
         if (hipMalloc(&p, bytes ? bytes : 16) != hipSuccess) {
             return nullptr;
         }
-        hipMemset(p, 0, bytes ? bytes : 16);
         allocs.push_back(p);
+        if (hipMemset(p, 0, bytes ? bytes : 16) != hipSuccess) {
+            return nullptr;
+        }
         return p;
     }
     bool Alloc(Arr *a, int rows, int cols, int type)
@@ -177,7 +180,7 @@ struct ts2_model {
     ~ts2_model()
     {
         for (void *p : allocs) {
-            hipFree(p);
+            (void)hipFree(p);
         }
     }
 };
@@ -833,7 +836,40 @@ int FinalBackward(ts2_model *M, void *s)
     h.epilogue = TS2_EPI_ROW_TILE_MAXNORM;
     h.tileScale = M->finalW.deltaTileScale.m;
     h.splitK = 1;
-    CK(ts2_gemm_nt(&h, s));
+    // One workgroup per CU at a time: the 256-row groups of the vocabulary beyond the last full round of the chip would take a round of
+    // their own at a fraction of the CUs.  They run as slices of the token axis instead (stored fp32 products, packed afterwards).
+    const int tilesM = VP / 256, tilesN = D / 256, cus = M->cuCount;
+    const int rowsPerRound = tilesN > 0 && cus % tilesN == 0 ? cus / tilesN : 0;
+    const int tailRows = h.kMajor && rowsPerRound > 0 && tilesM > rowsPerRound ? tilesM % rowsPerRound : 0;
+    int tailSplits = tailRows > 0 ? cus / (tailRows * tilesN) : 0;
+    tailSplits = tailSplits > 8 ? 8 : tailSplits;
+    if (tailSplits >= 2 && R / tailSplits >= 2048 && (size_t)tailSplits * tailRows * 256 * D <= M->sPartialFloats) {
+        const int mainM = (tilesM - tailRows) * 256, tailM = tailRows * 256;
+        h.m = mainM;
+        CK(ts2_gemm_nt(&h, s));
+        ts2_gemm_args t = h;
+        t.a.ptr = (uint8_t *)h.a.ptr + (size_t)mainM * 2; // columns mainM.. of the gradient [token][vocabulary]
+        t.a.x = tailM;
+        t.m = tailM;
+        Arr part = Flat(M->sPartial, tailSplits * tailM, D, TS2_F32);
+        t.c = part.m;
+        t.c.y = tailM;
+        t.cType = TS2_F32;
+        t.alpha = 1.f;
+        t.epilogue = TS2_EPI_STORE;
+        t.tileScale = ts2_mat{};
+        t.splitK = tailSplits;
+        t.splitSlabBytes = (int64_t)tailM * part.m.strideBytes;
+        CK(ts2_gemm_nt(&t, s));
+        ts2_mat dTail = M->finalW.delta.m, sTail = M->finalW.deltaTileScale.m;
+        dTail.ptr = (uint8_t *)dTail.ptr + (size_t)mainM * dTail.strideBytes;
+        dTail.y = tailM;
+        sTail.ptr = (uint8_t *)sTail.ptr + (size_t)mainM * 4; // tile scales are [D / 128][vocabulary row]
+        sTail.x = tailM;
+        CK(ts2_pack_delta(&part.m, tailSplits, t.splitSlabBytes, tailM, D, VEC, nullptr, &dTail, &sTail, s));
+    } else {
+        CK(ts2_gemm_nt(&h, s));
+    }
     return ts2_backprop_final_normalize(M->len, R, M->normState[depth].P(), M->mode, M->stateScale[depth].P(), M->dNormState.P(), M->stateGrad.P(),
         M->stateGradFast.P(), M->fastGradType, M->gradMaxNorm, s);
 }
@@ -876,6 +912,10 @@ extern "C" ts2_model *ts2_model_create(const ts2_model_config *cfg)
     M->cfg = *cfg;
     M->mode = cfg->mode;
     M->fastGradType = cfg->mode == TS2_I8 ? TS2_BF16 : TS2_E4M3;
+    if (ts2_device_info(&M->cuCount, nullptr) != TS2_OK || M->cuCount <= 0) {
+        delete M;
+        return nullptr;
+    }
     M->kTile = cfg->kTile > 0 ? cfg->kTile : 512;
     M->R = RoundUp(cfg->maxLen, M->kTile > 128 ? M->kTile : 128);
     int D = cfg->dim, H = cfg->headCount, F = cfg->ffnDim, X = cfg->expertDim, E = cfg->expertCount, V = cfg->vocab, R = M->R;
