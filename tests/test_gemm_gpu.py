@@ -503,6 +503,19 @@ def test_ring_pipeline_on_the_small_tile_equals_the_two_stage_loop(lib):
     a, b = codes((m, k)), codes((n, k))
     c16 = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
     both(lambda cfg: lib.gemm_nt(a, b, c16, L.E4M3, L.BF16, alpha=0.25, tile_config=cfg), [c16])
+    c32 = torch.zeros((m, n), device="cuda")
+    lib.gemm_nt(a, b, c32, L.E4M3, L.F32, alpha=0.25, tile_config=LOOP)
+    torch.cuda.synchronize()
+    assert torch.equal(c16, c32.bfloat16())  # and both are the rounded fp32 result (which leaves through another epilogue)
+    # live rows short of m, and a result whose rows start on 4-byte, not 16-byte, boundaries (the ring's 16-bit rows leave through LDS as
+    # 16-byte stores when they can)
+    both(lambda cfg: lib.gemm_nt(a, b, c16, L.E4M3, L.BF16, alpha=0.25, tile_config=cfg, m_live=500), [c16])
+    wide16 = torch.zeros((m, n + 2), dtype=torch.bfloat16, device="cuda")
+    wide16[:, n:] = 7
+    both(lambda cfg: lib.gemm_nt(a, b, wide16[:, :n], L.E4M3, L.BF16, alpha=0.25, tile_config=cfg), [wide16[:, :n]])
+    assert bool((wide16[:, n:] == 7).all())  # nothing written past the row's end
+    h16 = torch.zeros((m, n), dtype=torch.float16, device="cuda")
+    both(lambda cfg: lib.gemm_nt(a, b, h16, L.E4M3, L.F16, alpha=0.25, tile_config=cfg), [h16])
     cadd = torch.zeros((m, n), device="cuda")
     start = torch.randn((m, n), device="cuda", generator=g)
 

@@ -605,20 +605,27 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
 // rows go through the wave's own 32 KB of LDS (free after the main loop; 8-byte granules XOR-swizzled by the row so that the 32 rows
 // of a store hit different banks) and leave as 16-byte stores of whole 256-byte row segments.
 // NORM false: the plain 16-bit store (TStoreScaled) through the same staging; F16: IEEE half instead of bf16.
-template <int TYPE, bool NORM, bool F16, class TAcc>
-__device__ __forceinline__ void NormEpilogueRows(const GemmP &p, TAcc (&acc)[4][4], uint8_t *waveLds, int rowBase, int colBase, int wm, int wn,
+// WT = 2: the same for the 64x64 wave tile of the 128x128 ring kernel (plain 16-bit stores): rows of 128 bytes, 8 KB of the wave's stage
+// array, eight lanes per row on the way out.
+template <int TYPE, bool NORM, bool F16, int WT, class TAcc>
+__device__ __forceinline__ void NormEpilogueRows(const GemmP &p, TAcc (&acc)[WT][WT], uint8_t *waveLds, int rowBase, int colBase, int wm, int wn,
     int lane)
 {
+    static_assert(WT == 4 || !NORM, "a 128-column tile spans two waves of the 128x128 kernel: the normalising form is for the large tile");
+    constexpr int RW = 32 * WT;                 // rows and columns of the wave tile
+    constexpr int RB = RW * 2;                  // bytes of a staged row
+    constexpr int SWZ = WT == 4 ? 15 : 7;       // rows that differ in these bits (WT = 2: of r / 2) take different granule pairs
+    constexpr int SWS = WT == 4 ? 0 : 1;
     const int half = lane >> 5, l32 = lane & 31;
     float scale = p.alpha;
     if (p.alphaPtr) {
         scale *= *p.alphaPtr;
     }
     const int mLive = p.mLive > 0 ? p.mLive : p.m;
-    const int tile = (colBase + wn * 128) / TILE;
-    const int firstRow = rowBase + wm * 128;
+    const int tile = (colBase + wn * RW) / TILE;
+    const int firstRow = rowBase + wm * RW;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < WT; ++i) {
         const int r = i * 32 + l32; // row inside the wave tile
         const int row = firstRow + r;
         const bool live = row < mLive;
@@ -626,10 +633,10 @@ __device__ __forceinline__ void NormEpilogueRows(const GemmP &p, TAcc (&acc)[4][
         if (p.rowScale) {
             rs *= p.rowScale[row];
         }
-        float v[4][16];
+        float v[WT][16];
         float sum2 = 0;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < WT; ++j) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 v[j][e] = live ? (float)acc[i][j][e] * rs : 0.f;
@@ -645,7 +652,7 @@ __device__ __forceinline__ void NormEpilogueRows(const GemmP &p, TAcc (&acc)[4][
                 discr = __builtin_amdgcn_sqrtf(sum2 * (1.f / TILE)) * p.vecScale;
                 const float inv = __builtin_amdgcn_rcpf(discr);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
+                for (int j = 0; j < WT; ++j) {
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
                         v[j][e] *= inv;
@@ -659,7 +666,7 @@ __device__ __forceinline__ void NormEpilogueRows(const GemmP &p, TAcc (&acc)[4][
         if (NORM && p.rope && live) {
             const float *ropeRow = p.rope + (int64_t)row * p.ldRope;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < WT; ++j) {
 #pragma unroll
                 for (int e = 0; e < 16; e += 2) {
                     const float2 cs = *(const float2 *)(ropeRow + j * 32 + (e >> 2) * 8 + half * 4 + (e & 3));
@@ -670,37 +677,38 @@ __device__ __forceinline__ void NormEpilogueRows(const GemmP &p, TAcc (&acc)[4][
             }
         }
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < WT; ++j) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const int g = (j * 8 + q * 2 + half) ^ ((r & 15) << 1); // 8-byte granule of the row, swizzled
-                *(uint2 *)(waveLds + r * 256 + g * 8) = F16 ? make_uint2(PackF16x2(v[j][4 * q], v[j][4 * q + 1]), PackF16x2(v[j][4 * q + 2], v[j][4 * q + 3]))
-                                                            : make_uint2(PackBf16x2(v[j][4 * q], v[j][4 * q + 1]), PackBf16x2(v[j][4 * q + 2], v[j][4 * q + 3]));
+                const int g = (j * 8 + q * 2 + half) ^ (((r >> SWS) & SWZ) << 1); // 8-byte granule of the row, swizzled
+                *(uint2 *)(waveLds + r * RB + g * 8) = F16 ? make_uint2(PackF16x2(v[j][4 * q], v[j][4 * q + 1]), PackF16x2(v[j][4 * q + 2], v[j][4 * q + 3]))
+                                                           : make_uint2(PackBf16x2(v[j][4 * q], v[j][4 * q + 1]), PackBf16x2(v[j][4 * q + 2], v[j][4 * q + 3]));
             }
         }
     }
-    // rows back out: 16 lanes take one row's 256 bytes, four rows per store instruction
+    // rows back out: LPR lanes take one row's bytes, 64 / LPR rows per store instruction
     typedef unsigned v4u_t __attribute__((ext_vector_type(4)));
-    const int t = lane & 15, rsub = lane >> 4;
-    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(p.c + (int64_t)firstRow * p.ldc), 0, (int)(128 * p.ldc), 0x00020000);
+    constexpr int LPR = RB / 16, RPI = 64 / LPR;
+    const int t = lane % LPR, rsub = lane / LPR;
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(p.c + (int64_t)firstRow * p.ldc), 0, (int)(RW * p.ldc), 0x00020000);
     const int ldc = (int)p.ldc;
-    const int laneOff = rsub * ldc + (colBase + wn * 128) * 2 + t * 16;
+    const int laneOff = rsub * ldc + (colBase + wn * RW) * 2 + t * 16;
     const bool aligned16 = (((uintptr_t)p.c | (uintptr_t)p.ldc) & 15) == 0;
 #pragma unroll
-    for (int it = 0; it < 32; ++it) {
-        const int r = it * 4 + rsub;
-        const int g = (2 * t) ^ ((r & 15) << 1);
-        const uint4 d = *(const uint4 *)(waveLds + r * 256 + g * 8);
+    for (int it = 0; it < RW / RPI; ++it) {
+        const int r = it * RPI + rsub;
+        const int g = (2 * t) ^ (((r >> SWS) & SWZ) << 1);
+        const uint4 d = *(const uint4 *)(waveLds + r * RB + g * 8);
         if (!aligned16) {
             // (a result whose rows do not start on 16 bytes: the same data in 4-byte stores)
-            __builtin_amdgcn_raw_buffer_store_b32(d.x, rsrc, laneOff, it * 4 * ldc, 0);
-            __builtin_amdgcn_raw_buffer_store_b32(d.y, rsrc, laneOff, it * 4 * ldc + 4, 0);
-            __builtin_amdgcn_raw_buffer_store_b32(d.z, rsrc, laneOff, it * 4 * ldc + 8, 0);
-            __builtin_amdgcn_raw_buffer_store_b32(d.w, rsrc, laneOff, it * 4 * ldc + 12, 0);
+            __builtin_amdgcn_raw_buffer_store_b32(d.x, rsrc, laneOff, it * RPI * ldc, 0);
+            __builtin_amdgcn_raw_buffer_store_b32(d.y, rsrc, laneOff, it * RPI * ldc + 4, 0);
+            __builtin_amdgcn_raw_buffer_store_b32(d.z, rsrc, laneOff, it * RPI * ldc + 8, 0);
+            __builtin_amdgcn_raw_buffer_store_b32(d.w, rsrc, laneOff, it * RPI * ldc + 12, 0);
         } else if (p.streamC) {
-            __builtin_amdgcn_raw_buffer_store_b128((v4u_t){d.x, d.y, d.z, d.w}, rsrc, laneOff, it * 4 * ldc, 2);
+            __builtin_amdgcn_raw_buffer_store_b128((v4u_t){d.x, d.y, d.z, d.w}, rsrc, laneOff, it * RPI * ldc, 2);
         } else {
-            __builtin_amdgcn_raw_buffer_store_b128((v4u_t){d.x, d.y, d.z, d.w}, rsrc, laneOff, it * 4 * ldc, 0);
+            __builtin_amdgcn_raw_buffer_store_b128((v4u_t){d.x, d.y, d.z, d.w}, rsrc, laneOff, it * RPI * ldc, 0);
         }
     }
 }
@@ -956,6 +964,8 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN) / 4) GemmNTDirect(Gemm
     constexpr int NW = WM * WN; // waves per workgroup
     constexpr int BM = 32 * WTM * WM;
     constexpr int BN = 32 * WTN * WN;
+    // plain 16-bit results of the 128x128 e4m3 tile leave through the row-owning epilogue (a lane owns a row: operands swapped)
+    constexpr bool SWAPC = TYPE == T_FP8 && WTM == 2 && WTN == 2 && WM == 2 && WN == 2 && !KT && (CT == C_BF16 || CT == C_F16) && EPI == TS2_EPI_STORE;
     __shared__ __attribute__((aligned(1024))) uint8_t sA0[BM * BKB];
     __shared__ __attribute__((aligned(1024))) uint8_t sB0[BN * BKB];
     __shared__ __attribute__((aligned(1024))) uint8_t sA1[BM * BKB];
@@ -1082,7 +1092,7 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN) / 4) GemmNTDirect(Gemm
 #define MFMA_ROWS(SET, I0, I1)                                                                                                             \
     do {                                                                                                                                   \
         _Pragma("unroll") for (int i = I0; i < I1; ++i) _Pragma("unroll") for (int j = 0; j < WTN; ++j) acc[i][j] =                        \
-            mfma(fa[SET][i], fb[SET][j], acc[i][j]);                                                                                       \
+            mfma(SWAPC ? fb[SET][j] : fa[SET][i], SWAPC ? fa[SET][i] : fb[SET][j], acc[i][j]);                                             \
     } while (0)
 #define WAIT_VM0() __builtin_amdgcn_s_waitcnt(0x0F70) /* vmcnt(0): the direct loads have landed in LDS */
     const int tileSteps = KT ? p.kTileBytes / BKB : 0;
@@ -1193,7 +1203,12 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN) / 4) GemmNTDirect(Gemm
 #undef DIRECT_LOAD
 #undef WAIT_VM0
     __syncthreads();
-    Epilogue<TYPE, WTM, WTN, CT, EPI, KT>(p, acc, facc, sA0, rowBase, colBase, wm, wn, half, l32);
+    if constexpr (SWAPC) {
+        uint8_t *waveLds = wave == 0 ? sA0 : wave == 1 ? sB0 : wave == 2 ? sA1 : sB1;
+        NormEpilogueRows<TYPE, false, CT == C_F16, 2>(p, acc, waveLds, rowBase, colBase, wm, wn, lane);
+    } else {
+        Epilogue<TYPE, WTM, WTN, CT, EPI, KT>(p, acc, facc, sA0, rowBase, colBase, wm, wn, half, l32);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------------------------------------
@@ -1214,7 +1229,7 @@ template <int TYPE, int CT, int EPI, bool TN = false, int WT = 4> __global__ voi
     static_assert(WT == 4 || (WT == 2 && TYPE == T_FP8 && !TN), "the 128x128 ring takes e4m3 operands with the contraction along the rows");
     static_assert(!TN || TYPE != T_I8, "contraction-major operands: e4m3 and bf16");
     // the normalising epilogue of the large tile works on transposed blocks: the MFMAs take their operands the other way round
-    constexpr bool SWAPC = (CT == C_BF16NORM || ((CT == C_BF16 || CT == C_F16) && EPI == TS2_EPI_STORE)) && WT == 4 && !TN;
+    constexpr bool SWAPC = ((CT == C_BF16NORM && WT == 4) || ((CT == C_BF16 || CT == C_F16) && EPI == TS2_EPI_STORE)) && !TN;
     constexpr int ESZ = TYPE == T_BF16 ? 2 : 1;
     constexpr int KR = BKB / ESZ; // contraction rows of a step (K-major operands)
     __shared__ __attribute__((aligned(1024))) uint8_t sA0[BM * BKB];
@@ -1551,7 +1566,7 @@ template <int TYPE, int CT, int EPI, bool TN = false, int WT = 4> __global__ voi
     if constexpr (SWAPC) {
         // every wave stages its rows in a stage array of its own
         uint8_t *waveLds = wave == 0 ? sA0 : wave == 1 ? sA1 : wave == 2 ? sA2 : sB0;
-        NormEpilogueRows<TYPE, CT == C_BF16NORM, CT == C_F16>(p, acc, waveLds, rowBase, colBase, wm, wn, lane);
+        NormEpilogueRows<TYPE, CT == C_BF16NORM, CT == C_F16, WT>(p, acc, waveLds, rowBase, colBase, wm, wn, lane);
     } else {
         Epilogue<TYPE, WTM, WTN, CT, EPI, false>(p, acc, facc, sA0, rowBase, colBase, wm, wn, half, l32);
     }
