@@ -605,13 +605,13 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
 // rows go through the wave's own 32 KB of LDS (free after the main loop; 8-byte granules XOR-swizzled by the row so that the 32 rows
 // of a store hit different banks) and leave as 16-byte stores of whole 256-byte row segments.
 // NORM false: the plain 16-bit store (TStoreScaled) through the same staging; F16: IEEE half instead of bf16.
-// WT = 2: the same for the 64x64 wave tile of the 128x128 ring kernel (plain 16-bit stores): rows of 128 bytes, 8 KB of the wave's stage
-// array, eight lanes per row on the way out.
+// WT = 2: the same for the 64x64 wave tile of the 128x128 kernels: rows of 128 bytes, 8 KB of the wave's stage array, eight lanes per
+// row on the way out.  A 128-column tile spans the two waves of a row there: each leaves its 64-column sums of squares in xchg (LDS,
+// 4 x 64 floats outside the staged rows) and adds its neighbour's after one workgroup barrier.
 template <int TYPE, bool NORM, bool F16, int WT, class TAcc>
-__device__ __forceinline__ void NormEpilogueRows(const GemmP &p, TAcc (&acc)[WT][WT], uint8_t *waveLds, int rowBase, int colBase, int wm, int wn,
-    int lane)
+__device__ __forceinline__ void NormEpilogueRows(const GemmP &p, TAcc (&acc)[WT][WT], uint8_t *waveLds, float *xchg, int rowBase, int colBase,
+    int wm, int wn, int lane)
 {
-    static_assert(WT == 4 || !NORM, "a 128-column tile spans two waves of the 128x128 kernel: the normalising form is for the large tile");
     constexpr int RW = 32 * WT;                 // rows and columns of the wave tile
     constexpr int RB = RW * 2;                  // bytes of a staged row
     constexpr int SWZ = WT == 4 ? 15 : 7;       // rows that differ in these bits (WT = 2: of r / 2) take different granule pairs
@@ -624,6 +624,40 @@ __device__ __forceinline__ void NormEpilogueRows(const GemmP &p, TAcc (&acc)[WT]
     const int mLive = p.mLive > 0 ? p.mLive : p.m;
     const int tile = (colBase + wn * RW) / TILE;
     const int firstRow = rowBase + wm * RW;
+    float tileSum2[WT];
+    if constexpr (NORM && WT == 2) {
+        if (p.normalize) { // (uniform over the workgroup)
+            const int wave = wm * 2 + wn;
+#pragma unroll
+            for (int i = 0; i < WT; ++i) {
+                const bool live = firstRow + i * 32 + l32 < mLive;
+                float rs = scale;
+                if (p.rowScale) {
+                    rs *= p.rowScale[firstRow + i * 32 + l32];
+                }
+                float own = 0;
+#pragma unroll
+                for (int j = 0; j < WT; ++j) {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const float x = live ? (float)acc[i][j][e] * rs : 0.f;
+                        own += x * x;
+                    }
+                }
+                float a, b;
+                LaneSwap32(own, &a, &b);
+                tileSum2[i] = a + b;
+                if (half == 0) {
+                    xchg[wave * 64 + i * 32 + l32] = tileSum2[i];
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < WT; ++i) {
+                tileSum2[i] += xchg[(wave ^ 1) * 64 + i * 32 + l32];
+            }
+        }
+    }
 #pragma unroll
     for (int i = 0; i < WT; ++i) {
         const int r = i * 32 + l32; // row inside the wave tile
@@ -644,9 +678,13 @@ __device__ __forceinline__ void NormEpilogueRows(const GemmP &p, TAcc (&acc)[WT]
             }
         }
         if (NORM && p.normalize) {
-            float a, b;
-            LaneSwap32(sum2, &a, &b);
-            sum2 = a + b;
+            if constexpr (WT == 2) {
+                sum2 = tileSum2[i];
+            } else {
+                float a, b;
+                LaneSwap32(sum2, &a, &b);
+                sum2 = a + b;
+            }
             float discr = 0;
             if (sum2 > 0) {
                 discr = __builtin_amdgcn_sqrtf(sum2 * (1.f / TILE)) * p.vecScale;
@@ -659,7 +697,7 @@ __device__ __forceinline__ void NormEpilogueRows(const GemmP &p, TAcc (&acc)[WT]
                     }
                 }
             }
-            if (half == 0) {
+            if (half == 0 && (WT == 4 || wn == 0)) {
                 p.tileScale[(int64_t)tile * p.ldTileScale + row] = discr;
             }
         }
@@ -669,7 +707,7 @@ __device__ __forceinline__ void NormEpilogueRows(const GemmP &p, TAcc (&acc)[WT]
             for (int j = 0; j < WT; ++j) {
 #pragma unroll
                 for (int e = 0; e < 16; e += 2) {
-                    const float2 cs = *(const float2 *)(ropeRow + j * 32 + (e >> 2) * 8 + half * 4 + (e & 3));
+                    const float2 cs = *(const float2 *)(ropeRow + (WT == 2 ? wn * RW : 0) + j * 32 + (e >> 2) * 8 + half * 4 + (e & 3));
                     const float x = v[j][e], y = v[j][e + 1];
                     v[j][e] = x * cs.x - y * cs.y;
                     v[j][e + 1] = y * cs.x + x * cs.y;
@@ -965,7 +1003,8 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN) / 4) GemmNTDirect(Gemm
     constexpr int BM = 32 * WTM * WM;
     constexpr int BN = 32 * WTN * WN;
     // plain 16-bit results of the 128x128 e4m3 tile leave through the row-owning epilogue (a lane owns a row: operands swapped)
-    constexpr bool SWAPC = TYPE == T_FP8 && WTM == 2 && WTN == 2 && WM == 2 && WN == 2 && !KT && (CT == C_BF16 || CT == C_F16) && EPI == TS2_EPI_STORE;
+    constexpr bool SWAPC = TYPE == T_FP8 && WTM == 2 && WTN == 2 && WM == 2 && WN == 2 && !KT &&
+                           (CT == C_BF16NORM || ((CT == C_BF16 || CT == C_F16) && EPI == TS2_EPI_STORE));
     __shared__ __attribute__((aligned(1024))) uint8_t sA0[BM * BKB];
     __shared__ __attribute__((aligned(1024))) uint8_t sB0[BN * BKB];
     __shared__ __attribute__((aligned(1024))) uint8_t sA1[BM * BKB];
@@ -1205,7 +1244,7 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN) / 4) GemmNTDirect(Gemm
     __syncthreads();
     if constexpr (SWAPC) {
         uint8_t *waveLds = wave == 0 ? sA0 : wave == 1 ? sB0 : wave == 2 ? sA1 : sB1;
-        NormEpilogueRows<TYPE, false, CT == C_F16, 2>(p, acc, waveLds, rowBase, colBase, wm, wn, lane);
+        NormEpilogueRows<TYPE, CT == C_BF16NORM, CT == C_F16, 2>(p, acc, waveLds, (float *)(sA0 + 8192), rowBase, colBase, wm, wn, lane);
     } else {
         Epilogue<TYPE, WTM, WTN, CT, EPI, KT>(p, acc, facc, sA0, rowBase, colBase, wm, wn, half, l32);
     }
@@ -1229,7 +1268,7 @@ template <int TYPE, int CT, int EPI, bool TN = false, int WT = 4> __global__ voi
     static_assert(WT == 4 || (WT == 2 && TYPE == T_FP8 && !TN), "the 128x128 ring takes e4m3 operands with the contraction along the rows");
     static_assert(!TN || TYPE != T_I8, "contraction-major operands: e4m3 and bf16");
     // the normalising epilogue of the large tile works on transposed blocks: the MFMAs take their operands the other way round
-    constexpr bool SWAPC = ((CT == C_BF16NORM && WT == 4) || ((CT == C_BF16 || CT == C_F16) && EPI == TS2_EPI_STORE)) && !TN;
+    constexpr bool SWAPC = (CT == C_BF16NORM || ((CT == C_BF16 || CT == C_F16) && EPI == TS2_EPI_STORE)) && !TN;
     constexpr int ESZ = TYPE == T_BF16 ? 2 : 1;
     constexpr int KR = BKB / ESZ; // contraction rows of a step (K-major operands)
     __shared__ __attribute__((aligned(1024))) uint8_t sA0[BM * BKB];
@@ -1566,7 +1605,7 @@ template <int TYPE, int CT, int EPI, bool TN = false, int WT = 4> __global__ voi
     if constexpr (SWAPC) {
         // every wave stages its rows in a stage array of its own
         uint8_t *waveLds = wave == 0 ? sA0 : wave == 1 ? sA1 : wave == 2 ? sA2 : sB0;
-        NormEpilogueRows<TYPE, CT == C_BF16NORM, CT == C_F16, WT>(p, acc, waveLds, rowBase, colBase, wm, wn, lane);
+        NormEpilogueRows<TYPE, CT == C_BF16NORM, CT == C_F16, WT>(p, acc, waveLds, (float *)sB1, rowBase, colBase, wm, wn, lane);
     } else {
         Epilogue<TYPE, WTM, WTN, CT, EPI, false>(p, acc, facc, sA0, rowBase, colBase, wm, wn, half, l32);
     }
