@@ -751,6 +751,96 @@ __device__ __forceinline__ void NormEpilogueRows(const GemmP &p, TAcc (&acc)[WT]
     }
 }
 
+// The packed-delta epilogue (TStoreRowTileMaxNormalize, src/lib/cuda/cuda_matmul.cuh:530-559) of the 256x256 ring kernel in the same
+// row-owning form: the largest magnitude of a row's 128-column tile is 64 in-lane terms and one swap with the other half wave, four
+// consecutive columns are one 32-bit word of bytes, the 128-byte rows are staged in the wave's own LDS (words XOR-swizzled in groups
+// of four by the row) and leave as 16-byte stores, eight lanes per row; a tile's scales are 32 consecutive floats per store.  Same
+// arithmetic, element for element, as the lane = column form (maximum of |acc| times |scale|, /127, reciprocal, (acc * scale) * mult).
+template <class TAcc>
+__device__ __forceinline__ void PackEpilogueRows(const GemmP &p, TAcc (&acc)[4][4], uint8_t *waveLds, int rowBase, int colBase, int wm, int wn, int lane)
+{
+    const int half = lane >> 5, l32 = lane & 31;
+    float scale = p.alpha;
+    if (p.alphaPtr) {
+        scale *= *p.alphaPtr;
+    }
+    const int mLive = p.mLive > 0 ? p.mLive : p.m;
+    const int tile = (colBase + wn * 128) / TILE;
+    const int firstRow = rowBase + wm * 128;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = i * 32 + l32; // row inside the wave tile
+        const int row = firstRow + r;
+        float rs = scale;
+        if (p.rowScale) {
+            rs *= p.rowScale[row];
+        }
+        float mx = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                mx = fmaxf(mx, fabsf((float)acc[i][j][e]));
+            }
+        }
+        float a, b;
+        LaneSwap32(mx, &a, &b);
+        mx = fmaxf(a, b) * fabsf(rs);
+        float discr = 0, mult = 0;
+        if (mx > 0 && row < mLive) {
+            discr = mx / 127;
+            mult = 1 / discr;
+        }
+        if (half == 0) {
+            p.tileScale[(int64_t)tile * p.ldTileScale + row] = discr;
+        }
+        const int swz = ((r >> 1) & 7) << 2;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                uint32_t w = 0;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    w |= (uint32_t)(CvtToI8((float)acc[i][j][4 * q + c] * rs * mult) & 0xff) << (8 * c);
+                }
+                *(uint32_t *)(waveLds + r * 128 + (((j * 8 + q * 2 + half) ^ swz) << 2)) = w;
+            }
+        }
+    }
+    typedef unsigned v4u_t __attribute__((ext_vector_type(4)));
+    const int t = lane & 7, rsub = lane >> 3;
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(p.c + (int64_t)firstRow * p.ldc), 0, (int)(128 * p.ldc), 0x00020000);
+    const int ldc = (int)p.ldc;
+    const int laneOff = rsub * ldc + colBase + wn * 128 + t * 16;
+    const int alignBits = (int)(((uintptr_t)p.c | (uintptr_t)p.ldc) & 15);
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+        const int r = it * 8 + rsub;
+        const uint4 d = *(const uint4 *)(waveLds + r * 128 + (((4 * t) ^ (((r >> 1) & 7) << 2)) << 2));
+        if (alignBits == 0) {
+            if (p.streamC) {
+                __builtin_amdgcn_raw_buffer_store_b128((v4u_t){d.x, d.y, d.z, d.w}, rsrc, laneOff, it * 8 * ldc, 2);
+            } else {
+                __builtin_amdgcn_raw_buffer_store_b128((v4u_t){d.x, d.y, d.z, d.w}, rsrc, laneOff, it * 8 * ldc, 0);
+            }
+        } else if ((alignBits & 3) == 0) {
+            __builtin_amdgcn_raw_buffer_store_b32(d.x, rsrc, laneOff, it * 8 * ldc, 0);
+            __builtin_amdgcn_raw_buffer_store_b32(d.y, rsrc, laneOff, it * 8 * ldc + 4, 0);
+            __builtin_amdgcn_raw_buffer_store_b32(d.z, rsrc, laneOff, it * 8 * ldc + 8, 0);
+            __builtin_amdgcn_raw_buffer_store_b32(d.w, rsrc, laneOff, it * 8 * ldc + 12, 0);
+        } else {
+            // (rows that start off the 4-byte grid: byte stores)
+            const uint32_t w[4] = {d.x, d.y, d.z, d.w};
+            uint8_t *dst = p.c + (int64_t)(firstRow + r) * p.ldc + colBase + wn * 128 + t * 16;
+#pragma unroll
+            for (int c = 0; c < 16; ++c) {
+                dst[c] = (uint8_t)(w[c >> 2] >> (8 * (c & 3)));
+            }
+        }
+    }
+}
+
 template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT>
 __global__ void __launch_bounds__(256, 1) GemmNT(GemmP p)
 {
@@ -1267,8 +1357,8 @@ template <int TYPE, int CT, int EPI, bool TN = false, int WT = 4> __global__ voi
     constexpr int WTM = WT, WTN = WT, WN = 2, NW = 4, BM = 64 * WT, BN = 64 * WT;
     static_assert(WT == 4 || (WT == 2 && TYPE == T_FP8 && !TN), "the 128x128 ring takes e4m3 operands with the contraction along the rows");
     static_assert(!TN || TYPE != T_I8, "contraction-major operands: e4m3 and bf16");
-    // the normalising epilogue of the large tile works on transposed blocks: the MFMAs take their operands the other way round
-    constexpr bool SWAPC = (CT == C_BF16NORM || ((CT == C_BF16 || CT == C_F16) && EPI == TS2_EPI_STORE)) && !TN;
+    // the 16-bit and the packed-delta epilogues work on transposed blocks (a lane owns a row): the MFMAs take their operands the other way round
+    constexpr bool SWAPC = ((CT == C_BF16NORM || ((CT == C_BF16 || CT == C_F16) && EPI == TS2_EPI_STORE)) && !TN) || (CT == C_I8PACK && WT == 4);
     constexpr int ESZ = TYPE == T_BF16 ? 2 : 1;
     constexpr int KR = BKB / ESZ; // contraction rows of a step (K-major operands)
     __shared__ __attribute__((aligned(1024))) uint8_t sA0[BM * BKB];
@@ -1605,7 +1695,11 @@ template <int TYPE, int CT, int EPI, bool TN = false, int WT = 4> __global__ voi
     if constexpr (SWAPC) {
         // every wave stages its rows in a stage array of its own
         uint8_t *waveLds = wave == 0 ? sA0 : wave == 1 ? sA1 : wave == 2 ? sA2 : sB0;
-        NormEpilogueRows<TYPE, CT == C_BF16NORM, CT == C_F16, WT>(p, acc, waveLds, (float *)sB1, rowBase, colBase, wm, wn, lane);
+        if constexpr (CT == C_I8PACK) {
+            PackEpilogueRows(p, acc, waveLds, rowBase, colBase, wm, wn, lane);
+        } else {
+            NormEpilogueRows<TYPE, CT == C_BF16NORM, CT == C_F16, WT>(p, acc, waveLds, (float *)sB1, rowBase, colBase, wm, wn, lane);
+        }
     } else {
         Epilogue<TYPE, WTM, WTN, CT, EPI, false>(p, acc, facc, sA0, rowBase, colBase, wm, wn, half, l32);
     }
