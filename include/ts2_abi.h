@@ -68,6 +68,8 @@ enum ts2_epilogue {
  * abType: TS2_I8 (int32 accumulate, exact), TS2_E4M3 or TS2_BF16 (fp32 accumulate).
  * cType : TS2_F32, TS2_BF16, TS2_F16 (TS2_EPI_STORE only), TS2_I32 (raw accumulator, TS2_I8 inputs and TS2_EPI_STORE only) or TS2_I8
  *         (ROW_TILE_MAXNORM).
+ *         16-bit and TS2_I8 results: 128 rows of C within 2 GiB (row stride below 16 MiB), else TS2_ERR_UNSUPPORTED; 16-bit rows
+ *         4-byte aligned.
  * rowScale  (optional, [m], 16-byte aligned): per-row scale of A applied to the accumulator before the epilogue (the dX kernel).
  * kTileScale (optional, [k/kTile], TS2_I8 only): one scale per kTile contraction rows; each tile's int32 sum is exact and
  *             tiles are added in fp32 in tile order (the dW kernel).  kTile must be a multiple of 128.

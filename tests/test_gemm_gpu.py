@@ -155,6 +155,50 @@ def test_packed_delta_epilogue(lib, orc):
         assert diff.max() <= 1 and (diff != 0).mean() < 1e-3
 
 
+@pytest.mark.parametrize("k_major", [False, True])
+def test_packed_delta_epilogue_equals_the_packed_fp32_product(lib, k_major):
+    """e4m3 operands on the 256x256 tile: the fused ROW_TILE_MAXNORM epilogue against the same product stored in fp32 and packed by
+    ts2_pack_delta (the same arithmetic on the same fp32 sums: bit-identical bytes and scales), with a scale behind a pointer; live
+    rows short of m (bytes and scales of the rest are zero); and results whose rows start off the 16-byte and off the 4-byte grid
+    (the epilogue stores 16 bytes per lane where it can), nothing written past a row's end."""
+    print("case packed delta against pack_delta", k_major, flush=True)
+    import ctypes as C
+    from tscale2_amd import lib as L
+    m, n, k = 512, 768, 640
+    g = torch.Generator(device="cuda").manual_seed(77)
+
+    def codes(shape):
+        return (torch.randint(0, 120, shape, device="cuda", generator=g) | (torch.randint(0, 2, shape, device="cuda", generator=g) << 7)).to(torch.uint8)
+    a, b = (codes((k, m)), codes((k, n))) if k_major else (codes((m, k)), codes((n, k)))
+    if k_major:
+        a[:, 7] = 0
+    else:
+        a[7] = 0                                                    # a zero row: zero tiles, zero scales
+    kw = dict(m=m, n=n, k=k, k_major=True) if k_major else {}
+    sc = torch.tensor([1.7], device="cuda")
+    raw = torch.zeros((m, n), device="cuda")
+    lib.gemm_nt(a, b, raw, L.E4M3, L.F32, tile_config=1, **kw)
+    want = torch.zeros((m, n), dtype=torch.int8, device="cuda"); want_ts = torch.zeros((n // 128, m), device="cuda")
+    L.call("ts2_pack_delta", raw, 1, C.c_int64(0), m, n, 0.03, sc, want, want_ts)
+    got = torch.full((m, n), 3, dtype=torch.int8, device="cuda"); got_ts = torch.full((n // 128, m), -1.0, device="cuda")
+    lib.gemm_nt(a, b, got, L.E4M3, L.I8, alpha=0.03, alpha_ptr=sc, epilogue=L.EPI_ROW_TILE_MAXNORM, tile_scale=got_ts, tile_config=1, **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want) and torch.equal(got_ts, want_ts)
+    assert int(got.abs().max()) == 127 and bool((got[7] == 0).all()) and bool((got_ts[:, 7] == 0).all())
+    for pad in (4, 1):                                              # row stride n + pad bytes
+        wide = torch.full((m, n + pad), 5, dtype=torch.int8, device="cuda")
+        ts2 = torch.full((n // 128, m), -1.0, device="cuda")
+        lib.gemm_nt(a, b, wide[:, :n], L.E4M3, L.I8, alpha=0.03, alpha_ptr=sc, epilogue=L.EPI_ROW_TILE_MAXNORM, tile_scale=ts2, tile_config=1, **kw)
+        torch.cuda.synchronize()
+        assert torch.equal(wide[:, :n], want) and torch.equal(ts2, want_ts) and bool((wide[:, n:] == 5).all())
+    if not k_major:
+        live = 300
+        lib.gemm_nt(a, b, got, L.E4M3, L.I8, alpha=0.03, alpha_ptr=sc, epilogue=L.EPI_ROW_TILE_MAXNORM, tile_scale=got_ts, tile_config=1, m_live=live)
+        torch.cuda.synchronize()
+        assert torch.equal(got[:live], want[:live]) and torch.equal(got_ts[:, :live], want_ts[:, :live])
+        assert bool((got[live:] == 0).all()) and bool((got_ts[:, live:] == 0).all())
+
+
 def test_split_k_matches(lib, orc):
     print("case split-k", flush=True)
     from tscale2_amd import lib as L

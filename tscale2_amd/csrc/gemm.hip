@@ -2158,7 +2158,7 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
     if ((a->cType == TS2_BF16 || a->cType == TS2_F16) && (a->c.strideBytes & 3)) {
         return TS2_ERR_ALIGN; // bf16 results are stored two columns at a time
     }
-    if ((a->cType == TS2_BF16 || a->cType == TS2_F16) && (int64_t)128 * a->c.strideBytes >= ((int64_t)1 << 31)) {
+    if ((a->cType == TS2_BF16 || a->cType == TS2_F16 || a->cType == TS2_I8) && (int64_t)128 * a->c.strideBytes >= ((int64_t)1 << 31)) {
         return TS2_ERR_UNSUPPORTED; // the row stores address 128 rows of C from one 32-bit offset
     }
     int splitK = a->splitK > 1 ? a->splitK : 1;
