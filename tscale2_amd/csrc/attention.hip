@@ -526,10 +526,14 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
                 s[e] = 0;
                 dp[e] = 0;
             }
-            // phase 1: S^T = K Q^T and dP^T = V dO^T; the operands of step ds + 1 are requested before the products of step ds
+            // phase 1: S^T = K Q^T and dP^T = V dO^T; the operands of step ds + 1 are requested before the products of step ds.
+            // The wave raises its issue priority for its two MFMA phases: the SIMD's other wave then fills the gaps between this one's
+            // products with its arithmetic instead of delaying them (3 % on this kernel; the same in the forward and the dK/dV
+            // kernels measured nothing and a loss, and is not used there).
             v8bf fk[2], fv[2];
             fk[0] = FragRow(kt2, 0, 0, fl);
             fv[0] = FragRow(vt2, 0, 0, fl);
+            __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int ds = 0; ds < 8; ++ds) {
                 if (ds + 1 < 8) {
@@ -551,6 +555,7 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
             }
             __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+            __builtin_amdgcn_s_setprio(0);
             // phase 2: dS = w (dP - dScale) attDotScale ln2, w = 2^(logit - L): three instructions and the exponential per element
             // (without a slope the position term drops out of the logit)
             const float kc = ALIBI ? p.slope * (float)(k0 + half * 4 - myRow) - L : -L;
@@ -574,6 +579,7 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
                 }
             }
             const v8bf sb[2] = {PackB(dsv, 0), PackB(dsv, 1)};
+            __builtin_amdgcn_s_setprio(1);
             // phase 3: dQ^T += K^T dS^T, operands two products ahead
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
@@ -588,6 +594,7 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             }
             __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            __builtin_amdgcn_s_setprio(0);
             }
         }
     };
