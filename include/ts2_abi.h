@@ -96,7 +96,12 @@ typedef struct ts2_gemm_args {
      * store/accumulate results; with tile 3: the form BackpropDelta launches); bit 4 (16) two LDS stages instead of the ring on the
      * 256x256 tile (and on the 128x128 tile with TS2_E4M3 operands, which takes the ring from k = 1024 on); bits 5-6 tile-order
      * group 8 / 4 / 2 instead of the automatic choice; bit 7 (128) the ring on the 128x128 tile at any k; bits 9 / 10 (512 / 1024)
-     * plain / non-temporal stores of C instead of the choice by k. */
+     * plain / non-temporal stores of C instead of the choice by k; bit 11 (2048) the 256x128 kernel with 64-byte steps for two
+     * workgroups per CU (k a multiple of 64 bytes); bit 12 (4096) the persistent eight-wave kernel whose epilogue runs under the next
+     * tile's main loop (m % 256 = 0, k >= 1024 bytes; fp32 / 16-bit / raw int32 results, store or accumulate), bits 13-14 its
+     * workgroup count as CUs >> 2, 4, 6 (tests).  Bits 11 and 12 return TS2_ERR_UNSUPPORTED for calls their kernel cannot run.  With
+     * bits 0-4 clear the persistent kernel is also chosen automatically for stored results with 1024 <= k bytes < 4096 and at least
+     * 512 tiles of 256x128; bit 15 (32768) switches that off. */
     int32_t tileConfig;
     /* Expert-grouped products (TMoeMatMulKernelCall / TMoeDeltaMatMulKernelCall, src/gpt/compute/moe_matmul.cuh:47-215):
      * tileGroup [m/128] (device): rows of A and C are grouped by expert in 128-row tiles; tile i multiplies the B slab
