@@ -613,27 +613,46 @@ def bench_moe_fp8(args):
 
 
 def bench_gemm_fp8(args):
-    """the dominant kernel of the dense fp8 step alone (e4m3 32768 x 2048 x 8192, fp32 result) followed by the copy probe of 1 GiB: the
-    command the HBM-traffic counters (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) are collected on; the probe calibrates the counters"""
+    """one e4m3 product alone - by default the dominant kernel of the dense fp8 step (32768 x 2048 x 8192, fp32 result) - followed by the
+    copy probe of 1 GiB: the command the hardware counters (rocprofv3 --pmc) are collected on; the probe calibrates FETCH_SIZE / WRITE_SIZE.
+    --shape m,n,k, --result f32|bf16|norm and --tile-config (ts2_gemm_args.tileConfig: 32768 = never the persistent kernel, 4096 = always)
+    select other products of the step; the shader clock is sampled while the launches run."""
     import torch
     from tscale2_amd import lib as L
     lib = L.load()
-    n, dim, ffn = 32768, 2048, 8192
+    n, dim, ffn = [int(x) for x in args.shape.split(",")] if args.shape else (32768, 2048, 8192)
     a = torch.randint(0, 120, (n, ffn), dtype=torch.uint8, device="cuda"); b = torch.randint(0, 120, (dim, ffn), dtype=torch.uint8, device="cuda")
-    c = torch.empty((n, dim), dtype=torch.float32, device="cuda")
-    fn = lambda: lib.gemm_nt(a, b, c, L.E4M3, L.F32)  # noqa: E731
+    kw = {"tile_config": args.tile_config}
+    if args.result == "f32":
+        c = torch.empty((n, dim), dtype=torch.float32, device="cuda")
+        ct = L.F32
+    else:
+        c = torch.empty((n, dim), dtype=torch.int16, device="cuda")
+        ct = L.BF16
+        if args.result == "norm":
+            kw.update(epilogue=L.EPI_ROW_TILE_NORM, normalize=True, vec_scale=1 / 24.0, tile_scale=torch.empty((dim // 128, n), device="cuda"))
+    fn = lambda: lib.gemm_nt(a, b, c, L.E4M3, ct, **kw)  # noqa: E731
     for _ in range(args.warmup):
         fn()
     torch.cuda.synchronize()
     ms = event_time_ms(fn, args.steps)
     gops = 2.0 * n * dim * ffn
+    reps = max(20, int(40.0 / ms))
+
+    def many():
+        for _ in range(reps):
+            fn()
+    clock = L.probe_shader_clock(many, seconds=reps * ms * 1.3e-3)
     copy = L.probe_copy_rate(1 << 30)
+    default = not args.shape and args.result == "f32"
     roof = {"bound": "mfma", "achieved": gops / (ms * 1e-3) / 1e12, "peak": PEAK_FP8 / 1e12, "unit": "TFLOP/s", "frac": gops / (ms * 1e-3) / PEAK_FP8,
-            "traffic": profile_traffic("gemm_fp8_32768x2048x8192_hbm_traffic.txt"), "traffic_algorithmic": n * ffn + dim * ffn + n * dim * 4,
-            "kernel": "GemmNTRing<e4m3> %dx%dx%d" % (n, dim, ffn)}
+            "traffic": profile_traffic("gemm_fp8_32768x2048x8192_hbm_traffic.txt") if default else None,
+            "traffic_algorithmic": n * ffn + dim * ffn + n * dim * (4 if ct == L.F32 else 2),
+            "kernel": "e4m3 GEMM %dx%dx%d, %s result, tileConfig %d" % (n, dim, ffn, args.result, args.tile_config),
+            "shader_clock_mhz_median_min_max": clock}
     return {"metric": "e4m3 GEMM launches/sec on 1 MI355X; TFLOPS as % of MFMA peak", "value": 1e3 / ms, "unit": "launches/s", "n_gpus": 1,
             "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-            "dtype": "fp8_e4m3", "data": "synthetic", "config": {"workload": "e4m3 GEMM 32768 x 2048 x 8192 (dX of the FFN expand matrix), fp32 result"},
+            "dtype": "fp8_e4m3", "data": "synthetic", "config": {"workload": "e4m3 GEMM %d x %d x %d, %s result" % (n, dim, ffn, args.result)},
             "copy_probe_gbps": copy, "roofline": roof}
 
 
@@ -652,6 +671,9 @@ def main():
     ap.add_argument("--sort-rows", action="store_true", help="linear_i8_bwd: sort the gradient rows by scale before the delta product (the reference's order)")
     ap.add_argument("--no-extras", action="store_true", help="step_fp8: only the step and its dominant GEMM (no int8 GEMMs, bandwidth kernels, device "
                                                               "probes or CPU leg): the command a kernel trace of the step is taken on")
+    ap.add_argument("--shape", default="", help="gemm_fp8: m,n,k of the product (default 32768,2048,8192)")
+    ap.add_argument("--result", default="f32", choices=["f32", "bf16", "norm"], help="gemm_fp8: fp32 store, bf16 store, or row-tile normalised bf16")
+    ap.add_argument("--tile-config", type=int, default=0, help="gemm_fp8: ts2_gemm_args.tileConfig")
     ap.add_argument("--small", action="store_true", help="step_fp8 / moe_fp8: a reduced model for quick checks (not a valid benchmark figure)")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -165,3 +165,34 @@ extern "C" int ts2_probe_copy_rate(const void *src, void *dst, int64_t bytes, do
     *gbPerSecOut = 2.0 * bytes / (ms * 1e-3) / 1e9; // read + write
     return TS2_OK;
 }
+
+// One wave that samples the shader clock while other kernels run: every `periodTicks` ticks of the constant 100 MHz counter
+// (s_memrealtime) it records how far the core-clock counter (s_memtime) advanced.  Bounded: `samples` periods, then it exits.
+__global__ void ClockMonitor(uint64_t *out, int samples, int periodTicks)
+{
+    if (threadIdx.x != 0) {
+        return;
+    }
+    for (int i = 0; i < samples; ++i) {
+        const uint64_t r0 = __builtin_amdgcn_s_memrealtime();
+        const uint64_t c0 = __builtin_amdgcn_s_memtime();
+        uint64_t r1 = r0;
+        while (r1 - r0 < (uint64_t)periodTicks) {
+            __builtin_amdgcn_s_sleep(8);
+            r1 = __builtin_amdgcn_s_memrealtime();
+        }
+        const uint64_t c1 = __builtin_amdgcn_s_memtime();
+        out[2 * i] = r1 - r0;
+        out[2 * i + 1] = c1 - c0;
+    }
+}
+
+extern "C" int ts2_probe_clock_monitor(uint64_t *out, int32_t samples, int32_t periodTicks, void *streamV)
+{
+    if (!out || samples <= 0 || samples > (1 << 20) || periodTicks <= 0 || periodTicks > 100000000) {
+        return TS2_ERR_SHAPE;
+    }
+    hipLaunchKernelGGL(ClockMonitor, dim3(1), dim3(64), 0, (hipStream_t)streamV, out, samples, periodTicks);
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}

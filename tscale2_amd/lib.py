@@ -171,6 +171,31 @@ def probe_copy_rate(nbytes=1 << 30):
     return out.value
 
 
+def probe_shader_clock(run, seconds=0.25, period_us=100):
+    """MHz of the shader clock while run() keeps the GPU busy on the current stream: a one-wave monitor kernel on a second stream samples
+    the core-clock counter against the 100 MHz counter every period_us; returns (median, min, max) over the samples of the busy time."""
+    import torch
+    lib = load()
+    n = int(seconds * 1e6 / period_us)
+    out = torch.zeros(2 * n, dtype=torch.int64, device="cuda")
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        lib.check(_probe_lib().ts2_probe_clock_monitor(ptr(out), C.c_int32(n), C.c_int32(period_us * 100),
+                                                       C.c_void_p(side.cuda_stream)), "ts2_probe_clock_monitor")
+    e0 = torch.cuda.Event(enable_timing=True); e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    run()
+    e1.record()
+    torch.cuda.synchronize()
+    busy_ms = e0.elapsed_time(e1)
+    v = out.view(n, 2).double().cpu()
+    mhz = (v[:, 1] / v[:, 0] * 100.0)
+    k = max(1, min(n, int(busy_ms * 1e3 / period_us)))      # samples taken while run() was executing
+    body = mhz[k // 10: max(k // 10 + 1, k - k // 10)]       # (without the ramp at either end)
+    return float(body.median()), float(body.min()), float(body.max())
+
+
 class BwdBuffers(C.Structure):
     _fields_ = [("grad8", Mat), ("grad8RowScale", C.c_void_p), ("gradT", Mat), ("srcT", Mat), ("tileMax", C.c_void_p), ("tileScale", C.c_void_p),
                 ("transformT", Mat), ("partial", Mat), ("splits", C.c_int32), ("gradRowAbsMax", C.c_void_p),
