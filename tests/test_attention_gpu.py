@@ -113,6 +113,14 @@ def test_attention_remapped_block_order(L, orc):
     run_case(L, orc, frag_count=4, frag_len=256, window=200, heads=2, slope=0.25, seed=24, grad_type=L.BF16)
 
 
+@pytest.mark.parametrize("slope", [0.0, 0.01])
+def test_attention_one_sequence_of_2048_tokens(L, orc, slope):
+    """the sequence length of config[3] (and twice config[2]'s): full causal spans over sixteen 128-row blocks, statistics accumulated
+    over up to 2047 keys, the reverse ranges of the last blocks reaching back over the whole sequence, the position term at distance 2000"""
+    print("case att 2048 tokens, slope", slope, flush=True)
+    run_case(L, orc, frag_count=1, frag_len=2048, window=4096, heads=2, slope=slope, seed=25, grad_type=L.BF16)
+
+
 def test_rope_and_head_norm_passes(L, orc):
     print("case rope/norm passes", flush=True)
     r = np.random.default_rng(24)

@@ -150,3 +150,71 @@ def test_attention_at_full_size_treats_the_sequences_of_a_batch_independently(L)
     assert torch.equal(dv2.float(), dv.float() * 2)
     assert torch.equal(dk2.float(), dk.float() * 2)
     assert torch.equal(dq2.float(), dq.float() * 2)
+
+
+def test_moe_routing_gather_grouped_product_and_combine_at_the_size_of_the_moe_benchmark(L):
+    """config[4]: 65536 tokens routed to 2 of 64 experts (139264 grouped rows with every expert's rows padded to 128), width 1024, expert
+    width 512.  Routing tables by their invariants, ts2_moe_group_samples against a torch gather (bit-exact), the expert-grouped e4m3
+    product 139264 x 512 x 1024 through per-expert row and column checksums in float64, ts2_combine_experts against a torch gather-sum
+    (bit-exact).  Reference: src/gpt/compute/layer_moe.cu:203-272 (forward), moe_matmul.cuh:47-215 (grouped products)."""
+    import ctypes as C
+    from test_moe_gpu import route
+    print("case moe full size", flush=True)
+    lib = L.load()
+    len_, E, K, dim, xp = 65536, 64, 2, 1024, 512
+    _, t, tb, len_moe, host = route(L, len_, E, K, 61)
+    assert len_moe == 139264
+    sid, eo, tile = t["sid"].long(), host["eo"], host["tile"]
+    # every token is listed `selected` times, an expert's rows are a multiple of 128, a tile's expert is the owner of its rows
+    live = sid >= 0
+    assert int(live.sum()) == len_ * K
+    assert torch.equal(torch.bincount(sid[live], minlength=len_), torch.full((len_,), K, device="cuda"))
+    assert eo[0] == 0 and np.all(np.diff(eo[:E + 1]) % 128 == 0) and np.all(np.diff(eo[:E + 1]) >= 0)
+    owner = np.searchsorted(eo[1:E + 1], np.arange(len_moe // 128) * 128, side="right")
+    used = np.arange(len_moe // 128) * 128 < eo[E]
+    assert np.array_equal(tile[used], owner[used]) and np.all(tile[~used] == -1)
+    rows_e = torch.from_numpy(np.repeat(np.where(used, owner, E), 128)).cuda()          # expert of every grouped row (E = unused tail)
+    # pad rows (sid -1) lie at the end of each expert's range
+    for e in (0, 17, E - 1):
+        s = sid[eo[e]:eo[e + 1]]
+        nlive = int((s >= 0).sum())
+        assert bool((s[:nlive] >= 0).all()) and bool((s[nlive:] < 0).all())
+    # ---- gather
+    g = torch.Generator(device="cuda").manual_seed(62)
+    x8 = (torch.randn((len_, dim), device="cuda", generator=g) * 2).to(torch.float8_e4m3fn).view(torch.uint8)
+    grouped = torch.full((len_moe, dim), 77, dtype=torch.uint8, device="cuda")
+    L.call("ts2_moe_group_samples", len_moe, 1, x8, t["sid"], grouped)
+    want = torch.where(live[:, None], x8[sid.clamp(min=0)], torch.zeros((), dtype=torch.uint8, device="cuda"))
+    assert torch.equal(grouped, want)
+    # ---- grouped product: every 128-row tile multiplies its expert's [xp x dim] slab
+    w8 = (torch.randn((E * xp, dim), device="cuda", generator=g) * 2).to(torch.float8_e4m3fn).view(torch.uint8)
+    c = torch.full((len_moe, xp), 5.0, dtype=torch.float32, device="cuda")
+    lib.gemm_nt(grouped, w8, c, L.E4M3, L.F32, n=xp, tile_group=t["tile"], b_slab_bytes=xp * dim)
+    torch.cuda.synchronize()
+    assert bool((c[eo[E]:] == 5.0).all())                                               # skipped tiles leave C alone
+    a64 = grouped.view(torch.float8_e4m3fn).double()
+    w64 = w8.view(torch.float8_e4m3fn).double().view(E, xp, dim)
+    c64 = c.double()
+    scale = c64[:eo[E]].abs().max().item()
+    # row sums: sum_j C[i][j] = A[i] . (sum_j W_e[j])
+    wsum = torch.cat([w64.sum(1), torch.zeros((1, dim), dtype=torch.float64, device="cuda")])     # [E + 1][dim]
+    row = (a64 * wsum[rows_e]).sum(1)
+    assert (c64[:eo[E]].sum(1) - row[:eo[E]]).abs().max().item() <= 1e-4 * scale * np.sqrt(xp)
+    # column sums per expert: sum_{i in e} C[i][j] = (sum_{i in e} A[i]) . W_e[j]
+    asum = torch.zeros((E + 1, dim), dtype=torch.float64, device="cuda").index_add_(0, rows_e, a64)
+    csum = torch.zeros((E + 1, xp), dtype=torch.float64, device="cuda").index_add_(0, rows_e[:eo[E]], c64[:eo[E]])
+    col = torch.einsum("ed,exd->ex", asum[:E], w64)
+    per_expert = np.diff(eo[:E + 1]).max()
+    assert (csum[:E] - col).abs().max().item() <= 1e-4 * scale * np.sqrt(per_expert)
+    # one row recomputed directly
+    i = int(eo[23]) + 5
+    assert (c64[i] - w64[23] @ a64[i]).abs().max().item() <= 2e-4 * scale
+    # ---- combine: res = alpha * (*alphaPtr) * sum over a token's slots, in slot order
+    src = torch.randn((len_moe, dim), device="cuda", generator=g)
+    ap = torch.tensor([1.5], device="cuda")
+    res = torch.zeros((len_, dim), device="cuda")
+    L.call("ts2_combine_experts", len_, K, src, L.F32, C.byref(tb), 0.37, ap, res, 0)
+    torch.cuda.synchronize()
+    rows = torch.from_numpy(host["row"]).cuda().long()
+    want = (src[rows[:, 0]] + src[rows[:, 1]]) * (np.float32(0.37) * np.float32(1.5))
+    assert torch.equal(res, want)

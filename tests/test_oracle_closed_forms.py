@@ -174,16 +174,25 @@ def _loss(h):
 
 
 def _fd_ratio(h, mat, delta, r, eps):
-    """(<delta, D> / n_targets) / d(mean log p)/d(eps) along a random direction D of one dequantised matrix"""
-    d = r.standard_normal(mat.deq.shape).astype(np.float32)
-    d *= np.float32(np.sqrt((mat.deq.astype(np.float64) ** 2).mean()))
+    """(<delta, D> / n_targets) / d(mean log p)/d(eps) along a direction D of one dequantised matrix.  D is half random, half the
+    delta itself (both at the matrix' rms): the random half checks the delta's direction, the other half keeps the derivative well away
+    from zero, so that the ratio is conditioned well enough for a tolerance of 5e-3.  The derivative is the Richardson extrapolation of
+    the central differences at eps and eps / 2 (error O(eps^4)); the oracle returns the loss as a double."""
+    rms = np.float32(np.sqrt((mat.deq.astype(np.float64) ** 2).mean()))
+    d = r.standard_normal(mat.deq.shape).astype(np.float32) * rms * np.float32(0.5)
+    drms = np.sqrt((delta.astype(np.float64) ** 2).mean())
+    if drms > 0:
+        d += (delta.astype(np.float64) * (0.5 * rms / drms)).astype(np.float32)
     keep = mat.deq.copy()
-    mat.deq[...] = keep + eps * d
-    lp = _loss(h)
-    mat.deq[...] = keep - eps * d
-    lm = _loss(h)
-    mat.deq[...] = keep
-    fd = (lp - lm) / (2 * eps)
+
+    def central(e):
+        mat.deq[...] = keep + np.float32(e) * d
+        lp = _loss(h)
+        mat.deq[...] = keep - np.float32(e) * d
+        lm = _loss(h)
+        mat.deq[...] = keep
+        return (lp - lm) / (2 * e)
+    fd = (4 * central(eps / 2) - central(eps)) / 3
     an = (delta.astype(np.float64) * d).sum() / (h.target >= 0).sum()
     return an / fd, fd
 
@@ -198,7 +207,7 @@ def _check_ratio(h, mat, delta, expect, eps, what):
     for e in steps:
         ratio, fd = _fd_ratio(h, mat, delta, np.random.default_rng(seed), e)
         got.append((e, ratio, fd))
-    good = [g for g in got if abs(g[2]) > 1e-5 and abs(g[1] / expect - 1) < 4e-2]
+    good = [g for g in got if abs(g[2]) > 1e-5 and abs(g[1] / expect - 1) < 5e-3]
     assert len(good) >= need, (what, expect, got)
 
 

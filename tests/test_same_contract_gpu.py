@@ -20,10 +20,11 @@ from same_contract import SameContract, rep  # noqa: E402
 TOL_MAX = 1e-2   # max |device - model| / max |model| per tensor
 TOL_RMS = 5e-3   # rms of the difference / rms of the tensor
 # e4m3 mode: the MFMA fp32 accumulation carries about 4e-5 relative noise (the int8 sums are exact), which flips about 1 % of the bf16
-# activations by an ulp and through them about 0.1 % of the e4m3 codes (steps of 6 %): isolated elements off by one code.  Which
-# elements flip depends on the last bit of every kernel's arithmetic: the largest isolated error seen over kernel revisions is
-# 2.1e-2 of the tensor's maximum (one element of an FFN delta), the rms and the scale fit do not move
+# activations by an ulp and through them about 0.1 % of the e4m3 codes (steps of 6 %): isolated elements that inherit one flipped code.
+# The contract stays 1e-2 of the tensor's maximum; what is allowed beyond it is counted: at most 0.2 % of a tensor's elements may exceed
+# it, none may exceed 3e-2 (one flipped code of a large element; two would), and the rms and the scale fit must not move.
 TOL_MAX_E4M3 = 3e-2
+TOL_OUTLIERS_E4M3 = 2e-3
 TOL_RMS_E4M3 = 8e-3
 
 
@@ -45,9 +46,11 @@ def check_layers(h, k_tile=0):
     def cmp(what, got, ref, tol_max=TOL_MAX, tol_rms=TOL_RMS):
         rms, mx = rel_err(got, ref)
         fit, _ = scale_fit(got, ref)
-        print(f"{what}: rms {rms:.2e} max {mx:.2e} fit {fit:.6f}", flush=True)
-        if not (mx <= tol_max and rms <= tol_rms and abs(fit - 1) <= 1e-3):
-            bad.append((what, rms, mx, fit))
+        # elements beyond the contract's 1e-2 of the maximum (only the e4m3 layers' tensors are allowed any)
+        over = float((np.abs(got.astype(np.float64) - ref) > TOL_MAX * (np.abs(ref).max() + 1e-30)).mean())
+        print(f"{what}: rms {rms:.2e} max {mx:.2e} beyond 1e-2: {over:.2e} fit {fit:.6f}", flush=True)
+        if not (mx <= tol_max and rms <= tol_rms and abs(fit - 1) <= 1e-3 and over <= (TOL_OUTLIERS_E4M3 if tol_max > TOL_MAX else 0)):
+            bad.append((what, rms, mx, over, fit))
     try:
         m.backprop()  # a real step: realistic state and state gradient to feed every layer with
         torch.cuda.synchronize()
@@ -133,3 +136,11 @@ def test_layers_same_contract_moe():
     print("case same contract per layer: MoE", flush=True)
     check_layers(Harness(E4M3, dim=256, heads=2, ffn_tiles=2, depth=3, vocab=256, frag_count=4, frag_len=96, wide_window=64, experts=8,
                          selected=2, xp=256, seed=16, std=0.05))
+
+
+def test_layers_same_contract_moe_64_experts_width_512():
+    """the expert count and expert width of the MoE benchmark (64 experts, top-2, width 512 = four norm tiles per expert slab, which
+    runs the second pass of the gate / norm backward's tile loop and 64-way routing tables), on 768 tokens: 8192 grouped rows"""
+    print("case same contract per layer: MoE, 64 experts x 512", flush=True)
+    check_layers(Harness(E4M3, dim=512, heads=4, ffn_tiles=4, depth=3, vocab=256, frag_count=4, frag_len=192, wide_window=64, experts=64,
+                         selected=2, xp=512, seed=17, std=0.05))
