@@ -338,21 +338,19 @@ def bench_step_fp8(args):
     bf16 activations.  One step = forward + loss gradient + backward through all layers with every delta (no optimiser)."""
     import numpy as np
     import torch
-    from model_harness import LT_ATT, layer_shapes, schedule
-    from oracle_lib import Oracle
     from tscale2_amd import lib as L
     L.load()
-    orc = Oracle()
+    LT_ATT = 0
     dim, heads, ffn, depth, vocab, frags, frag_len, wide = 2048, 16, 8192, 12, 50304, 32, 1024, 1024
     if args.small:
         dim, heads, ffn, depth, vocab, frags, frag_len, wide = 512, 4, 2048, 4, 1024, 8, 512, 512
-    lt, la, ls, aw = schedule(orc, depth, 0, wide)
+    lt, la, ls, aw = L.model_schedule(depth, 0, wide)      # the library's own schedule and RoPE table: no oracle in the timed path
     n = frags * frag_len
     m = L.Model(L.E4M3, dim, heads, ffn, lt, la, ls, len(aw), vocab, vocab + 1, n)
     gen = torch.Generator(device="cuda").manual_seed(2)
     params = 0
     for d in range(len(lt)):
-        for i, (rows, cols) in enumerate(layer_shapes(int(lt[d]), dim, heads, ffn, 0, 0)):
+        for i, (rows, cols) in enumerate(L.layer_shapes(int(lt[d]), dim, heads, ffn, 0, 0)):
             fast, sc = _fast_weights(torch, rows, cols, True, gen)
             m.set_matrix(d, i, fast, sc)
             params += rows * cols
@@ -370,7 +368,7 @@ def bench_step_fp8(args):
     finishes = [(t - 1).astype(np.int32) for _ in aw]
     for a in range(len(aw)):
         finishes[a][t == frag0] = -1
-    m.set_batch(np.arange(n + 1, dtype=np.int32), (1 + tokens).astype(np.uint32).ravel(), tg.ravel(), starts, finishes, orc.fill_rope_buf(128, n))
+    m.set_batch(np.arange(n + 1, dtype=np.int32), (1 + tokens).astype(np.uint32).ravel(), tg.ravel(), starts, finishes, L.fill_rope_buf(128, n))
     for _ in range(args.warmup):
         m.backprop()
     torch.cuda.synchronize()
@@ -420,7 +418,8 @@ def bench_step_fp8(args):
     out["bandwidth_kernels"] = bandwidth_kernels()
     roof["device_sustained"] = sustained(L.E4M3)
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline_step(orc, dim, heads, ffn, lt, la, ls, aw, vocab)
+        from oracle_lib import Oracle            # the CPU leg only
+        out["cpu_baseline"] = cpu_baseline_step(Oracle(), dim, heads, ffn, lt, la, ls, aw, vocab)
     return out
 
 
@@ -548,9 +547,7 @@ def bench_moe_fp8(args):
     import numpy as np
     import torch
     from tscale2_amd import lib as L
-    from oracle_lib import Oracle
     L.load()
-    orc = Oracle()
     dim, xp, experts, selected, n, vocab = 1024, 512, 64, 2, 65536, 128
     if args.small:
         n = 8192
@@ -573,7 +570,7 @@ def bench_moe_fp8(args):
     tg = r.integers(0, vocab, n).astype(np.int32)
     t = np.arange(n, dtype=np.int32)
     m.set_batch(np.arange(n + 1, dtype=np.int32), (1 + t).astype(np.uint32), tg, [np.maximum(t - 1, 0).astype(np.int32)],
-                [(t - 1).astype(np.int32)], orc.fill_rope_buf(128, n))
+                [(t - 1).astype(np.int32)], L.fill_rope_buf(128, n))
     m.backprop()                                  # fills state, stateGrad and the gradient scales once
 
     def step():

@@ -552,6 +552,16 @@ typedef struct ts2_model_config {
     int32_t recompute;
 } ts2_model_config;
 
+/* Host helpers for setting a model up (no device work).
+ * ts2_model_schedule: the layer list a model depth stands for - InitAlibi, src/gpt/model_params/model_dim.cpp:82-158 (the ALIBI_V3
+ *   branch every model string of the reference selects): attention types {1, 64, wideWindow} (depth 1: the single-attention profiling
+ *   case), layers as (type, attention type, ALiBi slope).  moeExpertCount > 0 makes the MLPs behind the first groups MoE layers.
+ *   Returns the number of layers written (<= maxLayers, else TS2_ERR_SHAPE); attWidth must hold 3 entries.
+ * ts2_fill_rope_buf: the (cos, sin) table fp32 [ropeLen][width] of FillRopeBuf, src/gpt/att/rope.cpp:4-38 (theta 5e5), host memory. */
+int ts2_model_schedule(int32_t depth, int32_t moeExpertCount, int32_t wideWindow, int32_t maxLayers, int32_t *layerType, int32_t *layerAttId,
+    float *layerSlope, int32_t *attWidth, int32_t *attTypeCount);
+int ts2_fill_rope_buf(float *buf, int32_t width, int32_t ropeLen);
+
 ts2_model *ts2_model_create(const ts2_model_config *cfg);
 void ts2_model_destroy(ts2_model *m);
 /* matrixId: MP_ATT_{Q,K,V,GATE,COMBINER} = 0..4, MP_FFN_{EXPAND,GATE,CONTRACT} = 0..2, MP_MOE_{EXPAND,GATE,CONTRACT,SELECT} = 0..3

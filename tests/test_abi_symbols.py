@@ -38,7 +38,7 @@ def test_probe_library_exports_its_header_and_the_product_header_holds_no_probe(
     assert os.path.exists(PROBE_SO), "build the library first: python -m tscale2_amd.build"
     dll = C.CDLL(PROBE_SO)
     names = declared_functions(PROBE_HEADER)
-    assert names == ["ts2_probe_copy_rate", "ts2_probe_mfma_rate"]
+    assert names == ["ts2_probe_clock_monitor", "ts2_probe_copy_rate", "ts2_probe_mfma_rate"]
     assert not [n for n in names if not hasattr(dll, n)]
 
 
@@ -90,3 +90,20 @@ def test_every_entry_point_cites_the_interface_it_replaces():
     """each declaration is preceded by a comment naming a reference file:line, or says that it has no counterpart there"""
     text = open(HEADER).read()
     assert len(re.findall(r"[a-z_]+\.(?:cuh|cu|h|cpp):\d+", text)) >= 30
+
+
+def test_model_schedule_and_rope_table_equal_the_oracle():
+    """ts2_model_schedule / ts2_fill_rope_buf (host code of the library) against the oracle's restatements, which are bit-exact against
+    the reference build (tests/test_oracle_vs_reference.py): InitAlibi src/gpt/model_params/model_dim.cpp:82-158, FillRopeBuf
+    src/gpt/att/rope.cpp:4-38.  No GPU needed."""
+    import numpy as np
+    from oracle_lib import Oracle
+    from tscale2_amd import lib as L
+    orc = Oracle()
+    for depth, experts, wide in ((1, 0, 64), (1, 8, 256), (2, 0, 64), (3, 8, 64), (12, 0, 1024), (13, 0, 128), (24, 16, 512), (60, 0, 64)):
+        want = orc.model_schedule(None, depth, experts, wide)
+        lt, la, ls, aw = L.model_schedule(depth, experts, wide)
+        assert np.array_equal(lt, want["layer_type"]) and np.array_equal(la, want["layer_att_id"]), (depth, experts)
+        assert np.array_equal(ls, want["layer_slope"]) and np.array_equal(aw, want["att_width"]), (depth, experts)
+    for width, n in ((128, 300), (64, 17), (128, 2048)):
+        assert np.array_equal(L.fill_rope_buf(width, n), orc.fill_rope_buf(width, n))

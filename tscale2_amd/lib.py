@@ -137,6 +137,40 @@ def call(name, *args, check=True):
     return rc
 
 
+def model_schedule(depth, experts=0, wide_window=64):
+    """(layer_type, layer_att_id, layer_slope, att_width) of a model depth: ts2_model_schedule (host only, no GPU needed)"""
+    import numpy as np
+    lib = load()
+    cap = 4 * max(depth, 1) + 8
+    lt = np.zeros(cap, np.int32); la = np.zeros(cap, np.int32); ls = np.zeros(cap, np.float32); aw = np.zeros(3, np.int32)
+    cnt = C.c_int32(0)
+    n = lib.dll.ts2_model_schedule(C.c_int32(depth), C.c_int32(experts), C.c_int32(wide_window), C.c_int32(cap), lt.ctypes.data_as(C.c_void_p),
+                                   la.ctypes.data_as(C.c_void_p), ls.ctypes.data_as(C.c_void_p), aw.ctypes.data_as(C.c_void_p), C.byref(cnt))
+    if n < 0:
+        raise RuntimeError(f"ts2_model_schedule failed with code {n}")
+    return lt[:n].copy(), la[:n].copy(), ls[:n].copy(), aw[:cnt.value].copy()
+
+
+def layer_shapes(ltype, dim, heads, ffn, xp=0, experts=0):
+    """[out][in] shapes of a layer's matrices in ts2_model_set_matrix order (EnumLayerMatrices, src/gpt/model_params/model_dim.h:225-262):
+    attention Q, K, V, gate, combiner; FFN expand, gate, contract; MoE expand, gate, contract, select"""
+    q = heads * 128
+    if ltype == 0:
+        return [(q, dim), (q, dim), (q, dim), (q, dim), (dim, q)]
+    if ltype == 2:
+        return [(ffn, dim), (ffn, dim), (dim, ffn)]
+    return [(xp * experts, dim), (xp * experts, dim), (dim * experts, xp), (experts, dim)]
+
+
+def fill_rope_buf(width, rope_len):
+    """fp32 [rope_len][width] (cos, sin) table: ts2_fill_rope_buf (host only)"""
+    import numpy as np
+    lib = load()
+    buf = np.zeros((rope_len, width), np.float32)
+    lib.check(lib.dll.ts2_fill_rope_buf(buf.ctypes.data_as(C.c_void_p), C.c_int32(width), C.c_int32(rope_len)), "ts2_fill_rope_buf")
+    return buf
+
+
 _probe = None
 
 
