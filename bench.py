@@ -44,7 +44,9 @@ def sustained(ab_type):
     """What the device sustains with nothing else running: an MFMA-only kernel with per-lane random operand bits (the chip is power
     limited below its boost clock under such data) and a streaming copy.  Reported beside the published peaks, never instead of them."""
     from tscale2_amd import lib as L
+    clock = L.probe_shader_clock(lambda: L.probe_mfma_rate(ab_type, 1, 60000), seconds=0.3)
     return {"mfma_only_random_operands_tops": round(L.probe_mfma_rate(ab_type, 1, 100000), 1),
+            "mfma_only_random_operands_shader_clock_mhz": round(clock[0]),
             "mfma_only_constant_operands_tops": round(L.probe_mfma_rate(ab_type, 0, 100000), 1),
             "copy_read_plus_write_gbps": round(L.probe_copy_rate(1 << 30), 1)}
 
@@ -320,8 +322,13 @@ def fp8_backward_gemms(n, dim, ffn, iters=100, warm=20, only_dominant=False):
         torch.cuda.synchronize()
         ms = event_time_ms(fn, iters)
         ops = 2.0 * m * nn * k
+
+        def again():
+            for _ in range(iters):
+                fn()
+        clock = L.probe_shader_clock(again, seconds=ms * iters * 1.3e-3)     # the shader clock while the same launches run once more
         out.append({"product": name, "m": m, "n": nn, "k": k, "us": round(ms * 1e3, 1), "tflops": round(ops / (ms * 1e-3) / 1e12, 1),
-                    "frac_of_peak": round(ops / (ms * 1e-3) / PEAK_FP8, 3)})
+                    "frac_of_peak": round(ops / (ms * 1e-3) / PEAK_FP8, 3), "shader_clock_mhz": round(clock[0])})
         return ms, ops
     first = run("dX: dY[tokens x ffn] x W^T (FFN expand / gate), fp32 result", n, dim, ffn)
     if only_dominant:
@@ -417,6 +424,18 @@ def bench_step_fp8(args):
     torch.cuda.empty_cache()
     out["bandwidth_kernels"] = bandwidth_kernels()
     roof["device_sustained"] = sustained(L.E4M3)
+    # config[3] and config[4] beside the step (their own --workload lines carry the CPU legs): a few launches each
+    import copy
+    sub = copy.copy(args)
+    sub.no_cpu, sub.steps, sub.warmup, sub.small = True, 10, 3, False
+    a = bench_att_bwd(sub)
+    out["att_bwd"] = {"workload": a["config"]["workload"], "ms": a["ms_per_step"], "tokens_per_s": a["value"], "tflops": a["roofline"]["achieved"],
+                      "frac_of_bf16_peak": a["roofline"]["frac"], "kernel": a["roofline"]["kernel"]}
+    torch.cuda.empty_cache()
+    mo = bench_moe_fp8(sub)
+    out["moe_layer"] = {"workload": mo["config"]["workload"], "ms": mo["ms_per_step"], "tokens_per_s": mo["value"], "layer_tflops": mo["layer_tflops"],
+                        "grouped_product": mo["roofline"]["kernel"], "grouped_product_frac_of_fp8_peak": mo["roofline"]["frac"]}
+    torch.cuda.empty_cache()
     if not args.no_cpu:
         from oracle_lib import Oracle            # the CPU leg only
         out["cpu_baseline"] = cpu_baseline_step(Oracle(), dim, heads, ffn, lt, la, ls, aw, vocab)
