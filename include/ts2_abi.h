@@ -213,6 +213,15 @@ int ts2_normalize_vecs_row_max2(int32_t len, int32_t lenRound, const ts2_mat *sr
     const ts2_mat *dst, float *rowScale, float *rowAbsMax, void *stream);
 int ts2_tile_max_from_rows(int32_t len, const float *rowAbsMax, const float *rowMult, int32_t kTile, float *tileMax, void *stream);
 
+/* the same with the reference's dither (src/gpt/compute/row_scale.cuh:32-35 adds uniform noise in (-0.5, 0.5) before it rounds, which
+ * makes the int8 gradient unbiased): ditherSeed != 0 quantises dst = sat_i8(rne(fma(src, 1/scale, u))) with
+ * u(t, x) = (byte (x % 4) of H(ditherSeed, t, x / 4) - 127.5) / 256, H(s, r, c) = lowbias32(s ^ r * 0x9E3779B1 ^ c * 0x85EBCA6B),
+ * lowbias32(h): h ^= h >> 16; h *= 0x7FEB352D; h ^= h >> 15; h *= 0x846CA68B; h ^= h >> 16 - the reference draws its noise from an LCG
+ * seeded with the row's own bits; this stream is the library's own, the property (E[dst * scale] = src) is the reference's.
+ * ditherSeed 0 = ts2_normalize_vecs_row_max2. */
+int ts2_normalize_vecs_row_max_dither(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, const float *colScale,
+    const ts2_mat *dst, float *rowScale, float *rowAbsMax, uint32_t ditherSeed, void *stream);
+
 /* HistSortFloatsStableKernel, src/lib/cuda/cuda_sort.cu:115-186 (SortPositiveFloatsApproxStable as BackpropMulti calls it on the row
  * scales of the gradient, src/gpt/compute/matmul_fwdbwd.cuh:325): order[0..len) = the rows sorted ascending by the top 13 bits (sign,
  * exponent, four mantissa bits) of key[t] = rowAbsMax[t] * |rowMult[t]| (rowMult optional); rows that share those bits come in
@@ -233,6 +242,10 @@ int ts2_tile_absmax(int32_t len, const ts2_mat *src, int32_t srcType, const floa
  * rowIndex (optional, [lenRound], -1 = zero row) gathers source rows first (MoeGroupSamples, moe_kernels.cuh:89-143). */
 int ts2_transpose_quant(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, const float *rowMult, const float *tileMax,
     int32_t kTile, const int32_t *rowIndex, const ts2_mat *dstT, int32_t dstType, float *tileScale, void *stream);
+/* the same with the dither of ts2_normalize_vecs_row_max_dither in the requantisation (dstType TS2_I8): the noise of element (t, x) is
+ * u(t, x) with t the position in dstT's rows (after the gather through rowIndex), x the source column. */
+int ts2_transpose_quant_dither(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, const float *rowMult, const float *tileMax,
+    int32_t kTile, const int32_t *rowIndex, const ts2_mat *dstT, int32_t dstType, float *tileScale, uint32_t ditherSeed, void *stream);
 
 /* Compress (src/gpt/matrix/delta.cpp:155-179) of a sum of fp32 partial products: delta = packed(alpha * (*alphaPtr) * sum_i partial_i),
  * partial_i = fp32 [rows][cols] at partial->ptr + i*slabBytes; the same arithmetic as TS2_EPI_ROW_TILE_MAXNORM.  Used with the stored
@@ -251,8 +264,9 @@ int ts2_pack_delta(const ts2_mat *partial, int32_t splits, int64_t slabBytes, in
  *   srcT  [srcDim][lenRound] 8-bit                              (I8: Src8T;  E4M3: SrcE4T)
  *   tileMax, tileScale [lenRound/kTile] fp32                    (I8: SortedTileScale)
  *   transformT [srcDim][gradDim] 8-bit                          (TransformT)
- * Differences from the reference, by design: no random dither in the int8 quantisers, the sort of the rows is optional (sortRows;
- * without it each kTile consecutive tokens share the delta GEMM's scale) and exact int32 sums per k-tile added in fp32. */
+ * Differences from the reference, by design: the dither of the int8 quantisers is optional and drawn from the library's own
+ * counter-based stream (ditherSeed), the sort of the rows is optional (sortRows; without it each kTile consecutive tokens share the
+ * delta GEMM's scale) and exact int32 sums per k-tile added in fp32. */
 typedef struct ts2_matmul_bwd_buffers {
     ts2_mat grad8;
     float *grad8RowScale;
@@ -292,6 +306,10 @@ typedef struct ts2_matmul_bwd_buffers {
      * reads both operands as they are - contraction-major, ts2_gemm_args.kMajor - and neither is transposed: gradT, srcT and their
      * Valid flags are not used.  The result is bit-identical to the transposing sequence. */
     int32_t padRowsZero;
+    /* != 0 (I8): BackpropMulti and BackpropDelta quantise the gradient with the dither of ts2_normalize_vecs_row_max_dither /
+     * ts2_transpose_quant_dither under this seed (unbiased int8 gradients, as the reference's NormalizeVecsRowMaxWithNoise gives); 0 rounds
+     * to nearest.  A caller varies the seed from matrix to matrix and from step to step. */
+    uint32_t ditherSeed;
 } ts2_matmul_bwd_buffers;
 
 /* Bytes of every scratch member of ts2_matmul_bwd_buffers for one matrix, the sizes TInt8MatMulBwdBuffers / TFp8MatMulBwdBuffers allocate
@@ -550,6 +568,9 @@ typedef struct ts2_model_config {
     /* 0: every FFN and attention layer keeps what its forward pass computed for its backward pass when that fits into half of the
      * free device memory; 1: the backward recomputes it, as the reference's AddBackward does (layer_ffn.cu:83-113, layer_att.cu:160-226) */
     int32_t recompute;
+    /* != 0 (TS2_I8 models): the int8 quantisers of every linear backward dither (ts2_matmul_bwd_buffers.ditherSeed), each call under a
+     * seed of its own derived from this one and a call counter; 0: round to nearest */
+    uint32_t ditherSeed;
 } ts2_model_config;
 
 /* Host helpers for setting a model up (no device work).

@@ -17,7 +17,7 @@
  *   backprop_scale_experts, fwd/bwd_contract_matrix, layer_forward, layer_backward, final_backward, model_step
  *       -> their reference sources need cuda_runtime.h and cannot be compiled here; pinned by brute force over the code table,
  *          invariants, bilinear / adjoint identities and fp64 finite differences (tests/test_oracle_closed_forms.py).
- *   quant_rowmax_i8, quant_ktile_i8, gemm_i8_nt, gemm_i8_nt_rowscale, gemm_i8_nt_ktile, gemm_f32_nt, dequant_i8/e4m3, bf16_round,
+ *   quant_rowmax_i8(_noise), quant_ktile_i8(_noise), gemm_i8_nt, gemm_i8_nt_rowscale, gemm_i8_nt_ktile, gemm_f32_nt, dequant_i8/e4m3, bf16_round,
  *   softmax2, embedding_forward/backward, and the same-contract layer functions (orc_sc_*)
  *       -> this library's own contracts and helpers: closed forms against numpy round-half-even and int64 products, torch's bfloat16
  *          conversion, scipy's softmax, adjoint identities (tests/test_oracle_own_contract.py, tests/test_same_contract_cpu.py).
@@ -83,6 +83,8 @@ void orc_dequant_e4m3(const uint8_t *fast, float *w, int n, float scale);
 void orc_compress_delta(const float *data, int8_t *delta, float *tileScale, int ySize, int xSize);
 void orc_quant_rowmax_i8(const float *src, int8_t *dst, float *rowScale, int len, int dim);
 void orc_quant_ktile_i8(const float *src, int8_t *dst, float *tileScale, int len, int dim, int kTile);
+void orc_quant_rowmax_i8_noise(const float *src, const float *noise, int8_t *dst, float *rowScale, int len, int dim);
+void orc_quant_ktile_i8_noise(const float *src, const float *noise, int8_t *dst, float *tileScale, int len, int dim, int kTile);
 float orc_grad_mult(float maxNorm);
 float orc_bf16_round(float x);
 

@@ -254,6 +254,53 @@ void orc_quant_rowmax_i8(const float *src, int8_t *dst, float *rowScale, int len
     }
 }
 
+/* The same with the noise NormalizeVecsRowMaxKernel adds before it rounds (src/gpt/compute/row_scale.cuh:32-35:
+ * buf[d] = buf[d] * mult + rng.GenUniformFloat() - 0.5f): noise[t][x] in (-0.5, 0.5) is handed in by the caller (the reference draws it
+ * from an LCG seeded with the row's own bits; the library under test from a counter-based hash).  One fused multiply-add per element. */
+void orc_quant_rowmax_i8_noise(const float *src, const float *noise, int8_t *dst, float *rowScale, int len, int dim)
+{
+    for (int t = 0; t < len; ++t) {
+        float maxVal = 0;
+        for (int x = 0; x < dim; ++x) {
+            float a = fabsf(src[(size_t)t * dim + x]);
+            maxVal = maxVal > a ? maxVal : a;
+        }
+        float discrScale = 0;
+        float mult = 0;
+        if (maxVal > 0) {
+            discrScale = maxVal / 127;
+            mult = 1 / discrScale;
+        }
+        for (int x = 0; x < dim; ++x) {
+            dst[(size_t)t * dim + x] = orc_cvt_i8(fmaf(src[(size_t)t * dim + x], mult, noise[(size_t)t * dim + x]));
+        }
+        rowScale[t] = discrScale;
+    }
+}
+
+/* orc_quant_ktile_i8 (below) with the same noise in its requantisation */
+void orc_quant_ktile_i8_noise(const float *src, const float *noise, int8_t *dst, float *tileScale, int len, int dim, int kTile)
+{
+    for (int t0 = 0; t0 < len; t0 += kTile) {
+        int t1 = t0 + kTile < len ? t0 + kTile : len;
+        float maxVal = 0;
+        for (int t = t0; t < t1; ++t) {
+            for (int x = 0; x < dim; ++x) {
+                float a = fabsf(src[(size_t)t * dim + x]);
+                maxVal = maxVal > a ? maxVal : a;
+            }
+        }
+        float scale = maxVal > 0 ? maxVal / 127 : 1;
+        float mult = 1 / scale;
+        for (int t = t0; t < t1; ++t) {
+            for (int x = 0; x < dim; ++x) {
+                dst[(size_t)t * dim + x] = orc_cvt_i8(fmaf(src[(size_t)t * dim + x], mult, noise[(size_t)t * dim + x]));
+            }
+        }
+        tileScale[t0 / kTile] = scale;
+    }
+}
+
 /* Role of ShuffleMaxScaleTransposeKernel (src/gpt/compute/matmul_fwdbwd.cuh:209-280) without the sort and the dither: every
  * kTile consecutive rows share one scale = maxabs(tile)/127 (1 for an all-zero tile), requantised from the fp32 source.
  * Output stays row-major [len][dim]; the transposed copy the reference writes is a layout choice of its GEMM. */

@@ -143,10 +143,10 @@ class Harness:
         return loss
 
     # ---- device side
-    def device_model(self, k_tile=0, recompute=False):
+    def device_model(self, k_tile=0, recompute=False, dither_seed=0):
         from tscale2_amd import lib as L
         m = L.Model(self.mode, self.dim, self.heads, self.ffn, self.lt, self.la, self.ls, len(self.att_width), self.vocab, self.label_count,
-                    self.n, self.xp if self.experts else 0, self.experts, self.selected if self.experts else 0, k_tile, recompute)
+                    self.n, self.xp if self.experts else 0, self.experts, self.selected if self.experts else 0, k_tile, recompute, dither_seed)
         for d in range(self.depth):
             for i, q in enumerate(self.layers[d]):
                 m.set_matrix(d, i, q.fast, q.scale)

@@ -354,3 +354,82 @@ def test_transpose_and_ktile_quant(L, orc):
     np.testing.assert_allclose(tsc.cpu().numpy(), want_s, rtol=3e-7)
     got = dst.cpu().numpy()[:, :len_].T.astype(np.int32)
     np.testing.assert_array_equal(got, want_q)
+
+
+@pytest.mark.parametrize("src,dim", [("bf16", 1536), ("bf16", 4096), ("f32", 1280), ("bf16", 640)])
+def test_row_max_quantise_with_dither_equals_the_oracle_given_the_same_noise(L, orc, src, dim):
+    """ts2_normalize_vecs_row_max_dither: the reference rounds x / scale + u, u uniform in (-0.5, 0.5) (src/gpt/compute/row_scale.cuh:32-35).
+    The library's u is a counter-based hash of (seed, row, column); the oracle takes the same values as an array: bytes and scales must
+    agree bit for bit on the wave-per-row kernel (bf16, dim a multiple of 512) and on the workgroup-per-row kernel alike."""
+    from test_oracle_own_contract import dither_noise
+    print("case rowmax dither", src, dim, flush=True)
+    r = np.random.default_rng(dim)
+    len_, len_round, seed = 1000, 1024, 0x1234567
+    x = (r.standard_normal((len_, dim)) * r.random((len_, 1)) * 5).astype(np.float32)
+    x[11] = 0
+    if src == "bf16":
+        x16 = torch.from_numpy(x).bfloat16()
+        x = x16.float().numpy()
+        dsrc, ty = x16.cuda().view(torch.int16), L.BF16
+    else:
+        dsrc, ty = dev(x), L.F32
+    noise = dither_noise(seed, len_, dim)
+    want = np.zeros((len_, dim), np.int8); wscale = np.zeros(len_, np.float32)
+    orc.lib.orc_quant_rowmax_i8_noise(_ptr(np.ascontiguousarray(x)), _ptr(noise), _ptr(want), _ptr(wscale), len_, dim)
+    dst = torch.full((len_round, dim), 3, dtype=torch.int8, device="cuda")
+    rs = torch.full((len_round,), -1.0, device="cuda")
+    L.call("ts2_normalize_vecs_row_max_dither", len_, len_round, dsrc, ty, None, dst, rs, None, seed)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(rs.cpu().numpy()[:len_], wscale)
+    np.testing.assert_array_equal(dst.cpu().numpy()[:len_], want)
+    assert np.all(dst.cpu().numpy()[len_:] == 0)
+    plain = np.zeros((len_, dim), np.int8)
+    orc.lib.orc_quant_rowmax_i8(_ptr(np.ascontiguousarray(x)), _ptr(plain), _ptr(wscale), len_, dim)
+    assert 0.2 < (plain != want).mean() < 0.6                                   # the dither does move a good part of the bytes
+    # seed 0 is the deterministic quantiser
+    L.call("ts2_normalize_vecs_row_max_dither", len_, len_round, dsrc, ty, None, dst, rs, None, 0)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(dst.cpu().numpy()[:len_], plain)
+
+
+def test_dithered_quantiser_is_unbiased_on_the_device(L):
+    """E[q * scale] = x: rows of one constant (plus one extreme element that fixes the scale at 1) quantised under the dither average to
+    the constant; rounding to nearest gives the nearest integer instead."""
+    print("case rowmax dither unbiased", flush=True)
+    len_, dim = 4096, 512
+    for c in (0.3, -1.45, 17.02):
+        x = torch.full((len_, dim), c, device="cuda")
+        x[:, 0] = 127
+        dst = torch.zeros((len_, dim), dtype=torch.int8, device="cuda")
+        rs = torch.zeros(len_, device="cuda")
+        L.call("ts2_normalize_vecs_row_max_dither", len_, len_, x, L.F32, None, dst, rs, None, 4242)
+        torch.cuda.synchronize()
+        assert bool((rs == 1).all())
+        mean = dst[:, 1:].double().mean().item()
+        assert abs(mean - c) < 2e-3, (c, mean)
+        L.call("ts2_normalize_vecs_row_max_dither", len_, len_, x, L.F32, None, dst, rs, None, 0)
+        torch.cuda.synchronize()
+        assert dst[:, 1:].double().mean().item() == round(c)
+
+
+def test_transpose_and_ktile_quant_with_dither(L, orc):
+    from test_oracle_own_contract import dither_noise
+    print("case transpose dither", flush=True)
+    r = np.random.default_rng(16)
+    len_, len_round, dim, kt, seed = 700, 768, 256, 256, 99991
+    x16 = torch.from_numpy((r.standard_normal((len_, dim)) * (1 + 10 * r.random((len_, 1)))).astype(np.float32)).bfloat16()
+    x = x16.float().numpy()
+    rm = (r.random(len_) + 0.5).astype(np.float32)
+    xs = x * rm[:, None]
+    noise = dither_noise(seed, len_, dim)
+    want_q = np.zeros((len_, dim), np.int8); want_s = np.zeros(len_round // kt, np.float32)
+    orc.lib.orc_quant_ktile_i8_noise(_ptr(xs), _ptr(noise), _ptr(want_q), _ptr(want_s), len_, dim, kt)
+    tmax = torch.full((len_round // kt,), 7.0, device="cuda")
+    L.call("ts2_tile_absmax", len_, x16.cuda().view(torch.int16), L.BF16, dev(rm), kt, tmax, 1)
+    tsc = torch.zeros(len_round // kt, device="cuda")
+    dst = torch.full((dim, len_round), 5, dtype=torch.int8, device="cuda")
+    L.call("ts2_transpose_quant_dither", len_, len_round, x16.cuda().view(torch.int16), L.BF16, dev(rm), tmax, kt, None, dst, L.I8, tsc, seed)
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(tsc.cpu().numpy(), want_s, rtol=3e-7)
+    np.testing.assert_array_equal(dst.cpu().numpy()[:, :len_].T, want_q)
+    assert np.all(dst.cpu().numpy()[:, len_:] == 0)

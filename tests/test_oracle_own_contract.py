@@ -199,3 +199,67 @@ def test_hist_sort_reproduces_the_hash_of_the_reference_sort_test(orc):
     o2 = np.zeros(300, np.int32)
     orc.lib.orc_hist_sort_stable(_ptr(y), 300, _ptr(o2), 0)
     assert np.array_equal(o2, np.lexsort((np.arange(300), y)))
+
+
+def dither_noise(seed, rows, cols, row0=0):
+    """the library's dither stream (include/ts2_abi.h, ts2_normalize_vecs_row_max_dither): noise[t][x] = (byte (x % 4) of
+    lowbias32(seed ^ t * 0x9E3779B1 ^ (x / 4) * 0x85EBCA6B) - 127.5) / 256, in uint32 arithmetic"""
+    t = (np.arange(rows, dtype=np.uint64) + row0)[:, None]
+    c4 = (np.arange(cols, dtype=np.uint64) // 4)[None, :]
+    m = np.uint64(0xffffffff)
+    h = (np.uint64(seed) ^ ((t * np.uint64(0x9E3779B1)) & m) ^ ((c4 * np.uint64(0x85EBCA6B)) & m)) & m
+    h ^= h >> np.uint64(16)
+    h = (h * np.uint64(0x7FEB352D)) & m
+    h ^= h >> np.uint64(15)
+    h = (h * np.uint64(0x846CA68B)) & m
+    h ^= h >> np.uint64(16)
+    byte = (h >> (np.uint64(8) * (np.arange(cols, dtype=np.uint64) % np.uint64(4))[None, :])) & np.uint64(255)
+    return ((byte.astype(np.float32) - np.float32(127.5)) * np.float32(1 / 256)).astype(np.float32)
+
+
+def test_dithered_quantisers_closed_form_and_unbiased(orc):
+    """q = saturate(round-half-even(fma(x, 1/scale, noise))): equal to the plain quantiser for zero noise, equal to numpy's float64
+    evaluation rounded once (a fused multiply-add), and unbiased: the mean of q * scale over a uniform noise stream is x.
+    The hash stream itself is uniform over its 256 levels and independent between neighbouring columns and rows."""
+    r = np.random.default_rng(31)
+    x = heavy_rows(r, 23, 384)
+    q0 = np.zeros(x.shape, np.int8); s0 = np.zeros(23, np.float32)
+    orc.lib.orc_quant_rowmax_i8(_ptr(x), _ptr(q0), _ptr(s0), *x.shape)
+    zero = np.zeros_like(x)
+    q = np.full(x.shape, 99, np.int8); sc = np.full(23, -1, np.float32)
+    orc.lib.orc_quant_rowmax_i8_noise(_ptr(x), _ptr(zero), _ptr(q), _ptr(sc), *x.shape)
+    assert np.array_equal(q, q0) and np.array_equal(sc, s0)
+    noise = dither_noise(12345, *x.shape)
+    assert noise.min() >= -0.5 + 1 / 512 - 1e-7 and noise.max() <= 0.5 - 1 / 512 + 1e-7
+    orc.lib.orc_quant_rowmax_i8_noise(_ptr(x), _ptr(noise), _ptr(q), _ptr(sc), *x.shape)
+    mult = np.where(s0 > 0, np.float32(1) / np.where(s0 > 0, s0, 1), 0).astype(np.float32)
+    fused = (x.astype(np.float64) * mult[:, None].astype(np.float64) + noise.astype(np.float64)).astype(np.float32)   # one rounding
+    assert np.array_equal(q, np.clip(np.rint(fused), -128, 127).astype(np.int8))
+    assert np.array_equal(sc, s0)
+    # the stream: every level equally likely, no correlation between neighbours
+    big = dither_noise(777, 512, 2048)
+    levels = np.rint((big + 0.5) * 256 - 0.5).astype(np.int64)
+    counts = np.bincount(levels.ravel(), minlength=256)
+    assert counts.min() > 0.9 * big.size / 256 and counts.max() < 1.1 * big.size / 256
+    assert abs(big.mean()) < 1e-3
+    assert abs((big[:, 1:] * big[:, :-1]).mean()) < 2e-4 and abs((big[1:] * big[:-1]).mean()) < 2e-4
+    # unbiased: a constant row (plus one extreme element that fixes the scale at 1) under many noise rows
+    const = np.full((4096, 256), 0.3, np.float32)
+    const[:, 0] = 127
+    nz = dither_noise(99, *const.shape)
+    qc = np.zeros(const.shape, np.int8); scc = np.zeros(4096, np.float32)
+    orc.lib.orc_quant_rowmax_i8_noise(_ptr(const), _ptr(nz), _ptr(qc), _ptr(scc), *const.shape)
+    assert (scc == 1).all()
+    assert abs(qc[:, 1:].astype(np.float64).mean() - 0.3) < 2e-3               # round-to-nearest alone gives 0
+    # k-tile form: the same noise rule with one scale per tile
+    xk = heavy_rows(r, 16, 128)
+    nk = dither_noise(5, 16, 128)
+    qk = np.zeros(xk.shape, np.int8); sk = np.zeros(2, np.float32)
+    orc.lib.orc_quant_ktile_i8_noise(_ptr(xk), _ptr(nk), _ptr(qk), _ptr(sk), 16, 128, 8)
+    for t in range(2):
+        blk = xk[t * 8:(t + 1) * 8]
+        mx = np.abs(blk).max()
+        s = np.float32(mx) / np.float32(127) if mx > 0 else np.float32(1)
+        assert sk[t] == s
+        f = (blk.astype(np.float64) * np.float64(np.float32(1) / s) + nk[t * 8:(t + 1) * 8].astype(np.float64)).astype(np.float32)
+        assert np.array_equal(qk[t * 8:(t + 1) * 8], np.clip(np.rint(f), -128, 127).astype(np.int8))

@@ -86,6 +86,35 @@ __device__ __forceinline__ float E4m3ToFloat(uint32_t byte)
     return __builtin_amdgcn_cvt_f32_fp8((int)byte, 0);
 }
 
+// Dither of the int8 quantisers (the role of the uniform noise NormalizeVecsRowMaxKernel adds before it rounds,
+// src/gpt/compute/row_scale.cuh:32-35: rounding to nearest of x + u, u uniform in (-0.5, 0.5), is unbiased).  The noise is a counter-based
+// hash of (seed, row, column / 4): one 32-bit word serves four neighbouring columns, byte b standing for the offset (b - 127.5) / 256.
+// The offsets of a row depend on nothing but (seed, row, column), so a test can hand the same array to the CPU restatement.
+__device__ __forceinline__ uint32_t DitherWord(uint32_t seed, int row, int col4)
+{
+    uint32_t h = seed ^ ((uint32_t)row * 0x9E3779B1u) ^ ((uint32_t)col4 * 0x85EBCA6Bu);
+    h ^= h >> 16;
+    h *= 0x7FEB352Du;
+    h ^= h >> 15;
+    h *= 0x846CA68Bu;
+    h ^= h >> 16;
+    return h;
+}
+
+__device__ __forceinline__ float DitherOffset(uint32_t word, int j)
+{
+    return ((float)((word >> (8 * j)) & 255u) - 127.5f) * (1.f / 256);
+}
+
+// sat_i8(rne(x * mult + offset)) of four neighbouring columns, one fused multiply-add each
+__device__ __forceinline__ uint32_t QuantDither4(float x0, float x1, float x2, float x3, float mult, uint32_t word)
+{
+    return (uint32_t)(CvtToI8(__builtin_fmaf(x0, mult, DitherOffset(word, 0))) & 0xff) |
+           ((uint32_t)(CvtToI8(__builtin_fmaf(x1, mult, DitherOffset(word, 1))) & 0xff) << 8) |
+           ((uint32_t)(CvtToI8(__builtin_fmaf(x2, mult, DitherOffset(word, 2))) & 0xff) << 16) |
+           ((uint32_t)(CvtToI8(__builtin_fmaf(x3, mult, DitherOffset(word, 3))) & 0xff) << 24);
+}
+
 // Cross-lane exchange without the LDS crossbar: DPP modifiers inside a row of 16 lanes (they fold into the consuming VALU
 // instruction), v_permlane16_swap / v_permlane32_swap of gfx950 across rows.  A butterfly reduction over 1, 2, 4, 8 uses
 // quad_perm, quad_perm, row_half_mirror and row_mirror: once the quads (the 8-lane halves) hold one value each, the mirrored lane

@@ -699,7 +699,7 @@ __global__ void __launch_bounds__(256) BackpropLoLUAtt8(int len, int lenRound, i
 // flight.  Longer rows are read twice (the second read is served by L2).
 template <class TSrc, bool REG>
 __global__ void __launch_bounds__(256) NormalizeVecsRowMax(int len, int lenRound, int dim, Mat src, const float *colScale, Mat dst, float *rowScale,
-    float *rowAbsMax)
+    float *rowAbsMax, uint32_t seed)
 {
     __shared__ float red[2][4], redPlain[2][4];
     const int tid = threadIdx.x;
@@ -782,7 +782,11 @@ __global__ void __launch_bounds__(256) NormalizeVecsRowMax(int len, int lenRound
             for (int i = 0; i < 4; ++i) {
                 int col = tid * 4 + i * 1024;
                 if (col < dim) {
-                    Store4<TI8>(At<TI8>(dst, t, col), keep[i] * mult);
+                    if (seed) {
+                        *(uint32_t *)At<TI8>(dst, t, col) = QuantDither4(keep[i].x, keep[i].y, keep[i].z, keep[i].w, mult, DitherWord(seed, t, col >> 2));
+                    } else {
+                        Store4<TI8>(At<TI8>(dst, t, col), keep[i] * mult);
+                    }
                 }
             }
         } else {
@@ -791,7 +795,11 @@ __global__ void __launch_bounds__(256) NormalizeVecsRowMax(int len, int lenRound
                 if (colScale) {
                     v = v * Load4<TF32>(colScale + col);
                 }
-                Store4<TI8>(At<TI8>(dst, t, col), v * mult);
+                if (seed) {
+                    *(uint32_t *)At<TI8>(dst, t, col) = QuantDither4(v.x, v.y, v.z, v.w, mult, DitherWord(seed, t, col >> 2));
+                } else {
+                    Store4<TI8>(At<TI8>(dst, t, col), v * mult);
+                }
             }
         }
         if (tid == 0) {
@@ -804,7 +812,8 @@ __global__ void __launch_bounds__(256) NormalizeVecsRowMax(int len, int lenRound
 // consecutive elements (16-byte loads, 8-byte stores, each instruction of the wave covering 1 KB / 512 B of the row), the row
 // maxima are wave reductions, and no workgroup barrier or LDS exchange is left.  Same arithmetic per element as NormalizeVecsRowMax.
 template <int NCH>
-__global__ void __launch_bounds__(256) NormalizeRowsWave(int len, int lenRound, Mat src, const float *colScale, Mat dst, float *rowScale, float *rowAbsMax)
+__global__ void __launch_bounds__(256) NormalizeRowsWave(int len, int lenRound, Mat src, const float *colScale, Mat dst, float *rowScale, float *rowAbsMax,
+    uint32_t seed)
 {
     const int lane = threadIdx.x & 63;
     const int nWaves = gridDim.x * 4;
@@ -862,6 +871,13 @@ __global__ void __launch_bounds__(256) NormalizeRowsWave(int len, int lenRound, 
         }
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
+            if (seed) {
+                const int col4 = (i * 64 + lane) * 2;
+                *(uint2 *)(out + (i * 64 + lane) * 8) =
+                    make_uint2(QuantDither4(v[i][0].x, v[i][0].y, v[i][0].z, v[i][0].w, mult, DitherWord(seed, t, col4)),
+                        QuantDither4(v[i][1].x, v[i][1].y, v[i][1].z, v[i][1].w, mult, DitherWord(seed, t, col4 + 1)));
+                continue;
+            }
             F4 a = v[i][0] * mult, b = v[i][1] * mult;
             uint32_t lo = (uint32_t)(CvtToI8(a.x) & 0xff) | ((uint32_t)(CvtToI8(a.y) & 0xff) << 8) | ((uint32_t)(CvtToI8(a.z) & 0xff) << 16) |
                           ((uint32_t)(CvtToI8(a.w) & 0xff) << 24);
@@ -968,7 +984,7 @@ __global__ void __launch_bounds__(256) TileAbsMax(int len, int dim, Mat src, con
 // lanes cover the 128 bytes of one destination row.
 template <class TSrc, bool QUANT>
 __global__ void __launch_bounds__(256) TransposeQuant(int len, int lenRound, Mat src, const float *rowMult, const float *tileMax, int kTile,
-    const int *rowIndex, Mat dst, float *tileScale, const float *rowAbsMax)
+    const int *rowIndex, Mat dst, float *tileScale, const float *rowAbsMax, uint32_t seed)
 {
     constexpr int PITCH = 132;
     __shared__ __attribute__((aligned(16))) uint8_t buf[128 * PITCH];
@@ -1051,13 +1067,16 @@ __global__ void __launch_bounds__(256) TransposeQuant(int len, int lenRound, Mat
 #pragma unroll
                 for (int q = 0; q < EPL / 4; ++q) {
                     packed[q] = 0;
+                    // (the dither's row is the position in the contraction, its column the gradient's)
+                    const uint32_t word = seed ? DitherWord(seed, tBlock + r, (xBlock + lc * EPL) / 4 + q) : 0u;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         float x = f[q * 4 + e];
                         if (rowMult) {
                             x = x * rm[k];
                         }
-                        packed[q] |= (uint32_t)(CvtToI8(x * mult) & 0xff) << (8 * e);
+                        const float y = seed ? __builtin_fmaf(x, mult, DitherOffset(word, e)) : x * mult;
+                        packed[q] |= (uint32_t)(CvtToI8(y) & 0xff) << (8 * e);
                     }
                 }
                 *(uint32_t *)d = packed[0];
@@ -1549,8 +1568,14 @@ extern "C" int ts2_tile_max_from_rows(int32_t len, const float *rowAbsMax, const
     return TS2_OK;
 }
 
+extern "C" int ts2_normalize_vecs_row_max_dither(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, const float *colScale,
+    const ts2_mat *dst, float *rowScale, float *rowAbsMax, uint32_t ditherSeed, void *stream);
+
 extern "C" int ts2_normalize_vecs_row_max2(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, const float *colScale,
-    const ts2_mat *dst, float *rowScale, float *rowAbsMax, void *stream);
+    const ts2_mat *dst, float *rowScale, float *rowAbsMax, void *stream)
+{
+    return ts2_normalize_vecs_row_max_dither(len, lenRound, src, srcType, colScale, dst, rowScale, rowAbsMax, 0, stream);
+}
 
 extern "C" int ts2_normalize_vecs_row_max(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, const float *colScale,
     const ts2_mat *dst, float *rowScale, void *stream)
@@ -1558,8 +1583,8 @@ extern "C" int ts2_normalize_vecs_row_max(int32_t len, int32_t lenRound, const t
     return ts2_normalize_vecs_row_max2(len, lenRound, src, srcType, colScale, dst, rowScale, nullptr, stream);
 }
 
-extern "C" int ts2_normalize_vecs_row_max2(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, const float *colScale,
-    const ts2_mat *dst, float *rowScale, float *rowAbsMax, void *stream)
+extern "C" int ts2_normalize_vecs_row_max_dither(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, const float *colScale,
+    const ts2_mat *dst, float *rowScale, float *rowAbsMax, uint32_t ditherSeed, void *stream)
 {
     if (!src || !dst || !rowScale) {
         return TS2_ERR_NULL;
@@ -1574,7 +1599,7 @@ extern "C" int ts2_normalize_vecs_row_max2(int32_t len, int32_t lenRound, const 
         // with column scales a wave walks several rows (the scales stay in registers), else one row per wave
         const int wgs = (lenRound + 3) / 4;
         const dim3 grid(colScale && wgs > 2048 ? 2048 : wgs);
-#define LAUNCH_RW(N) hipLaunchKernelGGL((NormalizeRowsWave<N>), grid, dim3(256), 0, STREAM, len, lenRound, M(*src), colScale, M(*dst), rowScale, rowAbsMax)
+#define LAUNCH_RW(N) hipLaunchKernelGGL((NormalizeRowsWave<N>), grid, dim3(256), 0, STREAM, len, lenRound, M(*src), colScale, M(*dst), rowScale, rowAbsMax, ditherSeed)
         switch (dim / 512) {
         case 1: LAUNCH_RW(1); break;
         case 2: LAUNCH_RW(2); break;
@@ -1589,7 +1614,7 @@ extern "C" int ts2_normalize_vecs_row_max2(int32_t len, int32_t lenRound, const 
         TS2_CHECK_LAUNCH();
         return TS2_OK;
     }
-#define LAUNCH_RM(TS, REG) hipLaunchKernelGGL((NormalizeVecsRowMax<TS, REG>), dim3(lenRound < 4096 ? lenRound : 4096), dim3(256), 0, STREAM, len, lenRound, dim, M(*src), colScale, M(*dst), rowScale, rowAbsMax)
+#define LAUNCH_RM(TS, REG) hipLaunchKernelGGL((NormalizeVecsRowMax<TS, REG>), dim3(lenRound < 4096 ? lenRound : 4096), dim3(256), 0, STREAM, len, lenRound, dim, M(*src), colScale, M(*dst), rowScale, rowAbsMax, ditherSeed)
     if (srcType == TS2_BF16) {
         if (reg) {
             LAUNCH_RM(TBF16, true);
@@ -1645,11 +1670,17 @@ extern "C" int ts2_transpose_quant(int32_t len, int32_t lenRound, const ts2_mat 
     return Ts2TransposeQuantRows(len, lenRound, src, srcType, rowMult, tileMax, nullptr, kTile, rowIndex, dstT, dstType, tileScale, stream);
 }
 
+extern "C" int ts2_transpose_quant_dither(int32_t len, int32_t lenRound, const ts2_mat *src, int32_t srcType, const float *rowMult, const float *tileMax,
+    int32_t kTile, const int32_t *rowIndex, const ts2_mat *dstT, int32_t dstType, float *tileScale, uint32_t ditherSeed, void *stream)
+{
+    return Ts2TransposeQuantRows(len, lenRound, src, srcType, rowMult, tileMax, nullptr, kTile, rowIndex, dstT, dstType, tileScale, stream, ditherSeed);
+}
+
 // ts2_transpose_quant whose k-tile maxima may come from the row maxima instead (rowAbsMax, with tileMax null; with a row index: the
 // maxima of the rows gathered into the tile): the kernel then forms each k-tile's maximum itself and the separate
 // ts2_tile_max_from_rows launch is not needed
 int Ts2TransposeQuantRows(int len, int lenRound, const ts2_mat *src, int srcType, const float *rowMult, const float *tileMax, const float *rowAbsMax,
-    int kTile, const int *rowIndex, const ts2_mat *dstT, int dstType, float *tileScale, void *stream)
+    int kTile, const int *rowIndex, const ts2_mat *dstT, int dstType, float *tileScale, void *stream, uint32_t ditherSeed)
 {
     if (!src || !dstT) {
         return TS2_ERR_NULL;
@@ -1673,14 +1704,14 @@ int Ts2TransposeQuantRows(int len, int lenRound, const ts2_mat *src, int srcType
         }
         if (srcType == TS2_BF16) {
             hipLaunchKernelGGL((TransposeQuant<TBF16, true>), grid, dim3(256), 0, STREAM, len, lenRound, M(*src), rowMult, tileMax, kTile, rowIndex,
-                M(*dstT), tileScale, rowAbsMax);
+                M(*dstT), tileScale, rowAbsMax, ditherSeed);
         } else {
             hipLaunchKernelGGL((TransposeQuant<TF32, true>), grid, dim3(256), 0, STREAM, len, lenRound, M(*src), rowMult, tileMax, kTile, rowIndex,
-                M(*dstT), tileScale, rowAbsMax);
+                M(*dstT), tileScale, rowAbsMax, ditherSeed);
         }
     } else if (ElemSize(srcType) == 1 && dstType == srcType) {
         hipLaunchKernelGGL((TransposeQuant<TI8, false>), grid, dim3(256), 0, STREAM, len, lenRound, M(*src), nullptr, nullptr, 128, rowIndex,
-            M(*dstT), nullptr, nullptr);
+            M(*dstT), nullptr, nullptr, 0u);
     } else {
         return TS2_ERR_UNSUPPORTED;
     }

@@ -16,4 +16,4 @@ int Ts2ZeroRows(const ts2_mat *m, int rows, int rowBytes, void *stream);
 int Ts2FillFloats(float *p, int n, float v, void *stream);
 // ts2_transpose_quant with the k-tile maxima formed in the kernel from row maxima (rowAbsMax) when tileMax is null
 int Ts2TransposeQuantRows(int len, int lenRound, const ts2_mat *src, int srcType, const float *rowMult, const float *tileMax, const float *rowAbsMax,
-    int kTile, const int *rowIndex, const ts2_mat *dstT, int dstType, float *tileScale, void *stream);
+    int kTile, const int *rowIndex, const ts2_mat *dstT, int dstType, float *tileScale, void *stream, uint32_t ditherSeed = 0);

@@ -152,6 +152,7 @@ struct ts2_model {
     float *sPartial = 0;                     // fp32 slices of a delta product with few output tiles
     size_t sPartialFloats = 0;
     float *sRowScale = 0, *sTileMax = 0, *sTileScale = 0;
+    uint32_t ditherCalls = 0; // uses of the linear operator so far (seeds of the int8 dither)
     int maxW = 0, RP = 0; // RP = rows of the row-indexed scratch (max(R, lenMoe))
     int cuCount = 256;
 
@@ -217,6 +218,14 @@ ts2_matmul_bwd_buffers Scratch(ts2_model *M, int rows, int srcDim, int gradDim)
     b.tileMax = M->sTileMax;
     b.tileScale = M->sTileScale;
     b.transformT = Flat(M->sWT, srcDim, gradDim, M->mode).m;
+    if (M->cfg.ditherSeed) {
+        // every use of the operator draws its own noise: the call counter runs on from step to step
+        uint32_t h = M->cfg.ditherSeed + 0x9E3779B9u * ++M->ditherCalls;
+        h ^= h >> 15;
+        h *= 0x2C1B3C6Du;
+        h ^= h >> 12;
+        b.ditherSeed = h | 1u;
+    }
     return b;
 }
 

@@ -57,7 +57,8 @@ extern "C" int ts2_matmul_backprop_multi(int32_t mode, int32_t len, int32_t lenR
         if (!grad || !buf->grad8RowScale) {
             return TS2_ERR_NULL;
         }
-        int rc = ts2_normalize_vecs_row_max2(len, lenRound, grad, gradType, gradColScale, &buf->grad8, buf->grad8RowScale, buf->gradRowAbsMax, stream);
+        int rc = ts2_normalize_vecs_row_max_dither(len, lenRound, grad, gradType, gradColScale, &buf->grad8, buf->grad8RowScale, buf->gradRowAbsMax,
+            buf->ditherSeed, stream);
         if (rc) {
             return rc;
         }
@@ -180,18 +181,18 @@ extern "C" int ts2_matmul_backprop_delta(int32_t mode, int32_t len, int32_t lenR
                 return rc;
             }
             rc = Ts2TransposeQuantRows(len, lenRound, grad, gradType, srcRowScale, nullptr, buf->gradRowAbsMax, kTile, buf->rowOrder, &buf->gradT,
-                TS2_I8, buf->tileScale, stream);
+                TS2_I8, buf->tileScale, stream, buf->ditherSeed);
         } else if (buf->gradRowAbsMax && buf->gradRowAbsMaxValid) {
             // the k-tile maxima follow from the row maxima of the dX pass: the transposing quantiser forms them itself
             rc = Ts2TransposeQuantRows(len, lenRound, grad, gradType, srcRowScale, nullptr, buf->gradRowAbsMax, kTile, nullptr, &buf->gradT, TS2_I8,
-                buf->tileScale, stream);
+                buf->tileScale, stream, buf->ditherSeed);
         } else {
             rc = ts2_tile_absmax(len, grad, gradType, srcRowScale, kTile, buf->tileMax, 1, stream);
             if (rc) {
                 return rc;
             }
-            rc = ts2_transpose_quant(len, lenRound, grad, gradType, srcRowScale, buf->tileMax, kTile, nullptr, &buf->gradT, TS2_I8, buf->tileScale,
-                stream);
+            rc = ts2_transpose_quant_dither(len, lenRound, grad, gradType, srcRowScale, buf->tileMax, kTile, nullptr, &buf->gradT, TS2_I8, buf->tileScale,
+                buf->ditherSeed, stream);
         }
         if (rc) {
             return rc;

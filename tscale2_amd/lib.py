@@ -234,7 +234,8 @@ class BwdBuffers(C.Structure):
     _fields_ = [("grad8", Mat), ("grad8RowScale", C.c_void_p), ("gradT", Mat), ("srcT", Mat), ("tileMax", C.c_void_p), ("tileScale", C.c_void_p),
                 ("transformT", Mat), ("partial", Mat), ("splits", C.c_int32), ("gradRowAbsMax", C.c_void_p),
                 ("gradRowAbsMaxValid", C.c_int32), ("srcTValid", C.c_int32), ("gradTValid", C.c_int32), ("transformTValid", C.c_int32),
-                ("rowOrder", C.c_void_p), ("rowOrderTmp", C.c_void_p), ("sortRows", C.c_int32), ("padRowsZero", C.c_int32)]
+                ("rowOrder", C.c_void_p), ("rowOrderTmp", C.c_void_p), ("sortRows", C.c_int32), ("padRowsZero", C.c_int32),
+                ("ditherSeed", C.c_uint32)]
 
 
 class MatMulBuffers:
@@ -345,7 +346,7 @@ class ModelConfig(C.Structure):
     _fields_ = [("mode", C.c_int32), ("dim", C.c_int32), ("headCount", C.c_int32), ("ffnDim", C.c_int32), ("expertDim", C.c_int32),
                 ("expertCount", C.c_int32), ("moeSelected", C.c_int32), ("depth", C.c_int32), ("layerType", C.c_void_p),
                 ("layerAttId", C.c_void_p), ("layerSlope", C.c_void_p), ("attTypeCount", C.c_int32), ("vocab", C.c_int32),
-                ("labelCount", C.c_int32), ("maxLen", C.c_int32), ("kTile", C.c_int32), ("recompute", C.c_int32)]
+                ("labelCount", C.c_int32), ("maxLen", C.c_int32), ("kTile", C.c_int32), ("recompute", C.c_int32), ("ditherSeed", C.c_uint32)]
 
 
 class AddGradientParams(C.Structure):
@@ -359,7 +360,7 @@ class Model:
     """Step driver object of the library (ts2_model_*): owns device buffers, runs forward / backprop of a layer stack."""
 
     def __init__(self, mode, dim, heads, ffn_dim, layer_type, layer_att_id, layer_slope, att_type_count, vocab, label_count, max_len,
-                 expert_dim=0, expert_count=0, moe_selected=0, k_tile=0, recompute=False):
+                 expert_dim=0, expert_count=0, moe_selected=0, k_tile=0, recompute=False, dither_seed=0):
         import numpy as np
         self.lib = load()
         dll = self.lib.dll
@@ -368,7 +369,7 @@ class Model:
         self._la = np.ascontiguousarray(layer_att_id, np.int32)
         self._ls = np.ascontiguousarray(layer_slope, np.float32)
         cfg = ModelConfig(mode, dim, heads, ffn_dim, expert_dim, expert_count, moe_selected, len(self._lt), self._lt.ctypes.data,
-                          self._la.ctypes.data, self._ls.ctypes.data, att_type_count, vocab, label_count, max_len, k_tile, int(recompute))
+                          self._la.ctypes.data, self._ls.ctypes.data, att_type_count, vocab, label_count, max_len, k_tile, int(recompute), dither_seed)
         self.h = dll.ts2_model_create(C.byref(cfg))
         if not self.h:
             raise RuntimeError("ts2_model_create failed")
