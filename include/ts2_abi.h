@@ -225,8 +225,9 @@ int ts2_normalize_vecs_row_max_dither(int32_t len, int32_t lenRound, const ts2_m
 /* HistSortFloatsStableKernel, src/lib/cuda/cuda_sort.cu:115-186 (SortPositiveFloatsApproxStable as BackpropMulti calls it on the row
  * scales of the gradient, src/gpt/compute/matmul_fwdbwd.cuh:325): order[0..len) = the rows sorted ascending by the top 13 bits (sign,
  * exponent, four mantissa bits) of key[t] = rowAbsMax[t] * |rowMult[t]| (rowMult optional); rows that share those bits come in
- * descending row order, as in the reference (whose own test holds the hash of that order).  Deterministic.  tmp: len ints of scratch.
- * (The reference sorts fewer than 500 values exactly instead; here every length takes the histogram order.) */
+ * descending row order, as in the reference (whose own test holds the hash of that order).  len < 500: the exact order the reference
+ * takes there (PerformRegularSort, cuda_sort.cu:50-60,117-120): ascending by the whole key, equal keys in ascending row order.
+ * Deterministic.  tmp: len ints of scratch. */
 int ts2_sort_rows_by_scale(int32_t len, const float *rowAbsMax, const float *rowMult, int32_t *order, int32_t *tmp, void *stream);
 
 /* Per-k-tile abs-max of a [len][dim] matrix (optionally times rowMult[t]): tileMax[t/kTile] = max |src|, the first half of
@@ -448,7 +449,10 @@ int ts2_moe_route(int32_t len, int32_t lenMoe, int32_t experts, int32_t selected
  * TS2_MOE_ROUTE_STATIC_INTS ints (512 KiB) held by every GPU the library runs on until the process ends.  A call needs
  * ceil(len*selected/256) * experts <= TS2_MOE_ROUTE_STATIC_INTS (e.g. 65536 tokens, top-2, 64 experts: 32768) and returns TS2_ERR_SHAPE
  * beyond that.  The call allocates and frees nothing.  All calls on one GPU share that GPU's array: calls that may overlap on one GPU
- * (different streams, different host threads) race and must be ordered by the caller. */
+ * (different streams, different host threads) race and must be ordered by the caller.
+ * The first call on a device also resolves the array's address there and sets a kernel's LDS attribute; neither is a stream
+ * operation and neither belongs under stream capture.  ts2_device_info (and with it ts2_model_create) does both for the current
+ * device: call one of them, or make one eager call of this entry point, on each device before a capture that contains it. */
 #define TS2_MOE_ROUTE_STATIC_INTS 131072
 int ts2_moe_route_static(int32_t len, int32_t lenMoe, int32_t experts, int32_t selected, const ts2_mat *select, int32_t selectType,
     const ts2_moe_tables *tables, void *stream);
@@ -538,7 +542,10 @@ int ts2_opt_convert(const ts2_opt_matrix *m, void *stream);
 /* TAgpuCudaModelMatrix::AddDelta(TCudaPackedDeltaMatrix&, bm) with ApplyGradientImpl, agpu_cuda.cuh:484-590, on one device (its
  * all-reduces over devices drop out): backpropMode = TS2_BM_GRAD_ADD adds the delta to `grad`, otherwise it replaces it;
  * TS2_BM_GRAD_APPLY then updates the dispersion estimates, the moving average, the weights and the fast weights.  APPLY without ADD
- * reads the packed bytes directly and leaves `grad` untouched. */
+ * reads the packed bytes directly: `grad` is neither read nor written and may be an empty ts2_mat.  The reference leaves the unpacked
+ * delta in Grad on that path too (UnpackDeltaKernel<0>, agpu_cuda.cuh:579-585); here `grad` holds valid data only after a call with
+ * TS2_BM_GRAD_ADD or one without TS2_BM_GRAD_APPLY, so a caller that reads it, or mixes this call with ts2_unpack_delta /
+ * ts2_add_gradient on the same state, must use one of those. */
 int ts2_opt_add_delta(const ts2_opt_matrix *m, const ts2_mat *delta, const ts2_mat *tileScale, int32_t backpropMode,
     const ts2_add_gradient_params *params, void *stream);
 
@@ -673,7 +680,8 @@ int ts2_checkpoint_matrix(const ts2_checkpoint *c, int32_t layer, int32_t matrix
 int64_t ts2_pack_matrix_fp16(const float *matr, int32_t xSize, int32_t ySize, void *out, int64_t cap);
 int ts2_add_packed_matrix_fp16(float *matr, int32_t xSize, int32_t ySize, const void *in, int64_t size, float scale);
 
-/* peak dense MFMA rate the library prices its kernels against, in T(FL)OP/s, and the CU count it tiles for */
+/* CU count and nominal clock of the current device.  Also the library's per-device set-up call: it resolves what
+ * ts2_moe_route_static would otherwise resolve on its first call on this device (see there). */
 int ts2_device_info(int *cuCount, int *clockMHz);
 
 const char *ts2_version(void);

@@ -341,13 +341,15 @@ def test_row_sort_reproduces_the_reference_order(L, orc):
     got = _sort_dev(L, x)
     assert orc.lib.orc_sort_result_hash(_ptr(np.ascontiguousarray(got)), x.size) == 1749808112
     r = np.random.default_rng(31)
-    for n in (1, 63, 700, 5000, 32768, 70001):
+    for n in (1, 2, 63, 499, 500, 700, 5000, 32768, 70001):
         key = np.exp(r.standard_normal(n) * 3).astype(np.float32)
         key[r.random(n) < 0.05] = 0                                            # zero rows sort first
+        if n > 40:
+            key[30:40] = key[7]                                                # equal keys: ascending rows below 500, descending from 500 on
         mult = (r.standard_normal(n) * 2).astype(np.float32) if n % 2 else None  # the key is |mult| * max
         eff = key if mult is None else (key * np.abs(mult)).astype(np.float32)
         want = np.zeros(n, np.int32)
-        orc.lib.orc_hist_sort_stable(_ptr(eff), n, _ptr(want), 1)
+        orc.lib.orc_hist_sort_stable(_ptr(eff), n, _ptr(want), 0)           # fewer than 500: the exact sort, as in the reference
         np.testing.assert_array_equal(_sort_dev(L, key, mult), want)
 
 

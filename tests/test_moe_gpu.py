@@ -172,3 +172,120 @@ def test_gate_and_norm_backward_over_grouped_rows_matches_the_cpu_layer(lib, gra
         assert (err <= 4.2e-3 * np.abs(want[live]) + 2e-5 * np.abs(want[live]).max()).all(), (what, err.max())
     np.testing.assert_allclose(got_w[live], grad_moe[live, 0], rtol=2e-5, atol=2e-5 * np.abs(grad_moe).max())
     assert (got_vals[5, 128:256] == 0).all()
+
+
+def offset_view(t, elems=4):
+    """the same values at a base address that is 8 bytes off a 16-byte boundary: the entry points then take their four-element kernels"""
+    rows, cols = t.shape
+    buf = torch.zeros((rows, cols + 2 * elems), dtype=t.dtype, device=t.device)
+    view = buf[:, elems:elems + cols]
+    view.copy_(t)
+    assert view.data_ptr() % 16 == 8 and (view.stride(0) * view.element_size()) % 16 == 0
+    return view
+
+
+def e4m3_steps(orc, a, b):
+    """distance of two arrays of e4m3 codes in grid steps (positions on the sorted grid of the 254 finite values)"""
+    tab = orc.e4m3_table(hw=True).astype(np.float64)
+    fin = np.isfinite(tab)
+    order = np.full(256, -1, np.int64)
+    vals = np.unique(tab[fin])
+    order[fin] = np.searchsorted(vals, tab[fin])
+    assert (order[a] >= 0).all() and (order[b] >= 0).all()
+    return np.abs(order[a] - order[b])
+
+
+@pytest.mark.parametrize("X", [256, 1024])
+def test_lolu_moe_e4m3_sixteen_wide_kernel_equals_the_four_wide_kernel(lib, X):
+    """ts2_matrix_lolu_moe with an e4m3 result and 16-byte aligned operands runs the kernel of sixteen elements per lane; the same values
+    at an address 8 bytes off run the four-element kernel, itself checked against MatrixLoLUmoe of the CPU layer by the model tests.
+    Same arithmetic per element: the codes are equal."""
+    L = lib
+    len_, E, K = 700, 64, 2
+    print("case moe lolu e4m3", X, flush=True)
+    _, t, tb, len_moe, host = route(L, len_, E, K, 31)
+    r = np.random.default_rng(32)
+    gate = torch.from_numpy((r.standard_normal((len_moe, X)) * 1.5).astype(np.float32)).cuda().bfloat16()
+    vals = torch.from_numpy((r.standard_normal((len_moe, X)) * 24).astype(np.float32)).cuda().bfloat16()
+    fast = torch.full((len_moe, X), 0x55, dtype=torch.uint8, device="cuda")
+    slow = torch.full((len_moe, X), 0x55, dtype=torch.uint8, device="cuda")
+    L.call("ts2_matrix_lolu_moe", len_moe, t["sw"], gate, vals, 0.75, fast, L.E4M3)
+    L.call("ts2_matrix_lolu_moe", len_moe, t["sw"], offset_view(gate), offset_view(vals), 0.75, slow, L.E4M3)
+    torch.cuda.synchronize()
+    f, s = fast.cpu().numpy(), slow.cpu().numpy()
+    live = host["sid"] >= 0
+    assert np.array_equal(f, s)
+    assert (f[~live] == 0).all() and (f[live] != 0).mean() > 0.9
+    # and the values: vals * sigmoid(2 gate) * weight * 0.75, rounded to e4m3 (half a step of three mantissa bits)
+    orc = Oracle()
+    got = orc.e4m3_table(hw=True)[f[live]]
+    g = gate.float().cpu().numpy()[live]; v = vals.float().cpu().numpy()[live]
+    want = np.clip(v / (1 + np.exp(-2 * g.astype(np.float64))) * host["sw"][live][:, None] * 0.75, -448, 448)  # the conversion saturates
+    assert (np.abs(got - want) <= np.abs(want) * 2.0 ** -4 + 2.0 ** -10).all()
+
+
+@pytest.mark.parametrize("X", [256, 1024])
+def test_gate_and_norm_backward_e4m3_wave_kernel_equals_the_generic_kernel(lib, X):
+    """bf16 gradient in, e4m3 out (the fp8 model's types) runs the wave-per-row kernel; X = 1024 takes its tile loop twice, X = 256 leaves
+    half of each wave without a tile.  The same values at an address 8 bytes off run the generic kernel (checked against the CPU layer
+    above).  Per element the same arithmetic; the two 128-element tile sums are formed in a different order, so a code may move by one
+    step where a value sits on a rounding boundary, and the routing-weight gradient agrees to fp32 summation noise."""
+    L = lib
+    orc = Oracle()
+    len_, E, K = 700, 64, 2
+    print("case moe gate/norm backward e4m3", X, flush=True)
+    _, t, tb, len_moe, host = route(L, len_, E, K, 33)
+    r = np.random.default_rng(34)
+    tiles = X // 128
+    vals16 = torch.from_numpy((r.standard_normal((len_moe, X)) * 24).astype(np.float32)).cuda().bfloat16()
+    vals16[7, 128:256] = 0  # a zero tile
+    gate16 = torch.from_numpy((r.standard_normal((len_moe, X)) * 1.5).astype(np.float32)).cuda().bfloat16()
+    grad = torch.from_numpy((r.standard_normal((len_moe, X)) * 16).astype(np.float32)).cuda().bfloat16()
+    tsc = torch.from_numpy(np.exp(r.standard_normal((tiles, len_moe))).astype(np.float32)).cuda()
+    outs = []
+    for off in (False, True):
+        d_gate = torch.full((len_moe, X), 0x55, dtype=torch.uint8, device="cuda"); d_vals = torch.full_like(d_gate, 0x55)
+        dxw = torch.full((len_moe,), 9.0, device="cuda")
+        g, v, gr = (offset_view(x) if off else x for x in (gate16, vals16, grad))
+        L.call("ts2_backprop_row_tile_normalize_lolu_moe", len_moe, t["sw"], g, v, float(VEC), tsc, gr, L.BF16, 0.5, d_gate, d_vals, L.E4M3, dxw)
+        torch.cuda.synchronize()
+        outs.append((d_gate.cpu().numpy(), d_vals.cpu().numpy(), dxw.cpu().numpy()))
+    (fg, fv, fw), (sg, sv, sw) = outs
+    live = host["sid"] >= 0
+    assert (fg[~live] == 0).all() and (fv[~live] == 0).all() and (fw[~live] == 0).all()
+    assert np.array_equal(fg, sg)                      # no reduction enters the gate gradient
+    steps = e4m3_steps(orc, fv, sv)
+    assert steps.max() <= 1 and (steps != 0).mean() < 2e-3, (steps.max(), (steps != 0).mean())
+    assert (fv[7, 128:256] == 0).all() and (fv[live] != 0).mean() > 0.9
+    np.testing.assert_allclose(fw, sw, rtol=2e-5, atol=2e-5 * np.abs(sw).max())
+
+
+@pytest.mark.parametrize("selected", [5, 6])
+def test_combine_experts_bf16_beyond_four_slots(lib, selected):
+    """bf16 grouped rows, more than four selected experts: the eight-element kernel gathers the slots in batches of four and takes a
+    second batch.  The sum is in slot order, as numpy's."""
+    L = lib
+    len_, E, dim = 900, 16, 512
+    print("case moe combine bf16 slots", selected, flush=True)
+    _, t, tb, len_moe, host = route(L, len_, E, selected, 35)
+    r = np.random.default_rng(36)
+    src = torch.from_numpy(r.standard_normal((len_moe, dim)).astype(np.float32)).cuda().bfloat16()
+    srcf = src.float().cpu().numpy()
+    res0 = r.standard_normal((len_, dim)).astype(np.float32)
+    alpha = np.float32(0.37)
+    ap = torch.tensor([1.5], device="cuda")
+    s = alpha * np.float32(1.5)
+    for add in (0, 1):
+        res = torch.from_numpy(res0.copy()).cuda()
+        L.call("ts2_combine_experts", len_, selected, src, L.BF16, C.byref(tb), float(alpha), ap, res, add)
+        res4 = torch.from_numpy(res0.copy()).cuda()
+        L.call("ts2_combine_experts", len_, selected, offset_view(src), L.BF16, C.byref(tb), float(alpha), ap, res4, add)
+        torch.cuda.synchronize()
+        want = np.zeros((len_, dim), np.float32)
+        for k in range(selected):
+            want = want + srcf[host["row"][:, k]]
+        want = want * s
+        if add:
+            want = want + res0
+        assert np.array_equal(res.cpu().numpy(), want), add
+        assert np.array_equal(res4.cpu().numpy(), want), add

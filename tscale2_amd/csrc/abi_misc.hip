@@ -1,5 +1,6 @@
 // Library-level queries of the C ABI.
 #include "common.h"
+#include "internal.h"
 
 extern "C" int ts2_device_info(int *cuCount, int *clockMHz)
 {
@@ -17,7 +18,8 @@ extern "C" int ts2_device_info(int *cuCount, int *clockMHz)
     if (clockMHz) {
         *clockMHz = prop.clockRate / 1000;
     }
-    return TS2_OK;
+    // the library's per-device set-up that is not stream work, so that no later entry point has to do it under a caller's capture
+    return Ts2MoeRouteSetup();
 }
 
 extern "C" const char *ts2_version(void)

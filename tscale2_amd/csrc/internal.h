@@ -17,3 +17,5 @@ int Ts2FillFloats(float *p, int n, float v, void *stream);
 // ts2_transpose_quant with the k-tile maxima formed in the kernel from row maxima (rowAbsMax) when tileMax is null
 int Ts2TransposeQuantRows(int len, int lenRound, const ts2_mat *src, int srcType, const float *rowMult, const float *tileMax, const float *rowAbsMax,
     int kTile, const int *rowIndex, const ts2_mat *dstT, int dstType, float *tileScale, void *stream, uint32_t ditherSeed = 0);
+// resolves, for the current device, what ts2_moe_route_static otherwise resolves on its first call there (no stream operation)
+int Ts2MoeRouteSetup();

@@ -567,6 +567,13 @@ bool TablesOk(const ts2_moe_tables *t)
 
 // Routing tables from the select logits; blockCounts is the counting sort's scratch: [ceil(len*selected/RB)][experts] ints, every entry in
 // use written by MoeLocalRank before it is read, so it needs no clearing between calls.
+// the dynamic LDS size MoeOffsets may ask for (a function attribute, set once; not a stream operation)
+static bool MoeOffsetsLdsReady()
+{
+    static std::atomic<bool> attrDone{false};
+    return Ts2SetDynamicLds(attrDone, (const void *)MoeOffsets, 150 * 1024);
+}
+
 static int MoeRoute(int32_t len, int32_t lenMoe, int32_t experts, int32_t selected, const ts2_mat *select, int32_t selectType,
     const ts2_moe_tables *tb, int *blockCounts, void *stream)
 {
@@ -586,8 +593,7 @@ static int MoeRoute(int32_t len, int32_t lenMoe, int32_t experts, int32_t select
     TS2_CHECK_LAUNCH();
     const size_t tableBytes = (size_t)nBlocks * experts * 4;
     const int useLds = tableBytes <= 150 * 1024;
-    static std::atomic<bool> attrDone{false};
-    if (!Ts2SetDynamicLds(attrDone, (const void *)MoeOffsets, 150 * 1024)) {
+    if (!MoeOffsetsLdsReady()) {
         return TS2_ERR_LAUNCH;
     }
     hipLaunchKernelGGL(MoeOffsets, dim3(1), dim3(1024), useLds ? tableBytes : 0, STREAM, nBlocks, experts, lenMoe, blockCounts, tb->expertOffset,
@@ -649,6 +655,14 @@ int *MoeRouteScratch()
     return p;
 }
 } // namespace
+
+// Everything ts2_moe_route_static does on its first call on a device that is not a stream operation (the scratch symbol's address, which
+// loads the code object and registers the array, and MoeOffsets' LDS attribute), for callers that make that first call under stream
+// capture: ts2_device_info runs it for the current device.
+int Ts2MoeRouteSetup()
+{
+    return MoeRouteScratch() && MoeOffsetsLdsReady() ? TS2_OK : TS2_ERR_LAUNCH;
+}
 
 extern "C" int ts2_moe_route_static(int32_t len, int32_t lenMoe, int32_t experts, int32_t selected, const ts2_mat *select, int32_t selectType,
     const ts2_moe_tables *tb, void *stream)

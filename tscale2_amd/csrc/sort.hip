@@ -7,6 +7,10 @@
 // least-significant-digit radix passes (6 + 7 bits) over the rows taken in reverse order; a wave owns a contiguous run of positions,
 // ranks equal digits inside a 64-lane step with ballots and keeps per-(wave, digit) running offsets in LDS, so the result is
 // deterministic and independent of atomic ordering.  About 20 microseconds for 32768 rows.
+//
+// Fewer than 500 rows: the reference sorts exactly instead (PerformRegularSort, cuda_sort.cu:50-60,117-120: ascending by value, equal
+// values by ascending row, a strict total order, so its sorting network has one possible result).  Here each row counts the rows that
+// precede it in that order.
 #include "common.h"
 
 namespace
@@ -89,6 +93,31 @@ __device__ __forceinline__ void RadixPass(int len, const float *rowAbsMax, const
     }
 }
 
+constexpr int SORT_EXACT_BELOW = 500;
+
+__global__ void __launch_bounds__(512) ExactSortRows(int len, const float *rowAbsMax, const float *rowMult, int *order)
+{
+    __shared__ uint32_t key[512];
+    const int tid = threadIdx.x;
+    if (tid < len) {
+        float v = rowAbsMax[tid];
+        if (rowMult) {
+            v *= fabsf(rowMult[tid]);
+        }
+        key[tid] = __float_as_uint(fabsf(v)); // non-negative floats order as their bits
+    }
+    __syncthreads();
+    if (tid < len) {
+        const uint32_t mine = key[tid];
+        int rank = 0;
+        for (int j = 0; j < len; ++j) {
+            const uint32_t other = key[j];
+            rank += other < mine || (other == mine && j < tid);
+        }
+        order[rank] = tid;
+    }
+}
+
 __global__ void __launch_bounds__(SORT_THREADS) HistSortRows(int len, const float *rowAbsMax, const float *rowMult, int *order, int *tmp)
 {
     __shared__ int cnt[SORT_WAVES * 128];
@@ -107,6 +136,11 @@ extern "C" int ts2_sort_rows_by_scale(int32_t len, const float *rowAbsMax, const
     }
     if (len <= 0) {
         return TS2_ERR_SHAPE;
+    }
+    if (len < SORT_EXACT_BELOW) {
+        hipLaunchKernelGGL(ExactSortRows, dim3(1), dim3(512), 0, (hipStream_t)stream, len, rowAbsMax, rowMult, order);
+        TS2_CHECK_LAUNCH();
+        return TS2_OK;
     }
     hipLaunchKernelGGL(HistSortRows, dim3(1), dim3(SORT_THREADS), 0, (hipStream_t)stream, len, rowAbsMax, rowMult, order, tmp);
     TS2_CHECK_LAUNCH();
