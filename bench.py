@@ -548,7 +548,7 @@ def bench_att_bwd(args):
     pairs = B * H * (S * (S - 1) / 2)
     flop5 = 5 * 2.0 * pairs * 128
     roof = {"bound": "mfma", "achieved": flop5 / (ms * 1e-3) / 1e12, "peak": PEAK_BF16 / 1e12, "unit": "TFLOP/s", "frac": flop5 / (ms * 1e-3) / PEAK_BF16,
-            "traffic": None, "kernel": "AttGradQ + AttGradKV, 5-product causal count (7 products executed)"}
+            "traffic": None, "kernel": "AttGradQ + AttGradKV, 5-product causal count (7 products executed: S and dP once per kernel)"}
     out = {"metric": "attention backward tokens/sec on 1 MI355X; TFLOPS as % of MFMA peak", "value": n / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1,
            "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": "bf16", "data": "synthetic", "config": {"workload": "causal attention backward, 16 x 2048 tokens, 16 heads x 128, bf16"},

@@ -26,7 +26,7 @@
 //   * the wave's own rows (the B operands of the products that contract over d) stay in registers for the whole kernel, so every
 //     MFMA costs one 1 KB operand fetch from LDS.  With that every kernel fits 256 registers and 64-70 KB of LDS: two workgroups share
 //     a CU (the exponentials and conversions of one run between the products of the other), where one wave per SIMD waits out every
-//     LDS and MFMA latency itself.  The dK/dV kernel gets there by giving dK and dV to different waves.
+//     LDS and MFMA latency itself.  The dK/dV kernel gets there by giving dK and dV to different waves, which hand P over in LDS.
 //   * the register budget shapes the control flow: blocks of 32 rows that a wave does not see are skipped by loops of no trips, not
 //     by branches (the join after a branch makes the compiler copy the 64 accumulator registers); the two tile buffers are two
 //     copies of the code in one loop body (an operand fetch names its LDS array, so it never waits for the loads in flight into the
@@ -636,11 +636,48 @@ __device__ __forceinline__ int Half32MaxInt(int v)
 }
 
 // dK, dV: grid (lenRound/64, heads).  The workgroup owns 64 key rows and streams the query rows that reach them; its four waves are
-// two key blocks x two roles: one wave of a block accumulates dV^T += dO^T P (it needs S only), the other dK^T += Q^T dS (S and dP).
-// Both accumulators of a key block in one wave would need 128 registers and leave room for one wave per SIMD only; split, the kernel
-// recomputes S once more but runs two workgroups per CU.
+// two key blocks x two roles.  Both accumulators of a key block in one wave would need 128 registers and leave room for one wave per
+// SIMD only; split over two waves, the kernel runs two workgroups per CU, and the two waves share the four products evenly: the dV
+// wave forms S = Q K^T and the probabilities P and accumulates dV^T += dO^T P; the dK wave forms dP = dO V^T, takes P from the dV wave
+// through LDS (fp32, the very values it would have computed itself), forms dS and accumulates dK^T += Q^T dS.
+//
+// Hand-over of a 32 x 32 block of P (4 KB per key block, one slot): two counters in LDS per key block, `ready` = number of blocks
+// written by the dV wave, `taken` = number of blocks read by the dK wave.  The dV wave writes block n after taken >= n - 1 and then
+// sets ready = n; the dK wave reads block n after ready >= n and then sets taken = n.  A wave's LDS operations complete in the order
+// it issues them, so a counter is never seen before the data it covers.  Both waves of a pair skip the same blocks (the test
+// depends on the pair's keys and the tile's bounds only), so they count the same blocks; neither wait depends on anything the
+// waiting wave still has to do, and the tile barrier is reached by both after the same blocks.  The waits are bounded all the same:
+// a wave whose wait runs out stops waiting for the rest of the launch (its results are then wrong, which the tests would show,
+// but every wave finishes).
+__device__ __forceinline__ void WaitCounter(int ldsAddr, int want, int &waiting)
+{
+    if (waiting) {
+        int spins = 1 << 15;
+#pragma unroll 1
+        for (;;) {
+            int v;
+            asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(ldsAddr) : "memory");
+            if (__builtin_amdgcn_readfirstlane(v) >= want) {
+                break;
+            }
+            if (--spins == 0) {
+                waiting = 0;
+                break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+        }
+    }
+}
+
+__device__ __forceinline__ void SetCounter(int ldsAddr, int value)
+{
+    asm volatile("ds_write_b32 %0, %1" : : "v"(ldsAddr), "v"(value) : "memory");
+}
+
 template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGradKV(AttP p)
 {
+    __shared__ __attribute__((aligned(16))) float pBlock[2][4][64][4]; // [key block][quarter][lane][4 values]: P of the block in hand
+    __shared__ int pCount[2][2];                                          // [key block][ready, taken]
     __shared__ __attribute__((aligned(1024))) uint8_t qT0[TILE_BYTES], qT1[TILE_BYTES], oT0[TILE_BYTES], oT1[TILE_BYTES];
     __shared__ __attribute__((aligned(16))) float rawStat[2][4][TR];  // [slot][L, dScale, span start, span finish][query], as loaded
     // [slot][-L - slope * (q - keyBase), -dScale * attDotScale * ln2, span start (0x7fffffff if empty), span length][query]: one array,
@@ -658,6 +695,9 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
     const int qLo = p.revLo[block >> 1], qHi = p.revHi[block >> 1];
     const int tFirst = qHi >= qLo ? (qLo / TR) * TR : 1;
     const uint8_t *gq = p.q + hoff, *go = p.dO + hoff;
+    if (tid < 4) {
+        (&pCount[0][0])[tid] = 0; // visible to every wave after the first tile's barrier
+    }
     auto loadStats = [&](int t0, int slot) __attribute__((always_inline)) {
         if (wave == 0) {
             const int lane = FreshLaneId();
@@ -709,10 +749,11 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
     // operand fetch names the LDS array it reads (a fetch through a selected pointer would have to wait for the loads in flight)
     auto run = [&](auto roleTag) __attribute__((always_inline)) {
         constexpr int ROLE = decltype(roleTag)::value;
-        v8bf kf[8], vf[ROLE ? 8 : 1];
-        LoadOwnFrags(kf, p.k + (int64_t)(myRow - l32) * p.ldk + hoff, p.ldk, l32, half);
+        v8bf own[8]; // the wave's keys as B operands: K for S (dV wave), V for dP (dK wave)
         if constexpr (ROLE) {
-            LoadOwnFrags(vf, p.v + (int64_t)(myRow - l32) * p.ldv + hoff, p.ldv, l32, half);
+            LoadOwnFrags(own, p.v + (int64_t)(myRow - l32) * p.ldv + hoff, p.ldv, l32, half);
+        } else {
+            LoadOwnFrags(own, p.k + (int64_t)(myRow - l32) * p.ldk + hoff, p.ldk, l32, half);
         }
         float zero = 0; // opaque, as in AttGradQ
         asm volatile("" : "+v"(zero));
@@ -724,6 +765,11 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
                 acc[db][e] = zero;
             }
         }
+        // LDS addresses of the pair's block of P (this lane's 16 bytes of quarter 0) and of its two counters
+        v4f *const pMine = (v4f *)&pBlock[wave >> 1][0][lane][0]; // named through the array: known not to be a tile with loads in flight
+        const int readyAddr = (int)(uintptr_t)TS2_LDS_PTR(&pCount[wave >> 1][0]), takenAddr = readyAddr + 4;
+        int blockNo = 0, waiting = 1;
+        asm volatile("" : "+s"(waiting));
         if (tFirst <= qHi) {
             __builtin_amdgcn_s_waitcnt(0x0f70);
             digestStats(tFirst, 0);
@@ -747,49 +793,28 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
                 asm volatile("" : "+s"(trips));
 #pragma unroll 1
                 for (int trip = 0; trip < trips; ++trip) {
-                v16f s, dp;
+                ++blockNo;
+                v16f x; // S (dV wave) or dP (dK wave)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    s[e] = 0;
-                    dp[e] = 0;
+                    x[e] = 0;
                 }
-                const uint8_t *tt = ROLE ? qt2 : ot2; // the tile whose transpose the last product takes
+                const uint8_t *rt = ROLE ? ot2 : qt2; // the tile the first product reads by rows: dO for dP, Q for S
+                const uint8_t *tt = ROLE ? qt2 : ot2; // the tile whose transpose the second product takes: Q^T for dK, dO^T for dV
                 v8bf ft[3];
-                if constexpr (ROLE) {
-                    // S = Q K^T, dP = dO V^T; the operands of step ds + 1 are requested before the products of step ds (this role has
-                    // no registers left for a third set of operands)
-                    v8bf fq[2], fo[2];
-                    fq[0] = FragRow(qt2, 0, 0, fl);
-                    fo[0] = FragRow(ot2, 0, 0, fl);
-#pragma unroll
-                    for (int ds = 0; ds < 8; ++ds) {
-                        if (ds + 1 < 8) {
-                            fq[(ds + 1) & 1] = FragRow(qt2, 0, ds + 1, fl);
-                            fo[(ds + 1) & 1] = FragRow(ot2, 0, ds + 1, fl);
-                        }
-                        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fq[ds & 1], kf[ds], s, 0, 0, 0);
-                        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fo[ds & 1], vf[ds], dp, 0, 0, 0);
-                    }
-                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-#pragma unroll
-                    for (int ds = 0; ds < 7; ++ds) {
-                        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-                        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-                    }
-                    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-                } else {
-                    // S = Q K^T, operands three steps ahead (one product per step)
-                    v8bf fq[4];
+                {
+                    // operands three steps ahead (one product per step)
+                    v8bf fr[4];
 #pragma unroll
                     for (int ds = 0; ds < 3; ++ds) {
-                        fq[ds] = FragRow(qt2, 0, ds, fl);
+                        fr[ds] = FragRow(rt, 0, ds, fl);
                     }
 #pragma unroll
                     for (int ds = 0; ds < 8; ++ds) {
                         if (ds + 3 < 8) {
-                            fq[(ds + 3) & 3] = FragRow(qt2, 0, ds + 3, fl);
+                            fr[(ds + 3) & 3] = FragRow(rt, 0, ds + 3, fl);
                         }
-                        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fq[ds & 3], kf[ds], s, 0, 0, 0);
+                        x = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[ds & 3], own[ds], x, 0, 0, 0);
                     }
                     ft[0] = FragTr(tt, 0, 0, 0, fl);
                     ft[1] = FragTr(tt, 0, 0, 1, fl);
@@ -802,46 +827,61 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
                     __builtin_amdgcn_sched_group_barrier(0x008, 3, 0);
                     __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
                 }
-                // P (dV role) or dS (dK role) from the per-query statistics of the tile
                 float wv[16];
-                const float *ps = &st[slot][0][qb * 32 + half * 4];
+                if constexpr (ROLE == 0) {
+                    // P from the per-query statistics of the tile
+                    const float *ps = &st[slot][0][qb * 32 + half * 4];
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const float4 L4 = *(const float4 *)(ps + g * 8);
-                    const float Ls[4] = {L4.x, L4.y, L4.z, L4.w};
-                    float Ds[4] = {0, 0, 0, 0};
-                    if constexpr (ROLE) {
-                        const float4 D4 = *(const float4 *)(ps + TR + g * 8);
-                        Ds[0] = D4.x; Ds[1] = D4.y; Ds[2] = D4.z; Ds[3] = D4.w;
-                    }
-                    int Ss[4] = {0, 0, 0, 0};
-                    unsigned Ns[4] = {0, 0, 0, 0};
-                    if (!full) {
-                        const int4 S4 = *(const int4 *)(ps + 2 * TR + g * 8);
-                        const int4 N4 = *(const int4 *)(ps + 3 * TR + g * 8);
-                        Ss[0] = S4.x; Ss[1] = S4.y; Ss[2] = S4.z; Ss[3] = S4.w;
-                        Ns[0] = (unsigned)N4.x; Ns[1] = (unsigned)N4.y; Ns[2] = (unsigned)N4.z; Ns[3] = (unsigned)N4.w;
-                    }
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const int e = g * 4 + j;
-                        float w = __builtin_amdgcn_exp2f(fmaf(s[e], p.attDotScale, ALIBI ? Ls[j] + ck : Ls[j]));
+                    for (int g = 0; g < 4; ++g) {
+                        const float4 L4 = *(const float4 *)(ps + g * 8);
+                        const float Ls[4] = {L4.x, L4.y, L4.z, L4.w};
+                        int Ss[4] = {0, 0, 0, 0};
+                        unsigned Ns[4] = {0, 0, 0, 0};
                         if (!full) {
-                            w = (unsigned)(myRow - Ss[j]) <= Ns[j] ? w : 0.f;
+                            const int4 S4 = *(const int4 *)(ps + 2 * TR + g * 8);
+                            const int4 N4 = *(const int4 *)(ps + 3 * TR + g * 8);
+                            Ss[0] = S4.x; Ss[1] = S4.y; Ss[2] = S4.z; Ss[3] = S4.w;
+                            Ns[0] = (unsigned)N4.x; Ns[1] = (unsigned)N4.y; Ns[2] = (unsigned)N4.z; Ns[3] = (unsigned)N4.w;
                         }
-                        wv[e] = ROLE ? w * fmaf(dp[e], gmul, Ds[j]) : w;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const int e = g * 4 + j;
+                            float w = __builtin_amdgcn_exp2f(fmaf(x[e], p.attDotScale, ALIBI ? Ls[j] + ck : Ls[j]));
+                            if (!full) {
+                                w = (unsigned)(myRow - Ss[j]) <= Ns[j] ? w : 0.f;
+                            }
+                            wv[e] = w;
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
                     }
-                    // four queries at a time: without the fence the scheduler runs all sixteen side by side, and their temporaries
-                    // push the role that holds both K and V over its registers
-                    __builtin_amdgcn_sched_barrier(0);
+                    // hand the block over once the previous one has been taken
+                    WaitCounter(takenAddr, blockNo - 1, waiting);
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        pMine[g * 64] = v4f{wv[4 * g], wv[4 * g + 1], wv[4 * g + 2], wv[4 * g + 3]};
+                    }
+                    SetCounter(readyAddr, blockNo);
+                } else {
+                    // dS = P (dP attDotScale ln2 - dScale attDotScale ln2)
+                    WaitCounter(readyAddr, blockNo, waiting);
+                    v4f pw[4];
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        pw[g] = pMine[g * 64];
+                    }
+                    SetCounter(takenAddr, blockNo); // issued after the reads, so carried out after them
+                    const float *ps = &st[slot][1][qb * 32 + half * 4];
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const float4 D4 = *(const float4 *)(ps + g * 8);
+                        wv[4 * g] = pw[g].x * fmaf(x[4 * g], gmul, D4.x);
+                        wv[4 * g + 1] = pw[g].y * fmaf(x[4 * g + 1], gmul, D4.y);
+                        wv[4 * g + 2] = pw[g].z * fmaf(x[4 * g + 2], gmul, D4.z);
+                        wv[4 * g + 3] = pw[g].w * fmaf(x[4 * g + 3], gmul, D4.w);
+                    }
                 }
                 const v8bf wb[2] = {PackB(wv, 0), PackB(wv, 1)};
                 // dV^T += dO^T P, or dK^T += Q^T dS, operands two products ahead
-                if constexpr (ROLE) { // this role had no registers to hold them through the arithmetic above
-                    ft[0] = FragTr(tt, 0, 0, 0, fl);
-                    ft[1] = FragTr(tt, 0, 0, 1, fl);
-                    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-                }
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     if (i + 2 < 8) {
