@@ -73,8 +73,8 @@ enum ts2_epilogue {
  * rowScale  (optional, [m], 16-byte aligned): per-row scale of A applied to the accumulator before the epilogue (the dX kernel).
  * kTileScale (optional, [k/kTile], TS2_I8 only): one scale per kTile contraction rows; each tile's int32 sum is exact and
  *             tiles are added in fp32 in tile order (the dW kernel).  kTile must be a multiple of 128.
- * splitK    : >1 splits the contraction over workgroups; partial sums are added with fp32 atomics (TS2_EPI_ADD semantics on a
- *             C the caller has zeroed, or TS2_EPI_STORE with the library zero-filling first).  1 = deterministic.
+ * splitK    : >1 cuts the contraction into that many slices, each STORED to its own slab of C (splitSlabBytes, below; required:
+ *             partial sums are never added atomically, every result of the library is deterministic).
  * Requirements: k a multiple of 128 (8-bit) or 64 (bf16); m, n multiples of 128; 16-byte aligned rows.
  * Rows >= mLive of C are written as zeros when mLive < m (producers keep pad rows zero, src/lib/cuda/cuda_matmul.cuh:10).
  */
@@ -92,7 +92,7 @@ typedef struct ts2_gemm_args {
     ts2_mat tileScale; /* ROW_TILE_MAXNORM: fp32 [n/128][m] */
     int32_t splitK;
     /* bits 0-1: 0 = choose; 1 = 256x256 workgroup tile; 2 = 128x128; 3 = 256x128 (int8 with kTileScale, fp32 result).
-     * Comparison switches, all off in normal use: bit 2 (4) register-staged loader; bit 3 (8) eight waves per workgroup (256x256
+     * Comparison switches, all off in normal use: bit 2 (4) unused (TS2_ERR_UNSUPPORTED); bit 3 (8) eight waves per workgroup (256x256
      * store/accumulate results; with tile 3: the form BackpropDelta launches); bit 4 (16) two LDS stages instead of the ring on the
      * 256x256 tile (and on the 128x128 tile with TS2_E4M3 operands, which takes the ring from k = 1024 on); bits 5-6 tile-order
      * group 8 / 4 / 2 instead of the automatic choice; bit 7 (128) the ring on the 128x128 tile at any k; bits 9 / 10 (512 / 1024)
@@ -116,7 +116,7 @@ typedef struct ts2_gemm_args {
     int64_t cSlabBytes;
     int64_t tileScaleSlabBytes;
     /* splitK > 1 with splitSlabBytes != 0: slice i of the contraction is STORED to c + i*splitSlabBytes (fp32, TS2_EPI_STORE; slices
-     * are whole k-tiles) instead of being added atomically: deterministic, the caller sums the slices (ts2_pack_delta does). */
+     * are whole k-tiles): deterministic, the caller sums the slices (ts2_pack_delta does).  splitK > 1 without it is refused. */
     int64_t splitSlabBytes;
     /* TS2_EPI_ROW_TILE_NORM */
     int32_t normalize;

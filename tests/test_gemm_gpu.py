@@ -207,10 +207,16 @@ def test_split_k_matches(lib, orc):
     a = r.integers(-16, 17, (m, k), dtype=np.int8)
     b = r.integers(-16, 17, (n, k), dtype=np.int8)
     ref = orc_gemm_i8(orc, a, b).astype(np.float32)  # |sum| < 2^24: every fp32 partial sum is exact
-    tc = torch.full((m, n), 3.0, dtype=torch.float32, device="cuda")
-    lib.gemm_nt(torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(), tc, L.I8, L.F32, split_k=4)
+    ta, tb = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    tc = torch.full((4 * m, n), 3.0, dtype=torch.float32, device="cuda")
+    lib.gemm_nt(ta, tb, tc, L.I8, L.F32, split_k=4, split_slab_bytes=m * n * 4, m=m, n=n, k=k)
     torch.cuda.synchronize()
-    assert np.array_equal(tc.cpu().numpy(), ref)
+    slices = tc.cpu().numpy().reshape(4, m, n)
+    for i in range(4):  # every stored slice is the product over its quarter of the contraction
+        assert np.array_equal(slices[i], orc_gemm_i8(orc, a[:, i * 512:(i + 1) * 512], b[:, i * 512:(i + 1) * 512]).astype(np.float32)), i
+    assert np.array_equal(slices.sum(0), ref)
+    # slices are stored, never added atomically: without a slab the call is refused
+    assert lib.gemm_nt(ta, tb, tc[:m], L.I8, L.F32, split_k=4, check=False) == -3
 
 
 def test_rejects_bad_shapes(lib):

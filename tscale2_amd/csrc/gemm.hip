@@ -8,9 +8,8 @@
 //   * K advances 128 bytes per step; A and B tiles go global -> LDS with global_load_lds_dwordx4, no staging registers and no
 //     ds_write.  GemmNTRing (the 256x256 tile) keeps three stages of A and two of B (all 160 KB of LDS): A is loaded two steps
 //     ahead, B one, one load at a time between the MFMAs.  GemmNTDirect (the other tiles, k-tile scales, expert groups) has two
-//     stages.  Stages are separate static arrays so that operand reads of one never wait for the loads into another.  GemmNT
-//     (tileConfig bit 2, and the atomically accumulated split-K) stages through registers.  In all of them 16-byte chunks are
-//     XOR-swizzled by (row/2)%8: loader writes and ds_read_b128 operand fetches are bank-conflict free;
+//     stages.  Stages are separate static arrays so that operand reads of one never wait for the loads into another.  In all of
+//     them 16-byte chunks are XOR-swizzled by (row/2)%8: the deposited loads and the ds_read_b128 operand fetches are bank-conflict free;
 //   * operand fragments are read one K-slice ahead of the MFMAs that use them (two fragment sets), one barrier per step;
 //   * MFMA: v_mfma_i32_32x32x32_i8, v_mfma_f32_32x32x64_f8f6f4 (fp8 x fp8), v_mfma_f32_32x32x16_bf16;
 //   * workgroup ids are remapped so that each of the 8 XCDs (which receive ids round-robin) works on a compact band of C tiles
@@ -27,243 +26,9 @@ using namespace gemmk;
 namespace
 {
 
-template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT>
-__global__ void __launch_bounds__(256, 1) GemmNT(GemmP p)
-{
-    typedef typename AccT<TYPE>::type TAcc;
-    constexpr int BM = 64 * WTM;
-    constexpr int BN = 64 * WTN;
-    constexpr int LA = BM / 32; // 16-byte loads per thread for the A tile
-    constexpr int LB = BN / 32;
-    constexpr int STAGE = (BM + BN) * BKB;
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int wm = wave >> 1;
-    const int wn = wave & 1;
-
-    int tm, tn;
-    const int tilesMN = p.tilesM * p.tilesN;
-    int bid = blockIdx.x;
-    int split = 0;
-    if (p.splitK > 1) {
-        split = bid / tilesMN;
-        bid -= split * tilesMN;
-    }
-    MapTile(bid, tilesMN, p.tilesM, p.tilesN, &tm, &tn, p.mapGroup ? p.mapGroup : 8);
-    const int rowBase = tm * BM;
-    const int colBase = tn * BN;
-
-    // contraction range of this workgroup
-    int kSteps = p.kBytes / BKB;
-    int kBeg = 0;
-    if (p.tileGroup) {
-        // rows of one 128-row tile belong to one group (BM == 128 is enforced by the host); its B operand is that group's slab
-        int g = p.tileGroup[rowBase / TILE];
-        if (g < 0) {
-            return;
-        }
-        p.b += (int64_t)g * p.bSlab;
-    }
-    if (p.groupOffsets) {
-        // delta of one group: contraction over the group's own rows only
-        int g = blockIdx.y;
-        kBeg = p.groupOffsets[g] * (TYPE == T_BF16 ? 2 : 1) / BKB;
-        kSteps = p.groupOffsets[g + 1] * (TYPE == T_BF16 ? 2 : 1) / BKB - kBeg;
-        p.c += (int64_t)g * p.cSlab;
-        if (p.tileScale) {
-            p.tileScale += (int64_t)g * p.tileScaleSlab;
-        }
-    }
-    if (p.splitK > 1) {
-        int per = (kSteps + p.splitK - 1) / p.splitK;
-        if (KT) {
-            int tileSteps = p.kTileBytes / BKB;
-            per = (per + tileSteps - 1) / tileSteps * tileSteps;
-        }
-        kBeg = split * per;
-        int kEnd = kBeg + per < kSteps ? kBeg + per : kSteps;
-        kSteps = kEnd - kBeg;
-        if (kSteps <= 0) {
-            return;
-        }
-    }
-
-    // global load addressing: thread -> (row = tid/8 + 32*i, 16-byte chunk = tid%8)
-    const int lc = tid & 7;
-    const int lr = tid >> 3;
-    const uint8_t *gaBase = p.a + (int64_t)(rowBase + lr) * p.lda + (int64_t)kBeg * BKB + lc * 16;
-    const uint8_t *gbBase = p.b + (int64_t)(colBase + lr) * p.ldb + (int64_t)kBeg * BKB + lc * 16;
-    v4i ra[LA], rb[LB];
-
-    auto loadGlobal = [&](int step) {
-#pragma unroll
-        for (int i = 0; i < LA; ++i) {
-            ra[i] = *(const v4i *)(gaBase + (int64_t)i * 32 * p.lda + (int64_t)step * BKB);
-        }
-#pragma unroll
-        for (int i = 0; i < LB; ++i) {
-            rb[i] = *(const v4i *)(gbBase + (int64_t)i * 32 * p.ldb + (int64_t)step * BKB);
-        }
-    };
-    auto storeLds = [&](int stage) {
-        uint8_t *sa = lds + stage * STAGE;
-        uint8_t *sb = sa + BM * BKB;
-#pragma unroll
-        for (int i = 0; i < LA; ++i) {
-            *(v4i *)(sa + SwizzleOffset(lr + 32 * i, lc)) = ra[i];
-        }
-#pragma unroll
-        for (int i = 0; i < LB; ++i) {
-            *(v4i *)(sb + SwizzleOffset(lr + 32 * i, lc)) = rb[i];
-        }
-    };
-
-    TAcc acc[WTM][WTN];
-    v16f facc[KT ? WTM : 1][KT ? WTN : 1];
-#pragma unroll
-    for (int i = 0; i < WTM; ++i) {
-#pragma unroll
-        for (int j = 0; j < WTN; ++j) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                acc[i][j][e] = 0;
-            }
-        }
-    }
-    if (KT) {
-#pragma unroll
-        for (int i = 0; i < WTM; ++i) {
-#pragma unroll
-            for (int j = 0; j < WTN; ++j) {
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    facc[i][j][e] = 0;
-                }
-            }
-        }
-    }
-
-    const int half = lane >> 5;
-    const int l32 = lane & 31;
-    const int aRow0 = wm * (32 * WTM) + l32;
-    const int bRow0 = wn * (32 * WTN) + l32;
-
-    // MFMA operand fragments, two register sets: the set of slice s+1 is fetched from LDS while the MFMAs of slice s run
-    constexpr int NS = TYPE == T_FP8 ? 2 : 4; // K slices per step: 64 bytes (f8f6f4 32x32x64) or 32 bytes (i8 32x32x32, bf16 32x32x16)
-    typedef typename std::conditional<TYPE == T_FP8, v8i, v4i>::type TFrag;
-    TFrag fa[2][WTM], fb[2][WTN];
-    auto loadOne = [&](const uint8_t *base, int row, int sl) -> TFrag {
-        if constexpr (TYPE == T_FP8) {
-            int ch = sl * 4 + half * 2;
-            v4i lo = *(const v4i *)(base + SwizzleOffset(row, ch));
-            v4i hi = *(const v4i *)(base + SwizzleOffset(row, ch + 1));
-            return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        } else {
-            return *(const v4i *)(base + SwizzleOffset(row, sl * 2 + half));
-        }
-    };
-    auto mfma = [&](TFrag a, TFrag b, TAcc c) -> TAcc {
-        if constexpr (TYPE == T_I8) {
-            return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
-        } else if constexpr (TYPE == T_FP8) {
-            return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
-        } else {
-            return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
-        }
-    };
-#define LOAD_FRAGS(SET, STAGE, SL)                                                                                                         \
-    do {                                                                                                                                   \
-        const uint8_t *sa_ = lds + (STAGE)*STAGE_BYTES;                                                                                    \
-        const uint8_t *sb_ = sa_ + BM * BKB;                                                                                               \
-        _Pragma("unroll") for (int i = 0; i < WTM; ++i) fa[SET][i] = loadOne(sa_, aRow0 + 32 * i, SL);                                     \
-        _Pragma("unroll") for (int j = 0; j < WTN; ++j) fb[SET][j] = loadOne(sb_, bRow0 + 32 * j, SL);                                     \
-    } while (0)
-#define MFMA_ROWS(SET, I0, I1)                                                                                                             \
-    do {                                                                                                                                   \
-        _Pragma("unroll") for (int i = I0; i < I1; ++i) _Pragma("unroll") for (int j = 0; j < WTN; ++j) acc[i][j] =                        \
-            mfma(fa[SET][i], fb[SET][j], acc[i][j]);                                                                                       \
-    } while (0)
-
-    // main loop: LDS double buffered; global loads of step s+1 are in flight during step s, are written to LDS before the last
-    // slice's MFMAs, the barrier sits in the middle of that slice and the first fragments of step s+1 are fetched behind it
-    constexpr int STAGE_BYTES = STAGE;
-    if (kSteps > 0) {
-        loadGlobal(0);
-        storeLds(0);
-    }
-    __syncthreads();
-    if (kSteps > 0) {
-        LOAD_FRAGS(0, 0, 0);
-    }
-    const int tileSteps = KT ? p.kTileBytes / BKB : 0;
-    for (int s = 0; s < kSteps; ++s) {
-        const int cur = s & 1;
-        const bool more = s + 1 < kSteps;
-        if (more) {
-            loadGlobal(s + 1);
-        }
-#pragma unroll
-        for (int sl = 0; sl < NS - 1; ++sl) {
-            if ((sl & 1) == 0) {
-                LOAD_FRAGS(1, cur, sl + 1);
-                MFMA_ROWS(0, 0, WTM);
-            } else {
-                LOAD_FRAGS(0, cur, sl + 1);
-                MFMA_ROWS(1, 0, WTM);
-            }
-        }
-        // last slice lives in set 1 (NS is even)
-        if (more) {
-            storeLds(cur ^ 1);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        MFMA_ROWS(1, 0, WTM / 2);
-        __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();
-        if (more) {
-            LOAD_FRAGS(0, cur ^ 1, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0); // keep the LDS reads ahead of the remaining MFMAs, which hide their latency
-        MFMA_ROWS(1, WTM / 2, WTM);
-        if (KT) {
-            if ((kBeg + s + 1) % tileSteps == 0 || s + 1 == kSteps) {
-                float sc = p.kTileScale[(kBeg + s) / tileSteps];
-#pragma unroll
-                for (int i = 0; i < WTM; ++i) {
-#pragma unroll
-                    for (int j = 0; j < WTN; ++j) {
-#pragma unroll
-                        for (int e = 0; e < 16; ++e) {
-                            facc[i][j][e] += sc * (float)acc[i][j][e];
-                            acc[i][j][e] = 0;
-                        }
-                    }
-                }
-            }
-        }
-    }
-#undef LOAD_FRAGS
-#undef MFMA_ROWS
-    __syncthreads();
-
-    Epilogue<TYPE, WTM, WTN, CT, EPI, KT>(p, acc, facc, lds, rowBase, colBase, wm, wn, half, l32);
-}
-
-__global__ void ZeroRows(uint8_t *c, int64_t ldc, int rowBytes)
-{
-    uint8_t *row = c + (int64_t)blockIdx.x * ldc;
-    for (int x = threadIdx.x * 4; x < rowBytes; x += blockDim.x * 4) {
-        *(int *)(row + x) = 0;
-    }
-}
-
-
 // ---------------------------------------------------------------------------------------------------------------------------
-// Variant with direct global -> LDS loads (global_load_lds_dwordx4): no staging registers and no ds_write instructions.  A wave-level
-// load deposits 64 x 16 bytes contiguously in LDS, i.e. one block of 8 tile rows; which 16-byte chunk of the row a lane fetches is
+// Two-stage loop with direct global -> LDS loads (global_load_lds_dwordx4): no staging registers and no ds_write instructions.  A
+// wave-level load deposits 64 x 16 bytes contiguously in LDS, i.e. one block of 8 tile rows; which 16-byte chunk of the row a lane fetches is
 // chosen so that the block lands already XOR-swizzled.  The two LDS stages are separate static arrays: the compiler can then prove
 // that the operand reads of one stage do not alias the in-flight loads into the other and does not serialise them.
 
@@ -1104,14 +869,8 @@ template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT> int Launch(const
     GemmP q = p;
     q.tilesM = (p.m + BM - 1) / BM;
     q.tilesN = (p.n + BN - 1) / BN;
-    int ldsBytes = 2 * (BM + BN) * BKB;
-    auto kern = GemmNT<TYPE, WTM, WTN, CT, EPI, KT>;
-    static std::atomic<bool> attrDone{false}; // per instantiation
-    if (!Ts2SetDynamicLds(attrDone, (const void *)kern, ldsBytes)) {
-        return TS2_ERR_LAUNCH;
-    }
-    int nb = q.tilesM * q.tilesN * (p.splitK > 1 ? p.splitK : 1);
-    if (p.direct && p.splitK <= 1) {
+    int nb = q.tilesM * q.tilesN;
+    {
         int gy = p.groupOffsets ? p.splitK_groups : (p.splits > 1 ? p.splits : 1);
         // an XCD runs nb/8 consecutive tiles: group the order so that they cover about as many rows of A as of B
         {
@@ -1165,12 +924,6 @@ template <int TYPE, int WTM, int WTN, int CT, int EPI, bool KT> int Launch(const
         TS2_CHECK_LAUNCH();
         return TS2_OK;
     }
-    if (p.nSeg > 1 || p.kMajor) {
-        return TS2_ERR_UNSUPPORTED;
-    }
-    hipLaunchKernelGGL(kern, dim3(nb, p.groupOffsets ? p.splitK_groups : 1), dim3(256), ldsBytes, stream, q);
-    TS2_CHECK_LAUNCH();
-    return TS2_OK;
 }
 
 // 256x256 tile with 8 waves (2 x 4, wave tile 128x64): two waves per SIMD hide each other's LDS and barrier stalls
@@ -1347,8 +1100,11 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
         return TS2_ERR_UNSUPPORTED; // the row stores address 128 rows of C from one 32-bit offset
     }
     int splitK = a->splitK > 1 ? a->splitK : 1;
-    if (splitK > 1 && (a->cType != TS2_F32 || a->epilogue == TS2_EPI_ROW_TILE_MAXNORM)) {
-        return TS2_ERR_UNSUPPORTED;
+    if (splitK > 1 && !a->splitSlabBytes) {
+        return TS2_ERR_UNSUPPORTED; // slices of the contraction are stored, never added atomically
+    }
+    if (a->tileConfig & 4) {
+        return TS2_ERR_UNSUPPORTED; // was: the register-staged loader
     }
     if (a->epilogue == TS2_EPI_ROW_TILE_MAXNORM && (!a->tileScale.ptr || a->tileScale.y < a->n / 128 || a->tileScale.x < a->m)) {
         return TS2_ERR_SHAPE;
@@ -1424,7 +1180,7 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
         // stored (not atomically added) partial products: needs the direct kernel, fp32 results and slices of whole k-tiles
         int kStepsAll = (int)(((int64_t)a->k * esz) / BKB);
         int per = (kStepsAll + splitK - 1) / splitK;
-        if (splitK <= 1 || a->cType != TS2_F32 || a->epilogue != TS2_EPI_STORE || a->tileGroup || a->groupOffsets || (a->tileConfig & 4) ||
+        if (splitK <= 1 || a->cType != TS2_F32 || a->epilogue != TS2_EPI_STORE || a->tileGroup || a->groupOffsets ||
             (a->kTileScale && (per * BKB) % (a->kTile * esz)) || (a->splitSlabBytes & 7)) {
             return TS2_ERR_UNSUPPORTED;
         }
@@ -1433,7 +1189,6 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
         splitK = 1;
         p.splitK = 1;
     }
-    p.direct = (a->tileConfig & 4) ? 0 : 1; // bit 2 of tileConfig selects the register-staged loader (kept for comparison)
     p.mapGroup = ((a->tileConfig >> 5) & 3) == 1 ? 8 : ((a->tileConfig >> 5) & 3) == 2 ? 4 : ((a->tileConfig >> 5) & 3) == 3 ? 2 : 0;
     p.gridShrink = (a->tileConfig >> 13) & 3;
     p.noRing = (a->tileConfig & 16) ? 1 : 0; // bit 4: two-stage loop instead of the ring for the 256x256 tile (comparison)
@@ -1446,16 +1201,8 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
     // 128x128 tile, e4m3: the ring pipeline from a contraction of eight steps on (measured on the expert-grouped products: 136 -> 120 us
     // at K = 1024, no gain at K = 512); bit 7 of tileConfig asks for it at any length, bit 4 for the two-stage loop
     p.ring128 = !(a->tileConfig & 16) && ((a->tileConfig & 128) || (int64_t)a->k * esz >= 8 * BKB) ? 1 : 0;
-    if ((a->tileGroup || a->groupOffsets) && splitK > 1) {
-        return TS2_ERR_UNSUPPORTED;
-    }
     if (a->groupOffsets && a->groups <= 0) {
         return TS2_ERR_SHAPE;
-    }
-    if (splitK > 1 && a->epilogue == TS2_EPI_STORE) {
-        // partial sums are accumulated with atomics: clear the live rows first (with a fill kernel, which is safe under graph capture)
-        hipLaunchKernelGGL(ZeroRows, dim3(a->m), dim3(256), 0, stream, (uint8_t *)a->c.ptr, (int64_t)a->c.strideBytes, a->n * 4);
-        TS2_CHECK_LAUNCH();
     }
     {
         // the 256x128 kernel for two workgroups per CU: bit 11 of tileConfig asks for it (TS2_ERR_UNSUPPORTED if it cannot run the call)

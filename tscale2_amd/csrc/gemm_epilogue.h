@@ -31,7 +31,6 @@ struct GemmP {
     int64_t cSlab;           // bytes between the C blocks of consecutive groups
     int64_t tileScaleSlab;   // floats
     int splitK_groups;       // number of groups when groupOffsets is set
-    int direct;              // 1: direct global->LDS loader
     int noRing;              // 1: keep the two-stage loop for the 256x256 tile (comparison)
     int kMajor;              // 1: A is [k][m], B is [k][n] (fp8, ring kernel): operands are transposed by the LDS reads
     int streamC;             // results stored with the non-temporal hint
@@ -556,11 +555,7 @@ __device__ __forceinline__ void Epilogue(const GemmP &p, TAcc (&acc)[WTM][WTN], 
                                 float v = live ? accVal(i, j, e) * rs : 0.f;
                                 if constexpr (CT == C_F32) {
                                     float *d = (float *)dst + col;
-                                    if (p.splitK > 1) {
-                                        if (live) {
-                                            atomicAdd(d, v);
-                                        }
-                                    } else if (EPI == TS2_EPI_ADD) {
+                                    if (EPI == TS2_EPI_ADD) {
                                         if (live) {
                                             *d = old[ee][j] + v;
                                         }
