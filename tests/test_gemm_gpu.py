@@ -213,7 +213,7 @@ def test_split_k_matches(lib, orc):
     torch.cuda.synchronize()
     slices = tc.cpu().numpy().reshape(4, m, n)
     for i in range(4):  # every stored slice is the product over its quarter of the contraction
-        assert np.array_equal(slices[i], orc_gemm_i8(orc, a[:, i * 512:(i + 1) * 512], b[:, i * 512:(i + 1) * 512]).astype(np.float32)), i
+        assert np.array_equal(slices[i], orc_gemm_i8(orc, np.ascontiguousarray(a[:, i * 512:(i + 1) * 512]), np.ascontiguousarray(b[:, i * 512:(i + 1) * 512])).astype(np.float32)), i
     assert np.array_equal(slices.sum(0), ref)
     # slices are stored, never added atomically: without a slab the call is refused
     assert lib.gemm_nt(ta, tb, tc[:m], L.I8, L.F32, split_k=4, check=False) == -3
