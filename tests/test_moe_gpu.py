@@ -260,12 +260,13 @@ def test_gate_and_norm_backward_e4m3_wave_kernel_equals_the_generic_kernel(lib, 
     np.testing.assert_allclose(fw, sw, rtol=2e-5, atol=2e-5 * np.abs(sw).max())
 
 
-@pytest.mark.parametrize("selected", [5, 6])
-def test_combine_experts_bf16_beyond_four_slots(lib, selected):
-    """bf16 grouped rows, more than four selected experts: the eight-element kernel gathers the slots in batches of four and takes a
-    second batch.  The sum is in slot order, as numpy's."""
+@pytest.mark.parametrize("selected", [1, 3, 4, 5, 6])
+def test_combine_experts_bf16_slot_counts(lib, selected):
+    """bf16 grouped rows: up to four selected experts take the kernel with four tokens per lane (902 tokens: its last group of four is
+    half empty), more than four the kernel that gathers the slots in batches of four and takes a second batch.
+    The sum is in slot order, as numpy's."""
     L = lib
-    len_, E, dim = 900, 16, 512
+    len_, E, dim = 902 if selected < 5 else 900, 16, 512  # 902: the last group of four tokens is half empty
     print("case moe combine bf16 slots", selected, flush=True)
     _, t, tb, len_moe, host = route(L, len_, E, selected, 35)
     r = np.random.default_rng(36)

@@ -525,6 +525,86 @@ __global__ void __launch_bounds__(256) CombineExperts8(int len, int tiles, int s
     Store4<TF32>(At<TF32>(res, t, col + 4), r1);
 }
 
+// The same for up to KB (<= 4) selected experts with U consecutive tokens per lane: the three dependent loads that lead to a row's
+// data (slot -> expert, expert -> first row, row -> data) are issued for all U tokens side by side, so that U * selected row loads of
+// a lane are in flight together instead of `selected` at the end of one chain.
+template <int U, int KB>
+__global__ void __launch_bounds__(256) CombineExperts8U(int len, int tiles, int selected, Mat src, const int *sampleExpertIds,
+    const int *sampleExpertOffset, const int *expertOffset, float alpha, const float *alphaPtr, Mat res, int add)
+{
+    const long unit = ((long)blockIdx.x * 256 + threadIdx.x) >> 4;
+    const int l16 = threadIdx.x & 15;
+    const long nUnits = (long)((len + U - 1) / U) * tiles;
+    if (unit >= nUnits) {
+        return;
+    }
+    const int t0 = (int)(unit / tiles) * U, tile = (int)(unit % tiles);
+    const int col = tile * TILE + l16 * 8;
+    int ids[U][KB], off[U][KB], row[U][KB];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int k = 0; k < KB; ++k) {
+            const int t = t0 + u < len ? t0 + u : len - 1;
+            const int idx = t * selected + (k < selected ? k : selected - 1);
+            ids[u][k] = sampleExpertIds[idx];
+            off[u][k] = sampleExpertOffset[idx];
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int k = 0; k < KB; ++k) {
+            row[u][k] = expertOffset[ids[u][k]] + off[u][k];
+        }
+    }
+    uint4 v[U][KB];
+    F4 old0[U], old1[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int k = 0; k < KB; ++k) {
+            if (k < selected) {
+                v[u][k] = *(const uint4 *)At<TBF16>(src, row[u][k], col);
+            }
+        }
+        old0[u] = ZeroF4();
+        old1[u] = ZeroF4();
+        if (add && t0 + u < len) {
+            old0[u] = Load4<TF32>(At<TF32>(res, t0 + u, col));
+            old1[u] = Load4<TF32>(At<TF32>(res, t0 + u, col + 4));
+        }
+    }
+    float s = alpha;
+    if (alphaPtr) {
+        s *= *alphaPtr;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        if (t0 + u >= len) {
+            break;
+        }
+        float sum[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int k = 0; k < KB; ++k) {
+            if (k < selected) {
+                const uint32_t w[4] = {v[u][k].x, v[u][k].y, v[u][k].z, v[u][k].w};
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    sum[e] += (e & 1) ? __uint_as_float(w[e >> 1] & 0xffff0000u) : __uint_as_float(w[e >> 1] << 16);
+                }
+            }
+        }
+        F4 r0 = MakeF4(sum[0], sum[1], sum[2], sum[3]) * s, r1 = MakeF4(sum[4], sum[5], sum[6], sum[7]) * s;
+        if (add) {
+            r0 = r0 + old0[u];
+            r1 = r1 + old1[u];
+        }
+        Store4<TF32>(At<TF32>(res, t0 + u, col), r0);
+        Store4<TF32>(At<TF32>(res, t0 + u, col + 4), r1);
+    }
+}
+
 // 128x128 byte-tile transposes over a batch of slabs
 __global__ void __launch_bounds__(256) TransposeU8Batched(const uint8_t *src, int64_t srcStride, int64_t srcSlab, uint8_t *dst, int64_t dstStride,
     int64_t dstSlab)
@@ -802,6 +882,19 @@ extern "C" int ts2_combine_experts(int32_t len, int32_t selected, const ts2_mat 
     long units = (long)len * tiles;
     dim3 grid((unsigned)((units * 32 + 255) / 256));
     if (srcType == TS2_BF16 && Aligned16(src->ptr, src->strideBytes) && Aligned16(res->ptr, res->strideBytes)) {
+        if (selected <= 4) {
+            const long unitsU = (long)((len + 3) / 4) * tiles;
+            const dim3 gridU((unsigned)((unitsU * 16 + 255) / 256));
+            if (selected <= 2) {
+                hipLaunchKernelGGL((CombineExperts8U<4, 2>), gridU, dim3(256), 0, STREAM, len, tiles, selected, M(*src), tb->sampleExpertIds,
+                    tb->sampleExpertOffset, tb->expertOffset, alpha, alphaPtr, M(*res), add);
+            } else {
+                hipLaunchKernelGGL((CombineExperts8U<4, 4>), gridU, dim3(256), 0, STREAM, len, tiles, selected, M(*src), tb->sampleExpertIds,
+                    tb->sampleExpertOffset, tb->expertOffset, alpha, alphaPtr, M(*res), add);
+            }
+            TS2_CHECK_LAUNCH();
+            return TS2_OK;
+        }
         hipLaunchKernelGGL(CombineExperts8, dim3((unsigned)((units * 16 + 255) / 256)), dim3(256), 0, STREAM, len, tiles, selected, M(*src),
             tb->sampleExpertIds, tb->sampleExpertOffset, tb->expertOffset, alpha, alphaPtr, M(*res), add);
     } else if (srcType == TS2_BF16) {
