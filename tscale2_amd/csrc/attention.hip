@@ -688,7 +688,11 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
     int block, head;
     MapAttBlock(&block, &head);
     // co-resident workgroups get opposite role orders, so that a SIMD is not handed two waves of the longer role
-    const int role = (wave ^ (((blockIdx.x + blockIdx.y * gridDim.x) >> 8) & 1)) & 1; // 0: dV, 1: dK
+    const int rolePar = ((blockIdx.x + blockIdx.y * gridDim.x) >> 8) & 1;
+    const int role = (wave ^ rolePar) & 1; // 0: dV, 1: dK
+    // the wave that fetches and digests the per-query statistics of the coming tiles: the dK wave of the first key block, which
+    // spends part of every block waiting for P anyway
+    const int statWave = 1 ^ rolePar;
     const int keyBase = block * KVROWS;
     const int myRow = keyBase + (wave >> 1) * WROWS + l32; // my key
     const int64_t hoff = (int64_t)head * HD * 2;
@@ -699,7 +703,7 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
         (&pCount[0][0])[tid] = 0; // visible to every wave after the first tile's barrier
     }
     auto loadStats = [&](int t0, int slot) __attribute__((always_inline)) {
-        if (wave == 0) {
+        if (wave == statWave) {
             const int lane = FreshLaneId();
             const int64_t so = (int64_t)head * p.ldStat + t0 + lane;
             __builtin_amdgcn_global_load_lds(TS2_GLB_PTR(p.sumWeightLog + so), TS2_LDS_PTR(&rawStat[slot][0][0]), 4, 0, 0);
@@ -708,9 +712,9 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
             __builtin_amdgcn_global_load_lds(TS2_GLB_PTR(p.spanFinish + t0 + lane), TS2_LDS_PTR(&rawStat[slot][3][0]), 4, 0, 0);
         }
     };
-    // wave 0: raw statistics of the tile at t0 (slot) -> the form the products use
+    // the statistics wave: raw statistics of the tile at t0 (slot) -> the form the products use
     auto digestStats = [&](int t0, int slot) __attribute__((always_inline)) {
-        if (wave == 0) {
+        if (wave == statWave) {
             // the lane index is computed afresh: a value kept from the kernel's start would hold registers (or be spilled) across the
             // tile loop for the sake of these few instructions
             const int lane = FreshLaneId(), l32 = lane & 31, half = lane >> 5;
@@ -774,7 +778,106 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
             __builtin_amdgcn_s_waitcnt(0x0f70);
             digestStats(tFirst, 0);
         }
-        // one 64-query tile: the 32-query blocks of which some query sees a key of this wave
+        // ---- pieces of a 32 x 32 block --------------------------------------------------------------------------------------------
+        // first product: S = Q K^T (dV wave) or dP = dO V^T (dK wave), operands three steps ahead
+        auto firstProduct = [&](v16f &x, const uint8_t *rt) __attribute__((always_inline)) {
+            v8bf fr[4];
+#pragma unroll
+            for (int ds = 0; ds < 3; ++ds) {
+                fr[ds] = FragRow(rt, 0, ds, fl);
+            }
+#pragma unroll
+            for (int ds = 0; ds < 8; ++ds) {
+                if (ds + 3 < 8) {
+                    fr[(ds + 3) & 3] = FragRow(rt, 0, ds + 3, fl);
+                }
+                x = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[ds & 3], own[ds], x, 0, 0, 0);
+            }
+        };
+        // dV wave: P from S and the per-query statistics of the tile
+        auto probabilities = [&](const v16f &x, float (&wv)[16], int slot, int qb, auto fullTag) __attribute__((always_inline)) {
+            constexpr bool full = decltype(fullTag)::value; // every query of the block sees every key of the wave: no span tests
+            const float *ps = &st[slot][0][qb * 32 + half * 4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const float4 L4 = *(const float4 *)(ps + g * 8);
+                const float Ls[4] = {L4.x, L4.y, L4.z, L4.w};
+                int Ss[4] = {0, 0, 0, 0};
+                unsigned Ns[4] = {0, 0, 0, 0};
+                if (!full) {
+                    const int4 S4 = *(const int4 *)(ps + 2 * TR + g * 8);
+                    const int4 N4 = *(const int4 *)(ps + 3 * TR + g * 8);
+                    Ss[0] = S4.x; Ss[1] = S4.y; Ss[2] = S4.z; Ss[3] = S4.w;
+                    Ns[0] = (unsigned)N4.x; Ns[1] = (unsigned)N4.y; Ns[2] = (unsigned)N4.z; Ns[3] = (unsigned)N4.w;
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int e = g * 4 + j;
+                    float w = __builtin_amdgcn_exp2f(fmaf(x[e], p.attDotScale, ALIBI ? Ls[j] + ck : Ls[j]));
+                    if (!full) {
+                        w = (unsigned)(myRow - Ss[j]) <= Ns[j] ? w : 0.f;
+                    }
+                    wv[e] = w;
+                }
+            }
+        };
+        // pins values to the point of the call: without it the compiler sinks the arithmetic that makes them past the wait loops of the
+        // hand-over, to just before their first use, and nothing is left to issue between the products
+        auto pin16 = [&](float (&v)[16]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                asm volatile("" : "+v"(v[4 * g]), "+v"(v[4 * g + 1]), "+v"(v[4 * g + 2]), "+v"(v[4 * g + 3]));
+            }
+        };
+        // dV wave: hand block number n over once block n - 1 has been taken
+        auto giveP = [&](const float (&wv)[16], int n) __attribute__((always_inline)) {
+            WaitCounter(takenAddr, n - 1, waiting);
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                pMine[g * 64] = v4f{wv[4 * g], wv[4 * g + 1], wv[4 * g + 2], wv[4 * g + 3]};
+            }
+            SetCounter(readyAddr, n);
+        };
+        // dK wave: take block number n and form dS = P (dP attDotScale ln2 - dScale attDotScale ln2)
+        auto takeP = [&](const v16f &x, float (&wv)[16], int slot, int qb, int n) __attribute__((always_inline)) {
+            WaitCounter(readyAddr, n, waiting);
+            v4f pw[4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                pw[g] = pMine[g * 64];
+            }
+            SetCounter(takenAddr, n); // issued after the reads, so carried out after them
+            const float *ps = &st[slot][1][qb * 32 + half * 4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const float4 D4 = *(const float4 *)(ps + g * 8);
+                wv[4 * g] = pw[g][0] * fmaf(x[4 * g], gmul, D4.x);
+                wv[4 * g + 1] = pw[g][1] * fmaf(x[4 * g + 1], gmul, D4.y);
+                wv[4 * g + 2] = pw[g][2] * fmaf(x[4 * g + 2], gmul, D4.z);
+                wv[4 * g + 3] = pw[g][3] * fmaf(x[4 * g + 3], gmul, D4.w);
+            }
+        };
+        // second product: dV^T += dO^T P or dK^T += Q^T dS, operands four products ahead; the first four are requested by the caller
+        // (before the arithmetic that makes wb) with secondOperands
+        auto secondOperands = [&](v8bf (&ft)[5], const uint8_t *tt) __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                ft[i] = FragTr(tt, 0, i >> 2, i & 3, fl);
+            }
+        };
+        auto secondProduct = [&](v8bf (&ft)[5], const uint8_t *tt, const v8bf (&wb)[2]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                if (i + 4 < 8) {
+                    ft[(i + 4) % 5] = FragTr(tt, 0, (i + 4) >> 2, (i + 4) & 3, fl);
+                }
+                acc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ft[i % 5], wb[i >> 2], acc[i & 3], 0, 0, 0);
+            }
+        };
+        // one 64-query tile: the 32-query blocks of which some query sees a key of this wave.  When both blocks are seen (the usual
+        // case away from the edges of a span) they are worked on together, so that the wave always has instructions of one block
+        // to issue while it waits for a result of the other: both first products, then the arithmetic of block 0 between the
+        // products... (two waves per SIMD alone do not cover the latencies of a chain of dependent steps).
         auto tile = [&](const uint8_t *qt, const uint8_t *ot, int slot) __attribute__((always_inline)) {
             int bounds[2][4];
 #pragma unroll
@@ -784,117 +887,100 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
                     bounds[qb][j] = __builtin_amdgcn_readfirstlane(stT[slot][qb][j]);
                 }
             }
+            const bool seen0 = !(bounds[0][3] < kw0 || bounds[0][2] > kw0 + 31), seen1 = !(bounds[1][3] < kw0 || bounds[1][2] > kw0 + 31);
+            const bool full0 = bounds[0][0] <= kw0 && bounds[0][1] >= kw0 + 31, full1 = bounds[1][0] <= kw0 && bounds[1][1] >= kw0 + 31;
+            const uint8_t *rtile = ROLE ? ot : qt; // the tile the first product reads by rows: dO for dP, Q for S
+            const uint8_t *ttile = ROLE ? qt : ot; // the tile whose transpose the second product takes: Q^T for dK, dO^T for dV
+            // skipped by loops of no trips, not by branches (see AttGradQ)
+            const bool pair = seen0 && seen1 && full0 && full1;
+            int pairTrips = __builtin_amdgcn_readfirstlane((int)pair);
+            asm volatile("" : "+s"(pairTrips));
+#pragma unroll 1
+            for (int trip = 0; trip < pairTrips; ++trip) {
+                const int n0 = blockNo + 1, n1 = blockNo + 2;
+                blockNo += 2;
+                v16f x0, x1;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    x0[e] = 0;
+                    x1[e] = 0;
+                }
+                v8bf ft[5];
+                float wv[16];
+                firstProduct(x0, rtile);
+                firstProduct(x1, rtile + 32 * ROWB);
+                secondOperands(ft, ttile);
+                if constexpr (ROLE == 0) {
+                    float wv1[16];
+                    probabilities(x0, wv, slot, 0, std::true_type{});
+                    // the second first-product runs with the arithmetic of block 0 between its MFMAs
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    }
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
+                    }
+                    pin16(wv);
+                    giveP(wv, n0);
+                    const v8bf wb0[2] = {PackB(wv, 0), PackB(wv, 1)};
+                    probabilities(x1, wv1, slot, 1, std::true_type{});
+                    secondProduct(ft, ttile, wb0);
+                    // ... and the arithmetic of block 1 between the MFMAs of block 0's second product
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
+                    }
+                    secondOperands(ft, ttile + 32 * ROWB);
+                    pin16(wv1);
+                    giveP(wv1, n1);
+                    const v8bf wb1[2] = {PackB(wv1, 0), PackB(wv1, 1)};
+                    secondProduct(ft, ttile + 32 * ROWB, wb1);
+                } else {
+                    takeP(x0, wv, slot, 0, n0);
+                    const v8bf wb0[2] = {PackB(wv, 0), PackB(wv, 1)};
+                    secondProduct(ft, ttile, wb0);
+                    secondOperands(ft, ttile + 32 * ROWB);
+                    takeP(x1, wv, slot, 1, n1);
+                    const v8bf wb1[2] = {PackB(wv, 0), PackB(wv, 1)};
+                    secondProduct(ft, ttile + 32 * ROWB, wb1);
+                }
+            }
 #pragma unroll
             for (int qb = 0; qb < TR / 32; ++qb) {
-                const bool full = bounds[qb][0] <= kw0 && bounds[qb][1] >= kw0 + 31;
-                const uint8_t *qt2 = qt + qb * 32 * ROWB, *ot2 = ot + qb * 32 * ROWB;
-                // skipped by a loop of no trips, not by a branch (see AttGradQ)
-                int trips = __builtin_amdgcn_readfirstlane((int)!(bounds[qb][3] < kw0 || bounds[qb][2] > kw0 + 31));
+                const bool full = qb ? full1 : full0;
+                int trips = __builtin_amdgcn_readfirstlane((int)((qb ? seen1 : seen0) && !pair));
                 asm volatile("" : "+s"(trips));
 #pragma unroll 1
                 for (int trip = 0; trip < trips; ++trip) {
-                ++blockNo;
-                v16f x; // S (dV wave) or dP (dK wave)
+                    ++blockNo;
+                    v16f x;
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    x[e] = 0;
-                }
-                const uint8_t *rt = ROLE ? ot2 : qt2; // the tile the first product reads by rows: dO for dP, Q for S
-                const uint8_t *tt = ROLE ? qt2 : ot2; // the tile whose transpose the second product takes: Q^T for dK, dO^T for dV
-                v8bf ft[3];
-                {
-                    // operands three steps ahead (one product per step)
-                    v8bf fr[4];
-#pragma unroll
-                    for (int ds = 0; ds < 3; ++ds) {
-                        fr[ds] = FragRow(rt, 0, ds, fl);
+                    for (int e = 0; e < 16; ++e) {
+                        x[e] = 0;
                     }
-#pragma unroll
-                    for (int ds = 0; ds < 8; ++ds) {
-                        if (ds + 3 < 8) {
-                            fr[(ds + 3) & 3] = FragRow(rt, 0, ds + 3, fl);
+                    v8bf ft[5];
+                    float wv[16];
+                    firstProduct(x, rtile + qb * 32 * ROWB);
+                    secondOperands(ft, ttile + qb * 32 * ROWB);
+                    if constexpr (ROLE == 0) {
+                        if (full) {
+                            probabilities(x, wv, slot, qb, std::true_type{});
+                        } else {
+                            probabilities(x, wv, slot, qb, std::false_type{});
                         }
-                        x = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[ds & 3], own[ds], x, 0, 0, 0);
+                        giveP(wv, blockNo);
+                    } else {
+                        takeP(x, wv, slot, qb, blockNo);
                     }
-                    ft[0] = FragTr(tt, 0, 0, 0, fl);
-                    ft[1] = FragTr(tt, 0, 0, 1, fl);
-                    __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
-#pragma unroll
-                    for (int ds = 0; ds < 5; ++ds) {
-                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    }
-                    __builtin_amdgcn_sched_group_barrier(0x008, 3, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-                }
-                float wv[16];
-                if constexpr (ROLE == 0) {
-                    // P from the per-query statistics of the tile
-                    const float *ps = &st[slot][0][qb * 32 + half * 4];
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const float4 L4 = *(const float4 *)(ps + g * 8);
-                        const float Ls[4] = {L4.x, L4.y, L4.z, L4.w};
-                        int Ss[4] = {0, 0, 0, 0};
-                        unsigned Ns[4] = {0, 0, 0, 0};
-                        if (!full) {
-                            const int4 S4 = *(const int4 *)(ps + 2 * TR + g * 8);
-                            const int4 N4 = *(const int4 *)(ps + 3 * TR + g * 8);
-                            Ss[0] = S4.x; Ss[1] = S4.y; Ss[2] = S4.z; Ss[3] = S4.w;
-                            Ns[0] = (unsigned)N4.x; Ns[1] = (unsigned)N4.y; Ns[2] = (unsigned)N4.z; Ns[3] = (unsigned)N4.w;
-                        }
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            const int e = g * 4 + j;
-                            float w = __builtin_amdgcn_exp2f(fmaf(x[e], p.attDotScale, ALIBI ? Ls[j] + ck : Ls[j]));
-                            if (!full) {
-                                w = (unsigned)(myRow - Ss[j]) <= Ns[j] ? w : 0.f;
-                            }
-                            wv[e] = w;
-                        }
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                    // hand the block over once the previous one has been taken
-                    WaitCounter(takenAddr, blockNo - 1, waiting);
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        pMine[g * 64] = v4f{wv[4 * g], wv[4 * g + 1], wv[4 * g + 2], wv[4 * g + 3]};
-                    }
-                    SetCounter(readyAddr, blockNo);
-                } else {
-                    // dS = P (dP attDotScale ln2 - dScale attDotScale ln2)
-                    WaitCounter(readyAddr, blockNo, waiting);
-                    v4f pw[4];
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        pw[g] = pMine[g * 64];
-                    }
-                    SetCounter(takenAddr, blockNo); // issued after the reads, so carried out after them
-                    const float *ps = &st[slot][1][qb * 32 + half * 4];
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const float4 D4 = *(const float4 *)(ps + g * 8);
-                        wv[4 * g] = pw[g].x * fmaf(x[4 * g], gmul, D4.x);
-                        wv[4 * g + 1] = pw[g].y * fmaf(x[4 * g + 1], gmul, D4.y);
-                        wv[4 * g + 2] = pw[g].z * fmaf(x[4 * g + 2], gmul, D4.z);
-                        wv[4 * g + 3] = pw[g].w * fmaf(x[4 * g + 3], gmul, D4.w);
-                    }
-                }
-                const v8bf wb[2] = {PackB(wv, 0), PackB(wv, 1)};
-                // dV^T += dO^T P, or dK^T += Q^T dS, operands two products ahead
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    if (i + 2 < 8) {
-                        ft[(i + 2) % 3] = FragTr(tt, 0, (i + 2) >> 2, (i + 2) & 3, fl);
-                    }
-                    acc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ft[i % 3], wb[i >> 2], acc[i & 3], 0, 0, 0);
-                }
-#pragma unroll
-                for (int i = 0; i < 6; ++i) {
-                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                }
-                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+                    const v8bf wb[2] = {PackB(wv, 0), PackB(wv, 1)};
+                    secondProduct(ft, ttile + qb * 32 * ROWB, wb);
                 }
             }
         };
