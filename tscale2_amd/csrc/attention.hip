@@ -838,8 +838,19 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
             }
             SetCounter(readyAddr, n);
         };
-        // dK wave: take block number n and form dS = P (dP attDotScale ln2 - dScale attDotScale ln2)
+        // dK wave: take block number n and form dS = P (dP attDotScale ln2 - dScale attDotScale ln2); the factor that does not need P
+        // is formed before the wait
         auto takeP = [&](const v16f &x, float (&wv)[16], int slot, int qb, int n) __attribute__((always_inline)) {
+            const float *ps = &st[slot][1][qb * 32 + half * 4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const float4 D4 = *(const float4 *)(ps + g * 8);
+                wv[4 * g] = fmaf(x[4 * g], gmul, D4.x);
+                wv[4 * g + 1] = fmaf(x[4 * g + 1], gmul, D4.y);
+                wv[4 * g + 2] = fmaf(x[4 * g + 2], gmul, D4.z);
+                wv[4 * g + 3] = fmaf(x[4 * g + 3], gmul, D4.w);
+            }
+            pin16(wv);
             WaitCounter(readyAddr, n, waiting);
             v4f pw[4];
 #pragma unroll
@@ -847,14 +858,12 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
                 pw[g] = pMine[g * 64];
             }
             SetCounter(takenAddr, n); // issued after the reads, so carried out after them
-            const float *ps = &st[slot][1][qb * 32 + half * 4];
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const float4 D4 = *(const float4 *)(ps + g * 8);
-                wv[4 * g] = pw[g][0] * fmaf(x[4 * g], gmul, D4.x);
-                wv[4 * g + 1] = pw[g][1] * fmaf(x[4 * g + 1], gmul, D4.y);
-                wv[4 * g + 2] = pw[g][2] * fmaf(x[4 * g + 2], gmul, D4.z);
-                wv[4 * g + 3] = pw[g][3] * fmaf(x[4 * g + 3], gmul, D4.w);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    wv[4 * g + j] *= pw[g][j];
+                }
             }
         };
         // second product: dV^T += dO^T P or dK^T += Q^T dS, operands four products ahead; the first four are requested by the caller
