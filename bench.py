@@ -430,7 +430,7 @@ def bench_step_fp8(args):
     sub.no_cpu, sub.steps, sub.warmup, sub.small = True, 10, 3, False
     a = bench_att_bwd(sub)
     out["att_bwd"] = {"workload": a["config"]["workload"], "ms": a["ms_per_step"], "tokens_per_s": a["value"], "tflops": a["roofline"]["achieved"],
-                      "frac_of_bf16_peak": a["roofline"]["frac"], "kernel": a["roofline"]["kernel"]}
+                      "frac_of_bf16_peak": a["roofline"]["frac"], "kernel": a["roofline"]["kernel"], "kernels": a["kernels"]}
     torch.cuda.empty_cache()
     mo = bench_moe_fp8(sub)
     out["moe_layer"] = {"workload": mo["config"]["workload"], "ms": mo["ms_per_step"], "tokens_per_s": mo["value"], "layer_tflops": mo["layer_tflops"],
@@ -538,13 +538,16 @@ def bench_att_bwd(args):
     L.att_forward(n, H, q.view(i16), k.view(i16), v.view(i16), start, finish, sc, 0.0, val.view(i16), swl)
     ds.copy_((val.float() * do.float()).view(n, H, 128).sum(-1).t())
 
-    def step():
+    def step(which=3):
         L.att_backward(n, H, q.view(i16), k.view(i16), v.view(i16), do.view(i16), start, finish, rl, rh, sc, 0.0, swl, ds, dq.view(i16), dk.view(i16),
-                       dv.view(i16), L.BF16, 3)
+                       dv.view(i16), L.BF16, which)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
     ms = event_time_ms(step, args.steps)
+    # the two kernels on their own, after the timed region (the device is warm by then)
+    ms_dq = event_time_ms(lambda: step(1), args.steps)
+    ms_dkdv = event_time_ms(lambda: step(2), args.steps)
     pairs = B * H * (S * (S - 1) / 2)
     flop5 = 5 * 2.0 * pairs * 128
     roof = {"bound": "mfma", "achieved": flop5 / (ms * 1e-3) / 1e12, "peak": PEAK_BF16 / 1e12, "unit": "TFLOP/s", "frac": flop5 / (ms * 1e-3) / PEAK_BF16,
@@ -552,7 +555,7 @@ def bench_att_bwd(args):
     out = {"metric": "attention backward tokens/sec on 1 MI355X; TFLOPS as % of MFMA peak", "value": n / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1,
            "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": "bf16", "data": "synthetic", "config": {"workload": "causal attention backward, 16 x 2048 tokens, 16 heads x 128, bf16"},
-           "roofline": roof}
+           "roofline": roof, "kernels": {"dq_ms": ms_dq, "dkdv_ms": ms_dkdv, "dq_products": 3, "dkdv_products": 4}}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_att(H, B, S)
     return out
