@@ -393,6 +393,14 @@ typedef struct ts2_att_grad_args {
     ts2_mat dQ, dK, dV;           /* out, gradType = TS2_BF16 | TS2_F32 */
     int32_t gradType;
     int32_t which; /* bit 0: dQ (Fp16AttGradQ), bit 1: dK and dV (Fp16AttGradKV) */
+    /* optional, all three or none, used when which == 3: the score gradients dS leave the dK/dV kernel as 32 x 32 bf16 blocks (2 KB
+     * each) in dsScratch and dQ is a single product over them instead of a second evaluation of S and dP (5 products per backward
+     * instead of 7).  dsBase: [lenRound + 1] from ts2_att_build_ds_index on the same spans; dsScratch: 16-byte aligned,
+     * dsCapacityBlocks blocks of 2048 bytes, at least heads * ts2_att_ds_blocks(spans) (blocks beyond the capacity are dropped:
+     * wrong gradients for those rows, no access outside the array).  Without them the kernels of the two bits run independently. */
+    const int32_t *dsBase;
+    void *dsScratch;
+    int64_t dsCapacityBlocks;
 } ts2_att_grad_args;
 
 /* Fp16AttGradQ + Fp16AttGradKV, src/gpt/compute/gpu_att_fp16.cuh:60-358 (their norm/rope epilogues are
@@ -403,6 +411,13 @@ int ts2_att_backward(const ts2_att_grad_args *args, void *stream);
  * span touches it (replaces TransposeAttention + GroupAttention on the host, src/gpt/att/att.cpp:25-55, att.h:125-211). */
 int ts2_att_build_rev(int32_t len, int32_t lenRound, const int32_t *spanStart, const int32_t *spanFinish, int32_t *revLo, int32_t *revHi,
     void *stream);
+/* Numbering of the blocks of score gradients that ts2_att_backward can hand from its dK/dV kernel to its dQ kernel (no counterpart in
+ * the reference, whose two kernels each evaluate the scores): a block exists for every (32-query block, 32-key block) pair such that
+ * the key block lies between the earliest span start and the latest span finish of the query block's rows.  dsBase[q] = number of
+ * the first block of q's query block, dsBase[lenRound] = blocks per head; device arrays, spans of lenRound rows (empty: finish <
+ * start).  ts2_att_ds_blocks counts the blocks per head on the host from host copies of the same spans (to size the array). */
+int ts2_att_build_ds_index(int32_t lenRound, const int32_t *spanStart, const int32_t *spanFinish, int32_t *dsBase, void *stream);
+int64_t ts2_att_ds_blocks(int32_t lenRound, const int32_t *spanStartHost, const int32_t *spanFinishHost);
 
 /* TStoreRowTileNormalize / TStoreRowTileNormalizeRope as a stand-alone pass (src/lib/cuda/cuda_matmul.cuh:495-525,
  * src/gpt/compute/gpu_rope.cuh:25-60): per row and 128-wide head: v = src*srcMult; if normalize: scale = rms(v)*vecScale

@@ -89,6 +89,21 @@ def run_case(L, orc, frag_count, frag_len, window, heads, slope, seed, grad_type
         print(name, "rel err", err)
         assert err <= 1e-2, name
         assert np.all(g[n:] == 0), name
+    # the same with the score gradients handed from the dK/dV kernel to the dQ kernel (5 products instead of 7): dK and dV are the very
+    # same values, dQ is formed from dS rounded to bf16 where the other kernel rounds its own evaluation of it: equal to bf16 noise
+    print("  ... dQ from the dK/dV kernel's score gradients", flush=True)
+    ds_pair = L.att_ds_scratch(n_round, heads, ts, tf)
+    ds_pair[1].fill_(0x7f)  # NaN patterns where nothing is written
+    dq2, dk2, dv2 = torch.full_like(dq, 3.0), torch.full_like(dk, 3.0), torch.full_like(dv, 3.0)
+    L.att_backward(n, heads, tq.view(i16), tk.view(i16), tv.view(i16), tdv.view(i16), ts, tf, rev_lo, rev_hi, att_dot_scale, slope, swl, ds,
+                   vw(dq2), vw(dk2), vw(dv2), grad_type, ds=ds_pair)
+    torch.cuda.synchronize()
+    assert torch.equal(dk2, dk) and torch.equal(dv2, dv)
+    g2 = dq2.float().cpu().numpy()
+    err = np.abs(g2[:n] - ref["dq"]).max() / np.abs(ref["dq"]).max()
+    print("dq (from dS) rel err", err, "against the other kernel", np.abs(g2 - dq.float().cpu().numpy()).max() / np.abs(ref["dq"]).max())
+    assert err <= 1e-2 and np.all(g2[n:] == 0)
+    assert np.abs(g2 - dq.float().cpu().numpy()).max() <= 4e-3 * np.abs(ref["dq"]).max()
 
 
 def test_attention_window_and_slope(L, orc):

@@ -64,7 +64,14 @@ struct AttP {
     uint8_t *out0, *out1; // forward: valLookup; dQ kernel: dQ; dK/dV kernel: dK, dV
     int64_t ldo0, ldo1;
     int lenRound;
+    // score gradients handed from the dK/dV kernel to the dQ kernel (optional): per query row the number of its 32-query block's first
+    // block of dS (dsBase[lenRound] = blocks per head), the blocks themselves (2 KB each), and how many of them the array holds
+    const int *dsBase;
+    uint8_t *ds;
+    int64_t dsCap;
 };
+
+constexpr int DS_BLOCK_BYTES = 32 * 32 * 2; // a 32 x 32 block of dS in bf16
 
 // result registers 8*s .. 8*s+7 of a 32x32 block -> bf16 B operand whose slots match FragTr's row order
 __device__ __forceinline__ v8bf PackB(const float *x, int s)
@@ -674,16 +681,17 @@ __device__ __forceinline__ void SetCounter(int ldsAddr, int value)
     asm volatile("ds_write_b32 %0, %1" : : "v"(ldsAddr), "v"(value) : "memory");
 }
 
-template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGradKV(AttP p)
+template <bool F32, bool ALIBI, bool DS> __global__ void __launch_bounds__(256, 2) AttGradKV(AttP p)
 {
     __shared__ __attribute__((aligned(16))) float pBlock[2][4][64][4]; // [key block][quarter][lane][4 values]: P of the block in hand
     __shared__ int pCount[2][2];                                          // [key block][ready, taken]
     __shared__ __attribute__((aligned(1024))) uint8_t qT0[TILE_BYTES], qT1[TILE_BYTES], oT0[TILE_BYTES], oT1[TILE_BYTES];
-    __shared__ __attribute__((aligned(16))) float rawStat[2][4][TR];  // [slot][L, dScale, span start, span finish][query], as loaded
+    // [slot][L, dScale, span start, span finish, first dS block of the query's block][query], as loaded
+    __shared__ __attribute__((aligned(16))) float rawStat[2][DS ? 5 : 4][TR];
     // [slot][-L - slope * (q - keyBase), -dScale * attDotScale * ln2, span start (0x7fffffff if empty), span length][query]: one array,
     // one address register
     __shared__ __attribute__((aligned(16))) float st[2][4][TR];
-    __shared__ int stT[2][2][4];                                          // [slot][32-query block]: bounds over the block's queries
+    __shared__ int stT[2][2][5]; // [slot][32-query block]: bounds over the block's queries, first dS block
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l32 = lane & 31, half = lane >> 5;
     int block, head;
     MapAttBlock(&block, &head);
@@ -710,6 +718,9 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
             __builtin_amdgcn_global_load_lds(TS2_GLB_PTR(p.dScale + so), TS2_LDS_PTR(&rawStat[slot][1][0]), 4, 0, 0);
             __builtin_amdgcn_global_load_lds(TS2_GLB_PTR(p.spanStart + t0 + lane), TS2_LDS_PTR(&rawStat[slot][2][0]), 4, 0, 0);
             __builtin_amdgcn_global_load_lds(TS2_GLB_PTR(p.spanFinish + t0 + lane), TS2_LDS_PTR(&rawStat[slot][3][0]), 4, 0, 0);
+            if constexpr (DS) {
+                __builtin_amdgcn_global_load_lds(TS2_GLB_PTR(p.dsBase + t0 + lane), TS2_LDS_PTR(&rawStat[slot][DS ? 4 : 0][0]), 4, 0, 0);
+            }
         }
     };
     // the statistics wave: raw statistics of the tile at t0 (slot) -> the form the products use
@@ -734,6 +745,9 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
                 stT[slot][half][1] = b; // earliest finish
                 stT[slot][half][2] = c; // earliest start
                 stT[slot][half][3] = d; // latest finish
+                if constexpr (DS) {
+                    stT[slot][half][4] = __float_as_int(rawStat[slot][DS ? 4 : 0][lane]);
+                }
             }
         }
     };
@@ -749,6 +763,7 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
     const TFragLane fl = MakeFragLane(lane);
     const int kw0 = __builtin_amdgcn_readfirstlane(myRow - l32); // first key of this wave
     const float ck = p.slope * (float)(myRow - keyBase);
+    const int64_t dsHead = DS ? (int64_t)head * p.dsBase[p.lenRound] : 0; // first dS block of this head
     // the whole tile loop once per role, as separate code: no value of one role's path meets a value of the other's, and every
     // operand fetch names the LDS array it reads (a fetch through a selected pointer would have to wait for the loads in flight)
     auto run = [&](auto roleTag) __attribute__((always_inline)) {
@@ -866,6 +881,51 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
                 }
             }
         };
+        // dK wave: the block of dS goes to the dQ kernel, transposed on the way.  Here a lane is a key and its registers walk over the
+        // queries; the dQ kernel's lanes are queries.  The operand pair the wave is about to multiply with, taken as the A operand of
+        // two more MFMAs against the matching slices of the identity, comes back as dS^T with lane = query, registers = keys in the
+        // order of the other kernel's operand fetches (exact: every sum has one term, and the values are bf16 already).  Block
+        // number first(query block) + (this key block - first key block the query block sees); a lane's two operands of 16 bytes sit at
+        // lane * 16 and 1024 + lane * 16: a wave writes, and the dQ kernel's wave reads, 1 KB contiguous per instruction.
+        v8bf idB[2];
+        if constexpr (DS && ROLE == 1) {
+#pragma unroll
+            for (int sl = 0; sl < 2; ++sl) {
+                v4i r;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    // slot j of operand sl in a lane of half h stands for query 16 sl + (j >> 2) * 8 + 4 h + (j & 3)
+                    const int qa = 16 * sl + ((2 * w) >> 2) * 8 + 4 * half + ((2 * w) & 3), qb2 = qa + 1;
+                    r[w] = (qa == l32 ? 0x3f80 : 0) | (qb2 == l32 ? 0x3f800000 : 0);
+                }
+                idB[sl] = __builtin_bit_cast(v8bf, r);
+            }
+        }
+        auto giveDs = [&](const v8bf (&wb)[2], int slot, int qb) __attribute__((always_inline)) {
+            if constexpr (DS && ROLE == 1) {
+                const int first = __builtin_amdgcn_readfirstlane(stT[slot][qb][4]);
+                const int startMin = __builtin_amdgcn_readfirstlane(stT[slot][qb][2]);
+                const int64_t id = dsHead + first + ((kw0 >> 5) - (startMin >> 5));
+                v16f tr;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    tr[e] = 0;
+                }
+                tr = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[0], idB[0], tr, 0, 0, 0);
+                tr = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wb[1], idB[1], tr, 0, 0, 0);
+                float tv[16];
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    tv[e] = tr[e];
+                }
+                const v8bf o0 = PackB(tv, 0), o1 = PackB(tv, 1);
+                if (id >= 0 && id < p.dsCap) {
+                    uint8_t *dst = p.ds + id * DS_BLOCK_BYTES + lane * 16;
+                    *(v4i *)dst = __builtin_bit_cast(v4i, o0);
+                    *(v4i *)(dst + 1024) = __builtin_bit_cast(v4i, o1);
+                }
+            }
+        };
         // second product: dV^T += dO^T P or dK^T += Q^T dS, operands four products ahead; the first four are requested by the caller
         // (before the arithmetic that makes wb) with secondOperands
         auto secondOperands = [&](v8bf (&ft)[5], const uint8_t *tt) __attribute__((always_inline)) {
@@ -954,10 +1014,12 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
                 } else {
                     takeP(x0, wv, slot, 0, n0);
                     const v8bf wb0[2] = {PackB(wv, 0), PackB(wv, 1)};
+                    giveDs(wb0, slot, 0);
                     secondProduct(ft, ttile, wb0);
                     secondOperands(ft, ttile + 32 * ROWB);
                     takeP(x1, wv, slot, 1, n1);
                     const v8bf wb1[2] = {PackB(wv, 0), PackB(wv, 1)};
+                    giveDs(wb1, slot, 1);
                     secondProduct(ft, ttile + 32 * ROWB, wb1);
                 }
             }
@@ -989,6 +1051,9 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
                         takeP(x, wv, slot, qb, blockNo);
                     }
                     const v8bf wb[2] = {PackB(wv, 0), PackB(wv, 1)};
+                    if constexpr (ROLE == 1) {
+                        giveDs(wb, slot, qb);
+                    }
                     secondProduct(ft, ttile + qb * 32 * ROWB, wb);
                 }
             }
@@ -1032,6 +1097,163 @@ template <bool F32, bool ALIBI> __global__ void __launch_bounds__(256, 2) AttGra
         run(std::integral_constant<int, 1>{});
     } else {
         run(std::integral_constant<int, 0>{});
+    }
+}
+
+// dQ from the score gradients the dK/dV kernel left behind: dQ^T += K^T dS^T, one product per block, no statistics, no exponentials.
+// grid (lenRound/128, heads); a wave owns 32 query rows (as in AttGradQ) and streams the key tiles its rows reach through LDS.  Its blocks
+// of dS arrive transposed and in operand order (see giveDs), one after the other in memory: 32 bytes per lane and block straight into
+// registers.  The kernel is a stream of loads with 16 MFMAs per tile and wave, so everything is requested two tiles ahead: three
+// K buffers in LDS, three sets of dS registers, used in turn (three copies of the tile code per trip).  Every trip issues the same
+// number of loads - past the end of the range they re-read the last tile, and a block the wave does not see is replaced by block 0 -
+// so that "all but the newest eight" (vmcnt) at the top of a trip means that the tile and the blocks of this trip have landed.
+template <bool F32> __global__ void __launch_bounds__(256, 3) AttGradQFromDs(AttP p)
+{
+    __shared__ __attribute__((aligned(1024))) uint8_t kT0[TILE_BYTES], kT1[TILE_BYTES], kT2[TILE_BYTES];
+    __shared__ int red[8];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l32 = lane & 31;
+    int blk, head;
+    MapAttBlock(&blk, &head);
+    const int myRow = (gridDim.x - 1 - blk) * BROWS + wave * WROWS + l32; // long blocks first, as in AttGradQ
+    const int64_t hoff = (int64_t)head * HD * 2;
+    const int start = p.spanStart[myRow], finish = p.spanFinish[myRow];
+    int kLo, kHi;
+    BlockKeyRange(start, finish, tid, &kLo, &kHi, red);
+    kLo = __builtin_amdgcn_readfirstlane(kLo);
+    kHi = __builtin_amdgcn_readfirstlane(kHi);
+    if (kHi < kLo) { // no row of the workgroup has a span (wave-uniform, before any barrier of the loop)
+        v16f none[4];
+#pragma unroll
+        for (int db = 0; db < 4; ++db) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                none[db][e] = 0;
+            }
+        }
+        StoreOwnRows<F32>(p.out0 + (int64_t)(myRow - l32) * p.ldo0, p.ldo0, head * HD, none, 1.f, l32, lane >> 5);
+        return;
+    }
+    const int tFirst = (kLo / TR) * TR, tLast = (kHi / TR) * TR;
+    const uint8_t *gk = p.k + hoff;
+    const TRowSpan sp = MakeRowSpan(start, finish);
+    // this wave's blocks of dS: number first + (key block - first key block the wave's rows see), per head
+    const int64_t dsFirst = (int64_t)head * p.dsBase[p.lenRound] + __builtin_amdgcn_readfirstlane(p.dsBase[myRow]) - (sp.waveMinStart >> 5);
+    const uint8_t *dsLane = p.ds + lane * 16;
+    // requests for the tile at t0 (clamped to the last tile): its K rows, then the wave's two blocks of dS (block 0 for one it does not use)
+    auto request = [&](uint8_t *kt, v4i (&sb)[2][2], int t0) __attribute__((always_inline)) {
+        const int tt = t0 <= tLast ? t0 : tLast;
+        LoadTileDirect(kt, gk + (int64_t)tt * p.ldk, p.ldk, wave);
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            const int k0 = tt + kb * 32;
+            int64_t id = dsFirst + (k0 >> 5);
+            if (k0 > sp.waveMaxFinish || k0 + 31 < sp.waveMinStart || id < 0 || id >= p.dsCap) {
+                id = 0;
+            }
+            sb[kb][0] = *(const v4i *)(dsLane + id * DS_BLOCK_BYTES);
+            sb[kb][1] = *(const v4i *)(dsLane + id * DS_BLOCK_BYTES + 1024);
+        }
+    };
+    v4i sb0[2][2], sb1[2][2], sb2[2][2];
+    request(kT0, sb0, tFirst);
+    request(kT1, sb1, tFirst + TR);
+    const TFragLane fl = MakeFragLane(lane);
+    float zero = 0; // opaque, as in AttGradQ
+    asm volatile("" : "+v"(zero));
+    v16f acc[4];
+#pragma unroll
+    for (int db = 0; db < 4; ++db) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            acc[db][e] = zero;
+        }
+    }
+    auto tile = [&](const uint8_t *kt, const v4i (&sb)[2][2], int t0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int kb = 0; kb < TR / 32; ++kb) {
+            const int k0 = t0 + kb * 32;
+            const uint8_t *kt2 = kt + kb * 32 * ROWB;
+            int trips = __builtin_amdgcn_readfirstlane((int)!(k0 > sp.waveMaxFinish || k0 + 31 < sp.waveMinStart)); // (see AttGradQ)
+            asm volatile("" : "+s"(trips));
+#pragma unroll 1
+            for (int trip = 0; trip < trips; ++trip) {
+                const v8bf b[2] = {__builtin_bit_cast(v8bf, sb[kb][0]), __builtin_bit_cast(v8bf, sb[kb][1])};
+                v8bf ft[5];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    ft[i] = FragTr(kt2, 0, i >> 2, i & 3, fl);
+                }
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    if (i + 4 < 8) {
+                        ft[(i + 4) % 5] = FragTr(kt2, 0, (i + 4) >> 2, (i + 4) & 3, fl);
+                    }
+                    acc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ft[i % 5], b[i >> 2], acc[i & 3], 0, 0, 0);
+                }
+            }
+        }
+    };
+    // per trip: the loads of this tile have landed (all but the eight of the next one), for every wave; request the tile after next
+    // into the buffer every wave has just left; multiply
+#define DQ_TRIP(KC, SC, KN, SN)                                                                                                            \
+    __builtin_amdgcn_s_waitcnt(0x0f78); /* vmcnt(8) */                                                                                     \
+    __syncthreads();                                                                                                                       \
+    request(KN, SN, t0 + 2 * TR);                                                                                                          \
+    tile(KC, SC, t0);                                                                                                                      \
+    t0 += TR;                                                                                                                              \
+    if (t0 > kHi) {                                                                                                                        \
+        break;                                                                                                                             \
+    }
+    for (int t0 = tFirst;;) {
+        DQ_TRIP(kT0, sb0, kT2, sb2)
+        DQ_TRIP(kT1, sb1, kT0, sb0)
+        DQ_TRIP(kT2, sb2, kT1, sb1)
+    }
+#undef DQ_TRIP
+    __builtin_amdgcn_s_waitcnt(0x0f70); // the requests past the end land before the workgroup's LDS is given up
+    StoreOwnRows<F32>(p.out0 + (int64_t)(myRow - l32) * p.ldo0, p.ldo0, head * HD, acc, 1.f, l32, lane >> 5);
+}
+
+// dsBase[q] = number of the first block of dS of q's 32-query block, numbering the blocks (query block, key block it sees) in the
+// order of the query blocks; dsBase[lenRound] = their count.  A query block sees the key blocks from (earliest span start) / 32 to
+// (latest span finish) / 32 of its rows with a span.  One workgroup; a thread takes a run of query blocks.
+__global__ void __launch_bounds__(1024) DsIndexBuild(const int *spanStart, const int *spanFinish, int lenRound, int *dsBase)
+{
+    __shared__ int part[1024];
+    const int nqb = lenRound / 32, tid = threadIdx.x;
+    const int per = (nqb + 1023) / 1024, q0 = tid * per, q1 = min(nqb, q0 + per);
+    auto count = [&](int qb) {
+        int lo = 0x7fffffff, hi = -1;
+        for (int i = 0; i < 32; ++i) {
+            const int s = spanStart[qb * 32 + i], f = spanFinish[qb * 32 + i];
+            if (f >= s) {
+                lo = min(lo, s);
+                hi = max(hi, f);
+            }
+        }
+        return hi >= lo ? (hi >> 5) - (lo >> 5) + 1 : 0;
+    };
+    int sum = 0;
+    for (int qb = q0; qb < q1; ++qb) {
+        sum += count(qb);
+    }
+    part[tid] = sum;
+    __syncthreads();
+    for (int d = 1; d < 1024; d *= 2) { // inclusive scan
+        const int v = tid >= d ? part[tid - d] : 0;
+        __syncthreads();
+        part[tid] += v;
+        __syncthreads();
+    }
+    int run = part[tid] - sum;
+    for (int qb = q0; qb < q1; ++qb) {
+        for (int i = 0; i < 32; ++i) {
+            dsBase[qb * 32 + i] = run;
+        }
+        run += count(qb);
+    }
+    if (tid == 1023) {
+        dsBase[lenRound] = part[1023];
     }
 }
 
@@ -1094,6 +1316,39 @@ extern "C" int ts2_att_forward(const ts2_att_args *a, void *stream)
     return TS2_OK;
 }
 
+extern "C" int ts2_att_build_ds_index(int32_t lenRound, const int32_t *spanStart, const int32_t *spanFinish, int32_t *dsBase, void *stream)
+{
+    if (!spanStart || !spanFinish || !dsBase) {
+        return TS2_ERR_NULL;
+    }
+    if (lenRound <= 0 || lenRound % BROWS) {
+        return TS2_ERR_SHAPE;
+    }
+    hipLaunchKernelGGL(DsIndexBuild, dim3(1), dim3(1024), 0, (hipStream_t)stream, spanStart, spanFinish, lenRound, dsBase);
+    TS2_CHECK_LAUNCH();
+    return TS2_OK;
+}
+
+extern "C" int64_t ts2_att_ds_blocks(int32_t lenRound, const int32_t *spanStartHost, const int32_t *spanFinishHost)
+{
+    if (!spanStartHost || !spanFinishHost || lenRound <= 0 || lenRound % 32) {
+        return TS2_ERR_SHAPE;
+    }
+    int64_t total = 0;
+    for (int qb = 0; qb < lenRound / 32; ++qb) {
+        int lo = 0x7fffffff, hi = -1;
+        for (int i = 0; i < 32; ++i) {
+            const int s = spanStartHost[qb * 32 + i], f = spanFinishHost[qb * 32 + i];
+            if (f >= s) {
+                lo = s < lo ? s : lo;
+                hi = f > hi ? f : hi;
+            }
+        }
+        total += hi >= lo ? (hi >> 5) - (lo >> 5) + 1 : 0;
+    }
+    return total;
+}
+
 extern "C" int ts2_att_backward(const ts2_att_grad_args *a, void *stream)
 {
     if (!a || !a->spanStart || !a->spanFinish || !a->revLo || !a->revHi || !a->sumWeightLog.ptr || !a->dScale.ptr) {
@@ -1131,7 +1386,17 @@ extern "C" int ts2_att_backward(const ts2_att_grad_args *a, void *stream)
     p.ldStat = a->sumWeightLog.strideBytes / 4;
     p.lenRound = a->lenRound;
     const bool alibi = a->alibiSlope != 0; // the kernels without a slope leave the position term out of every logit
-    if (a->which & 1) {
+    // with a dS array the dK/dV kernel leaves its score gradients behind and dQ is one product over them (both must run: which == 3)
+    const bool viaDs = a->which == 3 && a->dsBase && a->dsScratch && a->dsCapacityBlocks > 0;
+    if (viaDs) {
+        if (((uintptr_t)a->dsScratch & 15) != 0) {
+            return TS2_ERR_ALIGN;
+        }
+        p.dsBase = a->dsBase;
+        p.ds = (uint8_t *)a->dsScratch;
+        p.dsCap = a->dsCapacityBlocks;
+    }
+    if ((a->which & 1) && !viaDs) {
         p.out0 = (uint8_t *)a->dQ.ptr;
         p.ldo0 = a->dQ.strideBytes;
         auto kernel = f32 ? (alibi ? AttGradQ<true, true> : AttGradQ<true, false>) : (alibi ? AttGradQ<false, true> : AttGradQ<false, false>);
@@ -1143,8 +1408,19 @@ extern "C" int ts2_att_backward(const ts2_att_grad_args *a, void *stream)
         p.ldo0 = a->dK.strideBytes;
         p.out1 = (uint8_t *)a->dV.ptr;
         p.ldo1 = a->dV.strideBytes;
-        auto kernel = f32 ? (alibi ? AttGradKV<true, true> : AttGradKV<true, false>) : (alibi ? AttGradKV<false, true> : AttGradKV<false, false>);
+        auto kernel = f32 ? (alibi ? AttGradKV<true, true, false> : AttGradKV<true, false, false>)
+                          : (alibi ? AttGradKV<false, true, false> : AttGradKV<false, false, false>);
+        if (viaDs) {
+            kernel = f32 ? (alibi ? AttGradKV<true, true, true> : AttGradKV<true, false, true>)
+                         : (alibi ? AttGradKV<false, true, true> : AttGradKV<false, false, true>);
+        }
         hipLaunchKernelGGL(kernel, dim3(a->lenRound / KVROWS, a->heads), dim3(256), 0, (hipStream_t)stream, p);
+        TS2_CHECK_LAUNCH();
+    }
+    if (viaDs) {
+        p.out0 = (uint8_t *)a->dQ.ptr;
+        p.ldo0 = a->dQ.strideBytes;
+        hipLaunchKernelGGL(f32 ? AttGradQFromDs<true> : AttGradQFromDs<false>, dim3(a->lenRound / BROWS, a->heads), dim3(256), 0, (hipStream_t)stream, p);
         TS2_CHECK_LAUNCH();
     }
     return TS2_OK;

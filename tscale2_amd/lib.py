@@ -323,7 +323,8 @@ class AttGradArgs(C.Structure):
     _fields_ = [("len", C.c_int32), ("lenRound", C.c_int32), ("heads", C.c_int32), ("q", Mat), ("k", Mat), ("v", Mat), ("dValLookup", Mat),
                 ("spanStart", C.c_void_p), ("spanFinish", C.c_void_p), ("revLo", C.c_void_p), ("revHi", C.c_void_p),
                 ("attDotScale", C.c_float), ("alibiSlope", C.c_float), ("sumWeightLog", Mat), ("dScale", Mat), ("dQ", Mat), ("dK", Mat),
-                ("dV", Mat), ("gradType", C.c_int32), ("which", C.c_int32)]
+                ("dV", Mat), ("gradType", C.c_int32), ("which", C.c_int32), ("dsBase", C.c_void_p), ("dsScratch", C.c_void_p),
+                ("dsCapacityBlocks", C.c_int64)]
 
 
 def att_forward(len_, heads, q, k, v, span_start, span_finish, att_dot_scale, slope, val_lookup, sum_weight_log):
@@ -334,12 +335,32 @@ def att_forward(len_, heads, q, k, v, span_start, span_finish, att_dot_scale, sl
 
 
 def att_backward(len_, heads, q, k, v, dval, span_start, span_finish, rev_lo, rev_hi, att_dot_scale, slope, sum_weight_log, dscale, dq, dk,
-                 dv, grad_type, which=3):
+                 dv, grad_type, which=3, ds=None):
+    """ds: optional (dsBase, dsScratch) pair - the index of ts2_att_build_ds_index and a uint8 tensor of whole 2048-byte blocks - with which
+    dQ is formed from the score gradients the dK/dV kernel leaves behind"""
     a = AttGradArgs(len_, q.shape[0], heads, mat(q), mat(k), mat(v), mat(dval), span_start.data_ptr(), span_finish.data_ptr(),
                     rev_lo.data_ptr(), rev_hi.data_ptr(), att_dot_scale, slope, mat(sum_weight_log), mat(dscale), mat(dq), mat(dk), mat(dv),
-                    grad_type, which)
+                    grad_type, which, None, None, 0)
+    if ds is not None:
+        a.dsBase, a.dsScratch, a.dsCapacityBlocks = ds[0].data_ptr(), ds[1].data_ptr(), ds[1].numel() // 2048
     lib = load()
     lib.check(lib.dll.ts2_att_backward(C.byref(a), lib.stream()), "ts2_att_backward")
+
+
+def att_ds_scratch(len_round, heads, span_start, span_finish):
+    """(dsBase, dsScratch) for att_backward(ds=...): the block index on the device and an array sized from the host copy of the spans"""
+    import torch
+    lib = load()
+    base = torch.empty(len_round + 1, dtype=torch.int32, device="cuda")
+    lib.check(lib.dll.ts2_att_build_ds_index(C.c_int32(len_round), C.c_void_p(span_start.data_ptr()), C.c_void_p(span_finish.data_ptr()),
+                                             C.c_void_p(base.data_ptr()), lib.stream()), "ts2_att_build_ds_index")
+    hs, hf = span_start.cpu().numpy(), span_finish.cpu().numpy()
+    lib.dll.ts2_att_ds_blocks.restype = C.c_int64
+    blocks = lib.dll.ts2_att_ds_blocks(C.c_int32(len_round), hs.ctypes.data_as(C.c_void_p), hf.ctypes.data_as(C.c_void_p))
+    if blocks < 0:
+        raise RuntimeError("ts2_att_ds_blocks failed")
+    scratch = torch.empty(max(int(blocks) * heads, 1) * 2048, dtype=torch.uint8, device="cuda")
+    return base, scratch
 
 
 class ModelConfig(C.Structure):
