@@ -538,9 +538,9 @@ def bench_att_bwd(args):
     L.att_forward(n, H, q.view(i16), k.view(i16), v.view(i16), start, finish, sc, 0.0, val.view(i16), swl)
     ds.copy_((val.float() * do.float()).view(n, H, 128).sum(-1).t())
 
-    def step(which=3):
+    def step(which=3, ds_pair=None):
         L.att_backward(n, H, q.view(i16), k.view(i16), v.view(i16), do.view(i16), start, finish, rl, rh, sc, 0.0, swl, ds, dq.view(i16), dk.view(i16),
-                       dv.view(i16), L.BF16, which)
+                       dv.view(i16), L.BF16, which, ds=ds_pair)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -548,6 +548,13 @@ def bench_att_bwd(args):
     # the two kernels on their own, after the timed region (the device is warm by then)
     ms_dq = event_time_ms(lambda: step(1), args.steps)
     ms_dkdv = event_time_ms(lambda: step(2), args.steps)
+    # the optional form with 5 products: dS handed from the dK/dV kernel to a one-product dQ kernel through a scratch array
+    pair = L.att_ds_scratch(n, H, start, finish)
+    step(3, pair)
+    torch.cuda.synchronize()
+    ms_five = event_time_ms(lambda: step(3, pair), args.steps)
+    ds_mb = pair[1].numel() / 1e6
+    del pair
     pairs = B * H * (S * (S - 1) / 2)
     flop5 = 5 * 2.0 * pairs * 128
     roof = {"bound": "mfma", "achieved": flop5 / (ms * 1e-3) / 1e12, "peak": PEAK_BF16 / 1e12, "unit": "TFLOP/s", "frac": flop5 / (ms * 1e-3) / PEAK_BF16,
@@ -555,7 +562,9 @@ def bench_att_bwd(args):
     out = {"metric": "attention backward tokens/sec on 1 MI355X; TFLOPS as % of MFMA peak", "value": n / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1,
            "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": "bf16", "data": "synthetic", "config": {"workload": "causal attention backward, 16 x 2048 tokens, 16 heads x 128, bf16"},
-           "roofline": roof, "kernels": {"dq_ms": ms_dq, "dkdv_ms": ms_dkdv, "dq_products": 3, "dkdv_products": 4}}
+           "roofline": roof, "kernels": {"dq_ms": ms_dq, "dkdv_ms": ms_dkdv, "dq_products": 3, "dkdv_products": 4},
+           "five_products": {"ms": ms_five, "scratch_mbytes": ds_mb,
+                             "note": "ts2_att_grad_args.dsScratch: dS leaves the dK/dV kernel as bf16 blocks, dQ is one product over them"}}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_att(H, B, S)
     return out
