@@ -36,10 +36,29 @@ def spans_to_ranges(sp, spans, n, n_round):
     return start, finish
 
 
-def run_case(L, orc, frag_count, frag_len, window, heads, slope, seed, grad_type):
+def ragged_spans(doc_lens, window):
+    """documents of unequal length back to back: token t of a document that starts at d0 sees [max(d0, t - window), t - 1]"""
+    n = int(sum(doc_lens))
+    sp = np.zeros(n + 1, np.int32)
+    spans = []
+    t = 0
+    for ln in doc_lens:
+        d0 = t
+        for _ in range(ln):
+            a, b = max(d0, t - window), t - 1
+            if b >= a:
+                spans.append((a, b))
+            sp[t + 1] = len(spans)
+            t += 1
+    return sp, np.array(spans, np.int32).reshape(-1, 2)
+
+
+def run_case(L, orc, frag_count, frag_len, window, heads, slope, seed, grad_type, custom_spans=None):
     n = frag_count * frag_len
+    sp, spans = causal_spans(frag_count, frag_len, window) if custom_spans is None else custom_spans
+    if custom_spans is not None:
+        n = sp.size - 1
     n_round = (n + 127) // 128 * 128
-    sp, spans = causal_spans(frag_count, frag_len, window)
     r = np.random.default_rng(seed)
     # q, v are unit-rms heads and k ~ N(0,1) in the model; scaled so that logits have a realistic spread
     q = bf16_round(r.standard_normal((n, heads * 128)).astype(np.float32))
@@ -126,6 +145,19 @@ def test_attention_remapped_block_order(L, orc):
     sequence, a slope, key ranges that start inside a 64-row tile"""
     print("case att remapped order", flush=True)
     run_case(L, orc, frag_count=4, frag_len=256, window=200, heads=2, slope=0.25, seed=24, grad_type=L.BF16)
+
+
+@pytest.mark.parametrize("window,slope,seed", [(96, 0.125, 31), (1000, 0.0, 32), (40, 0.0, 33)])
+def test_attention_ragged_documents(L, orc, window, slope, seed):
+    """documents of random lengths between 1 and 400 tokens: rows without a span (first tokens), 32-row blocks that straddle document
+    starts (seen partly by one key block of a workgroup and completely by the other, so the dK/dV waves take their two-block and
+    their one-block paths in turn and the hand-over counters run through both), windows that end inside a tile"""
+    print("case att ragged documents", window, slope, flush=True)
+    r = np.random.default_rng(seed)
+    lens = []
+    while sum(lens) < 1100:
+        lens.append(int(r.integers(1, 400)))
+    run_case(L, orc, 0, 0, window, heads=2, slope=slope, seed=seed, grad_type=L.BF16, custom_spans=ragged_spans(lens, window))
 
 
 @pytest.mark.parametrize("slope", [0.0, 0.01])
