@@ -167,19 +167,26 @@ __global__ void RevInit(int *revLo, int *revHi, int n)
     }
 }
 
+// a wave takes 64 consecutive queries and issues one atomic pair per key block that any of them reaches (the queries of a wave reach
+// much the same blocks: one atomic per query and block made the few hundred block entries the bottleneck)
 __global__ void RevBuild(const int *spanStart, const int *spanFinish, int len, int *revLo, int *revHi)
 {
-    int q = blockIdx.x * blockDim.x + threadIdx.x;
-    if (q >= len) {
-        return;
+    const int q = blockIdx.x * blockDim.x + threadIdx.x;
+    int s = 0, f = -1;
+    if (q < len) {
+        s = spanStart[q];
+        f = spanFinish[q];
     }
-    int s = spanStart[q], f = spanFinish[q];
-    if (f < s) {
-        return;
-    }
-    for (int b = s / BROWS; b <= f / BROWS; ++b) {
-        atomicMin(&revLo[b], q);
-        atomicMax(&revHi[b], q);
+    const bool some = f >= s;
+    const int bLo = some ? s / BROWS : 0x7fffffff, bHi = some ? f / BROWS : -1;
+    const int wLo = __builtin_amdgcn_readfirstlane(WaveMinInt(bLo)), wHi = __builtin_amdgcn_readfirstlane(WaveMaxInt(bHi));
+    for (int b = wLo; b <= wHi; ++b) {
+        const bool touch = some && b >= bLo && b <= bHi;
+        const int qMin = WaveMinInt(touch ? q : 0x7fffffff), qMax = WaveMaxInt(touch ? q : -1);
+        if ((threadIdx.x & 63) == 0 && qMax >= 0) {
+            atomicMin(&revLo[b], qMin);
+            atomicMax(&revHi[b], qMax);
+        }
     }
 }
 
