@@ -209,6 +209,13 @@ def test_moe_routing_gather_grouped_product_and_combine_at_the_size_of_the_moe_b
     # one row recomputed directly
     i = int(eo[23]) + 5
     assert (c64[i] - w64[23] @ a64[i]).abs().max().item() <= 2e-4 * scale
+    # the same product with a 16-bit result: at this size the library runs it on the persistent kernel with the operands exchanged;
+    # same accumulators, so the bf16 rows are the fp32 ones rounded
+    c16 = torch.full((len_moe, xp), 0x1234, dtype=torch.int16, device="cuda")
+    lib.gemm_nt(grouped, w8, c16, L.E4M3, L.BF16, n=xp, tile_group=t["tile"], b_slab_bytes=xp * dim)
+    torch.cuda.synchronize()
+    assert bool((c16[eo[E]:] == 0x1234).all())
+    assert torch.equal(c16[:eo[E]].view(torch.bfloat16), c[:eo[E]].bfloat16())
     # ---- combine: res = alpha * (*alphaPtr) * sum over a token's slots, in slot order
     src = torch.randn((len_moe, dim), device="cuda", generator=g)
     ap = torch.tensor([1.5], device="cuda")

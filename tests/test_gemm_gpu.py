@@ -452,6 +452,81 @@ def test_weight_slab_chosen_per_row_tile_is_bit_exact(lib, orc):
             assert np.array_equal(got[rows], orc_gemm_i8(orc, np.ascontiguousarray(a[rows]), np.ascontiguousarray(b[g * n:(g + 1) * n])))
 
 
+@pytest.mark.parametrize("n,k,shrink,c16", [(512, 1024, 1, "bf16"), (1024, 512, 2, "bf16"), (256, 640, 0, "f16"), (512, 2048, 2, "bf16")])
+def test_grouped_products_on_the_persistent_kernel(lib, n, k, shrink, c16):
+    """The expert-grouped e4m3 product with a 16-bit result on the persistent kernel (operands exchanged: a tile is 256 result columns
+    of one expert x the 128 tokens of a row tile): bit-identical to the 128x128 kernels (same contraction order per accumulator), tiles
+    without an expert leave C alone, rows from mLive on are zeros, per-token row scales.  shrink > 0 runs many tiles per workgroup
+    (the roles of the wave groups alternate, the operand ring wraps around tile boundaries)."""
+    print(f"case grouped persistent n={n} k={k} shrink={shrink} {c16}", flush=True)
+    from tscale2_amd import lib as L
+    g = torch.Generator(device="cuda").manual_seed(100 + n + k)
+    slabs, tiles = 5, 23
+    m = tiles * 128
+    r = np.random.default_rng(n + k)
+    tg = r.integers(0, slabs, tiles).astype(np.int32)
+    tg[[3, 11, 22]] = -1
+    tg[0], tg[1] = 4, 0
+    a = (torch.randn((m, k), device="cuda", generator=g) * 4).to(torch.float8_e4m3fn).view(torch.uint8)
+    b = (torch.randn((slabs * n, k), device="cuda", generator=g) * 4).to(torch.float8_e4m3fn).view(torch.uint8)
+    rs = torch.rand((m,), device="cuda", generator=g) + 0.5
+    ct = L.F16 if c16 == "f16" else L.BF16
+    tgd = torch.from_numpy(tg).cuda()
+    m_live = m - 128 - 37  # inside the last tile that has an expert
+    res = []
+    for cfg in (32768, 4096 | (shrink << 13)):
+        c = torch.full((m, n), 0x1234, dtype=torch.int16, device="cuda")
+        lib.gemm_nt(a, b, c, L.E4M3, ct, alpha=2e-3, row_scale=rs, n=n, tile_group=tgd, b_slab_bytes=n * k, m_live=m_live, tile_config=cfg)
+        torch.cuda.synchronize()
+        res.append(c)
+    old, new = res
+    assert torch.equal(old, new)
+    for t, e in enumerate(tg):
+        rows = new[t * 128:(t + 1) * 128]
+        if e < 0:
+            assert (rows == 0x1234).all(), t
+    assert (new[m_live:m - 128] == 0).all()
+    # and against the product itself on one tile
+    t = 1
+    view = torch.float16 if c16 == "f16" else torch.bfloat16
+    af = a[t * 128:(t + 1) * 128].view(torch.float8_e4m3fn).float()
+    bf = b[tg[t] * n:(tg[t] + 1) * n].view(torch.float8_e4m3fn).float()
+    want = (af @ bf.T) * 2e-3 * rs[t * 128:(t + 1) * 128, None]
+    assert torch.allclose(new[t * 128:(t + 1) * 128].view(view).float(), want, rtol=1e-2, atol=1e-3)
+
+
+@pytest.mark.parametrize("f0,f1", [(0.7, 0.3), (0.5, 0.5), (0.9, 0.0), (0.0, 0.4)])
+def test_grouped_sum_of_two_products_on_the_persistent_kernel(lib, f0, f1):
+    """C = alpha (f0 A0 B0_g^T + f1 A1 B1_g^T) per expert-grouped row tile (the dX of an expert's expand and gate matrices): the persistent
+    kernel runs the second product's steps behind the first's and rescales the accumulators at the seam, like the two-product form of
+    the 128x128 kernel - bit-identical to it, also with a zero factor on either product"""
+    print(f"case grouped two products {f0} {f1}", flush=True)
+    from tscale2_amd import lib as L
+    g = torch.Generator(device="cuda").manual_seed(7)
+    slabs, tiles, n, k = 4, 19, 512, 512
+    m = tiles * 128
+    tg = (np.arange(tiles) % slabs).astype(np.int32)
+    tg[5] = -1
+    mk = lambda r, c: (torch.randn((r, c), device="cuda", generator=g) * 4).to(torch.float8_e4m3fn).view(torch.uint8)
+    a0, a1, b0, b1 = mk(m, k), mk(m, k), mk(slabs * n, k), mk(slabs * n, k)
+    p0, p1 = torch.full((1,), f0, device="cuda"), torch.full((1,), f1, device="cuda")
+    tgd = torch.from_numpy(tg).cuda()
+    res = []
+    for cfg in (32768, 4096 | (2 << 13)):
+        c = torch.full((m, n), 0x1234, dtype=torch.int16, device="cuda")
+        lib.gemm_nt(a0, b0, c, L.E4M3, L.BF16, alpha=3e-3, alpha_ptr=p0, n=n, tile_group=tgd, b_slab_bytes=n * k, tile_config=cfg,
+                    segments=((a1, b1, 3e-3, p1),))
+        torch.cuda.synchronize()
+        res.append(c)
+    assert torch.equal(res[0], res[1])
+    assert (res[1][5 * 128:6 * 128] == 0x1234).all()
+    t = 2
+    rows = slice(t * 128, (t + 1) * 128)
+    f = lambda x: x.view(torch.float8_e4m3fn).float()
+    want = 3e-3 * (f0 * f(a0[rows]) @ f(b0[tg[t] * n:(tg[t] + 1) * n]).T + f1 * f(a1[rows]) @ f(b1[tg[t] * n:(tg[t] + 1) * n]).T)
+    assert torch.allclose(res[1][rows].view(torch.bfloat16).float(), want, rtol=1e-2, atol=2e-3)
+
+
 @pytest.mark.parametrize("zero_at", [(0,), (1,), (3,), (1, 2), (0, 1, 2, 3)])
 def test_products_with_a_zero_factor_contribute_nothing(zero_at):
     """a device-resident factor of zero (the scale of an all-zero matrix) on any of the products of a one-launch sum: the product is

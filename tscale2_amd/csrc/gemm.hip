@@ -1220,6 +1220,9 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
             if (ct < 0 || splitK > 1 || (a->tileConfig & (4 | 8 | 16))) {
                 return TS2_ERR_UNSUPPORTED;
             }
+            if (p.tileGroup) {
+                return RunPingGrouped(p, type, ct, epi, stream);
+            }
             return RunPing(p, type, ct, epi, stream);
         }
         if (a->tileConfig & 2048) {
@@ -1234,6 +1237,12 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
         // 482, fp32 546 -> 497; 32768 x 2048 x 2048 fp32 142 -> 127; equal at 4096 bytes and beyond.  Bit 15 of tileConfig keeps the
         // old kernels (comparison).
         static const bool noPersistent = getenv("TS2_GEMM_NO_PERSISTENT") != nullptr; // (comparison runs of whole models)
+        // Expert-grouped products with a 16-bit result: the persistent kernel on the exchanged operands (a tile = 256 result columns
+        // of one expert x the 128 tokens of a row tile) when the result has 256-column chunks and there are two tiles per CU.
+        if (!noPersistent && p.tileGroup && (a->tileConfig & (3 | 4 | 8 | 16 | 128 | 32768)) == 0 && ct >= 0 && splitK <= 1 &&
+            (int64_t)(a->m / 128) * (a->n / 256) >= 512 && PingGroupedCanRun(p, type, ct, epi)) {
+            return RunPingGrouped(p, type, ct, epi, stream);
+        }
         if (!noPersistent && (a->tileConfig & (3 | 4 | 8 | 16 | 32768)) == 0 && ct >= 0 && epi == TS2_EPI_STORE && splitK <= 1 && p.kBytes >= 1024 && p.kBytes < 4096 &&
             (ct == C_F32 || ct == C_BF16 || ct == C_F16 || ct == C_BF16NORM) && (int64_t)(a->m / 256) * (a->n / 128) >= 512 &&
             PingCanRun(p, type, ct, epi)) {

@@ -853,4 +853,6 @@ int RunTwin(const GemmP &p, int type, int ct, int epi, hipStream_t stream);
 // The persistent eight-wave kernel whose epilogue runs under the next tile's main loop (gemm_ping.hip)
 bool PingCanRun(const GemmP &p, int type, int ct, int epi);
 int RunPing(const GemmP &p, int type, int ct, int epi, hipStream_t stream);
+bool PingGroupedCanRun(const GemmP &p, int type, int ct, int epi);
+int RunPingGrouped(const GemmP &p, int type, int ct, int epi, hipStream_t stream);
 } // namespace gemmk

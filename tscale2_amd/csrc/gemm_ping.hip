@@ -51,7 +51,12 @@ __device__ __forceinline__ v4i MakeRsrc(const uint8_t *base, int64_t off, int by
     return r;
 }
 
-template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(512, 2) GemmNTPing(PingP pp)
+// GRP (expert-grouped products, e4m3, 16-bit result): the roles of the operands are exchanged.  The 256-row side of a tile holds rows
+// of the weight slab of the tile's expert (p.a = the slabs, p.bSlab apart), the 128-row side the 128 tokens of one row tile of the
+// expert-ordered activations (p.b), whose expert p.tileGroup names (-1: nothing is stored).  A block of accumulators is then C^T:
+// a lane owns a token and four consecutive result columns per register quad, and the wave's 64 columns of 32 tokens leave as whole
+// 128-byte row segments through 4 KB of the wave's own LDS, one token block per slot.
+template <int TYPE, int CT, int EPI, bool GRP = false> __global__ void __launch_bounds__(512, 2) GemmNTPing(PingP pp)
 {
     typedef typename AccT<TYPE>::type TAcc;
     const GemmP &p = pp.g;
@@ -59,7 +64,8 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(512, 2) G
     // the normalising epilogue works on transposed blocks (a lane owns a row): the MFMAs take their operands the other way round
     constexpr bool SWAPC = CT == C_BF16NORM;
     __shared__ __attribute__((aligned(1024))) uint8_t lds[PLDS];
-    __shared__ __attribute__((aligned(1024))) uint8_t ldsEpi[CT == C_BF16NORM ? 16384 : 16]; // 4 KB per wave of the storing group
+    static_assert(!GRP || ((CT == C_BF16 || CT == C_F16) && EPI == TS2_EPI_STORE && TYPE == T_FP8), "grouped: e4m3 operands, 16-bit result");
+    __shared__ __attribute__((aligned(1024))) uint8_t ldsEpi[CT == C_BF16NORM || GRP ? 16384 : 16]; // 4 KB per wave of the storing group
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -67,7 +73,31 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(512, 2) G
     const int group = wave >> 2; // waves w and w + 4 share a SIMD
     const int gw = wave & 3;
     const int half = lane >> 5, l32 = lane & 31;
-    const int kSlots = p.kBytes / PK;
+    // grouped products may add a second product of the same shapes into the same accumulators (p.nSeg == 2: operands segA[0], segB[0]):
+    // its steps follow the first product's, and at the seam the accumulators are brought to the second product's factor, which is the
+    // one the epilogue applies - the same arithmetic as the two-product form of the 128x128 kernel.  A second factor of zero (the scale
+    // of an all-zero matrix) leaves the first product alone.
+    const int kSlots1 = p.kBytes / PK;
+    bool twoProducts = false;
+    float seamRatio = 1.f, unitsOfSum = 0.f;
+    if constexpr (GRP) {
+        if (p.nSeg == 2) {
+            float cur = p.alpha, nxt = p.segAlpha[0];
+            if (p.alphaPtr) {
+                cur *= *p.alphaPtr;
+            }
+            if (p.segAlphaPtr[0]) {
+                nxt *= *p.segAlphaPtr[0];
+            }
+            unitsOfSum = cur;
+            if (nxt != 0) {
+                twoProducts = true;
+                unitsOfSum = nxt;
+                seamRatio = cur / nxt;
+            }
+        }
+    }
+    const int kSlots = twoProducts ? 2 * kSlots1 : kSlots1;
     const int myTiles = ((int)blockIdx.x < pp.nTiles) ? (pp.nTiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x : 0;
     const unsigned ldsBase = (unsigned)(uintptr_t)(TLds)lds;
     const int lda = (int)p.lda, ldb = (int)p.ldb;
@@ -86,12 +116,18 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(512, 2) G
         *rowBase = tm * PBM;
         *colBase = tn * PBN;
     };
-    auto tileRsrc = [&](int i, v4i *ra, v4i *rb) {
+    auto tileRsrcOf = [&](const uint8_t *baseA, const uint8_t *baseB, int i, v4i *ra, v4i *rb) {
         int rowBase, colBase;
         tileOrigin(i < myTiles ? i : myTiles - 1, &rowBase, &colBase);
-        *ra = MakeRsrc(p.a, (int64_t)rowBase * p.lda, (PBM - 1) * lda + p.kBytes);
-        *rb = MakeRsrc(p.b, (int64_t)colBase * p.ldb, (PBN - 1) * ldb + p.kBytes);
+        int64_t slab = 0;
+        if constexpr (GRP) {
+            const int g = p.tileGroup[colBase / PBN];
+            slab = g > 0 ? g * p.bSlab : 0; // (a tile without an expert multiplies the first slab and stores nothing)
+        }
+        *ra = MakeRsrc(baseA, slab + (int64_t)rowBase * p.lda, (PBM - 1) * lda + p.kBytes);
+        *rb = MakeRsrc(baseB, (int64_t)colBase * p.ldb, (PBN - 1) * ldb + p.kBytes);
     };
+    auto tileRsrc = [&](int i, v4i *ra, v4i *rb) { tileRsrcOf(p.a, p.b, i, ra, rb); };
 #define PING_LOAD(M0VAL, VOFF, RSRC, SOFF)                                                                                                 \
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(M0VAL), "v"(VOFF), "s"(RSRC), "s"(SOFF) : "memory")
     // load number I (0..11) of a step: the first 8 are A blocks gw + 4 * I, the others B blocks
@@ -224,7 +260,12 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(512, 2) G
     if (p.alphaPtr) {
         scale *= *p.alphaPtr;
     }
-    const int mLive = p.mLive > 0 ? p.mLive : p.m;
+    if constexpr (GRP) {
+        if (p.nSeg == 2) {
+            scale = unitsOfSum;
+        }
+    }
+    const int mLive = p.mLive > 0 ? p.mLive : GRP ? p.n : p.m;
     // old values of block (i, j) for the accumulating epilogue: fetched one piece ahead
     auto loadOld = [&](auto iTag, auto jTag, int rowBase, int colBase, float (&old)[16]) {
         constexpr int i = decltype(iTag)::value, j = decltype(jTag)::value;
@@ -306,7 +347,7 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(512, 2) G
     // piece of a block row normalises, rotates and packs the row's 128 columns (pk) and sends columns 0..63 on their way, the second
     // piece columns 64..127: the rows are staged in 4 KB of the wave's own LDS (128 bytes per row, 8-byte granules XOR-swizzled by the
     // row pair) and leave as 16-byte stores of whole 128-byte row segments, eight lanes per row.
-    uint8_t *waveEpi = ldsEpi + (CT == C_BF16NORM ? gw * 4096 : 0);
+    uint8_t *waveEpi = ldsEpi + (CT == C_BF16NORM || GRP ? gw * 4096 : 0);
     auto normPack = [&](auto iTag, int rowBase, int colBase, uint2 (&pk)[4][4]) {
         constexpr int i = decltype(iTag)::value;
         const int row = rowBase + gw * 64 + i * 32 + l32;
@@ -354,6 +395,46 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(512, 2) G
             }
         }
     };
+    // grouped products: token block j of the tile (32 tokens x the wave's 64 result columns); rowBase = first result column of the tile,
+    // colBase = its first token
+    auto grpFlush = [&](auto jTag, int rowBase, int colBase) {
+        constexpr int j = decltype(jTag)::value;
+        typedef unsigned v4u_t __attribute__((ext_vector_type(4)));
+        const int token = colBase + j * 32 + l32;
+        const bool live = token < mLive;
+        float rs = scale;
+        if (p.rowScale) {
+            rs *= p.rowScale[token];
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float v0 = live ? (float)acc[i][j][4 * q] * rs : 0.f, v1 = live ? (float)acc[i][j][4 * q + 1] * rs : 0.f;
+                const float v2 = live ? (float)acc[i][j][4 * q + 2] * rs : 0.f, v3 = live ? (float)acc[i][j][4 * q + 3] * rs : 0.f;
+                const int g = (i * 8 + q * 2 + half) ^ (((l32 >> 1) & 7) << 1);
+                *(uint2 *)(waveEpi + l32 * 128 + g * 8) =
+                    CT == C_F16 ? make_uint2(PackF16x2(v0, v1), PackF16x2(v2, v3)) : make_uint2(PackBf16x2(v0, v1), PackBf16x2(v2, v3));
+            }
+        }
+        const int firstToken = colBase + j * 32;
+        const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(p.c + (int64_t)firstToken * p.ldc), 0, (int)(32 * p.ldc), 0x00020000);
+        const int ldc = (int)p.ldc;
+        const int t8 = lane & 7, rsub = lane >> 3;
+        const int laneOff = rsub * ldc + (rowBase + gw * 64) * 2 + t8 * 16;
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int r = it * 8 + rsub;
+            const int g = (2 * t8) ^ (((r >> 1) & 7) << 1);
+            const uint4 d = *(const uint4 *)(waveEpi + r * 128 + g * 8);
+            const int so = it * 8 * ldc;
+            if (p.streamC) {
+                __builtin_amdgcn_raw_buffer_store_b128((v4u_t){d.x, d.y, d.z, d.w}, rsrc, laneOff, so, 2);
+            } else {
+                __builtin_amdgcn_raw_buffer_store_b128((v4u_t){d.x, d.y, d.z, d.w}, rsrc, laneOff, so, 0);
+            }
+        }
+    };
     // the whole epilogue of tile number t of this workgroup, one block per slot; nBarriers slot barriers are kept in all
     auto epiloguePhase = [&](int t, int nBarriers) {
         int rowBase, colBase;
@@ -371,7 +452,24 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(512, 2) G
     } while (0)
         // (the first piece waits for the loads this group issued in its last two slots as the multiplying group)
 #define WAIT_OWN_LOADS() asm volatile("s_waitcnt vmcnt(0)" ::: "memory")
-        if constexpr (CT == C_BF16NORM) {
+        if constexpr (GRP) {
+            const bool hasExpert = p.tileGroup[colBase / PBN] >= 0;
+#define GPIECE(J)                                                                                                                          \
+    do {                                                                                                                                   \
+        if ((J) == 0) {                                                                                                                    \
+            WAIT_OWN_LOADS();                                                                                                              \
+        }                                                                                                                                  \
+        if (hasExpert) {                                                                                                                   \
+            grpFlush(std::integral_constant<int, J>(), rowBase, colBase);                                                                  \
+        }                                                                                                                                  \
+        END_PIECE();                                                                                                                       \
+    } while (0)
+            GPIECE(0);
+            GPIECE(1);
+            GPIECE(2);
+            GPIECE(3);
+#undef GPIECE
+        } else if constexpr (CT == C_BF16NORM) {
             uint2 pk[4][4];
 #define NPIECE(I)                                                                                                                          \
     do {                                                                                                                                   \
@@ -477,14 +575,42 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(512, 2) G
             FENCE();
             tileRsrc(t, &ra, &rb);
             tileRsrc(t + 1, &na, &nb);
+            v4i ra2 = ra, rb2 = rb; // second product of a grouped sum
+            if constexpr (GRP) {
+                if (twoProducts) {
+                    tileRsrcOf(p.segA[0], p.segB[0], t, &ra2, &rb2);
+                }
+            }
             for (int s = 0; s < kSlots - 1; ++s) {
                 // step s + 2 of this tile, or step s + 2 - kSlots of the next one (of the last tile again when there is none: harmless,
                 // and the count of loads in flight stays the same)
                 const bool wrap = s + 2 >= kSlots;
-                const v4i la = wrap ? na : ra, lb = wrap ? nb : rb;
-                const int kOff = (wrap ? s + 2 - kSlots : s + 2) * PK;
+                const bool second = GRP && !wrap && s + 2 >= kSlots1;
+                const v4i la = wrap ? na : second ? ra2 : ra, lb = wrap ? nb : second ? rb2 : rb;
+                const int kOff = (wrap ? s + 2 - kSlots : second ? s + 2 - kSlots1 : s + 2) * PK;
                 SLOT(stC, stN, stL, la, lb, kOff, false);
                 ROTATE(1);
+                if constexpr (GRP) {
+                    if (twoProducts && s == kSlots1 - 1) {
+                        // the seam: the first product's sums in units of the second's factor (wait states of the last MFMAs spelled out)
+                        FENCE();
+                        asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+                        FENCE();
+#pragma unroll
+                        for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+                            for (int j = 0; j < WTN; ++j) {
+#pragma unroll
+                                for (int e = 0; e < 16; ++e) {
+                                    acc[i][j][e] *= seamRatio;
+                                }
+                            }
+                        }
+                        FENCE();
+                        asm volatile("s_nop 4" ::: "memory");
+                        FENCE();
+                    }
+                }
             }
             SLOT(stC, stN, stL, na, nb, PK, true); // loads step kSlots + 1 = step 1 of the next tile
             ROTATE(1);
@@ -509,7 +635,7 @@ template <int TYPE, int CT, int EPI> __global__ void __launch_bounds__(512, 2) G
 #undef PING_LOAD
 }
 
-template <int TYPE, int CT, int EPI> int LaunchPing(const GemmP &p, hipStream_t stream)
+template <int TYPE, int CT, int EPI, bool GRP = false> int LaunchPing(const GemmP &p, hipStream_t stream)
 {
     PingP q;
     q.g = p;
@@ -538,7 +664,7 @@ template <int TYPE, int CT, int EPI> int LaunchPing(const GemmP &p, hipStream_t 
         const int chunk = (grid % 8) == 0 ? grid / 8 : grid;
         q.g.mapGroup = chunk >= 128 ? 8 : chunk >= 16 ? 4 : 2;
     }
-    hipLaunchKernelGGL((GemmNTPing<TYPE, CT, EPI>), dim3(grid), dim3(512), 0, stream, q);
+    hipLaunchKernelGGL((GemmNTPing<TYPE, CT, EPI, GRP>), dim3(grid), dim3(512), 0, stream, q);
     TS2_CHECK_LAUNCH();
     return TS2_OK;
 }
@@ -589,6 +715,45 @@ bool PingCanRun(const GemmP &p, int type, int ct, int epi)
         return false; // a tile's rows are addressed from one 32-bit offset
     }
     return true;
+}
+
+// expert-grouped product C[m][n] = A[m][k] * B_g[n][k] with g = tileGroup[row / 128]: the persistent kernel on the exchanged operands
+bool PingGroupedCanRun(const GemmP &p, int type, int ct, int epi)
+{
+    if (!p.tileGroup || type != T_FP8 || (ct != C_BF16 && ct != C_F16) || epi != TS2_EPI_STORE) {
+        return false;
+    }
+    if (p.m % PBN || p.n % PBM || p.kBytes % PK || p.kBytes < 4 * PK) {
+        return false; // (a tile's epilogue is four pieces, one per slot of the next tile)
+    }
+    if (p.groupOffsets || p.kTileScale || p.kMajor || p.splitK > 1 || p.splits > 1 || p.nSeg > 2) {
+        return false;
+    }
+    if ((((uintptr_t)p.c | (uintptr_t)p.ldc) & 15) || (int64_t)32 * p.ldc >= ((int64_t)1 << 31)) {
+        return false;
+    }
+    if ((int64_t)(PBM - 1) * p.ldb + p.kBytes >= ((int64_t)1 << 31) || (int64_t)(PBN - 1) * p.lda + p.kBytes >= ((int64_t)1 << 31)) {
+        return false;
+    }
+    return true;
+}
+
+int RunPingGrouped(const GemmP &p, int type, int ct, int epi, hipStream_t stream)
+{
+    if (!PingGroupedCanRun(p, type, ct, epi)) {
+        return TS2_ERR_UNSUPPORTED;
+    }
+    GemmP q = p;
+    q.a = p.b;
+    q.lda = p.ldb;
+    q.b = p.a;
+    q.ldb = p.lda;
+    q.m = p.n;
+    q.n = p.m;
+    q.mLive = p.mLive > 0 ? p.mLive : p.m;
+    q.segA[0] = p.segB[0];
+    q.segB[0] = p.segA[0];
+    return ct == C_F16 ? LaunchPing<T_FP8, C_F16, TS2_EPI_STORE, true>(q, stream) : LaunchPing<T_FP8, C_BF16, TS2_EPI_STORE, true>(q, stream);
 }
 
 int RunPing(const GemmP &p, int type, int ct, int epi, hipStream_t stream)
