@@ -623,10 +623,10 @@ def bench_moe_fp8(args):
     c = torch.empty((rows, xp), dtype=torch.bfloat16, device="cuda")   # 16-bit results, as every grouped product of the layer stores them
     grp = (torch.arange(rows // 128, device="cuda", dtype=torch.int32) * experts // (rows // 128)).int().contiguous()
     grouped = lambda: lib.gemm_nt(a, b, c, L.E4M3, L.BF16, n=xp, tile_group=grp, b_slab_bytes=xp * dim)
-    for _ in range(20):
+    for _ in range(300):   # (a launch is under 0.1 ms: the clocks take some 20 ms of load to settle after the set-up above)
         grouped()
     torch.cuda.synchronize()
-    ms_g = event_time_ms(grouped, 100)
+    ms_g = event_time_ms(grouped, 300)
     gops = 2.0 * rows * xp * dim
     roof = {"bound": "mfma", "achieved": gops / (ms_g * 1e-3) / 1e12, "peak": PEAK_FP8 / 1e12, "unit": "TFLOP/s",
             "frac": gops / (ms_g * 1e-3) / PEAK_FP8, "traffic": None,

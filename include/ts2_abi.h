@@ -101,7 +101,10 @@ typedef struct ts2_gemm_args {
      * tile's main loop (m % 256 = 0, k >= 1024 bytes; fp32 / 16-bit / raw int32 results, store or accumulate), bits 13-14 its
      * workgroup count as CUs >> 2, 4, 6 (tests).  Bits 11 and 12 return TS2_ERR_UNSUPPORTED for calls their kernel cannot run.  With
      * bits 0-4 clear the persistent kernel is also chosen automatically for stored results with 1024 <= k bytes < 4096 and at least
-     * 512 tiles of 256x128; bit 15 (32768) switches that off. */
+     * 512 tiles of 256x128; bit 15 (32768) switches that off.  The same kernel, on exchanged operands, takes tileGroup products
+     * of TS2_E4M3 operands with a 16-bit stored result (plain or ROW_TILE_NORM; also with one further product) when n % 256 = 0,
+     * k >= 512 bytes, c and its stride are multiples of 16 bytes and (m/128)*(n/256) >= 512 - or when bit 12 asks for it;
+     * results are bit-identical to the 128x128 kernels'. */
     int32_t tileConfig;
     /* Expert-grouped products (TMoeMatMulKernelCall / TMoeDeltaMatMulKernelCall, src/gpt/compute/moe_matmul.cuh:47-215):
      * tileGroup [m/128] (device): rows of A and C are grouped by expert in 128-row tiles; tile i multiplies the B slab

@@ -495,6 +495,42 @@ def test_grouped_products_on_the_persistent_kernel(lib, n, k, shrink, c16):
     assert torch.allclose(new[t * 128:(t + 1) * 128].view(view).float(), want, rtol=1e-2, atol=1e-3)
 
 
+@pytest.mark.parametrize("n,k,tiles,shrink", [(512, 1024, 23, 1), (256, 512, 9, 2), (1024, 640, 8, 2), (256, 1024, 1, 0)])
+def test_grouped_normalised_products_on_the_persistent_kernel(lib, n, k, tiles, shrink):
+    """The expert-grouped product with the row-tile normalising epilogue (the experts' expand product) on the persistent kernel: a
+    token's 128-column tile is held by two waves, which exchange their sums of squares through LDS.  Normalised bf16 rows and tile
+    scales bit-identical to the 128x128 kernel's; odd and even numbers of tiles per workgroup (either wave group ends the list)."""
+    print(f"case grouped persistent normalised n={n} k={k} tiles={tiles} shrink={shrink}", flush=True)
+    from tscale2_amd import lib as L
+    g = torch.Generator(device="cuda").manual_seed(300 + n + k + tiles)
+    slabs = 3
+    m = tiles * 128
+    tg = (np.arange(tiles) * 7 % slabs).astype(np.int32)
+    if tiles > 4:
+        tg[4] = -1
+    a = (torch.randn((m, k), device="cuda", generator=g) * 4).to(torch.float8_e4m3fn).view(torch.uint8)
+    b = (torch.randn((slabs * n, k), device="cuda", generator=g) * 4).to(torch.float8_e4m3fn).view(torch.uint8)
+    tgd = torch.from_numpy(tg).cuda()
+    m_live = m - 50 if tg[-1] >= 0 else m
+    res = []
+    for cfg in (32768, 4096 | (shrink << 13)):
+        c = torch.full((m, n), 0x1234, dtype=torch.int16, device="cuda")
+        ts = torch.full((n // 128, m), -3.0, device="cuda")
+        lib.gemm_nt(a, b, c, L.E4M3, L.BF16, alpha=2e-3, n=n, tile_group=tgd, b_slab_bytes=n * k, m_live=m_live, tile_config=cfg,
+                    epilogue=L.EPI_ROW_TILE_NORM, normalize=True, vec_scale=1 / 24.0, tile_scale=ts)
+        torch.cuda.synchronize()
+        res.append((c, ts))
+    assert torch.equal(res[0][0], res[1][0])
+    assert torch.equal(res[0][1], res[1][1])
+    c, ts = res[1]
+    if tiles > 4:
+        assert (c[4 * 128:5 * 128] == 0x1234).all() and (ts[:, 4 * 128:5 * 128] == -3.0).all()
+    # normalised: mean square of a tile = (1 / vecScale)^2
+    t = 1 if tiles > 1 else 0
+    x = c[t * 128:t * 128 + 64].view(torch.bfloat16).float().view(64, n // 128, 128)
+    assert torch.allclose((x * x).mean(2), torch.full((64, n // 128), 576.0, device="cuda"), rtol=2e-2)
+
+
 @pytest.mark.parametrize("f0,f1", [(0.7, 0.3), (0.5, 0.5), (0.9, 0.0), (0.0, 0.4)])
 def test_grouped_sum_of_two_products_on_the_persistent_kernel(lib, f0, f1):
     """C = alpha (f0 A0 B0_g^T + f1 A1 B1_g^T) per expert-grouped row tile (the dX of an expert's expand and gate matrices): the persistent

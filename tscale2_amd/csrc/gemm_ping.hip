@@ -55,16 +55,19 @@ __device__ __forceinline__ v4i MakeRsrc(const uint8_t *base, int64_t off, int by
 // of the weight slab of the tile's expert (p.a = the slabs, p.bSlab apart), the 128-row side the 128 tokens of one row tile of the
 // expert-ordered activations (p.b), whose expert p.tileGroup names (-1: nothing is stored).  A block of accumulators is then C^T:
 // a lane owns a token and four consecutive result columns per register quad, and the wave's 64 columns of 32 tokens leave as whole
-// 128-byte row segments through 4 KB of the wave's own LDS, one token block per slot.
+// 128-byte row segments through 4 KB of the wave's own LDS, one token block per slot.  With the normalising epilogue a token's 128-column
+// tile spans two waves (64 columns each): in a first piece every wave leaves its sums of squares in its partner's LDS area, the slot
+// barrier separates that from the partner reading them, and the four token blocks follow.  The last tile of a workgroup has no slot
+// barriers left, so there the group that is already done keeps one barrier for the other's exchange.
 template <int TYPE, int CT, int EPI, bool GRP = false> __global__ void __launch_bounds__(512, 2) GemmNTPing(PingP pp)
 {
     typedef typename AccT<TYPE>::type TAcc;
     const GemmP &p = pp.g;
     constexpr int WTM = 2, WTN = 4;
     // the normalising epilogue works on transposed blocks (a lane owns a row): the MFMAs take their operands the other way round
-    constexpr bool SWAPC = CT == C_BF16NORM;
+    constexpr bool SWAPC = CT == C_BF16NORM && !GRP;
     __shared__ __attribute__((aligned(1024))) uint8_t lds[PLDS];
-    static_assert(!GRP || ((CT == C_BF16 || CT == C_F16) && EPI == TS2_EPI_STORE && TYPE == T_FP8), "grouped: e4m3 operands, 16-bit result");
+    static_assert(!GRP || ((CT == C_BF16 || CT == C_F16 || CT == C_BF16NORM) && EPI == TS2_EPI_STORE && TYPE == T_FP8), "grouped: e4m3 operands, 16-bit result");
     __shared__ __attribute__((aligned(1024))) uint8_t ldsEpi[CT == C_BF16NORM || GRP ? 16384 : 16]; // 4 KB per wave of the storing group
 
     const int tid = threadIdx.x;
@@ -397,7 +400,31 @@ template <int TYPE, int CT, int EPI, bool GRP = false> __global__ void __launch_
     };
     // grouped products: token block j of the tile (32 tokens x the wave's 64 result columns); rowBase = first result column of the tile,
     // colBase = its first token
-    auto grpFlush = [&](auto jTag, int rowBase, int colBase) {
+    // sums of squares of this wave's 64 columns for the tokens of the tile (lane = token l32 of block j; both half waves get the sum)
+    auto grpSums = [&](int colBase, float (&own)[4]) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int token = colBase + j * 32 + l32;
+            const bool live = token < mLive;
+            float rs = scale;
+            if (p.rowScale) {
+                rs *= p.rowScale[token];
+            }
+            float sum = 0;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const float x = live ? (float)acc[i][j][e] * rs : 0.f;
+                    sum += x * x;
+                }
+            }
+            float a, b;
+            LaneSwap32(sum, &a, &b);
+            own[j] = a + b;
+        }
+    };
+    auto grpFlush = [&](auto jTag, int rowBase, int colBase, float tileSum2) {
         constexpr int j = decltype(jTag)::value;
         typedef unsigned v4u_t __attribute__((ext_vector_type(4)));
         const int token = colBase + j * 32 + l32;
@@ -406,12 +433,24 @@ template <int TYPE, int CT, int EPI, bool GRP = false> __global__ void __launch_
         if (p.rowScale) {
             rs *= p.rowScale[token];
         }
+        float v[2][16];
+        if constexpr (CT == C_BF16NORM) {
+            TAcc two[2] = {acc[0][j], acc[1][j]};
+            NormRowValues<true, 2>(p, two, token, live, rs, (rowBase + gw * 64) / TILE, (gw & 1) * 64, half, (gw & 1) == 0, tileSum2, v);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    v[i][e] = live ? (float)acc[i][j][e] * rs : 0.f;
+                }
+            }
+        }
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const float v0 = live ? (float)acc[i][j][4 * q] * rs : 0.f, v1 = live ? (float)acc[i][j][4 * q + 1] * rs : 0.f;
-                const float v2 = live ? (float)acc[i][j][4 * q + 2] * rs : 0.f, v3 = live ? (float)acc[i][j][4 * q + 3] * rs : 0.f;
+                const float v0 = v[i][4 * q], v1 = v[i][4 * q + 1], v2 = v[i][4 * q + 2], v3 = v[i][4 * q + 3];
                 const int g = (i * 8 + q * 2 + half) ^ (((l32 >> 1) & 7) << 1);
                 *(uint2 *)(waveEpi + l32 * 128 + g * 8) =
                     CT == C_F16 ? make_uint2(PackF16x2(v0, v1), PackF16x2(v2, v3)) : make_uint2(PackBf16x2(v0, v1), PackBf16x2(v2, v3));
@@ -442,6 +481,7 @@ template <int TYPE, int CT, int EPI, bool GRP = false> __global__ void __launch_
         // the compiler does not see the MFMAs inside the asm statements: the wait states between the last one and the first read of a
         // result are spelled out
         asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+        FENCE(); // (no accumulator is read above this line)
         int done = 0;
 #define END_PIECE()                                                                                                                        \
     do {                                                                                                                                   \
@@ -454,13 +494,32 @@ template <int TYPE, int CT, int EPI, bool GRP = false> __global__ void __launch_
 #define WAIT_OWN_LOADS() asm volatile("s_waitcnt vmcnt(0)" ::: "memory")
         if constexpr (GRP) {
             const bool hasExpert = p.tileGroup[colBase / PBN] >= 0;
+            float tileSum2[4] = {0.f, 0.f, 0.f, 0.f};
+            if constexpr (CT == C_BF16NORM) {
+                float own[4];
+                grpSums(colBase, own);
+                WAIT_OWN_LOADS();
+                float *mine = (float *)waveEpi, *theirs = (float *)(ldsEpi + (gw ^ 1) * 4096);
+                if (half == 0) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        theirs[j * 32 + l32] = own[j];
+                    }
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                END_PIECE();
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    tileSum2[j] = own[j] + mine[j * 32 + l32];
+                }
+            }
 #define GPIECE(J)                                                                                                                          \
     do {                                                                                                                                   \
-        if ((J) == 0) {                                                                                                                    \
+        if ((J) == 0 && CT != C_BF16NORM) {                                                                                                \
             WAIT_OWN_LOADS();                                                                                                              \
         }                                                                                                                                  \
         if (hasExpert) {                                                                                                                   \
-            grpFlush(std::integral_constant<int, J>(), rowBase, colBase);                                                                  \
+            grpFlush(std::integral_constant<int, J>(), rowBase, colBase, tileSum2[J]);                                                     \
         }                                                                                                                                  \
         END_PIECE();                                                                                                                       \
     } while (0)
@@ -616,9 +675,14 @@ template <int TYPE, int CT, int EPI, bool GRP = false> __global__ void __launch_
             ROTATE(1);
             // ---- phase t + 1: store tile t, under the other group's tile if there is one
             const bool more = t + 1 < myTiles;
-            epiloguePhase(t, more ? kSlots : 0);
+            epiloguePhase(t, more ? kSlots : (GRP && CT == C_BF16NORM) ? 1 : 0);
             if (more) {
                 ROTATE(kSlots % 3);
+            }
+        }
+        if constexpr (GRP && CT == C_BF16NORM) {
+            if (((myTiles - 1) & 1) != group) {
+                SLOT_BARRIER(); // the other group's last epilogue exchanges its sums across this barrier
             }
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -720,7 +784,7 @@ bool PingCanRun(const GemmP &p, int type, int ct, int epi)
 // expert-grouped product C[m][n] = A[m][k] * B_g[n][k] with g = tileGroup[row / 128]: the persistent kernel on the exchanged operands
 bool PingGroupedCanRun(const GemmP &p, int type, int ct, int epi)
 {
-    if (!p.tileGroup || type != T_FP8 || (ct != C_BF16 && ct != C_F16) || epi != TS2_EPI_STORE) {
+    if (!p.tileGroup || type != T_FP8 || (ct != C_BF16 && ct != C_F16 && ct != C_BF16NORM) || epi != TS2_EPI_STORE || (ct == C_BF16NORM && p.nSeg > 1)) {
         return false;
     }
     if (p.m % PBN || p.n % PBM || p.kBytes % PK || p.kBytes < 4 * PK) {
@@ -753,7 +817,9 @@ int RunPingGrouped(const GemmP &p, int type, int ct, int epi, hipStream_t stream
     q.mLive = p.mLive > 0 ? p.mLive : p.m;
     q.segA[0] = p.segB[0];
     q.segB[0] = p.segA[0];
-    return ct == C_F16 ? LaunchPing<T_FP8, C_F16, TS2_EPI_STORE, true>(q, stream) : LaunchPing<T_FP8, C_BF16, TS2_EPI_STORE, true>(q, stream);
+    return ct == C_F16        ? LaunchPing<T_FP8, C_F16, TS2_EPI_STORE, true>(q, stream)
+           : ct == C_BF16NORM ? LaunchPing<T_FP8, C_BF16NORM, TS2_EPI_STORE, true>(q, stream)
+                              : LaunchPing<T_FP8, C_BF16, TS2_EPI_STORE, true>(q, stream);
 }
 
 int RunPing(const GemmP &p, int type, int ct, int epi, hipStream_t stream)
