@@ -28,6 +28,19 @@ PEAK_BF16 = 2.5e15
 PEAK_HBM = 8.0e12
 
 
+def settle(fn, ms=40.0):
+    """runs fn back to back for about `ms` milliseconds of GPU time, untimed.  After a pause in the launch stream (set-up, allocation,
+    a CPU leg) the shader clock needs some 20 ms of load to reach the value it then holds: launches timed before that read 10-25 %
+    slow (measured: a 76 us kernel at 114, 93, 84, 80, 79, 77, 76 us over its first blocks of 50 launches).  Every timed region of
+    kernels shorter than the warm-up steps of the command line starts behind this."""
+    import torch
+    torch.cuda.synchronize()
+    one = event_time_ms(fn, 1)
+    for _ in range(min(4000, int(ms / max(one, 1e-3)))):
+        fn()
+    torch.cuda.synchronize()
+
+
 def event_time_ms(fn, iters):
     import torch
     e0 = torch.cuda.Event(enable_timing=True)
@@ -136,7 +149,9 @@ def linear_i8_gemm_times(c, iters=20):
     """the two int8 MFMA GEMMs (dX and delta, 137.44 GOP each) timed alone with events on the launch stream"""
     from tscale2_amd import lib as L
     bufs, len_, src_dim, grad_dim, k_tile, splits = c["bufs"], c["len"], c["src_dim"], c["grad_dim"], c["k_tile"], c["splits"]
-    ms_dx = event_time_ms(lambda: bufs.backprop(len_, None, 1.0, None, c["dx"], L.F32), iters)
+    dx = lambda: bufs.backprop(len_, None, 1.0, None, c["dx"], L.F32)  # noqa: E731
+    settle(dx)
+    ms_dx = event_time_ms(dx, iters)
     tsc, gt, st = bufs.t["tileScale"], bufs.t["gradT"], bufs.t["srcT"]
     lib = L.load()
 
@@ -147,6 +162,7 @@ def linear_i8_gemm_times(c, iters=20):
                         tile_config=3 | 8, m=grad_dim)  # the configuration BackpropDelta launches: 256x128 tile, eight waves
         else:
             lib.gemm_nt(gt, st, bufs.delta, L.I8, L.I8, k_tile_scale=tsc, k_tile=k_tile, epilogue=L.EPI_ROW_TILE_MAXNORM, tile_scale=bufs.delta_tile_scale)
+    settle(dw)
     ms_dw = event_time_ms(dw, iters)
     gemm_ops = 2.0 * len_ * src_dim * grad_dim
     return {"shape": "dY[16384x4096] x W[4096x1024] and dY^T x X[16384x1024], int8 -> int32", "gop_per_launch": gemm_ops / 1e9,
@@ -174,7 +190,7 @@ def bench_linear_i8(args):
     step, len_ = c["step"], c["len"]
     for _ in range(args.warmup):
         step()
-    torch.cuda.synchronize()
+    settle(step)
     t0 = time.perf_counter()
     for _ in range(args.steps):
         step()
@@ -229,7 +245,7 @@ def bandwidth_kernels(iters=10):
 
     def add(name, nbytes, fn):
         fn()
-        torch.cuda.synchronize()
+        settle(fn, 25.0)
         ms = event_time_ms(fn, iters)
         res.append({"kernel": name, "mbytes": round(nbytes / 1e6, 1), "us": round(ms * 1e3, 1), "gbps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                     "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / PEAK_HBM, 3)})
@@ -300,7 +316,7 @@ def bandwidth_kernels(iters=10):
 
 def fp8_backward_gemms(n, dim, ffn, iters=100, warm=20, only_dominant=False):
     """the e4m3 backward GEMM shapes of the dense step, each timed alone with events over `iters` launches after `warm` untimed ones
-    (the device settles at its sustained clock within the first few milliseconds of such a run): dX of the FFN contract / expand
+    and 40 ms more of the same launches (settle()): dX of the FFN contract / expand
     matrices, the FFN delta (packed-delta epilogue) and the attention-width dX"""
     import torch
     from tscale2_amd import lib as L
@@ -319,7 +335,7 @@ def fp8_backward_gemms(n, dim, ffn, iters=100, warm=20, only_dominant=False):
             fn = lambda: lib.gemm_nt(a, b, c, L.E4M3, ctype or L.F32)  # noqa: E731
         for _ in range(warm):
             fn()
-        torch.cuda.synchronize()
+        settle(fn)
         ms = event_time_ms(fn, iters)
         ops = 2.0 * m * nn * k
 
@@ -427,7 +443,7 @@ def bench_step_fp8(args):
     # config[3] and config[4] beside the step (their own --workload lines carry the CPU legs): a few launches each
     import copy
     sub = copy.copy(args)
-    sub.no_cpu, sub.steps, sub.warmup, sub.small = True, 10, 3, False
+    sub.no_cpu, sub.steps, sub.warmup, sub.small = True, 20, 3, False
     a = bench_att_bwd(sub)
     out["att_bwd"] = {"workload": a["config"]["workload"], "ms": a["ms_per_step"], "tokens_per_s": a["value"], "tflops": a["roofline"]["achieved"],
                       "frac_of_bf16_peak": a["roofline"]["frac"], "kernel": a["roofline"]["kernel"], "kernels": a["kernels"]}
@@ -543,7 +559,7 @@ def bench_att_bwd(args):
                        dv.view(i16), L.BF16, which, ds=ds_pair)
     for _ in range(args.warmup):
         step()
-    torch.cuda.synchronize()
+    settle(step)
     ms = event_time_ms(step, args.steps)
     # the two kernels on their own, after the timed region (the device is warm by then)
     ms_dq = event_time_ms(lambda: step(1), args.steps)
@@ -609,7 +625,7 @@ def bench_moe_fp8(args):
         m.layer_backward(0)
     for _ in range(args.warmup):
         step()
-    torch.cuda.synchronize()
+    settle(step)
     ms = event_time_ms(step, args.steps)
     offs = m.read("expertOffset").ravel()
     per_expert = np.diff(offs[:experts + 1])
@@ -623,9 +639,7 @@ def bench_moe_fp8(args):
     c = torch.empty((rows, xp), dtype=torch.bfloat16, device="cuda")   # 16-bit results, as every grouped product of the layer stores them
     grp = (torch.arange(rows // 128, device="cuda", dtype=torch.int32) * experts // (rows // 128)).int().contiguous()
     grouped = lambda: lib.gemm_nt(a, b, c, L.E4M3, L.BF16, n=xp, tile_group=grp, b_slab_bytes=xp * dim)
-    for _ in range(300):   # (a launch is under 0.1 ms: the clocks take some 20 ms of load to settle after the set-up above)
-        grouped()
-    torch.cuda.synchronize()
+    settle(grouped)
     ms_g = event_time_ms(grouped, 300)
     gops = 2.0 * rows * xp * dim
     roof = {"bound": "mfma", "achieved": gops / (ms_g * 1e-3) / 1e12, "peak": PEAK_FP8 / 1e12, "unit": "TFLOP/s",
@@ -666,7 +680,7 @@ def bench_gemm_fp8(args):
     fn = lambda: lib.gemm_nt(a, b, c, L.E4M3, ct, **kw)  # noqa: E731
     for _ in range(args.warmup):
         fn()
-    torch.cuda.synchronize()
+    settle(fn)
     ms = event_time_ms(fn, args.steps)
     gops = 2.0 * n * dim * ffn
     reps = max(20, int(40.0 / ms))
