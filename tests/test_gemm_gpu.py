@@ -495,11 +495,12 @@ def test_grouped_products_on_the_persistent_kernel(lib, n, k, shrink, c16):
     assert torch.allclose(new[t * 128:(t + 1) * 128].view(view).float(), want, rtol=1e-2, atol=1e-3)
 
 
-@pytest.mark.parametrize("n,k,tiles,shrink", [(512, 1024, 23, 1), (256, 512, 9, 2), (1024, 640, 8, 2), (256, 1024, 1, 0)])
-def test_grouped_normalised_products_on_the_persistent_kernel(lib, n, k, tiles, shrink):
+@pytest.mark.parametrize("n,k,tiles,shrink,with_rope", [(512, 1024, 23, 1, False), (256, 512, 9, 2, False), (1024, 640, 8, 2, True), (256, 1024, 1, 0, False)])
+def test_grouped_normalised_products_on_the_persistent_kernel(lib, n, k, tiles, shrink, with_rope):
     """The expert-grouped product with the row-tile normalising epilogue (the experts' expand product) on the persistent kernel: a
     token's 128-column tile is held by two waves, which exchange their sums of squares through LDS.  Normalised bf16 rows and tile
-    scales bit-identical to the 128x128 kernel's; odd and even numbers of tiles per workgroup (either wave group ends the list)."""
+    scales bit-identical to the 128x128 kernel's, with and without the rotation of column pairs; odd and even numbers of tiles per
+    workgroup (either wave group ends the list)."""
     print(f"case grouped persistent normalised n={n} k={k} tiles={tiles} shrink={shrink}", flush=True)
     from tscale2_amd import lib as L
     g = torch.Generator(device="cuda").manual_seed(300 + n + k + tiles)
@@ -512,12 +513,16 @@ def test_grouped_normalised_products_on_the_persistent_kernel(lib, n, k, tiles, 
     b = (torch.randn((slabs * n, k), device="cuda", generator=g) * 4).to(torch.float8_e4m3fn).view(torch.uint8)
     tgd = torch.from_numpy(tg).cuda()
     m_live = m - 50 if tg[-1] >= 0 else m
+    rope = None
+    if with_rope:   # (cos, sin) pairs per row and column pair of a 128-wide tile
+        ang = torch.rand((m, 64), device="cuda", generator=g) * 6.28
+        rope = torch.stack((ang.cos(), ang.sin()), dim=2).reshape(m, 128).contiguous()
     res = []
     for cfg in (32768, 4096 | (shrink << 13)):
         c = torch.full((m, n), 0x1234, dtype=torch.int16, device="cuda")
         ts = torch.full((n // 128, m), -3.0, device="cuda")
         lib.gemm_nt(a, b, c, L.E4M3, L.BF16, alpha=2e-3, n=n, tile_group=tgd, b_slab_bytes=n * k, m_live=m_live, tile_config=cfg,
-                    epilogue=L.EPI_ROW_TILE_NORM, normalize=True, vec_scale=1 / 24.0, tile_scale=ts)
+                    epilogue=L.EPI_ROW_TILE_NORM, normalize=True, vec_scale=1 / 24.0, tile_scale=ts, rope=rope)
         torch.cuda.synchronize()
         res.append((c, ts))
     assert torch.equal(res[0][0], res[1][0])

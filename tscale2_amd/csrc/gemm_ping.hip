@@ -21,6 +21,8 @@
 //   * One fragment set, refilled in place: of the eight MFMAs of a 64-byte slice fa[0] is free after the fourth, fb[j] after (1,j),
 //     and each is fetched again - from the next slice, behind the barrier from the next stage - as soon as it is free.
 //   * Same contraction order per accumulator as every other kernel of the library, so results are bit-identical to theirs.
+//   * Expert-grouped products (the reference's TMoeMatMulKernelCall, src/gpt/compute/moe_matmul.cuh:47-120) run on the same schedule
+//     with the operands exchanged, see GRP below.
 #include "gemm_epilogue.h"
 
 using namespace gemmk;
