@@ -6,8 +6,8 @@ Default workload ("step_fp8") = the dense GPT forward + backward step the metric
 backward through every layer with every packed delta (no optimiser).  The same line carries the second half of the metric, the int8
 backward GEMMs of the linear-layer microbenchmark (`bwd_gemm_int8`: X i8 [16384x1024], dY [16384x4096], W i8 [4096x1024]) and the
 fused bandwidth kernels' GB/s (`bandwidth_kernels`).  All inputs are resident in HBM before a timed region starts.
-Other workloads: "linear_i8_bwd" (that microbenchmark as the step), "att_bwd", "moe_fp8", "gemm_fp8" (the dominant GEMM alone plus the
-copy probe: the command the HBM-traffic counters are collected on).
+Other workloads: "linear_i8_bwd" (that microbenchmark as the step), "att_bwd", "moe_fp8", "bandwidth" (the fused kernels alone) and
+"gemm_fp8" (the dominant GEMM alone); the last two end with the copy probe: the commands the HBM-traffic counters are collected on.
 
 python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
 """
@@ -223,7 +223,7 @@ def _fast_weights(torch, rows, cols, mode_e4m3, gen):
     return torch.clamp(torch.round(w), -128, 127).to(torch.int8).cpu().numpy(), 0.02
 
 
-def bandwidth_kernels(iters=10):
+def bandwidth_kernels(iters=10, settle_ms=25.0):
     """The fused bandwidth-bound kernels at the shapes of the dense fp8 step (32768 tokens, dim 2048, ffn 8192), of the int8
     linear-layer microbenchmark (16384 x 4096) and of the MoE layer (65536 tokens, top-2 of 64, dim 1024): algorithmic bytes (live
     elements x dtype size of every operand), event time, GB/s and the fraction of the 8 TB/s HBM peak.  Working sets are 0.2-2 GB,
@@ -235,6 +235,9 @@ def bandwidth_kernels(iters=10):
     Q = D
     f32, bf16, u8, i8 = torch.float32, torch.bfloat16, torch.uint8, torch.int8
     res = []
+    # (torch's generators are used once before the first launch of this library: under rocprofv3 their first use after it failed with
+    # "invalid device function")
+    torch.randn(4, device=dev); torch.randint(0, 2, (4,), device=dev); torch.rand(4, device=dev)
 
     def rnd(rows, cols, dt):
         if dt in (u8,):
@@ -245,7 +248,8 @@ def bandwidth_kernels(iters=10):
 
     def add(name, nbytes, fn):
         fn()
-        settle(fn, 25.0)
+        if settle_ms > 0:
+            settle(fn, settle_ms)
         ms = event_time_ms(fn, iters)
         res.append({"kernel": name, "mbytes": round(nbytes / 1e6, 1), "us": round(ms * 1e3, 1), "gbps": round(nbytes / (ms * 1e-3) / 1e9, 1),
                     "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / PEAK_HBM, 3)})
@@ -702,8 +706,29 @@ def bench_gemm_fp8(args):
             "copy_probe_gbps": copy, "roofline": roof}
 
 
+def bench_bandwidth(args):
+    """the fused bandwidth-bound kernels alone, followed by the copy probe of 1 GiB: the command their HBM counters (rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE) are collected on; the probe calibrates the counters.  `value` is the byte-weighted rate of the set.
+    With --steps below 5 the kernels are launched --steps times each after one warm-up launch and no settling loop (counter runs)."""
+    from tscale2_amd import lib as L
+    L.load()
+    few = args.steps < 5
+    res = bandwidth_kernels(iters=max(1, args.steps), settle_ms=0.0 if few else 25.0)
+    copy = L.probe_copy_rate(1 << 30)
+    nbytes = sum(r["mbytes"] for r in res) * 1e6
+    secs = sum(r["us"] for r in res) * 1e-6
+    worst = min(res, key=lambda r: r["frac_of_hbm_peak"])
+    roof = {"bound": "hbm", "achieved": nbytes / secs / 1e9, "peak": PEAK_HBM / 1e9, "unit": "GB/s", "frac": nbytes / secs / PEAK_HBM, "traffic": None,
+            "kernel": "all %d kernels, byte-weighted; lowest: %s (%.3f)" % (len(res), worst["kernel"], worst["frac_of_hbm_peak"])}
+    return {"metric": "fused gradient kernels, algorithmic GB/s on 1 MI355X as % of HBM peak", "value": nbytes / secs / 1e9, "unit": "GB/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": secs * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "mixed (fp32 / bf16 / e4m3 / int8 streams)", "data": "synthetic",
+            "config": {"workload": "the 13 fused bandwidth-bound kernels at the shapes of configs 1, 2 and 4, one launch series each"},
+            "copy_probe_gbps": copy, "bandwidth_kernels": res, "roofline": roof}
+
+
 WORKLOADS = {"linear_i8_bwd": bench_linear_i8, "step_fp8": bench_step_fp8, "att_bwd": bench_att_bwd, "moe_fp8": bench_moe_fp8,
-             "gemm_fp8": bench_gemm_fp8}
+             "gemm_fp8": bench_gemm_fp8, "bandwidth": bench_bandwidth}
 
 
 def main():

@@ -44,6 +44,10 @@ class Lib:
     def __init__(self, path=SO):
         if not os.path.exists(path):
             raise RuntimeError(f"{path} is missing: build it with `python -m tscale2_amd.build` (no CPU fallback exists)")
+        # torch ships its own copy of the HIP runtime.  It has to be in the process before this library is mapped: mapped first, the
+        # library binds to the system's copy, the process then holds two runtimes, and launches on torch's tensors fail with
+        # "invalid device function" (TS2_ERR_LAUNCH).
+        import torch  # noqa: F401
         self.dll = C.CDLL(path)
         self.dll.ts2_version.restype = C.c_char_p
 
