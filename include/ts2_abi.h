@@ -91,7 +91,9 @@ typedef struct ts2_gemm_args {
     int32_t epilogue;
     ts2_mat tileScale; /* ROW_TILE_MAXNORM: fp32 [n/128][m] */
     int32_t splitK;
-    /* bits 0-1: 0 = choose; 1 = 256x256 workgroup tile; 2 = 128x128; 3 = 256x128 (int8 with kTileScale, fp32 result).
+    /* bits 0-1: 0 = choose (256x256 when m, n are multiples of 256 and there are 192 tiles or more, except for TS2_E4M3 products with
+     * k <= 512, or k <= 1024 and TS2_EPI_ADD, which are mostly their epilogue and run on 128x128); 1 = 256x256 workgroup tile;
+     * 2 = 128x128; 3 = 256x128 (int8 with kTileScale, fp32 result).
      * Comparison switches, all off in normal use: bit 2 (4) unused (TS2_ERR_UNSUPPORTED); bit 3 (8) eight waves per workgroup (256x256
      * store/accumulate results; with tile 3: the form BackpropDelta launches); bit 4 (16) two LDS stages instead of the ring on the
      * 256x256 tile (and on the 128x128 tile with TS2_E4M3 operands, which takes the ring from k = 1024 on); bits 5-6 tile-order

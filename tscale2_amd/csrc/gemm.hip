@@ -1033,6 +1033,14 @@ template <int TYPE> int DispatchTile(const ts2_gemm_args *a, const GemmP &p, hip
         // 256x256 tiles only when they still fill the chip; the k-tile-scaled kernel keeps a second accumulator set and needs 128x128
         long tilesL = (long)(p.m / 256) * (p.n / 256) * (p.splitK > 1 ? p.splitK : 1) * (p.groupOffsets ? p.splitK_groups : 1);
         cfg = (tilesL >= 192 || p.nSeg > 1) ? 1 : 2;
+        // A short contraction is mostly its epilogue, which the 256x256 kernel (one workgroup per CU) overlaps with nothing; two or
+        // three workgroups of the 128x128 kernels per CU cover each other's.  Measured, e4m3, 65536 x 1024 and 32768 x 2048 results,
+        // 256x256 -> 128x128: accumulating into fp32 at K = 128 .. 1024 bytes 147-182 -> 115-150 us, into bf16 215-249 -> 128-175;
+        // stored bf16 at K <= 512 55-72 -> 32-53, stored fp32 at K <= 512 equal or better; at K = 1024 stored results are a toss-up.
+        if (TYPE == T_FP8 && p.nSeg == 1 && !p.kMajor && !a->kTileScale &&
+            (p.kBytes <= 512 || (p.kBytes <= 1024 && a->epilogue == TS2_EPI_ADD))) {
+            cfg = 2;
+        }
     }
     if (p.kMajor) {
         cfg = 1; // only the 256x256 ring kernel reads contraction-major operands
