@@ -95,6 +95,16 @@ def test_float_results_equal_the_ring_kernel_bit_for_bit(lib, ab, m, n, k, sh):
         lib.gemm_nt(a, b, gv, t, c_type, alpha=0.02, alpha_ptr=aptr, epilogue=epi, tile_config=PING | shrink(sh), m_live=m_live)
         torch.cuda.synchronize()
         assert torch.equal(gv, wv), (c_type, epi, m_live)
+    # 16-bit results whose rows do not start on 16 bytes (a view four columns into a wider array) leave as pairs of columns instead of
+    # row segments: same values, neighbours untouched
+    for c_type, dt in ((L.BF16, torch.bfloat16), (L.F16, torch.float16)):
+        wide = torch.full((m, n + 8), 7.0, device="cuda").to(dt)
+        want = torch.empty((m, n), device="cuda").to(dt)
+        lib.gemm_nt(a, b, want.view(torch.int16), t, c_type, alpha=0.02, alpha_ptr=aptr, tile_config=1, m_live=m - 37)
+        lib.gemm_nt(a, b, wide.view(torch.int16)[:, 4:4 + n], t, c_type, alpha=0.02, alpha_ptr=aptr, tile_config=PING | shrink(sh), m_live=m - 37)
+        torch.cuda.synchronize()
+        assert torch.equal(wide[:, 4:4 + n].view(torch.int16), want.view(torch.int16)), c_type
+        assert bool((wide[:, :4] == 7.0).all()) and bool((wide[:, 4 + n:] == 7.0).all())
     got = torch.empty((m, n), device="cuda")
     lib.gemm_nt(a, b, got, t, L.F32, tile_config=PING | shrink(sh))
     torch.cuda.synchronize()

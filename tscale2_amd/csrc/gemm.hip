@@ -1158,6 +1158,7 @@ extern "C" int ts2_gemm_nt(const ts2_gemm_args *a, void *streamPtr)
         }
     }
     p.nSeg = 1;
+    p.rowsF16 = 0;
     if (a->extraSegments) {
         const bool bigTile = (a->m % 256) == 0 && (a->n % 256) == 0 && (a->tileConfig & 3) <= 1 && !(a->tileConfig & (4 | 8 | 16)) && !a->tileGroup;
         // the 128x128 tile (chosen with tileConfig 2, or implied by tileGroup) takes one further product

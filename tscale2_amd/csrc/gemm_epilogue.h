@@ -49,6 +49,7 @@ struct GemmP {
     const uint8_t *segA[3], *segB[3];
     float segAlpha[3];
     const float *segAlphaPtr[3];
+    int rowsF16; // persistent kernel, row-owning epilogue: the 16-bit rows are IEEE half instead of bf16
 };
 
 enum { T_I8 = 0, T_FP8 = 1, T_BF16 = 2 };
